@@ -1,0 +1,725 @@
+"""Seeded op cases shared by the CPU suite (oracle vs numpy closed forms) and the GPU
+suite (HipBackend vs oracle).
+
+Every case is `Case(name, run, expect, kind)`:
+  run(be)   -> list of numpy arrays produced through the Backend API of `be`
+  expect()  -> the same list computed by numpy (closed form / float64), or None when
+               only backend-vs-backend comparison makes sense
+  kind      -> "exact" (bit-exact: integer, shape, index ops and IEEE-exact f32 ops),
+               "ew"    (f32 element-wise math: rtol 1e-4, atol 1e-6),
+               "red"   (matmul / sum: 1e-3 of the natural scale of the result)
+The tolerances are the ones the north-star states: bit-exact for integer/shape/index
+ops, rtol 1e-4 for f32 element-wise, 1e-3 relative for matmul and reductions.
+"""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import Callable, List, Optional
+
+import numpy as np
+
+from catgrad_amd import _abi as A
+
+F32_MIN = np.float32(-3.4028234663852886e38)
+
+
+@dataclass
+class Case:
+    name: str
+    run: Callable
+    expect: Optional[Callable]
+    kind: str = "exact"
+    scale: Optional[Callable] = None  # for "red": per-element magnitude bound
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+def f32(seed, shape, scale=1.0):
+    return (rng(seed).standard_normal(shape) * scale).astype(np.float32)
+
+
+def u32(seed, shape, hi=2**32):
+    return rng(seed).integers(0, hi, size=shape, dtype=np.uint64).astype(np.uint32)
+
+
+def total_key(x):
+    b = x.astype(np.float32).view(np.int32).astype(np.int64)
+    return np.where(b < 0, b ^ 0x7FFFFFFF, b)
+
+
+def argmax_last(x):
+    """Reference rule (ndarray.rs:670-694): max_by(total_cmp) => last of equal maxima."""
+    key = total_key(x) if x.dtype == np.float32 else x.astype(np.int64)
+    n = key.shape[-1]
+    rev = key[..., ::-1]
+    return (n - 1 - np.argmax(rev, axis=-1)).astype(np.uint32)[..., None]
+
+
+def max_last_f32(x):
+    """fold from f32::MIN with f32::max: NaN ignored (ndarray.rs:656-661)."""
+    y = np.where(np.isnan(x), F32_MIN, x)
+    return np.maximum(np.max(y, axis=-1, keepdims=True, initial=F32_MIN), F32_MIN).astype(np.float32)
+
+
+def rust_f32_as_u32(x):
+    x64 = x.astype(np.float64)
+    out = np.zeros(x.shape, dtype=np.uint32)
+    ok = ~np.isnan(x64)
+    clipped = np.clip(np.trunc(np.where(ok, x64, 0.0)), 0.0, 4294967295.0)
+    return np.where(ok, clipped, 0).astype(np.uint64).astype(np.uint32)
+
+
+def wrapping_pow(a, e):
+    a = a.astype(np.uint64)
+    out = np.ones_like(a)
+    e = e.copy()
+    M = np.uint64(0xFFFFFFFF)
+    for _ in range(32):
+        out = np.where(e & 1, (out * a) & M, out)
+        a = (a * a) & M
+        e = e >> 1
+    return out.astype(np.uint32)
+
+
+def topk_ref(x, k):
+    key = total_key(x)
+    idx = np.argsort(-key, axis=-1, kind="stable")[..., :k]
+    return np.take_along_axis(x, idx, axis=-1), idx.astype(np.uint32)
+
+
+# ---------------------------------------------------------------------------------------
+CASES: List[Case] = []
+
+
+def case(name, kind="exact", scale=None):
+    def deco(pair):
+        run, expect = pair()
+        CASES.append(Case(name, run, expect, kind, scale))
+        return pair
+
+    return deco
+
+
+def N(be, *ts):
+    return [be.to_numpy(t) for t in ts]
+
+
+# ---- creation ----------------------------------------------------------------------------
+for _n in (0, 1, 5, 2304, 70001):
+    @case(f"arange_{_n}")
+    def _(n=_n):
+        return (lambda be: N(be, be.arange(n))), (lambda: [np.arange(n, dtype=np.uint32)])
+
+for _shape in ([], [1], [3, 0, 2], [16, 4, 8, 0, 64], [7, 5]):
+    for _dt, _np in ((A.F32, np.float32), (A.U32, np.uint32)):
+        @case(f"zeros_{_dt}_{'x'.join(map(str, _shape)) or 'scalar'}")
+        def _(shape=_shape, dt=_dt, npdt=_np):
+            return (lambda be: N(be, be.zeros(shape, dt))), (lambda: [np.zeros(shape, dtype=npdt)])
+
+
+@case("from_vec_roundtrip")
+def _():
+    a, b, s = f32(1, (3, 5, 7)), u32(2, (4, 6)), np.float32(2.5).reshape(())
+    return (lambda be: N(be, be.from_numpy(a), be.from_numpy(b), be.from_numpy(s))), (lambda: [a, b, s])
+
+
+# ---- cast -----------------------------------------------------------------------------------
+CAST_F = np.array([0.0, -0.0, 0.9, 1.5, -1.5, 2.9999998, 16777217.0, 4294967040.0, 4294967296.0, 1e20, -1e20,
+                   np.nan, np.inf, -np.inf, 1e-40, 3.5e9], dtype=np.float32)
+CAST_U = np.array([0, 1, 16777216, 16777217, 16777218, 16777219, 2147483648 + 129, 4294967295, 4294967167,
+                   4294967168, 33554435], dtype=np.uint32)
+
+
+@case("cast_f32_to_u32_rust_as")
+def _():
+    return (lambda be: N(be, be.cast(be.from_numpy(CAST_F), A.U32))), (lambda: [rust_f32_as_u32(CAST_F)])
+
+
+@case("cast_u32_to_f32_rne")
+def _():
+    return (lambda be: N(be, be.cast(be.from_numpy(CAST_U), A.F32))), (lambda: [CAST_U.astype(np.float32)])
+
+
+@case("cast_identity_and_random")
+def _():
+    a = f32(3, (33, 17), 1000.0)
+    u = u32(4, (129,))
+    return (
+        lambda be: N(be, be.cast(be.from_numpy(a), A.F32), be.cast(be.from_numpy(a), A.U32),
+                     be.cast(be.from_numpy(u), A.U32), be.cast(be.from_numpy(u), A.F32)),
+        lambda: [a, rust_f32_as_u32(a), u, u.astype(np.float32)],
+    )
+
+
+# ---- binary -----------------------------------------------------------------------------------
+SPECIAL = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, np.nan, 1e-45, 3.4e38, -3.4e38, 0.5, 2.0], dtype=np.float32)
+
+
+def _bin_f32(name, npf, kind="exact"):
+    @case(f"{name}_f32", kind)
+    def _():
+        a, b = f32(10, (37, 65)), f32(11, (37, 65))
+        sa, sb = np.meshgrid(SPECIAL, SPECIAL)
+        sa, sb = np.ascontiguousarray(sa), np.ascontiguousarray(sb)
+
+        def run(be):
+            return N(be, getattr(be, name)(be.from_numpy(a), be.from_numpy(b)),
+                     getattr(be, name)(be.from_numpy(sa), be.from_numpy(sb)))
+
+        def expect():
+            with np.errstate(all="ignore"):
+                return [npf(a, b), npf(sa, sb)]
+
+        return run, expect
+
+
+_bin_f32("add", lambda a, b: a + b)
+_bin_f32("sub", lambda a, b: a - b)
+_bin_f32("mul", lambda a, b: a * b)
+_bin_f32("div", lambda a, b: a / b)
+_bin_f32("lt", lambda a, b: (a < b).astype(np.float32))
+_bin_f32("gt", lambda a, b: (a > b).astype(np.float32))
+_bin_f32("gte", lambda a, b: (a >= b).astype(np.float32))
+_bin_f32("lte", lambda a, b: (a <= b).astype(np.float32))
+_bin_f32("eq", lambda a, b: (a == b).astype(np.float32))
+
+
+def _bin_u32(name, npf):
+    @case(f"{name}_u32")
+    def _():
+        a, b = u32(12, (19, 33)), u32(13, (19, 33))
+        b[0, :8] = a[0, :8]
+        if name == "div":
+            b[b == 0] = 7
+        if name == "pow":
+            a[:, :16] %= 7
+            b %= 40
+
+        def run(be):
+            return N(be, getattr(be, name)(be.from_numpy(a), be.from_numpy(b)))
+
+        return run, (lambda: [npf(a, b)])
+
+
+_bin_u32("add", lambda a, b: a + b)
+_bin_u32("sub", lambda a, b: a - b)
+_bin_u32("mul", lambda a, b: a * b)
+_bin_u32("div", lambda a, b: a // b)
+_bin_u32("pow", wrapping_pow)
+_bin_u32("lt", lambda a, b: (a < b).astype(np.uint32))
+_bin_u32("gt", lambda a, b: (a > b).astype(np.uint32))
+_bin_u32("gte", lambda a, b: (a >= b).astype(np.uint32))
+_bin_u32("lte", lambda a, b: (a <= b).astype(np.uint32))
+_bin_u32("eq", lambda a, b: (a == b).astype(np.uint32))
+
+
+@case("pow_f32", "ew")
+def _():
+    a = np.abs(f32(14, (41, 23))) + 0.01
+    b = f32(15, (41, 23), 2.0)
+    th = np.full((32,), 500000.0, np.float32)
+    ex = (np.arange(32, dtype=np.float32) * np.float32(2.0 / 64))
+
+    def run(be):
+        return N(be, be.pow(be.from_numpy(a), be.from_numpy(b)), be.pow(be.from_numpy(th), be.from_numpy(ex)),
+                 be.pow(be.from_numpy(a), be.from_numpy(np.full_like(a, 0.5))))
+
+    def expect():
+        return [np.power(a.astype(np.float64), b.astype(np.float64)),
+                np.power(th.astype(np.float64), ex.astype(np.float64)), np.sqrt(a.astype(np.float64))]
+
+    return run, expect
+
+
+@case("pow_f32_special")
+def _():
+    a = np.array([-8.0, -2.0, 0.0, 2.0, 1.0, -1.0, 4.0], dtype=np.float32)
+    b = np.array([1.0 / 3, 0.5, 0.0, 3.0, np.nan, 2.0, 0.5], dtype=np.float32)
+
+    def run(be):
+        return N(be, be.pow(be.from_numpy(a), be.from_numpy(b)))
+
+    # negative base with fractional exponent is NaN (Rust powf); exact small powers
+    return run, (lambda: [np.array([np.nan, np.nan, 1.0, 8.0, 1.0, 1.0, 2.0], dtype=np.float32)])
+
+
+# ---- where --------------------------------------------------------------------------------------
+@case("where_f32_nan_mask")
+def _():
+    m = f32(16, (29, 31))
+    m[0, :4] = [np.nan, 0.0, -0.0, 1e-45]
+    x, y = f32(17, (29, 31)), f32(18, (29, 31))
+    return (lambda be: N(be, be.where_cond(be.from_numpy(m), be.from_numpy(x), be.from_numpy(y)))), (
+        lambda: [np.where(m > 0, x, y)])
+
+
+@case("where_u32")
+def _():
+    m, x, y = u32(19, (64,), 3), u32(20, (64,)), u32(21, (64,))
+    return (lambda be: N(be, be.where_cond(be.from_numpy(m), be.from_numpy(x), be.from_numpy(y)))), (
+        lambda: [np.where(m != 0, x, y)])
+
+
+# ---- unary ----------------------------------------------------------------------------------------
+@case("neg_floor_round_exact")
+def _():
+    a = f32(22, (45, 37), 10.0)
+    a[0, :8] = [0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 8388608.5, -0.0]
+    u = u32(23, (77,))
+    u[0] = 0
+
+    def run(be):
+        t = be.from_numpy(a)
+        return N(be, be.neg(t), be.floor(t), be.round(t), be.neg(be.from_numpy(u)))
+
+    return run, (lambda: [-a, np.floor(a), np.rint(a), (np.uint64(2**32) - u.astype(np.uint64)).astype(np.uint32)])
+
+
+@case("exp_log_f32", "ew")
+def _():
+    a = f32(24, (63, 65), 8.0)
+    p = np.abs(f32(25, (63, 65), 50.0)) + 1e-6
+
+    def run(be):
+        return N(be, be.exp(be.from_numpy(a)), be.log(be.from_numpy(p)))
+
+    return run, (lambda: [np.exp(a.astype(np.float64)), np.log(p.astype(np.float64))])
+
+
+@case("sin_cos_rope_range", "ew")
+def _():
+    a = (rng(26).uniform(-2304.0, 2304.0, size=(128, 65))).astype(np.float32)
+
+    def run(be):
+        return N(be, be.sin(be.from_numpy(a)), be.cos(be.from_numpy(a)))
+
+    return run, (lambda: [np.sin(a.astype(np.float64)), np.cos(a.astype(np.float64))])
+
+
+@case("exp_log_special")
+def _():
+    a = np.array([-np.inf, np.inf, 0.0, -200.0, 100.0], dtype=np.float32)
+    lg = np.array([0.0, -1.0, np.inf, 1.0], dtype=np.float32)
+
+    def run(be):
+        return N(be, be.exp(be.from_numpy(a)), be.log(be.from_numpy(lg)))
+
+    return run, (lambda: [np.array([0.0, np.inf, 1.0, 0.0, np.inf], np.float32),
+                          np.array([-np.inf, np.nan, np.inf, 0.0], np.float32)])
+
+
+# ---- views: broadcast / reshape / transpose / slice ---------------------------------------------------
+@case("broadcast_patterns")
+def _():
+    s = np.float32(3.25).reshape(())
+    col, row = f32(30, (6, 5, 1)), f32(31, (8,))
+    w = f32(32, (7, 9))
+    kv = f32(33, (2, 3, 1, 5, 4))
+
+    def run(be):
+        return N(be, be.broadcast(be.from_numpy(s), (4, 3)), be.broadcast(be.from_numpy(col), (6, 5, 8)),
+                 be.broadcast(be.from_numpy(row), (6, 5, 8)),
+                 be.broadcast(be.transpose(be.from_numpy(w), 0, 1), (3, 9, 7)),
+                 be.broadcast(be.from_numpy(kv), (2, 3, 4, 5, 4)), be.broadcast(be.from_numpy(row), (0, 8)))
+
+    def expect():
+        return [np.broadcast_to(s, (4, 3)), np.broadcast_to(col, (6, 5, 8)), np.broadcast_to(row, (6, 5, 8)),
+                np.broadcast_to(w.T, (3, 9, 7)), np.broadcast_to(kv, (2, 3, 4, 5, 4)), np.zeros((0, 8), np.float32)]
+
+    return run, expect
+
+
+@case("reshape_of_views")
+def _():
+    a = f32(34, (4, 6, 5, 8))
+    u = u32(35, (12, 10))
+
+    def run(be):
+        t = be.from_numpy(a)
+        return N(be,
+                 be.reshape(t, (24, 40)),
+                 be.reshape(be.transpose(t, 1, 2), (4, 5, 48)),
+                 be.reshape(be.slice(t, 3, 2, 4), (4, 6, 20)),
+                 be.reshape(be.slice(t, 1, 1, 3), (12, 40)),
+                 be.reshape(be.broadcast(be.reshape(be.slice(t, 1, 0, 1), (4, 1, 1, 5, 8)), (4, 1, 3, 5, 8)), (4, 3, 5, 8)),
+                 be.reshape(be.reshape(t, (4, 1, 6, 1, 40)), (4, 6, 40)),
+                 be.reshape(be.transpose(be.from_numpy(u), 0, 1), (120,)),
+                 be.reshape(be.transpose(be.transpose(t, 0, 3), 1, 2), (8 * 5, 6 * 4)))
+
+    def expect():
+        return [a.reshape(24, 40), a.transpose(0, 2, 1, 3).reshape(4, 5, 48), a[..., 2:6].reshape(4, 6, 20),
+                a[:, 1:4].reshape(12, 40),
+                np.broadcast_to(a[:, 0:1].reshape(4, 1, 1, 5, 8), (4, 1, 3, 5, 8)).reshape(4, 3, 5, 8),
+                a.reshape(4, 6, 40), u.T.reshape(120), a.transpose(3, 2, 1, 0).reshape(40, 24)]
+
+    return run, expect
+
+
+@case("transpose_slice_chain")
+def _():
+    a = f32(36, (5, 7, 9))
+
+    def run(be):
+        t = be.from_numpy(a)
+        return N(be, be.transpose(t, 0, 2), be.transpose(t, 1, 1), be.slice(t, 0, 4, 1), be.slice(t, 2, 9, 0),
+                 be.slice(be.transpose(be.slice(t, 1, 2, 4), 1, 2), 1, 3, 5),
+                 be.add(be.transpose(t, 0, 1), be.transpose(t, 0, 1)))
+
+    def expect():
+        return [a.transpose(2, 1, 0), a, a[4:5], a[:, :, 9:9], a[:, 2:6].transpose(0, 2, 1)[:, 3:8],
+                a.transpose(1, 0, 2) * 2]
+
+    return run, expect
+
+
+@case("elementwise_on_strided_operands")
+def _():
+    a, b = f32(37, (6, 10, 12)), f32(38, (10, 6, 12))
+    g = f32(39, (12,))
+    c = f32(40, (6, 10, 1))
+
+    def run(be):
+        ta, tb = be.from_numpy(a), be.from_numpy(b)
+        return N(be,
+                 be.mul(ta, be.transpose(tb, 0, 1)),
+                 be.mul(ta, be.broadcast(be.from_numpy(g), (6, 10, 12))),
+                 be.div(ta, be.broadcast(be.from_numpy(c), (6, 10, 12))),
+                 be.add(be.slice(ta, 2, 0, 6), be.neg(be.slice(ta, 2, 6, 6))),
+                 be.sub(be.broadcast(be.from_numpy(np.float32(1.5).reshape(())), (6, 10, 12)), ta),
+                 be.exp(be.transpose(be.slice(ta, 1, 1, 8), 0, 2)))
+
+    def expect():
+        return [a * b.transpose(1, 0, 2), a * g, a / c, a[..., :6] + (-a[..., 6:]), np.float32(1.5) - a,
+                np.exp(a[:, 1:9].transpose(2, 1, 0).astype(np.float64))]
+
+    return run, expect
+
+
+CASES[-1].kind = "ew"
+
+
+# ---- concat / index -------------------------------------------------------------------------------------
+@case("concat_all_dims")
+def _():
+    a, b0, b1, b2 = f32(41, (3, 4, 5)), f32(42, (2, 4, 5)), f32(43, (3, 6, 5)), f32(44, (3, 4, 1))
+    e = np.zeros((3, 0, 5), np.float32)
+    u1, u2 = u32(45, (4, 3)), u32(46, (4, 2))
+
+    def run(be):
+        ta = be.from_numpy(a)
+        return N(be, be.concat(ta, be.from_numpy(b0), 0), be.concat(ta, be.from_numpy(b1), 1),
+                 be.concat(ta, be.from_numpy(b2), 2), be.concat(be.from_numpy(e), ta, 1),
+                 be.concat(ta, be.from_numpy(e), 1), be.concat(be.from_numpy(u1), be.from_numpy(u2), 1),
+                 be.concat(be.neg(be.slice(ta, 2, 3, 2)), be.slice(ta, 2, 0, 3), 2),
+                 be.concat(be.transpose(ta, 0, 1), be.transpose(ta, 0, 1), 2))
+
+    def expect():
+        return [np.concatenate([a, b0], 0), np.concatenate([a, b1], 1), np.concatenate([a, b2], 2), a, a,
+                np.concatenate([u1, u2], 1), np.concatenate([-a[..., 3:], a[..., :3]], 2),
+                np.concatenate([a.transpose(1, 0, 2)] * 2, 2)]
+
+    return run, expect
+
+
+@case("kv_restack_chain")
+def _():
+    layers = [f32(50 + i, (2, 3, 4, 8)) for i in range(5)]
+
+    def run(be):
+        out = be.reshape(be.from_numpy(layers[0]), (1, 2, 3, 4, 8))
+        for l in layers[1:]:
+            out = be.concat(out, be.reshape(be.from_numpy(l), (1, 2, 3, 4, 8)), 0)
+        return N(be, out)
+
+    return run, (lambda: [np.stack(layers)])
+
+
+@case("index_gather")
+def _():
+    w = f32(60, (50, 16))
+    ids = u32(61, (23,), 50)
+    ids[:3] = [49, 0, 49]
+    x3 = u32(62, (4, 6, 5))
+    i1, i2 = np.array([5, 0, 0, 3], np.uint32), np.array([4, 4, 1], np.uint32)
+
+    def run(be):
+        tw, tx = be.from_numpy(w), be.from_numpy(x3)
+        return N(be, be.index(tw, 0, be.from_numpy(ids)), be.index(tx, 1, be.from_numpy(i1)),
+                 be.index(tx, 2, be.from_numpy(i2)), be.index(be.transpose(tw, 0, 1), 1, be.from_numpy(ids)),
+                 be.index(tw, 0, be.from_numpy(np.zeros((0,), np.uint32))),
+                 be.index(tw, 0, be.slice(be.from_numpy(ids), 0, 3, 7)))
+
+    def expect():
+        return [w[ids], x3[:, i1], x3[:, :, i2], w.T[:, ids], np.zeros((0, 16), np.float32), w[ids[3:10]]]
+
+    return run, expect
+
+
+# ---- reductions ---------------------------------------------------------------------------------------------
+@case("max_rules")
+def _():
+    a = f32(70, (9, 130))
+    a[0, :] = np.nan
+    a[1, :] = -np.inf
+    a[2, 5] = np.nan
+    a[3, 7] = np.inf
+    u = u32(71, (5, 67))
+    one = f32(72, (6,))
+    e = np.zeros((3, 0), np.float32)
+
+    def run(be):
+        return N(be, be.max(be.from_numpy(a)), be.max(be.from_numpy(u)), be.max(be.from_numpy(one)),
+                 be.max(be.from_numpy(e)), be.max(be.transpose(be.from_numpy(a), 0, 1)))
+
+    def expect():
+        return [max_last_f32(a), u.max(axis=-1, keepdims=True), max_last_f32(one), np.full((3, 1), F32_MIN),
+                max_last_f32(a.T)]
+
+    return run, expect
+
+
+@case("argmax_rules")
+def _():
+    a = f32(73, (11, 257))
+    a[0, :] = 1.0  # all tied -> last index
+    a[1, 3] = a[1, 200] = 99.0
+    a[2, :] = -0.0
+    a[2, 17] = 0.0  # +0 beats -0
+    a[3, 40] = np.nan  # +NaN is the greatest
+    a[4, 9] = np.inf
+    a[5, :] = -np.inf
+    neg_nan = np.array([0xFFC00000], dtype=np.uint32).view(np.float32)[0]
+    a[6, 100] = neg_nan  # -NaN is the least
+    u = u32(74, (6, 33), 5)
+    big = f32(75, (2, 128256), 0.02)
+
+    def run(be):
+        return N(be, be.argmax(be.from_numpy(a)), be.argmax(be.from_numpy(u)), be.argmax(be.from_numpy(big)),
+                 be.argmax(be.slice(be.transpose(be.from_numpy(a), 0, 1), 0, 10, 100)))
+
+    def expect():
+        return [argmax_last(a), argmax_last(u), argmax_last(big), argmax_last(np.ascontiguousarray(a.T[10:110]))]
+
+    return run, expect
+
+
+@case("sum_u32_and_small_f32")
+def _():
+    u = u32(76, (7, 300))
+    ints = rng(77).integers(-8, 9, size=(5, 4, 100)).astype(np.float32)  # exact in any order
+    e = np.zeros((4, 0), np.float32)
+
+    def run(be):
+        return N(be, be.sum(be.from_numpy(u)), be.sum(be.from_numpy(ints)), be.sum(be.from_numpy(e)),
+                 be.sum(be.transpose(be.from_numpy(ints), 1, 2)), be.sum(be.from_numpy(ints[0, 0])))
+
+    def expect():
+        return [u.sum(axis=-1, keepdims=True, dtype=np.uint32), ints.sum(-1, keepdims=True), np.zeros((4, 1), np.float32),
+                ints.transpose(0, 2, 1).sum(-1, keepdims=True), ints[0, 0].sum(keepdims=True)]
+
+    return run, expect
+
+
+def _sum_scale(arrs):
+    return lambda: [np.abs(a.astype(np.float64)).sum(-1, keepdims=True) for a in arrs]
+
+
+_SUM_IN = [f32(78, (33, 2048)), f32(79, (3, 5, 77)), np.square(f32(80, (16, 576)))]
+
+
+@case("sum_f32", "red", _sum_scale(_SUM_IN))
+def _():
+    def run(be):
+        return N(be, *[be.sum(be.from_numpy(a)) for a in _SUM_IN])
+
+    return run, (lambda: [a.astype(np.float64).sum(-1, keepdims=True) for a in _SUM_IN])
+
+
+@case("topk_rules")
+def _():
+    a = f32(81, (6, 40))
+    a[0, :] = 2.0
+    a[1, 5] = a[1, 30] = 50.0
+    big = f32(82, (3, 4, 128))
+
+    def run(be):
+        v1, i1 = be.topk(be.from_numpy(a), 4)
+        v2, i2 = be.topk(be.from_numpy(big), 8)
+        v3, i3 = be.topk(be.from_numpy(a), 40)
+        return N(be, v1, i1, v2, i2, v3, i3)
+
+    def expect():
+        return [*topk_ref(a, 4), *topk_ref(big, 8), *topk_ref(a, 40)]
+
+    return run, expect
+
+
+# ---- matmul ---------------------------------------------------------------------------------------------------
+def _mm_case(name, ashape, bshape, prep=None, seed=90):
+    a, b = f32(seed, ashape), f32(seed + 1, bshape)
+    prep = prep or (lambda be, ta, tb: (ta, tb, a, b))
+
+    def build(be):
+        ta, tb = be.from_numpy(a), be.from_numpy(b)
+        return prep(be, ta, tb)
+
+    def run(be):
+        x, y, _, _ = build(be)
+        return N(be, be.matmul(x, y))
+
+    def views():
+        class NP:  # numpy stand-in for the few view ops `prep` uses
+            @staticmethod
+            def transpose(t, i, j):
+                return np.swapaxes(t, i, j)
+
+            @staticmethod
+            def broadcast(t, s):
+                return np.broadcast_to(t, s)
+
+            @staticmethod
+            def reshape(t, s):
+                return t.reshape(s)
+
+            @staticmethod
+            def slice(t, d, s, l):
+                ix = [slice(None)] * t.ndim
+                ix[d] = slice(s, s + l)
+                return t[tuple(ix)]
+
+        x, y, _, _ = prep(NP, a, b)
+        return x.astype(np.float64), y.astype(np.float64)
+
+    def expect():
+        x, y = views()
+        return [x @ y]
+
+    def scale():
+        x, y = views()
+        return [np.abs(x) @ np.abs(y)]
+
+    CASES.append(Case(name, run, expect, "red", scale))
+
+
+_mm_case("mm_2d", (70, 50), (50, 90))
+_mm_case("mm_batched_3d", (5, 33, 65), (5, 65, 17))
+_mm_case("mm_two_batch_dims", (2, 3, 40, 24), (2, 3, 24, 56))
+_mm_case("mm_k1_and_m1", (4, 1, 1), (4, 1, 9))
+_mm_case("mm_decode_gemv", (4, 1, 576), (4, 576, 300))
+_mm_case("mm_linear_weight_view", (3, 20, 64), (48, 64),
+         lambda be, x, w: (x, be.broadcast(be.transpose(w, 0, 1), (3, 64, 48)), None, None))
+_mm_case("mm_linear_decode", (4, 1, 256), (1000, 256),
+         lambda be, x, w: (x, be.broadcast(be.transpose(w, 0, 1), (4, 256, 1000)), None, None))
+_mm_case("mm_attention_scores", (2, 40, 6, 32), (2, 56, 6, 32),
+         lambda be, q, k: (be.transpose(q, 1, 2), be.transpose(be.transpose(k, 1, 2), 2, 3), None, None))
+_mm_case("mm_attention_context", (2, 6, 40, 56), (2, 56, 6, 32),
+         lambda be, p, v: (p, be.transpose(v, 1, 2), None, None))
+_mm_case("mm_repeat_kv_rhs", (2, 6, 5, 16), (2, 2, 1, 16, 12),
+         lambda be, q, kv: (q, be.reshape(be.broadcast(kv, (2, 2, 3, 16, 12)), (2, 6, 16, 12)), None, None))
+_mm_case("mm_transposed_lhs", (3, 64, 30), (3, 64, 20), lambda be, a, b: (be.transpose(a, 1, 2), b, None, None))
+_mm_case("mm_sliced_operands", (2, 50, 80), (2, 80, 70),
+         lambda be, a, b: (be.slice(a, 2, 8, 64), be.slice(be.slice(b, 1, 8, 64), 2, 3, 33), None, None))
+_mm_case("mm_k_over_256", (2, 16, 700), (2, 700, 24))
+_mm_case("mm_tile_edges", (1, 129, 67), (1, 67, 131))
+_mm_case("mm_big_tile", (2, 256, 128), (2, 128, 384))
+
+
+@case("mm_u32_wrapping")
+def _():
+    a, b = u32(95, (2, 5, 7)), u32(96, (2, 7, 3))
+
+    def run(be):
+        return N(be, be.matmul(be.from_numpy(a), be.from_numpy(b)))
+
+    def expect():
+        return [(a.astype(np.uint64)[..., :, :, None] * b.astype(np.uint64)[..., None, :, :]).sum(-2).astype(np.uint32)]
+
+    return run, expect
+
+
+@case("mm_zero_extents")
+def _():
+    def run(be):
+        return N(be, be.matmul(be.zeros((2, 0, 4), A.F32), be.zeros((2, 4, 3), A.F32)),
+                 be.matmul(be.from_numpy(f32(97, (2, 3, 0))), be.from_numpy(f32(98, (2, 0, 5)))))
+
+    return run, (lambda: [np.zeros((2, 0, 3), np.float32), np.zeros((2, 3, 5), np.float32)])
+
+
+# ---- host read-backs ------------------------------------------------------------------------------------------------
+@case("to_bool_and_compare")
+def _():
+    a = f32(99, (13, 7))
+
+    def run(be):
+        t = be.from_numpy(a)
+        z = be.zeros((4, 4), A.F32)
+        nanv = be.from_numpy(np.array([np.nan, -1.0, 0.0], np.float32))
+        res = [be.to_bool(t), be.to_bool(z), be.to_bool(nanv), be.to_bool(be.from_numpy(np.array([0, 0, 2], np.uint32))),
+               be.to_bool(be.zeros((3,), A.U32)), be.to_bool(be.from_numpy(np.float32(5.0).reshape(()))),
+               be.compare(t, be.from_numpy(a)), be.compare(t, be.from_numpy(a + 1)),
+               be.compare(be.transpose(t, 0, 1), be.from_numpy(np.ascontiguousarray(a.T))),
+               be.compare(t, be.reshape(t, (7, 13))), be.compare(nanv, nanv), be.compare(z, be.zeros((4, 4), A.F32))]
+        return [np.array(res, dtype=np.uint32)]
+
+    return run, (lambda: [np.array([1, 0, 0, 1, 0, 1, 1, 0, 1, 0, 0, 1], np.uint32)])
+
+
+# ---- composites (stdlib definitions) vs float64 formulas -------------------------------------------------------------
+def softmax_ops(be, x):
+    """`nn::softmax` (catgrad/src/stdlib/nn/mod.rs:168-179) as backend calls."""
+    shp = x.shape
+    m = be.broadcast(be.max(x), shp)
+    ex = be.exp(be.sub(x, m))
+    s = be.broadcast(be.sum(ex), shp)
+    return be.div(ex, s)
+
+
+@case("softmax_with_f32_min_entry", "ew")
+def _():
+    a = f32(100, (7, 96), 3.0)
+    a[0, 5] = F32_MIN  # masked entry as built by causal_mask (helpers/tensors.rs:207-224)
+
+    def run(be):
+        y = softmax_ops(be, be.from_numpy(a))
+        return N(be, y, be.sum(y))
+
+    def expect():
+        x = a.astype(np.float64)
+        e = np.exp(x - x.max(-1, keepdims=True))
+        p = e / e.sum(-1, keepdims=True)
+        return [p, np.ones((7, 1))]
+
+    return run, expect
+
+
+def by_name(name):
+    for c in CASES:
+        if c.name == name:
+            return c
+    raise KeyError(name)
+
+
+def assert_close(kind, got, exp, scale=None, name=""):
+    """Tolerance of each kind, written out (see module docstring)."""
+    got, exp = np.asarray(got), np.asarray(exp)
+    assert got.shape == exp.shape, f"{name}: shape {got.shape} != {exp.shape}"
+    if kind == "exact":
+        if got.dtype == np.float32:
+            e32 = exp.astype(np.float32)
+            nan_ok = np.isnan(got) & np.isnan(e32)
+            same = (got == e32) | nan_ok
+            assert same.all(), f"{name}: {np.count_nonzero(~same)} f32 mismatches, first at {np.argwhere(~same)[:3].tolist()}"
+        else:
+            np.testing.assert_array_equal(got, exp.astype(got.dtype), err_msg=name)
+    elif kind == "ew":
+        np.testing.assert_allclose(got.astype(np.float64), exp.astype(np.float64), rtol=1e-4, atol=1e-6, err_msg=name)
+    elif kind == "red":
+        s = np.asarray(scale, dtype=np.float64) if scale is not None else np.abs(exp.astype(np.float64))
+        err = np.abs(got.astype(np.float64) - exp.astype(np.float64))
+        bound = 1e-3 * np.maximum(s, 1e-30)
+        assert (err <= bound).all(), f"{name}: max err/scale {np.max(err / np.maximum(s, 1e-30)):.3e} > 1e-3"
+    else:
+        raise ValueError(kind)
