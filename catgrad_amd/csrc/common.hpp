@@ -1,0 +1,170 @@
+// Internal declarations shared by the host runtime and the kernel launchers of
+// libcatgrad_hip.so.  Nothing here is part of the C ABI (include/catgrad_hip.h).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <atomic>
+#include <cstdint>
+#include <cstring>
+#include <map>
+#include <mutex>
+#include <string>
+
+#include "../../include/catgrad_hip.h"
+
+namespace cg {
+
+constexpr int kMaxRank = CG_MAX_RANK;
+
+int fail(int code, const char *fmt, ...) __attribute__((format(printf, 2, 3)));
+int hip_fail(hipError_t e, const char *what);
+
+#define CG_HIP(expr)                                          \
+    do {                                                      \
+        hipError_t _e = (expr);                               \
+        if (_e != hipSuccess) return cg::hip_fail(_e, #expr); \
+    } while (0)
+
+// Bits the kernels set in the backend's host-mapped fault word; reported by the next
+// call that waits for the device.
+enum : uint32_t { kFaultIndexRange = 1u, kFaultDivZero = 2u };
+
+// Device memory pool: size-class free lists on one stream.  A block freed while
+// kernels that use it are still queued may be handed out again at once, because every
+// later user is ordered behind them on the same stream.
+class Pool {
+  public:
+    int alloc(size_t bytes, void **ptr, size_t *cls);
+    void free(void *ptr, size_t cls);
+    void trim();
+    void stats(size_t *in_use, size_t *cached);
+    static size_t size_class(size_t bytes);
+
+  private:
+    std::mutex mu_;
+    std::multimap<size_t, void *> free_;
+    size_t in_use_ = 0, cached_ = 0;
+};
+
+} // namespace cg
+
+struct cg_backend {
+    int device = 0;
+    hipStream_t stream = nullptr;
+    cg::Pool pool;
+    uint32_t *fault_host = nullptr; // pinned, device-visible
+    uint32_t *fault_dev = nullptr;
+    uint32_t *flag_dev = nullptr;   // 4-byte scratch for to_bool / compare
+    uint32_t *flag_host = nullptr;  // pinned landing zone for it
+    std::string name;
+};
+
+namespace cg {
+
+struct Buffer {
+    std::atomic<long> rc{1};
+    void *ptr = nullptr;
+    size_t cls = 0;
+    cg_backend *be = nullptr;
+};
+
+} // namespace cg
+
+// A strided view of a device buffer.  Strides and offset are in elements; a stride of
+// 0 is a broadcast axis.  `uniform` marks a tensor all of whose elements equal `ubits`
+// (rank-0 constants, zeros, and every view of them): such tensors own no memory until a
+// kernel needs to address them, and kernels take their value as an immediate.
+struct cg_tensor {
+    std::atomic<long> rc{1};
+    cg_backend *be = nullptr;
+    cg::Buffer *buf = nullptr;
+    cg_dtype dt = CG_F32;
+    int rank = 0;
+    int64_t dims[cg::kMaxRank] = {0};
+    int64_t strides[cg::kMaxRank] = {0};
+    int64_t offset = 0;
+    bool uniform = false;
+    uint32_t ubits = 0;
+};
+
+namespace cg {
+
+inline int64_t numel(const cg_tensor *t) {
+    int64_t n = 1;
+    for (int i = 0; i < t->rank; i++) n *= t->dims[i];
+    return n;
+}
+bool is_contiguous(const cg_tensor *t);
+void release(cg_tensor *t);
+inline void retain(cg_tensor *t) { t->rc.fetch_add(1, std::memory_order_relaxed); }
+// Fresh row-major tensor with pool memory (none when numel == 0).
+int new_dense(cg_backend *be, cg_dtype dt, const int64_t *dims, int rank, cg_tensor **out);
+// Fresh uniform tensor (no memory).
+cg_tensor *new_uniform(cg_backend *be, cg_dtype dt, const int64_t *dims, int rank, uint32_t bits);
+// New handle sharing t's buffer and metadata.
+cg_tensor *new_view(const cg_tensor *t);
+// Device address of element 0 of the view; allocates the 4-byte backing word of a
+// uniform tensor on first use.
+int device_ptr(const cg_tensor *t, const void **ptr);
+
+// ---- magic-number division for 32-bit indices (Granlund-Montgomery round-up) ----
+struct FastDiv {
+    uint32_t d, m, s1, s2;
+};
+FastDiv make_fastdiv(uint32_t d);
+
+// ---- launch descriptors ------------------------------------------------------------
+constexpr int kMaxOuter = kMaxRank - 1;
+
+struct Operand {
+    const char *ptr;           // byte address of the view's first element (null if uniform)
+    int64_t os[kMaxOuter];     // element strides of the outer axes, innermost first
+    int64_t is;                // element stride of the inner axis
+    uint32_t uniform;          // 1: take `ubits`, never dereference ptr
+    uint32_t ubits;
+};
+
+struct EwGeom {
+    uint32_t nouter;           // collapsed rank - 1
+    uint32_t inner;            // extent of the inner axis
+    uint32_t ipr;              // work items per row (inner / VEC)
+    uint32_t vec;              // 1 or 4 elements per work item
+    FastDiv ipr_div;
+    uint32_t od[kMaxOuter];    // outer extents, innermost first
+    FastDiv odiv[kMaxOuter];
+    uint64_t total;            // work items
+};
+
+// Collapses the iteration space shared by `n` views of identical shape (views[0] is
+// the output) and fills geometry + operands.  Returns CG_ERR_UNSUPPORTED when the
+// space exceeds 2^32-1 work items.
+int plan_elementwise(const cg_tensor *const *views, int n, EwGeom *g, Operand *ops);
+
+// ---- kernel launchers (ew.hip, reduce.hip, matmul.hip) -------------------------------
+enum EwOp : int {
+    // unary (CG_NEG.. order of cg_unary_op)
+    kNeg = 0, kSin, kCos, kExp, kLog, kFloor, kRound,
+    // binary (order of cg_binary_op) offset by 16
+    kAdd = 16, kSub, kMul, kDiv, kPow, kLt, kGt, kGte, kLte, kEq,
+    kWhere = 32,
+    kCastF2U = 40, kCastU2F, kCopy
+};
+
+// out = op(ins...) element-wise; all views have out's shape.  `out` may be a strided view.
+int launch_elementwise(cg_backend *be, int op, cg_dtype dt, const cg_tensor *out, const cg_tensor *const *ins, int nin);
+int launch_arange(cg_backend *be, cg_tensor *out);
+int launch_fill_word(cg_backend *be, void *ptr, uint32_t bits);
+// out[outer, j, inner] = x[outer, idx[j], inner]
+int launch_gather(cg_backend *be, const cg_tensor *x, int dim, const cg_tensor *idx, cg_tensor *out);
+
+enum ReduceKind : int { kSum = 0, kMax = 1, kArgmax = 2 };
+int launch_reduce(cg_backend *be, int kind, const cg_tensor *x, cg_tensor *out);
+int launch_topk(cg_backend *be, const cg_tensor *x, int64_t k, cg_tensor *vals, cg_tensor *idxs);
+// *flag_dev = any(x > 0) / any(x != y)
+int launch_any_positive(cg_backend *be, const cg_tensor *x);
+int launch_any_diff(cg_backend *be, const cg_tensor *x, const cg_tensor *y);
+
+int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_tensor *out);
+
+} // namespace cg

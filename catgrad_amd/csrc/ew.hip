@@ -1,0 +1,297 @@
+// Element-wise, cast, strided-copy, gather and iota kernels for gfx950.
+//
+// One kernel shape serves every map over views of a common logical shape: the host
+// collapses the iteration space (plan_elementwise) to "rows x inner"; a work item is
+// one 16-byte vector (or one element) of the output; each lane handles UNROLL items a
+// block-stride apart so that every wave keeps several 16-byte loads per operand in
+// flight; operands are addressed through their own strides, so broadcast (stride 0),
+// transposed and sliced views are consumed in place and constants arrive as kernel
+// arguments.  All of these kernels are HBM-bound: 4 B read per operand element + 4 B
+// written per output element.
+//
+// Arithmetic follows NdArrayBackend (catgrad/src/interpreter/backend/ndarray.rs):
+// IEEE f32 with one rounding per operation (the file is compiled with
+// -ffp-contract=off), accurate libm-grade sin/cos/exp/log/pow, wrapping u32.
+#include "common.hpp"
+#include "device_utils.hpp"
+
+namespace cg {
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kUnroll = 4;
+
+// Rust `f32 as u32` (ndarray.rs:155): truncate, saturate, NaN -> 0.
+__device__ __forceinline__ uint32_t f32_as_u32(float v) {
+    if (!(v == v) || v <= 0.0f) return 0u;
+    if (v >= 4294967296.0f) return 0xFFFFFFFFu;
+    return (uint32_t)v;
+}
+
+__device__ __forceinline__ uint32_t wrapping_pow(uint32_t a, uint32_t e) {
+    uint32_t acc = 1;
+    while (e) {
+        if (e & 1) acc *= a;
+        a *= a;
+        e >>= 1;
+    }
+    return acc;
+}
+
+// One scalar application of OP on raw 32-bit words.  F = operands are f32.
+template <int OP, bool F>
+__device__ __forceinline__ uint32_t apply(uint32_t a, uint32_t b, uint32_t c, uint32_t *fault) {
+    (void)b;
+    (void)c;
+    (void)fault;
+    if constexpr (OP == kCopy) return a;
+    if constexpr (OP == kCastF2U) return f32_as_u32(asf(a));
+    if constexpr (OP == kCastU2F) return asu((float)a); // round to nearest even
+    if constexpr (OP == kWhere) return F ? (asf(a) > 0.0f ? b : c) : (a != 0 ? b : c);
+    if constexpr (F) {
+        float x = asf(a), y = asf(b);
+        if constexpr (OP == kNeg) return a ^ 0x80000000u;
+        if constexpr (OP == kSin) return asu(sinf(x));
+        if constexpr (OP == kCos) return asu(cosf(x));
+        if constexpr (OP == kExp) return asu(expf(x));
+        if constexpr (OP == kLog) return asu(logf(x));
+        if constexpr (OP == kFloor) return asu(floorf(x));
+        if constexpr (OP == kRound) return asu(rintf(x)); // ties to even (ndarray.rs:646-648)
+        if constexpr (OP == kAdd) return asu(x + y);
+        if constexpr (OP == kSub) return asu(x - y);
+        if constexpr (OP == kMul) return asu(x * y);
+        if constexpr (OP == kDiv) return asu(x / y);
+        if constexpr (OP == kPow) return asu(powf(x, y));
+        if constexpr (OP == kLt) return asu(x < y ? 1.0f : 0.0f);
+        if constexpr (OP == kGt) return asu(x > y ? 1.0f : 0.0f);
+        if constexpr (OP == kGte) return asu(x >= y ? 1.0f : 0.0f);
+        if constexpr (OP == kLte) return asu(x <= y ? 1.0f : 0.0f);
+        if constexpr (OP == kEq) return asu(x == y ? 1.0f : 0.0f);
+    } else {
+        if constexpr (OP == kNeg) return 0u - a;
+        if constexpr (OP == kAdd) return a + b;
+        if constexpr (OP == kSub) return a - b;
+        if constexpr (OP == kMul) return a * b;
+        if constexpr (OP == kDiv) {
+            if (b == 0) {
+                *fault = kFaultDivZero; // reported by the next waiting call
+                return 0u;
+            }
+            return a / b;
+        }
+        if constexpr (OP == kPow) return wrapping_pow(a, b);
+        if constexpr (OP == kLt) return a < b;
+        if constexpr (OP == kGt) return a > b;
+        if constexpr (OP == kGte) return a >= b;
+        if constexpr (OP == kLte) return a <= b;
+        if constexpr (OP == kEq) return a == b;
+    }
+    return 0u;
+}
+
+struct EwArgs {
+    EwGeom g;
+    Operand out;
+    Operand in[3];
+    uint32_t *fault;
+};
+
+// FLAT: the iteration space collapsed to a single axis (no index arithmetic at all).
+template <int OP, bool F, int NIN, int VEC, bool FLAT>
+__global__ __launch_bounds__(kBlock) void ew_kernel(const EwArgs a) {
+    const uint64_t base = (uint64_t)blockIdx.x * (kBlock * kUnroll) + threadIdx.x;
+    int64_t off[kUnroll][4];
+    bool live[kUnroll];
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++) {
+        uint64_t v64 = base + (uint64_t)u * kBlock;
+        live[u] = v64 < a.g.total;
+        uint32_t v = (uint32_t)v64;
+        if (FLAT) {
+            int64_t e = (int64_t)v * VEC;
+            off[u][0] = e * a.out.is;
+#pragma unroll
+            for (int k = 0; k < NIN; k++) off[u][k + 1] = e * a.in[k].is;
+        } else {
+            uint32_t row = fastdiv(v, a.g.ipr_div);
+            int64_t e = (int64_t)(v - row * a.g.ipr) * VEC;
+            int64_t oo = e * a.out.is;
+            int64_t oi[3];
+#pragma unroll
+            for (int k = 0; k < NIN; k++) oi[k] = e * a.in[k].is;
+            for (uint32_t d = 0; d < a.g.nouter; d++) {
+                uint32_t q = fastdiv(row, a.g.odiv[d]);
+                int64_t i = (int64_t)(row - q * a.g.od[d]);
+                row = q;
+                oo += i * a.out.os[d];
+#pragma unroll
+                for (int k = 0; k < NIN; k++) oi[k] += i * a.in[k].os[d];
+            }
+            off[u][0] = oo;
+#pragma unroll
+            for (int k = 0; k < NIN; k++) off[u][k + 1] = oi[k];
+        }
+    }
+    uint32_t x[kUnroll][3][VEC];
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++)
+        if (live[u]) {
+#pragma unroll
+            for (int k = 0; k < NIN; k++) load_words<VEC>(a.in[k], off[u][k + 1], x[u][k]);
+        }
+#pragma unroll
+    for (int u = 0; u < kUnroll; u++)
+        if (live[u]) {
+            uint32_t r[VEC];
+#pragma unroll
+            for (int j = 0; j < VEC; j++)
+                r[j] = apply<OP, F>(x[u][0][j], NIN > 1 ? x[u][1 % NIN][j] : 0u, NIN > 2 ? x[u][2 % NIN][j] : 0u, a.fault);
+            store_words<VEC>(a.out, off[u][0], r);
+        }
+}
+
+template <int OP, bool F, int NIN> int launch_variants(cg_backend *be, const EwArgs &a) {
+    uint64_t per_block = (uint64_t)kBlock * kUnroll;
+    uint64_t blocks = (a.g.total + per_block - 1) / per_block;
+    if (blocks == 0) return CG_OK;
+    dim3 grid((uint32_t)blocks), block(kBlock);
+    bool flat = a.g.nouter == 0;
+    if (a.g.vec == 4) {
+        if (flat)
+            hipLaunchKernelGGL((ew_kernel<OP, F, NIN, 4, true>), grid, block, 0, be->stream, a);
+        else
+            hipLaunchKernelGGL((ew_kernel<OP, F, NIN, 4, false>), grid, block, 0, be->stream, a);
+    } else {
+        if (flat)
+            hipLaunchKernelGGL((ew_kernel<OP, F, NIN, 1, true>), grid, block, 0, be->stream, a);
+        else
+            hipLaunchKernelGGL((ew_kernel<OP, F, NIN, 1, false>), grid, block, 0, be->stream, a);
+    }
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CG_OK : hip_fail(e, "element-wise kernel launch");
+}
+
+template <int OP, int NIN> int launch_by_dtype(cg_backend *be, cg_dtype dt, const EwArgs &a) {
+    return dt == CG_F32 ? launch_variants<OP, true, NIN>(be, a) : launch_variants<OP, false, NIN>(be, a);
+}
+
+__global__ void arange_kernel(uint32_t *out, uint32_t n) {
+    uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) out[i] = i;
+}
+
+__global__ void fill_word_kernel(uint32_t *p, uint32_t bits) { *p = bits; }
+
+// out[o, j, :] = x[o, idx[j], :]  with x row-major [outer, D, inner]
+template <int VEC>
+__global__ __launch_bounds__(kBlock) void gather_kernel(const uint32_t *__restrict__ x, const uint32_t *__restrict__ idx,
+                                                        int64_t idx_stride, uint32_t *__restrict__ out, uint32_t D,
+                                                        uint32_t inner, FastDiv ipr_div, uint32_t ipr, FastDiv j_div,
+                                                        uint32_t J, uint64_t total, uint32_t *fault) {
+    uint64_t v64 = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (v64 >= total) return;
+    uint32_t v = (uint32_t)v64;
+    uint32_t row = fastdiv(v, ipr_div);
+    uint32_t c = (v - row * ipr) * VEC;
+    uint32_t o = fastdiv(row, j_div);
+    uint32_t j = row - o * J;
+    uint32_t id = idx[(int64_t)j * idx_stride];
+    uint32_t *dst = out + (uint64_t)row * inner + c;
+    if (id >= D) { // the reference panics (ndarray `select`); report and write zeros
+        *fault = kFaultIndexRange;
+        if (VEC == 4)
+            *reinterpret_cast<uint4 *>(dst) = make_uint4(0, 0, 0, 0);
+        else
+            *dst = 0;
+        return;
+    }
+    const uint32_t *src = x + ((uint64_t)o * D + id) * inner + c;
+    if (VEC == 4)
+        *reinterpret_cast<uint4 *>(dst) = *reinterpret_cast<const uint4 *>(src);
+    else
+        *dst = *src;
+}
+
+} // namespace
+
+int launch_elementwise(cg_backend *be, int op, cg_dtype dt, const cg_tensor *out, const cg_tensor *const *ins, int nin) {
+    const cg_tensor *views[4] = {out, nullptr, nullptr, nullptr};
+    for (int k = 0; k < nin; k++) views[k + 1] = ins[k];
+    EwArgs a;
+    memset(&a, 0, sizeof a);
+    Operand ops[4];
+    int rc = plan_elementwise(views, nin + 1, &a.g, ops);
+    if (rc) return rc;
+    a.out = ops[0];
+    for (int k = 0; k < nin; k++) a.in[k] = ops[k + 1];
+    a.fault = be->fault_dev;
+    switch (op) {
+#define CG_EW1(OP) case OP: return launch_by_dtype<OP, 1>(be, dt, a);
+#define CG_EW2(OP) case OP: return launch_by_dtype<OP, 2>(be, dt, a);
+    CG_EW1(kNeg)
+    case kSin: return launch_variants<kSin, true, 1>(be, a);
+    case kCos: return launch_variants<kCos, true, 1>(be, a);
+    case kExp: return launch_variants<kExp, true, 1>(be, a);
+    case kLog: return launch_variants<kLog, true, 1>(be, a);
+    case kFloor: return launch_variants<kFloor, true, 1>(be, a);
+    case kRound: return launch_variants<kRound, true, 1>(be, a);
+    CG_EW2(kAdd) CG_EW2(kSub) CG_EW2(kMul) CG_EW2(kDiv) CG_EW2(kPow)
+    CG_EW2(kLt) CG_EW2(kGt) CG_EW2(kGte) CG_EW2(kLte) CG_EW2(kEq)
+    case kWhere: return launch_by_dtype<kWhere, 3>(be, dt, a);
+    case kCastF2U: return launch_variants<kCastF2U, true, 1>(be, a);
+    case kCastU2F: return launch_variants<kCastU2F, false, 1>(be, a);
+    case kCopy: return launch_variants<kCopy, false, 1>(be, a);
+#undef CG_EW1
+#undef CG_EW2
+    default: return fail(CG_ERR_ARG, "unknown element-wise op %d", op);
+    }
+}
+
+int launch_arange(cg_backend *be, cg_tensor *out) {
+    uint32_t n = (uint32_t)out->dims[0];
+    hipLaunchKernelGGL(arange_kernel, dim3((n + 255) / 256), dim3(256), 0, be->stream,
+                       static_cast<uint32_t *>(out->buf->ptr), n);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CG_OK : hip_fail(e, "arange launch");
+}
+
+int launch_fill_word(cg_backend *be, void *ptr, uint32_t bits) {
+    hipLaunchKernelGGL(fill_word_kernel, dim3(1), dim3(1), 0, be->stream, static_cast<uint32_t *>(ptr), bits);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CG_OK : hip_fail(e, "fill launch");
+}
+
+int launch_gather(cg_backend *be, const cg_tensor *x, int dim, const cg_tensor *idx, cg_tensor *out) {
+    int64_t outer = 1, inner = 1;
+    for (int i = 0; i < dim; i++) outer *= x->dims[i];
+    for (int i = dim + 1; i < x->rank; i++) inner *= x->dims[i];
+    int64_t D = x->dims[dim], J = out->dims[dim];
+    if (D > 0xFFFFFFFFll || inner > 0xFFFFFFFFll || outer * J > 0xFFFFFFFFll)
+        return fail(CG_ERR_UNSUPPORTED, "index: extents above 2^32-1");
+    const void *xp, *ip;
+    int rc = device_ptr(x, &xp);
+    if (rc) return rc;
+    rc = device_ptr(idx, &ip);
+    if (rc) return rc;
+    int64_t istride = idx->uniform ? 0 : (idx->rank == 1 ? idx->strides[0] : 1);
+    uint32_t *op = static_cast<uint32_t *>(out->buf->ptr);
+    bool vec4 = inner % 4 == 0 && reinterpret_cast<uintptr_t>(xp) % 16 == 0;
+    uint32_t vec = vec4 ? 4 : 1;
+    uint32_t ipr = (uint32_t)(inner / vec);
+    uint64_t total = (uint64_t)outer * J * ipr;
+    if (total > 0xFFFFFFFFull) return fail(CG_ERR_UNSUPPORTED, "index: launch above 2^32-1 work items");
+    dim3 grid((uint32_t)((total + kBlock - 1) / kBlock)), block(kBlock);
+    if (vec4)
+        hipLaunchKernelGGL((gather_kernel<4>), grid, block, 0, be->stream, static_cast<const uint32_t *>(xp),
+                           static_cast<const uint32_t *>(ip), istride, op, (uint32_t)D, (uint32_t)inner,
+                           make_fastdiv(ipr), ipr, make_fastdiv((uint32_t)J), (uint32_t)J, total, be->fault_dev);
+    else
+        hipLaunchKernelGGL((gather_kernel<1>), grid, block, 0, be->stream, static_cast<const uint32_t *>(xp),
+                           static_cast<const uint32_t *>(ip), istride, op, (uint32_t)D, (uint32_t)inner,
+                           make_fastdiv(ipr), ipr, make_fastdiv((uint32_t)J), (uint32_t)J, total, be->fault_dev);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CG_OK : hip_fail(e, "gather launch");
+}
+
+} // namespace cg

@@ -1,0 +1,394 @@
+// Batched matrix multiply for gfx950: C[b, M, N] = A[b, M, K] * B[b, K, N], f32.
+//
+// Operands are consumed through their strides: row/column strides of A and B are
+// arbitrary (transposed views cost nothing), every batch axis has its own stride per
+// operand (0 = shared), so `linear`'s transposed, batch-broadcast weight view
+// (catgrad/src/stdlib/nn/mod.rs:182-204) and attention's [B, h, S, hd] head views
+// (catgrad-llm-models/src/models/llama.rs:285-345) are multiplied in place.  When the
+// right-hand side is shared by the whole batch and the left-hand side's batch and row
+// axes form one run, the batch is folded into M (one tall GEMM instead of B small ones).
+//
+// Kernels
+//   mfma_gemm_kernel   128x128x16 macro tile, 256 threads = 2x2 waves, each wave a 64x64
+//                      quadrant as 2x2 v_mfma_f32_32x32x2_f32 accumulators (64 VGPRs).
+//                      A and B tiles are staged K-fastest in LDS (pitch 20 words: the
+//                      128-bit fragment reads of 8 consecutive rows hit 32 distinct
+//                      banks), two LDS buffers, next tile's global loads in flight during
+//                      the MFMAs.  MFMA-bound: 2*M*N*K flop.
+//   skinny_kt_kernel   M <= 8 with K-contiguous B rows (decode-time linear layers and
+//                      q.K^T): one wave per output column, 16-byte loads along K, wave
+//                      shuffle reduction.  HBM-bound: 4*K*N bytes of B.
+//   simple_gemm_kernel u32 (wrapping) and any shape the others decline.
+//
+// Accumulation is f32 with fused multiply-add; the summation order differs from the
+// reference's `matrixmultiply::sgemm`, which is why the contract for matmul is 1e-3
+// relative (ndarray.rs:750-816 makes no promise on order either).
+#include "common.hpp"
+#include "device_utils.hpp"
+
+namespace cg {
+
+namespace {
+
+constexpr int kMaxBatchAxes = 6;
+
+struct MmArgs {
+    const uint32_t *A;
+    const uint32_t *B;
+    uint32_t *C;
+    uint32_t M, N, K;
+    int64_t a_sm, a_sk, b_sk, b_sn;
+    uint32_t nb;                    // collapsed batch axes
+    uint32_t bd[kMaxBatchAxes];     // extents, innermost first
+    FastDiv bdiv[kMaxBatchAxes];
+    int64_t a_bs[kMaxBatchAxes], b_bs[kMaxBatchAxes];
+    uint32_t batch;
+    uint32_t a_vec, b_vec;          // 16-byte loads along the unit-stride axis are legal
+};
+
+__device__ __forceinline__ void batch_offsets(const MmArgs &a, uint32_t b, int64_t &oa, int64_t &ob) {
+    oa = 0;
+    ob = 0;
+    for (uint32_t d = 0; d < a.nb; d++) {
+        uint32_t q = fastdiv(b, a.bdiv[d]);
+        int64_t i = (int64_t)(b - q * a.bd[d]);
+        b = q;
+        oa += i * a.a_bs[d];
+        ob += i * a.b_bs[d];
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// MFMA kernel
+// ------------------------------------------------------------------------------------------
+constexpr int BM = 128, BN = 128, BK = 16;
+constexpr int PITCH = BK + 4; // words per LDS row
+constexpr int kThreads = 256;
+
+typedef float float4v __attribute__((ext_vector_type(4)));
+typedef float float16v __attribute__((ext_vector_type(16)));
+
+// Loads one 128 x 16 tile (rows along `R` with stride s_r, k with stride s_k) into
+// registers: 2 x float4 per thread.  Layout of the 512 float4 slots of a tile:
+//   K-contiguous source (s_k == 1): slot = row*4 + kq      (float4 along k)
+//   R-contiguous source (s_r == 1): slot = k*32 + rq       (float4 along rows)
+//   otherwise                      : as K-contiguous, element by element
+struct TileRegs {
+    float4v v[2];
+};
+
+__device__ __forceinline__ float ld_guard(const uint32_t *p, bool ok) { return ok ? asf(*p) : 0.0f; }
+
+template <bool ROWS_FAST>
+__device__ __forceinline__ void load_tile(TileRegs &t, const uint32_t *base, int64_t s_r, int64_t s_k, uint32_t r0,
+                                          uint32_t k0, uint32_t R, uint32_t K, bool vec_ok) {
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        uint32_t slot = threadIdx.x + h * kThreads;
+        if (!ROWS_FAST) {
+            uint32_t row = r0 + slot / 4, k = k0 + (slot % 4) * 4;
+            const uint32_t *p = base + (int64_t)row * s_r + (int64_t)k * s_k;
+            if (vec_ok && row < R && k + 3 < K) {
+                t.v[h] = *reinterpret_cast<const float4v *>(p);
+            } else {
+                bool rok = row < R;
+                t.v[h][0] = ld_guard(p, rok && k < K);
+                t.v[h][1] = ld_guard(p + s_k, rok && k + 1 < K);
+                t.v[h][2] = ld_guard(p + 2 * s_k, rok && k + 2 < K);
+                t.v[h][3] = ld_guard(p + 3 * s_k, rok && k + 3 < K);
+            }
+        } else {
+            uint32_t k = k0 + slot / 32, row = r0 + (slot % 32) * 4;
+            const uint32_t *p = base + (int64_t)row * s_r + (int64_t)k * s_k;
+            if (vec_ok && k < K && row + 3 < R) {
+                t.v[h] = *reinterpret_cast<const float4v *>(p);
+            } else {
+                bool kok = k < K;
+                t.v[h][0] = ld_guard(p, kok && row < R);
+                t.v[h][1] = ld_guard(p + s_r, kok && row + 1 < R);
+                t.v[h][2] = ld_guard(p + 2 * s_r, kok && row + 2 < R);
+                t.v[h][3] = ld_guard(p + 3 * s_r, kok && row + 3 < R);
+            }
+        }
+    }
+}
+
+// Stores the registers K-fastest into an LDS tile [128][PITCH].
+template <bool ROWS_FAST> __device__ __forceinline__ void store_tile(const TileRegs &t, float *lds) {
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        uint32_t slot = threadIdx.x + h * kThreads;
+        if (!ROWS_FAST) {
+            uint32_t row = slot / 4, k = (slot % 4) * 4;
+            *reinterpret_cast<float4v *>(lds + row * PITCH + k) = t.v[h];
+        } else {
+            uint32_t k = slot / 32, row = (slot % 32) * 4;
+            lds[(row + 0) * PITCH + k] = t.v[h][0];
+            lds[(row + 1) * PITCH + k] = t.v[h][1];
+            lds[(row + 2) * PITCH + k] = t.v[h][2];
+            lds[(row + 3) * PITCH + k] = t.v[h][3];
+        }
+    }
+}
+
+template <bool A_MFAST, bool B_NFAST> __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
+    __shared__ float lds_a[2][BM * PITCH];
+    __shared__ float lds_b[2][BN * PITCH];
+
+    const uint32_t tiles_n = (a.N + BN - 1) / BN;
+    const uint32_t tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x % tiles_n;
+    const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
+    int64_t oa, ob;
+    batch_offsets(a, blockIdx.y, oa, ob);
+    const uint32_t *A = a.A + oa;
+    const uint32_t *B = a.B + ob;
+    uint32_t *C = a.C + (uint64_t)blockIdx.y * a.M * a.N;
+
+    const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    const uint32_t wm = (wave / 2) * 64, wn = (wave % 2) * 64; // wave quadrant
+    const uint32_t li = lane % 32, lg = lane / 32;
+
+    float16v acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+
+    TileRegs ra, rb;
+    const uint32_t nk = (a.K + BK - 1) / BK;
+    load_tile<A_MFAST>(ra, A, a.a_sm, a.a_sk, m0, 0, a.M, a.K, a.a_vec);
+    load_tile<B_NFAST>(rb, B, a.b_sn, a.b_sk, n0, 0, a.N, a.K, a.b_vec);
+    store_tile<A_MFAST>(ra, lds_a[0]);
+    store_tile<B_NFAST>(rb, lds_b[0]);
+    __syncthreads();
+
+    for (uint32_t kt = 0; kt < nk; kt++) {
+        const uint32_t cur = kt & 1;
+        if (kt + 1 < nk) {
+            load_tile<A_MFAST>(ra, A, a.a_sm, a.a_sk, m0, (kt + 1) * BK, a.M, a.K, a.a_vec);
+            load_tile<B_NFAST>(rb, B, a.b_sn, a.b_sk, n0, (kt + 1) * BK, a.N, a.K, a.b_vec);
+        }
+        const float *la = lds_a[cur], *lb = lds_b[cur];
+#pragma unroll
+        for (int kc = 0; kc < BK / 8; kc++) {
+            // lane group g supplies k = 8*kc + 4*g + t to the t-th MFMA of this chunk, for
+            // A and B alike, so one 128-bit LDS read feeds four MFMAs.
+            float4v fa[2], fb[2];
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+                fa[i] = *reinterpret_cast<const float4v *>(la + (wm + i * 32 + li) * PITCH + kc * 8 + lg * 4);
+#pragma unroll
+            for (int j = 0; j < 2; j++)
+                fb[j] = *reinterpret_cast<const float4v *>(lb + (wn + j * 32 + li) * PITCH + kc * 8 + lg * 4);
+#pragma unroll
+            for (int t = 0; t < 4; t++)
+#pragma unroll
+                for (int i = 0; i < 2; i++)
+#pragma unroll
+                    for (int j = 0; j < 2; j++)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][t], fb[j][t], acc[i][j], 0, 0, 0);
+        }
+        if (kt + 1 < nk) {
+            store_tile<A_MFAST>(ra, lds_a[cur ^ 1]);
+            store_tile<B_NFAST>(rb, lds_b[cur ^ 1]);
+        }
+        __syncthreads();
+    }
+
+    // D layout of v_mfma_f32_32x32x2_f32: lane (li, lg), register v -> row 8*(v/4) + 4*lg + v%4, col li
+#pragma unroll
+    for (int i = 0; i < 2; i++)
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            uint32_t col = n0 + wn + j * 32 + li;
+            if (col < a.N) {
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    uint32_t row = m0 + wm + i * 32 + 8 * (v / 4) + 4 * lg + (v % 4);
+                    if (row < a.M) C[(uint64_t)row * a.N + col] = asu(acc[i][j][v]);
+                }
+            }
+        }
+}
+
+// ------------------------------------------------------------------------------------------
+// Skinny kernel: M <= 8, B rows K-contiguous (b_sk == 1).  One wave per output column.
+// ------------------------------------------------------------------------------------------
+template <int MM> __global__ __launch_bounds__(kThreads) void skinny_kt_kernel(const MmArgs a) {
+    const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    const uint32_t n = blockIdx.x * (kThreads / 64) + wave;
+    if (n >= a.N) return;
+    int64_t oa, ob;
+    batch_offsets(a, blockIdx.y, oa, ob);
+    const uint32_t *A = a.A + oa;
+    const uint32_t *Brow = a.B + ob + (int64_t)n * a.b_sn;
+    float acc[MM];
+#pragma unroll
+    for (int m = 0; m < MM; m++) acc[m] = 0.0f;
+    const bool vec = a.b_vec && a.a_vec && a.a_sk == 1 && (a.K % 4 == 0);
+    if (vec) {
+        for (uint32_t k = lane * 4; k < a.K; k += 256) {
+            float4v b = *reinterpret_cast<const float4v *>(Brow + k);
+#pragma unroll
+            for (int m = 0; m < MM; m++) {
+                if ((uint32_t)m < a.M) {
+                    float4v x = *reinterpret_cast<const float4v *>(A + (int64_t)m * a.a_sm + k);
+                    acc[m] = fmaf(x[0], b[0], acc[m]);
+                    acc[m] = fmaf(x[1], b[1], acc[m]);
+                    acc[m] = fmaf(x[2], b[2], acc[m]);
+                    acc[m] = fmaf(x[3], b[3], acc[m]);
+                }
+            }
+        }
+    } else {
+        for (uint32_t k = lane; k < a.K; k += 64) {
+            float b = asf(Brow[k]);
+#pragma unroll
+            for (int m = 0; m < MM; m++)
+                if ((uint32_t)m < a.M) acc[m] = fmaf(asf(A[(int64_t)m * a.a_sm + (int64_t)k * a.a_sk]), b, acc[m]);
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < MM; m++) {
+        float v = acc[m];
+#pragma unroll
+        for (int s = 32; s >= 1; s >>= 1) v += __shfl_xor(v, s);
+        if (lane == 0 && (uint32_t)m < a.M) a.C[((uint64_t)blockIdx.y * a.M + m) * a.N + n] = asu(v);
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// Plain kernel: one thread per output element.  u32 with wrapping arithmetic
+// (ndarray.rs:181) and the f32 shapes nothing else takes.
+// ------------------------------------------------------------------------------------------
+template <bool F> __global__ __launch_bounds__(kThreads) void simple_gemm_kernel(const MmArgs a) {
+    uint64_t e = (uint64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (e >= (uint64_t)a.M * a.N) return;
+    uint32_t m = (uint32_t)(e / a.N), n = (uint32_t)(e % a.N);
+    int64_t oa, ob;
+    batch_offsets(a, blockIdx.y, oa, ob);
+    const uint32_t *A = a.A + oa + (int64_t)m * a.a_sm;
+    const uint32_t *B = a.B + ob + (int64_t)n * a.b_sn;
+    uint32_t r;
+    if (F) {
+        float s = 0.0f;
+        for (uint32_t k = 0; k < a.K; k++) s = fmaf(asf(A[(int64_t)k * a.a_sk]), asf(B[(int64_t)k * a.b_sk]), s);
+        r = asu(s);
+    } else {
+        uint32_t s = 0;
+        for (uint32_t k = 0; k < a.K; k++) s += A[(int64_t)k * a.a_sk] * B[(int64_t)k * a.b_sk];
+        r = s;
+    }
+    a.C[(uint64_t)blockIdx.y * a.M * a.N + e] = r;
+}
+
+} // namespace
+
+int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_tensor *out) {
+    const int r = x->rank;
+    int64_t M = x->dims[r - 2], K = x->dims[r - 1], N = y->dims[r - 1];
+    MmArgs a;
+    memset(&a, 0, sizeof a);
+    const void *pa, *pb;
+    int rc = device_ptr(x, &pa);
+    if (rc) return rc;
+    rc = device_ptr(y, &pb);
+    if (rc) return rc;
+    a.A = static_cast<const uint32_t *>(pa);
+    a.B = static_cast<const uint32_t *>(pb);
+    a.C = static_cast<uint32_t *>(out->buf->ptr);
+    auto stride = [](const cg_tensor *t, int ax) -> int64_t { return t->uniform ? 0 : t->strides[ax]; };
+    a.a_sm = stride(x, r - 2);
+    a.a_sk = stride(x, r - 1);
+    a.b_sk = stride(y, r - 2);
+    a.b_sn = stride(y, r - 1);
+
+    // collapse the batch axes of A and B together (C is row-major, so it follows)
+    int64_t bd[kMaxRank], sa[kMaxRank], sb[kMaxRank];
+    int w = 0;
+    for (int i = 0; i < r - 2; i++) {
+        if (x->dims[i] == 1) continue;
+        int64_t d = x->dims[i], s1 = stride(x, i), s2 = stride(y, i);
+        if (w > 0 && sa[w - 1] == s1 * d && sb[w - 1] == s2 * d) {
+            bd[w - 1] *= d;
+            sa[w - 1] = s1;
+            sb[w - 1] = s2;
+        } else {
+            bd[w] = d;
+            sa[w] = s1;
+            sb[w] = s2;
+            w++;
+        }
+    }
+    // fold the innermost batch axis into M when B ignores it and A walks it as more rows
+    while (w > 0 && sb[w - 1] == 0 && (M == 1 || sa[w - 1] == a.a_sm * M)) {
+        if (M == 1) a.a_sm = sa[w - 1];
+        M *= bd[w - 1];
+        w--;
+    }
+    if (w > kMaxBatchAxes) return fail(CG_ERR_UNSUPPORTED, "matmul: more than %d non-mergeable batch axes", kMaxBatchAxes);
+    int64_t batch = 1;
+    for (int i = 0; i < w; i++) batch *= bd[i];
+    if (M > 0x7FFFFFFFll || N > 0x7FFFFFFFll || K > 0x7FFFFFFFll || batch > 65535ll * 1024)
+        return fail(CG_ERR_UNSUPPORTED, "matmul: extent above 2^31-1");
+    a.M = (uint32_t)M;
+    a.N = (uint32_t)N;
+    a.K = (uint32_t)K;
+    a.nb = (uint32_t)w;
+    a.batch = (uint32_t)batch;
+    bool a_al = reinterpret_cast<uintptr_t>(pa) % 16 == 0, b_al = reinterpret_cast<uintptr_t>(pb) % 16 == 0;
+    for (int d = 0; d < w; d++) {
+        a.bd[d] = (uint32_t)bd[w - 1 - d];
+        a.bdiv[d] = make_fastdiv(a.bd[d]);
+        a.a_bs[d] = sa[w - 1 - d];
+        a.b_bs[d] = sb[w - 1 - d];
+        if (a.a_bs[d] % 4) a_al = false;
+        if (a.b_bs[d] % 4) b_al = false;
+    }
+    // 16-byte loads run along the unit-stride axis; the other axis' stride must keep alignment
+    const bool a_kfast = a.a_sk == 1 || K == 1, a_mfast = !a_kfast && a.a_sm == 1;
+    const bool b_kfast = a.b_sk == 1 || K == 1, b_nfast = !b_kfast && a.b_sn == 1;
+    a.a_vec = a_al && ((a.a_sk == 1 && a.a_sm % 4 == 0) || (a_mfast && a.a_sk % 4 == 0));
+    a.b_vec = b_al && ((a.b_sk == 1 && a.b_sn % 4 == 0) || (b_nfast && a.b_sk % 4 == 0));
+
+    if (batch > 65535) return fail(CG_ERR_UNSUPPORTED, "matmul: more than 65535 batch entries after folding");
+    const bool f32 = x->dt == CG_F32;
+    hipStream_t s = be->stream;
+    if (K == 0 || !f32) {
+        uint64_t elems = (uint64_t)M * N;
+        dim3 grid((uint32_t)((elems + kThreads - 1) / kThreads), (uint32_t)batch);
+        if (f32)
+            hipLaunchKernelGGL((simple_gemm_kernel<true>), grid, dim3(kThreads), 0, s, a);
+        else
+            hipLaunchKernelGGL((simple_gemm_kernel<false>), grid, dim3(kThreads), 0, s, a);
+    } else if (M <= 8 && a.b_sk == 1) {
+        dim3 grid((uint32_t)((N + 3) / 4), (uint32_t)batch);
+        if (M <= 1)
+            hipLaunchKernelGGL((skinny_kt_kernel<1>), grid, dim3(kThreads), 0, s, a);
+        else if (M <= 4)
+            hipLaunchKernelGGL((skinny_kt_kernel<4>), grid, dim3(kThreads), 0, s, a);
+        else
+            hipLaunchKernelGGL((skinny_kt_kernel<8>), grid, dim3(kThreads), 0, s, a);
+    } else {
+        uint64_t tiles = (uint64_t)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+        if (tiles > 0x7FFFFFFFull) return fail(CG_ERR_UNSUPPORTED, "matmul: too many tiles");
+        dim3 grid((uint32_t)tiles, (uint32_t)batch);
+        if (a_mfast) {
+            if (b_nfast)
+                hipLaunchKernelGGL((mfma_gemm_kernel<true, true>), grid, dim3(kThreads), 0, s, a);
+            else
+                hipLaunchKernelGGL((mfma_gemm_kernel<true, false>), grid, dim3(kThreads), 0, s, a);
+        } else {
+            if (b_nfast)
+                hipLaunchKernelGGL((mfma_gemm_kernel<false, true>), grid, dim3(kThreads), 0, s, a);
+            else
+                hipLaunchKernelGGL((mfma_gemm_kernel<false, false>), grid, dim3(kThreads), 0, s, a);
+        }
+    }
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CG_OK : hip_fail(e, "matmul launch");
+}
+
+} // namespace cg

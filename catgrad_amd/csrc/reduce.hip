@@ -1,0 +1,342 @@
+// Last-axis reductions for gfx950: sum, max, argmax, top-k, and the host-visible
+// predicates behind to_bool / compare.
+//
+// Layout: a strided view is seen as rows x n; rows are addressed through the view's own
+// outer strides, the reduced axis through its stride, so transposed / sliced inputs are
+// reduced in place.  TPR lanes cooperate on one row (4, 16, 64 lanes of one wave, or the
+// 256 lanes of a block); each lane strides over the row with 16-byte loads when the row
+// is unit-stride and aligned; lanes combine with wave64 cross-lane shuffles and, for
+// TPR = 256, a 4-entry LDS exchange.  HBM-bound: 4 B read per element, 4 B written per row.
+//
+// Semantics follow NdArrayBackend (catgrad/src/interpreter/backend/ndarray.rs:656-730):
+//   max     folds from f32::MIN with NaN-ignoring max; u32 from 0
+//   argmax  `max_by(total_cmp)`: the LAST of equal maxima; +0 > -0; +NaN greatest
+//   topk    stable descending sort by total_cmp: ties in order of appearance
+//   sum     f32 in tree order (the reference's own order is sequential/8-way; both are
+//           within the 1e-3 relative contract), u32 wrapping
+#include "common.hpp"
+#include "device_utils.hpp"
+
+namespace cg {
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr float kF32Min = -3.4028234663852886e38f;
+
+struct RowsArgs {
+    const char *x;
+    uint32_t *out;
+    uint32_t rows, n;
+    int64_t sn;           // stride of the reduced axis (elements)
+    uint32_t nouter;
+    uint32_t od[kMaxOuter];
+    FastDiv odiv[kMaxOuter];
+    int64_t os[kMaxOuter];
+    uint32_t vec;         // 4: rows are unit-stride and 16-byte aligned
+};
+
+__device__ __forceinline__ int32_t total_key(uint32_t bits) { // Rust f32::total_cmp
+    int32_t b = (int32_t)bits;
+    return b ^ (int32_t)(((uint32_t)(b >> 31)) >> 1);
+}
+
+// Accumulator per reduction kind.  K: 0 sum, 1 max, 2 argmax.  F: f32 input.
+template <int K, bool F> struct Acc;
+
+template <> struct Acc<kSum, true> {
+    float v = 0.0f;
+    __device__ void take(uint32_t w, uint32_t) { v += asf(w); }
+    __device__ void merge(const Acc &o) { v += o.v; }
+    __device__ uint32_t result() const { return asu(v); }
+    __device__ Acc shfl(int m) const { Acc r; r.v = __shfl_xor(v, m); return r; }
+    __device__ long long pack() const { return (long long)asu(v); }
+    __device__ static Acc unpack(long long b) { Acc r; r.v = asf((uint32_t)b); return r; }
+};
+template <> struct Acc<kSum, false> {
+    uint32_t v = 0;
+    __device__ void take(uint32_t w, uint32_t) { v += w; }
+    __device__ void merge(const Acc &o) { v += o.v; }
+    __device__ uint32_t result() const { return v; }
+    __device__ Acc shfl(int m) const { Acc r; r.v = __shfl_xor(v, m); return r; }
+    __device__ long long pack() const { return (long long)v; }
+    __device__ static Acc unpack(long long b) { Acc r; r.v = (uint32_t)b; return r; }
+};
+template <> struct Acc<kMax, true> {
+    float v = kF32Min;
+    __device__ void take(uint32_t w, uint32_t) { v = fmaxf(v, asf(w)); } // NaN operand ignored
+    __device__ void merge(const Acc &o) { v = fmaxf(v, o.v); }
+    __device__ uint32_t result() const { return asu(v); }
+    __device__ Acc shfl(int m) const { Acc r; r.v = __shfl_xor(v, m); return r; }
+    __device__ long long pack() const { return (long long)asu(v); }
+    __device__ static Acc unpack(long long b) { Acc r; r.v = asf((uint32_t)b); return r; }
+};
+template <> struct Acc<kMax, false> {
+    uint32_t v = 0;
+    __device__ void take(uint32_t w, uint32_t) { v = w > v ? w : v; }
+    __device__ void merge(const Acc &o) { v = o.v > v ? o.v : v; }
+    __device__ uint32_t result() const { return v; }
+    __device__ Acc shfl(int m) const { Acc r; r.v = __shfl_xor(v, m); return r; }
+    __device__ long long pack() const { return (long long)v; }
+    __device__ static Acc unpack(long long b) { Acc r; r.v = (uint32_t)b; return r; }
+};
+// argmax: (order key, index) packed so that a signed 64-bit max picks the greatest key
+// and, among equal keys, the greatest index.
+template <bool F> struct Acc<kArgmax, F> {
+    long long c = (long long)0x8000000000000000ll;
+    __device__ void take(uint32_t w, uint32_t idx) {
+        int32_t key = F ? total_key(w) : (int32_t)(w ^ 0x80000000u);
+        long long p = ((long long)key << 32) | (long long)idx;
+        c = p > c ? p : c;
+    }
+    __device__ void merge(const Acc &o) { c = o.c > c ? o.c : c; }
+    __device__ uint32_t result() const { return (uint32_t)(c & 0xFFFFFFFFll); }
+    __device__ Acc shfl(int m) const {
+        Acc r;
+        int lo = __shfl_xor((int)(c & 0xFFFFFFFFll), m);
+        int hi = __shfl_xor((int)(c >> 32), m);
+        r.c = ((long long)hi << 32) | (long long)(uint32_t)lo;
+        return r;
+    }
+    __device__ long long pack() const { return c; }
+    __device__ static Acc unpack(long long b) { Acc r; r.c = b; return r; }
+};
+
+template <int K, bool F, int TPR> __global__ __launch_bounds__(kBlock) void reduce_rows_kernel(const RowsArgs a) {
+    constexpr int RPB = kBlock / TPR; // rows per block
+    const uint32_t lane = threadIdx.x % TPR;
+    const uint32_t row = blockIdx.x * RPB + threadIdx.x / TPR;
+    const bool live = row < a.rows;
+    Acc<K, F> acc;
+    if (live) {
+        const uint32_t *p = reinterpret_cast<const uint32_t *>(a.x) + row_offset(row, a.nouter, a.od, a.odiv, a.os);
+        if (a.vec == 4) {
+            const uint32_t nv = a.n / 4;
+            // two independent 16-byte loads in flight per lane per trip
+            uint32_t i = lane;
+            for (; i + TPR < nv; i += 2 * TPR) {
+                uint4 t0 = reinterpret_cast<const uint4 *>(p)[i];
+                uint4 t1 = reinterpret_cast<const uint4 *>(p)[i + TPR];
+                acc.take(t0.x, 4 * i);
+                acc.take(t0.y, 4 * i + 1);
+                acc.take(t0.z, 4 * i + 2);
+                acc.take(t0.w, 4 * i + 3);
+                acc.take(t1.x, 4 * (i + TPR));
+                acc.take(t1.y, 4 * (i + TPR) + 1);
+                acc.take(t1.z, 4 * (i + TPR) + 2);
+                acc.take(t1.w, 4 * (i + TPR) + 3);
+            }
+            if (i < nv) {
+                uint4 t0 = reinterpret_cast<const uint4 *>(p)[i];
+                acc.take(t0.x, 4 * i);
+                acc.take(t0.y, 4 * i + 1);
+                acc.take(t0.z, 4 * i + 2);
+                acc.take(t0.w, 4 * i + 3);
+            }
+        } else {
+            for (uint32_t i = lane; i < a.n; i += TPR) acc.take(p[(int64_t)i * a.sn], i);
+        }
+    }
+    constexpr int W = TPR < 64 ? TPR : 64;
+#pragma unroll
+    for (int m = W / 2; m >= 1; m >>= 1) acc.merge(acc.shfl(m));
+    if constexpr (TPR > 64) {
+        __shared__ long long part[kBlock / 64];
+        if (threadIdx.x % 64 == 0) part[threadIdx.x / 64] = acc.pack();
+        __syncthreads();
+        if (threadIdx.x == 0) {
+#pragma unroll
+            for (int w = 1; w < kBlock / 64; w++) acc.merge(Acc<K, F>::unpack(part[w]));
+        }
+    }
+    if (live && lane == 0) a.out[row] = acc.result();
+}
+
+// top-k by repeated selection: element e precedes f when key(e) > key(f), or the keys
+// are equal and e appears first.  One block per row; k passes over the row.
+__global__ __launch_bounds__(kBlock) void topk_kernel(const RowsArgs a, uint32_t k, uint32_t *idx_out) {
+    const uint32_t row = blockIdx.x;
+    const uint32_t *p = reinterpret_cast<const uint32_t *>(a.x) + row_offset(row, a.nouter, a.od, a.odiv, a.os);
+    __shared__ long long part[kBlock / 64];
+    __shared__ long long chosen;
+    long long prev = 0x7FFFFFFFFFFFFFFFll;
+    for (uint32_t j = 0; j < k; j++) {
+        long long best = (long long)0x8000000000000000ll;
+        for (uint32_t i = threadIdx.x; i < a.n; i += kBlock) {
+            uint32_t w = p[(int64_t)i * a.sn];
+            long long c = ((long long)total_key(w) << 32) | (long long)(0xFFFFFFFFu - i);
+            if (c < prev && c > best) best = c;
+        }
+#pragma unroll
+        for (int m = 32; m >= 1; m >>= 1) {
+            int lo = __shfl_xor((int)(best & 0xFFFFFFFFll), m);
+            int hi = __shfl_xor((int)(best >> 32), m);
+            long long o = ((long long)hi << 32) | (long long)(uint32_t)lo;
+            best = o > best ? o : best;
+        }
+        if (threadIdx.x % 64 == 0) part[threadIdx.x / 64] = best;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            for (int w = 1; w < kBlock / 64; w++) best = part[w] > best ? part[w] : best;
+            uint32_t i = 0xFFFFFFFFu - (uint32_t)(best & 0xFFFFFFFFll);
+            a.out[(uint64_t)row * k + j] = p[(int64_t)i * a.sn];
+            idx_out[(uint64_t)row * k + j] = i;
+            chosen = best;
+        }
+        __syncthreads();
+        prev = chosen;
+        __syncthreads();
+    }
+}
+
+struct AnyArgs {
+    EwGeom g;
+    Operand x, y;
+    uint32_t *flag;
+};
+
+// MODE 0: any(x > 0) (f32) / any(x != 0) (u32).  MODE 1: any(x != y) with IEEE
+// inequality for f32 (NaN differs from everything, -0 equals +0).
+template <int MODE, bool F, int VEC> __global__ __launch_bounds__(kBlock) void any_kernel(const AnyArgs a) {
+    uint64_t v64 = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (v64 >= a.g.total) return;
+    uint32_t v = (uint32_t)v64;
+    uint32_t row = fastdiv(v, a.g.ipr_div);
+    int64_t e = (int64_t)(v - row * a.g.ipr) * VEC;
+    int64_t ox = e * a.x.is, oy = e * a.y.is;
+    for (uint32_t d = 0; d < a.g.nouter; d++) {
+        uint32_t q = fastdiv(row, a.g.odiv[d]);
+        int64_t i = (int64_t)(row - q * a.g.od[d]);
+        row = q;
+        ox += i * a.x.os[d];
+        oy += i * a.y.os[d];
+    }
+    uint32_t xs[VEC], ys[VEC];
+    load_words<VEC>(a.x, ox, xs);
+    if (MODE == 1) load_words<VEC>(a.y, oy, ys);
+    bool hit = false;
+#pragma unroll
+    for (int j = 0; j < VEC; j++) {
+        if (MODE == 0)
+            hit |= F ? asf(xs[j]) > 0.0f : xs[j] != 0u;
+        else
+            hit |= F ? !(asf(xs[j]) == asf(ys[j])) : xs[j] != ys[j];
+    }
+    if (hit) *a.flag = 1u;
+}
+
+int fill_rows_args(const cg_tensor *x, RowsArgs *a) {
+    memset(a, 0, sizeof *a);
+    const void *p;
+    int rc = device_ptr(x, &p);
+    if (rc) return rc;
+    a->x = static_cast<const char *>(p);
+    int r = x->rank;
+    int64_t n = x->dims[r - 1];
+    a->sn = x->uniform ? 0 : x->strides[r - 1];
+    // collapse the outer axes of this one view
+    int64_t dims[kMaxRank], st[kMaxRank];
+    int w = 0;
+    for (int i = 0; i < r - 1; i++) {
+        if (x->dims[i] == 1) continue;
+        int64_t s = x->uniform ? 0 : x->strides[i];
+        if (w > 0 && st[w - 1] == s * x->dims[i]) {
+            dims[w - 1] *= x->dims[i];
+            st[w - 1] = s;
+        } else {
+            dims[w] = x->dims[i];
+            st[w] = s;
+            w++;
+        }
+    }
+    int64_t rows = 1;
+    for (int i = 0; i < w; i++) rows *= dims[i];
+    if (rows > 0xFFFFFFFFll || n > 0x3FFFFFFFll) return fail(CG_ERR_UNSUPPORTED, "reduction extents above 2^32-1");
+    a->rows = (uint32_t)rows;
+    a->n = (uint32_t)n;
+    a->nouter = (uint32_t)w;
+    bool vec = !x->uniform && a->sn == 1 && n % 4 == 0 && reinterpret_cast<uintptr_t>(p) % 16 == 0;
+    for (int d = 0; d < w; d++) {
+        a->od[d] = (uint32_t)dims[w - 1 - d];
+        a->odiv[d] = make_fastdiv(a->od[d]);
+        a->os[d] = st[w - 1 - d];
+        if (a->os[d] % 4) vec = false;
+    }
+    a->vec = vec ? 4 : 1;
+    return CG_OK;
+}
+
+template <int K, bool F> int launch_rows(cg_backend *be, const RowsArgs &a) {
+    // lanes per row: enough that a lane sees about eight elements, within {4,16,64,256}
+    uint32_t want = (a.n + 7) / 8;
+    int tpr = want <= 4 ? 4 : want <= 16 ? 16 : want <= 64 ? 64 : 256;
+    uint32_t rpb = kBlock / tpr;
+    dim3 grid((a.rows + rpb - 1) / rpb), block(kBlock);
+    switch (tpr) {
+    case 4: hipLaunchKernelGGL((reduce_rows_kernel<K, F, 4>), grid, block, 0, be->stream, a); break;
+    case 16: hipLaunchKernelGGL((reduce_rows_kernel<K, F, 16>), grid, block, 0, be->stream, a); break;
+    case 64: hipLaunchKernelGGL((reduce_rows_kernel<K, F, 64>), grid, block, 0, be->stream, a); break;
+    default: hipLaunchKernelGGL((reduce_rows_kernel<K, F, 256>), grid, block, 0, be->stream, a); break;
+    }
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CG_OK : hip_fail(e, "reduction launch");
+}
+
+} // namespace
+
+int launch_reduce(cg_backend *be, int kind, const cg_tensor *x, cg_tensor *out) {
+    RowsArgs a;
+    int rc = fill_rows_args(x, &a);
+    if (rc) return rc;
+    a.out = static_cast<uint32_t *>(out->buf->ptr);
+    bool f = x->dt == CG_F32;
+    switch (kind) {
+    case kSum: return f ? launch_rows<kSum, true>(be, a) : launch_rows<kSum, false>(be, a);
+    case kMax: return f ? launch_rows<kMax, true>(be, a) : launch_rows<kMax, false>(be, a);
+    case kArgmax: return f ? launch_rows<kArgmax, true>(be, a) : launch_rows<kArgmax, false>(be, a);
+    default: return fail(CG_ERR_ARG, "unknown reduction %d", kind);
+    }
+}
+
+int launch_topk(cg_backend *be, const cg_tensor *x, int64_t k, cg_tensor *vals, cg_tensor *idxs) {
+    RowsArgs a;
+    int rc = fill_rows_args(x, &a);
+    if (rc) return rc;
+    a.out = static_cast<uint32_t *>(vals->buf->ptr);
+    hipLaunchKernelGGL(topk_kernel, dim3(a.rows), dim3(kBlock), 0, be->stream, a, (uint32_t)k,
+                       static_cast<uint32_t *>(idxs->buf->ptr));
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CG_OK : hip_fail(e, "topk launch");
+}
+
+static int launch_any(cg_backend *be, int mode, const cg_tensor *x, const cg_tensor *y) {
+    int rc = launch_fill_word(be, be->flag_dev, 0);
+    if (rc) return rc;
+    const cg_tensor *views[2] = {x, y ? y : x};
+    AnyArgs a;
+    memset(&a, 0, sizeof a);
+    Operand ops[2];
+    rc = plan_elementwise(views, 2, &a.g, ops);
+    if (rc) return rc;
+    a.x = ops[0];
+    a.y = ops[1];
+    a.flag = be->flag_dev;
+    dim3 grid((uint32_t)((a.g.total + kBlock - 1) / kBlock)), block(kBlock);
+    bool f = x->dt == CG_F32;
+#define CG_ANY(MODE, F, VEC) hipLaunchKernelGGL((any_kernel<MODE, F, VEC>), grid, block, 0, be->stream, a)
+    if (mode == 0) {
+        if (a.g.vec == 4) { if (f) CG_ANY(0, true, 4); else CG_ANY(0, false, 4); }
+        else { if (f) CG_ANY(0, true, 1); else CG_ANY(0, false, 1); }
+    } else {
+        if (a.g.vec == 4) { if (f) CG_ANY(1, true, 4); else CG_ANY(1, false, 4); }
+        else { if (f) CG_ANY(1, true, 1); else CG_ANY(1, false, 1); }
+    }
+#undef CG_ANY
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CG_OK : hip_fail(e, "predicate launch");
+}
+
+int launch_any_positive(cg_backend *be, const cg_tensor *x) { return launch_any(be, 0, x, nullptr); }
+int launch_any_diff(cg_backend *be, const cg_tensor *x, const cg_tensor *y) { return launch_any(be, 1, x, y); }
+
+} // namespace cg

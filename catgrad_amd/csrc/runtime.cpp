@@ -1,0 +1,1083 @@
+// Host runtime of libcatgrad_hip.so: backend lifetime, device pool, tensor handles,
+// zero-copy view algebra, argument checking and the C ABI entry points.  Arithmetic
+// lives in the kernel files (ew.hip, reduce.hip, matmul.hip).
+//
+// The semantics implemented here follow catgrad's NdArrayBackend
+// (reference: catgrad/src/interpreter/backend/ndarray.rs); each entry point cites the
+// lines it replaces.  Unlike that backend, transpose / slice / broadcast / reshape are
+// views whenever strides allow, constants never touch device memory, and nothing
+// copies a shared buffer before using it.
+#include "common.hpp"
+
+#include <algorithm>
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <vector>
+
+namespace cg {
+
+static thread_local std::string g_err;
+static std::mutex g_lazy_mu; // guards lazy backing of uniform tensors
+
+int fail(int code, const char *fmt, ...) {
+    char buf[512];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    g_err = buf;
+    return code;
+}
+
+int hip_fail(hipError_t e, const char *what) {
+    return fail(CG_ERR_DEVICE, "HIP error %d (%s) in %s", (int)e, hipGetErrorString(e), what);
+}
+
+// ---- pool -------------------------------------------------------------------------
+size_t Pool::size_class(size_t bytes) {
+    // 512 B minimum, then eight classes per octave: at most 12.5 % slack and few enough
+    // distinct sizes that the growing shapes of a decode loop keep hitting the lists.
+    if (bytes <= 512) return 512;
+    int e = 63 - __builtin_clzll(bytes);
+    size_t step = (size_t)1 << (e - 3);
+    return (bytes + step - 1) & ~(step - 1);
+}
+
+int Pool::alloc(size_t bytes, void **ptr, size_t *cls) {
+    size_t c = size_class(bytes);
+    {
+        std::lock_guard<std::mutex> lk(mu_);
+        auto it = free_.lower_bound(c);
+        if (it != free_.end() && it->first <= c + c / 4) {
+            *ptr = it->second;
+            *cls = it->first;
+            cached_ -= it->first;
+            in_use_ += it->first;
+            free_.erase(it);
+            return CG_OK;
+        }
+    }
+    void *p = nullptr;
+    hipError_t e = hipMalloc(&p, c);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        trim();
+        e = hipMalloc(&p, c);
+        if (e != hipSuccess) return hip_fail(e, "hipMalloc");
+    }
+    std::lock_guard<std::mutex> lk(mu_);
+    in_use_ += c;
+    *ptr = p;
+    *cls = c;
+    return CG_OK;
+}
+
+void Pool::free(void *ptr, size_t cls) {
+    std::lock_guard<std::mutex> lk(mu_);
+    free_.emplace(cls, ptr);
+    in_use_ -= cls;
+    cached_ += cls;
+}
+
+void Pool::trim() {
+    std::multimap<size_t, void *> take;
+    {
+        std::lock_guard<std::mutex> lk(mu_);
+        take.swap(free_);
+        cached_ = 0;
+    }
+    for (auto &kv : take) (void)hipFree(kv.second);
+}
+
+void Pool::stats(size_t *in_use, size_t *cached) {
+    std::lock_guard<std::mutex> lk(mu_);
+    if (in_use) *in_use = in_use_;
+    if (cached) *cached = cached_;
+}
+
+// ---- tensors ----------------------------------------------------------------------
+bool is_contiguous(const cg_tensor *t) {
+    if (numel(t) == 0) return true;
+    int64_t s = 1;
+    for (int i = t->rank - 1; i >= 0; i--) {
+        if (t->dims[i] != 1 && t->strides[i] != s) return false;
+        s *= t->dims[i];
+    }
+    return true;
+}
+
+static void buffer_release(Buffer *b) {
+    if (b && b->rc.fetch_sub(1) == 1) {
+        if (b->ptr) b->be->pool.free(b->ptr, b->cls);
+        delete b;
+    }
+}
+
+void release(cg_tensor *t) {
+    if (!t) return;
+    if (t->rc.fetch_sub(1) == 1) {
+        buffer_release(t->buf);
+        delete t;
+    }
+}
+
+static void set_row_major(cg_tensor *t) {
+    int64_t s = 1;
+    for (int i = t->rank - 1; i >= 0; i--) {
+        t->strides[i] = s;
+        s *= t->dims[i];
+    }
+}
+
+int new_dense(cg_backend *be, cg_dtype dt, const int64_t *dims, int rank, cg_tensor **out) {
+    cg_tensor *t = new cg_tensor;
+    t->be = be;
+    t->dt = dt;
+    t->rank = rank;
+    for (int i = 0; i < rank; i++) t->dims[i] = dims[i];
+    set_row_major(t);
+    int64_t n = numel(t);
+    if (n > 0) {
+        Buffer *b = new Buffer;
+        b->be = be;
+        int rc = be->pool.alloc((size_t)n * 4, &b->ptr, &b->cls);
+        if (rc) {
+            delete b;
+            delete t;
+            return rc;
+        }
+        t->buf = b;
+    }
+    *out = t;
+    return CG_OK;
+}
+
+cg_tensor *new_uniform(cg_backend *be, cg_dtype dt, const int64_t *dims, int rank, uint32_t bits) {
+    cg_tensor *t = new cg_tensor;
+    t->be = be;
+    t->dt = dt;
+    t->rank = rank;
+    for (int i = 0; i < rank; i++) {
+        t->dims[i] = dims[i];
+        t->strides[i] = 0;
+    }
+    t->uniform = true;
+    t->ubits = bits;
+    return t;
+}
+
+cg_tensor *new_view(const cg_tensor *t) {
+    cg_tensor *v = new cg_tensor;
+    v->be = t->be;
+    v->buf = t->buf;
+    if (v->buf) v->buf->rc.fetch_add(1);
+    v->dt = t->dt;
+    v->rank = t->rank;
+    memcpy(v->dims, t->dims, sizeof v->dims);
+    memcpy(v->strides, t->strides, sizeof v->strides);
+    v->offset = t->offset;
+    v->uniform = t->uniform;
+    v->ubits = t->ubits;
+    return v;
+}
+
+int device_ptr(const cg_tensor *t, const void **ptr) {
+    if (!t->buf) {
+        if (!t->uniform || numel(t) == 0) {
+            *ptr = nullptr;
+            return CG_OK;
+        }
+        std::lock_guard<std::mutex> lk(g_lazy_mu);
+        if (!t->buf) {
+            Buffer *b = new Buffer;
+            b->be = t->be;
+            int rc = t->be->pool.alloc(4, &b->ptr, &b->cls);
+            if (rc) {
+                delete b;
+                return rc;
+            }
+            rc = launch_fill_word(t->be, b->ptr, t->ubits);
+            if (rc) {
+                buffer_release(b);
+                return rc;
+            }
+            const_cast<cg_tensor *>(t)->buf = b;
+        }
+    }
+    *ptr = static_cast<const char *>(t->buf->ptr) + t->offset * 4;
+    return CG_OK;
+}
+
+FastDiv make_fastdiv(uint32_t d) {
+    FastDiv f;
+    f.d = d;
+    uint32_t l = 0;
+    while (l < 32 && ((uint64_t)1 << l) < d) l++;
+    f.m = (uint32_t)((((uint64_t)1 << 32) * (((uint64_t)1 << l) - d)) / d + 1);
+    f.s1 = l < 1 ? l : 1;
+    f.s2 = l > 0 ? l - 1 : 0;
+    return f;
+}
+
+int plan_elementwise(const cg_tensor *const *views, int n, EwGeom *g, Operand *ops) {
+    const cg_tensor *out = views[0];
+    int r = 0;
+    int64_t dims[kMaxRank];
+    int64_t st[4][kMaxRank];
+    for (int i = 0; i < out->rank; i++) {
+        if (out->dims[i] == 1) continue;
+        dims[r] = out->dims[i];
+        for (int k = 0; k < n; k++) st[k][r] = views[k]->uniform ? 0 : views[k]->strides[i];
+        r++;
+    }
+    // merge axis i+1 into axis i when every operand steps through them as one run
+    int w = 0;
+    for (int i = 0; i < r; i++) {
+        if (w > 0) {
+            bool ok = true;
+            for (int k = 0; k < n && ok; k++) ok = st[k][w - 1] == st[k][i] * dims[i];
+            if (ok) {
+                dims[w - 1] *= dims[i];
+                for (int k = 0; k < n; k++) st[k][w - 1] = st[k][i];
+                continue;
+            }
+        }
+        dims[w] = dims[i];
+        for (int k = 0; k < n; k++) st[k][w] = st[k][i];
+        w++;
+    }
+    r = w;
+    if (r == 0) {
+        r = 1;
+        dims[0] = 1;
+        for (int k = 0; k < n; k++) st[k][0] = 1;
+    }
+    for (int i = 0; i < r; i++)
+        if (dims[i] > 0xFFFFFFFFll) return fail(CG_ERR_UNSUPPORTED, "axis extent above 2^32-1 elements");
+    int64_t inner = dims[r - 1];
+    bool vec4 = inner % 4 == 0;
+    for (int k = 0; k < n; k++) {
+        Operand &o = ops[k];
+        memset(&o, 0, sizeof o);
+        o.uniform = views[k]->uniform ? 1u : 0u;
+        o.ubits = views[k]->ubits;
+        if (!o.uniform) {
+            const void *p;
+            int rc = device_ptr(views[k], &p);
+            if (rc) return rc;
+            o.ptr = static_cast<const char *>(p);
+        }
+        o.is = st[k][r - 1];
+        for (int d = 0; d < r - 1; d++) o.os[d] = st[k][r - 2 - d];
+        if (!o.uniform && o.is == 1) {
+            if (reinterpret_cast<uintptr_t>(o.ptr) % 16) vec4 = false;
+            for (int d = 0; d < r - 1; d++)
+                if (o.os[d] % 4) vec4 = false;
+        }
+    }
+    g->nouter = (uint32_t)(r - 1);
+    g->inner = (uint32_t)inner;
+    g->vec = vec4 ? 4 : 1;
+    g->ipr = (uint32_t)(inner / g->vec);
+    g->ipr_div = make_fastdiv(g->ipr ? g->ipr : 1);
+    uint64_t total = g->ipr;
+    for (int d = 0; d < r - 1; d++) {
+        g->od[d] = (uint32_t)dims[r - 2 - d];
+        g->odiv[d] = make_fastdiv(g->od[d]);
+        total *= g->od[d];
+    }
+    if (total > 0xFFFFFFFFull) return fail(CG_ERR_UNSUPPORTED, "element-wise launch above 2^32-1 work items");
+    g->total = total;
+    return CG_OK;
+}
+
+// ---- helpers for the entry points -------------------------------------------------------
+struct Consume { // the consumed reference of a tensor argument (move semantics of the ABI)
+    cg_tensor *t;
+    explicit Consume(cg_tensor *t) : t(t) {}
+    ~Consume() { release(t); }
+};
+
+static const char *kTodo = "f16, bf16, and fp8 are not supported (todo!() in the reference NdArrayBackend)";
+static bool supported(cg_dtype d) { return d == CG_F32 || d == CG_U32; }
+
+static bool same_shape(const cg_tensor *a, const cg_tensor *b) {
+    if (a->rank != b->rank) return false;
+    for (int i = 0; i < a->rank; i++)
+        if (a->dims[i] != b->dims[i]) return false;
+    return true;
+}
+
+static int wait_and_check(cg_backend *be) {
+    CG_HIP(hipStreamSynchronize(be->stream));
+    uint32_t f = *reinterpret_cast<volatile uint32_t *>(be->fault_host);
+    if (f) {
+        *reinterpret_cast<volatile uint32_t *>(be->fault_host) = 0;
+        if (f & kFaultIndexRange) return fail(CG_ERR_RANGE, "index: index out of bounds (detected on device)");
+        if (f & kFaultDivZero) return fail(CG_ERR_RANGE, "attempt to divide by zero (detected on device)");
+    }
+    return CG_OK;
+}
+
+// Row-major copy of a view (the materialising half of reshape / to_vec).
+static int materialize(cg_backend *be, const cg_tensor *x, cg_tensor **out) {
+    cg_tensor *o;
+    int rc = new_dense(be, x->dt, x->dims, x->rank, &o);
+    if (rc) return rc;
+    if (numel(x) > 0) {
+        const cg_tensor *ins[1] = {x};
+        rc = launch_elementwise(be, kCopy, x->dt, o, ins, 1);
+        if (rc) {
+            release(o);
+            return rc;
+        }
+    }
+    *out = o;
+    return CG_OK;
+}
+
+// numpy-style "reshape without copying": new strides for `dims` if the view allows it.
+static bool try_view_reshape(const cg_tensor *x, const int64_t *dims, int rank, int64_t *strides) {
+    int64_t od[kMaxRank], os[kMaxRank];
+    int on = 0;
+    for (int i = 0; i < x->rank; i++)
+        if (x->dims[i] != 1) {
+            od[on] = x->dims[i];
+            os[on] = x->strides[i];
+            on++;
+        }
+    int oi = 0, ni = 0;
+    while (ni < rank && oi < on) {
+        int64_t np = dims[ni], op = od[oi];
+        int oj = oi + 1, nj = ni + 1;
+        while (np != op) {
+            if (np < op) {
+                if (nj >= rank) return false;
+                np *= dims[nj++];
+            } else {
+                if (oj >= on) return false;
+                op *= od[oj++];
+            }
+        }
+        for (int k = oi; k < oj - 1; k++)
+            if (os[k] != os[k + 1] * od[k + 1]) return false;
+        int64_t s = os[oj - 1];
+        for (int k = nj - 1; k >= ni; k--) {
+            strides[k] = s;
+            s *= dims[k];
+        }
+        oi = oj;
+        ni = nj;
+    }
+    if (oi < on) return false;
+    for (; ni < rank; ni++) {
+        if (dims[ni] != 1) return false;
+        strides[ni] = 0;
+    }
+    return true;
+}
+
+static uint32_t f32_as_u32_host(float v) { // Rust `as`: saturating, NaN -> 0
+    if (!(v == v) || v <= 0.0f) return 0;
+    if (v >= 4294967296.0f) return 0xFFFFFFFFu;
+    return (uint32_t)v;
+}
+static float bits_f(uint32_t b) {
+    float f;
+    memcpy(&f, &b, 4);
+    return f;
+}
+static uint32_t f_bits(float f) {
+    uint32_t b;
+    memcpy(&b, &f, 4);
+    return b;
+}
+
+// Exactly-rounded scalar ops are folded on the host when every operand is uniform
+// (IEEE add/sub/mul/div and comparisons give the same bits on host and device).
+static bool fold_binary(int op, cg_dtype dt, uint32_t a, uint32_t b, uint32_t *r, bool *divzero) {
+    if (dt == CG_F32) {
+        float x = bits_f(a), y = bits_f(b);
+        switch (op) {
+        case CG_ADD: *r = f_bits(x + y); return true;
+        case CG_SUB: *r = f_bits(x - y); return true;
+        case CG_MUL: *r = f_bits(x * y); return true;
+        case CG_DIV: *r = f_bits(x / y); return true;
+        case CG_LT: *r = f_bits(x < y ? 1.0f : 0.0f); return true;
+        case CG_GT: *r = f_bits(x > y ? 1.0f : 0.0f); return true;
+        case CG_GTE: *r = f_bits(x >= y ? 1.0f : 0.0f); return true;
+        case CG_LTE: *r = f_bits(x <= y ? 1.0f : 0.0f); return true;
+        case CG_EQ: *r = f_bits(x == y ? 1.0f : 0.0f); return true;
+        default: return false; // pow goes to the device so that one libm serves all elements
+        }
+    }
+    switch (op) {
+    case CG_ADD: *r = a + b; return true;
+    case CG_SUB: *r = a - b; return true;
+    case CG_MUL: *r = a * b; return true;
+    case CG_DIV:
+        if (b == 0) {
+            *divzero = true;
+            return true;
+        }
+        *r = a / b;
+        return true;
+    case CG_POW: {
+        uint32_t acc = 1, base = a, e = b;
+        while (e) {
+            if (e & 1) acc *= base;
+            base *= base;
+            e >>= 1;
+        }
+        *r = acc;
+        return true;
+    }
+    case CG_LT: *r = a < b; return true;
+    case CG_GT: *r = a > b; return true;
+    case CG_GTE: *r = a >= b; return true;
+    case CG_LTE: *r = a <= b; return true;
+    case CG_EQ: *r = a == b; return true;
+    default: return false;
+    }
+}
+
+} // namespace cg
+
+using namespace cg;
+
+extern "C" {
+
+// ---- backend lifetime ----------------------------------------------------------------
+int cg_backend_create(int device, cg_backend **out) {
+    if (!out) return fail(CG_ERR_ARG, "null out");
+    int count = 0;
+    hipError_t e = hipGetDeviceCount(&count);
+    if (e != hipSuccess || count <= 0) {
+        (void)hipGetLastError();
+        return fail(CG_ERR_DEVICE, "no HIP device available (hipGetDeviceCount: %s); HipBackend has no CPU fallback",
+                    hipGetErrorString(e));
+    }
+    if (device < 0 || device >= count) return fail(CG_ERR_ARG, "device %d out of range (%d devices)", device, count);
+    CG_HIP(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    CG_HIP(hipGetDeviceProperties(&prop, device));
+    cg_backend *b = new cg_backend;
+    b->device = device;
+    CG_HIP(hipStreamCreateWithFlags(&b->stream, hipStreamNonBlocking));
+    CG_HIP(hipHostMalloc((void **)&b->fault_host, 64, hipHostMallocMapped));
+    memset(b->fault_host, 0, 64);
+    CG_HIP(hipHostGetDevicePointer((void **)&b->fault_dev, b->fault_host, 0));
+    CG_HIP(hipHostMalloc((void **)&b->flag_host, 64, hipHostMallocDefault));
+    CG_HIP(hipMalloc((void **)&b->flag_dev, 64));
+    char name[256];
+    snprintf(name, sizeof name, "hip:%s (%s, %d CUs)", prop.gcnArchName, prop.name, prop.multiProcessorCount);
+    b->name = name;
+    *out = b;
+    return CG_OK;
+}
+
+void cg_backend_destroy(cg_backend *b) {
+    if (!b) return;
+    (void)hipSetDevice(b->device);
+    (void)hipStreamSynchronize(b->stream);
+    b->pool.trim();
+    (void)hipFree(b->flag_dev);
+    (void)hipHostFree(b->flag_host);
+    (void)hipHostFree(b->fault_host);
+    (void)hipStreamDestroy(b->stream);
+    delete b;
+}
+
+const char *cg_last_error(void) { return g_err.c_str(); }
+const char *cg_backend_name(cg_backend *b) { return b ? b->name.c_str() : ""; }
+
+int cg_sync(cg_backend *b) {
+    if (!b) return fail(CG_ERR_ARG, "null backend");
+    return wait_and_check(b);
+}
+
+int cg_pool_stats(cg_backend *b, size_t *bytes_in_use, size_t *bytes_cached) {
+    if (!b) return fail(CG_ERR_ARG, "null backend");
+    b->pool.stats(bytes_in_use, bytes_cached);
+    return CG_OK;
+}
+
+int cg_pool_trim(cg_backend *b) {
+    if (!b) return fail(CG_ERR_ARG, "null backend");
+    CG_HIP(hipStreamSynchronize(b->stream));
+    b->pool.trim();
+    return CG_OK;
+}
+
+// ---- handles -------------------------------------------------------------------------
+void cg_tensor_retain(cg_tensor *t) {
+    if (t) retain(t);
+}
+void cg_tensor_release(cg_tensor *t) { release(t); }
+size_t cg_tensor_rank(const cg_tensor *t) { return (size_t)t->rank; }
+void cg_tensor_shape(const cg_tensor *t, size_t *dims) {
+    for (int i = 0; i < t->rank; i++) dims[i] = (size_t)t->dims[i];
+}
+cg_dtype cg_tensor_dtype(const cg_tensor *t) { return t->dt; }
+size_t cg_tensor_numel(const cg_tensor *t) { return (size_t)numel(t); }
+int cg_tensor_is_contiguous(const cg_tensor *t) { return (t->uniform && numel(t) > 1) ? 0 : (is_contiguous(t) ? 1 : 0); }
+
+// ---- creation --------------------------------------------------------------------------
+static int check_dims(const size_t *dims, size_t rank, int64_t *d64) {
+    if (rank > CG_MAX_RANK) return fail(CG_ERR_ARG, "rank %zu above CG_MAX_RANK", rank);
+    if (rank && !dims) return fail(CG_ERR_ARG, "null dims");
+    for (size_t i = 0; i < rank; i++) d64[i] = (int64_t)dims[i];
+    return CG_OK;
+}
+
+// ndarray.rs:71-84 — a zero tensor is a uniform constant: no memory, no memset.
+int cg_zeros(cg_backend *b, cg_dtype dtype, const size_t *dims, size_t rank, cg_tensor **out) {
+    if (!b || !out) return fail(CG_ERR_ARG, "null argument");
+    if (!supported(dtype)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
+    int64_t d[kMaxRank];
+    int rc = check_dims(dims, rank, d);
+    if (rc) return rc;
+    *out = new_uniform(b, dtype, d, (int)rank, 0);
+    return CG_OK;
+}
+
+// ndarray.rs:86-96,122-132 and interpreter/mod.rs:28-30.  One-element tensors (the
+// `Scalar` / `NatToU32` constants of tensor_op.rs:64-87) stay on the host as uniforms.
+int cg_from_host(cg_backend *b, cg_dtype dtype, const void *data, size_t len, const size_t *dims, size_t rank,
+                 cg_tensor **out) {
+    if (!b || !out) return fail(CG_ERR_ARG, "null argument");
+    if (!supported(dtype)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
+    int64_t d[kMaxRank];
+    int rc = check_dims(dims, rank, d);
+    if (rc) return rc;
+    size_t n = 1;
+    for (size_t i = 0; i < rank; i++) n *= dims[i];
+    if (n != len) return fail(CG_ERR_SHAPE, "ShapeError");
+    if (n && !data) return fail(CG_ERR_ARG, "null data");
+    if (n == 1) {
+        uint32_t bits;
+        memcpy(&bits, data, 4);
+        *out = new_uniform(b, dtype, d, (int)rank, bits);
+        return CG_OK;
+    }
+    cg_tensor *t;
+    rc = new_dense(b, dtype, d, (int)rank, &t);
+    if (rc) return rc;
+    if (n) {
+        CG_HIP(hipSetDevice(b->device));
+        hipError_t e = hipMemcpyAsync(t->buf->ptr, data, n * 4, hipMemcpyHostToDevice, b->stream);
+        if (e == hipSuccess) e = hipStreamSynchronize(b->stream); // caller may free `data` on return
+        if (e != hipSuccess) {
+            release(t);
+            return hip_fail(e, "host to device copy");
+        }
+    }
+    *out = t;
+    return CG_OK;
+}
+
+// ndarray.rs:134-138.  The reference builds the range in f32 and casts; for
+// end <= 2^24 that is the integer iota produced here.  Larger ends are rejected
+// rather than reproducing the reference's rounding artefacts.
+int cg_arange(cg_backend *b, size_t end, cg_tensor **out) {
+    if (!b || !out) return fail(CG_ERR_ARG, "null argument");
+    if (end > (1u << 24)) return fail(CG_ERR_UNSUPPORTED, "arange: end above 2^24 is inexact in the reference");
+    int64_t d[1] = {(int64_t)end};
+    cg_tensor *t;
+    int rc = new_dense(b, CG_U32, d, 1, &t);
+    if (rc) return rc;
+    if (end) {
+        rc = launch_arange(b, t);
+        if (rc) {
+            release(t);
+            return rc;
+        }
+    }
+    *out = t;
+    return CG_OK;
+}
+
+// ---- read-back -----------------------------------------------------------------------------
+static int copy_out(cg_backend *b, const cg_tensor *t, void *dst, size_t len) {
+    if (len == 0) return wait_and_check(b);
+    if (t->uniform) {
+        uint32_t *d = static_cast<uint32_t *>(dst);
+        for (size_t i = 0; i < len; i++) d[i] = t->ubits;
+        return wait_and_check(b);
+    }
+    cg_tensor *tmp = nullptr;
+    const cg_tensor *src = t;
+    if (!is_contiguous(t)) {
+        int rc = materialize(b, t, &tmp);
+        if (rc) return rc;
+        src = tmp;
+    }
+    const void *p;
+    int rc = device_ptr(src, &p);
+    if (!rc) {
+        hipError_t e = hipMemcpyAsync(dst, p, len * 4, hipMemcpyDeviceToHost, b->stream);
+        rc = e == hipSuccess ? wait_and_check(b) : hip_fail(e, "device to host copy");
+    }
+    release(tmp);
+    return rc;
+}
+
+// ndarray.rs:50-58.  Non-contiguous views are materialised first (the reference panics).
+int cg_to_host(cg_backend *b, const cg_tensor *t, void *dst, size_t len) {
+    if (!b || !t || (!dst && len)) return fail(CG_ERR_ARG, "null argument");
+    if ((int64_t)len != numel(t)) return fail(CG_ERR_SHAPE, "to_vec: length mismatch");
+    CG_HIP(hipSetDevice(b->device));
+    return copy_out(b, t, dst, len);
+}
+
+static int read_flag(cg_backend *b, int *out) {
+    CG_HIP(hipMemcpyAsync(b->flag_host, b->flag_dev, 4, hipMemcpyDeviceToHost, b->stream));
+    int rc = wait_and_check(b);
+    if (rc) return rc;
+    *out = *b->flag_host != 0;
+    return CG_OK;
+}
+
+// ndarray.rs:140-149
+int cg_to_bool(cg_backend *b, const cg_tensor *t, int *out) {
+    if (!b || !t || !out) return fail(CG_ERR_ARG, "null argument");
+    if (!supported(t->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
+    CG_HIP(hipSetDevice(b->device));
+    if (numel(t) == 0) {
+        *out = 0;
+        return wait_and_check(b);
+    }
+    if (t->uniform) {
+        *out = t->dt == CG_F32 ? bits_f(t->ubits) > 0.0f : t->ubits != 0;
+        return wait_and_check(b);
+    }
+    int rc = launch_any_positive(b, t);
+    if (rc) return rc;
+    return read_flag(b, out);
+}
+
+// ndarray.rs:534-541
+int cg_compare(cg_backend *b, const cg_tensor *x, const cg_tensor *y, int *out) {
+    if (!b || !x || !y || !out) return fail(CG_ERR_ARG, "null argument");
+    if (!supported(x->dt) || !supported(y->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
+    if (x->dt != y->dt) return fail(CG_ERR_DTYPE, "compare: dtype mismatch");
+    CG_HIP(hipSetDevice(b->device));
+    if (!same_shape(x, y)) {
+        *out = 0;
+        return wait_and_check(b);
+    }
+    if (numel(x) == 0) {
+        *out = 1;
+        return wait_and_check(b);
+    }
+    int rc = launch_any_diff(b, x, y);
+    if (rc) return rc;
+    int diff = 0;
+    rc = read_flag(b, &diff);
+    *out = !diff;
+    return rc;
+}
+
+// ndarray.rs:60-69 — free-form debug rendering: dtype, shape and the first 16 elements.
+int cg_format_tensor(cg_backend *b, const cg_tensor *t, char *buf, size_t cap) {
+    if (!b || !t || !buf || !cap) return fail(CG_ERR_ARG, "null argument");
+    CG_HIP(hipSetDevice(b->device));
+    size_t n = (size_t)numel(t);
+    std::vector<uint32_t> host(n);
+    int rc = copy_out(b, t, host.data(), n);
+    if (rc) return rc;
+    std::string s = t->dt == CG_F32 ? "f32[" : "u32[";
+    for (int i = 0; i < t->rank; i++) s += (i ? "," : "") + std::to_string(t->dims[i]);
+    s += "] [";
+    size_t shown = std::min<size_t>(n, 16);
+    char tmp[48];
+    for (size_t i = 0; i < shown; i++) {
+        if (t->dt == CG_F32)
+            snprintf(tmp, sizeof tmp, "%s%.9g", i ? ", " : "", bits_f(host[i]));
+        else
+            snprintf(tmp, sizeof tmp, "%s%u", i ? ", " : "", host[i]);
+        s += tmp;
+    }
+    s += n > shown ? ", ...]" : "]";
+    snprintf(buf, cap, "%s", s.c_str());
+    return CG_OK;
+}
+
+// ---- element-wise ------------------------------------------------------------------------------
+static int ew_result(cg_backend *b, int op, cg_dtype compute_dt, cg_dtype out_dt, const cg_tensor *shape_of,
+                     const cg_tensor *const *ins, int nin, cg_tensor **out) {
+    cg_tensor *o;
+    int rc = new_dense(b, out_dt, shape_of->dims, shape_of->rank, &o);
+    if (rc) return rc;
+    if (numel(o) > 0) {
+        rc = launch_elementwise(b, op, compute_dt, o, ins, nin);
+        if (rc) {
+            release(o);
+            return rc;
+        }
+    }
+    *out = o;
+    return CG_OK;
+}
+
+// ndarray.rs:151-174
+int cg_cast(cg_backend *b, cg_tensor *x, cg_dtype target, cg_tensor **out) {
+    Consume cx(x);
+    if (!b || !x || !out) return fail(CG_ERR_ARG, "null argument");
+    if (!supported(target) || !supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
+    if (target == x->dt) { // identity: hand the same handle back
+        retain(x);
+        *out = x;
+        return CG_OK;
+    }
+    if (x->uniform) {
+        uint32_t r = target == CG_U32 ? f32_as_u32_host(bits_f(x->ubits)) : f_bits((float)x->ubits);
+        *out = new_uniform(b, target, x->dims, x->rank, r);
+        return CG_OK;
+    }
+    CG_HIP(hipSetDevice(b->device));
+    const cg_tensor *ins[1] = {x};
+    return ew_result(b, target == CG_U32 ? kCastF2U : kCastU2F, x->dt, target, x, ins, 1, out);
+}
+
+// ndarray.rs:352-407, 630-648
+int cg_unary(cg_backend *b, cg_unary_op op, cg_tensor *x, cg_tensor **out) {
+    Consume cx(x);
+    if (!b || !x || !out) return fail(CG_ERR_ARG, "null argument");
+    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
+    if ((int)op < CG_NEG || (int)op > CG_ROUND) return fail(CG_ERR_ARG, "unknown unary op %d", (int)op);
+    if (x->dt == CG_U32 && op != CG_NEG) {
+        static const char *names[] = {"neg", "sin", "cos", "exp", "log", "floor", "round"};
+        return fail(CG_ERR_DTYPE, "Invalid input types for %s", names[op]);
+    }
+    if (x->uniform && op == CG_NEG) {
+        uint32_t r = x->dt == CG_F32 ? (x->ubits ^ 0x80000000u) : (0u - x->ubits);
+        *out = new_uniform(b, x->dt, x->dims, x->rank, r);
+        return CG_OK;
+    }
+    CG_HIP(hipSetDevice(b->device));
+    const cg_tensor *ins[1] = {x};
+    return ew_result(b, kNeg + (int)op, x->dt, x->dt, x, ins, 1, out);
+}
+
+// ndarray.rs:185-323, 598-654
+int cg_binary(cg_backend *b, cg_binary_op op, cg_tensor *x, cg_tensor *y, cg_tensor **out) {
+    Consume cx(x), cy(y);
+    if (!b || !x || !y || !out) return fail(CG_ERR_ARG, "null argument");
+    if (!supported(x->dt) || !supported(y->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
+    if ((int)op < CG_ADD || (int)op > CG_EQ) return fail(CG_ERR_ARG, "unknown binary op %d", (int)op);
+    if (x->dt != y->dt) return fail(CG_ERR_DTYPE, "TypeError: mixed dtypes in a binary operation");
+    if (!same_shape(x, y)) return fail(CG_ERR_SHAPE, "Shape mismatch in operation");
+    if (x->uniform && y->uniform && numel(x) > 0) {
+        uint32_t r = 0;
+        bool divzero = false;
+        if (fold_binary(op, x->dt, x->ubits, y->ubits, &r, &divzero)) {
+            if (divzero) return fail(CG_ERR_RANGE, "attempt to divide by zero");
+            *out = new_uniform(b, x->dt, x->dims, x->rank, r);
+            return CG_OK;
+        }
+    }
+    CG_HIP(hipSetDevice(b->device));
+    const cg_tensor *ins[2] = {x, y};
+    return ew_result(b, kAdd + (int)op, x->dt, x->dt, x, ins, 2, out);
+}
+
+// ndarray.rs:325-350
+int cg_where(cg_backend *b, cg_tensor *mask, cg_tensor *x, cg_tensor *y, cg_tensor **out) {
+    Consume cm(mask), cx(x), cy(y);
+    if (!b || !mask || !x || !y || !out) return fail(CG_ERR_ARG, "null argument");
+    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
+    if (mask->dt != x->dt || y->dt != x->dt) return fail(CG_ERR_DTYPE, "TypeError: mixed dtypes in where");
+    if (!same_shape(mask, x) || !same_shape(x, y)) return fail(CG_ERR_SHAPE, "Shape mismatch in operation");
+    CG_HIP(hipSetDevice(b->device));
+    const cg_tensor *ins[3] = {mask, x, y};
+    return ew_result(b, kWhere, x->dt, x->dt, x, ins, 3, out);
+}
+
+// ---- contraction / reductions ---------------------------------------------------------------------
+// ndarray.rs:176-183, 750-816
+int cg_matmul(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **out) {
+    Consume cx(x), cy(y);
+    if (!b || !x || !y || !out) return fail(CG_ERR_ARG, "null argument");
+    if (!supported(x->dt) || !supported(y->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
+    if (x->dt != y->dt) return fail(CG_ERR_DTYPE, "TypeError: mixed dtypes in matmul");
+    if (x->rank < 2) return fail(CG_ERR_SHAPE, "batched_matmul: lhs must be at least rank 2");
+    if (y->rank < 2) return fail(CG_ERR_SHAPE, "batched_matmul: rhs must be at least rank 2");
+    int r = x->rank;
+    if (x->dims[r - 1] != y->dims[y->rank - 2])
+        return fail(CG_ERR_SHAPE, "batched_matmul: incompatible matrix dimensions");
+    if (x->rank != y->rank) return fail(CG_ERR_SHAPE, "batched_matmul: batch dimensions must match");
+    for (int i = 0; i < r - 2; i++)
+        if (x->dims[i] != y->dims[i]) return fail(CG_ERR_SHAPE, "batched_matmul: batch dimensions must match");
+    int64_t od[kMaxRank];
+    for (int i = 0; i < r - 2; i++) od[i] = x->dims[i];
+    od[r - 2] = x->dims[r - 2];
+    od[r - 1] = y->dims[r - 1];
+    CG_HIP(hipSetDevice(b->device));
+    cg_tensor *o;
+    int rc = new_dense(b, x->dt, od, r, &o);
+    if (rc) return rc;
+    if (numel(o) > 0) {
+        rc = launch_matmul(b, x, y, o);
+        if (rc) {
+            release(o);
+            return rc;
+        }
+    }
+    *out = o;
+    return CG_OK;
+}
+
+static int reduce_entry(cg_backend *b, int kind, const char *what, cg_tensor *x, cg_tensor **out) {
+    Consume cx(x);
+    if (!b || !x || !out) return fail(CG_ERR_ARG, "null argument");
+    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
+    if (x->rank == 0) return fail(CG_ERR_SHAPE, "%s: rank-0 tensor has no last axis", what);
+    if (kind == kArgmax && x->dims[x->rank - 1] == 0)
+        return fail(CG_ERR_SHAPE, "argmax: called `Option::unwrap()` on a `None` value (empty axis)");
+    int64_t od[kMaxRank];
+    memcpy(od, x->dims, sizeof od);
+    od[x->rank - 1] = 1;
+    CG_HIP(hipSetDevice(b->device));
+    cg_tensor *o;
+    int rc = new_dense(b, kind == kArgmax ? CG_U32 : x->dt, od, x->rank, &o);
+    if (rc) return rc;
+    if (numel(o) > 0) {
+        rc = launch_reduce(b, kind, x, o);
+        if (rc) {
+            release(o);
+            return rc;
+        }
+    }
+    *out = o;
+    return CG_OK;
+}
+
+// ndarray.rs:418-425, 723-730
+int cg_sum(cg_backend *b, cg_tensor *x, cg_tensor **out) { return reduce_entry(b, kSum, "sum", x, out); }
+// ndarray.rs:409-416, 656-668
+int cg_max(cg_backend *b, cg_tensor *x, cg_tensor **out) { return reduce_entry(b, kMax, "max", x, out); }
+// ndarray.rs:427-434, 670-694
+int cg_argmax(cg_backend *b, cg_tensor *x, cg_tensor **out) { return reduce_entry(b, kArgmax, "argmax", x, out); }
+
+// ndarray.rs:436-446, 696-721
+int cg_topk(cg_backend *b, cg_tensor *x, size_t k, cg_tensor **values, cg_tensor **indices) {
+    Consume cx(x);
+    if (!b || !x || !values || !indices) return fail(CG_ERR_ARG, "null argument");
+    if (x->dt == CG_U32) return fail(CG_ERR_DTYPE, "Unsupported type for topk");
+    if (x->dt != CG_F32) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
+    if (x->rank == 0) return fail(CG_ERR_SHAPE, "topk: rank-0 tensor has no last axis");
+    int64_t n = x->dims[x->rank - 1];
+    if (n == 0) return fail(CG_ERR_SHAPE, "topk: attempt to divide by zero (empty last axis)");
+    if ((int64_t)k > n) return fail(CG_ERR_SHAPE, "topk: k larger than the last axis");
+    int64_t od[kMaxRank];
+    memcpy(od, x->dims, sizeof od);
+    od[x->rank - 1] = (int64_t)k;
+    CG_HIP(hipSetDevice(b->device));
+    cg_tensor *v, *i;
+    int rc = new_dense(b, CG_F32, od, x->rank, &v);
+    if (rc) return rc;
+    rc = new_dense(b, CG_U32, od, x->rank, &i);
+    if (rc) {
+        release(v);
+        return rc;
+    }
+    if (numel(v) > 0) {
+        rc = launch_topk(b, x, (int64_t)k, v, i);
+        if (rc) {
+            release(v);
+            release(i);
+            return rc;
+        }
+    }
+    *values = v;
+    *indices = i;
+    return CG_OK;
+}
+
+// ---- shape and indexing ---------------------------------------------------------------------------
+// ndarray.rs:448-455, 553-559 — a stride-0 view; the reference materialises.
+int cg_broadcast(cg_backend *b, cg_tensor *x, const size_t *dims, size_t rank, cg_tensor **out) {
+    Consume cx(x);
+    if (!b || !x || !out) return fail(CG_ERR_ARG, "null argument");
+    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
+    int64_t d[kMaxRank];
+    int rc = check_dims(dims, rank, d);
+    if (rc) return rc;
+    if ((size_t)x->rank > rank) return fail(CG_ERR_SHAPE, "broadcast: incompatible shape (rank)");
+    int shift = (int)rank - x->rank;
+    for (int i = 0; i < x->rank; i++)
+        if (x->dims[i] != d[i + shift] && x->dims[i] != 1)
+            return fail(CG_ERR_SHAPE, "broadcast: incompatible shape (axis %d: %lld -> %lld)", i, (long long)x->dims[i],
+                        (long long)d[i + shift]);
+    cg_tensor *v = new_view(x);
+    v->rank = (int)rank;
+    for (int i = 0; i < (int)rank; i++) {
+        int j = i - shift;
+        v->dims[i] = d[i];
+        v->strides[i] = (j >= 0 && x->dims[j] == d[i] && !x->uniform) ? x->strides[j] : 0;
+    }
+    *out = v;
+    return CG_OK;
+}
+
+// ndarray.rs:504-511, 545-551 — a view when the strides allow it, else one row-major copy.
+int cg_reshape(cg_backend *b, cg_tensor *x, const size_t *dims, size_t rank, cg_tensor **out) {
+    Consume cx(x);
+    if (!b || !x || !out) return fail(CG_ERR_ARG, "null argument");
+    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
+    int64_t d[kMaxRank];
+    int rc = check_dims(dims, rank, d);
+    if (rc) return rc;
+    int64_t n = 1;
+    for (size_t i = 0; i < rank; i++) n *= d[i];
+    if (n != numel(x)) return fail(CG_ERR_SHAPE, "reshape: element count mismatch");
+    if (n == 0 || x->uniform) {
+        cg_tensor *v = new_view(x);
+        v->rank = (int)rank;
+        for (size_t i = 0; i < rank; i++) {
+            v->dims[i] = d[i];
+            v->strides[i] = 0;
+        }
+        if (n == 0 && !x->uniform) set_row_major(v);
+        *out = v;
+        return CG_OK;
+    }
+    int64_t st[kMaxRank];
+    if (try_view_reshape(x, d, (int)rank, st)) {
+        cg_tensor *v = new_view(x);
+        v->rank = (int)rank;
+        for (size_t i = 0; i < rank; i++) {
+            v->dims[i] = d[i];
+            v->strides[i] = st[i];
+        }
+        *out = v;
+        return CG_OK;
+    }
+    CG_HIP(hipSetDevice(b->device));
+    cg_tensor *m;
+    rc = materialize(b, x, &m);
+    if (rc) return rc;
+    m->rank = (int)rank;
+    for (size_t i = 0; i < rank; i++) m->dims[i] = d[i];
+    set_row_major(m);
+    *out = m;
+    return CG_OK;
+}
+
+// ndarray.rs:457-464, 561-569
+int cg_transpose(cg_backend *b, cg_tensor *x, size_t dim0, size_t dim1, cg_tensor **out) {
+    Consume cx(x);
+    if (!b || !x || !out) return fail(CG_ERR_ARG, "null argument");
+    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
+    if (dim0 >= (size_t)x->rank || dim1 >= (size_t)x->rank) return fail(CG_ERR_RANGE, "transpose: axis out of range");
+    cg_tensor *v = new_view(x);
+    std::swap(v->dims[dim0], v->dims[dim1]);
+    std::swap(v->strides[dim0], v->strides[dim1]);
+    *out = v;
+    return CG_OK;
+}
+
+// ndarray.rs:489-502, 581-588
+int cg_slice(cg_backend *b, cg_tensor *x, size_t dim, size_t start, size_t len, cg_tensor **out) {
+    Consume cx(x);
+    if (!b || !x || !out) return fail(CG_ERR_ARG, "null argument");
+    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
+    if (dim >= (size_t)x->rank) return fail(CG_ERR_RANGE, "slice: axis out of range");
+    if ((int64_t)start > x->dims[dim] || (int64_t)len > x->dims[dim] - (int64_t)start)
+        return fail(CG_ERR_RANGE, "slice: range out of bounds");
+    cg_tensor *v = new_view(x);
+    v->dims[dim] = (int64_t)len;
+    v->offset += (int64_t)start * x->strides[dim];
+    *out = v;
+    return CG_OK;
+}
+
+// ndarray.rs:513-532, 590-596 — two strided copies into the halves of a fresh tensor.
+int cg_concat(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor **out) {
+    Consume cx(x), cy(y);
+    if (!b || !x || !y || !out) return fail(CG_ERR_ARG, "null argument");
+    if (!supported(x->dt) || !supported(y->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
+    if (x->dt != y->dt) return fail(CG_ERR_DTYPE, "Incompatible types for concatenation");
+    if (x->rank != y->rank || dim >= (size_t)x->rank) return fail(CG_ERR_SHAPE, "concat: incompatible shapes");
+    for (int i = 0; i < x->rank; i++)
+        if ((size_t)i != dim && x->dims[i] != y->dims[i]) return fail(CG_ERR_SHAPE, "concat: incompatible shapes");
+    int64_t od[kMaxRank];
+    memcpy(od, x->dims, sizeof od);
+    od[dim] = x->dims[dim] + y->dims[dim];
+    CG_HIP(hipSetDevice(b->device));
+    cg_tensor *o;
+    int rc = new_dense(b, x->dt, od, x->rank, &o);
+    if (rc) return rc;
+    const cg_tensor *parts[2] = {x, y};
+    int64_t at = 0;
+    for (int p = 0; p < 2 && !rc; p++) {
+        const cg_tensor *src = parts[p];
+        if (numel(src) > 0) {
+            cg_tensor half = cg_tensor(); // stack view of the output's slice; never released
+            half.be = b;
+            half.buf = o->buf;
+            half.dt = o->dt;
+            half.rank = o->rank;
+            memcpy(half.dims, src->dims, sizeof half.dims);
+            memcpy(half.strides, o->strides, sizeof half.strides);
+            half.offset = at * o->strides[dim];
+            const cg_tensor *ins[1] = {src};
+            rc = launch_elementwise(b, kCopy, o->dt, &half, ins, 1);
+        }
+        at += src->dims[dim];
+    }
+    if (rc) {
+        release(o);
+        return rc;
+    }
+    *out = o;
+    return CG_OK;
+}
+
+// ndarray.rs:466-487, 571-579 — gather; out-of-range indices are detected by the kernel
+// and reported by the next call that waits for the device.
+int cg_index(cg_backend *b, cg_tensor *x, size_t dim, cg_tensor *indices, cg_tensor **out) {
+    Consume cx(x), ci(indices);
+    if (!b || !x || !indices || !out) return fail(CG_ERR_ARG, "null argument");
+    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
+    if (indices->dt != CG_U32) return fail(CG_ERR_DTYPE, "Invalid input types for indexing");
+    if (dim >= (size_t)x->rank) return fail(CG_ERR_RANGE, "index: axis out of range");
+    CG_HIP(hipSetDevice(b->device));
+    int64_t J = numel(indices);
+    int64_t od[kMaxRank];
+    memcpy(od, x->dims, sizeof od);
+    od[dim] = J;
+    cg_tensor *o;
+    int rc = new_dense(b, x->dt, od, x->rank, &o);
+    if (rc) return rc;
+    if (numel(o) > 0) {
+        if (x->dims[dim] == 0) {
+            release(o);
+            return fail(CG_ERR_RANGE, "index: index out of bounds for an axis of length 0");
+        }
+        // the gather kernel wants a row-major source and a 1-D index vector
+        cg_tensor *xs = nullptr, *is = nullptr;
+        const cg_tensor *src = x, *idx = indices;
+        if (!is_contiguous(x) || x->uniform) {
+            rc = materialize(b, x, &xs);
+            src = xs;
+        }
+        if (!rc && indices->rank != 1) {
+            rc = materialize(b, indices, &is);
+            idx = is;
+        }
+        if (!rc) rc = launch_gather(b, src, (int)dim, idx, o);
+        release(xs);
+        release(is);
+        if (rc) {
+            release(o);
+            return rc;
+        }
+    }
+    *out = o;
+    return CG_OK;
+}
+
+} // extern "C"

@@ -1,0 +1,159 @@
+"""Parity tests proper: HipBackend (through the C ABI) against the CPU oracle on the
+same seeded inputs, and against the reference's known answers.
+
+Tolerances (written out in cases.assert_close): bit-exact for integer / shape / index
+ops and IEEE-exact f32 ops; rtol 1e-4 (+1e-6 abs) for f32 element-wise math; 1e-3 of
+the natural scale for matmul and sum."""
+import numpy as np
+import pytest
+
+from catgrad_amd import BackendPanic, ShapeError
+from catgrad_amd import _abi as A
+from cases import CASES, assert_close
+from kat_runner import KATS, apply, check_case
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("case", CASES, ids=lambda c: c.name)
+def test_hip_matches_oracle(hip, oracle, case):
+    print(f"case={case.name}", flush=True)
+    got = case.run(hip)
+    ref = case.run(oracle)
+    scales = case.scale() if case.scale else [None] * len(ref)
+    assert len(got) == len(ref)
+    for i, (g, e, s) in enumerate(zip(got, ref, scales)):
+        assert g.dtype == e.dtype
+        assert_close(case.kind, g, e, s, f"{case.name}[{i}]")
+
+
+@pytest.mark.parametrize("case", [c for c in CASES if c.expect is not None], ids=lambda c: c.name)
+def test_hip_matches_closed_form(hip, case):
+    print(f"case={case.name}", flush=True)
+    got = case.run(hip)
+    exp = case.expect()
+    scales = case.scale() if case.scale else [None] * len(exp)
+    for i, (g, e, s) in enumerate(zip(got, exp, scales)):
+        assert_close(case.kind, g, e, s, f"{case.name}[{i}]")
+
+
+@pytest.mark.parametrize("case", KATS["cases"], ids=lambda c: c["name"])
+def test_hip_reference_kat(hip, case):
+    check_case(hip, case)
+
+
+@pytest.mark.parametrize("case", KATS["errors"], ids=lambda c: c["name"])
+def test_hip_reference_error(hip, case):
+    with pytest.raises(BackendPanic) as e:
+        apply(hip, case)
+    if "message" in case:
+        assert case["message"] in str(e.value)
+
+
+def test_from_vec_shape_error(hip):
+    with pytest.raises(ShapeError):
+        hip.ndarray_from_vec_f32([1.0, 2.0, 3.0], (2, 2))
+    with pytest.raises(ShapeError):
+        hip.ndarray_from_vec_u32([1, 2, 3, 4], (3,))
+
+
+def test_error_paths(hip):
+    x = hip.from_numpy(np.arange(12, dtype=np.float32).reshape(3, 4))
+    u = hip.from_numpy(np.arange(12, dtype=np.uint32).reshape(3, 4))
+    for bad in (
+        lambda: hip.add(x, u),
+        lambda: hip.sin(u),
+        lambda: hip.topk(u, 2),
+        lambda: hip.topk(x, 5),
+        lambda: hip.matmul(x, x),
+        lambda: hip.matmul(x, hip.reshape(x, (1, 4, 3))),
+        lambda: hip.slice(x, 1, 3, 2),
+        lambda: hip.slice(x, 2, 0, 1),
+        lambda: hip.transpose(x, 0, 2),
+        lambda: hip.reshape(x, (5, 2)),
+        lambda: hip.concat(x, hip.reshape(x, (4, 3)), 0),
+        lambda: hip.index(x, 0, x),
+        lambda: hip.max(hip.from_numpy(np.float32(1).reshape(()))),
+        lambda: hip.argmax(hip.zeros((3, 0), A.F32)),
+        lambda: hip.zeros((2, 2), A.F16),
+        lambda: hip.cast(x, A.BF16),
+        lambda: hip.div(hip.broadcast(hip.from_numpy(np.uint32(3).reshape(())), (2,)),
+                        hip.zeros((2,), A.U32)),
+    ):
+        with pytest.raises(BackendPanic):
+            bad()
+
+
+def test_deferred_device_faults(hip):
+    """Gather index out of range and u32 division by zero are detected by the kernel and
+    reported by the next call that waits for the device (the reference panics at once)."""
+    w = hip.from_numpy(np.arange(20, dtype=np.float32).reshape(5, 4))
+    bad = hip.index(w, 0, hip.from_numpy(np.array([1, 7], np.uint32)))
+    with pytest.raises(BackendPanic, match="out of bounds"):
+        hip.sync()
+    np.testing.assert_array_equal(hip.to_numpy(bad)[0], np.arange(4, 8, dtype=np.float32))
+    a = hip.from_numpy(np.array([4, 6, 8], np.uint32))
+    q = hip.div(a, hip.from_numpy(np.array([2, 0, 4], np.uint32)))
+    with pytest.raises(BackendPanic, match="divide by zero"):
+        hip.to_vec(q)
+    hip.sync()  # the fault word was cleared
+
+
+def test_clone_is_refcount_and_values_survive_release(hip):
+    x = hip.from_numpy(np.arange(6, dtype=np.float32).reshape(2, 3))
+    y = x.clone()
+    t = hip.transpose(x.move(), 0, 1)
+    del y
+    np.testing.assert_array_equal(hip.to_numpy(t), np.arange(6, dtype=np.float32).reshape(2, 3).T)
+
+
+def test_pool_returns_to_baseline(hip):
+    hip.sync()
+    base, _ = hip.pool_stats()
+    for _ in range(3):
+        a = hip.from_numpy(np.ones((257, 129), np.float32))
+        b = hip.exp(hip.add(a, a))
+        c = hip.sum(b)
+        hip.to_numpy(c)
+        del a, b, c
+    now, cached = hip.pool_stats()
+    assert now == base
+    assert cached > 0
+
+
+def test_format_tensor(hip):
+    s = hip.format_tensor(hip.from_numpy(np.array([[1.5, 2.0]], np.float32)))
+    assert "f32[1,2]" in s and "1.5" in s
+
+
+# ---- full-size checks through size-independent properties -----------------------------------
+def test_microbench_shapes_properties(hip):
+    """Config-2 shapes: linearity / invariants instead of a CPU recomputation."""
+    rng = np.random.default_rng(0)
+    n = 8192
+    row = rng.standard_normal((1, n)).astype(np.float32)
+    big = hip.broadcast(hip.from_numpy(row), (4096, n))
+    # sum over the last axis of a row-broadcast tensor: every row gives the same value
+    s = hip.to_numpy(hip.sum(big))
+    ref = np.float64(row.astype(np.float64).sum())
+    assert s.shape == (4096, 1)
+    assert np.all(s == s[0])
+    assert abs(float(s[0, 0]) - ref) <= 1e-3 * np.abs(row).astype(np.float64).sum()
+    m = hip.to_numpy(hip.max(big))
+    assert np.all(m == row.max())
+    am = hip.to_numpy(hip.argmax(big))
+    assert np.all(am == np.uint32(n - 1 - np.argmax(row[0, ::-1])))
+    # exp(a + b) == exp(a) * exp(b) on [8192, 8192]
+    a = hip.from_numpy((rng.standard_normal((n, n)) * 0.5).astype(np.float32))
+    b = hip.from_numpy((rng.standard_normal((n, n)) * 0.5).astype(np.float32))
+    lhs = hip.exp(hip.add(a, b))
+    rhs = hip.mul(hip.exp(a), hip.exp(b))
+    d = hip.to_numpy(hip.max(hip.reshape(hip.div(hip.sub(lhs.clone(), rhs), lhs), (1, n * n))))
+    assert float(d[0, 0]) < 1e-5
+    # bmm [16,1024,1024]: (A B) 1 == A (B 1)
+    A_ = hip.from_numpy(rng.standard_normal((16, 1024, 1024)).astype(np.float32))
+    B_ = hip.from_numpy(rng.standard_normal((16, 1024, 1024)).astype(np.float32))
+    ones = hip.broadcast(hip.from_numpy(np.float32(1).reshape(())), (16, 1024, 1))
+    left = hip.to_numpy(hip.matmul(hip.matmul(A_, B_), ones))
+    right = hip.to_numpy(hip.matmul(A_, hip.matmul(B_, ones)))
+    np.testing.assert_allclose(left, right, rtol=0, atol=1e-3 * 1024 * 32)
