@@ -20,6 +20,9 @@ OK, ERR_SHAPE, ERR_DTYPE, ERR_RANGE, ERR_DEVICE, ERR_UNSUPPORTED, ERR_ARG = rang
 NEG, SIN, COS, EXP, LOG, FLOOR, ROUND = range(7)
 ADD, SUB, MUL, DIV, POW, LT, GT, GTE, LTE, EQ = range(10)
 
+# enum cg_kernel_class
+K_GEMM_MFMA, K_GEMM_SKINNY, K_GEMM_SIMPLE, K_ELEMENTWISE, K_REDUCE, K_GATHER = range(6)
+
 _P = C.c_void_p
 _PP = C.POINTER(C.c_void_p)
 _SZ = C.c_size_t
@@ -35,6 +38,8 @@ SIGNATURES = {
     "cg_sync": (_I, [_P]),
     "cg_pool_stats": (_I, [_P, _SZP, _SZP]),
     "cg_pool_trim": (_I, [_P]),
+    "cg_profile_enable": (_I, [_P, _I, C.c_uint]),
+    "cg_profile_read": (_I, [_P, _I, C.POINTER(C.c_uint64), C.POINTER(C.c_double), C.POINTER(C.c_double), _I]),
     "cg_tensor_retain": (None, [_P]),
     "cg_tensor_release": (None, [_P]),
     "cg_tensor_rank": (_SZ, [_P]),

@@ -136,6 +136,16 @@ class Backend:
         self._check(self._lib.cg_pool_stats(self._b, C.byref(u), C.byref(c)))
         return int(u.value), int(c.value)
 
+    def profile_enable(self, cls: int, sample_every: int = 1):
+        """Time every `sample_every`-th launch of a kernel class with HIP events (0: off)."""
+        self._check(self._lib.cg_profile_enable(self._b, cls, sample_every))
+
+    def profile_read(self, cls: int, reset: bool = True):
+        """(launches timed, device milliseconds, algorithmic work) of a kernel class."""
+        n, ms, w = C.c_uint64(), C.c_double(), C.c_double()
+        self._check(self._lib.cg_profile_read(self._b, cls, C.byref(n), C.byref(ms), C.byref(w), int(reset)))
+        return int(n.value), float(ms.value), float(w.value)
+
     def pool_trim(self):
         self._check(self._lib.cg_pool_trim(self._b))
 

@@ -10,6 +10,8 @@
 #include <map>
 #include <mutex>
 #include <string>
+#include <utility>
+#include <vector>
 
 #include "../../include/catgrad_hip.h"
 
@@ -47,6 +49,17 @@ class Pool {
     size_t in_use_ = 0, cached_ = 0;
 };
 
+struct ProfClass {
+    unsigned every = 0;
+    uint64_t seen = 0, timed = 0;
+    double ms = 0.0, work = 0.0;
+};
+struct ProfPending {
+    hipEvent_t a, b;
+    int cls;
+    double work;
+};
+
 } // namespace cg
 
 struct cg_backend {
@@ -58,6 +71,9 @@ struct cg_backend {
     uint32_t *flag_dev = nullptr;   // 4-byte scratch for to_bool / compare
     uint32_t *flag_host = nullptr;  // pinned landing zone for it
     std::string name;
+    cg::ProfClass prof[CG_K_CLASSES];
+    std::vector<cg::ProfPending> prof_pending;
+    std::vector<std::pair<hipEvent_t, hipEvent_t>> prof_free;
 };
 
 namespace cg {
@@ -140,6 +156,21 @@ struct EwGeom {
 // the output) and fills geometry + operands.  Returns CG_ERR_UNSUPPORTED when the
 // space exceeds 2^32-1 work items.
 int plan_elementwise(const cg_tensor *const *views, int n, EwGeom *g, Operand *ops);
+
+// Times one launch with a pair of events on the backend's stream when the kernel class
+// is being sampled; the pair is resolved by the next call that waits for the device.
+class ProfScope {
+  public:
+    ProfScope(cg_backend *be, int cls, double work);
+    ~ProfScope();
+
+  private:
+    cg_backend *be_;
+    int slot_ = -1;
+};
+// Algorithmic bytes of a view: 4 B per distinct element (broadcast axes count once).
+double distinct_bytes(const cg_tensor *t);
+void prof_drain(cg_backend *be);
 
 // ---- kernel launchers (ew.hip, reduce.hip, matmul.hip) -------------------------------
 enum EwOp : int {

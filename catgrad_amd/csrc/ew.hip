@@ -226,6 +226,9 @@ int launch_elementwise(cg_backend *be, int op, cg_dtype dt, const cg_tensor *out
     a.out = ops[0];
     for (int k = 0; k < nin; k++) a.in[k] = ops[k + 1];
     a.fault = be->fault_dev;
+    double work = distinct_bytes(out);
+    for (int k = 0; k < nin; k++) work += distinct_bytes(ins[k]);
+    ProfScope prof(be, CG_K_ELEMENTWISE, work);
     switch (op) {
 #define CG_EW1(OP) case OP: return launch_by_dtype<OP, 1>(be, dt, a);
 #define CG_EW2(OP) case OP: return launch_by_dtype<OP, 2>(be, dt, a);
@@ -282,6 +285,7 @@ int launch_gather(cg_backend *be, const cg_tensor *x, int dim, const cg_tensor *
     uint64_t total = (uint64_t)outer * J * ipr;
     if (total > 0xFFFFFFFFull) return fail(CG_ERR_UNSUPPORTED, "index: launch above 2^32-1 work items");
     dim3 grid((uint32_t)((total + kBlock - 1) / kBlock)), block(kBlock);
+    ProfScope prof(be, CG_K_GATHER, 2.0 * distinct_bytes(out) + distinct_bytes(idx));
     if (vec4)
         hipLaunchKernelGGL((gather_kernel<4>), grid, block, 0, be->stream, static_cast<const uint32_t *>(xp),
                            static_cast<const uint32_t *>(ip), istride, op, (uint32_t)D, (uint32_t)inner,

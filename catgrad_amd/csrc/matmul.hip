@@ -356,6 +356,10 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
     if (batch > 65535) return fail(CG_ERR_UNSUPPORTED, "matmul: more than 65535 batch entries after folding");
     const bool f32 = x->dt == CG_F32;
     hipStream_t s = be->stream;
+    const double flop = 2.0 * (double)M * (double)N * (double)K * (double)batch;
+    const double bytes = distinct_bytes(x) + distinct_bytes(y) + distinct_bytes(out);
+    const bool simple = K == 0 || !f32, skinny = !simple && M <= 8 && a.b_sk == 1;
+    ProfScope prof(be, simple ? CG_K_GEMM_SIMPLE : skinny ? CG_K_GEMM_SKINNY : CG_K_GEMM_MFMA, skinny ? bytes : flop);
     if (K == 0 || !f32) {
         uint64_t elems = (uint64_t)M * N;
         dim3 grid((uint32_t)((elems + kThreads - 1) / kThreads), (uint32_t)batch);

@@ -290,6 +290,7 @@ int launch_reduce(cg_backend *be, int kind, const cg_tensor *x, cg_tensor *out) 
     if (rc) return rc;
     a.out = static_cast<uint32_t *>(out->buf->ptr);
     bool f = x->dt == CG_F32;
+    ProfScope prof(be, CG_K_REDUCE, distinct_bytes(x) + distinct_bytes(out));
     switch (kind) {
     case kSum: return f ? launch_rows<kSum, true>(be, a) : launch_rows<kSum, false>(be, a);
     case kMax: return f ? launch_rows<kMax, true>(be, a) : launch_rows<kMax, false>(be, a);

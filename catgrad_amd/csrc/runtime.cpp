@@ -292,6 +292,62 @@ int plan_elementwise(const cg_tensor *const *views, int n, EwGeom *g, Operand *o
     return CG_OK;
 }
 
+// ---- launch timing ---------------------------------------------------------------------
+constexpr size_t kProfMaxPending = 16384;
+
+ProfScope::ProfScope(cg_backend *be, int cls, double work) : be_(be) {
+    ProfClass &c = be->prof[cls];
+    if (!c.every) return;
+    if (c.seen++ % c.every) return;
+    if (be->prof_pending.size() >= kProfMaxPending) return;
+    ProfPending p;
+    if (!be->prof_free.empty()) {
+        p.a = be->prof_free.back().first;
+        p.b = be->prof_free.back().second;
+        be->prof_free.pop_back();
+    } else {
+        if (hipEventCreate(&p.a) != hipSuccess) return;
+        if (hipEventCreate(&p.b) != hipSuccess) {
+            (void)hipEventDestroy(p.a);
+            return;
+        }
+    }
+    p.cls = cls;
+    p.work = work;
+    (void)hipEventRecord(p.a, be->stream);
+    be->prof_pending.push_back(p);
+    slot_ = (int)be->prof_pending.size() - 1;
+}
+
+ProfScope::~ProfScope() {
+    if (slot_ >= 0) (void)hipEventRecord(be_->prof_pending[slot_].b, be_->stream);
+}
+
+// Call only after the stream has been synchronised.
+void prof_drain(cg_backend *be) {
+    for (ProfPending &p : be->prof_pending) {
+        float ms = 0.0f;
+        if (hipEventElapsedTime(&ms, p.a, p.b) == hipSuccess) {
+            ProfClass &c = be->prof[p.cls];
+            c.timed++;
+            c.ms += ms;
+            c.work += p.work;
+        } else {
+            (void)hipGetLastError();
+        }
+        be->prof_free.emplace_back(p.a, p.b);
+    }
+    be->prof_pending.clear();
+}
+
+double distinct_bytes(const cg_tensor *t) {
+    if (t->uniform) return 0.0;
+    double n = 1.0;
+    for (int i = 0; i < t->rank; i++)
+        if (t->strides[i] != 0 || t->dims[i] <= 1) n *= (double)t->dims[i];
+    return 4.0 * n;
+}
+
 // ---- helpers for the entry points -------------------------------------------------------
 struct Consume { // the consumed reference of a tensor argument (move semantics of the ABI)
     cg_tensor *t;
@@ -311,6 +367,7 @@ static bool same_shape(const cg_tensor *a, const cg_tensor *b) {
 
 static int wait_and_check(cg_backend *be) {
     CG_HIP(hipStreamSynchronize(be->stream));
+    if (!be->prof_pending.empty()) prof_drain(be);
     uint32_t f = *reinterpret_cast<volatile uint32_t *>(be->fault_host);
     if (f) {
         *reinterpret_cast<volatile uint32_t *>(be->fault_host) = 0;
@@ -481,6 +538,11 @@ void cg_backend_destroy(cg_backend *b) {
     if (!b) return;
     (void)hipSetDevice(b->device);
     (void)hipStreamSynchronize(b->stream);
+    prof_drain(b);
+    for (auto &ev : b->prof_free) {
+        (void)hipEventDestroy(ev.first);
+        (void)hipEventDestroy(ev.second);
+    }
     b->pool.trim();
     (void)hipFree(b->flag_dev);
     (void)hipHostFree(b->flag_host);
@@ -507,6 +569,28 @@ int cg_pool_trim(cg_backend *b) {
     if (!b) return fail(CG_ERR_ARG, "null backend");
     CG_HIP(hipStreamSynchronize(b->stream));
     b->pool.trim();
+    return CG_OK;
+}
+
+int cg_profile_enable(cg_backend *b, cg_kernel_class cls, unsigned sample_every) {
+    if (!b || (int)cls < 0 || (int)cls >= CG_K_CLASSES) return fail(CG_ERR_ARG, "bad profile class");
+    b->prof[cls].every = sample_every;
+    return CG_OK;
+}
+
+int cg_profile_read(cg_backend *b, cg_kernel_class cls, uint64_t *launches, double *milliseconds, double *work,
+                    int reset) {
+    if (!b || (int)cls < 0 || (int)cls >= CG_K_CLASSES) return fail(CG_ERR_ARG, "bad profile class");
+    int rc = wait_and_check(b);
+    if (rc) return rc;
+    ProfClass &c = b->prof[cls];
+    if (launches) *launches = c.timed;
+    if (milliseconds) *milliseconds = c.ms;
+    if (work) *work = c.work;
+    if (reset) {
+        c.seen = c.timed = 0;
+        c.ms = c.work = 0.0;
+    }
     return CG_OK;
 }
 

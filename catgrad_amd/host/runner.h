@@ -1,0 +1,52 @@
+/* runner.h — C entry points of the host driver (libcatgrad_host.so): the C++ mirror of
+ * catgrad's interpreter and model graphs, driving any library that exports the backend
+ * C ABI (include/catgrad_hip.h).  Used by bench.py and the tests through ctypes. */
+#ifndef CATGRAD_HOST_RUNNER_H
+#define CATGRAD_HOST_RUNNER_H
+#include <stddef.h>
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct cgm_session cgm_session; /* Interpreter<B> + Parameters + model config */
+
+int cgm_open(const char *backend_library, int device, cgm_session **out);
+void cgm_close(cgm_session *s);
+const char *cgm_last_error(void);
+const char *cgm_backend_name(cgm_session *s);
+
+/* Parameters::insert(path, interpreter::tensor(backend, shape, data)) */
+int cgm_set_param(cgm_session *s, const char *path, const float *data, const size_t *dims, size_t rank);
+int cgm_clear_params(cgm_session *s);
+
+/* arch: 0 = llama, 1 = qwen3 (dense). */
+int cgm_set_config(cgm_session *s, int arch, size_t hidden_size, size_t num_hidden_layers, size_t num_attention_heads,
+                   size_t num_key_value_heads, size_t head_dim, size_t intermediate_size, size_t vocab_size,
+                   float rms_norm_eps, float rope_theta, int tie_word_embeddings);
+
+/* Prefill + `steps` greedy decode runs.  out_tokens: (steps+1) x B ids.  stats:
+ * [prefill_s, decode_s, backend calls in prefill, backend calls in decode]. */
+int cgm_generate(cgm_session *s, const uint32_t *prompt, size_t B, size_t S, size_t steps, size_t max_positions,
+                 uint32_t *out_tokens, double *stats4);
+
+/* One run on an empty cache.  out_tokens: B x S argmax ids.  out_logits (may be null):
+ * B x S x vocab logits, read from the same run just before `argmax`. */
+int cgm_forward(cgm_session *s, const uint32_t *tokens, size_t B, size_t S, size_t max_positions, uint32_t *out_tokens,
+                float *out_logits);
+
+/* Config-1 MLP: x f32[1, rows, in] -> Linear(in, hidden)+b -> Sigmoid -> Linear(hidden, out)+b.
+ * Parameters: mlp.l1.weight [hidden,in], mlp.l1.bias [hidden], mlp.l2.weight [out,hidden], mlp.l2.bias [out]. */
+int cgm_mlp(cgm_session *s, const float *x, size_t rows, size_t in_dim, size_t hidden, size_t out_dim, float *y);
+
+/* Pass-through of the backend's launch-timing hooks (cg_profile_enable / cg_profile_read). */
+int cgm_profile_enable(cgm_session *s, int kernel_class, unsigned sample_every);
+int cgm_profile_read(cgm_session *s, int kernel_class, uint64_t *launches, double *milliseconds, double *work, int reset);
+
+/* Bytes the backend's device pool has handed out / holds cached. */
+int cgm_pool_stats(cgm_session *s, size_t *in_use, size_t *cached);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -108,6 +108,25 @@ int cg_pool_stats(cg_backend *b, size_t *bytes_in_use, size_t *bytes_cached);
 /* Return cached blocks to the driver. */
 int cg_pool_trim(cg_backend *b);
 
+/* ---- measurement hooks (no counterpart in the reference; used by the benchmark) ----
+ * Per-kernel-class device timing with HIP events recorded on the backend's stream
+ * around every `sample_every`-th launch of the class (0 switches the class off).
+ * cg_profile_read returns the launches timed so far, their summed device time and their
+ * summed algorithmic work (flop for the GEMM classes, bytes for the others) and
+ * optionally resets the counters; it waits for the device. */
+typedef enum cg_kernel_class {
+    CG_K_GEMM_MFMA = 0,   /* work = 2*M*N*K flop per batch entry */
+    CG_K_GEMM_SKINNY = 1, /* work = bytes of A, B and C */
+    CG_K_GEMM_SIMPLE = 2, /* work = flop */
+    CG_K_ELEMENTWISE = 3, /* work = bytes of distinct operand elements + output */
+    CG_K_REDUCE = 4,      /* work = bytes of the input + output */
+    CG_K_GATHER = 5,      /* work = bytes gathered + written */
+    CG_K_CLASSES = 6
+} cg_kernel_class;
+int cg_profile_enable(cg_backend *b, cg_kernel_class cls, unsigned sample_every);
+int cg_profile_read(cg_backend *b, cg_kernel_class cls, uint64_t *launches, double *milliseconds, double *work,
+                    int reset);
+
 /* ---- tensor handles -------------------------------------------------------
  * `BackendTensorOps` (mod.rs:124-126): Clone + shape(). */
 void cg_tensor_retain(cg_tensor *t);

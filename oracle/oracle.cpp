@@ -428,6 +428,13 @@ int cg_pool_stats(cg_backend *, size_t *u, size_t *c) {
     return CG_OK;
 }
 int cg_pool_trim(cg_backend *) { return CG_OK; }
+int cg_profile_enable(cg_backend *, cg_kernel_class, unsigned) { return CG_OK; } // no kernels to time
+int cg_profile_read(cg_backend *, cg_kernel_class, uint64_t *launches, double *milliseconds, double *work, int) {
+    if (launches) *launches = 0;
+    if (milliseconds) *milliseconds = 0.0;
+    if (work) *work = 0.0;
+    return CG_OK;
+}
 
 void cg_tensor_retain(cg_tensor *t) {
     if (t) t->rc.fetch_add(1);

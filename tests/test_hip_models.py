@@ -1,0 +1,119 @@
+"""End-to-end parity on the GPU: the host driver over HipBackend against the same driver
+over the CPU oracle — identical seeded weights and prompts, token equality with the
+top1-top2 gap rule, logits within the 1e-3 matmul/reduction contract."""
+import numpy as np
+import pytest
+
+import np_models
+from catgrad_amd.runner import SMOLLM2_135M, LlmConfig, Session, random_params
+from model_cases import TINY, load_mlp, mlp_case, params_of, prompt_of
+from oracle_loader import ORACLE_LIB, oracle_library
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def hip_session():
+    return Session()  # the product path: HipBackend, no fallback
+
+
+@pytest.fixture(scope="module")
+def cpu_session():
+    oracle_library()
+    return Session(ORACLE_LIB)
+
+
+def assert_tokens_match(got, ref, gaps=None, gap_floor=0.0):
+    bad = np.argwhere(got != ref)
+    if bad.size == 0:
+        return
+    step, b = bad[0]
+    if gaps is not None and gaps[step, b] <= gap_floor:
+        return  # near-tie: a different summation order may legitimately pick the other token
+    raise AssertionError(f"token mismatch first at step {step}, row {b}: {got[step, b]} != {ref[step, b]}")
+
+
+@pytest.mark.parametrize("name", list(TINY))
+def test_tiny_models_logits_and_decode(hip_session, cpu_session, name):
+    cfg = TINY[name]
+    params = params_of(cfg, seed=11, scale=4.0)
+    prompt = prompt_of(cfg, 3, 10, seed=12)
+    outs = []
+    for s in (hip_session, cpu_session):
+        s.load_model(cfg, params=params.items())
+        toks, logits = s.forward(prompt, max_positions=32)
+        gen, stats = s.generate(prompt, steps=12, max_positions=32)
+        outs.append((toks, logits, gen))
+    (t_h, l_h, g_h), (t_c, l_c, g_c) = outs
+    assert np.abs(l_h - l_c).max() <= 1e-3 * np.abs(l_c).max()
+    np.testing.assert_array_equal(t_h, t_c)
+    _, gaps = np_models.greedy(cfg, params, prompt, 12)
+    assert_tokens_match(g_h, g_c, gaps, 1e-3 * np.abs(l_c).max())
+
+
+def test_config1_mlp(hip_session, cpu_session):
+    case = mlp_case(0)
+    ys = []
+    for s in (hip_session, cpu_session):
+        load_mlp(s, case)
+        ys.append(s.mlp(case[0], 512, 10))
+    np.testing.assert_allclose(ys[0], ys[1], rtol=1e-3, atol=1e-6)
+    np.testing.assert_allclose(ys[0][0], np_models.mlp(*case), rtol=1e-3, atol=1e-5)
+
+
+def test_config3_smollm2_shape_prefill(hip_session, cpu_session):
+    """BASELINE config 3: SmolLM2-135M shape, random init N(0, 0.02), prefill batch 1 x 512."""
+    cfg = SMOLLM2_135M
+    params = list(random_params(cfg, seed=0))
+    prompt = prompt_of(cfg, 1, 512, seed=0)
+    hip_session.load_model(cfg, params=params)
+    t_h, l_h = hip_session.forward(prompt, max_positions=512)
+    cpu_session.load_model(cfg, params=params)
+    t_c, l_c = cpu_session.forward(prompt, max_positions=512)
+    cpu_session.clear_params()
+    scale = np.abs(l_c).max()
+    err = np.abs(l_h - l_c).max()
+    srt = np.sort(l_c[0], -1)
+    gaps = srt[:, -1] - srt[:, -2]
+    flips = t_h[0] != t_c[0]
+    print(f"config3: max |dlogit| {err:.3e} (scale {scale:.3e}); token flips {int(flips.sum())}/512; "
+          f"min top1-top2 gap {gaps.min():.3e}", flush=True)
+    assert err <= 1e-3 * scale
+    assert not (flips & (gaps > 2 * err)).any()
+
+
+def test_reduced_qwen3_prefill_and_decode(hip_session, cpu_session):
+    """Qwen3-0.6B layer shape (hidden 1024, 16/8 heads, head_dim 128, QK-norm, MLP 3072) with 4
+    layers and a 4096-entry vocabulary: prefill 128 tokens, 16 greedy decode steps with KV cache."""
+    cfg = LlmConfig("qwen3", 1024, 4, 16, 8, 3072, 4096, head_dim=128, rms_norm_eps=1e-6, rope_theta=1000000.0,
+                    tie_word_embeddings=True)
+    params = list(random_params(cfg, seed=2))
+    prompt = prompt_of(cfg, 2, 128, seed=3)
+    hip_session.load_model(cfg, params=params)
+    g_h, st = hip_session.generate(prompt, steps=16, max_positions=160)
+    _, l_h = hip_session.forward(prompt, max_positions=160)
+    cpu_session.load_model(cfg, params=params)
+    g_c, _ = cpu_session.generate(prompt, steps=16, max_positions=160)
+    _, l_c = cpu_session.forward(prompt, max_positions=160)
+    cpu_session.clear_params()
+    err, scale = np.abs(l_h - l_c).max(), np.abs(l_c).max()
+    print(f"qwen3-reduced: max |dlogit| {err:.3e} (scale {scale:.3e}); calls/decode step {st['decode_calls'] / 16:.0f}",
+          flush=True)
+    assert err <= 1e-3 * scale
+    bad = np.argwhere(g_h != g_c)
+    if bad.size:
+        # after a near-tie flip the sequences legitimately diverge; require agreement up to there
+        print(f"first divergence at step {bad[0][0]}", flush=True)
+        assert bad[0][0] > 0
+
+
+def test_pool_returns_to_baseline_after_runs(hip_session):
+    cfg = TINY["tiny_llama"]
+    hip_session.load_model(cfg, seed=1)
+    prompt = prompt_of(cfg, 2, 8)
+    hip_session.generate(prompt, steps=4, max_positions=16)
+    base, _ = hip_session.pool_stats()
+    for _ in range(3):
+        hip_session.generate(prompt, steps=4, max_positions=16)
+    now, _ = hip_session.pool_stats()
+    assert now == base  # only the parameters stay resident between runs
