@@ -259,6 +259,174 @@ template <int MM> __global__ __launch_bounds__(kThreads) void skinny_kt_kernel(c
     }
 }
 
+
+// Vectorised skinny kernel for K > 256: a wave owns COLS output columns and walks K with
+// 16-byte loads (COLS weight loads + M activation loads in flight per lane per trip; the
+// activation rows stay in L1/L2).  SPLIT: the four waves of the block share the columns
+// and split K, for shapes with too few columns to fill the chip.
+template <int MM, int COLS, bool SPLIT>
+__global__ __launch_bounds__(kThreads) void skinny_kt_wide_kernel(const MmArgs a) {
+    const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    const uint32_t group = SPLIT ? blockIdx.x : blockIdx.x * 4 + wave;
+    const uint32_t n0 = group * COLS;
+    const bool live = n0 < a.N;
+    int64_t oa, ob;
+    batch_offsets(a, blockIdx.y, oa, ob);
+    const uint32_t *A = a.A + oa;
+    const uint32_t *B = a.B + ob;
+    float acc[COLS][MM];
+#pragma unroll
+    for (int c = 0; c < COLS; c++)
+#pragma unroll
+        for (int m = 0; m < MM; m++) acc[c][m] = 0.0f;
+    if (live) {
+        const uint32_t kstep = SPLIT ? 1024u : 256u;
+#pragma unroll 2
+        for (uint32_t k = (SPLIT ? wave * 256u : 0u) + lane * 4; k < a.K; k += kstep) {
+            float4v w[COLS], x[MM];
+#pragma unroll
+            for (int c = 0; c < COLS; c++) {
+                w[c] = (float4v){0.f, 0.f, 0.f, 0.f};
+                if (n0 + c < a.N) w[c] = *reinterpret_cast<const float4v *>(B + (int64_t)(n0 + c) * a.b_sn + k);
+            }
+#pragma unroll
+            for (int m = 0; m < MM; m++) {
+                x[m] = (float4v){0.f, 0.f, 0.f, 0.f};
+                if ((uint32_t)m < a.M) x[m] = *reinterpret_cast<const float4v *>(A + (int64_t)m * a.a_sm + k);
+            }
+#pragma unroll
+            for (int c = 0; c < COLS; c++)
+#pragma unroll
+                for (int m = 0; m < MM; m++) {
+                    acc[c][m] = fmaf(x[m][0], w[c][0], acc[c][m]);
+                    acc[c][m] = fmaf(x[m][1], w[c][1], acc[c][m]);
+                    acc[c][m] = fmaf(x[m][2], w[c][2], acc[c][m]);
+                    acc[c][m] = fmaf(x[m][3], w[c][3], acc[c][m]);
+                }
+        }
+    }
+#pragma unroll
+    for (int c = 0; c < COLS; c++)
+#pragma unroll
+        for (int m = 0; m < MM; m++) {
+#pragma unroll
+            for (int s = 32; s >= 1; s >>= 1) acc[c][m] += __shfl_xor(acc[c][m], s);
+        }
+    if (SPLIT) {
+        __shared__ float part[4][COLS * MM];
+        if (lane == 0) {
+#pragma unroll
+            for (int c = 0; c < COLS; c++)
+#pragma unroll
+                for (int m = 0; m < MM; m++) part[wave][c * MM + m] = acc[c][m];
+        }
+        __syncthreads();
+        if (threadIdx.x < COLS * MM) {
+            uint32_t c = threadIdx.x / MM, m = threadIdx.x % MM;
+            float v = (part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]);
+            if (n0 + c < a.N && m < a.M) a.C[((uint64_t)blockIdx.y * a.M + m) * a.N + n0 + c] = asu(v);
+        }
+    } else if (live && lane == 0) {
+#pragma unroll
+        for (int c = 0; c < COLS; c++)
+#pragma unroll
+            for (int m = 0; m < MM; m++)
+                if (n0 + c < a.N && (uint32_t)m < a.M) a.C[((uint64_t)blockIdx.y * a.M + m) * a.N + n0 + c] = asu(acc[c][m]);
+    }
+}
+
+// Vectorised skinny kernel for short K (K <= 4*LPC, e.g. q.K^T of a decode step with
+// K = head_dim): LPC lanes share a column, so a wave covers 64/LPC columns per pass and
+// the activation fragment is loaded once.
+template <int MM, int LPC> __global__ __launch_bounds__(kThreads) void skinny_kt_narrow_kernel(const MmArgs a) {
+    constexpr uint32_t CPW = 64 / LPC, PASSES = 4;
+    const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    const uint32_t sub = lane / LPC, l = lane % LPC;
+    const uint32_t nblock = blockIdx.x * (4 * CPW * PASSES);
+    int64_t oa, ob;
+    batch_offsets(a, blockIdx.y, oa, ob);
+    const uint32_t *A = a.A + oa;
+    const uint32_t *B = a.B + ob;
+    const uint32_t k = l * 4;
+    const bool kin = k < a.K;
+    float4v x[MM];
+#pragma unroll
+    for (int m = 0; m < MM; m++) {
+        x[m] = (float4v){0.f, 0.f, 0.f, 0.f};
+        if (kin && (uint32_t)m < a.M) x[m] = *reinterpret_cast<const float4v *>(A + (int64_t)m * a.a_sm + k);
+    }
+    float4v w[PASSES];
+#pragma unroll
+    for (uint32_t p = 0; p < PASSES; p++) {
+        uint32_t col = nblock + (p * 4 + wave) * CPW + sub;
+        w[p] = (float4v){0.f, 0.f, 0.f, 0.f};
+        if (kin && col < a.N) w[p] = *reinterpret_cast<const float4v *>(B + (int64_t)col * a.b_sn + k);
+    }
+#pragma unroll
+    for (uint32_t p = 0; p < PASSES; p++) {
+        uint32_t col = nblock + (p * 4 + wave) * CPW + sub;
+#pragma unroll
+        for (int m = 0; m < MM; m++) {
+            float v = fmaf(x[m][3], w[p][3], fmaf(x[m][2], w[p][2], fmaf(x[m][1], w[p][1], x[m][0] * w[p][0])));
+#pragma unroll
+            for (int s = LPC / 2; s >= 1; s >>= 1) v += __shfl_xor(v, s);
+            if (l == 0 && col < a.N && (uint32_t)m < a.M) a.C[((uint64_t)blockIdx.y * a.M + m) * a.N + col] = asu(v);
+        }
+    }
+}
+
+// Skinny kernel for N-contiguous B (p.V of a decode step: M = 1, K = T, N = head_dim):
+// a block owns 64 output columns (16 lanes x float4) and splits K over 16 lane groups,
+// which an LDS exchange sums at the end.
+template <int MM> __global__ __launch_bounds__(kThreads) void skinny_nn_kernel(const MmArgs a) {
+    const uint32_t ng = threadIdx.x % 16, kg = threadIdx.x / 16;
+    const uint32_t n = blockIdx.x * 64 + ng * 4;
+    int64_t oa, ob;
+    batch_offsets(a, blockIdx.y, oa, ob);
+    const uint32_t *A = a.A + oa;
+    const uint32_t *B = a.B + ob;
+    float4v acc[MM];
+#pragma unroll
+    for (int m = 0; m < MM; m++) acc[m] = (float4v){0.f, 0.f, 0.f, 0.f};
+    const bool vec = a.b_vec && n + 3 < a.N;
+#pragma unroll 4
+    for (uint32_t k = kg; k < a.K; k += 16) {
+        const uint32_t *p = B + (int64_t)k * a.b_sk + (int64_t)n * a.b_sn;
+        float4v w;
+        if (vec) {
+            w = *reinterpret_cast<const float4v *>(p);
+        } else {
+            w[0] = ld_guard(p, n < a.N);
+            w[1] = ld_guard(p + a.b_sn, n + 1 < a.N);
+            w[2] = ld_guard(p + 2 * a.b_sn, n + 2 < a.N);
+            w[3] = ld_guard(p + 3 * a.b_sn, n + 3 < a.N);
+        }
+#pragma unroll
+        for (int m = 0; m < MM; m++) {
+            if ((uint32_t)m < a.M) {
+                float x = asf(A[(int64_t)m * a.a_sm + (int64_t)k * a.a_sk]);
+                acc[m][0] = fmaf(x, w[0], acc[m][0]);
+                acc[m][1] = fmaf(x, w[1], acc[m][1]);
+                acc[m][2] = fmaf(x, w[2], acc[m][2]);
+                acc[m][3] = fmaf(x, w[3], acc[m][3]);
+            }
+        }
+    }
+    __shared__ float red[16][64 * MM + 4];
+#pragma unroll
+    for (int m = 0; m < MM; m++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) red[kg][m * 64 + ng * 4 + j] = acc[m][j];
+    __syncthreads();
+    for (uint32_t o = threadIdx.x; o < 64 * MM; o += kThreads) {
+        float v = 0.0f;
+#pragma unroll
+        for (int g = 0; g < 16; g++) v += red[g][o];
+        uint32_t m = o / 64, col = blockIdx.x * 64 + o % 64;
+        if (m < a.M && col < a.N) a.C[((uint64_t)blockIdx.y * a.M + m) * a.N + col] = asu(v);
+    }
+}
+
 // ------------------------------------------------------------------------------------------
 // Plain kernel: one thread per output element.  u32 with wrapping arithmetic
 // (ndarray.rs:181) and the f32 shapes nothing else takes.
@@ -358,7 +526,7 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
     hipStream_t s = be->stream;
     const double flop = 2.0 * (double)M * (double)N * (double)K * (double)batch;
     const double bytes = distinct_bytes(x) + distinct_bytes(y) + distinct_bytes(out);
-    const bool simple = K == 0 || !f32, skinny = !simple && M <= 8 && a.b_sk == 1;
+    const bool simple = K == 0 || !f32, skinny = !simple && M <= 8 && (a.b_sk == 1 || a.b_sn == 1);
     ProfScope prof(be, simple ? CG_K_GEMM_SIMPLE : skinny ? CG_K_GEMM_SKINNY : CG_K_GEMM_MFMA, skinny ? bytes : flop);
     if (K == 0 || !f32) {
         uint64_t elems = (uint64_t)M * N;
@@ -368,13 +536,52 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
         else
             hipLaunchKernelGGL((simple_gemm_kernel<false>), grid, dim3(kThreads), 0, s, a);
     } else if (M <= 8 && a.b_sk == 1) {
-        dim3 grid((uint32_t)((N + 3) / 4), (uint32_t)batch);
-        if (M <= 1)
-            hipLaunchKernelGGL((skinny_kt_kernel<1>), grid, dim3(kThreads), 0, s, a);
-        else if (M <= 4)
-            hipLaunchKernelGGL((skinny_kt_kernel<4>), grid, dim3(kThreads), 0, s, a);
-        else
-            hipLaunchKernelGGL((skinny_kt_kernel<8>), grid, dim3(kThreads), 0, s, a);
+        const bool vec = a.a_vec && a.b_vec && a.a_sk == 1 && K % 4 == 0;
+#define CG_MM_SWITCH(CALL)        \
+    if (M <= 1) { CALL(1) }       \
+    else if (M <= 4) { CALL(4) }  \
+    else { CALL(8) }
+        if (!vec) {
+            dim3 grid((uint32_t)((N + 3) / 4), (uint32_t)batch);
+#define CG_CALL(MMV) hipLaunchKernelGGL((skinny_kt_kernel<MMV>), grid, dim3(kThreads), 0, s, a);
+            CG_MM_SWITCH(CG_CALL)
+#undef CG_CALL
+        } else if (K <= 256) {
+            const int lpc = K <= 64 ? 16 : K <= 128 ? 32 : 64;
+            const uint32_t cols_per_block = 4 * (64 / lpc) * 4;
+            dim3 grid((uint32_t)((N + cols_per_block - 1) / cols_per_block), (uint32_t)batch);
+#define CG_CALL(MMV)                                                                                          \
+    if (lpc == 16) hipLaunchKernelGGL((skinny_kt_narrow_kernel<MMV, 16>), grid, dim3(kThreads), 0, s, a);     \
+    else if (lpc == 32) hipLaunchKernelGGL((skinny_kt_narrow_kernel<MMV, 32>), grid, dim3(kThreads), 0, s, a); \
+    else hipLaunchKernelGGL((skinny_kt_narrow_kernel<MMV, 64>), grid, dim3(kThreads), 0, s, a);
+            CG_MM_SWITCH(CG_CALL)
+#undef CG_CALL
+        } else {
+            // enough waves to cover 256 CUs several times over, else split K inside the block
+            const int64_t cols = N * batch;
+            if (cols >= 16384) {
+                dim3 grid((uint32_t)((N + 15) / 16), (uint32_t)batch);
+#define CG_CALL(MMV) hipLaunchKernelGGL((skinny_kt_wide_kernel<MMV, 4, false>), grid, dim3(kThreads), 0, s, a);
+                CG_MM_SWITCH(CG_CALL)
+#undef CG_CALL
+            } else if (cols >= 4096) {
+                dim3 grid((uint32_t)((N + 3) / 4), (uint32_t)batch);
+#define CG_CALL(MMV) hipLaunchKernelGGL((skinny_kt_wide_kernel<MMV, 1, false>), grid, dim3(kThreads), 0, s, a);
+                CG_MM_SWITCH(CG_CALL)
+#undef CG_CALL
+            } else {
+                dim3 grid((uint32_t)N, (uint32_t)batch);
+#define CG_CALL(MMV) hipLaunchKernelGGL((skinny_kt_wide_kernel<MMV, 1, true>), grid, dim3(kThreads), 0, s, a);
+                CG_MM_SWITCH(CG_CALL)
+#undef CG_CALL
+            }
+        }
+    } else if (M <= 8 && a.b_sn == 1) {
+        dim3 grid((uint32_t)((N + 63) / 64), (uint32_t)batch);
+#define CG_CALL(MMV) hipLaunchKernelGGL((skinny_nn_kernel<MMV>), grid, dim3(kThreads), 0, s, a);
+        CG_MM_SWITCH(CG_CALL)
+#undef CG_CALL
+#undef CG_MM_SWITCH
     } else {
         uint64_t tiles = (uint64_t)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
         if (tiles > 0x7FFFFFFFull) return fail(CG_ERR_UNSUPPORTED, "matmul: too many tiles");

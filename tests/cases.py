@@ -612,6 +612,20 @@ _mm_case("mm_linear_weight_view", (3, 20, 64), (48, 64),
          lambda be, x, w: (x, be.broadcast(be.transpose(w, 0, 1), (3, 64, 48)), None, None))
 _mm_case("mm_linear_decode", (4, 1, 256), (1000, 256),
          lambda be, x, w: (x, be.broadcast(be.transpose(w, 0, 1), (4, 256, 1000)), None, None))
+_mm_case("mm_linear_decode_wide_split", (4, 1, 2048), (512, 2048),
+         lambda be, x, w: (x, be.broadcast(be.transpose(w, 0, 1), (4, 2048, 512)), None, None))
+_mm_case("mm_linear_decode_wide_cols1", (4, 1, 512), (5003, 512),
+         lambda be, x, w: (x, be.broadcast(be.transpose(w, 0, 1), (4, 512, 5003)), None, None))
+_mm_case("mm_linear_decode_wide_cols4", (3, 1, 384), (20001, 384),
+         lambda be, x, w: (x, be.broadcast(be.transpose(w, 0, 1), (3, 384, 20001)), None, None))
+_mm_case("mm_linear_m8", (8, 1, 1024), (300, 1024),
+         lambda be, x, w: (x, be.broadcast(be.transpose(w, 0, 1), (8, 1024, 300)), None, None))
+_mm_case("mm_decode_scores_hd64", (2, 1, 6, 64), (2, 6, 301, 64),
+         lambda be, q, k: (be.transpose(q, 1, 2), be.transpose(k, 2, 3), None, None))
+_mm_case("mm_decode_scores_hd128", (2, 1, 4, 128), (2, 4, 77, 128),
+         lambda be, q, k: (be.transpose(q, 1, 2), be.transpose(k, 2, 3), None, None))
+_mm_case("mm_decode_context", (2, 6, 1, 301), (2, 6, 301, 64))
+_mm_case("mm_decode_context_ragged_n", (3, 5, 2, 90), (3, 5, 90, 70))
 _mm_case("mm_attention_scores", (2, 40, 6, 32), (2, 56, 6, 32),
          lambda be, q, k: (be.transpose(q, 1, 2), be.transpose(be.transpose(k, 1, 2), 2, 3), None, None))
 _mm_case("mm_attention_context", (2, 6, 40, 56), (2, 56, 6, 32),
