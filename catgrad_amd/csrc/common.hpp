@@ -115,7 +115,8 @@ bool is_contiguous(const cg_tensor *t);
 void release(cg_tensor *t);
 inline void retain(cg_tensor *t) { t->rc.fetch_add(1, std::memory_order_relaxed); }
 // Fresh row-major tensor with pool memory (none when numel == 0).
-int new_dense(cg_backend *be, cg_dtype dt, const int64_t *dims, int rank, cg_tensor **out);
+// `reserve_elems` asks for a buffer with room for at least that many elements.
+int new_dense(cg_backend *be, cg_dtype dt, const int64_t *dims, int rank, cg_tensor **out, int64_t reserve_elems = 0);
 // Fresh uniform tensor (no memory).
 cg_tensor *new_uniform(cg_backend *be, cg_dtype dt, const int64_t *dims, int rank, uint32_t bits);
 // New handle sharing t's buffer and metadata.

@@ -26,6 +26,8 @@
 #include "common.hpp"
 #include "device_utils.hpp"
 
+#include <algorithm>
+
 namespace cg {
 
 namespace {
@@ -378,7 +380,8 @@ template <int MM, int LPC> __global__ __launch_bounds__(kThreads) void skinny_kt
 // Skinny kernel for N-contiguous B (p.V of a decode step: M = 1, K = T, N = head_dim):
 // a block owns 64 output columns (16 lanes x float4) and splits K over 16 lane groups,
 // which an LDS exchange sums at the end.
-template <int MM> __global__ __launch_bounds__(kThreads) void skinny_nn_kernel(const MmArgs a) {
+template <int MM>
+__global__ __launch_bounds__(kThreads) void skinny_nn_kernel(const MmArgs a, uint32_t *dst, uint32_t kchunk) {
     const uint32_t ng = threadIdx.x % 16, kg = threadIdx.x / 16;
     const uint32_t n = blockIdx.x * 64 + ng * 4;
     int64_t oa, ob;
@@ -389,8 +392,9 @@ template <int MM> __global__ __launch_bounds__(kThreads) void skinny_nn_kernel(c
 #pragma unroll
     for (int m = 0; m < MM; m++) acc[m] = (float4v){0.f, 0.f, 0.f, 0.f};
     const bool vec = a.b_vec && n + 3 < a.N;
+    const uint32_t kbeg = blockIdx.z * kchunk, kend = min(a.K, kbeg + kchunk);
 #pragma unroll 4
-    for (uint32_t k = kg; k < a.K; k += 16) {
+    for (uint32_t k = kbeg + kg; k < kend; k += 16) {
         const uint32_t *p = B + (int64_t)k * a.b_sk + (int64_t)n * a.b_sn;
         float4v w;
         if (vec) {
@@ -423,8 +427,21 @@ template <int MM> __global__ __launch_bounds__(kThreads) void skinny_nn_kernel(c
 #pragma unroll
         for (int g = 0; g < 16; g++) v += red[g][o];
         uint32_t m = o / 64, col = blockIdx.x * 64 + o % 64;
-        if (m < a.M && col < a.N) a.C[((uint64_t)blockIdx.y * a.M + m) * a.N + col] = asu(v);
+        // dst is C itself (gridDim.z == 1) or the [batch][gridDim.z][M][N] partial sums
+        if (m < a.M && col < a.N)
+            dst[(((uint64_t)blockIdx.y * gridDim.z + blockIdx.z) * a.M + m) * a.N + col] = asu(v);
     }
+}
+
+// C[b][e] = sum over s of part[b][s][e]   (e < M*N)
+__global__ __launch_bounds__(kThreads) void splitk_reduce_kernel(const uint32_t *part, uint32_t *C, uint32_t splits,
+                                                                 uint32_t mn, uint64_t total) {
+    uint64_t i = (uint64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (i >= total) return;
+    uint64_t b = i / mn, e = i % mn;
+    float v = 0.0f;
+    for (uint32_t s = 0; s < splits; s++) v += asf(part[(b * splits + s) * mn + e]);
+    C[i] = asu(v);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -564,7 +581,7 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
 #define CG_CALL(MMV) hipLaunchKernelGGL((skinny_kt_wide_kernel<MMV, 4, false>), grid, dim3(kThreads), 0, s, a);
                 CG_MM_SWITCH(CG_CALL)
 #undef CG_CALL
-            } else if (cols >= 4096) {
+            } else if (cols >= 2048) {
                 dim3 grid((uint32_t)((N + 3) / 4), (uint32_t)batch);
 #define CG_CALL(MMV) hipLaunchKernelGGL((skinny_kt_wide_kernel<MMV, 1, false>), grid, dim3(kThreads), 0, s, a);
                 CG_MM_SWITCH(CG_CALL)
@@ -577,10 +594,31 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
             }
         }
     } else if (M <= 8 && a.b_sn == 1) {
-        dim3 grid((uint32_t)((N + 63) / 64), (uint32_t)batch);
-#define CG_CALL(MMV) hipLaunchKernelGGL((skinny_nn_kernel<MMV>), grid, dim3(kThreads), 0, s, a);
+        // split K over grid.z until about 2048 blocks are in flight (>= 128 k-rows each)
+        const int64_t blocks_xy = ((N + 63) / 64) * batch;
+        int64_t splits = std::min<int64_t>(std::min<int64_t>((2048 + blocks_xy - 1) / blocks_xy, (K + 127) / 128), 64);
+        if (splits < 1) splits = 1;
+        const uint32_t kchunk = (uint32_t)((((K + splits - 1) / splits) + 15) / 16 * 16);
+        splits = (K + kchunk - 1) / kchunk;
+        void *scratch = nullptr;
+        size_t scratch_cls = 0;
+        uint32_t *dst = a.C;
+        if (splits > 1) {
+            int prc = be->pool.alloc((size_t)batch * splits * M * N * 4, &scratch, &scratch_cls);
+            if (prc) return prc;
+            dst = static_cast<uint32_t *>(scratch);
+        }
+        dim3 grid((uint32_t)((N + 63) / 64), (uint32_t)batch, (uint32_t)splits);
+#define CG_CALL(MMV) hipLaunchKernelGGL((skinny_nn_kernel<MMV>), grid, dim3(kThreads), 0, s, a, dst, kchunk);
         CG_MM_SWITCH(CG_CALL)
 #undef CG_CALL
+        if (splits > 1) {
+            uint64_t total = (uint64_t)batch * M * N;
+            hipLaunchKernelGGL(splitk_reduce_kernel, dim3((uint32_t)((total + kThreads - 1) / kThreads)), dim3(kThreads),
+                               0, s, static_cast<const uint32_t *>(scratch), a.C, (uint32_t)splits, (uint32_t)(M * N),
+                               total);
+            be->pool.free(scratch, scratch_cls); // stream-ordered: later users queue behind the reduce
+        }
 #undef CG_MM_SWITCH
     } else {
         uint64_t tiles = (uint64_t)((M + BM - 1) / BM) * ((N + BN - 1) / BN);

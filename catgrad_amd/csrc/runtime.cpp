@@ -130,7 +130,7 @@ static void set_row_major(cg_tensor *t) {
     }
 }
 
-int new_dense(cg_backend *be, cg_dtype dt, const int64_t *dims, int rank, cg_tensor **out) {
+int new_dense(cg_backend *be, cg_dtype dt, const int64_t *dims, int rank, cg_tensor **out, int64_t reserve_elems) {
     cg_tensor *t = new cg_tensor;
     t->be = be;
     t->dt = dt;
@@ -141,7 +141,7 @@ int new_dense(cg_backend *be, cg_dtype dt, const int64_t *dims, int rank, cg_ten
     if (n > 0) {
         Buffer *b = new Buffer;
         b->be = be;
-        int rc = be->pool.alloc((size_t)n * 4, &b->ptr, &b->cls);
+        int rc = be->pool.alloc((size_t)(n > reserve_elems ? n : reserve_elems) * 4, &b->ptr, &b->cls);
         if (rc) {
             delete b;
             delete t;
@@ -1090,16 +1090,60 @@ int cg_concat(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor *
     int64_t od[kMaxRank];
     memcpy(od, x->dims, sizeof od);
     od[dim] = x->dims[dim] + y->dims[dim];
+    // an empty operand contributes nothing: the other operand IS the result (tensors are
+    // immutable, so handing the same handle back is indistinguishable from a copy)
+    if (x->dims[dim] == 0) {
+        retain(y);
+        *out = y;
+        return CG_OK;
+    }
+    if (y->dims[dim] == 0) {
+        retain(x);
+        *out = x;
+        return CG_OK;
+    }
     CG_HIP(hipSetDevice(b->device));
+    int64_t nx = numel(x), ny = numel(y);
+    bool outermost = true; // `dim` is the outermost axis with extent > 1: y lands right after x in memory
+    for (size_t i = 0; i < dim; i++) outermost = outermost && od[i] == 1;
+    // Growing a stack along its outermost axis (the per-layer restack of the KV cache,
+    // helpers/cache.rs:64-74): when this call holds the only reference to x and x's buffer
+    // has room behind it, y is appended in place and x's handle is returned with the larger
+    // extent — one copy of y instead of a copy of everything accumulated so far.
+    if (outermost && nx > 0 && ny > 0 && !x->uniform && x->rc.load() == 1 && x->buf && x->buf->rc.load() == 1 &&
+        x->offset == 0 && is_contiguous(x) && (size_t)(nx + ny) * 4 <= x->buf->cls) {
+        cg_tensor tail;
+        tail.be = b;
+        tail.buf = x->buf;
+        tail.dt = x->dt;
+        tail.rank = y->rank;
+        memcpy(tail.dims, y->dims, sizeof tail.dims);
+        int64_t st = 1;
+        for (int i = y->rank - 1; i >= 0; i--) {
+            tail.strides[i] = st;
+            st *= y->dims[i];
+        }
+        tail.offset = nx;
+        const cg_tensor *ins[1] = {y};
+        int rc = launch_elementwise(b, kCopy, x->dt, &tail, ins, 1);
+        tail.buf = nullptr;
+        if (rc) return rc;
+        x->dims[dim] = od[dim];
+        set_row_major(x);
+        retain(x);
+        *out = x;
+        return CG_OK;
+    }
     cg_tensor *o;
-    int rc = new_dense(b, x->dt, od, x->rank, &o);
+    // a stack that starts growing gets room for as much again, so later appends stay in place
+    int rc = new_dense(b, x->dt, od, x->rank, &o, outermost ? 2 * (nx + ny) : 0);
     if (rc) return rc;
     const cg_tensor *parts[2] = {x, y};
     int64_t at = 0;
     for (int p = 0; p < 2 && !rc; p++) {
         const cg_tensor *src = parts[p];
         if (numel(src) > 0) {
-            cg_tensor half = cg_tensor(); // stack view of the output's slice; never released
+            cg_tensor half; // stack view of the output's slice; never released
             half.be = b;
             half.buf = o->buf;
             half.dt = o->dt;

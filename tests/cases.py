@@ -436,6 +436,27 @@ def _():
     return run, (lambda: [np.stack(layers)])
 
 
+@case("kv_restack_chain_moved_operands")
+def _():
+    """Same chain with the growing stack MOVED into every concat, as the interpreter does:
+    uniquely owned stacks may be appended to in place."""
+    layers = [f32(70 + i, (2, 3, 4, 8)) for i in range(9)]
+
+    def run(be):
+        out = be.reshape(be.from_numpy(layers[0]).move(), (1, 2, 3, 4, 8))
+        keep = None
+        for n, l in enumerate(layers[1:]):
+            out = be.concat(out.move(), be.reshape(be.from_numpy(l).move(), (1, 2, 3, 4, 8)).move(), 0)
+            if n == 3:
+                keep = out.clone()  # a second holder: the next append must not disturb it
+        flat = be.concat(be.from_numpy(layers[0].reshape(-1)).move(), be.from_numpy(layers[1].reshape(-1)).move(), 0)
+        flat = be.concat(flat.move(), be.from_numpy(layers[2].reshape(-1)).move(), 0)
+        return N(be, out, keep, flat)
+
+    return run, (lambda: [np.stack(layers), np.stack(layers[:5]),
+                          np.concatenate([l.reshape(-1) for l in layers[:3]])])
+
+
 @case("index_gather")
 def _():
     w = f32(60, (50, 16))
