@@ -81,7 +81,10 @@ def micro_bench(iters=20):
 
 def cpu_baseline(cfg, params, B, sample_prefill, sample_decode, seed):
     """The oracle on this box's host cores (it is single-threaded, like NdArrayBackend) on a
-    bounded sample of the workload: same model, same batch, a short prompt and few steps."""
+    bounded sample of the workload: same model, a short prompt and few steps, at the
+    batch size the reference's own CLI uses (1; catgrad-llm/examples/llama/main.rs:947-951).
+    With batch 4 one forward pass alone takes about a minute of CPU time, most of it
+    materialising the batch-broadcast weight views."""
     from catgrad_amd.runner import Session
 
     lib = os.path.join(ROOT, "oracle", "liboracle.so")
@@ -98,7 +101,7 @@ def cpu_baseline(cfg, params, B, sample_prefill, sample_decode, seed):
     return {
         "value": round(tokens / (st["prefill_s"] + st["decode_s"]), 3), "unit": "tok/s", "cores": 1,
         "host_cores": os.cpu_count(), "kind": "port",
-        "sample": f"same model and batch {B}; prefill {sample_prefill} tokens/seq + {sample_decode} decode steps "
+        "sample": f"same model, batch {B}; prefill {sample_prefill} tokens/seq + {sample_decode} decode steps "
                   f"({wall:.1f} s of CPU work); prefill {B * sample_prefill / st['prefill_s']:.2f} tok/s, "
                   f"decode {B * sample_decode / max(st['decode_s'], 1e-9):.3f} tok/s",
     }
@@ -115,12 +118,27 @@ def main():
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-micro", action="store_true")
-    ap.add_argument("--cpu-sample", type=int, nargs=2, default=[8, 1], metavar=("PREFILL", "DECODE"))
+    ap.add_argument("--cpu-sample", type=int, nargs=3, default=[1, 16, 2], metavar=("BATCH", "PREFILL", "DECODE"))
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="only run a strided copy of known size (268435456 B read + 268435456 B written per launch), "
+                         "the yardstick for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this backend runs on ONE GPU; every box in this build has one GPU and the path has no "
               "collective step. Run with --gpus 1.", file=sys.stderr)
         sys.exit(2)
+
+    if args.calibrate_copy:
+        from catgrad_amd import HipBackend
+
+        be = HipBackend(0)
+        x = be.from_numpy(np.zeros((8192, 8192 + 4), dtype=np.float32))
+        for _ in range(10):
+            be.reshape(be.slice(x, 1, 0, 8192), (8192 * 8192,))
+        be.sync()
+        print(json.dumps({"calibration": "ew_kernel<copy> 10 launches", "read_bytes": 8192 * 8192 * 4,
+                          "write_bytes": 8192 * 8192 * 4}))
+        return
 
     import torch  # device-wide synchronisation around the timed region
 
@@ -211,7 +229,7 @@ def main():
     if not args.no_micro:
         result["micro"] = micro_bench()
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(cfg, params, B, args.cpu_sample[0], args.cpu_sample[1], args.seed)
+        result["cpu_baseline"] = cpu_baseline(cfg, params, *args.cpu_sample, args.seed)
     print(json.dumps(result))
 
 

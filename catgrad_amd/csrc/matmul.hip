@@ -66,6 +66,7 @@ __device__ __forceinline__ void batch_offsets(const MmArgs &a, uint32_t b, int64
 constexpr int BM = 128, BN = 128, BK = 16;
 constexpr int PITCH = BK + 4; // words per LDS row
 constexpr int kThreads = 256;
+constexpr uint32_t kXcds = 8, kGroupM = 8;
 
 typedef float float4v __attribute__((ext_vector_type(4)));
 typedef float float16v __attribute__((ext_vector_type(16)));
@@ -137,8 +138,24 @@ template <bool A_MFAST, bool B_NFAST> __global__ __launch_bounds__(kThreads) voi
     __shared__ float lds_a[2][BM * PITCH];
     __shared__ float lds_b[2][BN * PITCH];
 
-    const uint32_t tiles_n = (a.N + BN - 1) / BN;
-    const uint32_t tile_m = blockIdx.x / tiles_n, tile_n = blockIdx.x % tiles_n;
+    // Tile order.  Workgroups are dealt round-robin to the 8 XCDs, each with its own L2, so
+    // the linear id is first regrouped to give every XCD one contiguous run of tiles; inside
+    // the run tiles advance down a column of kGroupM row-tiles before moving to the next
+    // column-tile, so that the tiles in flight on one XCD share A and B panels in its L2
+    // instead of each streaming its own from HBM.
+    const uint32_t tiles_n = (a.N + BN - 1) / BN, tiles_m = (a.M + BM - 1) / BM;
+    const uint32_t ntiles = tiles_m * tiles_n;
+    uint32_t lin;
+    {
+        const uint32_t xcd = blockIdx.x % kXcds, slot = blockIdx.x / kXcds;
+        const uint32_t q = ntiles / kXcds, r = ntiles % kXcds;
+        lin = xcd * q + (xcd < r ? xcd : r) + slot;
+    }
+    const uint32_t per_group = kGroupM * tiles_n;
+    const uint32_t group = lin / per_group, in_group = lin % per_group;
+    const uint32_t first_m = group * kGroupM;
+    const uint32_t gsize = (tiles_m - first_m) < kGroupM ? (tiles_m - first_m) : kGroupM;
+    const uint32_t tile_m = first_m + in_group % gsize, tile_n = in_group / gsize;
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
     int64_t oa, ob;
     batch_offsets(a, blockIdx.y, oa, ob);
