@@ -60,9 +60,9 @@ def micro_bench(iters=20):
     n = 8192
     a = be.from_numpy(rng.standard_normal((n, n), dtype=np.float32))
     b = be.from_numpy(rng.standard_normal((n, n), dtype=np.float32))
-    run("add_f32_8192x8192", A.K_ELEMENTWISE, lambda: be.add(a, b), "GB/s")
-    run("mul_f32_8192x8192", A.K_ELEMENTWISE, lambda: be.mul(a, b), "GB/s")
-    run("exp_f32_8192x8192", A.K_ELEMENTWISE, lambda: be.exp(a), "GB/s")
+    run("add_f32_8192x8192", A.K_ELEMENTWISE, lambda: be.realize(be.add(a, b)), "GB/s")
+    run("mul_f32_8192x8192", A.K_ELEMENTWISE, lambda: be.realize(be.mul(a, b)), "GB/s")
+    run("exp_f32_8192x8192", A.K_ELEMENTWISE, lambda: be.realize(be.exp(a)), "GB/s")
     del a, b
     r = be.from_numpy(rng.standard_normal((4096, n), dtype=np.float32))
     run("sum_last_4096x8192", A.K_REDUCE, lambda: be.sum(r), "GB/s")

@@ -136,6 +136,11 @@ class Backend:
         self._check(self._lib.cg_pool_stats(self._b, C.byref(u), C.byref(c)))
         return int(u.value), int(c.value)
 
+    def realize(self, x: "Tensor") -> "Tensor":
+        """Queue the computation of a lazily evaluated element-wise result now."""
+        self._check(self._lib.cg_realize(self._b, x._h))
+        return x
+
     def profile_enable(self, cls: int, sample_every: int = 1):
         """Time every `sample_every`-th launch of a kernel class with HIP events (0: off)."""
         self._check(self._lib.cg_profile_enable(self._b, cls, sample_every))

@@ -71,6 +71,7 @@ struct cg_backend {
     uint32_t *flag_dev = nullptr;   // 4-byte scratch for to_bool / compare
     uint32_t *flag_host = nullptr;  // pinned landing zone for it
     std::string name;
+    bool fuse = true; // defer element-wise ops and fuse them (CG_FUSE=0 switches it off)
     cg::ProfClass prof[CG_K_CLASSES];
     std::vector<cg::ProfPending> prof_pending;
     std::vector<std::pair<hipEvent_t, hipEvent_t>> prof_free;
@@ -87,6 +88,10 @@ struct Buffer {
 
 } // namespace cg
 
+namespace cg {
+struct Pending;
+}
+
 // A strided view of a device buffer.  Strides and offset are in elements; a stride of
 // 0 is a broadcast axis.  `uniform` marks a tensor all of whose elements equal `ubits`
 // (rank-0 constants, zeros, and every view of them): such tensors own no memory until a
@@ -102,6 +107,8 @@ struct cg_tensor {
     int64_t offset = 0;
     bool uniform = false;
     uint32_t ubits = 0;
+    // A deferred element-wise result: no buffer yet, `pend` says how to compute it.
+    cg::Pending *pend = nullptr;
 };
 
 namespace cg {
@@ -153,6 +160,52 @@ struct EwGeom {
     uint64_t total;            // work items
 };
 
+// ---- deferred element-wise expressions ------------------------------------------------
+// Element-wise results are not computed when the op is issued: the handle carries a small
+// program over "leaf" views (concrete strided views or constants, all of the result's
+// shape).  A consumer that is itself element-wise splices the program into its own; a
+// reduction evaluates it while reading; anything else (matmul, concat, gather, read-back)
+// materialises it with ONE launch of the interpreter kernel.  Each element goes through
+// exactly the operations, in the order, that the separate ops would have applied, so
+// results are bit-identical to unfused execution.
+constexpr int kMaxLeaves = 8, kMaxInstr = 24, kMaxViews = kMaxLeaves + 1;
+
+struct Instr {
+    uint8_t op;      // EwOp code, | kInstrU32 when the operands are u32
+    uint8_t a, b, c; // registers: < kMaxLeaves = leaf, else kMaxLeaves + instruction index
+};
+constexpr uint8_t kInstrU32 = 0x80;
+
+struct LeafView {
+    Buffer *buf = nullptr; // retained; null for uniform leaves
+    int64_t strides[kMaxRank] = {0};
+    int64_t offset = 0;
+    bool uniform = false;
+    uint32_t ubits = 0;
+};
+
+struct Pending {
+    int nleaf = 0, ninstr = 0;
+    bool expensive = false; // holds div / pow / exp / log / sin / cos
+    LeafView leaf[kMaxLeaves];
+    Instr ins[kMaxInstr];
+    Pending() = default;
+    Pending(const Pending &o);
+    Pending &operator=(const Pending &) = delete;
+    ~Pending();
+};
+
+struct ViewDesc {
+    const int64_t *strides;
+    bool uniform;
+    uint32_t ubits;
+    const char *ptr; // device address of the view's first element (unused when uniform)
+};
+// Collapses the iteration space shared by `n` views of shape `dims` (v[0] is the output)
+// and fills geometry + operands.  keep_last_axis: never merge the last axis into the one
+// before it (reductions need it on its own).
+int plan_views(const int64_t *dims, int rank, const ViewDesc *v, int n, bool keep_last_axis, EwGeom *g, Operand *ops);
+
 // Collapses the iteration space shared by `n` views of identical shape (views[0] is
 // the output) and fills geometry + operands.  Returns CG_ERR_UNSUPPORTED when the
 // space exceeds 2^32-1 work items.
@@ -185,6 +238,11 @@ enum EwOp : int {
 
 // out = op(ins...) element-wise; all views have out's shape.  `out` may be a strided view.
 int launch_elementwise(cg_backend *be, int op, cg_dtype dt, const cg_tensor *out, const cg_tensor *const *ins, int nin);
+// Evaluates `p` for every element of shape `dims` into `out` (a dense or strided view of that shape).
+int launch_fused(cg_backend *be, const cg_tensor *out, const Pending &p);
+// Last-axis reduction of the value of `p` (shape dims/rank) into the dense tensor `out`.
+int launch_fused_reduce(cg_backend *be, int kind, bool f32, const Pending &p, const int64_t *dims, int rank,
+                        cg_tensor *out);
 int launch_arange(cg_backend *be, cg_tensor *out);
 int launch_fill_word(cg_backend *be, void *ptr, uint32_t bits);
 // out[outer, j, inner] = x[outer, idx[j], inner]

@@ -46,6 +46,74 @@ template <int VEC> __device__ __forceinline__ void store_words(const Operand &o,
 }
 
 
+// Rust `f32 as u32` (ndarray.rs:155): truncate, saturate, NaN -> 0.
+__device__ __forceinline__ uint32_t f32_as_u32(float v) {
+    if (!(v == v) || v <= 0.0f) return 0u;
+    if (v >= 4294967296.0f) return 0xFFFFFFFFu;
+    return (uint32_t)v;
+}
+
+__device__ __forceinline__ uint32_t wrapping_pow(uint32_t a, uint32_t e) {
+    uint32_t acc = 1;
+    while (e) {
+        if (e & 1) acc *= a;
+        a *= a;
+        e >>= 1;
+    }
+    return acc;
+}
+
+// One scalar application of OP on raw 32-bit words.  F = operands are f32.
+template <int OP, bool F>
+__device__ __forceinline__ uint32_t apply(uint32_t a, uint32_t b, uint32_t c, uint32_t *fault) {
+    (void)b;
+    (void)c;
+    (void)fault;
+    if constexpr (OP == kCopy) return a;
+    if constexpr (OP == kCastF2U) return f32_as_u32(asf(a));
+    if constexpr (OP == kCastU2F) return asu((float)a); // round to nearest even
+    if constexpr (OP == kWhere) return F ? (asf(a) > 0.0f ? b : c) : (a != 0 ? b : c);
+    if constexpr (F) {
+        float x = asf(a), y = asf(b);
+        if constexpr (OP == kNeg) return a ^ 0x80000000u;
+        if constexpr (OP == kSin) return asu(sinf(x));
+        if constexpr (OP == kCos) return asu(cosf(x));
+        if constexpr (OP == kExp) return asu(expf(x));
+        if constexpr (OP == kLog) return asu(logf(x));
+        if constexpr (OP == kFloor) return asu(floorf(x));
+        if constexpr (OP == kRound) return asu(rintf(x)); // ties to even (ndarray.rs:646-648)
+        if constexpr (OP == kAdd) return asu(x + y);
+        if constexpr (OP == kSub) return asu(x - y);
+        if constexpr (OP == kMul) return asu(x * y);
+        if constexpr (OP == kDiv) return asu(x / y);
+        if constexpr (OP == kPow) return asu(powf(x, y));
+        if constexpr (OP == kLt) return asu(x < y ? 1.0f : 0.0f);
+        if constexpr (OP == kGt) return asu(x > y ? 1.0f : 0.0f);
+        if constexpr (OP == kGte) return asu(x >= y ? 1.0f : 0.0f);
+        if constexpr (OP == kLte) return asu(x <= y ? 1.0f : 0.0f);
+        if constexpr (OP == kEq) return asu(x == y ? 1.0f : 0.0f);
+    } else {
+        if constexpr (OP == kNeg) return 0u - a;
+        if constexpr (OP == kAdd) return a + b;
+        if constexpr (OP == kSub) return a - b;
+        if constexpr (OP == kMul) return a * b;
+        if constexpr (OP == kDiv) {
+            if (b == 0) {
+                *fault = kFaultDivZero; // reported by the next waiting call
+                return 0u;
+            }
+            return a / b;
+        }
+        if constexpr (OP == kPow) return wrapping_pow(a, b);
+        if constexpr (OP == kLt) return a < b;
+        if constexpr (OP == kGt) return a > b;
+        if constexpr (OP == kGte) return a >= b;
+        if constexpr (OP == kLte) return a <= b;
+        if constexpr (OP == kEq) return a == b;
+    }
+    return 0u;
+}
+
 // Offset (in elements) of row `row` of a view whose outer axes are described by
 // (od, odiv, os), innermost first.
 __device__ __forceinline__ int64_t row_offset(uint32_t row, uint32_t nouter, const uint32_t *od, const FastDiv *odiv,

@@ -1,0 +1,314 @@
+// Interpreter kernels for deferred element-wise expressions (see `Pending` in common.hpp).
+//
+// A program is a short list of instructions over a register file of 32 values per
+// element: registers 0..7 are the leaves (strided views or immediates, loaded once),
+// register 8+i is the result of instruction i.  Every lane runs the same program, so the
+// register numbers and op codes are wave-uniform: the register file lives in VGPRs and is
+// indexed with scalar (uniform) indices, and the op switch is a scalar branch.  Arithmetic
+// is the same `apply<OP, F>` the single-op kernels use, applied in the same order, so a
+// fused chain is bit-identical to the chain of separate kernels — it just reads every leaf
+// once and writes once.
+//
+//   fused_kernel         value of the program -> dense or strided output      (HBM-bound:
+//                        4 B per distinct leaf element + 4 B per output element)
+//   fused_reduce_kernel  sum / max / argmax over the last axis of the value   (HBM-bound:
+//                        4 B per distinct leaf element + 4 B per row)
+#include "common.hpp"
+#include "device_utils.hpp"
+
+namespace cg {
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr float kF32Min = -3.4028234663852886e38f;
+
+typedef uint32_t regfile __attribute__((ext_vector_type(32)));
+
+struct FusedArgs {
+    EwGeom g;
+    Operand out;
+    Operand leaf[kMaxLeaves];
+    uint32_t nleaf, ninstr;
+    Instr ins[kMaxInstr];
+    uint32_t *fault;
+    // reductions only
+    uint32_t rows, n;
+};
+
+// One instruction on one element.  op is wave-uniform.
+__device__ __forceinline__ uint32_t apply_rt(uint32_t op, uint32_t a, uint32_t b, uint32_t c, uint32_t *fault) {
+#define CG_F(OP) case OP: return apply<OP, true>(a, b, c, fault);
+#define CG_U(OP) case (OP | kInstrU32): return apply<OP, false>(a, b, c, fault);
+    switch (op) {
+        CG_F(kNeg) CG_F(kSin) CG_F(kCos) CG_F(kExp) CG_F(kLog) CG_F(kFloor) CG_F(kRound)
+        CG_F(kAdd) CG_F(kSub) CG_F(kMul) CG_F(kDiv) CG_F(kPow)
+        CG_F(kLt) CG_F(kGt) CG_F(kGte) CG_F(kLte) CG_F(kEq) CG_F(kWhere) CG_F(kCastF2U)
+        CG_U(kNeg) CG_U(kAdd) CG_U(kSub) CG_U(kMul) CG_U(kDiv) CG_U(kPow)
+        CG_U(kLt) CG_U(kGt) CG_U(kGte) CG_U(kLte) CG_U(kEq) CG_U(kWhere) CG_U(kCastU2F)
+    default: return a; // kCopy
+    }
+#undef CG_F
+#undef CG_U
+}
+
+// Loads the leaves of one work item and runs the program; result in res[VEC].
+template <int VEC>
+__device__ __forceinline__ void eval_program(const FusedArgs &a, const int64_t (&off)[kMaxLeaves], uint32_t (&res)[VEC]) {
+    regfile r[VEC];
+#pragma unroll
+    for (int l = 0; l < kMaxLeaves; l++) {
+        if ((uint32_t)l < a.nleaf) {
+            uint32_t t[VEC];
+            load_words<VEC>(a.leaf[l], off[l], t);
+#pragma unroll
+            for (int j = 0; j < VEC; j++) r[j][l] = t[j];
+        }
+    }
+    uint32_t last = 0;
+    for (uint32_t i = 0; i < a.ninstr; i++) {
+        const Instr in = a.ins[i];
+        last = kMaxLeaves + i;
+#pragma unroll
+        for (int j = 0; j < VEC; j++) {
+            uint32_t x = r[j][in.a], y = r[j][in.b], z = r[j][in.c];
+            r[j][last] = apply_rt(in.op, x, y, z, a.fault);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; j++) res[j] = r[j][last];
+}
+
+template <int VEC> __global__ __launch_bounds__(kBlock) void fused_kernel(const FusedArgs a) {
+    const uint64_t v64 = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (v64 >= a.g.total) return;
+    const uint32_t v = (uint32_t)v64;
+    uint32_t row = fastdiv(v, a.g.ipr_div);
+    const int64_t e = (int64_t)(v - row * a.g.ipr) * VEC;
+    int64_t oo = e * a.out.is;
+    int64_t off[kMaxLeaves];
+#pragma unroll
+    for (int l = 0; l < kMaxLeaves; l++) off[l] = (uint32_t)l < a.nleaf ? e * a.leaf[l].is : 0;
+    for (uint32_t d = 0; d < a.g.nouter; d++) {
+        const uint32_t q = fastdiv(row, a.g.odiv[d]);
+        const int64_t i = (int64_t)(row - q * a.g.od[d]);
+        row = q;
+        oo += i * a.out.os[d];
+#pragma unroll
+        for (int l = 0; l < kMaxLeaves; l++)
+            if ((uint32_t)l < a.nleaf) off[l] += i * a.leaf[l].os[d];
+    }
+    uint32_t res[VEC];
+    eval_program<VEC>(a, off, res);
+    store_words<VEC>(a.out, oo, res);
+}
+
+// ---- reduction over the last axis of a program's value --------------------------------------
+__device__ __forceinline__ int32_t total_key(uint32_t bits) { // Rust f32::total_cmp
+    int32_t b = (int32_t)bits;
+    return b ^ (int32_t)(((uint32_t)(b >> 31)) >> 1);
+}
+
+// kind 0 sum, 1 max, 2 argmax; f32 flag picks the arithmetic.  One 64-bit accumulator serves
+// all six cases so that the kernel is not instantiated per case.
+struct RedAcc {
+    long long c;
+    __device__ static RedAcc init(int kind, bool f) {
+        RedAcc r;
+        if (kind == kSum) r.c = 0;
+        else if (kind == kMax) r.c = f ? (long long)asu(kF32Min) : 0;
+        else r.c = (long long)0x8000000000000000ll;
+        return r;
+    }
+    __device__ void take(int kind, bool f, uint32_t w, uint32_t idx) {
+        if (kind == kSum) {
+            c = f ? (long long)asu(asf((uint32_t)c) + asf(w)) : (long long)(uint32_t)((uint32_t)c + w);
+        } else if (kind == kMax) {
+            if (f) c = (long long)asu(fmaxf(asf((uint32_t)c), asf(w)));
+            else c = w > (uint32_t)c ? (long long)w : c;
+        } else {
+            int32_t key = f ? total_key(w) : (int32_t)(w ^ 0x80000000u);
+            long long p = ((long long)key << 32) | (long long)idx;
+            c = p > c ? p : c;
+        }
+    }
+    __device__ void merge(int kind, bool f, const RedAcc &o) {
+        if (kind == kSum) {
+            c = f ? (long long)asu(asf((uint32_t)c) + asf((uint32_t)o.c)) : (long long)(uint32_t)((uint32_t)c + (uint32_t)o.c);
+        } else if (kind == kMax) {
+            if (f) c = (long long)asu(fmaxf(asf((uint32_t)c), asf((uint32_t)o.c)));
+            else c = (uint32_t)o.c > (uint32_t)c ? o.c : c;
+        } else {
+            c = o.c > c ? o.c : c;
+        }
+    }
+    __device__ RedAcc shfl(int m) const {
+        RedAcc r;
+        int lo = __shfl_xor((int)(c & 0xFFFFFFFFll), m);
+        int hi = __shfl_xor((int)(c >> 32), m);
+        r.c = ((long long)hi << 32) | (long long)(uint32_t)lo;
+        return r;
+    }
+};
+
+template <int VEC, int TPR>
+__global__ __launch_bounds__(kBlock) void fused_reduce_kernel(const FusedArgs a, uint32_t *out, int kind, int f32) {
+    constexpr int RPB = kBlock / TPR;
+    const uint32_t lane = threadIdx.x % TPR;
+    const uint32_t row = blockIdx.x * RPB + threadIdx.x / TPR;
+    const bool live = row < a.rows;
+    const bool f = f32 != 0;
+    RedAcc acc = RedAcc::init(kind, f);
+    if (live) {
+        int64_t base[kMaxLeaves];
+#pragma unroll
+        for (int l = 0; l < kMaxLeaves; l++) base[l] = 0;
+        uint32_t rr = row;
+        for (uint32_t d = 0; d < a.g.nouter; d++) {
+            const uint32_t q = fastdiv(rr, a.g.odiv[d]);
+            const int64_t i = (int64_t)(rr - q * a.g.od[d]);
+            rr = q;
+#pragma unroll
+            for (int l = 0; l < kMaxLeaves; l++)
+                if ((uint32_t)l < a.nleaf) base[l] += i * a.leaf[l].os[d];
+        }
+        const uint32_t items = a.n / VEC;
+        for (uint32_t it = lane; it < items; it += TPR) {
+            int64_t off[kMaxLeaves];
+#pragma unroll
+            for (int l = 0; l < kMaxLeaves; l++)
+                off[l] = (uint32_t)l < a.nleaf ? base[l] + (int64_t)it * VEC * a.leaf[l].is : 0;
+            uint32_t res[VEC];
+            eval_program<VEC>(a, off, res);
+#pragma unroll
+            for (int j = 0; j < VEC; j++) acc.take(kind, f, res[j], it * VEC + j);
+        }
+    }
+    constexpr int W = TPR < 64 ? TPR : 64;
+#pragma unroll
+    for (int m = W / 2; m >= 1; m >>= 1) acc.merge(kind, f, acc.shfl(m));
+    if constexpr (TPR > 64) {
+        __shared__ long long part[kBlock / 64];
+        if (threadIdx.x % 64 == 0) part[threadIdx.x / 64] = acc.c;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+#pragma unroll
+            for (int w = 1; w < kBlock / 64; w++) {
+                RedAcc o;
+                o.c = part[w];
+                acc.merge(kind, f, o);
+            }
+        }
+    }
+    if (live && lane == 0) out[row] = (uint32_t)(acc.c & 0xFFFFFFFFll);
+}
+
+int fill_args(cg_backend *be, const Pending &p, const int64_t *dims, int rank, const cg_tensor *out, bool keep_last,
+              FusedArgs *a, double *leaf_bytes) {
+    memset(a, 0, sizeof *a);
+    ViewDesc v[kMaxViews];
+    int64_t out_strides[kMaxRank];
+    if (out) {
+        const void *op;
+        int rc = device_ptr(out, &op);
+        if (rc) return rc;
+        v[0].strides = out->strides;
+        v[0].uniform = false;
+        v[0].ubits = 0;
+        v[0].ptr = static_cast<const char *>(op);
+    } else { // reductions plan over the leaves only; a stand-in output keeps the planner's shape
+        int64_t s = 1;
+        for (int i = rank - 1; i >= 0; i--) {
+            out_strides[i] = s;
+            s *= dims[i];
+        }
+        v[0].strides = out_strides;
+        v[0].uniform = false;
+        v[0].ubits = 0;
+        v[0].ptr = nullptr;
+    }
+    double bytes = 0.0;
+    for (int l = 0; l < p.nleaf; l++) {
+        const LeafView &lv = p.leaf[l];
+        v[l + 1].strides = lv.strides;
+        v[l + 1].uniform = lv.uniform;
+        v[l + 1].ubits = lv.ubits;
+        v[l + 1].ptr = lv.uniform ? nullptr : static_cast<const char *>(lv.buf->ptr) + lv.offset * 4;
+        if (!lv.uniform) {
+            double n = 1.0;
+            for (int i = 0; i < rank; i++)
+                if (lv.strides[i] != 0 || dims[i] <= 1) n *= (double)dims[i];
+            bytes += 4.0 * n;
+        }
+    }
+    Operand ops[kMaxViews];
+    int rc = plan_views(dims, rank, v, p.nleaf + 1, keep_last, &a->g, ops);
+    if (rc) return rc;
+    a->out = ops[0];
+    for (int l = 0; l < p.nleaf; l++) a->leaf[l] = ops[l + 1];
+    a->nleaf = (uint32_t)p.nleaf;
+    a->ninstr = (uint32_t)p.ninstr;
+    for (int i = 0; i < p.ninstr; i++) a->ins[i] = p.ins[i];
+    a->fault = be->fault_dev;
+    *leaf_bytes = bytes;
+    return CG_OK;
+}
+
+} // namespace
+
+int launch_fused(cg_backend *be, const cg_tensor *out, const Pending &p) {
+    FusedArgs a;
+    double bytes;
+    int rc = fill_args(be, p, out->dims, out->rank, out, false, &a, &bytes);
+    if (rc) return rc;
+    if (a.g.total == 0) return CG_OK;
+    ProfScope prof(be, CG_K_ELEMENTWISE, bytes + distinct_bytes(out));
+    dim3 grid((uint32_t)((a.g.total + kBlock - 1) / kBlock)), block(kBlock);
+    if (a.g.vec == 4)
+        hipLaunchKernelGGL((fused_kernel<4>), grid, block, 0, be->stream, a);
+    else
+        hipLaunchKernelGGL((fused_kernel<1>), grid, block, 0, be->stream, a);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CG_OK : hip_fail(e, "fused element-wise launch");
+}
+
+int launch_fused_reduce(cg_backend *be, int kind, bool f32, const Pending &p, const int64_t *dims, int rank,
+                        cg_tensor *out) {
+    FusedArgs a;
+    double bytes;
+    int rc = fill_args(be, p, dims, rank, nullptr, true, &a, &bytes);
+    if (rc) return rc;
+    a.n = a.g.inner;
+    uint64_t rows = 1;
+    for (uint32_t d = 0; d < a.g.nouter; d++) rows *= a.g.od[d];
+    if (rows > 0xFFFFFFFFull) return fail(CG_ERR_UNSUPPORTED, "reduction extents above 2^32-1");
+    a.rows = (uint32_t)rows;
+    uint32_t *op = static_cast<uint32_t *>(out->buf->ptr);
+    ProfScope prof(be, CG_K_REDUCE, bytes + distinct_bytes(out));
+    uint32_t want = (a.n + 7) / 8;
+    int tpr = want <= 4 ? 4 : want <= 16 ? 16 : want <= 64 ? 64 : 256;
+    uint32_t rpb = kBlock / tpr;
+    dim3 grid((a.rows + rpb - 1) / rpb), block(kBlock);
+    const int f = f32 ? 1 : 0;
+#define CG_LAUNCH(VEC, TPR) hipLaunchKernelGGL((fused_reduce_kernel<VEC, TPR>), grid, block, 0, be->stream, a, op, kind, f)
+    if (a.g.vec == 4) {
+        switch (tpr) {
+        case 4: CG_LAUNCH(4, 4); break;
+        case 16: CG_LAUNCH(4, 16); break;
+        case 64: CG_LAUNCH(4, 64); break;
+        default: CG_LAUNCH(4, 256); break;
+        }
+    } else {
+        switch (tpr) {
+        case 4: CG_LAUNCH(1, 4); break;
+        case 16: CG_LAUNCH(1, 16); break;
+        case 64: CG_LAUNCH(1, 64); break;
+        default: CG_LAUNCH(1, 256); break;
+        }
+    }
+#undef CG_LAUNCH
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CG_OK : hip_fail(e, "fused reduction launch");
+}
+
+} // namespace cg

@@ -13,6 +13,7 @@
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <vector>
 
 namespace cg {
@@ -114,10 +115,23 @@ static void buffer_release(Buffer *b) {
     }
 }
 
+Pending::Pending(const Pending &o) : nleaf(o.nleaf), ninstr(o.ninstr), expensive(o.expensive) {
+    for (int l = 0; l < nleaf; l++) {
+        leaf[l] = o.leaf[l];
+        if (leaf[l].buf) leaf[l].buf->rc.fetch_add(1);
+    }
+    for (int i = 0; i < ninstr; i++) ins[i] = o.ins[i];
+}
+
+Pending::~Pending() {
+    for (int l = 0; l < nleaf; l++) buffer_release(leaf[l].buf);
+}
+
 void release(cg_tensor *t) {
     if (!t) return;
     if (t->rc.fetch_sub(1) == 1) {
         buffer_release(t->buf);
+        delete t->pend;
         delete t;
     }
 }
@@ -183,6 +197,7 @@ cg_tensor *new_view(const cg_tensor *t) {
 }
 
 int device_ptr(const cg_tensor *t, const void **ptr) {
+    if (t->pend) return fail(CG_ERR_ARG, "internal error: address of a deferred tensor requested");
     if (!t->buf) {
         if (!t->uniform || numel(t) == 0) {
             *ptr = nullptr;
@@ -220,21 +235,26 @@ FastDiv make_fastdiv(uint32_t d) {
     return f;
 }
 
-int plan_elementwise(const cg_tensor *const *views, int n, EwGeom *g, Operand *ops) {
-    const cg_tensor *out = views[0];
+int plan_views(const int64_t *vdims, int vrank, const ViewDesc *v, int n, bool keep_last_axis, EwGeom *g,
+               Operand *ops) {
     int r = 0;
     int64_t dims[kMaxRank];
-    int64_t st[4][kMaxRank];
-    for (int i = 0; i < out->rank; i++) {
-        if (out->dims[i] == 1) continue;
-        dims[r] = out->dims[i];
-        for (int k = 0; k < n; k++) st[k][r] = views[k]->uniform ? 0 : views[k]->strides[i];
+    int64_t st[kMaxViews][kMaxRank];
+    bool last_kept = false;
+    for (int i = 0; i < vrank; i++) {
+        const bool is_last = i == vrank - 1;
+        if (vdims[i] == 1 && !(keep_last_axis && is_last)) continue;
+        dims[r] = vdims[i];
+        for (int k = 0; k < n; k++) st[k][r] = v[k].uniform ? 0 : v[k].strides[i];
+        if (is_last) last_kept = true;
         r++;
     }
+    (void)last_kept;
     // merge axis i+1 into axis i when every operand steps through them as one run
     int w = 0;
     for (int i = 0; i < r; i++) {
-        if (w > 0) {
+        const bool protect = keep_last_axis && i == r - 1;
+        if (w > 0 && !protect) {
             bool ok = true;
             for (int k = 0; k < n && ok; k++) ok = st[k][w - 1] == st[k][i] * dims[i];
             if (ok) {
@@ -260,14 +280,9 @@ int plan_elementwise(const cg_tensor *const *views, int n, EwGeom *g, Operand *o
     for (int k = 0; k < n; k++) {
         Operand &o = ops[k];
         memset(&o, 0, sizeof o);
-        o.uniform = views[k]->uniform ? 1u : 0u;
-        o.ubits = views[k]->ubits;
-        if (!o.uniform) {
-            const void *p;
-            int rc = device_ptr(views[k], &p);
-            if (rc) return rc;
-            o.ptr = static_cast<const char *>(p);
-        }
+        o.uniform = v[k].uniform ? 1u : 0u;
+        o.ubits = v[k].ubits;
+        o.ptr = v[k].uniform ? nullptr : v[k].ptr;
         o.is = st[k][r - 1];
         for (int d = 0; d < r - 1; d++) o.os[d] = st[k][r - 2 - d];
         if (!o.uniform && o.is == 1) {
@@ -290,6 +305,23 @@ int plan_elementwise(const cg_tensor *const *views, int n, EwGeom *g, Operand *o
     if (total > 0xFFFFFFFFull) return fail(CG_ERR_UNSUPPORTED, "element-wise launch above 2^32-1 work items");
     g->total = total;
     return CG_OK;
+}
+
+int plan_elementwise(const cg_tensor *const *views, int n, EwGeom *g, Operand *ops) {
+    ViewDesc v[kMaxViews];
+    for (int k = 0; k < n; k++) {
+        v[k].strides = views[k]->strides;
+        v[k].uniform = views[k]->uniform;
+        v[k].ubits = views[k]->ubits;
+        v[k].ptr = nullptr;
+        if (!views[k]->uniform) {
+            const void *p;
+            int rc = device_ptr(views[k], &p);
+            if (rc) return rc;
+            v[k].ptr = static_cast<const char *>(p);
+        }
+    }
+    return plan_views(views[0]->dims, views[0]->rank, v, n, false, g, ops);
 }
 
 // ---- launch timing ---------------------------------------------------------------------
@@ -384,7 +416,7 @@ static int materialize(cg_backend *be, const cg_tensor *x, cg_tensor **out) {
     if (rc) return rc;
     if (numel(x) > 0) {
         const cg_tensor *ins[1] = {x};
-        rc = launch_elementwise(be, kCopy, x->dt, o, ins, 1);
+        rc = x->pend ? launch_fused(be, o, *x->pend) : launch_elementwise(be, kCopy, x->dt, o, ins, 1);
         if (rc) {
             release(o);
             return rc;
@@ -395,13 +427,14 @@ static int materialize(cg_backend *be, const cg_tensor *x, cg_tensor **out) {
 }
 
 // numpy-style "reshape without copying": new strides for `dims` if the view allows it.
-static bool try_view_reshape(const cg_tensor *x, const int64_t *dims, int rank, int64_t *strides) {
+static bool try_view_reshape(const int64_t *xdims, const int64_t *xstrides, int xrank, const int64_t *dims, int rank,
+                             int64_t *strides) {
     int64_t od[kMaxRank], os[kMaxRank];
     int on = 0;
-    for (int i = 0; i < x->rank; i++)
-        if (x->dims[i] != 1) {
-            od[on] = x->dims[i];
-            os[on] = x->strides[i];
+    for (int i = 0; i < xrank; i++)
+        if (xdims[i] != 1) {
+            od[on] = xdims[i];
+            os[on] = xstrides[i];
             on++;
         }
     int oi = 0, ni = 0;
@@ -433,6 +466,235 @@ static bool try_view_reshape(const cg_tensor *x, const int64_t *dims, int rank, 
         strides[ni] = 0;
     }
     return true;
+}
+
+// ---- deferred element-wise expressions (see common.hpp) ---------------------------------
+static bool is_expensive(int op) {
+    return op == kDiv || op == kPow || op == kExp || op == kLog || op == kSin || op == kCos;
+}
+// Cheap enough to evaluate once per consumer instead of being written out and re-read.
+static bool cheap(const Pending *p) { return !p->expensive && p->ninstr <= 4 && p->nleaf <= 3; }
+
+static void leaf_as_tensor(const Pending &p, int l, const cg_tensor *shape_of, cg_dtype dt, cg_tensor *t) {
+    const LeafView &lv = p.leaf[l];
+    t->be = shape_of->be;
+    t->buf = lv.buf;
+    t->dt = dt;
+    t->rank = shape_of->rank;
+    memcpy(t->dims, shape_of->dims, sizeof t->dims);
+    memcpy(t->strides, lv.strides, sizeof t->strides);
+    t->offset = lv.offset;
+    t->uniform = lv.uniform;
+    t->ubits = lv.ubits;
+}
+
+// Runs the program of `p` into `dst` (a dense or strided view of p's shape).  A single
+// instruction goes to the specialised single-op kernel.
+static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p) {
+    if (p.ninstr == 1) {
+        const Instr in = p.ins[0];
+        const int op = in.op & ~kInstrU32;
+        const cg_dtype dt = (in.op & kInstrU32) ? CG_U32 : CG_F32;
+        const int nin = op == kWhere ? 3 : (op >= kAdd && op <= kEq) ? 2 : 1;
+        cg_tensor tmp[3];
+        const cg_tensor *ins[3];
+        const uint8_t regs[3] = {in.a, in.b, in.c};
+        for (int k = 0; k < nin; k++) {
+            leaf_as_tensor(p, regs[k], dst, dt, &tmp[k]);
+            ins[k] = &tmp[k];
+        }
+        int rc = launch_elementwise(be, op, dt, dst, ins, nin);
+        for (int k = 0; k < nin; k++) tmp[k].buf = nullptr;
+        return rc;
+    }
+    return launch_fused(be, dst, p);
+}
+
+// Turns a deferred tensor into a concrete one, in place (every holder of the handle sees it).
+static int ensure_concrete(cg_tensor *t) {
+    if (!t->pend) return CG_OK;
+    std::lock_guard<std::mutex> lk(g_lazy_mu);
+    if (!t->pend) return CG_OK;
+    cg_backend *be = t->be;
+    hipError_t he = hipSetDevice(be->device);
+    if (he != hipSuccess) return hip_fail(he, "hipSetDevice");
+    Buffer *b = new Buffer;
+    b->be = be;
+    int rc = be->pool.alloc((size_t)numel(t) * 4, &b->ptr, &b->cls);
+    if (rc) {
+        delete b;
+        return rc;
+    }
+    cg_tensor dst;
+    dst.be = be;
+    dst.buf = b;
+    dst.dt = t->dt;
+    dst.rank = t->rank;
+    memcpy(dst.dims, t->dims, sizeof dst.dims);
+    set_row_major(&dst);
+    rc = run_pending(be, &dst, *t->pend);
+    dst.buf = nullptr;
+    if (rc) {
+        buffer_release(b);
+        return rc;
+    }
+    Pending *old = t->pend;
+    t->buf = b;
+    t->offset = 0;
+    set_row_major(t);
+    t->pend = nullptr;
+    delete old;
+    return CG_OK;
+}
+
+static bool same_leaf(const LeafView &a, const LeafView &b, const cg_tensor *shape_of) {
+    if (a.uniform != b.uniform) return false;
+    if (a.uniform) return a.ubits == b.ubits;
+    if (a.buf != b.buf || a.offset != b.offset) return false;
+    for (int i = 0; i < shape_of->rank; i++)
+        if (shape_of->dims[i] > 1 && a.strides[i] != b.strides[i]) return false;
+    return true;
+}
+
+static int add_leaf(Pending *p, const LeafView &lv, const cg_tensor *shape_of) {
+    for (int l = 0; l < p->nleaf; l++)
+        if (same_leaf(p->leaf[l], lv, shape_of)) return l;
+    p->leaf[p->nleaf] = lv;
+    if (lv.buf) lv.buf->rc.fetch_add(1);
+    return p->nleaf++;
+}
+
+// The result of applying `op` element-wise to `ins` (all of ins[0]'s shape) as a deferred
+// tensor.  Deferred inputs that this call owns alone, or that are cheap, are spliced in;
+// other deferred inputs are made concrete first so that their value is computed once.
+static int defer_elementwise(cg_backend *be, int op, cg_dtype in_dt, cg_dtype out_dt, cg_tensor *const *ins, int nin,
+                             cg_tensor **out) {
+    const cg_tensor *shape_of = ins[0];
+    if (numel(shape_of) == 0) return new_dense(be, out_dt, shape_of->dims, shape_of->rank, out);
+    bool splice[3] = {false, false, false};
+    for (int k = 0; k < nin; k++) {
+        cg_tensor *x = ins[k];
+        if (!x->pend) continue;
+        long mine = 0; // references to x that this very call consumes
+        for (int j = 0; j < nin; j++) mine += ins[j] == x;
+        if (x->rc.load() <= mine || cheap(x->pend)) {
+            splice[k] = true;
+        } else {
+            int rc = ensure_concrete(x);
+            if (rc) return rc;
+        }
+    }
+    for (;;) { // shrink until the program fits
+        int leaves = 0, instrs = 1, worst = -1;
+        for (int k = 0; k < nin; k++) {
+            bool dup = false;
+            for (int j = 0; j < k; j++) dup = dup || ins[j] == ins[k];
+            if (dup) continue;
+            if (splice[k]) {
+                leaves += ins[k]->pend->nleaf;
+                instrs += ins[k]->pend->ninstr;
+                if (worst < 0 || ins[k]->pend->ninstr > ins[worst]->pend->ninstr) worst = k;
+            } else {
+                leaves += 1;
+            }
+        }
+        if ((leaves <= kMaxLeaves && instrs <= kMaxInstr) || worst < 0) break;
+        int rc = ensure_concrete(ins[worst]);
+        if (rc) return rc;
+        for (int k = 0; k < nin; k++)
+            if (ins[k] == ins[worst]) splice[k] = false;
+    }
+    Pending *p = new Pending;
+    uint8_t reg[3] = {0, 0, 0};
+    for (int k = 0; k < nin; k++) {
+        cg_tensor *x = ins[k];
+        bool done = false;
+        for (int j = 0; j < k && !done; j++)
+            if (ins[j] == x) {
+                reg[k] = reg[j];
+                done = true;
+            }
+        if (done) continue;
+        if (splice[k] && x->pend) {
+            const Pending *src = x->pend;
+            uint8_t lmap[kMaxLeaves];
+            for (int l = 0; l < src->nleaf; l++) lmap[l] = (uint8_t)add_leaf(p, src->leaf[l], shape_of);
+            const int base = p->ninstr;
+            auto remap = [&](uint8_t r) -> uint8_t {
+                return r < kMaxLeaves ? lmap[r] : (uint8_t)(r + base);
+            };
+            for (int i = 0; i < src->ninstr; i++) {
+                Instr in = src->ins[i];
+                const int sop = in.op & ~kInstrU32;
+                const int snin = sop == kWhere ? 3 : (sop >= kAdd && sop <= kEq) ? 2 : 1;
+                in.a = remap(in.a);
+                in.b = snin > 1 ? remap(in.b) : in.a;
+                in.c = snin > 2 ? remap(in.c) : in.a;
+                p->ins[p->ninstr++] = in;
+            }
+            p->expensive = p->expensive || src->expensive;
+            reg[k] = (uint8_t)(kMaxLeaves + p->ninstr - 1);
+        } else {
+            LeafView lv;
+            lv.uniform = x->uniform;
+            lv.ubits = x->ubits;
+            if (!x->uniform) {
+                lv.buf = x->buf;
+                memcpy(lv.strides, x->strides, sizeof lv.strides);
+                lv.offset = x->offset;
+            }
+            reg[k] = (uint8_t)add_leaf(p, lv, shape_of);
+        }
+    }
+    Instr in;
+    in.op = (uint8_t)(op | (in_dt == CG_U32 ? kInstrU32 : 0));
+    in.a = reg[0];
+    in.b = nin > 1 ? reg[1] : reg[0];
+    in.c = nin > 2 ? reg[2] : reg[0];
+    p->ins[p->ninstr++] = in;
+    p->expensive = p->expensive || is_expensive(op);
+    cg_tensor *t = new cg_tensor;
+    t->be = be;
+    t->dt = out_dt;
+    t->rank = shape_of->rank;
+    memcpy(t->dims, shape_of->dims, sizeof t->dims);
+    set_row_major(t);
+    t->pend = p;
+    *out = t;
+    return CG_OK;
+}
+
+// A view of a deferred tensor is the same program over re-strided leaves.  `fn` rewrites
+// one leaf (strides/offset) for the new shape; returns false when that leaf cannot be
+// viewed that way (then the tensor is made concrete and the caller takes the normal path).
+template <class F>
+static int pending_view(cg_tensor *x, const int64_t *dims, int rank, F &&fn, cg_tensor **out, bool *handled) {
+    *handled = false;
+    if (!x->pend) return CG_OK;
+    int64_t n = 1;
+    for (int i = 0; i < rank; i++) n *= dims[i];
+    const bool grows = n > numel(x);
+    if ((x->rc.load() > 1 && !cheap(x->pend)) || (grows && x->pend->expensive && n > 65536) || n == 0) {
+        return ensure_concrete(x); // compute once, then view the buffer
+    }
+    Pending *p = new Pending(*x->pend);
+    for (int l = 0; l < p->nleaf; l++) {
+        if (p->leaf[l].uniform) continue;
+        if (!fn(p->leaf[l])) {
+            delete p;
+            return ensure_concrete(x);
+        }
+    }
+    cg_tensor *t = new cg_tensor;
+    t->be = x->be;
+    t->dt = x->dt;
+    t->rank = rank;
+    for (int i = 0; i < rank; i++) t->dims[i] = dims[i];
+    set_row_major(t);
+    t->pend = p;
+    *out = t;
+    *handled = true;
+    return CG_OK;
 }
 
 static uint32_t f32_as_u32_host(float v) { // Rust `as`: saturating, NaN -> 0
@@ -527,8 +789,11 @@ int cg_backend_create(int device, cg_backend **out) {
     CG_HIP(hipHostGetDevicePointer((void **)&b->fault_dev, b->fault_host, 0));
     CG_HIP(hipHostMalloc((void **)&b->flag_host, 64, hipHostMallocDefault));
     CG_HIP(hipMalloc((void **)&b->flag_dev, 64));
+    const char *fuse = getenv("CG_FUSE"); // CG_FUSE=0: run every element-wise op as its own kernel
+    b->fuse = !(fuse && fuse[0] == '0');
     char name[256];
-    snprintf(name, sizeof name, "hip:%s (%s, %d CUs)", prop.gcnArchName, prop.name, prop.multiProcessorCount);
+    snprintf(name, sizeof name, "hip:%s (%s, %d CUs)%s", prop.gcnArchName, prop.name, prop.multiProcessorCount,
+             b->fuse ? "" : " [unfused]");
     b->name = name;
     *out = b;
     return CG_OK;
@@ -578,6 +843,11 @@ int cg_profile_enable(cg_backend *b, cg_kernel_class cls, unsigned sample_every)
     return CG_OK;
 }
 
+int cg_realize(cg_backend *b, cg_tensor *t) {
+    if (!b || !t) return fail(CG_ERR_ARG, "null argument");
+    return ensure_concrete(t);
+}
+
 int cg_profile_read(cg_backend *b, cg_kernel_class cls, uint64_t *launches, double *milliseconds, double *work,
                     int reset) {
     if (!b || (int)cls < 0 || (int)cls >= CG_K_CLASSES) return fail(CG_ERR_ARG, "bad profile class");
@@ -605,7 +875,10 @@ void cg_tensor_shape(const cg_tensor *t, size_t *dims) {
 }
 cg_dtype cg_tensor_dtype(const cg_tensor *t) { return t->dt; }
 size_t cg_tensor_numel(const cg_tensor *t) { return (size_t)numel(t); }
-int cg_tensor_is_contiguous(const cg_tensor *t) { return (t->uniform && numel(t) > 1) ? 0 : (is_contiguous(t) ? 1 : 0); }
+int cg_tensor_is_contiguous(const cg_tensor *t) {
+    if (t->pend) return 1; // a deferred result is row-major once computed
+    return (t->uniform && numel(t) > 1) ? 0 : (is_contiguous(t) ? 1 : 0);
+}
 
 // ---- creation --------------------------------------------------------------------------
 static int check_dims(const size_t *dims, size_t rank, int64_t *d64) {
@@ -685,6 +958,10 @@ int cg_arange(cg_backend *b, size_t end, cg_tensor **out) {
 // ---- read-back -----------------------------------------------------------------------------
 static int copy_out(cg_backend *b, const cg_tensor *t, void *dst, size_t len) {
     if (len == 0) return wait_and_check(b);
+    if (t->pend) {
+        int rc = ensure_concrete(const_cast<cg_tensor *>(t));
+        if (rc) return rc;
+    }
     if (t->uniform) {
         uint32_t *d = static_cast<uint32_t *>(dst);
         for (size_t i = 0; i < len; i++) d[i] = t->ubits;
@@ -736,7 +1013,9 @@ int cg_to_bool(cg_backend *b, const cg_tensor *t, int *out) {
         *out = t->dt == CG_F32 ? bits_f(t->ubits) > 0.0f : t->ubits != 0;
         return wait_and_check(b);
     }
-    int rc = launch_any_positive(b, t);
+    int rc = ensure_concrete(const_cast<cg_tensor *>(t));
+    if (rc) return rc;
+    rc = launch_any_positive(b, t);
     if (rc) return rc;
     return read_flag(b, out);
 }
@@ -755,7 +1034,9 @@ int cg_compare(cg_backend *b, const cg_tensor *x, const cg_tensor *y, int *out) 
         *out = 1;
         return wait_and_check(b);
     }
-    int rc = launch_any_diff(b, x, y);
+    int rc = ensure_concrete(const_cast<cg_tensor *>(x));
+    if (!rc) rc = ensure_concrete(const_cast<cg_tensor *>(y));
+    if (!rc) rc = launch_any_diff(b, x, y);
     if (rc) return rc;
     int diff = 0;
     rc = read_flag(b, &diff);
@@ -791,6 +1072,7 @@ int cg_format_tensor(cg_backend *b, const cg_tensor *t, char *buf, size_t cap) {
 // ---- element-wise ------------------------------------------------------------------------------
 static int ew_result(cg_backend *b, int op, cg_dtype compute_dt, cg_dtype out_dt, const cg_tensor *shape_of,
                      const cg_tensor *const *ins, int nin, cg_tensor **out) {
+    if (b->fuse) return defer_elementwise(b, op, compute_dt, out_dt, const_cast<cg_tensor *const *>(ins), nin, out);
     cg_tensor *o;
     int rc = new_dense(b, out_dt, shape_of->dims, shape_of->rank, &o);
     if (rc) return rc;
@@ -899,8 +1181,11 @@ int cg_matmul(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **out) {
     od[r - 2] = x->dims[r - 2];
     od[r - 1] = y->dims[r - 1];
     CG_HIP(hipSetDevice(b->device));
+    int rc = ensure_concrete(x);
+    if (!rc) rc = ensure_concrete(y);
+    if (rc) return rc;
     cg_tensor *o;
-    int rc = new_dense(b, x->dt, od, r, &o);
+    rc = new_dense(b, x->dt, od, r, &o);
     if (rc) return rc;
     if (numel(o) > 0) {
         rc = launch_matmul(b, x, y, o);
@@ -928,7 +1213,12 @@ static int reduce_entry(cg_backend *b, int kind, const char *what, cg_tensor *x,
     int rc = new_dense(b, kind == kArgmax ? CG_U32 : x->dt, od, x->rank, &o);
     if (rc) return rc;
     if (numel(o) > 0) {
-        rc = launch_reduce(b, kind, x, o);
+        if (x->pend && (x->rc.load() == 1 || cheap(x->pend))) {
+            rc = launch_fused_reduce(b, kind, x->dt == CG_F32, *x->pend, x->dims, x->rank, o);
+        } else {
+            rc = ensure_concrete(x);
+            if (!rc) rc = launch_reduce(b, kind, x, o);
+        }
         if (rc) {
             release(o);
             return rc;
@@ -960,7 +1250,9 @@ int cg_topk(cg_backend *b, cg_tensor *x, size_t k, cg_tensor **values, cg_tensor
     od[x->rank - 1] = (int64_t)k;
     CG_HIP(hipSetDevice(b->device));
     cg_tensor *v, *i;
-    int rc = new_dense(b, CG_F32, od, x->rank, &v);
+    int rc = ensure_concrete(x);
+    if (rc) return rc;
+    rc = new_dense(b, CG_F32, od, x->rank, &v);
     if (rc) return rc;
     rc = new_dense(b, CG_U32, od, x->rank, &i);
     if (rc) {
@@ -995,6 +1287,19 @@ int cg_broadcast(cg_backend *b, cg_tensor *x, const size_t *dims, size_t rank, c
         if (x->dims[i] != d[i + shift] && x->dims[i] != 1)
             return fail(CG_ERR_SHAPE, "broadcast: incompatible shape (axis %d: %lld -> %lld)", i, (long long)x->dims[i],
                         (long long)d[i + shift]);
+    if (x->pend) {
+        bool handled;
+        rc = pending_view(x, d, (int)rank, [&](LeafView &lv) {
+            int64_t ns[kMaxRank];
+            for (int i = 0; i < (int)rank; i++) {
+                int j = i - shift;
+                ns[i] = (j >= 0 && x->dims[j] == d[i]) ? lv.strides[j] : 0;
+            }
+            memcpy(lv.strides, ns, sizeof(int64_t) * rank);
+            return true;
+        }, out, &handled);
+        if (rc || handled) return rc;
+    }
     cg_tensor *v = new_view(x);
     v->rank = (int)rank;
     for (int i = 0; i < (int)rank; i++) {
@@ -1017,6 +1322,17 @@ int cg_reshape(cg_backend *b, cg_tensor *x, const size_t *dims, size_t rank, cg_
     int64_t n = 1;
     for (size_t i = 0; i < rank; i++) n *= d[i];
     if (n != numel(x)) return fail(CG_ERR_SHAPE, "reshape: element count mismatch");
+    if (x->pend) {
+        bool handled;
+        rc = pending_view(x, d, (int)rank, [&](LeafView &lv) {
+            int64_t ns[kMaxRank];
+            if (!try_view_reshape(x->dims, lv.strides, x->rank, d, (int)rank, ns)) return false;
+            memset(lv.strides, 0, sizeof lv.strides);
+            memcpy(lv.strides, ns, sizeof(int64_t) * rank);
+            return true;
+        }, out, &handled);
+        if (rc || handled) return rc;
+    }
     if (n == 0 || x->uniform) {
         cg_tensor *v = new_view(x);
         v->rank = (int)rank;
@@ -1029,7 +1345,7 @@ int cg_reshape(cg_backend *b, cg_tensor *x, const size_t *dims, size_t rank, cg_
         return CG_OK;
     }
     int64_t st[kMaxRank];
-    if (try_view_reshape(x, d, (int)rank, st)) {
+    if (try_view_reshape(x->dims, x->strides, x->rank, d, (int)rank, st)) {
         cg_tensor *v = new_view(x);
         v->rank = (int)rank;
         for (size_t i = 0; i < rank; i++) {
@@ -1056,6 +1372,17 @@ int cg_transpose(cg_backend *b, cg_tensor *x, size_t dim0, size_t dim1, cg_tenso
     if (!b || !x || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
     if (dim0 >= (size_t)x->rank || dim1 >= (size_t)x->rank) return fail(CG_ERR_RANGE, "transpose: axis out of range");
+    if (x->pend) {
+        int64_t nd[kMaxRank];
+        memcpy(nd, x->dims, sizeof nd);
+        std::swap(nd[dim0], nd[dim1]);
+        bool handled;
+        int rc = pending_view(x, nd, x->rank, [&](LeafView &lv) {
+            std::swap(lv.strides[dim0], lv.strides[dim1]);
+            return true;
+        }, out, &handled);
+        if (rc || handled) return rc;
+    }
     cg_tensor *v = new_view(x);
     std::swap(v->dims[dim0], v->dims[dim1]);
     std::swap(v->strides[dim0], v->strides[dim1]);
@@ -1071,6 +1398,17 @@ int cg_slice(cg_backend *b, cg_tensor *x, size_t dim, size_t start, size_t len, 
     if (dim >= (size_t)x->rank) return fail(CG_ERR_RANGE, "slice: axis out of range");
     if ((int64_t)start > x->dims[dim] || (int64_t)len > x->dims[dim] - (int64_t)start)
         return fail(CG_ERR_RANGE, "slice: range out of bounds");
+    if (x->pend) {
+        int64_t nd[kMaxRank];
+        memcpy(nd, x->dims, sizeof nd);
+        nd[dim] = (int64_t)len;
+        bool handled;
+        int rc = pending_view(x, nd, x->rank, [&](LeafView &lv) {
+            lv.offset += (int64_t)start * lv.strides[dim];
+            return true;
+        }, out, &handled);
+        if (rc || handled) return rc;
+    }
     cg_tensor *v = new_view(x);
     v->dims[dim] = (int64_t)len;
     v->offset += (int64_t)start * x->strides[dim];
@@ -1125,7 +1463,9 @@ int cg_concat(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor *
         }
         tail.offset = nx;
         const cg_tensor *ins[1] = {y};
-        int rc = launch_elementwise(b, kCopy, x->dt, &tail, ins, 1);
+        int rc = CG_OK;
+        if (y->pend && y->rc.load() > 1 && !cheap(y->pend)) rc = ensure_concrete(y);
+        if (!rc) rc = y->pend ? run_pending(b, &tail, *y->pend) : launch_elementwise(b, kCopy, x->dt, &tail, ins, 1);
         tail.buf = nullptr;
         if (rc) return rc;
         x->dims[dim] = od[dim];
@@ -1152,7 +1492,9 @@ int cg_concat(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor *
             memcpy(half.strides, o->strides, sizeof half.strides);
             half.offset = at * o->strides[dim];
             const cg_tensor *ins[1] = {src};
-            rc = launch_elementwise(b, kCopy, o->dt, &half, ins, 1);
+            if (src->pend && src->rc.load() > 1 && !cheap(src->pend)) rc = ensure_concrete(const_cast<cg_tensor *>(src));
+            // a deferred operand is evaluated straight into its half of the result
+            if (!rc) rc = src->pend ? run_pending(b, &half, *src->pend) : launch_elementwise(b, kCopy, o->dt, &half, ins, 1);
         }
         at += src->dims[dim];
     }
@@ -1188,7 +1530,9 @@ int cg_index(cg_backend *b, cg_tensor *x, size_t dim, cg_tensor *indices, cg_ten
         // the gather kernel wants a row-major source and a 1-D index vector
         cg_tensor *xs = nullptr, *is = nullptr;
         const cg_tensor *src = x, *idx = indices;
-        if (!is_contiguous(x) || x->uniform) {
+        rc = ensure_concrete(x);
+        if (!rc) rc = ensure_concrete(indices);
+        if (!rc && (!is_contiguous(x) || x->uniform)) {
             rc = materialize(b, x, &xs);
             src = xs;
         }

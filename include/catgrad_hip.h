@@ -124,6 +124,10 @@ typedef enum cg_kernel_class {
     CG_K_CLASSES = 6
 } cg_kernel_class;
 int cg_profile_enable(cg_backend *b, cg_kernel_class cls, unsigned sample_every);
+/* Element-wise results are computed lazily (fused into their consumer); cg_realize queues
+ * the computation of `t` now, as any non-element-wise consumer or read-back would.
+ * Borrows `t`.  Used by the op micro-benchmarks to time a single op. */
+int cg_realize(cg_backend *b, cg_tensor *t);
 int cg_profile_read(cg_backend *b, cg_kernel_class cls, uint64_t *launches, double *milliseconds, double *work,
                     int reset);
 
