@@ -238,6 +238,8 @@ enum EwOp : int {
 
 // out = op(ins...) element-wise; all views have out's shape.  `out` may be a strided view.
 int launch_elementwise(cg_backend *be, int op, cg_dtype dt, const cg_tensor *out, const cg_tensor *const *ins, int nin);
+// True when the program of `p` can be register-allocated for the interpreter kernels.
+bool fused_program_fits(const Pending &p);
 // Evaluates `p` for every element of shape `dims` into `out` (a dense or strided view of that shape).
 int launch_fused(cg_backend *be, const cg_tensor *out, const Pending &p);
 // Last-axis reduction of the value of `p` (shape dims/rank) into the dense tensor `out`.

@@ -1,8 +1,8 @@
 // Interpreter kernels for deferred element-wise expressions (see `Pending` in common.hpp).
 //
-// A program is a short list of instructions over a register file of 32 values per
-// element: registers 0..7 are the leaves (strided views or immediates, loaded once),
-// register 8+i is the result of instruction i.  Every lane runs the same program, so the
+// A program is a short list of instructions over a register file of 16 values per
+// element: the leaves (strided views or immediates, loaded once) occupy the first
+// registers, every instruction names its destination (allocated on the host).  Every lane runs the same program, so the
 // register numbers and op codes are wave-uniform: the register file lives in VGPRs and is
 // indexed with scalar (uniform) indices, and the op switch is a scalar branch.  Arithmetic
 // is the same `apply<OP, F>` the single-op kernels use, applied in the same order, so a
@@ -23,37 +23,62 @@ namespace {
 constexpr int kBlock = 256;
 constexpr float kF32Min = -3.4028234663852886e38f;
 
-typedef uint32_t regfile __attribute__((ext_vector_type(32)));
+typedef uint32_t regfile __attribute__((ext_vector_type(16)));
+
+// Program after register allocation: leaves sit in registers 0..nleaf-1, each instruction
+// names its destination.
+struct PInstr {
+    uint8_t op, a, b, c, dst, pad[3];
+};
 
 struct FusedArgs {
     EwGeom g;
     Operand out;
     Operand leaf[kMaxLeaves];
     uint32_t nleaf, ninstr;
-    Instr ins[kMaxInstr];
+    PInstr ins[kMaxInstr];
     uint32_t *fault;
     // reductions only
     uint32_t rows, n;
 };
 
-// One instruction on one element.  op is wave-uniform.
-__device__ __forceinline__ uint32_t apply_rt(uint32_t op, uint32_t a, uint32_t b, uint32_t c, uint32_t *fault) {
-#define CG_F(OP) case OP: return apply<OP, true>(a, b, c, fault);
-#define CG_U(OP) case (OP | kInstrU32): return apply<OP, false>(a, b, c, fault);
+// One instruction on the VEC elements of a work item.  op is wave-uniform, so the switch is
+// a scalar branch, and the VEC applications inside a case are independent (they interleave
+// in the pipeline).  FULL adds the long routines (sin, cos, log, pow, u32 pow); programs
+// without them run the lean instantiation, which needs fewer registers and less code.
+template <int VEC, bool FULL>
+__device__ __forceinline__ void apply_rt(uint32_t op, const uint32_t (&x)[VEC], const uint32_t (&y)[VEC],
+                                         const uint32_t (&z)[VEC], uint32_t (&o)[VEC], uint32_t *fault) {
+#define CG_CASE(CODE, OP, F)                                                        \
+    case CODE:                                                                      \
+        _Pragma("unroll") for (int j = 0; j < VEC; j++) o[j] = apply<OP, F>(x[j], y[j], z[j], fault); \
+        return;
+#define CG_F(OP) CG_CASE(OP, OP, true)
+#define CG_U(OP) CG_CASE((OP | kInstrU32), OP, false)
+    if (FULL) {
+        switch (op) {
+            CG_F(kSin) CG_F(kCos) CG_F(kLog) CG_F(kPow) CG_U(kPow)
+        default: break;
+        }
+    }
     switch (op) {
-        CG_F(kNeg) CG_F(kSin) CG_F(kCos) CG_F(kExp) CG_F(kLog) CG_F(kFloor) CG_F(kRound)
-        CG_F(kAdd) CG_F(kSub) CG_F(kMul) CG_F(kDiv) CG_F(kPow)
+        CG_F(kNeg) CG_F(kExp) CG_F(kFloor) CG_F(kRound)
+        CG_F(kAdd) CG_F(kSub) CG_F(kMul) CG_F(kDiv)
         CG_F(kLt) CG_F(kGt) CG_F(kGte) CG_F(kLte) CG_F(kEq) CG_F(kWhere) CG_F(kCastF2U)
-        CG_U(kNeg) CG_U(kAdd) CG_U(kSub) CG_U(kMul) CG_U(kDiv) CG_U(kPow)
+        CG_U(kNeg) CG_U(kAdd) CG_U(kSub) CG_U(kMul) CG_U(kDiv)
         CG_U(kLt) CG_U(kGt) CG_U(kGte) CG_U(kLte) CG_U(kEq) CG_U(kWhere) CG_U(kCastU2F)
-    default: return a; // kCopy
+    default:
+#pragma unroll
+        for (int j = 0; j < VEC; j++) o[j] = x[j]; // kCopy
+        return;
     }
 #undef CG_F
 #undef CG_U
+#undef CG_CASE
 }
 
 // Loads the leaves of one work item and runs the program; result in res[VEC].
-template <int VEC>
+template <int VEC, bool FULL>
 __device__ __forceinline__ void eval_program(const FusedArgs &a, const int64_t (&off)[kMaxLeaves], uint32_t (&res)[VEC]) {
     regfile r[VEC];
 #pragma unroll
@@ -65,21 +90,27 @@ __device__ __forceinline__ void eval_program(const FusedArgs &a, const int64_t (
             for (int j = 0; j < VEC; j++) r[j][l] = t[j];
         }
     }
-    uint32_t last = 0;
+    PInstr in = a.ins[0];
     for (uint32_t i = 0; i < a.ninstr; i++) {
-        const Instr in = a.ins[i];
-        last = kMaxLeaves + i;
+        const PInstr cur = in;
+        if (i + 1 < a.ninstr) in = a.ins[i + 1]; // next instruction word on its way while this one runs
+        uint32_t x[VEC], y[VEC], z[VEC], o[VEC];
 #pragma unroll
         for (int j = 0; j < VEC; j++) {
-            uint32_t x = r[j][in.a], y = r[j][in.b], z = r[j][in.c];
-            r[j][last] = apply_rt(in.op, x, y, z, a.fault);
+            x[j] = r[j][cur.a];
+            y[j] = r[j][cur.b];
+            z[j] = r[j][cur.c];
+        }
+        apply_rt<VEC, FULL>(cur.op, x, y, z, o, a.fault);
+#pragma unroll
+        for (int j = 0; j < VEC; j++) {
+            r[j][cur.dst] = o[j];
+            res[j] = o[j];
         }
     }
-#pragma unroll
-    for (int j = 0; j < VEC; j++) res[j] = r[j][last];
 }
 
-template <int VEC> __global__ __launch_bounds__(kBlock) void fused_kernel(const FusedArgs a) {
+template <int VEC, bool FULL> __global__ __launch_bounds__(kBlock) void fused_kernel(const FusedArgs a) {
     const uint64_t v64 = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
     if (v64 >= a.g.total) return;
     const uint32_t v = (uint32_t)v64;
@@ -99,7 +130,7 @@ template <int VEC> __global__ __launch_bounds__(kBlock) void fused_kernel(const 
             if ((uint32_t)l < a.nleaf) off[l] += i * a.leaf[l].os[d];
     }
     uint32_t res[VEC];
-    eval_program<VEC>(a, off, res);
+    eval_program<VEC, FULL>(a, off, res);
     store_words<VEC>(a.out, oo, res);
 }
 
@@ -151,7 +182,7 @@ struct RedAcc {
     }
 };
 
-template <int VEC, int TPR>
+template <int VEC, int TPR, bool FULL>
 __global__ __launch_bounds__(kBlock) void fused_reduce_kernel(const FusedArgs a, uint32_t *out, int kind, int f32) {
     constexpr int RPB = kBlock / TPR;
     const uint32_t lane = threadIdx.x % TPR;
@@ -179,7 +210,7 @@ __global__ __launch_bounds__(kBlock) void fused_reduce_kernel(const FusedArgs a,
             for (int l = 0; l < kMaxLeaves; l++)
                 off[l] = (uint32_t)l < a.nleaf ? base[l] + (int64_t)it * VEC * a.leaf[l].is : 0;
             uint32_t res[VEC];
-            eval_program<VEC>(a, off, res);
+            eval_program<VEC, FULL>(a, off, res);
 #pragma unroll
             for (int j = 0; j < VEC; j++) acc.take(kind, f, res[j], it * VEC + j);
         }
@@ -203,8 +234,38 @@ __global__ __launch_bounds__(kBlock) void fused_reduce_kernel(const FusedArgs a,
     if (live && lane == 0) out[row] = (uint32_t)(acc.c & 0xFFFFFFFFll);
 }
 
+// Linear-scan register allocation over the 16-entry register file: leaves take 0..nleaf-1,
+// an instruction's destination is any register whose value has no later use (an operand's
+// own register qualifies: it is read before the result is written).  False if 16 do not suffice.
+bool allocate_registers(const Pending &p, uint8_t *phys) {
+    constexpr int kRegs = 16;
+    int last_use[kMaxLeaves + kMaxInstr];
+    for (int i = 0; i < kMaxLeaves + kMaxInstr; i++) last_use[i] = -1;
+    for (int i = 0; i < p.ninstr; i++) {
+        last_use[p.ins[i].a] = i;
+        last_use[p.ins[i].b] = i;
+        last_use[p.ins[i].c] = i;
+    }
+    if (p.ninstr > 0) last_use[kMaxLeaves + p.ninstr - 1] = p.ninstr; // the result
+    int owner[kRegs];
+    for (int r = 0; r < kRegs; r++) owner[r] = -1;
+    for (int l = 0; l < p.nleaf; l++) {
+        phys[l] = (uint8_t)l;
+        owner[l] = l;
+    }
+    for (int i = 0; i < p.ninstr; i++) {
+        int pick = -1;
+        for (int r = 0; r < kRegs && pick < 0; r++)
+            if (owner[r] < 0 || last_use[owner[r]] <= i) pick = r;
+        if (pick < 0) return false;
+        owner[pick] = kMaxLeaves + i;
+        phys[kMaxLeaves + i] = (uint8_t)pick;
+    }
+    return true;
+}
+
 int fill_args(cg_backend *be, const Pending &p, const int64_t *dims, int rank, const cg_tensor *out, bool keep_last,
-              FusedArgs *a, double *leaf_bytes) {
+              FusedArgs *a, double *leaf_bytes, bool *full) {
     memset(a, 0, sizeof *a);
     ViewDesc v[kMaxViews];
     int64_t out_strides[kMaxRank];
@@ -248,7 +309,22 @@ int fill_args(cg_backend *be, const Pending &p, const int64_t *dims, int rank, c
     for (int l = 0; l < p.nleaf; l++) a->leaf[l] = ops[l + 1];
     a->nleaf = (uint32_t)p.nleaf;
     a->ninstr = (uint32_t)p.ninstr;
-    for (int i = 0; i < p.ninstr; i++) a->ins[i] = p.ins[i];
+    uint8_t phys[kMaxLeaves + kMaxInstr];
+    if (!allocate_registers(p, phys)) return fail(CG_ERR_ARG, "internal error: fused program needs too many registers");
+    *full = false;
+    for (int i = 0; i < p.ninstr; i++) {
+        const Instr &in = p.ins[i];
+        PInstr q;
+        memset(&q, 0, sizeof q);
+        q.op = in.op;
+        q.a = phys[in.a];
+        q.b = phys[in.b];
+        q.c = phys[in.c];
+        q.dst = phys[kMaxLeaves + i];
+        a->ins[i] = q;
+        const int op = in.op & ~kInstrU32;
+        *full = *full || op == kSin || op == kCos || op == kLog || op == kPow;
+    }
     a->fault = be->fault_dev;
     *leaf_bytes = bytes;
     return CG_OK;
@@ -256,18 +332,31 @@ int fill_args(cg_backend *be, const Pending &p, const int64_t *dims, int rank, c
 
 } // namespace
 
+bool fused_program_fits(const Pending &p) {
+    uint8_t phys[kMaxLeaves + kMaxInstr];
+    return allocate_registers(p, phys);
+}
+
 int launch_fused(cg_backend *be, const cg_tensor *out, const Pending &p) {
     FusedArgs a;
     double bytes;
-    int rc = fill_args(be, p, out->dims, out->rank, out, false, &a, &bytes);
+    bool full;
+    int rc = fill_args(be, p, out->dims, out->rank, out, false, &a, &bytes, &full);
     if (rc) return rc;
     if (a.g.total == 0) return CG_OK;
     ProfScope prof(be, CG_K_ELEMENTWISE, bytes + distinct_bytes(out));
     dim3 grid((uint32_t)((a.g.total + kBlock - 1) / kBlock)), block(kBlock);
-    if (a.g.vec == 4)
-        hipLaunchKernelGGL((fused_kernel<4>), grid, block, 0, be->stream, a);
-    else
-        hipLaunchKernelGGL((fused_kernel<1>), grid, block, 0, be->stream, a);
+    if (a.g.vec == 4) {
+        if (full)
+            hipLaunchKernelGGL((fused_kernel<4, true>), grid, block, 0, be->stream, a);
+        else
+            hipLaunchKernelGGL((fused_kernel<4, false>), grid, block, 0, be->stream, a);
+    } else {
+        if (full)
+            hipLaunchKernelGGL((fused_kernel<1, true>), grid, block, 0, be->stream, a);
+        else
+            hipLaunchKernelGGL((fused_kernel<1, false>), grid, block, 0, be->stream, a);
+    }
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? CG_OK : hip_fail(e, "fused element-wise launch");
 }
@@ -276,7 +365,8 @@ int launch_fused_reduce(cg_backend *be, int kind, bool f32, const Pending &p, co
                         cg_tensor *out) {
     FusedArgs a;
     double bytes;
-    int rc = fill_args(be, p, dims, rank, nullptr, true, &a, &bytes);
+    bool full;
+    int rc = fill_args(be, p, dims, rank, nullptr, true, &a, &bytes, &full);
     if (rc) return rc;
     a.n = a.g.inner;
     uint64_t rows = 1;
@@ -290,7 +380,13 @@ int launch_fused_reduce(cg_backend *be, int kind, bool f32, const Pending &p, co
     uint32_t rpb = kBlock / tpr;
     dim3 grid((a.rows + rpb - 1) / rpb), block(kBlock);
     const int f = f32 ? 1 : 0;
-#define CG_LAUNCH(VEC, TPR) hipLaunchKernelGGL((fused_reduce_kernel<VEC, TPR>), grid, block, 0, be->stream, a, op, kind, f)
+#define CG_LAUNCH(VEC, TPR)                                                                                  \
+    do {                                                                                                     \
+        if (full)                                                                                            \
+            hipLaunchKernelGGL((fused_reduce_kernel<VEC, TPR, true>), grid, block, 0, be->stream, a, op, kind, f);  \
+        else                                                                                                 \
+            hipLaunchKernelGGL((fused_reduce_kernel<VEC, TPR, false>), grid, block, 0, be->stream, a, op, kind, f); \
+    } while (0)
     if (a.g.vec == 4) {
         switch (tpr) {
         case 4: CG_LAUNCH(4, 4); break;

@@ -653,6 +653,16 @@ static int defer_elementwise(cg_backend *be, int op, cg_dtype in_dt, cg_dtype ou
     in.c = nin > 2 ? reg[2] : reg[0];
     p->ins[p->ninstr++] = in;
     p->expensive = p->expensive || is_expensive(op);
+    if (!fused_program_fits(*p)) { // too many live values: compute the largest deferred input first and retry
+        delete p;
+        int worst = -1;
+        for (int k = 0; k < nin; k++)
+            if (ins[k]->pend && (worst < 0 || ins[k]->pend->ninstr > ins[worst]->pend->ninstr)) worst = k;
+        if (worst < 0) return fail(CG_ERR_ARG, "internal error: single instruction does not fit");
+        int rc = ensure_concrete(ins[worst]);
+        if (rc) return rc;
+        return defer_elementwise(be, op, in_dt, out_dt, ins, nin, out);
+    }
     cg_tensor *t = new cg_tensor;
     t->be = be;
     t->dt = out_dt;
