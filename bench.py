@@ -51,7 +51,7 @@ def micro_bench(iters=20):
             fn()
         n, ms, work = be.profile_read(cls, reset=True)
         be.profile_enable(cls, 0)
-        per = ms / max(n, 1) * 1e-3
+        per = max(ms / max(n, 1) * 1e-3, 1e-12)
         rate = work / max(n, 1) / per
         peak = MFMA_F32_PEAK if unit == "TFLOP/s" else HBM_PEAK
         out[name] = {"us": round(per * 1e6, 2), "achieved": round(rate / (1e12 if unit == "TFLOP/s" else 1e9), 2),
@@ -70,7 +70,7 @@ def micro_bench(iters=20):
     del r
     row = be.from_numpy(rng.standard_normal((1, n), dtype=np.float32))
     run("broadcast_1x8192_to_4096x8192_materialised", A.K_ELEMENTWISE,
-        lambda: be.reshape(be.broadcast(row, (4096, n)), (4096 * n,)), "GB/s")
+        lambda: be.realize(be.reshape(be.broadcast(row, (4096, n)), (4096 * n,))), "GB/s")
     x = be.from_numpy(rng.standard_normal((16, 1024, 1024), dtype=np.float32))
     y = be.from_numpy(rng.standard_normal((16, 1024, 1024), dtype=np.float32))
     run("bmm_f32_16x1024x1024x1024", A.K_GEMM_MFMA, lambda: be.matmul(x, y), "TFLOP/s")

@@ -109,6 +109,15 @@ struct cg_tensor {
     uint32_t ubits = 0;
     // A deferred element-wise result: no buffer yet, `pend` says how to compute it.
     cg::Pending *pend = nullptr;
+    // Split axis: logical axis `split` (extent outer * split_inner) is addressed as
+    // (i / split_inner) * split_os + (i % split_inner) * strides[split].  This is what
+    // `reshape` makes of two adjacent axes that cannot share one stride — the merged
+    // [kvH, rep] axis of repeat_kv, whose `rep` part has stride 0 — so that the batched
+    // GEMM can walk the two parts as separate batch axes instead of reading a 4x copy.
+    // Only transpose / slice (other axes) / broadcast / matmul understand it; every
+    // other consumer first turns the tensor into a plain dense one.
+    int split = -1;
+    int64_t split_inner = 0, split_os = 0;
 };
 
 namespace cg {

@@ -507,12 +507,12 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
     a.b_sk = stride(y, r - 2);
     a.b_sn = stride(y, r - 1);
 
-    // collapse the batch axes of A and B together (C is row-major, so it follows)
-    int64_t bd[kMaxRank], sa[kMaxRank], sb[kMaxRank];
+    // collapse the batch axes of A and B together (C is row-major, so it follows); a split axis of
+    // either operand contributes its two parts as separate axes
+    int64_t bd[kMaxRank + 1], sa[kMaxRank + 1], sb[kMaxRank + 1];
     int w = 0;
-    for (int i = 0; i < r - 2; i++) {
-        if (x->dims[i] == 1) continue;
-        int64_t d = x->dims[i], s1 = stride(x, i), s2 = stride(y, i);
+    auto push_axis = [&](int64_t d, int64_t s1, int64_t s2) {
+        if (d == 1) return;
         if (w > 0 && sa[w - 1] == s1 * d && sb[w - 1] == s2 * d) {
             bd[w - 1] *= d;
             sa[w - 1] = s1;
@@ -522,6 +522,17 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
             sa[w] = s1;
             sb[w] = s2;
             w++;
+        }
+    };
+    for (int i = 0; i < r - 2; i++) {
+        const int64_t d = x->dims[i], s1 = stride(x, i), s2 = stride(y, i);
+        const bool xs = x->split == i, ys = y->split == i;
+        if (xs || ys) {
+            const int64_t inner = xs ? x->split_inner : y->split_inner;
+            push_axis(d / inner, xs ? x->split_os : s1 * inner, ys ? y->split_os : s2 * inner);
+            push_axis(inner, s1, s2);
+        } else {
+            push_axis(d, s1, s2);
         }
     }
     // fold the innermost batch axis into M when B ignores it and A walks it as more rows

@@ -100,6 +100,7 @@ void Pool::stats(size_t *in_use, size_t *cached) {
 // ---- tensors ----------------------------------------------------------------------
 bool is_contiguous(const cg_tensor *t) {
     if (numel(t) == 0) return true;
+    if (t->split >= 0) return false;
     int64_t s = 1;
     for (int i = t->rank - 1; i >= 0; i--) {
         if (t->dims[i] != 1 && t->strides[i] != s) return false;
@@ -193,6 +194,9 @@ cg_tensor *new_view(const cg_tensor *t) {
     v->offset = t->offset;
     v->uniform = t->uniform;
     v->ubits = t->ubits;
+    v->split = t->split;
+    v->split_inner = t->split_inner;
+    v->split_os = t->split_os;
     return v;
 }
 
@@ -414,7 +418,41 @@ static int materialize(cg_backend *be, const cg_tensor *x, cg_tensor **out) {
     cg_tensor *o;
     int rc = new_dense(be, x->dt, x->dims, x->rank, &o);
     if (rc) return rc;
-    if (numel(x) > 0) {
+    if (numel(x) > 0 && x->split >= 0) {
+        // copy through the physical (rank + 1) shape: the split axis becomes two axes on both sides
+        cg_tensor src, dst;
+        const int a = x->split, r = x->rank;
+        src.be = dst.be = be;
+        src.buf = x->buf;
+        dst.buf = o->buf;
+        src.dt = dst.dt = x->dt;
+        src.rank = dst.rank = r + 1;
+        src.offset = x->offset;
+        for (int i = 0, j = 0; i < r; i++) {
+            if (i == a) {
+                src.dims[j] = dst.dims[j] = x->dims[i] / x->split_inner;
+                src.strides[j] = x->split_os;
+                dst.strides[j] = o->strides[i] * x->split_inner;
+                j++;
+                src.dims[j] = dst.dims[j] = x->split_inner;
+                src.strides[j] = x->strides[i];
+                dst.strides[j] = o->strides[i];
+                j++;
+            } else {
+                src.dims[j] = dst.dims[j] = x->dims[i];
+                src.strides[j] = x->strides[i];
+                dst.strides[j] = o->strides[i];
+                j++;
+            }
+        }
+        const cg_tensor *ins[1] = {&src};
+        rc = launch_elementwise(be, kCopy, x->dt, &dst, ins, 1);
+        src.buf = dst.buf = nullptr;
+        if (rc) {
+            release(o);
+            return rc;
+        }
+    } else if (numel(x) > 0) {
         const cg_tensor *ins[1] = {x};
         rc = x->pend ? launch_fused(be, o, *x->pend) : launch_elementwise(be, kCopy, x->dt, o, ins, 1);
         if (rc) {
@@ -512,6 +550,21 @@ static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p) {
 
 // Turns a deferred tensor into a concrete one, in place (every holder of the handle sees it).
 static int ensure_concrete(cg_tensor *t) {
+    if (t->split >= 0) { // a split-axis view becomes a plain dense tensor, in place
+        std::lock_guard<std::mutex> lk(g_lazy_mu);
+        if (t->split < 0) return CG_OK;
+        cg_tensor *m;
+        int rc = materialize(t->be, t, &m);
+        if (rc) return rc;
+        buffer_release(t->buf);
+        t->buf = m->buf;
+        m->buf = nullptr;
+        t->offset = 0;
+        t->split = -1;
+        set_row_major(t);
+        release(m);
+        return CG_OK;
+    }
     if (!t->pend) return CG_OK;
     std::lock_guard<std::mutex> lk(g_lazy_mu);
     if (!t->pend) return CG_OK;
@@ -574,6 +627,10 @@ static int defer_elementwise(cg_backend *be, int op, cg_dtype in_dt, cg_dtype ou
     bool splice[3] = {false, false, false};
     for (int k = 0; k < nin; k++) {
         cg_tensor *x = ins[k];
+        if (x->split >= 0) {
+            int rc = ensure_concrete(x);
+            if (rc) return rc;
+        }
         if (!x->pend) continue;
         long mine = 0; // references to x that this very call consumes
         for (int j = 0; j < nin; j++) mine += ins[j] == x;
@@ -1083,6 +1140,10 @@ int cg_format_tensor(cg_backend *b, const cg_tensor *t, char *buf, size_t cap) {
 static int ew_result(cg_backend *b, int op, cg_dtype compute_dt, cg_dtype out_dt, const cg_tensor *shape_of,
                      const cg_tensor *const *ins, int nin, cg_tensor **out) {
     if (b->fuse) return defer_elementwise(b, op, compute_dt, out_dt, const_cast<cg_tensor *const *>(ins), nin, out);
+    for (int k = 0; k < nin; k++) {
+        int erc = ensure_concrete(const_cast<cg_tensor *>(ins[k]));
+        if (erc) return erc;
+    }
     cg_tensor *o;
     int rc = new_dense(b, out_dt, shape_of->dims, shape_of->rank, &o);
     if (rc) return rc;
@@ -1191,8 +1252,13 @@ int cg_matmul(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **out) {
     od[r - 2] = x->dims[r - 2];
     od[r - 1] = y->dims[r - 1];
     CG_HIP(hipSetDevice(b->device));
-    int rc = ensure_concrete(x);
-    if (!rc) rc = ensure_concrete(y);
+    // deferred operands are computed now; a split axis may stay if it is a batch axis (the GEMM walks
+    // its two parts as separate batch axes) and the two operands do not disagree about it
+    int rc = CG_OK;
+    if (x->pend || x->split >= r - 2) rc = ensure_concrete(x);
+    if (!rc && (y->pend || y->split >= r - 2)) rc = ensure_concrete(y);
+    if (!rc && x->split >= 0 && y->split >= 0 && (x->split != y->split || x->split_inner != y->split_inner))
+        rc = ensure_concrete(y);
     if (rc) return rc;
     cg_tensor *o;
     rc = new_dense(b, x->dt, od, r, &o);
@@ -1317,6 +1383,7 @@ int cg_broadcast(cg_backend *b, cg_tensor *x, const size_t *dims, size_t rank, c
         v->dims[i] = d[i];
         v->strides[i] = (j >= 0 && x->dims[j] == d[i] && !x->uniform) ? x->strides[j] : 0;
     }
+    if (v->split >= 0) v->split += shift;
     *out = v;
     return CG_OK;
 }
@@ -1343,6 +1410,10 @@ int cg_reshape(cg_backend *b, cg_tensor *x, const size_t *dims, size_t rank, cg_
         }, out, &handled);
         if (rc || handled) return rc;
     }
+    if (x->split >= 0) {
+        rc = ensure_concrete(x);
+        if (rc) return rc;
+    }
     if (n == 0 || x->uniform) {
         cg_tensor *v = new_view(x);
         v->rank = (int)rank;
@@ -1364,6 +1435,28 @@ int cg_reshape(cg_backend *b, cg_tensor *x, const size_t *dims, size_t rank, cg_
         }
         *out = v;
         return CG_OK;
+    }
+    // Two adjacent axes that cannot share a stride but are merged by the new shape (everything else
+    // unchanged) stay a view with a split axis; this is repeat_kv's [kvH, rep] -> [kvH * rep]
+    // (catgrad-llm-models/src/helpers/tensors.rs:128-151), which then costs no copy.
+    if ((int)rank == x->rank - 1 && !x->pend) {
+        for (int a = 0; a + 1 < x->rank; a++) {
+            bool ok = d[a] == x->dims[a] * x->dims[a + 1];
+            for (int i = 0; i < a && ok; i++) ok = d[i] == x->dims[i];
+            for (int i = a + 2; i < x->rank && ok; i++) ok = d[i - 1] == x->dims[i];
+            if (!ok) continue;
+            cg_tensor *v = new_view(x);
+            v->rank = (int)rank;
+            for (int i = 0; i < (int)rank; i++) {
+                v->dims[i] = d[i];
+                v->strides[i] = i < a ? x->strides[i] : x->strides[i + 1];
+            }
+            v->split = a;
+            v->split_inner = x->dims[a + 1];
+            v->split_os = x->strides[a];
+            *out = v;
+            return CG_OK;
+        }
     }
     CG_HIP(hipSetDevice(b->device));
     cg_tensor *m;
@@ -1396,6 +1489,8 @@ int cg_transpose(cg_backend *b, cg_tensor *x, size_t dim0, size_t dim1, cg_tenso
     cg_tensor *v = new_view(x);
     std::swap(v->dims[dim0], v->dims[dim1]);
     std::swap(v->strides[dim0], v->strides[dim1]);
+    if (v->split == (int)dim0) v->split = (int)dim1;
+    else if (v->split == (int)dim1) v->split = (int)dim0;
     *out = v;
     return CG_OK;
 }
@@ -1419,6 +1514,10 @@ int cg_slice(cg_backend *b, cg_tensor *x, size_t dim, size_t start, size_t len, 
         }, out, &handled);
         if (rc || handled) return rc;
     }
+    if (x->split == (int)dim) {
+        int rc = ensure_concrete(x);
+        if (rc) return rc;
+    }
     cg_tensor *v = new_view(x);
     v->dims[dim] = (int64_t)len;
     v->offset += (int64_t)start * x->strides[dim];
@@ -1435,6 +1534,11 @@ int cg_concat(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor *
     if (x->rank != y->rank || dim >= (size_t)x->rank) return fail(CG_ERR_SHAPE, "concat: incompatible shapes");
     for (int i = 0; i < x->rank; i++)
         if ((size_t)i != dim && x->dims[i] != y->dims[i]) return fail(CG_ERR_SHAPE, "concat: incompatible shapes");
+    if (x->split >= 0 || y->split >= 0) {
+        int erc = x->split >= 0 ? ensure_concrete(x) : CG_OK;
+        if (!erc && y->split >= 0) erc = ensure_concrete(y);
+        if (erc) return erc;
+    }
     int64_t od[kMaxRank];
     memcpy(od, x->dims, sizeof od);
     od[dim] = x->dims[dim] + y->dims[dim];

@@ -357,6 +357,32 @@ def _():
     return run, expect
 
 
+@case("repeat_kv_views_through_other_ops")
+def _():
+    """reshape(broadcast(x)) that merges a stride-0 axis into its neighbour, consumed by everything
+    except matmul (which has its own cases)."""
+    x = rng(120).integers(-9, 10, size=(2, 3, 1, 5, 8)).astype(np.float32)  # integer-valued: sums are exact
+    y = rng(121).integers(-9, 10, size=(2, 12, 5, 8)).astype(np.float32)
+
+    def rep(be):
+        return be.reshape(be.broadcast(be.from_numpy(x), (2, 3, 4, 5, 8)), (2, 12, 5, 8))
+
+    def run(be):
+        ty = be.from_numpy(y)
+        return N(be, rep(be), be.transpose(rep(be), 1, 2), be.slice(rep(be), 1, 2, 7), be.slice(rep(be), 3, 1, 4),
+                 be.add(rep(be), ty), be.sum(rep(be)), be.concat(rep(be), ty, 1), be.reshape(rep(be), (24, 40)),
+                 be.max(be.transpose(rep(be), 1, 3)), be.broadcast(rep(be), (3, 2, 12, 5, 8)),
+                 be.index(rep(be), 1, be.from_numpy(np.array([11, 0, 5], np.uint32))))
+
+    def expect():
+        r = np.repeat(x[:, :, 0], 4, axis=1)
+        return [r, r.transpose(0, 2, 1, 3), r[:, 2:9], r[..., 1:5], r + y, r.sum(-1, keepdims=True),
+                np.concatenate([r, y], 1), r.reshape(24, 40), r.transpose(0, 3, 2, 1).max(-1, keepdims=True),
+                np.broadcast_to(r, (3, 2, 12, 5, 8)), r[:, [11, 0, 5]]]
+
+    return run, expect
+
+
 @case("transpose_slice_chain")
 def _():
     a = f32(36, (5, 7, 9))
@@ -653,6 +679,12 @@ _mm_case("mm_attention_context", (2, 6, 40, 56), (2, 56, 6, 32),
          lambda be, p, v: (p, be.transpose(v, 1, 2), None, None))
 _mm_case("mm_repeat_kv_rhs", (2, 6, 5, 16), (2, 2, 1, 16, 12),
          lambda be, q, kv: (q, be.reshape(be.broadcast(kv, (2, 2, 3, 16, 12)), (2, 6, 16, 12)), None, None))
+_mm_case("mm_repeat_kv_transposed_rhs", (2, 6, 5, 16), (2, 2, 1, 12, 16),
+         lambda be, q, kv: (q, be.transpose(be.reshape(be.broadcast(kv, (2, 2, 3, 12, 16)), (2, 6, 12, 16)), 2, 3),
+                            None, None))
+_mm_case("mm_repeat_kv_both_operands", (2, 2, 1, 5, 16), (2, 2, 1, 16, 12),
+         lambda be, q, kv: (be.reshape(be.broadcast(q, (2, 2, 3, 5, 16)), (2, 6, 5, 16)),
+                            be.reshape(be.broadcast(kv, (2, 2, 3, 16, 12)), (2, 6, 16, 12)), None, None))
 _mm_case("mm_transposed_lhs", (3, 64, 30), (3, 64, 20), lambda be, a, b: (be.transpose(a, 1, 2), b, None, None))
 _mm_case("mm_sliced_operands", (2, 50, 80), (2, 80, 70),
          lambda be, a, b: (be.slice(a, 2, 8, 64), be.slice(be.slice(b, 1, 8, 64), 2, 3, 33), None, None))
