@@ -55,6 +55,8 @@ class Tensor:
     # BackendTensorOps::shape (backend/mod.rs:124-126)
     @property
     def shape(self) -> tuple:
+        if self._h is None:
+            raise ValueError("use of a moved tensor")
         lib = self._be._lib
         r = lib.cg_tensor_rank(self._h)
         buf = (C.c_size_t * max(r, 1))()

@@ -79,11 +79,22 @@ struct cg_backend {
 
 namespace cg {
 
+// Row-block structure of a buffer that grows by appended rows (a KV cache): the buffer is
+// [nblocks][C][R] elements, block b holds fill[b] valid rows of R elements, rows at and
+// beyond fill[b] are free and no view covers them.  `concat` along the row axis appends
+// in place at that frontier.
+struct RowStore {
+    int64_t R = 0, C = 0, nblocks = 0;
+    std::vector<int64_t> fill;
+};
+
 struct Buffer {
     std::atomic<long> rc{1};
     void *ptr = nullptr;
     size_t cls = 0;
     cg_backend *be = nullptr;
+    RowStore *rs = nullptr;      // owned
+    Buffer *successor = nullptr; // retained: the roomier buffer that blocks of this one migrate to on append
 };
 
 } // namespace cg

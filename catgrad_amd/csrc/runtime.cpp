@@ -110,9 +110,12 @@ bool is_contiguous(const cg_tensor *t) {
 }
 
 static void buffer_release(Buffer *b) {
-    if (b && b->rc.fetch_sub(1) == 1) {
+    while (b && b->rc.fetch_sub(1) == 1) {
         if (b->ptr) b->be->pool.free(b->ptr, b->cls);
+        Buffer *next = b->successor;
+        delete b->rs;
         delete b;
+        b = next; // drop the reference this buffer held on its successor
     }
 }
 
@@ -826,6 +829,168 @@ static bool fold_binary(int op, cg_dtype dt, uint32_t a, uint32_t b, uint32_t *r
     case CG_EQ: *r = a == b; return true;
     default: return false;
     }
+}
+
+
+// ---- zero-copy concat: adjacent views, and appended rows -----------------------------------
+// concat(x, y, dim) of two views of ONE buffer where y starts exactly where x ends along `dim`
+// and all other axes are laid out alike is just the wider view.  (This is how the per-layer KV
+// entries, once they live in one row store, restack into the [L, B, kvH, T, hd] cache for free.)
+static bool try_adjacent_merge(cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor **out) {
+    if (!x->buf || x->buf != y->buf || x->uniform || y->uniform || x->split >= 0 || y->split >= 0) return false;
+    const int64_t xd = x->dims[dim], yd = y->dims[dim];
+    for (int i = 0; i < x->rank; i++) {
+        if ((size_t)i == dim) continue;
+        if (x->dims[i] > 1 && x->strides[i] != y->strides[i]) return false;
+    }
+    const int64_t gap = y->offset - x->offset;
+    int64_t sd;
+    if (xd > 1) sd = x->strides[dim];
+    else if (yd > 1) sd = y->strides[dim];
+    else sd = gap;
+    if (sd <= 0 || gap != xd * sd) return false;
+    if (xd > 1 && x->strides[dim] != sd) return false;
+    if (yd > 1 && y->strides[dim] != sd) return false;
+    cg_tensor *v = new_view(x);
+    v->dims[dim] = xd + yd;
+    v->strides[dim] = sd;
+    *out = v;
+    return true;
+}
+
+// concat(x, y, dim) that appends a few rows to every block of a blocked tensor (the KV update
+// `concat(cached [B, kvH, T, hd], new [B, kvH, s, hd], 2)`, helpers/cache.rs:30-39).  With a row
+// store behind x and x at its frontier the rows are written in place; otherwise x's blocks
+// migrate, together with the new rows, into the buffer's roomier successor (one copy per 256+
+// appended rows instead of one per append).  Returns false when the pattern does not apply.
+static bool try_row_append(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor **out, int *status) {
+    *status = CG_OK;
+    if (!x->buf || x->pend || x->uniform || x->split >= 0 || y->split >= 0 || y->uniform) return false;
+    const int r = x->rank;
+    const int64_t xd = x->dims[dim], yd = y->dims[dim];
+    if (xd <= 0 || yd <= 0 || yd * 4 > xd) return false; // append-like only
+    int64_t R = 1;
+    for (int j = r - 1; j > (int)dim; j--) { // inner axes dense row-major
+        if (x->dims[j] > 1 && x->strides[j] != R) return false;
+        R *= x->dims[j];
+    }
+    if (xd > 1 && x->strides[dim] != R) return false;
+    int64_t outer = 1, min_os = 0;
+    for (int i = 0; i < (int)dim; i++) {
+        if (x->dims[i] <= 1) continue;
+        outer *= x->dims[i];
+        if (x->strides[i] <= 0) return false;
+        if (min_os == 0 || x->strides[i] < min_os) min_os = x->strides[i];
+    }
+    if (outer <= 1 || outer > 65536 || min_os % R) return false;
+    if (numel(x) * 4 < 65536) return false; // not worth the bookkeeping
+    Buffer *src = x->buf;
+    RowStore *rs = src->rs;
+    const int64_t C = rs ? rs->C : min_os / R;
+    if (rs && rs->R != R) return false;
+    if (C < xd || x->offset % (C * R)) return false;
+    for (int i = 0; i < (int)dim; i++)
+        if (x->dims[i] > 1 && x->strides[i] % (C * R)) return false;
+    if (!rs && xd != C) return false; // a partial view of a plain buffer: its "slack" is someone's data
+    const int64_t src_blocks = (int64_t)(src->cls / 4) / (C * R);
+    // blocks touched, in row-major order of the outer index
+    std::vector<int64_t> blocks((size_t)outer);
+    {
+        int64_t idx[kMaxRank] = {0};
+        for (int64_t o = 0; o < outer; o++) {
+            int64_t off = x->offset;
+            for (int i = 0; i < (int)dim; i++) off += idx[i] * x->strides[i];
+            blocks[(size_t)o] = off / (C * R);
+            if (blocks[(size_t)o] >= (rs ? rs->nblocks : src_blocks)) return false;
+            for (int i = (int)dim - 1; i >= 0; i--) {
+                if (x->dims[i] <= 1) continue;
+                if (++idx[i] < x->dims[i]) break;
+                idx[i] = 0;
+            }
+        }
+    }
+    hipError_t he = hipSetDevice(b->device);
+    if (he != hipSuccess) {
+        *status = hip_fail(he, "hipSetDevice");
+        return true;
+    }
+    if (y->pend && y->rc.load() > 1 && !cheap(y->pend)) {
+        *status = ensure_concrete(y);
+        if (*status) return true;
+    }
+    auto write_rows = [&](Buffer *dstbuf, int64_t dC, int64_t row0, const cg_tensor *src_t) -> int {
+        // destination: the rows [row0, row0 + rows) of x's blocks inside dstbuf (block capacity dC)
+        cg_tensor dst;
+        dst.be = b;
+        dst.buf = dstbuf;
+        dst.dt = x->dt;
+        dst.rank = r;
+        memcpy(dst.dims, src_t->dims, sizeof dst.dims);
+        for (int i = 0; i < r; i++) {
+            if (i < (int)dim) dst.strides[i] = x->dims[i] > 1 ? x->strides[i] / (C * R) * (dC * R) : 0;
+            else dst.strides[i] = i == (int)dim ? R : x->strides[i];
+        }
+        dst.offset = x->offset / (C * R) * (dC * R) + row0 * R;
+        const cg_tensor *ins[1] = {src_t};
+        int rc = src_t->pend ? run_pending(b, &dst, *src_t->pend) : launch_elementwise(b, kCopy, x->dt, &dst, ins, 1);
+        dst.buf = nullptr;
+        return rc;
+    };
+    bool at_frontier = rs != nullptr && xd + yd <= C;
+    for (int64_t o = 0; o < outer && at_frontier; o++) at_frontier = rs->fill[(size_t)blocks[(size_t)o]] == xd;
+    Buffer *dstbuf = src;
+    int64_t dC = C;
+    if (at_frontier) {
+        *status = write_rows(src, C, xd, y);
+        if (*status) return true;
+        for (int64_t o = 0; o < outer; o++) rs->fill[(size_t)blocks[(size_t)o]] = xd + yd;
+    } else {
+        if (!src->successor) {
+            const int64_t nb = rs ? rs->nblocks : src_blocks;
+            int64_t grow = (xd + yd) / 8;
+            if (grow < 256) grow = 256;
+            Buffer *nbuf = new Buffer;
+            nbuf->be = b;
+            nbuf->rs = new RowStore;
+            nbuf->rs->R = R;
+            nbuf->rs->C = xd + yd + grow;
+            nbuf->rs->nblocks = nb;
+            nbuf->rs->fill.assign((size_t)nb, 0);
+            int rc = b->pool.alloc((size_t)(nb * nbuf->rs->C * R) * 4, &nbuf->ptr, &nbuf->cls);
+            if (rc) {
+                delete nbuf->rs;
+                delete nbuf;
+                *status = rc;
+                return true;
+            }
+            src->successor = nbuf;
+        }
+        dstbuf = src->successor;
+        RowStore *ds = dstbuf->rs;
+        if (ds->R != R || ds->C < xd + yd) return false;
+        for (int64_t o = 0; o < outer; o++)
+            if (ds->fill[(size_t)blocks[(size_t)o]] != 0) return false; // somebody already migrated these blocks
+        dC = ds->C;
+        *status = write_rows(dstbuf, dC, 0, x);
+        if (!*status) *status = write_rows(dstbuf, dC, xd, y);
+        if (*status) return true;
+        for (int64_t o = 0; o < outer; o++) ds->fill[(size_t)blocks[(size_t)o]] = xd + yd;
+    }
+    cg_tensor *v = new cg_tensor;
+    v->be = b;
+    v->buf = dstbuf;
+    dstbuf->rc.fetch_add(1);
+    v->dt = x->dt;
+    v->rank = r;
+    memcpy(v->dims, x->dims, sizeof v->dims);
+    v->dims[dim] = xd + yd;
+    for (int i = 0; i < r; i++) {
+        if (i < (int)dim) v->strides[i] = x->dims[i] > 1 ? x->strides[i] / (C * R) * (dC * R) : x->strides[i];
+        else v->strides[i] = i == (int)dim ? R : x->strides[i];
+    }
+    v->offset = x->offset / (C * R) * (dC * R);
+    *out = v;
+    return true;
 }
 
 } // namespace cg
@@ -1553,6 +1718,11 @@ int cg_concat(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor *
         retain(x);
         *out = x;
         return CG_OK;
+    }
+    if (try_adjacent_merge(x, y, dim, out)) return CG_OK;
+    {
+        int arc;
+        if (try_row_append(b, x, y, dim, out, &arc)) return arc;
     }
     CG_HIP(hipSetDevice(b->device));
     int64_t nx = numel(x), ny = numel(y);

@@ -483,6 +483,70 @@ def _():
                           np.concatenate([l.reshape(-1) for l in layers[:3]])])
 
 
+@case("kv_cache_growth_loop")
+def _():
+    """The KV-cache dance of helpers/cache.rs over several steps: per-layer slice + squeeze of the stacked
+    cache, concat of new rows along the sequence axis, restack along axis 0 — with operands moved as the
+    interpreter does.  Also: an earlier cache stays valid, and two different appends to the same base agree
+    with numpy (the second one must not see the first one's rows)."""
+    L, B, H, T0, D = 3, 2, 2, 64, 64
+    base = f32(130, (L, B, H, T0, D))
+    news = [[f32(131 + 10 * s + l, (B, H, 1 + (s % 2), D)) for l in range(L)] for s in range(6)]
+    fork = f32(199, (B, H, 2, D))
+
+    def run(be):
+        cache = be.from_numpy(base)
+        old = []
+        forked = None
+        for s in range(6):
+            layers = []
+            for l in range(L):
+                c = be.reshape(be.slice(cache, 0, l, 1).move(), (B, H, cache.shape[3], D))
+                if s == 2 and l == 1:
+                    forked = be.concat(c, be.from_numpy(fork).move(), 2)  # c borrowed: a second append follows
+                layers.append(be.concat(c.move(), be.from_numpy(news[s][l]).move(), 2))
+            shp = (1, B, H, layers[0].shape[2], D)
+            out = be.reshape(layers[0].move(), shp)
+            for l in range(1, L):
+                out = be.concat(out.move(), be.reshape(layers[l].move(), shp).move(), 0)
+            if s in (0, 3):
+                old.append(cache.clone())
+            cache = out
+        return N(be, cache, forked, *old)
+
+    def expect():
+        c = base
+        olds, forked = [], None
+        for s in range(6):
+            if s == 2:
+                forked = np.concatenate([c[1], fork], 2)
+            if s in (0, 3):
+                olds.append(c)
+            c = np.stack([np.concatenate([c[l], news[s][l]], 2) for l in range(L)])
+        return [c, forked, *olds]
+
+    return run, expect
+
+
+@case("concat_adjacent_views_merge")
+def _():
+    a = f32(140, (6, 4, 10))
+
+    def run(be):
+        t = be.from_numpy(a)
+        return N(be, be.concat(be.slice(t, 0, 0, 2), be.slice(t, 0, 2, 3), 0),
+                 be.concat(be.slice(t, 2, 1, 4), be.slice(t, 2, 5, 5), 2),
+                 be.concat(be.slice(t, 1, 0, 1), be.slice(t, 1, 1, 1), 1),
+                 be.concat(be.slice(t, 0, 1, 2), be.slice(t, 0, 4, 2), 0),   # not adjacent: must copy
+                 be.concat(be.slice(t, 2, 0, 5), be.slice(t, 2, 0, 5), 2))   # same view twice
+
+    def expect():
+        return [a[0:5], a[:, :, 1:10], a[:, 0:2], np.concatenate([a[1:3], a[4:6]], 0),
+                np.concatenate([a[..., :5], a[..., :5]], 2)]
+
+    return run, expect
+
+
 @case("index_gather")
 def _():
     w = f32(60, (50, 16))
