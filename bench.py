@@ -211,7 +211,7 @@ def main():
         "backend_calls": {"prefill": calls[0], "per_decode_step": round(calls[1] / max(T, 1), 1)},
         "backend": sess.backend_name,
         "roofline": {
-            "kernel": "mfma_gemm_kernel (f32 v_mfma_f32_32x32x2, 128x128x16 tiles)",
+            "kernel": "mfma_gemm_kernel (f32 v_mfma_f32_32x32x2, 128x128x32 tiles)",
             "bound": "mfma", "achieved": round(mfma_rate / 1e12, 3), "peak": MFMA_F32_PEAK / 1e12, "unit": "TFLOP/s",
             "frac": round(mfma_rate / MFMA_F32_PEAK, 4), "traffic": None,
             "launches_timed": n_m, "avg_launch_ms": round(ms_m / max(n_m, 1), 4),

@@ -206,7 +206,7 @@ struct LeafView {
 
 struct Pending {
     int nleaf = 0, ninstr = 0;
-    bool expensive = false; // holds div / pow / exp / log / sin / cos
+    bool expensive = false; // holds pow / exp / log / sin / cos
     LeafView leaf[kMaxLeaves];
     Instr ins[kMaxInstr];
     Pending() = default;
@@ -224,7 +224,8 @@ struct ViewDesc {
 // Collapses the iteration space shared by `n` views of shape `dims` (v[0] is the output)
 // and fills geometry + operands.  keep_last_axis: never merge the last axis into the one
 // before it (reductions need it on its own).
-int plan_views(const int64_t *dims, int rank, const ViewDesc *v, int n, bool keep_last_axis, EwGeom *g, Operand *ops);
+int plan_views(const int64_t *dims, int rank, const ViewDesc *v, int n, bool keep_last_axis, EwGeom *g, Operand *ops,
+               bool allow_vec4 = true);
 
 // Collapses the iteration space shared by `n` views of identical shape (views[0] is
 // the output) and fills geometry + operands.  Returns CG_ERR_UNSUPPORTED when the

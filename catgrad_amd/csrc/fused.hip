@@ -303,7 +303,11 @@ int fill_args(cg_backend *be, const Pending &p, const int64_t *dims, int rank, c
         }
     }
     Operand ops[kMaxViews];
-    int rc = plan_views(dims, rank, v, p.nleaf + 1, keep_last, &a->g, ops);
+    // Small problems are latency-bound: one element per lane keeps each lane's serial chain
+    // (operand moves, long routines) four times shorter and still fills the chip.
+    int64_t elems = 1;
+    for (int i = 0; i < rank; i++) elems *= dims[i];
+    int rc = plan_views(dims, rank, v, p.nleaf + 1, keep_last, &a->g, ops, keep_last || elems > 32768);
     if (rc) return rc;
     a->out = ops[0];
     for (int l = 0; l < p.nleaf; l++) a->leaf[l] = ops[l + 1];

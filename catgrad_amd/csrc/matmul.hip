@@ -63,21 +63,24 @@ __device__ __forceinline__ void batch_offsets(const MmArgs &a, uint32_t b, int64
 // ------------------------------------------------------------------------------------------
 // MFMA kernel
 // ------------------------------------------------------------------------------------------
-constexpr int BM = 128, BN = 128, BK = 16;
-constexpr int PITCH = BK + 4; // words per LDS row
+constexpr int BM = 128, BN = 128, BK = 32;
+constexpr int PITCH = BK + 4; // words per LDS row: row r starts at bank 4r mod 32
+constexpr int kSlots = BM * BK / 4 / 256; // 16-byte slots of a tile per thread
+constexpr size_t kGemmLdsBytes = 2 * (BM + BN) * PITCH * sizeof(float);
 constexpr int kThreads = 256;
 constexpr uint32_t kXcds = 8, kGroupM = 8;
 
 typedef float float4v __attribute__((ext_vector_type(4)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 
-// Loads one 128 x 16 tile (rows along `R` with stride s_r, k with stride s_k) into
-// registers: 2 x float4 per thread.  Layout of the 512 float4 slots of a tile:
-//   K-contiguous source (s_k == 1): slot = row*4 + kq      (float4 along k)
-//   R-contiguous source (s_r == 1): slot = k*32 + rq       (float4 along rows)
+// Loads one 128 x BK tile (rows along `R` with stride s_r, k with stride s_k) into
+// registers: kSlots x float4 per thread.  Layout of the float4 slots of a tile:
+//   K-contiguous source (s_k == 1): slot = row*(BK/4) + kq  (float4 along k; 8 lanes read
+//                                                            128 contiguous bytes of a row)
+//   R-contiguous source (s_r == 1): slot = k*32 + rq        (float4 along rows)
 //   otherwise                      : as K-contiguous, element by element
 struct TileRegs {
-    float4v v[2];
+    float4v v[kSlots];
 };
 
 __device__ __forceinline__ float ld_guard(const uint32_t *p, bool ok) { return ok ? asf(*p) : 0.0f; }
@@ -86,10 +89,10 @@ template <bool ROWS_FAST>
 __device__ __forceinline__ void load_tile(TileRegs &t, const uint32_t *base, int64_t s_r, int64_t s_k, uint32_t r0,
                                           uint32_t k0, uint32_t R, uint32_t K, bool vec_ok) {
 #pragma unroll
-    for (int h = 0; h < 2; h++) {
+    for (int h = 0; h < kSlots; h++) {
         uint32_t slot = threadIdx.x + h * kThreads;
         if (!ROWS_FAST) {
-            uint32_t row = r0 + slot / 4, k = k0 + (slot % 4) * 4;
+            uint32_t row = r0 + slot / (BK / 4), k = k0 + (slot % (BK / 4)) * 4;
             const uint32_t *p = base + (int64_t)row * s_r + (int64_t)k * s_k;
             if (vec_ok && row < R && k + 3 < K) {
                 t.v[h] = *reinterpret_cast<const float4v *>(p);
@@ -119,10 +122,10 @@ __device__ __forceinline__ void load_tile(TileRegs &t, const uint32_t *base, int
 // Stores the registers K-fastest into an LDS tile [128][PITCH].
 template <bool ROWS_FAST> __device__ __forceinline__ void store_tile(const TileRegs &t, float *lds) {
 #pragma unroll
-    for (int h = 0; h < 2; h++) {
+    for (int h = 0; h < kSlots; h++) {
         uint32_t slot = threadIdx.x + h * kThreads;
         if (!ROWS_FAST) {
-            uint32_t row = slot / 4, k = (slot % 4) * 4;
+            uint32_t row = slot / (BK / 4), k = (slot % (BK / 4)) * 4;
             *reinterpret_cast<float4v *>(lds + row * PITCH + k) = t.v[h];
         } else {
             uint32_t k = slot / 32, row = (slot % 32) * 4;
@@ -135,8 +138,9 @@ template <bool ROWS_FAST> __device__ __forceinline__ void store_tile(const TileR
 }
 
 template <bool A_MFAST, bool B_NFAST> __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
-    __shared__ float lds_a[2][BM * PITCH];
-    __shared__ float lds_b[2][BN * PITCH];
+    extern __shared__ float lds_dyn[]; // [2][BM][PITCH] for A, then [2][BN][PITCH] for B
+    auto lds_a = [&](uint32_t buf) { return lds_dyn + buf * (BM * PITCH); };
+    auto lds_b = [&](uint32_t buf) { return lds_dyn + 2 * BM * PITCH + buf * (BN * PITCH); };
 
     // Tile order.  Workgroups are dealt round-robin to the 8 XCDs, each with its own L2, so
     // the linear id is first regrouped to give every XCD one contiguous run of tiles; inside
@@ -179,8 +183,8 @@ template <bool A_MFAST, bool B_NFAST> __global__ __launch_bounds__(kThreads) voi
     const uint32_t nk = (a.K + BK - 1) / BK;
     load_tile<A_MFAST>(ra, A, a.a_sm, a.a_sk, m0, 0, a.M, a.K, a.a_vec);
     load_tile<B_NFAST>(rb, B, a.b_sn, a.b_sk, n0, 0, a.N, a.K, a.b_vec);
-    store_tile<A_MFAST>(ra, lds_a[0]);
-    store_tile<B_NFAST>(rb, lds_b[0]);
+    store_tile<A_MFAST>(ra, lds_a(0));
+    store_tile<B_NFAST>(rb, lds_b(0));
     __syncthreads();
 
     for (uint32_t kt = 0; kt < nk; kt++) {
@@ -189,7 +193,7 @@ template <bool A_MFAST, bool B_NFAST> __global__ __launch_bounds__(kThreads) voi
             load_tile<A_MFAST>(ra, A, a.a_sm, a.a_sk, m0, (kt + 1) * BK, a.M, a.K, a.a_vec);
             load_tile<B_NFAST>(rb, B, a.b_sn, a.b_sk, n0, (kt + 1) * BK, a.N, a.K, a.b_vec);
         }
-        const float *la = lds_a[cur], *lb = lds_b[cur];
+        const float *la = lds_a(cur), *lb = lds_b(cur);
 #pragma unroll
         for (int kc = 0; kc < BK / 8; kc++) {
             // lane group g supplies k = 8*kc + 4*g + t to the t-th MFMA of this chunk, for
@@ -210,8 +214,8 @@ template <bool A_MFAST, bool B_NFAST> __global__ __launch_bounds__(kThreads) voi
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][t], fb[j][t], acc[i][j], 0, 0, 0);
         }
         if (kt + 1 < nk) {
-            store_tile<A_MFAST>(ra, lds_a[cur ^ 1]);
-            store_tile<B_NFAST>(rb, lds_b[cur ^ 1]);
+            store_tile<A_MFAST>(ra, lds_a(cur ^ 1));
+            store_tile<B_NFAST>(rb, lds_b(cur ^ 1));
         }
         __syncthreads();
     }
@@ -652,16 +656,29 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
         uint64_t tiles = (uint64_t)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
         if (tiles > 0x7FFFFFFFull) return fail(CG_ERR_UNSUPPORTED, "matmul: too many tiles");
         dim3 grid((uint32_t)tiles, (uint32_t)batch);
+        static const bool lds_ok = [] { // the tiles need more than the default 64 KiB of dynamic LDS
+            bool ok = true;
+            ok &= hipFuncSetAttribute(reinterpret_cast<const void *>(&mfma_gemm_kernel<true, true>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGemmLdsBytes) == hipSuccess;
+            ok &= hipFuncSetAttribute(reinterpret_cast<const void *>(&mfma_gemm_kernel<true, false>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGemmLdsBytes) == hipSuccess;
+            ok &= hipFuncSetAttribute(reinterpret_cast<const void *>(&mfma_gemm_kernel<false, true>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGemmLdsBytes) == hipSuccess;
+            ok &= hipFuncSetAttribute(reinterpret_cast<const void *>(&mfma_gemm_kernel<false, false>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGemmLdsBytes) == hipSuccess;
+            return ok;
+        }();
+        if (!lds_ok) return fail(CG_ERR_DEVICE, "matmul: cannot reserve %zu bytes of LDS", kGemmLdsBytes);
         if (a_mfast) {
             if (b_nfast)
-                hipLaunchKernelGGL((mfma_gemm_kernel<true, true>), grid, dim3(kThreads), 0, s, a);
+                hipLaunchKernelGGL((mfma_gemm_kernel<true, true>), grid, dim3(kThreads), kGemmLdsBytes, s, a);
             else
-                hipLaunchKernelGGL((mfma_gemm_kernel<true, false>), grid, dim3(kThreads), 0, s, a);
+                hipLaunchKernelGGL((mfma_gemm_kernel<true, false>), grid, dim3(kThreads), kGemmLdsBytes, s, a);
         } else {
             if (b_nfast)
-                hipLaunchKernelGGL((mfma_gemm_kernel<false, true>), grid, dim3(kThreads), 0, s, a);
+                hipLaunchKernelGGL((mfma_gemm_kernel<false, true>), grid, dim3(kThreads), kGemmLdsBytes, s, a);
             else
-                hipLaunchKernelGGL((mfma_gemm_kernel<false, false>), grid, dim3(kThreads), 0, s, a);
+                hipLaunchKernelGGL((mfma_gemm_kernel<false, false>), grid, dim3(kThreads), kGemmLdsBytes, s, a);
         }
     }
     hipError_t e = hipGetLastError();

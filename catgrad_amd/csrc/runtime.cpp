@@ -243,7 +243,7 @@ FastDiv make_fastdiv(uint32_t d) {
 }
 
 int plan_views(const int64_t *vdims, int vrank, const ViewDesc *v, int n, bool keep_last_axis, EwGeom *g,
-               Operand *ops) {
+               Operand *ops, bool allow_vec4) {
     int r = 0;
     int64_t dims[kMaxRank];
     int64_t st[kMaxViews][kMaxRank];
@@ -283,7 +283,7 @@ int plan_views(const int64_t *vdims, int vrank, const ViewDesc *v, int n, bool k
     for (int i = 0; i < r; i++)
         if (dims[i] > 0xFFFFFFFFll) return fail(CG_ERR_UNSUPPORTED, "axis extent above 2^32-1 elements");
     int64_t inner = dims[r - 1];
-    bool vec4 = inner % 4 == 0;
+    bool vec4 = allow_vec4 && inner % 4 == 0;
     for (int k = 0; k < n; k++) {
         Operand &o = ops[k];
         memset(&o, 0, sizeof o);
@@ -510,9 +510,7 @@ static bool try_view_reshape(const int64_t *xdims, const int64_t *xstrides, int 
 }
 
 // ---- deferred element-wise expressions (see common.hpp) ---------------------------------
-static bool is_expensive(int op) {
-    return op == kDiv || op == kPow || op == kExp || op == kLog || op == kSin || op == kCos;
-}
+static bool is_expensive(int op) { return op == kPow || op == kExp || op == kLog || op == kSin || op == kCos; }
 // Cheap enough to evaluate once per consumer instead of being written out and re-read.
 static bool cheap(const Pending *p) { return !p->expensive && p->ninstr <= 4 && p->nleaf <= 3; }
 
