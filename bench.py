@@ -65,8 +65,8 @@ def micro_bench(iters=20):
     run("exp_f32_8192x8192", A.K_ELEMENTWISE, lambda: be.realize(be.exp(a)), "GB/s")
     del a, b
     r = be.from_numpy(rng.standard_normal((4096, n), dtype=np.float32))
-    run("sum_last_4096x8192", A.K_REDUCE, lambda: be.sum(r), "GB/s")
-    run("max_last_4096x8192", A.K_REDUCE, lambda: be.max(r), "GB/s")
+    run("sum_last_4096x8192", A.K_REDUCE, lambda: be.realize(be.sum(r)), "GB/s")
+    run("max_last_4096x8192", A.K_REDUCE, lambda: be.realize(be.max(r)), "GB/s")
     del r
     row = be.from_numpy(rng.standard_normal((1, n), dtype=np.float32))
     run("broadcast_1x8192_to_4096x8192_materialised", A.K_ELEMENTWISE,

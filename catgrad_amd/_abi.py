@@ -40,6 +40,7 @@ SIGNATURES = {
     "cg_pool_trim": (_I, [_P]),
     "cg_profile_enable": (_I, [_P, _I, C.c_uint]),
     "cg_realize": (_I, [_P, _P]),
+    "cg_program_stats": (_I, [_P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), _I]),
     "cg_profile_read": (_I, [_P, _I, C.POINTER(C.c_uint64), C.POINTER(C.c_double), C.POINTER(C.c_double), _I]),
     "cg_tensor_retain": (None, [_P]),
     "cg_tensor_release": (None, [_P]),

@@ -143,6 +143,12 @@ class Backend:
         self._check(self._lib.cg_realize(self._b, x._h))
         return x
 
+    def program_stats(self, reset: bool = True):
+        """(compiled, interpreted) launches of fused programs since the last reset."""
+        c, i = C.c_uint64(), C.c_uint64()
+        self._check(self._lib.cg_program_stats(self._b, C.byref(c), C.byref(i), int(reset)))
+        return int(c.value), int(i.value)
+
     def profile_enable(self, cls: int, sample_every: int = 1):
         """Time every `sample_every`-th launch of a kernel class with HIP events (0: off)."""
         self._check(self._lib.cg_profile_enable(self._b, cls, sample_every))

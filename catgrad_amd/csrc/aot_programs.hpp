@@ -1,0 +1,267 @@
+// Ahead-of-time specialised kernels for deferred programs (included by fused.hip, inside
+// its anonymous namespace, after FusedArgs and the row helpers).
+//
+// The interpreter kernels run any program, but pay for decoding: operand moves through an
+// indexed register file and a branch per instruction.  The decoder graphs of the model
+// families produce only a handful of distinct programs (RMS norm with and without the
+// residual adds in front, soft-max over masked scores, SiLU gating, rotary embedding, the
+// residual sums), and they produce them for every layer of every step.  Each of those is
+// listed here in the very encoding `Pending` uses, and the compiler turns it into
+// straight-line code: `apply<OP, F>` per instruction, in program order, so results are
+// bit-identical to the interpreter and to unfused execution.  A program that is not listed
+// runs in the interpreter; CG_TRACE_PROGRAMS=1 prints programs in this notation.
+#pragma once
+
+#include <utility>
+
+#define CG_PROGRAM(NAME, NLEAF, ...)                                   \
+    struct NAME {                                                      \
+        static constexpr int nleaf = NLEAF;                            \
+        static constexpr uint8_t code[][4] = {__VA_ARGS__};            \
+        static constexpr int ninstr = (int)(sizeof(code) / 4);         \
+        static constexpr const char *name = #NAME;                     \
+    };
+
+// op codes: 0 neg, 3 exp, 16 add, 17 sub, 18 mul, 19 div, 20 pow, 48 row-sum, 49 row-max;
+// +128 = u32 operands (149 = u32 lt, 169 = cast u32 -> f32).  Registers 0..7 are leaves,
+// 8 + i is the result of instruction i.
+
+// ---- element-wise ------------------------------------------------------------------------
+// x * cos + rotate_half(x) * sin                         (rotary embedding)
+CG_PROGRAM(MapRope, 4, {18, 0, 1, 0}, {18, 2, 3, 2}, {16, 8, 9, 8})
+// g * (1 / (1 + exp(-g))) * u                            (SiLU gate times up projection)
+CG_PROGRAM(MapSiluMul, 3, {0, 0, 0, 0}, {3, 8, 8, 8}, {16, 1, 9, 1}, {19, 1, 10, 1}, {18, 0, 11, 0}, {18, 12, 2, 12})
+// residual stream after three adds, in the two operand orders the layer loop produces
+CG_PROGRAM(MapResidual3a, 4, {16, 1, 2, 1}, {16, 0, 8, 0}, {16, 9, 3, 9})
+CG_PROGRAM(MapResidual3b, 4, {16, 1, 2, 1}, {16, 8, 3, 8}, {16, 0, 9, 0})
+
+// ---- with row reduces ------------------------------------------------------------------------
+// x / sqrt(sum(x*x)/n + eps) * gamma                     (RMS norm)
+CG_PROGRAM(RowsRmsNorm, 5, {18, 0, 0, 0}, {48, 8, 8, 8}, {19, 9, 1, 9}, {16, 10, 2, 10}, {20, 11, 3, 11}, {19, 0, 12, 0},
+           {18, 13, 4, 13})
+// the same on h = a + b, and on h = a + (b + c) / (a + b) + c
+CG_PROGRAM(RowsRmsNormAdd, 6, {16, 0, 1, 0}, {18, 8, 8, 8}, {48, 9, 9, 9}, {19, 10, 2, 10}, {16, 11, 3, 11},
+           {20, 12, 4, 12}, {19, 8, 13, 8}, {18, 14, 5, 14})
+CG_PROGRAM(RowsRmsNormAdd2a, 7, {16, 1, 2, 1}, {16, 0, 8, 0}, {18, 9, 9, 9}, {48, 10, 10, 10}, {19, 11, 3, 11},
+           {16, 12, 4, 12}, {20, 13, 5, 13}, {19, 9, 14, 9}, {18, 15, 6, 15})
+CG_PROGRAM(RowsRmsNormAdd2b, 7, {16, 0, 1, 0}, {16, 8, 2, 8}, {18, 9, 9, 9}, {48, 10, 10, 10}, {19, 11, 3, 11},
+           {16, 12, 4, 12}, {20, 13, 5, 13}, {19, 9, 14, 9}, {18, 15, 6, 15})
+// softmax(s / d + f32(j < i) * m): attention scores, causal mask built from two index vectors
+CG_PROGRAM(RowsSoftmaxCausal, 5, {19, 0, 1, 0}, {149, 2, 3, 2}, {169, 9, 9, 9}, {18, 10, 4, 10}, {16, 8, 11, 8},
+           {49, 12, 12, 12}, {17, 12, 13, 12}, {3, 14, 14, 14}, {48, 15, 15, 15}, {19, 15, 16, 15})
+
+template <class... P> struct ProgramList {};
+using MapPrograms = ProgramList<MapRope, MapSiluMul, MapResidual3a, MapResidual3b>;
+using RowsPrograms = ProgramList<RowsRmsNorm, RowsRmsNormAdd, RowsRmsNormAdd2a, RowsRmsNormAdd2b, RowsSoftmaxCausal>;
+
+template <class P> bool program_matches(const Pending &p) {
+    if (p.nleaf != P::nleaf || p.ninstr != P::ninstr) return false;
+    for (int i = 0; i < P::ninstr; i++) {
+        const Instr &in = p.ins[i];
+        if (in.op != P::code[i][0] || in.a != P::code[i][1] || in.b != P::code[i][2] || in.c != P::code[i][3])
+            return false;
+    }
+    return true;
+}
+
+// ---- compile-time evaluation ------------------------------------------------------------------
+template <class P> constexpr int reduces_before(int i) {
+    int n = 0;
+    for (int k = 0; k < i; k++) n += is_row_reduce(P::code[k][0]) ? 1 : 0;
+    return n;
+}
+// index of row reduce number `phase`; ninstr when the program has no such reduce
+template <class P> constexpr int reduce_index(int phase) {
+    int n = 0;
+    for (int k = 0; k < P::ninstr; k++)
+        if (is_row_reduce(P::code[k][0]) && n++ == phase) return k;
+    return P::ninstr;
+}
+
+template <class P, int VEC> struct Values {
+    uint32_t v[kMaxLeaves + P::ninstr][VEC];
+};
+
+template <class P, int VEC, int I>
+__device__ __forceinline__ void aot_step(Values<P, VEC> &s, const uint32_t (&rs)[kMaxRowReduce], uint32_t *fault) {
+    constexpr int op = P::code[I][0];
+    constexpr int a = P::code[I][1], b = P::code[I][2], c = P::code[I][3];
+    if constexpr (is_row_reduce(op)) {
+        constexpr int k = reduces_before<P>(I);
+#pragma unroll
+        for (int j = 0; j < VEC; j++) s.v[kMaxLeaves + I][j] = rs[k];
+    } else {
+#pragma unroll
+        for (int j = 0; j < VEC; j++)
+            s.v[kMaxLeaves + I][j] = apply<(op & ~kInstrU32), !(op & kInstrU32)>(s.v[a][j], s.v[b][j], s.v[c][j], fault);
+    }
+}
+
+template <class P, int VEC, int... I>
+__device__ __forceinline__ void aot_run(Values<P, VEC> &s, const uint32_t (&rs)[kMaxRowReduce], uint32_t *fault,
+                                        std::integer_sequence<int, I...>) {
+    (aot_step<P, VEC, I>(s, rs, fault), ...);
+}
+
+template <class P, int VEC>
+__device__ __forceinline__ void aot_load(const FusedArgs &a, const int64_t (&off)[P::nleaf], Values<P, VEC> &s) {
+#pragma unroll
+    for (int l = 0; l < P::nleaf; l++) load_words<VEC>(a.leaf[l], off[l], s.v[l]);
+}
+
+// ---- element-wise kernel: the geometry of fused_kernel, the program compiled in ----------------------
+template <class P, int VEC> __global__ __launch_bounds__(kBlock) void aot_map_kernel(const FusedArgs a) {
+    const uint64_t v64 = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (v64 >= a.g.total) return;
+    const uint32_t v = (uint32_t)v64;
+    uint32_t row = fastdiv(v, a.g.ipr_div);
+    const int64_t e = (int64_t)(v - row * a.g.ipr) * VEC;
+    int64_t oo = e * a.out.is;
+    int64_t off[P::nleaf];
+#pragma unroll
+    for (int l = 0; l < P::nleaf; l++) off[l] = e * a.leaf[l].is;
+    for (uint32_t d = 0; d < a.g.nouter; d++) {
+        const uint32_t q = fastdiv(row, a.g.odiv[d]);
+        const int64_t i = (int64_t)(row - q * a.g.od[d]);
+        row = q;
+        oo += i * a.out.os[d];
+#pragma unroll
+        for (int l = 0; l < P::nleaf; l++) off[l] += i * a.leaf[l].os[d];
+    }
+    Values<P, VEC> s;
+    aot_load<P, VEC>(a, off, s);
+    const uint32_t rs[kMaxRowReduce] = {0, 0, 0};
+    aot_run<P, VEC>(s, rs, a.fault, std::make_integer_sequence<int, P::ninstr>{});
+    store_words<VEC>(a.out, oo, s.v[kMaxLeaves + P::ninstr - 1]);
+}
+
+// ---- row kernel: the phases of fused_rows_kernel, unrolled at compile time -----------------------------
+template <class P, int VEC, int TPR, int PHASE>
+__device__ __forceinline__ void aot_rows_phase(const FusedArgs &a, const int64_t (&base)[P::nleaf], uint32_t lane, bool live,
+                                               uint32_t items, uint32_t (&rs)[kMaxRowReduce]) {
+    constexpr int ri = reduce_index<P>(PHASE);
+    constexpr int rop = P::code[ri][0];
+    constexpr bool is_max = (rop & ~kInstrU32) == kRowMax, f = !(rop & kInstrU32);
+    constexpr int src = P::code[ri][1];
+    uint32_t acc = row_init(is_max, f);
+    if (live) {
+        for (uint32_t it = lane; it < items; it += TPR) {
+            int64_t off[P::nleaf];
+#pragma unroll
+            for (int l = 0; l < P::nleaf; l++) off[l] = base[l] + (int64_t)it * VEC * a.leaf[l].is;
+            Values<P, VEC> s;
+            aot_load<P, VEC>(a, off, s);
+            aot_run<P, VEC>(s, rs, a.fault, std::make_integer_sequence<int, ri>{});
+#pragma unroll
+            for (int j = 0; j < VEC; j++) acc = row_merge(is_max, f, acc, s.v[src][j]);
+        }
+    }
+    constexpr int W = TPR < 64 ? TPR : 64;
+#pragma unroll
+    for (int m = W / 2; m >= 1; m >>= 1) acc = row_merge(is_max, f, acc, (uint32_t)__shfl_xor((int)acc, m));
+    if constexpr (TPR > 64) {
+        __shared__ uint32_t part[kBlock / 64];
+        if (threadIdx.x % 64 == 0) part[threadIdx.x / 64] = acc;
+        __syncthreads();
+        acc = part[0];
+#pragma unroll
+        for (int w = 1; w < kBlock / 64; w++) acc = row_merge(is_max, f, acc, part[w]);
+        __syncthreads();
+    }
+    rs[PHASE] = acc;
+}
+
+template <class P, int VEC, int TPR, int... PH>
+__device__ __forceinline__ void aot_rows_phases(const FusedArgs &a, const int64_t (&base)[P::nleaf], uint32_t lane, bool live,
+                                                uint32_t items, uint32_t (&rs)[kMaxRowReduce],
+                                                std::integer_sequence<int, PH...>) {
+    (aot_rows_phase<P, VEC, TPR, PH>(a, base, lane, live, items, rs), ...);
+}
+
+template <class P, int VEC, int TPR>
+__global__ __launch_bounds__(kBlock) void aot_rows_kernel(const FusedArgs a, uint32_t *rowout) {
+    constexpr int RPB = kBlock / TPR;
+    constexpr int NRED = reduces_before<P>(P::ninstr);
+    const uint32_t lane = threadIdx.x % TPR;
+    const uint32_t row = blockIdx.x * RPB + threadIdx.x / TPR;
+    const bool live = row < a.rows;
+    int64_t base[P::nleaf];
+#pragma unroll
+    for (int l = 0; l < P::nleaf; l++) base[l] = 0;
+    int64_t obase = 0;
+    if (live) {
+        uint32_t rr = row;
+        for (uint32_t d = 0; d < a.g.nouter; d++) {
+            const uint32_t q = fastdiv(rr, a.g.odiv[d]);
+            const int64_t i = (int64_t)(rr - q * a.g.od[d]);
+            rr = q;
+            obase += i * a.out.os[d];
+#pragma unroll
+            for (int l = 0; l < P::nleaf; l++) base[l] += i * a.leaf[l].os[d];
+        }
+    }
+    const uint32_t items = a.n / VEC;
+    uint32_t rs[kMaxRowReduce] = {0, 0, 0};
+    aot_rows_phases<P, VEC, TPR>(a, base, lane, live, items, rs, std::make_integer_sequence<int, NRED>{});
+    if (!live) return;
+    if (a.reduced) {
+        if (lane == 0) {
+            Values<P, VEC> s;
+            aot_load<P, VEC>(a, base, s);
+            aot_run<P, VEC>(s, rs, a.fault, std::make_integer_sequence<int, P::ninstr>{});
+            rowout[row] = s.v[kMaxLeaves + P::ninstr - 1][0];
+        }
+        return;
+    }
+    for (uint32_t it = lane; it < items; it += TPR) {
+        int64_t off[P::nleaf];
+#pragma unroll
+        for (int l = 0; l < P::nleaf; l++) off[l] = base[l] + (int64_t)it * VEC * a.leaf[l].is;
+        Values<P, VEC> s;
+        aot_load<P, VEC>(a, off, s);
+        aot_run<P, VEC>(s, rs, a.fault, std::make_integer_sequence<int, P::ninstr>{});
+        store_words<VEC>(a.out, obase + (int64_t)it * VEC * a.out.is, s.v[kMaxLeaves + P::ninstr - 1]);
+    }
+}
+
+// ---- dispatch ---------------------------------------------------------------------------------------
+template <class P> void aot_map_launch(const FusedArgs &a, dim3 grid, hipStream_t s) {
+    if (a.g.vec == 4)
+        hipLaunchKernelGGL((aot_map_kernel<P, 4>), grid, dim3(kBlock), 0, s, a);
+    else
+        hipLaunchKernelGGL((aot_map_kernel<P, 1>), grid, dim3(kBlock), 0, s, a);
+}
+inline bool aot_map_dispatch(const Pending &, const FusedArgs &, dim3, hipStream_t, ProgramList<>) { return false; }
+template <class P, class... Rest>
+bool aot_map_dispatch(const Pending &p, const FusedArgs &a, dim3 grid, hipStream_t s, ProgramList<P, Rest...>) {
+    if (program_matches<P>(p)) {
+        aot_map_launch<P>(a, grid, s);
+        return true;
+    }
+    return aot_map_dispatch(p, a, grid, s, ProgramList<Rest...>{});
+}
+
+template <class P, int VEC> void aot_rows_launch(const FusedArgs &a, uint32_t *rowout, int tpr, dim3 grid, hipStream_t s) {
+    if (tpr == 16)
+        hipLaunchKernelGGL((aot_rows_kernel<P, VEC, 16>), grid, dim3(kBlock), 0, s, a, rowout);
+    else if (tpr == 64)
+        hipLaunchKernelGGL((aot_rows_kernel<P, VEC, 64>), grid, dim3(kBlock), 0, s, a, rowout);
+    else
+        hipLaunchKernelGGL((aot_rows_kernel<P, VEC, 256>), grid, dim3(kBlock), 0, s, a, rowout);
+}
+inline bool aot_rows_dispatch(const Pending &, const FusedArgs &, uint32_t *, int, dim3, hipStream_t, ProgramList<>) {
+    return false;
+}
+// tpr: lanes per row, one of 16 / 64 / 256 (shorter rows stay with the interpreter)
+template <class P, class... Rest>
+bool aot_rows_dispatch(const Pending &p, const FusedArgs &a, uint32_t *rowout, int tpr, dim3 grid, hipStream_t s,
+                       ProgramList<P, Rest...>) {
+    if (program_matches<P>(p)) {
+        if (a.g.vec == 4)
+            aot_rows_launch<P, 4>(a, rowout, tpr, grid, s);
+        else
+            aot_rows_launch<P, 1>(a, rowout, tpr, grid, s);
+        return true;
+    }
+    return aot_rows_dispatch(p, a, rowout, tpr, grid, s, ProgramList<Rest...>{});
+}

@@ -72,6 +72,9 @@ struct cg_backend {
     uint32_t *flag_host = nullptr;  // pinned landing zone for it
     std::string name;
     bool fuse = true; // defer element-wise ops and fuse them (CG_FUSE=0 switches it off)
+    bool aot = true;  // use the compiled kernels for listed programs (CG_AOT=0: interpreter only)
+    uint64_t programs_compiled = 0, programs_interpreted = 0; // launches of fused programs, by kernel kind
+    bool trace_programs = false; // CG_TRACE_PROGRAMS=1: print each distinct deferred program once, to stderr
     cg::ProfClass prof[CG_K_CLASSES];
     std::vector<cg::ProfPending> prof_pending;
     std::vector<std::pair<hipEvent_t, hipEvent_t>> prof_free;
@@ -188,7 +191,16 @@ struct EwGeom {
 // materialises it with ONE launch of the interpreter kernel.  Each element goes through
 // exactly the operations, in the order, that the separate ops would have applied, so
 // results are bit-identical to unfused execution.
-constexpr int kMaxLeaves = 8, kMaxInstr = 24, kMaxViews = kMaxLeaves + 1;
+//
+// `sum` and `max` over the last axis are deferred too, as row-reduce instructions: the
+// value of such an instruction is the reduction of its operand over the row (the last axis
+// of the program's iteration space) and is the same for every element of the row.  The
+// tensor a reduction returns has last extent 1 while its program still iterates over rows
+// of `rowlen` elements (`reduced`); broadcasting it back to the row shape yields an
+// ordinary full-shape program again, so max -> sub -> exp -> sum -> div (softmax) or
+// square -> sum -> scale -> sqrt -> div (RMS norm) collapse into ONE kernel in which a
+// workgroup walks its row once per reduction and once more to produce the output.
+constexpr int kMaxLeaves = 8, kMaxInstr = 24, kMaxViews = kMaxLeaves + 1, kMaxRowReduce = 3;
 
 struct Instr {
     uint8_t op;      // EwOp code, | kInstrU32 when the operands are u32
@@ -207,6 +219,10 @@ struct LeafView {
 struct Pending {
     int nleaf = 0, ninstr = 0;
     bool expensive = false; // holds pow / exp / log / sin / cos
+    int nred = 0;           // row-reduce instructions in the program
+    int64_t rowlen = 0;     // extent of the last axis of the iteration space (set when nred > 0)
+    bool reduced = false;   // the tensor's own last extent is 1: its value is the row-uniform result
+    bool overflow = false;  // set while building when the leaf or instruction table ran out
     LeafView leaf[kMaxLeaves];
     Instr ins[kMaxInstr];
     Pending() = default;
@@ -254,8 +270,11 @@ enum EwOp : int {
     // binary (order of cg_binary_op) offset by 16
     kAdd = 16, kSub, kMul, kDiv, kPow, kLt, kGt, kGte, kLte, kEq,
     kWhere = 32,
-    kCastF2U = 40, kCastU2F, kCopy
+    kCastF2U = 40, kCastU2F, kCopy,
+    // row reductions inside deferred programs (operand a; the result is uniform along the row)
+    kRowSum = 48, kRowMax
 };
+constexpr bool is_row_reduce(int op) { return (op & ~0x80) == kRowSum || (op & ~0x80) == kRowMax; }
 
 // out = op(ins...) element-wise; all views have out's shape.  `out` may be a strided view.
 int launch_elementwise(cg_backend *be, int op, cg_dtype dt, const cg_tensor *out, const cg_tensor *const *ins, int nin);
@@ -263,9 +282,13 @@ int launch_elementwise(cg_backend *be, int op, cg_dtype dt, const cg_tensor *out
 bool fused_program_fits(const Pending &p);
 // Evaluates `p` for every element of shape `dims` into `out` (a dense or strided view of that shape).
 int launch_fused(cg_backend *be, const cg_tensor *out, const Pending &p);
-// Last-axis reduction of the value of `p` (shape dims/rank) into the dense tensor `out`.
-int launch_fused_reduce(cg_backend *be, int kind, bool f32, const Pending &p, const int64_t *dims, int rank,
+// Last-axis reduction of the value of the first `ninstr` instructions of `p` (shape dims/rank)
+// into the dense tensor `out`.
+int launch_fused_reduce(cg_backend *be, int kind, bool f32, const Pending &p, int ninstr, const int64_t *dims, int rank,
                         cg_tensor *out);
+// Evaluates a program with row-reduce instructions over the iteration space `dims` (last axis = row).
+// reduced: `out` is dense with one element per row; else `out` is a (strided) view of shape `dims`.
+int launch_fused_rows(cg_backend *be, const cg_tensor *out, const Pending &p, const int64_t *dims, int rank);
 int launch_arange(cg_backend *be, cg_tensor *out);
 int launch_fill_word(cg_backend *be, void *ptr, uint32_t bits);
 // out[outer, j, inner] = x[outer, idx[j], inner]

@@ -16,6 +16,10 @@
 #include "common.hpp"
 #include "device_utils.hpp"
 
+#include <mutex>
+#include <set>
+#include <string>
+
 namespace cg {
 
 namespace {
@@ -40,6 +44,9 @@ struct FusedArgs {
     uint32_t *fault;
     // reductions only
     uint32_t rows, n;
+    // programs with row-reduce instructions only
+    uint32_t nred, reduced;
+    uint8_t red_op[4]; // op code of the k-th row reduce
 };
 
 // One instruction on the VEC elements of a work item.  op is wave-uniform, so the switch is
@@ -234,6 +241,153 @@ __global__ __launch_bounds__(kBlock) void fused_reduce_kernel(const FusedArgs a,
     if (live && lane == 0) out[row] = (uint32_t)(acc.c & 0xFFFFFFFFll);
 }
 
+// ---- programs with row-reduce instructions -----------------------------------------------------
+__device__ __forceinline__ uint32_t row_init(bool is_max, bool f) { return is_max && f ? asu(kF32Min) : 0u; }
+__device__ __forceinline__ uint32_t row_merge(bool is_max, bool f, uint32_t c, uint32_t w) {
+    if (is_max) return f ? asu(fmaxf(asf(c), asf(w))) : (w > c ? w : c);
+    return f ? asu(asf(c) + asf(w)) : c + w;
+}
+
+// Runs the program on one work item up to row reduce number `phase`: earlier reduces take
+// their finished row value from rs, the operand of reduce `phase` is returned in res (true),
+// and with phase == nred the whole program runs and res is its value (false).
+template <int VEC, bool FULL>
+__device__ __forceinline__ bool eval_rows(const FusedArgs &a, const int64_t (&off)[kMaxLeaves],
+                                          const uint32_t (&rs)[kMaxRowReduce], uint32_t phase, uint32_t (&res)[VEC]) {
+    regfile r[VEC];
+#pragma unroll
+    for (int l = 0; l < kMaxLeaves; l++) {
+        if ((uint32_t)l < a.nleaf) {
+            uint32_t t[VEC];
+            load_words<VEC>(a.leaf[l], off[l], t);
+#pragma unroll
+            for (int j = 0; j < VEC; j++) r[j][l] = t[j];
+        }
+    }
+    uint32_t seen = 0;
+    PInstr in = a.ins[0];
+    for (uint32_t i = 0; i < a.ninstr; i++) {
+        const PInstr cur = in;
+        if (i + 1 < a.ninstr) in = a.ins[i + 1];
+        if (is_row_reduce(cur.op)) {
+            if (seen == phase) {
+#pragma unroll
+                for (int j = 0; j < VEC; j++) res[j] = r[j][cur.a];
+                return true;
+            }
+            const uint32_t v = seen == 0 ? rs[0] : seen == 1 ? rs[1] : rs[2];
+#pragma unroll
+            for (int j = 0; j < VEC; j++) {
+                r[j][cur.dst] = v;
+                res[j] = v;
+            }
+            seen++;
+            continue;
+        }
+        uint32_t x[VEC], y[VEC], z[VEC], o[VEC];
+#pragma unroll
+        for (int j = 0; j < VEC; j++) {
+            x[j] = r[j][cur.a];
+            y[j] = r[j][cur.b];
+            z[j] = r[j][cur.c];
+        }
+        apply_rt<VEC, FULL>(cur.op, x, y, z, o, a.fault);
+#pragma unroll
+        for (int j = 0; j < VEC; j++) {
+            r[j][cur.dst] = o[j];
+            res[j] = o[j];
+        }
+    }
+    return false;
+}
+
+// TPR lanes share a row.  For each row reduce in program order the lanes walk the row,
+// evaluate the program up to that reduce and combine; a last walk evaluates the whole
+// program and stores the row (or, for a reduced result, lane 0 stores the row's value).
+// Leaves are re-read on every walk: a row is a few KiB and stays in L1/L2.
+template <int VEC, int TPR, bool FULL>
+__global__ __launch_bounds__(kBlock) void fused_rows_kernel(const FusedArgs a, uint32_t *rowout) {
+    constexpr int RPB = kBlock / TPR;
+    const uint32_t lane = threadIdx.x % TPR;
+    const uint32_t row = blockIdx.x * RPB + threadIdx.x / TPR;
+    const bool live = row < a.rows;
+    int64_t base[kMaxLeaves];
+#pragma unroll
+    for (int l = 0; l < kMaxLeaves; l++) base[l] = 0;
+    int64_t obase = 0;
+    if (live) {
+        uint32_t rr = row;
+        for (uint32_t d = 0; d < a.g.nouter; d++) {
+            const uint32_t q = fastdiv(rr, a.g.odiv[d]);
+            const int64_t i = (int64_t)(rr - q * a.g.od[d]);
+            rr = q;
+            obase += i * a.out.os[d];
+#pragma unroll
+            for (int l = 0; l < kMaxLeaves; l++)
+                if ((uint32_t)l < a.nleaf) base[l] += i * a.leaf[l].os[d];
+        }
+    }
+    const uint32_t items = a.n / VEC;
+    uint32_t rs[kMaxRowReduce] = {0, 0, 0};
+    for (uint32_t phase = 0; phase < a.nred; phase++) {
+        const uint32_t rop = a.red_op[phase];
+        const bool is_max = (rop & ~kInstrU32) == kRowMax, f = !(rop & kInstrU32);
+        uint32_t acc = row_init(is_max, f);
+        if (live) {
+            for (uint32_t it = lane; it < items; it += TPR) {
+                int64_t off[kMaxLeaves];
+#pragma unroll
+                for (int l = 0; l < kMaxLeaves; l++)
+                    off[l] = (uint32_t)l < a.nleaf ? base[l] + (int64_t)it * VEC * a.leaf[l].is : 0;
+                uint32_t res[VEC];
+                eval_rows<VEC, FULL>(a, off, rs, phase, res);
+#pragma unroll
+                for (int j = 0; j < VEC; j++) acc = row_merge(is_max, f, acc, res[j]);
+            }
+        }
+        // xor butterfly: both partners add the same two values, so every lane of the row ends
+        // with the same bits
+        constexpr int W = TPR < 64 ? TPR : 64;
+#pragma unroll
+        for (int m = W / 2; m >= 1; m >>= 1) acc = row_merge(is_max, f, acc, (uint32_t)__shfl_xor((int)acc, m));
+        if constexpr (TPR > 64) {
+            __shared__ uint32_t part[kBlock / 64];
+            if (threadIdx.x % 64 == 0) part[threadIdx.x / 64] = acc;
+            __syncthreads();
+            acc = part[0];
+#pragma unroll
+            for (int w = 1; w < kBlock / 64; w++) acc = row_merge(is_max, f, acc, part[w]);
+            __syncthreads();
+        }
+        if (phase == 0) rs[0] = acc;
+        else if (phase == 1) rs[1] = acc;
+        else rs[2] = acc;
+    }
+    if (!live) return;
+    if (a.reduced) {
+        if (lane == 0) {
+            int64_t off[kMaxLeaves];
+#pragma unroll
+            for (int l = 0; l < kMaxLeaves; l++) off[l] = base[l];
+            uint32_t res[VEC];
+            eval_rows<VEC, FULL>(a, off, rs, a.nred, res);
+            rowout[row] = res[0];
+        }
+        return;
+    }
+    for (uint32_t it = lane; it < items; it += TPR) {
+        int64_t off[kMaxLeaves];
+#pragma unroll
+        for (int l = 0; l < kMaxLeaves; l++)
+            off[l] = (uint32_t)l < a.nleaf ? base[l] + (int64_t)it * VEC * a.leaf[l].is : 0;
+        uint32_t res[VEC];
+        eval_rows<VEC, FULL>(a, off, rs, a.nred, res);
+        store_words<VEC>(a.out, obase + (int64_t)it * VEC * a.out.is, res);
+    }
+}
+
+#include "aot_programs.hpp"
+
 // Linear-scan register allocation over the 16-entry register file: leaves take 0..nleaf-1,
 // an instruction's destination is any register whose value has no later use (an operand's
 // own register qualifies: it is read before the result is written).  False if 16 do not suffice.
@@ -265,7 +419,8 @@ bool allocate_registers(const Pending &p, uint8_t *phys) {
 }
 
 int fill_args(cg_backend *be, const Pending &p, const int64_t *dims, int rank, const cg_tensor *out, bool keep_last,
-              FusedArgs *a, double *leaf_bytes, bool *full) {
+              FusedArgs *a, double *leaf_bytes, bool *full, int ninstr = -1) {
+    if (ninstr < 0) ninstr = p.ninstr;
     memset(a, 0, sizeof *a);
     ViewDesc v[kMaxViews];
     int64_t out_strides[kMaxRank];
@@ -312,11 +467,11 @@ int fill_args(cg_backend *be, const Pending &p, const int64_t *dims, int rank, c
     a->out = ops[0];
     for (int l = 0; l < p.nleaf; l++) a->leaf[l] = ops[l + 1];
     a->nleaf = (uint32_t)p.nleaf;
-    a->ninstr = (uint32_t)p.ninstr;
+    a->ninstr = (uint32_t)ninstr;
     uint8_t phys[kMaxLeaves + kMaxInstr];
     if (!allocate_registers(p, phys)) return fail(CG_ERR_ARG, "internal error: fused program needs too many registers");
     *full = false;
-    for (int i = 0; i < p.ninstr; i++) {
+    for (int i = 0; i < ninstr; i++) {
         const Instr &in = p.ins[i];
         PInstr q;
         memset(&q, 0, sizeof q);
@@ -328,10 +483,39 @@ int fill_args(cg_backend *be, const Pending &p, const int64_t *dims, int rank, c
         a->ins[i] = q;
         const int op = in.op & ~kInstrU32;
         *full = *full || op == kSin || op == kCos || op == kLog || op == kPow;
+        if (is_row_reduce(op)) {
+            if (a->nred >= (uint32_t)kMaxRowReduce) return fail(CG_ERR_ARG, "internal error: too many row reduces");
+            a->red_op[a->nred++] = in.op;
+        }
     }
     a->fault = be->fault_dev;
     *leaf_bytes = bytes;
     return CG_OK;
+}
+
+// CG_TRACE_PROGRAMS=1: each distinct program, once, in the order of first execution.
+void trace_program(cg_backend *be, const Pending &p, int ninstr, const char *how, const int64_t *dims, int rank) {
+    if (!be->trace_programs) return;
+    static std::mutex mu;
+    static std::set<std::string> seen;
+    std::string key = how;
+    char buf[64];
+    snprintf(buf, sizeof buf, " nleaf=%d ninstr=%d code=", p.nleaf, ninstr);
+    key += buf;
+    for (int i = 0; i < ninstr; i++) {
+        snprintf(buf, sizeof buf, "{%d,%d,%d,%d},", p.ins[i].op, p.ins[i].a, p.ins[i].b, p.ins[i].c);
+        key += buf;
+    }
+    std::lock_guard<std::mutex> lk(mu);
+    if (!seen.insert(key).second) return;
+    std::string where = " uniform=";
+    for (int l = 0; l < p.nleaf; l++) where += p.leaf[l].uniform ? '1' : '0';
+    where += " dims=[";
+    for (int i = 0; i < rank; i++) {
+        snprintf(buf, sizeof buf, "%s%lld", i ? "," : "", (long long)dims[i]);
+        where += buf;
+    }
+    fprintf(stderr, "[cg program] %s%s]\n", key.c_str(), where.c_str());
 }
 
 } // namespace
@@ -348,8 +532,15 @@ int launch_fused(cg_backend *be, const cg_tensor *out, const Pending &p) {
     int rc = fill_args(be, p, out->dims, out->rank, out, false, &a, &bytes, &full);
     if (rc) return rc;
     if (a.g.total == 0) return CG_OK;
+    trace_program(be, p, p.ninstr, "map", out->dims, out->rank);
     ProfScope prof(be, CG_K_ELEMENTWISE, bytes + distinct_bytes(out));
     dim3 grid((uint32_t)((a.g.total + kBlock - 1) / kBlock)), block(kBlock);
+    if (be->aot && aot_map_dispatch(p, a, grid, be->stream, MapPrograms{})) {
+        be->programs_compiled++;
+        hipError_t e = hipGetLastError();
+        return e == hipSuccess ? CG_OK : hip_fail(e, "compiled element-wise launch");
+    }
+    be->programs_interpreted++;
     if (a.g.vec == 4) {
         if (full)
             hipLaunchKernelGGL((fused_kernel<4, true>), grid, block, 0, be->stream, a);
@@ -365,12 +556,12 @@ int launch_fused(cg_backend *be, const cg_tensor *out, const Pending &p) {
     return e == hipSuccess ? CG_OK : hip_fail(e, "fused element-wise launch");
 }
 
-int launch_fused_reduce(cg_backend *be, int kind, bool f32, const Pending &p, const int64_t *dims, int rank,
+int launch_fused_reduce(cg_backend *be, int kind, bool f32, const Pending &p, int ninstr, const int64_t *dims, int rank,
                         cg_tensor *out) {
     FusedArgs a;
     double bytes;
     bool full;
-    int rc = fill_args(be, p, dims, rank, nullptr, true, &a, &bytes, &full);
+    int rc = fill_args(be, p, dims, rank, nullptr, true, &a, &bytes, &full, ninstr);
     if (rc) return rc;
     a.n = a.g.inner;
     uint64_t rows = 1;
@@ -378,6 +569,8 @@ int launch_fused_reduce(cg_backend *be, int kind, bool f32, const Pending &p, co
     if (rows > 0xFFFFFFFFull) return fail(CG_ERR_UNSUPPORTED, "reduction extents above 2^32-1");
     a.rows = (uint32_t)rows;
     uint32_t *op = static_cast<uint32_t *>(out->buf->ptr);
+    be->programs_interpreted++;
+    trace_program(be, p, ninstr, kind == kSum ? "reduce-sum" : kind == kMax ? "reduce-max" : "reduce-argmax", dims, rank);
     ProfScope prof(be, CG_K_REDUCE, bytes + distinct_bytes(out));
     uint32_t want = (a.n + 7) / 8;
     int tpr = want <= 4 ? 4 : want <= 16 ? 16 : want <= 64 ? 64 : 256;
@@ -409,6 +602,66 @@ int launch_fused_reduce(cg_backend *be, int kind, bool f32, const Pending &p, co
 #undef CG_LAUNCH
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? CG_OK : hip_fail(e, "fused reduction launch");
+}
+
+int launch_fused_rows(cg_backend *be, const cg_tensor *out, const Pending &p, const int64_t *dims, int rank) {
+    FusedArgs a;
+    double bytes;
+    bool full;
+    int rc = fill_args(be, p, dims, rank, p.reduced ? nullptr : out, true, &a, &bytes, &full);
+    if (rc) return rc;
+    a.n = a.g.inner;
+    a.reduced = p.reduced ? 1 : 0;
+    uint64_t rows = 1;
+    for (uint32_t d = 0; d < a.g.nouter; d++) rows *= a.g.od[d];
+    if (rows > 0xFFFFFFFFull) return fail(CG_ERR_UNSUPPORTED, "reduction extents above 2^32-1");
+    a.rows = (uint32_t)rows;
+    if (a.rows == 0 || a.n == 0) return CG_OK;
+    uint32_t *rowout = nullptr;
+    if (p.reduced) {
+        if (!is_contiguous(out)) return fail(CG_ERR_ARG, "internal error: row results need a dense destination");
+        const void *op;
+        rc = device_ptr(out, &op);
+        if (rc) return rc;
+        rowout = static_cast<uint32_t *>(const_cast<void *>(op));
+    }
+    trace_program(be, p, p.ninstr, p.reduced ? "rows-reduced" : "rows", dims, rank);
+    ProfScope prof(be, CG_K_ELEMENTWISE, bytes + distinct_bytes(out));
+    uint32_t want = (a.n + 7) / 8;
+    int tpr = want <= 4 ? 4 : want <= 16 ? 16 : want <= 64 ? 64 : 256;
+    uint32_t rpb = kBlock / tpr;
+    dim3 grid((a.rows + rpb - 1) / rpb), block(kBlock);
+    if (be->aot && tpr >= 16 && aot_rows_dispatch(p, a, rowout, tpr, grid, be->stream, RowsPrograms{})) {
+        be->programs_compiled++;
+        hipError_t e = hipGetLastError();
+        return e == hipSuccess ? CG_OK : hip_fail(e, "compiled row-program launch");
+    }
+    be->programs_interpreted++;
+#define CG_LAUNCH(VEC, TPR)                                                                           \
+    do {                                                                                              \
+        if (full)                                                                                     \
+            hipLaunchKernelGGL((fused_rows_kernel<VEC, TPR, true>), grid, block, 0, be->stream, a, rowout);  \
+        else                                                                                          \
+            hipLaunchKernelGGL((fused_rows_kernel<VEC, TPR, false>), grid, block, 0, be->stream, a, rowout); \
+    } while (0)
+    if (a.g.vec == 4) {
+        switch (tpr) {
+        case 4: CG_LAUNCH(4, 4); break;
+        case 16: CG_LAUNCH(4, 16); break;
+        case 64: CG_LAUNCH(4, 64); break;
+        default: CG_LAUNCH(4, 256); break;
+        }
+    } else {
+        switch (tpr) {
+        case 4: CG_LAUNCH(1, 4); break;
+        case 16: CG_LAUNCH(1, 16); break;
+        case 64: CG_LAUNCH(1, 64); break;
+        default: CG_LAUNCH(1, 256); break;
+        }
+    }
+#undef CG_LAUNCH
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CG_OK : hip_fail(e, "fused row-program launch");
 }
 
 } // namespace cg

@@ -119,7 +119,8 @@ static void buffer_release(Buffer *b) {
     }
 }
 
-Pending::Pending(const Pending &o) : nleaf(o.nleaf), ninstr(o.ninstr), expensive(o.expensive) {
+Pending::Pending(const Pending &o)
+    : nleaf(o.nleaf), ninstr(o.ninstr), expensive(o.expensive), nred(o.nred), rowlen(o.rowlen), reduced(o.reduced) {
     for (int l = 0; l < nleaf; l++) {
         leaf[l] = o.leaf[l];
         if (leaf[l].buf) leaf[l].buf->rc.fetch_add(1);
@@ -416,6 +417,8 @@ static int wait_and_check(cg_backend *be) {
     return CG_OK;
 }
 
+static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p);
+
 // Row-major copy of a view (the materialising half of reshape / to_vec).
 static int materialize(cg_backend *be, const cg_tensor *x, cg_tensor **out) {
     cg_tensor *o;
@@ -457,7 +460,7 @@ static int materialize(cg_backend *be, const cg_tensor *x, cg_tensor **out) {
         }
     } else if (numel(x) > 0) {
         const cg_tensor *ins[1] = {x};
-        rc = x->pend ? launch_fused(be, o, *x->pend) : launch_elementwise(be, kCopy, x->dt, o, ins, 1);
+        rc = x->pend ? run_pending(be, o, *x->pend) : launch_elementwise(be, kCopy, x->dt, o, ins, 1);
         if (rc) {
             release(o);
             return rc;
@@ -512,7 +515,7 @@ static bool try_view_reshape(const int64_t *xdims, const int64_t *xstrides, int 
 // ---- deferred element-wise expressions (see common.hpp) ---------------------------------
 static bool is_expensive(int op) { return op == kPow || op == kExp || op == kLog || op == kSin || op == kCos; }
 // Cheap enough to evaluate once per consumer instead of being written out and re-read.
-static bool cheap(const Pending *p) { return !p->expensive && p->ninstr <= 4 && p->nleaf <= 3; }
+static bool cheap(const Pending *p) { return !p->expensive && p->nred == 0 && p->ninstr <= 4 && p->nleaf <= 3; }
 
 static void leaf_as_tensor(const Pending &p, int l, const cg_tensor *shape_of, cg_dtype dt, cg_tensor *t) {
     const LeafView &lv = p.leaf[l];
@@ -530,6 +533,31 @@ static void leaf_as_tensor(const Pending &p, int l, const cg_tensor *shape_of, c
 // Runs the program of `p` into `dst` (a dense or strided view of p's shape).  A single
 // instruction goes to the specialised single-op kernel.
 static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p) {
+    if (p.nred > 0) {
+        // the iteration space: dst's shape, with the row restored when dst holds one value per row
+        cg_tensor space;
+        space.rank = dst->rank;
+        memcpy(space.dims, dst->dims, sizeof space.dims);
+        if (p.reduced) space.dims[space.rank - 1] = p.rowlen;
+        const Instr last = p.ins[p.ninstr - 1];
+        if (p.reduced && p.nred == 1 && is_row_reduce(last.op) && is_contiguous(dst)) {
+            // a lone reduction: the dedicated reduction kernels
+            const int kind = (last.op & ~kInstrU32) == kRowMax ? kMax : kSum;
+            const bool f32 = !(last.op & kInstrU32);
+            cg_tensor *out = const_cast<cg_tensor *>(dst);
+            if (p.ninstr == 1 && !p.leaf[last.a].uniform) {
+                cg_tensor leaf;
+                leaf_as_tensor(p, last.a, &space, f32 ? CG_F32 : CG_U32, &leaf);
+                leaf.be = be;
+                int rc = launch_reduce(be, kind, &leaf, out);
+                leaf.buf = nullptr;
+                return rc;
+            }
+            if (p.ninstr > 1 && last.a == kMaxLeaves + p.ninstr - 2)
+                return launch_fused_reduce(be, kind, f32, p, p.ninstr - 1, space.dims, space.rank, out);
+        }
+        return launch_fused_rows(be, dst, p, space.dims, space.rank);
+    }
     if (p.ninstr == 1) {
         const Instr in = p.ins[0];
         const int op = in.op & ~kInstrU32;
@@ -601,21 +629,72 @@ static int ensure_concrete(cg_tensor *t) {
     return CG_OK;
 }
 
-static bool same_leaf(const LeafView &a, const LeafView &b, const cg_tensor *shape_of) {
+static bool same_leaf(const LeafView &a, const LeafView &b, const int64_t *dims, int rank) {
     if (a.uniform != b.uniform) return false;
     if (a.uniform) return a.ubits == b.ubits;
     if (a.buf != b.buf || a.offset != b.offset) return false;
-    for (int i = 0; i < shape_of->rank; i++)
-        if (shape_of->dims[i] > 1 && a.strides[i] != b.strides[i]) return false;
+    for (int i = 0; i < rank; i++)
+        if (dims[i] > 1 && a.strides[i] != b.strides[i]) return false;
     return true;
 }
 
-static int add_leaf(Pending *p, const LeafView &lv, const cg_tensor *shape_of) {
+static int add_leaf(Pending *p, const LeafView &lv, const int64_t *dims, int rank) {
     for (int l = 0; l < p->nleaf; l++)
-        if (same_leaf(p->leaf[l], lv, shape_of)) return l;
+        if (same_leaf(p->leaf[l], lv, dims, rank)) return l;
+    if (p->nleaf == kMaxLeaves) {
+        p->overflow = true;
+        return 0;
+    }
     p->leaf[p->nleaf] = lv;
     if (lv.buf) lv.buf->rc.fetch_add(1);
     return p->nleaf++;
+}
+
+static int instr_arity(int op) {
+    op &= ~kInstrU32;
+    return op == kWhere ? 3 : (op >= kAdd && op <= kEq) ? 2 : 1;
+}
+
+// Appends `in` unless the program already computes the very same thing; returns its register.
+static uint8_t emit_instr(Pending *p, Instr in) {
+    const int n = instr_arity(in.op);
+    if (n < 2) in.b = in.a;
+    if (n < 3) in.c = in.a;
+    for (int i = 0; i < p->ninstr; i++) {
+        const Instr &o = p->ins[i];
+        if (o.op == in.op && o.a == in.a && o.b == in.b && o.c == in.c) return (uint8_t)(kMaxLeaves + i);
+    }
+    if (p->ninstr == kMaxInstr) {
+        p->overflow = true;
+        return (uint8_t)kMaxLeaves;
+    }
+    p->ins[p->ninstr] = in;
+    if (is_row_reduce(in.op)) p->nred++;
+    p->expensive = p->expensive || is_expensive(in.op & ~kInstrU32);
+    return (uint8_t)(kMaxLeaves + p->ninstr++);
+}
+
+// Copies the program of `src` into `p` (leaves merged, repeated work shared); returns the
+// register of its result.  zero_last: src is a plain program over [.., 1] entering a space
+// whose last axis is a row, so its leaves do not move along that axis.
+static uint8_t splice_program(Pending *p, const Pending *src, const int64_t *dims, int rank, bool zero_last) {
+    uint8_t lmap[kMaxLeaves], rmap[kMaxInstr];
+    for (int l = 0; l < src->nleaf; l++) {
+        LeafView lv = src->leaf[l];
+        if (zero_last) lv.strides[rank - 1] = 0;
+        lmap[l] = (uint8_t)add_leaf(p, lv, dims, rank);
+    }
+    auto remap = [&](uint8_t r) -> uint8_t { return r < kMaxLeaves ? lmap[r] : rmap[r - kMaxLeaves]; };
+    uint8_t last = 0;
+    for (int i = 0; i < src->ninstr; i++) {
+        Instr in = src->ins[i];
+        const int n = instr_arity(in.op);
+        in.a = remap(in.a);
+        in.b = n > 1 ? remap(in.b) : in.a;
+        in.c = n > 2 ? remap(in.c) : in.a;
+        last = rmap[i] = emit_instr(p, in);
+    }
+    return last;
 }
 
 // The result of applying `op` element-wise to `ins` (all of ins[0]'s shape) as a deferred
@@ -625,7 +704,9 @@ static int defer_elementwise(cg_backend *be, int op, cg_dtype in_dt, cg_dtype ou
                              cg_tensor **out) {
     const cg_tensor *shape_of = ins[0];
     if (numel(shape_of) == 0) return new_dense(be, out_dt, shape_of->dims, shape_of->rank, out);
+    const int rank = shape_of->rank;
     bool splice[3] = {false, false, false};
+    int64_t rowlen = 0; // > 0: the operands hold one value per row of this length
     for (int k = 0; k < nin; k++) {
         cg_tensor *x = ins[k];
         if (x->split >= 0) {
@@ -635,97 +716,137 @@ static int defer_elementwise(cg_backend *be, int op, cg_dtype in_dt, cg_dtype ou
         if (!x->pend) continue;
         long mine = 0; // references to x that this very call consumes
         for (int j = 0; j < nin; j++) mine += ins[j] == x;
-        if (x->rc.load() <= mine || cheap(x->pend)) {
+        bool ok = x->rc.load() <= mine || cheap(x->pend);
+        if (ok && x->pend->reduced) { // row results of different row lengths do not mix
+            if (rowlen == 0) rowlen = x->pend->rowlen;
+            else ok = rowlen == x->pend->rowlen;
+        }
+        if (ok) {
             splice[k] = true;
         } else {
             int rc = ensure_concrete(x);
             if (rc) return rc;
         }
     }
-    for (;;) { // shrink until the program fits
-        int leaves = 0, instrs = 1, worst = -1;
-        for (int k = 0; k < nin; k++) {
-            bool dup = false;
-            for (int j = 0; j < k; j++) dup = dup || ins[j] == ins[k];
-            if (dup) continue;
-            if (splice[k]) {
-                leaves += ins[k]->pend->nleaf;
-                instrs += ins[k]->pend->ninstr;
-                if (worst < 0 || ins[k]->pend->ninstr > ins[worst]->pend->ninstr) worst = k;
-            } else {
-                leaves += 1;
-            }
-        }
-        if ((leaves <= kMaxLeaves && instrs <= kMaxInstr) || worst < 0) break;
-        int rc = ensure_concrete(ins[worst]);
-        if (rc) return rc;
-        for (int k = 0; k < nin; k++)
-            if (ins[k] == ins[worst]) splice[k] = false;
-    }
-    Pending *p = new Pending;
-    uint8_t reg[3] = {0, 0, 0};
-    for (int k = 0; k < nin; k++) {
+    // a full-shape row program over rows of length 1 cannot join a space whose rows are longer
+    for (int k = 0; k < nin && rowlen > 0; k++) {
         cg_tensor *x = ins[k];
-        bool done = false;
-        for (int j = 0; j < k && !done; j++)
-            if (ins[j] == x) {
-                reg[k] = reg[j];
-                done = true;
-            }
-        if (done) continue;
-        if (splice[k] && x->pend) {
-            const Pending *src = x->pend;
-            uint8_t lmap[kMaxLeaves];
-            for (int l = 0; l < src->nleaf; l++) lmap[l] = (uint8_t)add_leaf(p, src->leaf[l], shape_of);
-            const int base = p->ninstr;
-            auto remap = [&](uint8_t r) -> uint8_t {
-                return r < kMaxLeaves ? lmap[r] : (uint8_t)(r + base);
-            };
-            for (int i = 0; i < src->ninstr; i++) {
-                Instr in = src->ins[i];
-                const int sop = in.op & ~kInstrU32;
-                const int snin = sop == kWhere ? 3 : (sop >= kAdd && sop <= kEq) ? 2 : 1;
-                in.a = remap(in.a);
-                in.b = snin > 1 ? remap(in.b) : in.a;
-                in.c = snin > 2 ? remap(in.c) : in.a;
-                p->ins[p->ninstr++] = in;
-            }
-            p->expensive = p->expensive || src->expensive;
-            reg[k] = (uint8_t)(kMaxLeaves + p->ninstr - 1);
-        } else {
-            LeafView lv;
-            lv.uniform = x->uniform;
-            lv.ubits = x->ubits;
-            if (!x->uniform) {
-                lv.buf = x->buf;
-                memcpy(lv.strides, x->strides, sizeof lv.strides);
-                lv.offset = x->offset;
-            }
-            reg[k] = (uint8_t)add_leaf(p, lv, shape_of);
+        if (splice[k] && x->pend->nred > 0 && !x->pend->reduced) {
+            int rc = ensure_concrete(x);
+            if (rc) return rc;
+            for (int j = 0; j < nin; j++)
+                if (ins[j] == x) splice[j] = false;
         }
     }
-    Instr in;
-    in.op = (uint8_t)(op | (in_dt == CG_U32 ? kInstrU32 : 0));
-    in.a = reg[0];
-    in.b = nin > 1 ? reg[1] : reg[0];
-    in.c = nin > 2 ? reg[2] : reg[0];
-    p->ins[p->ninstr++] = in;
-    p->expensive = p->expensive || is_expensive(op);
-    if (!fused_program_fits(*p)) { // too many live values: compute the largest deferred input first and retry
+    Pending *p = nullptr;
+    for (;;) { // build; while the program does not fit, compute the largest deferred input first and rebuild
+        int64_t rl = 0;
+        for (int k = 0; k < nin; k++)
+            if (splice[k] && ins[k]->pend->reduced) rl = ins[k]->pend->rowlen;
+        int64_t sdims[kMaxRank]; // the program's iteration space
+        memcpy(sdims, shape_of->dims, sizeof sdims);
+        if (rl > 0) sdims[rank - 1] = rl;
+        p = new Pending;
+        uint8_t reg[3] = {0, 0, 0};
+        for (int k = 0; k < nin; k++) {
+            cg_tensor *x = ins[k];
+            bool done = false;
+            for (int j = 0; j < k && !done; j++)
+                if (ins[j] == x) {
+                    reg[k] = reg[j];
+                    done = true;
+                }
+            if (done) continue;
+            if (splice[k]) {
+                reg[k] = splice_program(p, x->pend, sdims, rank, rl > 0 && !x->pend->reduced);
+            } else {
+                LeafView lv;
+                lv.uniform = x->uniform;
+                lv.ubits = x->ubits;
+                if (!x->uniform) {
+                    lv.buf = x->buf;
+                    memcpy(lv.strides, x->strides, sizeof lv.strides);
+                    if (rl > 0) lv.strides[rank - 1] = 0;
+                    lv.offset = x->offset;
+                }
+                reg[k] = (uint8_t)add_leaf(p, lv, sdims, rank);
+            }
+        }
+        Instr in;
+        in.op = (uint8_t)(op | (in_dt == CG_U32 ? kInstrU32 : 0));
+        in.a = reg[0];
+        in.b = nin > 1 ? reg[1] : reg[0];
+        in.c = nin > 2 ? reg[2] : reg[0];
+        emit_instr(p, in);
+        if (p->nred > 0) {
+            p->rowlen = sdims[rank - 1];
+            p->reduced = rl > 0;
+        }
+        if (!p->overflow && p->nred <= kMaxRowReduce && fused_program_fits(*p)) break;
         delete p;
         int worst = -1;
         for (int k = 0; k < nin; k++)
-            if (ins[k]->pend && (worst < 0 || ins[k]->pend->ninstr > ins[worst]->pend->ninstr)) worst = k;
+            if (splice[k] && (worst < 0 || ins[k]->pend->ninstr > ins[worst]->pend->ninstr)) worst = k;
         if (worst < 0) return fail(CG_ERR_ARG, "internal error: single instruction does not fit");
-        int rc = ensure_concrete(ins[worst]);
+        cg_tensor *w = ins[worst];
+        int rc = ensure_concrete(w);
         if (rc) return rc;
-        return defer_elementwise(be, op, in_dt, out_dt, ins, nin, out);
+        for (int k = 0; k < nin; k++)
+            if (ins[k] == w) splice[k] = false;
     }
     cg_tensor *t = new cg_tensor;
     t->be = be;
     t->dt = out_dt;
-    t->rank = shape_of->rank;
+    t->rank = rank;
     memcpy(t->dims, shape_of->dims, sizeof t->dims);
+    set_row_major(t);
+    t->pend = p;
+    *out = t;
+    return CG_OK;
+}
+
+// The deferred sum / max of x over its last axis (extent >= 1): x's program, or x as a leaf,
+// plus one row-reduce instruction.  *out stays null when the program would not fit.
+static int defer_reduce(cg_backend *be, int kind, cg_tensor *x, const int64_t *odims, cg_tensor **out) {
+    *out = nullptr;
+    const int rank = x->rank;
+    if (x->split >= 0 || (x->pend && x->pend->reduced)) {
+        int rc = ensure_concrete(x);
+        if (rc) return rc;
+    }
+    Pending *p;
+    uint8_t src;
+    if (x->pend) {
+        if (x->pend->nred >= kMaxRowReduce || x->pend->ninstr >= kMaxInstr) return CG_OK;
+        p = new Pending(*x->pend);
+        src = (uint8_t)(kMaxLeaves + p->ninstr - 1);
+    } else {
+        p = new Pending;
+        LeafView lv;
+        lv.uniform = x->uniform;
+        lv.ubits = x->ubits;
+        if (!x->uniform) {
+            lv.buf = x->buf;
+            memcpy(lv.strides, x->strides, sizeof lv.strides);
+            lv.offset = x->offset;
+        }
+        src = (uint8_t)add_leaf(p, lv, x->dims, rank);
+    }
+    Instr in;
+    in.op = (uint8_t)((kind == kMax ? kRowMax : kRowSum) | (x->dt == CG_U32 ? kInstrU32 : 0));
+    in.a = in.b = in.c = src;
+    emit_instr(p, in);
+    p->rowlen = x->dims[rank - 1];
+    p->reduced = true;
+    if (!fused_program_fits(*p)) {
+        delete p;
+        return CG_OK;
+    }
+    cg_tensor *t = new cg_tensor;
+    t->be = be;
+    t->dt = x->dt;
+    t->rank = rank;
+    memcpy(t->dims, odims, sizeof t->dims);
     set_row_major(t);
     t->pend = p;
     *out = t;
@@ -739,6 +860,7 @@ template <class F>
 static int pending_view(cg_tensor *x, const int64_t *dims, int rank, F &&fn, cg_tensor **out, bool *handled) {
     *handled = false;
     if (!x->pend) return CG_OK;
+    if (x->pend->nred > 0) return ensure_concrete(x); // rows do not survive re-striding
     int64_t n = 1;
     for (int i = 0; i < rank; i++) n *= dims[i];
     const bool grows = n > numel(x);
@@ -912,7 +1034,7 @@ static bool try_row_append(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim
         *status = hip_fail(he, "hipSetDevice");
         return true;
     }
-    if (y->pend && y->rc.load() > 1 && !cheap(y->pend)) {
+    if (y->pend && ((y->rc.load() > 1 && !cheap(y->pend)) || y->pend->reduced)) {
         *status = ensure_concrete(y);
         if (*status) return true;
     }
@@ -1021,6 +1143,10 @@ int cg_backend_create(int device, cg_backend **out) {
     CG_HIP(hipMalloc((void **)&b->flag_dev, 64));
     const char *fuse = getenv("CG_FUSE"); // CG_FUSE=0: run every element-wise op as its own kernel
     b->fuse = !(fuse && fuse[0] == '0');
+    const char *aot = getenv("CG_AOT");
+    b->aot = !(aot && aot[0] == '0');
+    const char *trace = getenv("CG_TRACE_PROGRAMS");
+    b->trace_programs = trace && trace[0] == '1';
     char name[256];
     snprintf(name, sizeof name, "hip:%s (%s, %d CUs)%s", prop.gcnArchName, prop.name, prop.multiProcessorCount,
              b->fuse ? "" : " [unfused]");
@@ -1070,6 +1196,14 @@ int cg_pool_trim(cg_backend *b) {
 int cg_profile_enable(cg_backend *b, cg_kernel_class cls, unsigned sample_every) {
     if (!b || (int)cls < 0 || (int)cls >= CG_K_CLASSES) return fail(CG_ERR_ARG, "bad profile class");
     b->prof[cls].every = sample_every;
+    return CG_OK;
+}
+
+int cg_program_stats(cg_backend *b, uint64_t *compiled, uint64_t *interpreted, int reset) {
+    if (!b) return fail(CG_ERR_ARG, "null backend");
+    if (compiled) *compiled = b->programs_compiled;
+    if (interpreted) *interpreted = b->programs_interpreted;
+    if (reset) b->programs_compiled = b->programs_interpreted = 0;
     return CG_OK;
 }
 
@@ -1449,11 +1583,16 @@ static int reduce_entry(cg_backend *b, int kind, const char *what, cg_tensor *x,
     od[x->rank - 1] = 1;
     CG_HIP(hipSetDevice(b->device));
     cg_tensor *o;
-    int rc = new_dense(b, kind == kArgmax ? CG_U32 : x->dt, od, x->rank, &o);
+    int rc;
+    if (b->fuse && kind != kArgmax && numel(x) > 0) {
+        rc = defer_reduce(b, kind, x, od, out);
+        if (rc || *out) return rc;
+    }
+    rc = new_dense(b, kind == kArgmax ? CG_U32 : x->dt, od, x->rank, &o);
     if (rc) return rc;
     if (numel(o) > 0) {
-        if (x->pend && (x->rc.load() == 1 || cheap(x->pend))) {
-            rc = launch_fused_reduce(b, kind, x->dt == CG_F32, *x->pend, x->dims, x->rank, o);
+        if (x->pend && x->pend->nred == 0 && (x->rc.load() == 1 || cheap(x->pend))) {
+            rc = launch_fused_reduce(b, kind, x->dt == CG_F32, *x->pend, x->pend->ninstr, x->dims, x->rank, o);
         } else {
             rc = ensure_concrete(x);
             if (!rc) rc = launch_reduce(b, kind, x, o);
@@ -1526,6 +1665,24 @@ int cg_broadcast(cg_backend *b, cg_tensor *x, const size_t *dims, size_t rank, c
         if (x->dims[i] != d[i + shift] && x->dims[i] != 1)
             return fail(CG_ERR_SHAPE, "broadcast: incompatible shape (axis %d: %lld -> %lld)", i, (long long)x->dims[i],
                         (long long)d[i + shift]);
+    if (x->pend && x->pend->reduced && x->rc.load() == 1 && (int)rank == x->rank && d[rank - 1] == x->pend->rowlen) {
+        // row results broadcast back over their rows: the same program, seen at full shape
+        bool same = true;
+        for (int i = 0; i + 1 < (int)rank; i++) same = same && d[i] == x->dims[i];
+        if (same) {
+            Pending *p = new Pending(*x->pend);
+            p->reduced = false;
+            cg_tensor *t = new cg_tensor;
+            t->be = b;
+            t->dt = x->dt;
+            t->rank = (int)rank;
+            memcpy(t->dims, d, sizeof(int64_t) * rank);
+            set_row_major(t);
+            t->pend = p;
+            *out = t;
+            return CG_OK;
+        }
+    }
     if (x->pend) {
         bool handled;
         rc = pending_view(x, d, (int)rank, [&](LeafView &lv) {
@@ -1746,7 +1903,7 @@ int cg_concat(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor *
         tail.offset = nx;
         const cg_tensor *ins[1] = {y};
         int rc = CG_OK;
-        if (y->pend && y->rc.load() > 1 && !cheap(y->pend)) rc = ensure_concrete(y);
+        if (y->pend && ((y->rc.load() > 1 && !cheap(y->pend)) || y->pend->reduced)) rc = ensure_concrete(y);
         if (!rc) rc = y->pend ? run_pending(b, &tail, *y->pend) : launch_elementwise(b, kCopy, x->dt, &tail, ins, 1);
         tail.buf = nullptr;
         if (rc) return rc;
@@ -1774,7 +1931,7 @@ int cg_concat(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor *
             memcpy(half.strides, o->strides, sizeof half.strides);
             half.offset = at * o->strides[dim];
             const cg_tensor *ins[1] = {src};
-            if (src->pend && src->rc.load() > 1 && !cheap(src->pend)) rc = ensure_concrete(const_cast<cg_tensor *>(src));
+            if (src->pend && ((src->rc.load() > 1 && !cheap(src->pend)) || src->pend->reduced)) rc = ensure_concrete(const_cast<cg_tensor *>(src));
             // a deferred operand is evaluated straight into its half of the result
             if (!rc) rc = src->pend ? run_pending(b, &half, *src->pend) : launch_elementwise(b, kCopy, o->dt, &half, ins, 1);
         }

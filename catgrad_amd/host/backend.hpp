@@ -34,7 +34,7 @@ struct ShapeError : Panic { // BackendError::ShapeError (backend/mod.rs:129-132)
 struct Abi {
 #define CGH_FN(name) decltype(&::name) name = nullptr;
     CGH_FN(cg_backend_create) CGH_FN(cg_backend_destroy) CGH_FN(cg_last_error) CGH_FN(cg_backend_name) CGH_FN(cg_sync)
-    CGH_FN(cg_pool_stats) CGH_FN(cg_pool_trim) CGH_FN(cg_tensor_retain) CGH_FN(cg_tensor_release)
+    CGH_FN(cg_pool_stats) CGH_FN(cg_program_stats) CGH_FN(cg_pool_trim) CGH_FN(cg_tensor_retain) CGH_FN(cg_tensor_release)
     CGH_FN(cg_tensor_rank) CGH_FN(cg_tensor_shape) CGH_FN(cg_tensor_dtype) CGH_FN(cg_tensor_numel)
     CGH_FN(cg_tensor_is_contiguous) CGH_FN(cg_zeros) CGH_FN(cg_from_host) CGH_FN(cg_arange) CGH_FN(cg_to_host)
     CGH_FN(cg_to_bool) CGH_FN(cg_compare) CGH_FN(cg_format_tensor) CGH_FN(cg_cast) CGH_FN(cg_unary)
@@ -51,7 +51,7 @@ struct Abi {
     name = reinterpret_cast<decltype(name)>(dlsym(handle, #name));                       \
     if (!name) throw std::runtime_error(std::string("missing symbol ") + #name + " in " + path);
         CGH_LOAD(cg_backend_create) CGH_LOAD(cg_backend_destroy) CGH_LOAD(cg_last_error) CGH_LOAD(cg_backend_name)
-        CGH_LOAD(cg_sync) CGH_LOAD(cg_pool_stats) CGH_LOAD(cg_pool_trim) CGH_LOAD(cg_tensor_retain)
+        CGH_LOAD(cg_sync) CGH_LOAD(cg_pool_stats) CGH_LOAD(cg_program_stats) CGH_LOAD(cg_pool_trim) CGH_LOAD(cg_tensor_retain)
         CGH_LOAD(cg_tensor_release) CGH_LOAD(cg_tensor_rank) CGH_LOAD(cg_tensor_shape) CGH_LOAD(cg_tensor_dtype)
         CGH_LOAD(cg_tensor_numel) CGH_LOAD(cg_tensor_is_contiguous) CGH_LOAD(cg_zeros) CGH_LOAD(cg_from_host)
         CGH_LOAD(cg_arange) CGH_LOAD(cg_to_host) CGH_LOAD(cg_to_bool) CGH_LOAD(cg_compare) CGH_LOAD(cg_format_tensor)
@@ -224,6 +224,9 @@ class Backend {
         check(abi_.cg_profile_read(b_, (cg_kernel_class)cls, n, ms, work, reset));
     }
     void pool_stats(size_t *in_use, size_t *cached) { check(abi_.cg_pool_stats(b_, in_use, cached)); }
+    void program_stats(uint64_t *compiled, uint64_t *interpreted, int reset) {
+        check(abi_.cg_program_stats(b_, compiled, interpreted, reset));
+    }
 
   private:
     template <class F> Tensor out(F &&f) {

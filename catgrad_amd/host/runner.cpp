@@ -134,4 +134,8 @@ int cgm_pool_stats(cgm_session *s, size_t *in_use, size_t *cached) {
     return guarded([&] { s->interp->backend.pool_stats(in_use, cached); });
 }
 
+int cgm_program_stats(cgm_session *s, uint64_t *compiled, uint64_t *interpreted, int reset) {
+    return guarded([&] { s->interp->backend.program_stats(compiled, interpreted, reset); });
+}
+
 } // extern "C"

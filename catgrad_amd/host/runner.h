@@ -46,6 +46,9 @@ int cgm_profile_read(cgm_session *s, int kernel_class, uint64_t *launches, doubl
 /* Bytes the backend's device pool has handed out / holds cached. */
 int cgm_pool_stats(cgm_session *s, size_t *in_use, size_t *cached);
 
+/* Launches of fused programs since the last reset: compiled ahead of time / interpreted. */
+int cgm_program_stats(cgm_session *s, uint64_t *compiled, uint64_t *interpreted, int reset);
+
 #ifdef __cplusplus
 }
 #endif

@@ -39,6 +39,7 @@ def _host():
             "cgm_forward": (C.c_int, [P, P, SZ, SZ, SZ, P, P]),
             "cgm_mlp": (C.c_int, [P, P, SZ, SZ, SZ, SZ, P]),
             "cgm_pool_stats": (C.c_int, [P, SZP, SZP]),
+            "cgm_program_stats": (C.c_int, [P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.c_int]),
             "cgm_profile_enable": (C.c_int, [P, C.c_int, C.c_uint]),
             "cgm_profile_read": (C.c_int, [P, C.c_int, C.POINTER(C.c_uint64), C.POINTER(C.c_double),
                                            C.POINTER(C.c_double), C.c_int]),
@@ -202,6 +203,12 @@ class Session:
         n, ms, w = C.c_uint64(), C.c_double(), C.c_double()
         self._check(self._lib.cgm_profile_read(self._s, cls, C.byref(n), C.byref(ms), C.byref(w), int(reset)))
         return int(n.value), float(ms.value), float(w.value)
+
+    def program_stats(self, reset: bool = True):
+        """(compiled, interpreted) launches of fused programs since the last reset."""
+        c, i = C.c_uint64(), C.c_uint64()
+        self._check(self._lib.cgm_program_stats(self._s, C.byref(c), C.byref(i), int(reset)))
+        return int(c.value), int(i.value)
 
     def pool_stats(self):
         u, c = C.c_size_t(), C.c_size_t()

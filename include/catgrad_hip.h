@@ -130,6 +130,11 @@ int cg_profile_enable(cg_backend *b, cg_kernel_class cls, unsigned sample_every)
 int cg_realize(cg_backend *b, cg_tensor *t);
 int cg_profile_read(cg_backend *b, cg_kernel_class cls, uint64_t *launches, double *milliseconds, double *work,
                     int reset);
+/* Launches of fused (deferred) programs since the last reset: through a kernel compiled
+ * ahead of time for that very program, and through the interpreter kernels.  No counterpart
+ * in the reference (it has no fusion); the conformance tests use it to check that the
+ * programs of the decoder graphs still match the compiled ones. */
+int cg_program_stats(cg_backend *b, uint64_t *compiled, uint64_t *interpreted, int reset);
 
 /* ---- tensor handles -------------------------------------------------------
  * `BackendTensorOps` (mod.rs:124-126): Clone + shape(). */

@@ -430,6 +430,11 @@ int cg_pool_stats(cg_backend *, size_t *u, size_t *c) {
 int cg_pool_trim(cg_backend *) { return CG_OK; }
 int cg_profile_enable(cg_backend *, cg_kernel_class, unsigned) { return CG_OK; } // no kernels to time
 int cg_realize(cg_backend *, cg_tensor *) { return CG_OK; } // every result is already computed
+int cg_program_stats(cg_backend *, uint64_t *compiled, uint64_t *interpreted, int) { // nothing is fused here
+    if (compiled) *compiled = 0;
+    if (interpreted) *interpreted = 0;
+    return CG_OK;
+}
 int cg_profile_read(cg_backend *, cg_kernel_class, uint64_t *launches, double *milliseconds, double *work, int) {
     if (launches) *launches = 0;
     if (milliseconds) *milliseconds = 0.0;

@@ -7,6 +7,7 @@ Every case is `Case(name, run, expect, kind)`:
                only backend-vs-backend comparison makes sense
   kind      -> "exact" (bit-exact: integer, shape, index ops and IEEE-exact f32 ops),
                "ew"    (f32 element-wise math: rtol 1e-4, atol 1e-6),
+               "ew_abs" (element-wise math fed by a row sum: rtol 1e-4, atol 1e-5),
                "red"   (matmul / sum: 1e-3 of the natural scale of the result)
 The tolerances are the ones the north-star states: bit-exact for integer/shape/index
 ops, rtol 1e-4 for f32 element-wise, 1e-3 relative for matmul and reductions.
@@ -826,6 +827,202 @@ def _():
     return run, expect
 
 
+# ---- deferred row programs: sum / max that stay inside a fused expression -----------------------------
+def _const(be, v, shape, dt=np.float32):
+    return be.broadcast(be.from_numpy(np.array(v, dt)), shape)
+
+
+def _np_softmax(x):
+    x = x.astype(np.float64)
+    e = np.exp(x - x.max(-1, keepdims=True))
+    return e / e.sum(-1, keepdims=True)
+
+
+for _shape in ((1, 5), (3, 7, 33), (4, 8, 1, 260), (2, 3000), (5, 1), (130, 4), (2, 3, 2052)):
+    @case(f"rows_softmax_{'x'.join(map(str, _shape))}", "ew")
+    def _(shape=_shape):
+        a = f32(200 + len(shape) + shape[-1], shape, 2.0)
+        return (lambda be: N(be, softmax_ops(be, be.from_numpy(a)))), (lambda: [_np_softmax(a)])
+
+
+@case("rows_attention_softmax_scale_mask", "ew")
+def _():
+    """softmax(scores * scale + mask) with the mask broadcast over batch and heads, scores a strided view."""
+    B, H, S, T = 2, 3, 5, 64
+    sc = f32(210, (B, S, H, T), 1.5)
+    mask = np.where(np.arange(T)[None, :] <= np.arange(S)[:, None] + (T - S), 0.0, F32_MIN).astype(np.float32)
+
+    def run(be):
+        x = be.transpose(be.from_numpy(sc), 1, 2)  # [B,H,S,T] view
+        shp = (B, H, S, T)
+        x = be.mul(x, _const(be, 0.125, shp))
+        x = be.add(x, be.broadcast(be.from_numpy(mask.reshape(1, 1, S, T)), shp))
+        return N(be, softmax_ops(be, x))
+
+    return run, (lambda: [_np_softmax(sc.transpose(0, 2, 1, 3).astype(np.float64) * 0.125 + mask)])
+
+
+for _n in (64, 576, 2048):
+    @case(f"rows_rmsnorm_{_n}", "ew")
+    def _(n=_n):
+        x = f32(220 + n, (3, 2, n), 1.7)
+        r = f32(221 + n, (3, 2, n), 0.3)
+        g = f32(222 + n, (n,), 1.0)
+
+        def run(be):
+            shp = (3, 2, n)
+            h = be.add(be.from_numpy(x), be.from_numpy(r))  # residual add feeding the norm
+            s = be.sum(be.mul(h, h))
+            mean = be.div(s, _const(be, float(n), (3, 2, 1)))
+            rms = be.pow(be.add(mean, _const(be, 1e-5, (3, 2, 1))), _const(be, 0.5, (3, 2, 1)))
+            y = be.div(h, be.broadcast(rms, shp))
+            return N(be, be.mul(y, be.broadcast(be.from_numpy(g), shp)), h)
+
+        def expect():
+            h = (x + r).astype(np.float64)
+            y = h / np.sqrt((h * h).mean(-1, keepdims=True) + np.float64(np.float32(1e-5)))
+            return [y * g, x + r]
+
+        return run, expect
+
+
+@case("rows_reduced_results_alone", "red")
+def _():
+    """Row results that are read back without being broadcast: a lone reduce, ops then reduce,
+    reduce then ops, and ops on two row results."""
+    a = np.abs(f32(230, (6, 5, 130), 1.0)) + np.float32(0.5)
+    b = np.abs(f32(231, (6, 5, 130), 1.0)) + np.float32(0.5)
+    w = f32(232, (6, 5, 1), 1.0)
+
+    def run(be):
+        ta, tb, tw = be.from_numpy(a), be.from_numpy(b), be.from_numpy(w)
+        s1 = be.sum(ta)
+        s2 = be.sum(be.mul(ta, tb))
+        s3 = be.add(be.div(be.sum(ta), _const(be, 130.0, (6, 5, 1))), tw)
+        s4 = be.div(be.sum(be.mul(ta, tb)), be.max(tb))
+        s5 = be.mul(be.max(ta), be.exp(be.neg(be.max(ta))))
+        return N(be, s1, s2, s3, s4, s5, be.max(ta))
+
+    def expect():
+        A64, B64 = a.astype(np.float64), b.astype(np.float64)
+        m = A64.max(-1, keepdims=True)
+        return [A64.sum(-1, keepdims=True), (A64 * B64).sum(-1, keepdims=True), A64.mean(-1, keepdims=True) + w,
+                (A64 * B64).sum(-1, keepdims=True) / B64.max(-1, keepdims=True), m * np.exp(-m), m]
+
+    return run, expect
+
+
+@case("rows_u32_wrapping")
+def _():
+    a = u32(240, (4, 3, 37))
+
+    def run(be):
+        t = be.from_numpy(a)
+        shp = (4, 3, 37)
+        y = be.add(t, be.broadcast(be.sum(t), shp))
+        z = be.sub(be.broadcast(be.max(t), shp), t)
+        q = be.div(be.broadcast(be.max(t), shp), be.add(t, _const(be, 1, shp, np.uint32)))
+        return N(be, y, z, q, be.add(be.sum(t), be.max(t)))
+
+    def expect():
+        s = a.astype(np.uint64).sum(-1, keepdims=True).astype(np.uint32)
+        m = a.max(-1, keepdims=True)
+        d = (a.astype(np.uint64) + 1).astype(np.uint32)
+        with np.errstate(divide="ignore"):
+            q = np.where(d == 0, 0, m // np.maximum(d, 1)).astype(np.uint32)
+        return [a + s, m - a, q, s + m]
+
+    return run, expect
+
+
+@case("rows_shared_and_viewed_results", "ew")
+def _():
+    """Row results with several users, and views / concats of row programs (which end the deferral)."""
+    a = f32(250, (3, 4, 24), 1.0)
+    b = f32(251, (3, 4, 24), 1.0)
+
+    def run(be):
+        ta, tb = be.from_numpy(a), be.from_numpy(b)
+        shp = (3, 4, 24)
+        m = be.max(ta)
+        bm = be.broadcast(m, shp)
+        o1 = be.sub(ta, bm)
+        o2 = be.add(tb, bm)                               # bm used twice
+        o3 = be.add(be.transpose(m, 0, 1), _const(be, 1.0, (4, 3, 1)))   # view of a row result
+        sm = softmax_ops(be, ta)
+        o4 = be.transpose(sm, 1, 2)                       # view of a full row program
+        o5 = be.concat(softmax_ops(be, tb), ta, 2)        # row program written into a strided destination
+        o6 = be.concat(be.sum(ta), be.max(tb), 2)         # row results as concat operands
+        o7 = be.reshape(softmax_ops(be, ta), (12, 24))
+        o8 = be.slice(softmax_ops(be, ta), 2, 3, 7)
+        o9 = be.broadcast(be.sum(ta), (3, 4, 5))          # row result broadcast to another length
+        o10 = be.broadcast(be.sum(ta), (2, 3, 4, 24))     # ... and with a rank increase
+        return N(be, o1, o2, o3, o4, o5, o6, o7, o8, o9, o10)
+
+    def expect():
+        A64, B64 = a.astype(np.float64), b.astype(np.float64)
+        m = A64.max(-1, keepdims=True)
+        s = A64.sum(-1, keepdims=True)
+        return [A64 - m, B64 + m, m.transpose(1, 0, 2) + 1.0, _np_softmax(a).transpose(0, 2, 1),
+                np.concatenate([_np_softmax(b), A64], 2), np.concatenate([s, B64.max(-1, keepdims=True)], 2),
+                _np_softmax(a).reshape(12, 24), _np_softmax(a)[:, :, 3:10], np.broadcast_to(s, (3, 4, 5)),
+                np.broadcast_to(s, (2, 3, 4, 24))]
+
+    return run, expect
+CASES[-1].kind = "ew_abs"
+
+
+@case("rows_many_reduces_and_mixed_lengths", "ew")
+def _():
+    """Three reduces in one program, a fourth that does not fit, layer-norm style centring, and row
+    results of different row lengths meeting in one op."""
+    a = f32(260, (5, 48), 1.0)
+    c = np.abs(f32(261, (5, 20), 1.0)) + np.float32(1.0)
+
+    def run(be):
+        ta, tc = be.from_numpy(a), be.from_numpy(c)
+        shp = (5, 48)
+        y = softmax_ops(be, ta)
+        z = be.div(y, be.broadcast(be.max(y), shp))             # 3 reduces
+        z4 = be.sum(z)                                           # a 4th
+        mean = be.div(be.sum(ta), _const(be, 48.0, (5, 1)))
+        cen = be.sub(ta, be.broadcast(mean, shp))
+        var = be.div(be.sum(be.mul(cen, cen)), _const(be, 48.0, (5, 1)))
+        ln = be.div(cen, be.broadcast(be.pow(be.add(var, _const(be, 1e-5, (5, 1))), _const(be, 0.5, (5, 1))), shp))
+        mix = be.add(be.sum(tc), be.max(ta))                     # row lengths 20 and 48
+        return N(be, z, z4, ln, mix)
+
+    def expect():
+        A64 = a.astype(np.float64)
+        y = _np_softmax(a)
+        z = y / y.max(-1, keepdims=True)
+        cen = A64 - A64.mean(-1, keepdims=True)
+        ln = cen / np.sqrt((cen * cen).mean(-1, keepdims=True) + np.float64(np.float32(1e-5)))
+        return [z, z.sum(-1, keepdims=True), ln, c.astype(np.float64).sum(-1, keepdims=True) + A64.max(-1, keepdims=True)]
+
+    return run, expect
+CASES[-1].kind = "ew_abs"
+
+
+@case("rows_degenerate_extents")
+def _():
+    a = rng(270).integers(-9, 10, size=(4, 1)).astype(np.float32)
+    e = np.zeros((0, 7), np.float32)
+
+    def run(be):
+        ta, te = be.from_numpy(a), be.from_numpy(e)
+        o1 = be.add(be.broadcast(be.sum(ta), (4, 1)), ta)
+        o2 = be.sub(ta, be.broadcast(be.max(ta), (4, 1)))
+        o3 = be.broadcast(be.sum(te), (0, 7))
+        z = be.zeros((3, 0), A.F32)
+        return N(be, o1, o2, o3, be.sum(z), be.max(z), be.add(be.sum(z), be.max(be.zeros((3, 5), A.F32))))
+
+    def expect():
+        return [a + a, a - a, e, np.zeros((3, 1), np.float32), np.full((3, 1), F32_MIN), np.zeros((3, 1), np.float32)]
+
+    return run, expect
+
+
 def by_name(name):
     for c in CASES:
         if c.name == name:
@@ -847,6 +1044,8 @@ def assert_close(kind, got, exp, scale=None, name=""):
             np.testing.assert_array_equal(got, exp.astype(got.dtype), err_msg=name)
     elif kind == "ew":
         np.testing.assert_allclose(got.astype(np.float64), exp.astype(np.float64), rtol=1e-4, atol=1e-6, err_msg=name)
+    elif kind == "ew_abs":  # element-wise math downstream of a row sum: the sum's rounding shows as absolute error
+        np.testing.assert_allclose(got.astype(np.float64), exp.astype(np.float64), rtol=1e-4, atol=1e-5, err_msg=name)
     elif kind == "red":
         s = np.asarray(scale, dtype=np.float64) if scale is not None else np.abs(exp.astype(np.float64))
         err = np.abs(got.astype(np.float64) - exp.astype(np.float64))

@@ -1,6 +1,8 @@
 """End-to-end parity on the GPU: the host driver over HipBackend against the same driver
 over the CPU oracle — identical seeded weights and prompts, token equality with the
 top1-top2 gap rule, logits within the 1e-3 matmul/reduction contract."""
+import os
+
 import numpy as np
 import pytest
 
@@ -21,6 +23,17 @@ def hip_session():
 def cpu_session():
     oracle_library()
     return Session(ORACLE_LIB)
+
+
+@pytest.fixture(scope="module")
+def interp_session():
+    """HipBackend with the ahead-of-time compiled programs switched off: every fused program
+    runs in the interpreter kernels."""
+    os.environ["CG_AOT"] = "0"
+    try:
+        return Session()
+    finally:
+        del os.environ["CG_AOT"]
 
 
 def assert_tokens_match(got, ref, gaps=None, gap_floor=0.0):
@@ -117,3 +130,33 @@ def test_pool_returns_to_baseline_after_runs(hip_session):
         hip_session.generate(prompt, steps=4, max_positions=16)
     now, _ = hip_session.pool_stats()
     assert now == base  # only the parameters stay resident between runs
+
+
+@pytest.mark.parametrize("arch", ["llama", "qwen3"])
+def test_decoder_programs_are_compiled_and_match_the_interpreter(hip_session, interp_session, arch):
+    """The fused programs that the decoder graphs produce per layer are the ones compiled ahead of
+    time: the number of interpreted launches does not grow with the layer count, and the compiled
+    kernels give bit-identical logits to the interpreter."""
+    interpreted = []
+    for layers in (2, 5):
+        cfg = LlmConfig(arch, 256, layers, 8, 4, 512, 384, head_dim=64, rope_theta=500000.0, tie_word_embeddings=True)
+        params = list(random_params(cfg, seed=5))
+        prompt = prompt_of(cfg, 2, 48, seed=6)
+        hip_session.load_model(cfg, params=params)
+        hip_session.program_stats()
+        g_h, _ = hip_session.generate(prompt, steps=6, max_positions=64)
+        comp, interp = hip_session.program_stats()
+        _, l_h = hip_session.forward(prompt, max_positions=64)
+        interp_session.load_model(cfg, params=params)
+        interp_session.program_stats()
+        g_i, _ = interp_session.generate(prompt, steps=6, max_positions=64)
+        comp_i, interp_i = interp_session.program_stats()
+        _, l_i = interp_session.forward(prompt, max_positions=64)
+        interp_session.clear_params()
+        print(f"{arch} x{layers}: compiled {comp}, interpreted {interp}; with CG_AOT=0: {comp_i}, {interp_i}", flush=True)
+        assert comp_i == 0 and interp_i == comp + interp
+        assert comp >= 7 * layers * 5  # at least five programs per layer and run
+        interpreted.append(interp)
+        np.testing.assert_array_equal(l_h, l_i)
+        np.testing.assert_array_equal(g_h, g_i)
+    assert interpreted[0] == interpreted[1]
