@@ -9,15 +9,19 @@
 // axes form one run, the batch is folded into M (one tall GEMM instead of B small ones).
 //
 // Kernels
-//   mfma_gemm_kernel   128x128x16 macro tile, 256 threads = 2x2 waves, each wave a 64x64
+//   mfma_gemm_kernel   128x128x32 macro tile, 256 threads = 2x2 waves, each wave a 64x64
 //                      quadrant as 2x2 v_mfma_f32_32x32x2_f32 accumulators (64 VGPRs).
-//                      A and B tiles are staged K-fastest in LDS (pitch 20 words: the
-//                      128-bit fragment reads of 8 consecutive rows hit 32 distinct
-//                      banks), two LDS buffers, next tile's global loads in flight during
-//                      the MFMAs.  MFMA-bound: 2*M*N*K flop.
-//   skinny_kt_kernel   M <= 8 with K-contiguous B rows (decode-time linear layers and
-//                      q.K^T): one wave per output column, 16-byte loads along K, wave
-//                      shuffle reduction.  HBM-bound: 4*K*N bytes of B.
+//                      A and B tiles are staged K-fastest in LDS (pitch 36 words: 128-bit
+//                      fragment reads and tile stores are both free of bank conflicts),
+//                      two LDS buffers (72 KiB, dynamic), next tile's global loads in
+//                      flight during the MFMAs.  MFMA-bound: 2*M*N*K flop.
+//   skinny_kt_*        M <= 8 with K-contiguous B rows (decode-time linear layers and
+//                      q.K^T): a wave per output column (or per 4 columns, or a column per
+//                      16/32 lanes for short K), 16-byte loads along K, wave shuffle
+//                      reduction; skinny_kt_mfma_xreg_kernel does the gate/up-sized
+//                      products on the 4x4x1 matrix instruction.  HBM-bound: 4*K*N bytes of B.
+//   skinny_nn_kernel   M <= 8 with N-contiguous B rows (p.V of a decode step), split over K
+//                      with a second pass that adds the partial sums.
 //   simple_gemm_kernel u32 (wrapping) and any shape the others decline.
 //
 // Accumulation is f32 with fused multiply-add; the summation order differs from the
@@ -358,6 +362,85 @@ __global__ __launch_bounds__(kThreads) void skinny_kt_wide_kernel(const MmArgs a
     }
 }
 
+// Skinny kernel on the 4x4x1 matrix instruction (16 independent 4x4 outer products per
+// issue): lane (b, j) = (lane / 4, lane % 4) feeds weight W[n0 + j][k] and activation
+// X[j][k] for the k values of block b, so one 16-byte weight load per lane drives four
+// instructions that update all 4 (rows) x 4 (columns) partial sums of the block.  Against
+// the FMA kernels this needs a quarter of the vector issue slots.  The four waves of a
+// workgroup split each 2048-wide chunk of k, keep their share of the chunk's activations
+// in registers (8 x 16 bytes per lane and row group) and reuse it for CG groups of four
+// columns, so the activation rows are fetched once per 4 * CG columns.
+template <int MM, int CG>
+__global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_kernel(const MmArgs a) {
+    constexpr int G = MM / 4;
+    const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    const uint32_t j = lane % 4, b = lane / 4;
+    const uint32_t n0 = blockIdx.x * (4 * CG);
+    int64_t oa, ob;
+    batch_offsets(a, blockIdx.y, oa, ob);
+    const uint32_t *wrow[CG];
+#pragma unroll
+    for (int c = 0; c < CG; c++) wrow[c] = a.B + ob + (int64_t)min(n0 + 4 * c + j, a.N - 1) * a.b_sn;
+    const uint32_t *xrow[G];
+#pragma unroll
+    for (int g = 0; g < G; g++) xrow[g] = a.A + oa + (int64_t)min((uint32_t)(4 * g) + j, a.M - 1) * a.a_sm;
+    float4v acc[CG][G];
+#pragma unroll
+    for (int c = 0; c < CG; c++)
+#pragma unroll
+        for (int g = 0; g < G; g++) acc[c][g] = (float4v){0.f, 0.f, 0.f, 0.f};
+    const uint32_t kb = (wave * 16 + b) * 4;
+    for (uint32_t k0 = 0; k0 < a.K; k0 += 2048) {
+        float4v xr[G][8];
+#pragma unroll
+        for (int t = 0; t < 8; t++) {
+            const uint32_t k = k0 + kb + 256 * t;
+#pragma unroll
+            for (int g = 0; g < G; g++) {
+                xr[g][t] = (float4v){0.f, 0.f, 0.f, 0.f};
+                if (k < a.K) xr[g][t] = *reinterpret_cast<const float4v *>(xrow[g] + k);
+            }
+        }
+#pragma unroll
+        for (int c = 0; c < CG; c++) {
+            float4v w[8];
+#pragma unroll
+            for (int t = 0; t < 8; t++) {
+                const uint32_t k = k0 + kb + 256 * t;
+                w[t] = (float4v){0.f, 0.f, 0.f, 0.f};
+                if (k < a.K) w[t] = *reinterpret_cast<const float4v *>(wrow[c] + k);
+            }
+#pragma unroll
+            for (int t = 0; t < 8; t++)
+#pragma unroll
+                for (int g = 0; g < G; g++) {
+                    acc[c][g] = __builtin_amdgcn_mfma_f32_4x4x1f32(xr[g][t][0], w[t][0], acc[c][g], 0, 0, 0);
+                    acc[c][g] = __builtin_amdgcn_mfma_f32_4x4x1f32(xr[g][t][1], w[t][1], acc[c][g], 0, 0, 0);
+                    acc[c][g] = __builtin_amdgcn_mfma_f32_4x4x1f32(xr[g][t][2], w[t][2], acc[c][g], 0, 0, 0);
+                    acc[c][g] = __builtin_amdgcn_mfma_f32_4x4x1f32(xr[g][t][3], w[t][3], acc[c][g], 0, 0, 0);
+                }
+        }
+    }
+    __shared__ float part[4][CG * MM * 4];
+#pragma unroll
+    for (int c = 0; c < CG; c++)
+#pragma unroll
+        for (int g = 0; g < G; g++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                float v = acc[c][g][i];
+#pragma unroll
+                for (int s = 32; s >= 4; s >>= 1) v += __shfl_xor(v, s);
+                if (lane < 4) part[wave][(c * MM + 4 * g + i) * 4 + j] = v;
+            }
+    __syncthreads();
+    if (threadIdx.x < CG * MM * 4) {
+        const uint32_t c = threadIdx.x / (MM * 4), m = threadIdx.x / 4 % MM, col = n0 + 4 * c + threadIdx.x % 4;
+        const float v = (part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]);
+        if (col < a.N && m < a.M) a.C[((uint64_t)blockIdx.y * a.M + m) * a.N + col] = asu(v);
+    }
+}
+
 // Vectorised skinny kernel for short K (K <= 4*LPC, e.g. q.K^T of a decode step with
 // K = head_dim): LPC lanes share a column, so a wave covers 64/LPC columns per pass and
 // the activation fragment is loaded once.
@@ -613,6 +696,9 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
 #define CG_CALL(MMV) hipLaunchKernelGGL((skinny_kt_wide_kernel<MMV, 4, false>), grid, dim3(kThreads), 0, s, a);
                 CG_MM_SWITCH(CG_CALL)
 #undef CG_CALL
+            } else if (cols >= 8192 && M <= 4) { // gate / up projections of a decode step
+                dim3 grid((uint32_t)((N + 7) / 8), (uint32_t)batch);
+                hipLaunchKernelGGL((skinny_kt_mfma_xreg_kernel<4, 2>), grid, dim3(kThreads), 0, s, a);
             } else if (cols >= 2048) {
                 dim3 grid((uint32_t)((N + 3) / 4), (uint32_t)batch);
 #define CG_CALL(MMV) hipLaunchKernelGGL((skinny_kt_wide_kernel<MMV, 1, false>), grid, dim3(kThreads), 0, s, a);

@@ -730,6 +730,10 @@ _mm_case("mm_linear_decode_wide_cols1", (4, 1, 512), (5003, 512),
          lambda be, x, w: (x, be.broadcast(be.transpose(w, 0, 1), (4, 512, 5003)), None, None))
 _mm_case("mm_linear_decode_wide_cols4", (3, 1, 384), (20001, 384),
          lambda be, x, w: (x, be.broadcast(be.transpose(w, 0, 1), (3, 384, 20001)), None, None))
+_mm_case("mm_linear_decode_mfma_4x4", (4, 1, 388), (8201, 388),   # ragged N and K: clamped rows, zero-filled k tail
+         lambda be, x, w: (x, be.broadcast(be.transpose(w, 0, 1), (4, 388, 8201)), None, None))
+_mm_case("mm_linear_decode_mfma_4x4_m3_k2304", (3, 1, 2304), (8192, 2304),   # two k chunks, M < 4
+         lambda be, x, w: (x, be.broadcast(be.transpose(w, 0, 1), (3, 2304, 8192)), None, None))
 _mm_case("mm_linear_m8", (8, 1, 1024), (300, 1024),
          lambda be, x, w: (x, be.broadcast(be.transpose(w, 0, 1), (8, 1024, 300)), None, None))
 _mm_case("mm_decode_scores_hd64", (2, 1, 6, 64), (2, 6, 301, 64),
