@@ -67,33 +67,33 @@ __device__ __forceinline__ void batch_offsets(const MmArgs &a, uint32_t b, int64
 // ------------------------------------------------------------------------------------------
 // MFMA kernel
 // ------------------------------------------------------------------------------------------
-constexpr int BM = 128, BN = 128, BK = 32;
+constexpr int BM = 128, BN = 128, BK = 32; // BN = 64 in the narrow variant
 constexpr int PITCH = BK + 4; // words per LDS row: row r starts at bank 4r mod 32
-constexpr int kSlots = BM * BK / 4 / 256; // 16-byte slots of a tile per thread
-constexpr size_t kGemmLdsBytes = 2 * (BM + BN) * PITCH * sizeof(float);
+constexpr size_t gemm_lds_bytes(int bn) { return 2 * (size_t)(BM + bn) * PITCH * sizeof(float); }
 constexpr int kThreads = 256;
 constexpr uint32_t kXcds = 8, kGroupM = 8;
 
 typedef float float4v __attribute__((ext_vector_type(4)));
 typedef float float16v __attribute__((ext_vector_type(16)));
 
-// Loads one 128 x BK tile (rows along `R` with stride s_r, k with stride s_k) into
-// registers: kSlots x float4 per thread.  Layout of the float4 slots of a tile:
+// Loads one TR x BK tile (rows along `R` with stride s_r, k with stride s_k) into
+// registers: TR*BK/4/256 float4 slots per thread.  Layout of the float4 slots of a tile:
 //   K-contiguous source (s_k == 1): slot = row*(BK/4) + kq  (float4 along k; 8 lanes read
 //                                                            128 contiguous bytes of a row)
-//   R-contiguous source (s_r == 1): slot = k*32 + rq        (float4 along rows)
+//   R-contiguous source (s_r == 1): slot = k*(TR/4) + rq    (float4 along rows)
 //   otherwise                      : as K-contiguous, element by element
-struct TileRegs {
-    float4v v[kSlots];
+template <int TR> struct TileRegs {
+    static constexpr int slots = TR * BK / 4 / 256;
+    float4v v[slots];
 };
 
 __device__ __forceinline__ float ld_guard(const uint32_t *p, bool ok) { return ok ? asf(*p) : 0.0f; }
 
-template <bool ROWS_FAST>
-__device__ __forceinline__ void load_tile(TileRegs &t, const uint32_t *base, int64_t s_r, int64_t s_k, uint32_t r0,
+template <bool ROWS_FAST, int TR>
+__device__ __forceinline__ void load_tile(TileRegs<TR> &t, const uint32_t *base, int64_t s_r, int64_t s_k, uint32_t r0,
                                           uint32_t k0, uint32_t R, uint32_t K, bool vec_ok) {
 #pragma unroll
-    for (int h = 0; h < kSlots; h++) {
+    for (int h = 0; h < TileRegs<TR>::slots; h++) {
         uint32_t slot = threadIdx.x + h * kThreads;
         if (!ROWS_FAST) {
             uint32_t row = r0 + slot / (BK / 4), k = k0 + (slot % (BK / 4)) * 4;
@@ -108,7 +108,7 @@ __device__ __forceinline__ void load_tile(TileRegs &t, const uint32_t *base, int
                 t.v[h][3] = ld_guard(p + 3 * s_k, rok && k + 3 < K);
             }
         } else {
-            uint32_t k = k0 + slot / 32, row = r0 + (slot % 32) * 4;
+            uint32_t k = k0 + slot / (TR / 4), row = r0 + (slot % (TR / 4)) * 4;
             const uint32_t *p = base + (int64_t)row * s_r + (int64_t)k * s_k;
             if (vec_ok && k < K && row + 3 < R) {
                 t.v[h] = *reinterpret_cast<const float4v *>(p);
@@ -123,16 +123,16 @@ __device__ __forceinline__ void load_tile(TileRegs &t, const uint32_t *base, int
     }
 }
 
-// Stores the registers K-fastest into an LDS tile [128][PITCH].
-template <bool ROWS_FAST> __device__ __forceinline__ void store_tile(const TileRegs &t, float *lds) {
+// Stores the registers K-fastest into an LDS tile [TR][PITCH].
+template <bool ROWS_FAST, int TR> __device__ __forceinline__ void store_tile(const TileRegs<TR> &t, float *lds) {
 #pragma unroll
-    for (int h = 0; h < kSlots; h++) {
+    for (int h = 0; h < TileRegs<TR>::slots; h++) {
         uint32_t slot = threadIdx.x + h * kThreads;
         if (!ROWS_FAST) {
             uint32_t row = slot / (BK / 4), k = (slot % (BK / 4)) * 4;
             *reinterpret_cast<float4v *>(lds + row * PITCH + k) = t.v[h];
         } else {
-            uint32_t k = slot / 32, row = (slot % 32) * 4;
+            uint32_t k = slot / (TR / 4), row = (slot % (TR / 4)) * 4;
             lds[(row + 0) * PITCH + k] = t.v[h][0];
             lds[(row + 1) * PITCH + k] = t.v[h][1];
             lds[(row + 2) * PITCH + k] = t.v[h][2];
@@ -141,7 +141,11 @@ template <bool ROWS_FAST> __device__ __forceinline__ void store_tile(const TileR
     }
 }
 
-template <bool A_MFAST, bool B_NFAST> __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
+// NT: 32-column MFMA tiles per wave.  2: the 128 x 128 macro tile; 1: 128 x 64 (each wave a
+// 64 x 32 strip) for products whose N is a small multiple of 64, such as p.V with head_dim 64.
+template <bool A_MFAST, bool B_NFAST, int NT>
+__global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
+    constexpr int BN = 64 * NT; // shadows the wide default
     extern __shared__ float lds_dyn[]; // [2][BM][PITCH] for A, then [2][BN][PITCH] for B
     auto lds_a = [&](uint32_t buf) { return lds_dyn + buf * (BM * PITCH); };
     auto lds_b = [&](uint32_t buf) { return lds_dyn + 2 * BM * PITCH + buf * (BN * PITCH); };
@@ -172,18 +176,19 @@ template <bool A_MFAST, bool B_NFAST> __global__ __launch_bounds__(kThreads) voi
     uint32_t *C = a.C + (uint64_t)blockIdx.y * a.M * a.N;
 
     const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x % 64;
-    const uint32_t wm = (wave / 2) * 64, wn = (wave % 2) * 64; // wave quadrant
+    const uint32_t wm = (wave / 2) * 64, wn = (wave % 2) * (32 * NT); // wave quadrant
     const uint32_t li = lane % 32, lg = lane / 32;
 
-    float16v acc[2][2];
+    float16v acc[2][NT];
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++)
+        for (int j = 0; j < NT; j++)
 #pragma unroll
             for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
 
-    TileRegs ra, rb;
+    TileRegs<BM> ra;
+    TileRegs<BN> rb;
     const uint32_t nk = (a.K + BK - 1) / BK;
     load_tile<A_MFAST>(ra, A, a.a_sm, a.a_sk, m0, 0, a.M, a.K, a.a_vec);
     load_tile<B_NFAST>(rb, B, a.b_sn, a.b_sk, n0, 0, a.N, a.K, a.b_vec);
@@ -202,19 +207,19 @@ template <bool A_MFAST, bool B_NFAST> __global__ __launch_bounds__(kThreads) voi
         for (int kc = 0; kc < BK / 8; kc++) {
             // lane group g supplies k = 8*kc + 4*g + t to the t-th MFMA of this chunk, for
             // A and B alike, so one 128-bit LDS read feeds four MFMAs.
-            float4v fa[2], fb[2];
+            float4v fa[2], fb[NT];
 #pragma unroll
             for (int i = 0; i < 2; i++)
                 fa[i] = *reinterpret_cast<const float4v *>(la + (wm + i * 32 + li) * PITCH + kc * 8 + lg * 4);
 #pragma unroll
-            for (int j = 0; j < 2; j++)
+            for (int j = 0; j < NT; j++)
                 fb[j] = *reinterpret_cast<const float4v *>(lb + (wn + j * 32 + li) * PITCH + kc * 8 + lg * 4);
 #pragma unroll
             for (int t = 0; t < 4; t++)
 #pragma unroll
                 for (int i = 0; i < 2; i++)
 #pragma unroll
-                    for (int j = 0; j < 2; j++)
+                    for (int j = 0; j < NT; j++)
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][t], fb[j][t], acc[i][j], 0, 0, 0);
         }
         if (kt + 1 < nk) {
@@ -228,7 +233,7 @@ template <bool A_MFAST, bool B_NFAST> __global__ __launch_bounds__(kThreads) voi
 #pragma unroll
     for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
+        for (int j = 0; j < NT; j++) {
             uint32_t col = n0 + wn + j * 32 + li;
             if (col < a.N) {
 #pragma unroll
@@ -739,33 +744,40 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
         }
 #undef CG_MM_SWITCH
     } else {
-        uint64_t tiles = (uint64_t)((M + BM - 1) / BM) * ((N + BN - 1) / BN);
+        // the narrow tile when the wide one would leave over a seventh of its columns empty
+        const int64_t cols128 = (N + 127) / 128 * 128, cols64 = (N + 63) / 64 * 64;
+        const bool narrow = cols128 * 7 > cols64 * 8;
+        const int bn = narrow ? 64 : 128;
+        uint64_t tiles = (uint64_t)((M + BM - 1) / BM) * ((N + bn - 1) / bn);
         if (tiles > 0x7FFFFFFFull) return fail(CG_ERR_UNSUPPORTED, "matmul: too many tiles");
         dim3 grid((uint32_t)tiles, (uint32_t)batch);
         static const bool lds_ok = [] { // the tiles need more than the default 64 KiB of dynamic LDS
             bool ok = true;
-            ok &= hipFuncSetAttribute(reinterpret_cast<const void *>(&mfma_gemm_kernel<true, true>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGemmLdsBytes) == hipSuccess;
-            ok &= hipFuncSetAttribute(reinterpret_cast<const void *>(&mfma_gemm_kernel<true, false>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGemmLdsBytes) == hipSuccess;
-            ok &= hipFuncSetAttribute(reinterpret_cast<const void *>(&mfma_gemm_kernel<false, true>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGemmLdsBytes) == hipSuccess;
-            ok &= hipFuncSetAttribute(reinterpret_cast<const void *>(&mfma_gemm_kernel<false, false>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGemmLdsBytes) == hipSuccess;
+#define CG_LDS(AF, BF)                                                                                                \
+    ok &= hipFuncSetAttribute(reinterpret_cast<const void *>(&mfma_gemm_kernel<AF, BF, 2>),                           \
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds_bytes(128)) == hipSuccess;    \
+    ok &= hipFuncSetAttribute(reinterpret_cast<const void *>(&mfma_gemm_kernel<AF, BF, 1>),                           \
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds_bytes(64)) == hipSuccess;
+            CG_LDS(true, true) CG_LDS(true, false) CG_LDS(false, true) CG_LDS(false, false)
+#undef CG_LDS
             return ok;
         }();
-        if (!lds_ok) return fail(CG_ERR_DEVICE, "matmul: cannot reserve %zu bytes of LDS", kGemmLdsBytes);
+        if (!lds_ok) return fail(CG_ERR_DEVICE, "matmul: cannot reserve %zu bytes of LDS", gemm_lds_bytes(128));
+#define CG_GEMM(AF, BF)                                                                                            \
+    do {                                                                                                           \
+        if (narrow)                                                                                                \
+            hipLaunchKernelGGL((mfma_gemm_kernel<AF, BF, 1>), grid, dim3(kThreads), gemm_lds_bytes(64), s, a);     \
+        else                                                                                                       \
+            hipLaunchKernelGGL((mfma_gemm_kernel<AF, BF, 2>), grid, dim3(kThreads), gemm_lds_bytes(128), s, a);    \
+    } while (0)
         if (a_mfast) {
-            if (b_nfast)
-                hipLaunchKernelGGL((mfma_gemm_kernel<true, true>), grid, dim3(kThreads), kGemmLdsBytes, s, a);
-            else
-                hipLaunchKernelGGL((mfma_gemm_kernel<true, false>), grid, dim3(kThreads), kGemmLdsBytes, s, a);
+            if (b_nfast) CG_GEMM(true, true);
+            else CG_GEMM(true, false);
         } else {
-            if (b_nfast)
-                hipLaunchKernelGGL((mfma_gemm_kernel<false, true>), grid, dim3(kThreads), kGemmLdsBytes, s, a);
-            else
-                hipLaunchKernelGGL((mfma_gemm_kernel<false, false>), grid, dim3(kThreads), kGemmLdsBytes, s, a);
+            if (b_nfast) CG_GEMM(false, true);
+            else CG_GEMM(false, false);
         }
+#undef CG_GEMM
     }
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? CG_OK : hip_fail(e, "matmul launch");
