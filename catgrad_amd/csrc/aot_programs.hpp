@@ -14,40 +14,42 @@
 
 #include <utility>
 
-#define CG_PROGRAM(NAME, NLEAF, ...)                                   \
+#define CG_PROGRAM(NAME, NLEAF, UNIFORM, ...)                          \
     struct NAME {                                                      \
         static constexpr int nleaf = NLEAF;                            \
+        static constexpr unsigned uniform = UNIFORM; /* bit l: leaf l is a constant */ \
         static constexpr uint8_t code[][4] = {__VA_ARGS__};            \
         static constexpr int ninstr = (int)(sizeof(code) / 4);         \
-        static constexpr const char *name = #NAME;                     \
     };
 
 // op codes: 0 neg, 3 exp, 16 add, 17 sub, 18 mul, 19 div, 20 pow, 48 row-sum, 49 row-max;
 // +128 = u32 operands (149 = u32 lt, 169 = cast u32 -> f32).  Registers 0..7 are leaves,
-// 8 + i is the result of instruction i.
+// 8 + i is the result of instruction i.  Which leaves are constants is part of a program's
+// identity: the compiler then sees that whatever depends only on constants and row results
+// (the square root of an RMS norm) does not change along a row and computes it once.
 
 // ---- element-wise ------------------------------------------------------------------------
 // x * cos + rotate_half(x) * sin                         (rotary embedding)
-CG_PROGRAM(MapRope, 4, {18, 0, 1, 0}, {18, 2, 3, 2}, {16, 8, 9, 8})
+CG_PROGRAM(MapRope, 4, 0x0, {18, 0, 1, 0}, {18, 2, 3, 2}, {16, 8, 9, 8})
 // g * (1 / (1 + exp(-g))) * u                            (SiLU gate times up projection)
-CG_PROGRAM(MapSiluMul, 3, {0, 0, 0, 0}, {3, 8, 8, 8}, {16, 1, 9, 1}, {19, 1, 10, 1}, {18, 0, 11, 0}, {18, 12, 2, 12})
+CG_PROGRAM(MapSiluMul, 3, 0x2, {0, 0, 0, 0}, {3, 8, 8, 8}, {16, 1, 9, 1}, {19, 1, 10, 1}, {18, 0, 11, 0}, {18, 12, 2, 12})
 // residual stream after three adds, in the two operand orders the layer loop produces
-CG_PROGRAM(MapResidual3a, 4, {16, 1, 2, 1}, {16, 0, 8, 0}, {16, 9, 3, 9})
-CG_PROGRAM(MapResidual3b, 4, {16, 1, 2, 1}, {16, 8, 3, 8}, {16, 0, 9, 0})
+CG_PROGRAM(MapResidual3a, 4, 0x0, {16, 1, 2, 1}, {16, 0, 8, 0}, {16, 9, 3, 9})
+CG_PROGRAM(MapResidual3b, 4, 0x0, {16, 1, 2, 1}, {16, 8, 3, 8}, {16, 0, 9, 0})
 
 // ---- with row reduces ------------------------------------------------------------------------
 // x / sqrt(sum(x*x)/n + eps) * gamma                     (RMS norm)
-CG_PROGRAM(RowsRmsNorm, 5, {18, 0, 0, 0}, {48, 8, 8, 8}, {19, 9, 1, 9}, {16, 10, 2, 10}, {20, 11, 3, 11}, {19, 0, 12, 0},
-           {18, 13, 4, 13})
+CG_PROGRAM(RowsRmsNorm, 5, 0xE, {18, 0, 0, 0}, {48, 8, 8, 8}, {19, 9, 1, 9}, {16, 10, 2, 10}, {20, 11, 3, 11},
+           {19, 0, 12, 0}, {18, 13, 4, 13})
 // the same on h = a + b, and on h = a + (b + c) / (a + b) + c
-CG_PROGRAM(RowsRmsNormAdd, 6, {16, 0, 1, 0}, {18, 8, 8, 8}, {48, 9, 9, 9}, {19, 10, 2, 10}, {16, 11, 3, 11},
+CG_PROGRAM(RowsRmsNormAdd, 6, 0x1C, {16, 0, 1, 0}, {18, 8, 8, 8}, {48, 9, 9, 9}, {19, 10, 2, 10}, {16, 11, 3, 11},
            {20, 12, 4, 12}, {19, 8, 13, 8}, {18, 14, 5, 14})
-CG_PROGRAM(RowsRmsNormAdd2a, 7, {16, 1, 2, 1}, {16, 0, 8, 0}, {18, 9, 9, 9}, {48, 10, 10, 10}, {19, 11, 3, 11},
+CG_PROGRAM(RowsRmsNormAdd2a, 7, 0x38, {16, 1, 2, 1}, {16, 0, 8, 0}, {18, 9, 9, 9}, {48, 10, 10, 10}, {19, 11, 3, 11},
            {16, 12, 4, 12}, {20, 13, 5, 13}, {19, 9, 14, 9}, {18, 15, 6, 15})
-CG_PROGRAM(RowsRmsNormAdd2b, 7, {16, 0, 1, 0}, {16, 8, 2, 8}, {18, 9, 9, 9}, {48, 10, 10, 10}, {19, 11, 3, 11},
+CG_PROGRAM(RowsRmsNormAdd2b, 7, 0x38, {16, 0, 1, 0}, {16, 8, 2, 8}, {18, 9, 9, 9}, {48, 10, 10, 10}, {19, 11, 3, 11},
            {16, 12, 4, 12}, {20, 13, 5, 13}, {19, 9, 14, 9}, {18, 15, 6, 15})
 // softmax(s / d + f32(j < i) * m): attention scores, causal mask built from two index vectors
-CG_PROGRAM(RowsSoftmaxCausal, 5, {19, 0, 1, 0}, {149, 2, 3, 2}, {169, 9, 9, 9}, {18, 10, 4, 10}, {16, 8, 11, 8},
+CG_PROGRAM(RowsSoftmaxCausal, 5, 0x12, {19, 0, 1, 0}, {149, 2, 3, 2}, {169, 9, 9, 9}, {18, 10, 4, 10}, {16, 8, 11, 8},
            {49, 12, 12, 12}, {17, 12, 13, 12}, {3, 14, 14, 14}, {48, 15, 15, 15}, {19, 15, 16, 15})
 
 template <class... P> struct ProgramList {};
@@ -56,6 +58,8 @@ using RowsPrograms = ProgramList<RowsRmsNorm, RowsRmsNormAdd, RowsRmsNormAdd2a, 
 
 template <class P> bool program_matches(const Pending &p) {
     if (p.nleaf != P::nleaf || p.ninstr != P::ninstr) return false;
+    for (int l = 0; l < P::nleaf; l++)
+        if (p.leaf[l].uniform != (((P::uniform >> l) & 1u) != 0)) return false;
     for (int i = 0; i < P::ninstr; i++) {
         const Instr &in = p.ins[i];
         if (in.op != P::code[i][0] || in.a != P::code[i][1] || in.b != P::code[i][2] || in.c != P::code[i][3])
@@ -106,7 +110,14 @@ __device__ __forceinline__ void aot_run(Values<P, VEC> &s, const uint32_t (&rs)[
 template <class P, int VEC>
 __device__ __forceinline__ void aot_load(const FusedArgs &a, const int64_t (&off)[P::nleaf], Values<P, VEC> &s) {
 #pragma unroll
-    for (int l = 0; l < P::nleaf; l++) load_words<VEC>(a.leaf[l], off[l], s.v[l]);
+    for (int l = 0; l < P::nleaf; l++) {
+        if ((P::uniform >> l) & 1u) {
+#pragma unroll
+            for (int j = 0; j < VEC; j++) s.v[l][j] = a.leaf[l].ubits;
+        } else {
+            load_words<VEC>(a.leaf[l], off[l], s.v[l]);
+        }
+    }
 }
 
 // ---- element-wise kernel: the geometry of fused_kernel, the program compiled in ----------------------
@@ -136,49 +147,94 @@ template <class P, int VEC> __global__ __launch_bounds__(kBlock) void aot_map_ke
 }
 
 // ---- row kernel: the phases of fused_rows_kernel, unrolled at compile time -----------------------------
-template <class P, int VEC, int TPR, int PHASE>
-__device__ __forceinline__ void aot_rows_phase(const FusedArgs &a, const int64_t (&base)[P::nleaf], uint32_t lane, bool live,
-                                               uint32_t items, uint32_t (&rs)[kMaxRowReduce]) {
-    constexpr int ri = reduce_index<P>(PHASE);
-    constexpr int rop = P::code[ri][0];
-    constexpr bool is_max = (rop & ~kInstrU32) == kRowMax, f = !(rop & kInstrU32);
-    constexpr int src = P::code[ri][1];
-    uint32_t acc = row_init(is_max, f);
-    if (live) {
-        for (uint32_t it = lane; it < items; it += TPR) {
-            int64_t off[P::nleaf];
+// CI > 0: a lane keeps the leaf words of its (at most CI) work items in registers, so the
+// row is read from memory once however many reduces the program has.  CI == 0: rows too long
+// for that; every walk re-reads the leaves (from L1/L2).
+template <class P, int VEC> struct LeafWords {
+    uint32_t v[P::nleaf][VEC];
+};
+
+template <class P, int VEC>
+__device__ __forceinline__ void aot_fetch(const FusedArgs &a, const int64_t (&base)[P::nleaf], uint32_t it,
+                                          LeafWords<P, VEC> &w) {
 #pragma unroll
-            for (int l = 0; l < P::nleaf; l++) off[l] = base[l] + (int64_t)it * VEC * a.leaf[l].is;
-            Values<P, VEC> s;
-            aot_load<P, VEC>(a, off, s);
-            aot_run<P, VEC>(s, rs, a.fault, std::make_integer_sequence<int, ri>{});
+    for (int l = 0; l < P::nleaf; l++) {
+        if ((P::uniform >> l) & 1u) {
 #pragma unroll
-            for (int j = 0; j < VEC; j++) acc = row_merge(is_max, f, acc, s.v[src][j]);
+            for (int j = 0; j < VEC; j++) w.v[l][j] = a.leaf[l].ubits;
+        } else {
+            load_words<VEC>(a.leaf[l], base[l] + (int64_t)it * VEC * a.leaf[l].is, w.v[l]);
         }
     }
+}
+
+// Value of instructions [0, UPTO) on one work item; returns the register file.
+template <class P, int VEC, int UPTO>
+__device__ __forceinline__ Values<P, VEC> aot_eval(const LeafWords<P, VEC> &w, const uint32_t (&rs)[kMaxRowReduce],
+                                                   uint32_t *fault) {
+    Values<P, VEC> s;
+#pragma unroll
+    for (int l = 0; l < P::nleaf; l++)
+#pragma unroll
+        for (int j = 0; j < VEC; j++) s.v[l][j] = w.v[l][j];
+    aot_run<P, VEC>(s, rs, fault, std::make_integer_sequence<int, UPTO>{});
+    return s;
+}
+
+template <bool IS_MAX, bool F, int TPR> __device__ __forceinline__ uint32_t aot_row_combine(uint32_t acc) {
     constexpr int W = TPR < 64 ? TPR : 64;
 #pragma unroll
-    for (int m = W / 2; m >= 1; m >>= 1) acc = row_merge(is_max, f, acc, (uint32_t)__shfl_xor((int)acc, m));
+    for (int m = W / 2; m >= 1; m >>= 1) acc = row_merge(IS_MAX, F, acc, (uint32_t)__shfl_xor((int)acc, m));
     if constexpr (TPR > 64) {
         __shared__ uint32_t part[kBlock / 64];
         if (threadIdx.x % 64 == 0) part[threadIdx.x / 64] = acc;
         __syncthreads();
         acc = part[0];
 #pragma unroll
-        for (int w = 1; w < kBlock / 64; w++) acc = row_merge(is_max, f, acc, part[w]);
+        for (int w = 1; w < kBlock / 64; w++) acc = row_merge(IS_MAX, F, acc, part[w]);
         __syncthreads();
     }
-    rs[PHASE] = acc;
+    return acc;
 }
 
-template <class P, int VEC, int TPR, int... PH>
+template <class P, int VEC, int TPR, int CI, int PHASE>
+__device__ __forceinline__ void aot_rows_phase(const FusedArgs &a, const int64_t (&base)[P::nleaf], uint32_t lane, bool live,
+                                               uint32_t items, const LeafWords<P, VEC> (&cache)[CI > 0 ? CI : 1],
+                                               uint32_t (&rs)[kMaxRowReduce]) {
+    constexpr int ri = reduce_index<P>(PHASE);
+    constexpr int rop = P::code[ri][0];
+    constexpr bool is_max = (rop & ~kInstrU32) == kRowMax, f = !(rop & kInstrU32);
+    constexpr int src = P::code[ri][1];
+    uint32_t acc = row_init(is_max, f);
+    if constexpr (CI > 0) {
+#pragma unroll
+        for (int c = 0; c < CI; c++) {
+            if (live && lane + c * TPR < items) {
+                const Values<P, VEC> s = aot_eval<P, VEC, ri>(cache[c], rs, a.fault);
+#pragma unroll
+                for (int j = 0; j < VEC; j++) acc = row_merge(is_max, f, acc, s.v[src][j]);
+            }
+        }
+    } else if (live) {
+        for (uint32_t it = lane; it < items; it += TPR) {
+            LeafWords<P, VEC> w;
+            aot_fetch<P, VEC>(a, base, it, w);
+            const Values<P, VEC> s = aot_eval<P, VEC, ri>(w, rs, a.fault);
+#pragma unroll
+            for (int j = 0; j < VEC; j++) acc = row_merge(is_max, f, acc, s.v[src][j]);
+        }
+    }
+    rs[PHASE] = aot_row_combine<is_max, f, TPR>(acc);
+}
+
+template <class P, int VEC, int TPR, int CI, int... PH>
 __device__ __forceinline__ void aot_rows_phases(const FusedArgs &a, const int64_t (&base)[P::nleaf], uint32_t lane, bool live,
-                                                uint32_t items, uint32_t (&rs)[kMaxRowReduce],
-                                                std::integer_sequence<int, PH...>) {
-    (aot_rows_phase<P, VEC, TPR, PH>(a, base, lane, live, items, rs), ...);
+                                                uint32_t items, const LeafWords<P, VEC> (&cache)[CI > 0 ? CI : 1],
+                                                uint32_t (&rs)[kMaxRowReduce], std::integer_sequence<int, PH...>) {
+    (aot_rows_phase<P, VEC, TPR, CI, PH>(a, base, lane, live, items, cache, rs), ...);
 }
 
-template <class P, int VEC, int TPR>
+template <class P, int VEC, int TPR, int CI>
 __global__ __launch_bounds__(kBlock) void aot_rows_kernel(const FusedArgs a, uint32_t *rowout) {
     constexpr int RPB = kBlock / TPR;
     constexpr int NRED = reduces_before<P>(P::ninstr);
@@ -201,26 +257,40 @@ __global__ __launch_bounds__(kBlock) void aot_rows_kernel(const FusedArgs a, uin
         }
     }
     const uint32_t items = a.n / VEC;
+    LeafWords<P, VEC> cache[CI > 0 ? CI : 1];
+    if constexpr (CI > 0) {
+#pragma unroll
+        for (int c = 0; c < CI; c++)
+            if (live && lane + c * TPR < items) aot_fetch<P, VEC>(a, base, lane + c * TPR, cache[c]);
+    }
     uint32_t rs[kMaxRowReduce] = {0, 0, 0};
-    aot_rows_phases<P, VEC, TPR>(a, base, lane, live, items, rs, std::make_integer_sequence<int, NRED>{});
+    aot_rows_phases<P, VEC, TPR, CI>(a, base, lane, live, items, cache, rs, std::make_integer_sequence<int, NRED>{});
     if (!live) return;
     if (a.reduced) {
         if (lane == 0) {
-            Values<P, VEC> s;
-            aot_load<P, VEC>(a, base, s);
-            aot_run<P, VEC>(s, rs, a.fault, std::make_integer_sequence<int, P::ninstr>{});
+            LeafWords<P, VEC> w;
+            aot_fetch<P, VEC>(a, base, 0, w);
+            const Values<P, VEC> s = aot_eval<P, VEC, P::ninstr>(w, rs, a.fault);
             rowout[row] = s.v[kMaxLeaves + P::ninstr - 1][0];
         }
         return;
     }
-    for (uint32_t it = lane; it < items; it += TPR) {
-        int64_t off[P::nleaf];
+    if constexpr (CI > 0) {
 #pragma unroll
-        for (int l = 0; l < P::nleaf; l++) off[l] = base[l] + (int64_t)it * VEC * a.leaf[l].is;
-        Values<P, VEC> s;
-        aot_load<P, VEC>(a, off, s);
-        aot_run<P, VEC>(s, rs, a.fault, std::make_integer_sequence<int, P::ninstr>{});
-        store_words<VEC>(a.out, obase + (int64_t)it * VEC * a.out.is, s.v[kMaxLeaves + P::ninstr - 1]);
+        for (int c = 0; c < CI; c++) {
+            const uint32_t it = lane + c * TPR;
+            if (it < items) {
+                const Values<P, VEC> s = aot_eval<P, VEC, P::ninstr>(cache[c], rs, a.fault);
+                store_words<VEC>(a.out, obase + (int64_t)it * VEC * a.out.is, s.v[kMaxLeaves + P::ninstr - 1]);
+            }
+        }
+    } else {
+        for (uint32_t it = lane; it < items; it += TPR) {
+            LeafWords<P, VEC> w;
+            aot_fetch<P, VEC>(a, base, it, w);
+            const Values<P, VEC> s = aot_eval<P, VEC, P::ninstr>(w, rs, a.fault);
+            store_words<VEC>(a.out, obase + (int64_t)it * VEC * a.out.is, s.v[kMaxLeaves + P::ninstr - 1]);
+        }
     }
 }
 
@@ -241,13 +311,22 @@ bool aot_map_dispatch(const Pending &p, const FusedArgs &a, dim3 grid, hipStream
     return aot_map_dispatch(p, a, grid, s, ProgramList<Rest...>{});
 }
 
+// Cached items per lane: 3 vectors of four (rows up to 12 * TPR elements) or 10 single
+// elements (rows up to 10 * TPR); longer rows take the re-reading instantiation.
 template <class P, int VEC> void aot_rows_launch(const FusedArgs &a, uint32_t *rowout, int tpr, dim3 grid, hipStream_t s) {
-    if (tpr == 16)
-        hipLaunchKernelGGL((aot_rows_kernel<P, VEC, 16>), grid, dim3(kBlock), 0, s, a, rowout);
-    else if (tpr == 64)
-        hipLaunchKernelGGL((aot_rows_kernel<P, VEC, 64>), grid, dim3(kBlock), 0, s, a, rowout);
-    else
-        hipLaunchKernelGGL((aot_rows_kernel<P, VEC, 256>), grid, dim3(kBlock), 0, s, a, rowout);
+    constexpr int CI = VEC == 4 ? 3 : 10;
+    const bool fits = (uint64_t)(a.n / VEC) <= (uint64_t)CI * (uint32_t)tpr;
+#define CG_ROWS(TPR)                                                                                        \
+    do {                                                                                                    \
+        if (fits)                                                                                           \
+            hipLaunchKernelGGL((aot_rows_kernel<P, VEC, TPR, CI>), grid, dim3(kBlock), 0, s, a, rowout);     \
+        else                                                                                                \
+            hipLaunchKernelGGL((aot_rows_kernel<P, VEC, TPR, 0>), grid, dim3(kBlock), 0, s, a, rowout);      \
+    } while (0)
+    if (tpr == 16) CG_ROWS(16);
+    else if (tpr == 64) CG_ROWS(64);
+    else CG_ROWS(256);
+#undef CG_ROWS
 }
 inline bool aot_rows_dispatch(const Pending &, const FusedArgs &, uint32_t *, int, dim3, hipStream_t, ProgramList<>) {
     return false;
