@@ -33,6 +33,12 @@ HBM_PEAK = 8.0e12       # B/s, MI355X HBM3E
 MFMA_F32_PEAK = 157.3e12  # flop/s, MI355X dense f32 matrix
 
 
+# HBM bytes per mfma_gemm_kernel launch of this workload's prefill, from rocprofv3 FETCH_SIZE / WRITE_SIZE passes
+# scaled by a copy kernel of known size (profiles/mfma_gemm_llama1b_prefill_pmc.txt); counters cannot be read
+# from inside this process, so the figure is carried here and only reported for the profiled shape.
+MFMA_GEMM_TRAFFIC_PER_LAUNCH = 1.627e9
+
+
 def micro_bench(iters=20):
     """configs[1]: device time per launch from HIP events, algorithmic bytes / flop."""
     from catgrad_amd import HipBackend, _abi as A
@@ -134,7 +140,7 @@ def main():
         be = HipBackend(0)
         x = be.from_numpy(np.zeros((8192, 8192 + 4), dtype=np.float32))
         for _ in range(10):
-            be.reshape(be.slice(x, 1, 0, 8192), (8192 * 8192,))
+            be.realize(be.reshape(be.slice(x, 1, 0, 8192), (8192 * 8192,)))
         be.sync()
         print(json.dumps({"calibration": "ew_kernel<copy> 10 launches", "read_bytes": 8192 * 8192 * 4,
                           "write_bytes": 8192 * 8192 * 4}))
@@ -185,6 +191,15 @@ def main():
 
     K = args.steps
     total_tokens = K * B * (S + T)
+    # algorithmic bytes of a decode step: the matmul weights (lm_head included) once, plus K and V
+    # of every layer at the mean cache length of the decode phase
+    hd = cfg.head_dim or cfg.hidden_size // cfg.num_attention_heads
+    weight_elems = cfg.num_hidden_layers * (
+        2 * cfg.hidden_size * cfg.num_attention_heads * hd + 2 * cfg.hidden_size * cfg.num_key_value_heads * hd
+        + 3 * cfg.hidden_size * cfg.intermediate_size) + cfg.vocab_size * cfg.hidden_size
+    kv_elems = 2 * cfg.num_hidden_layers * B * cfg.num_key_value_heads * (S + T / 2.0) * hd
+    step_bytes = int(4 * (weight_elems + kv_elems))
+    step_rate = step_bytes / (tg_s / K / T) if T and tg_s else 0.0
     result = {
         "metric": "tok/s prefill+decode, Llama-3.2-1B-shape f32; % HBM & MFMA roofline",
         "value": round(total_tokens / (pp_s + tg_s), 2),
@@ -213,15 +228,20 @@ def main():
         "roofline": {
             "kernel": "mfma_gemm_kernel (f32 v_mfma_f32_32x32x2, 128x128x32 tiles)",
             "bound": "mfma", "achieved": round(mfma_rate / 1e12, 3), "peak": MFMA_F32_PEAK / 1e12, "unit": "TFLOP/s",
-            "frac": round(mfma_rate / MFMA_F32_PEAK, 4), "traffic": None,
+            "frac": round(mfma_rate / MFMA_F32_PEAK, 4),
+            "traffic": MFMA_GEMM_TRAFFIC_PER_LAUNCH if (B, S) == (4, 2048) else None,
             "launches_timed": n_m, "avg_launch_ms": round(ms_m / max(n_m, 1), 4),
             "flop_per_launch_avg": flop_m / max(n_m, 1),
         },
         "decode_roofline": {
-            "kernel": "skinny_kt_kernel (M<=8 GEMV-like, K-contiguous weights)",
-            "bound": "hbm", "achieved": round(skinny_rate / 1e9, 2), "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-            "frac": round(skinny_rate / HBM_PEAK, 4), "traffic": None,
-            "launches_timed": n_s, "avg_launch_us": round(ms_s / max(n_s, 1) * 1e3, 3),
+            "scope": "one decode step, all kernels: every weight matrix and the KV cache are read once",
+            "bound": "hbm", "bytes_per_step": step_bytes, "achieved": round(step_rate / 1e9, 2), "peak": HBM_PEAK / 1e9,
+            "unit": "GB/s", "frac": round(step_rate / HBM_PEAK, 4),
+            "skinny_gemm_kernels": {
+                "kernels": "skinny_kt_wide / skinny_kt_mfma_xreg / skinny_kt_narrow / skinny_nn (M <= 8)",
+                "achieved": round(skinny_rate / 1e9, 2), "unit": "GB/s", "frac": round(skinny_rate / HBM_PEAK, 4),
+                "launches_timed": n_s, "avg_launch_us": round(ms_s / max(n_s, 1) * 1e3, 3),
+            },
         },
         "first_tokens": tokens[:2].tolist() if tokens is not None else None,
     }
