@@ -12,7 +12,8 @@ __device__ __forceinline__ uint32_t fastdiv(uint32_t n, const FastDiv &f) {
 __device__ __forceinline__ float asf(uint32_t b) { return __uint_as_float(b); }
 __device__ __forceinline__ uint32_t asu(float f) { return __float_as_uint(f); }
 
-template <int VEC> __device__ __forceinline__ void load_words(const Operand &o, int64_t off, uint32_t (&r)[VEC]) {
+template <int VEC, bool STREAM = false>
+__device__ __forceinline__ void load_words(const Operand &o, int64_t off, uint32_t (&r)[VEC]) {
     if (o.uniform) {
 #pragma unroll
         for (int j = 0; j < VEC; j++) r[j] = o.ubits;
@@ -20,11 +21,12 @@ template <int VEC> __device__ __forceinline__ void load_words(const Operand &o, 
     }
     const uint32_t *p = reinterpret_cast<const uint32_t *>(o.ptr) + off;
     if (VEC == 4 && o.is == 1) {
-        uint4 t = *reinterpret_cast<const uint4 *>(p);
-        r[0] = t.x;
-        r[1 % VEC] = t.y;
-        r[2 % VEC] = t.z;
-        r[3 % VEC] = t.w;
+        typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+        u4 t = STREAM ? __builtin_nontemporal_load(reinterpret_cast<const u4 *>(p)) : *reinterpret_cast<const u4 *>(p);
+        r[0] = t[0];
+        r[1 % VEC] = t[1];
+        r[2 % VEC] = t[2];
+        r[3 % VEC] = t[3];
     } else if (o.is == 0) {
         uint32_t t = *p;
 #pragma unroll
@@ -35,10 +37,19 @@ template <int VEC> __device__ __forceinline__ void load_words(const Operand &o, 
     }
 }
 
-template <int VEC> __device__ __forceinline__ void store_words(const Operand &o, int64_t off, const uint32_t (&r)[VEC]) {
+// STREAM: the output is far larger than the caches; non-temporal stores keep it from
+// evicting the operands that are still being read.
+template <int VEC, bool STREAM = false>
+__device__ __forceinline__ void store_words(const Operand &o, int64_t off, const uint32_t (&r)[VEC]) {
     uint32_t *p = reinterpret_cast<uint32_t *>(const_cast<char *>(o.ptr)) + off;
     if (VEC == 4 && o.is == 1) {
-        *reinterpret_cast<uint4 *>(p) = make_uint4(r[0], r[1 % VEC], r[2 % VEC], r[3 % VEC]);
+        if (STREAM) {
+            typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+            u4 v = {r[0], r[1 % VEC], r[2 % VEC], r[3 % VEC]};
+            __builtin_nontemporal_store(v, reinterpret_cast<u4 *>(p));
+        } else {
+            *reinterpret_cast<uint4 *>(p) = make_uint4(r[0], r[1 % VEC], r[2 % VEC], r[3 % VEC]);
+        }
     } else {
 #pragma unroll
         for (int j = 0; j < VEC; j++) p[(int64_t)j * o.is] = r[j];

@@ -21,6 +21,7 @@ namespace {
 
 constexpr int kBlock = 256;
 constexpr int kUnroll = 4;
+constexpr uint64_t kStreamItems = 4u << 20; // work items (64 MiB of 16-byte vectors) from which outputs stream past the caches
 
 struct EwArgs {
     EwGeom g;
@@ -70,7 +71,12 @@ __global__ __launch_bounds__(kBlock) void ew_kernel(const EwArgs a) {
     for (int u = 0; u < kUnroll; u++)
         if (live[u]) {
 #pragma unroll
-            for (int k = 0; k < NIN; k++) load_words<VEC>(a.in[k], off[u][k + 1], x[u][k]);
+            for (int k = 0; k < NIN; k++) {
+                // fully collapsed space: a unit-stride operand is read exactly once, so it need not
+                // displace anything from the caches either
+                if (FLAT && a.g.total >= kStreamItems) load_words<VEC, true>(a.in[k], off[u][k + 1], x[u][k]);
+                else load_words<VEC>(a.in[k], off[u][k + 1], x[u][k]);
+            }
         }
 #pragma unroll
     for (int u = 0; u < kUnroll; u++)
@@ -79,7 +85,8 @@ __global__ __launch_bounds__(kBlock) void ew_kernel(const EwArgs a) {
 #pragma unroll
             for (int j = 0; j < VEC; j++)
                 r[j] = apply<OP, F>(x[u][0][j], NIN > 1 ? x[u][1 % NIN][j] : 0u, NIN > 2 ? x[u][2 % NIN][j] : 0u, a.fault);
-            store_words<VEC>(a.out, off[u][0], r);
+            if (a.g.total >= kStreamItems) store_words<VEC, true>(a.out, off[u][0], r);
+            else store_words<VEC>(a.out, off[u][0], r);
         }
 }
 
