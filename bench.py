@@ -159,7 +159,11 @@ def main():
     B, S, T = args.batch, args.prefill, args.decode
     params = list(random_params(cfg, args.seed))
     sess = Session()
+    t_up = time.perf_counter()
     sess.load_model(cfg, params=params)
+    sess.sync()
+    t_up = time.perf_counter() - t_up
+    weight_bytes = sum(int(w.size) * 4 for _, w in params)
     prompt = np.random.default_rng(args.seed).integers(0, cfg.vocab_size, size=(B, S), dtype=np.uint32)
 
     for _ in range(args.warmup):
@@ -244,6 +248,9 @@ def main():
             },
         },
         "first_tokens": tokens[:2].tolist() if tokens is not None else None,
+        # not part of `value`: the one-off upload of the weights from pageable host memory through the
+        # backend's pinned staging buffers (the PCIe-inclusive cost of a cold start)
+        "weights_upload": {"bytes": weight_bytes, "seconds": round(t_up, 3), "GB_per_s": round(weight_bytes / t_up / 1e9, 2)},
     }
     sess.close()
     if not args.no_micro:

@@ -51,6 +51,7 @@ SIGNATURES = {
     "cg_tensor_is_contiguous": (_I, [_P]),
     "cg_zeros": (_I, [_P, _I, _SZP, _SZ, _PP]),
     "cg_from_host": (_I, [_P, _I, _P, _SZ, _SZP, _SZ, _PP]),
+    "cg_from_host_bf16_as_f32": (_I, [_P, _P, _SZ, _SZP, _SZ, _PP]),
     "cg_arange": (_I, [_P, _SZ, _PP]),
     "cg_to_host": (_I, [_P, _P, _P, _SZ]),
     "cg_to_bool": (_I, [_P, _P, C.POINTER(_I)]),

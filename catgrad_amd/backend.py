@@ -188,6 +188,14 @@ class Backend:
     def ndarray_from_vec_fp8(self, data, shape) -> Tensor:
         return self._from_vec(A.F8, np.uint8, data, shape)
 
+    def from_bf16_bits(self, bits, shape) -> Tensor:
+        """Weight ingest (catgrad-llm/src/utils/mod.rs:158-168): an f32 tensor from bfloat16 bit
+        patterns (uint16); the widening happens in the backend."""
+        arr = np.ascontiguousarray(np.asarray(bits, dtype=np.uint16).reshape(-1))
+        d, r = A.dims_array(shape)
+        ptr = arr.ctypes.data_as(C.c_void_p)
+        return self._op(lambda b, o: self._lib.cg_from_host_bf16_as_f32(b, ptr, arr.size, d, r, o))
+
     def from_numpy(self, arr) -> Tensor:
         """`interpreter::tensor` (catgrad/src/interpreter/mod.rs:23-33) for a numpy array."""
         arr = np.asarray(arr)

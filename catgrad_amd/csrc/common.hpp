@@ -70,6 +70,11 @@ struct cg_backend {
     uint32_t *fault_dev = nullptr;
     uint32_t *flag_dev = nullptr;   // 4-byte scratch for to_bool / compare
     uint32_t *flag_host = nullptr;  // pinned landing zone for it
+    // host-to-device staging: two pinned buffers used in turn, each guarded by an event
+    void *stage[2] = {nullptr, nullptr};
+    hipEvent_t stage_ev[2] = {nullptr, nullptr};
+    bool stage_busy[2] = {false, false};
+    unsigned stage_next = 0;
     std::string name;
     bool fuse = true; // defer element-wise ops and fuse them (CG_FUSE=0 switches it off)
     bool aot = true;  // use the compiled kernels for listed programs (CG_AOT=0: interpreter only)
@@ -81,6 +86,8 @@ struct cg_backend {
 };
 
 namespace cg {
+
+constexpr size_t kStageBytes = 16u << 20; // size of each pinned host-to-device staging buffer
 
 // Row-block structure of a buffer that grows by appended rows (a KV cache): the buffer is
 // [nblocks][C][R] elements, block b holds fill[b] valid rows of R elements, rows at and
@@ -291,6 +298,8 @@ int launch_fused_reduce(cg_backend *be, int kind, bool f32, const Pending &p, in
 int launch_fused_rows(cg_backend *be, const cg_tensor *out, const Pending &p, const int64_t *dims, int rank);
 int launch_arange(cg_backend *be, cg_tensor *out);
 int launch_fill_word(cg_backend *be, void *ptr, uint32_t bits);
+// dst[i] = (uint32_t)src[i] << 16 : bfloat16 bit patterns widened to f32
+int launch_bf16_widen(cg_backend *be, const void *src, void *dst, uint64_t n);
 // out[outer, j, inner] = x[outer, idx[j], inner]
 int launch_gather(cg_backend *be, const cg_tensor *x, int dim, const cg_tensor *idx, cg_tensor *out);
 

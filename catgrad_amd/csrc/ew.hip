@@ -15,6 +15,8 @@
 #include "common.hpp"
 #include "device_utils.hpp"
 
+#include <algorithm>
+
 namespace cg {
 
 namespace {
@@ -122,6 +124,24 @@ __global__ void arange_kernel(uint32_t *out, uint32_t n) {
 
 __global__ void fill_word_kernel(uint32_t *p, uint32_t bits) { *p = bits; }
 
+// 8 bfloat16 per lane and trip: one 16-byte load, two 16-byte stores.  HBM-bound: 2 B read + 4 B written per element.
+__global__ __launch_bounds__(kBlock) void bf16_widen_kernel(const uint16_t *__restrict__ src, uint32_t *__restrict__ dst,
+                                                            uint64_t n) {
+    const uint64_t groups = n / 8;
+    for (uint64_t g = (uint64_t)blockIdx.x * kBlock + threadIdx.x; g < groups; g += (uint64_t)gridDim.x * kBlock) {
+        const uint4 v = reinterpret_cast<const uint4 *>(src)[g];
+        uint4 lo, hi;
+        lo.x = v.x << 16; lo.y = v.x & 0xFFFF0000u; lo.z = v.y << 16; lo.w = v.y & 0xFFFF0000u;
+        hi.x = v.z << 16; hi.y = v.z & 0xFFFF0000u; hi.z = v.w << 16; hi.w = v.w & 0xFFFF0000u;
+        reinterpret_cast<uint4 *>(dst)[2 * g] = lo;
+        reinterpret_cast<uint4 *>(dst)[2 * g + 1] = hi;
+    }
+    if (blockIdx.x == 0 && threadIdx.x < n % 8) { // ragged tail
+        const uint64_t i = groups * 8 + threadIdx.x;
+        dst[i] = (uint32_t)src[i] << 16;
+    }
+}
+
 // out[o, j, :] = x[o, idx[j], :]  with x row-major [outer, D, inner]
 template <int VEC>
 __global__ __launch_bounds__(kBlock) void gather_kernel(const uint32_t *__restrict__ x, const uint32_t *__restrict__ idx,
@@ -196,6 +216,16 @@ int launch_arange(cg_backend *be, cg_tensor *out) {
                        static_cast<uint32_t *>(out->buf->ptr), n);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? CG_OK : hip_fail(e, "arange launch");
+}
+
+int launch_bf16_widen(cg_backend *be, const void *src, void *dst, uint64_t n) {
+    if (n == 0) return CG_OK;
+    const uint64_t groups = n / 8;
+    const uint32_t blocks = (uint32_t)std::min<uint64_t>(std::max<uint64_t>((groups + kBlock - 1) / kBlock, 1), 8192);
+    hipLaunchKernelGGL(bf16_widen_kernel, dim3(blocks), dim3(kBlock), 0, be->stream, static_cast<const uint16_t *>(src),
+                       static_cast<uint32_t *>(dst), n);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CG_OK : hip_fail(e, "bf16 widen launch");
 }
 
 int launch_fill_word(cg_backend *be, void *ptr, uint32_t bits) {

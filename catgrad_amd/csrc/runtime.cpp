@@ -1166,6 +1166,10 @@ void cg_backend_destroy(cg_backend *b) {
     }
     b->pool.trim();
     (void)hipFree(b->flag_dev);
+    for (int i = 0; i < 2; i++) {
+        if (b->stage[i]) (void)hipHostFree(b->stage[i]);
+        if (b->stage_ev[i]) (void)hipEventDestroy(b->stage_ev[i]);
+    }
     (void)hipHostFree(b->flag_host);
     (void)hipHostFree(b->fault_host);
     (void)hipStreamDestroy(b->stream);
@@ -1265,6 +1269,29 @@ int cg_zeros(cg_backend *b, cg_dtype dtype, const size_t *dims, size_t rank, cg_
 
 // ndarray.rs:86-96,122-132 and interpreter/mod.rs:28-30.  One-element tensors (the
 // `Scalar` / `NatToU32` constants of tensor_op.rs:64-87) stay on the host as uniforms.
+// Host memory to device memory through the backend's two pinned staging buffers: the host
+// copy into one buffer overlaps the DMA out of the other, nothing waits for the device unless
+// a buffer is still in flight, and `src` may be freed on return.
+static int staged_upload(cg_backend *b, void *dst, const void *src, size_t bytes) {
+    const char *s = static_cast<const char *>(src);
+    char *d = static_cast<char *>(dst);
+    for (size_t off = 0; off < bytes; off += kStageBytes) {
+        const size_t chunk = std::min(kStageBytes, bytes - off);
+        const unsigned i = b->stage_next;
+        b->stage_next ^= 1u;
+        if (!b->stage[i]) {
+            CG_HIP(hipHostMalloc(&b->stage[i], kStageBytes, hipHostMallocDefault));
+            CG_HIP(hipEventCreateWithFlags(&b->stage_ev[i], hipEventDisableTiming));
+        }
+        if (b->stage_busy[i]) CG_HIP(hipEventSynchronize(b->stage_ev[i]));
+        memcpy(b->stage[i], s + off, chunk);
+        CG_HIP(hipMemcpyAsync(d + off, b->stage[i], chunk, hipMemcpyHostToDevice, b->stream));
+        CG_HIP(hipEventRecord(b->stage_ev[i], b->stream));
+        b->stage_busy[i] = true;
+    }
+    return CG_OK;
+}
+
 int cg_from_host(cg_backend *b, cg_dtype dtype, const void *data, size_t len, const size_t *dims, size_t rank,
                  cg_tensor **out) {
     if (!b || !out) return fail(CG_ERR_ARG, "null argument");
@@ -1287,11 +1314,46 @@ int cg_from_host(cg_backend *b, cg_dtype dtype, const void *data, size_t len, co
     if (rc) return rc;
     if (n) {
         CG_HIP(hipSetDevice(b->device));
-        hipError_t e = hipMemcpyAsync(t->buf->ptr, data, n * 4, hipMemcpyHostToDevice, b->stream);
-        if (e == hipSuccess) e = hipStreamSynchronize(b->stream); // caller may free `data` on return
-        if (e != hipSuccess) {
+        rc = staged_upload(b, t->buf->ptr, data, n * 4);
+        if (rc) {
             release(t);
-            return hip_fail(e, "host to device copy");
+            return rc;
+        }
+    }
+    *out = t;
+    return CG_OK;
+}
+
+int cg_from_host_bf16_as_f32(cg_backend *b, const uint16_t *bits, size_t len, const size_t *dims, size_t rank,
+                             cg_tensor **out) {
+    if (!b || !out) return fail(CG_ERR_ARG, "null argument");
+    int64_t d[kMaxRank];
+    int rc = check_dims(dims, rank, d);
+    if (rc) return rc;
+    size_t n = 1;
+    for (size_t i = 0; i < rank; i++) n *= dims[i];
+    if (n != len) return fail(CG_ERR_SHAPE, "ShapeError");
+    if (n && !bits) return fail(CG_ERR_ARG, "null data");
+    if (n == 1) {
+        *out = new_uniform(b, CG_F32, d, (int)rank, (uint32_t)bits[0] << 16);
+        return CG_OK;
+    }
+    cg_tensor *t;
+    rc = new_dense(b, CG_F32, d, (int)rank, &t);
+    if (rc) return rc;
+    if (n) {
+        CG_HIP(hipSetDevice(b->device));
+        void *tmp = nullptr;
+        size_t cls = 0;
+        rc = b->pool.alloc(n * 2, &tmp, &cls);
+        if (!rc) {
+            rc = staged_upload(b, tmp, bits, n * 2);
+            if (!rc) rc = launch_bf16_widen(b, tmp, t->buf->ptr, n);
+            b->pool.free(tmp, cls); // stream-ordered: later users queue behind the widening kernel
+        }
+        if (rc) {
+            release(t);
+            return rc;
         }
     }
     *out = t;

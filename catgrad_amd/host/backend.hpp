@@ -36,7 +36,7 @@ struct Abi {
     CGH_FN(cg_backend_create) CGH_FN(cg_backend_destroy) CGH_FN(cg_last_error) CGH_FN(cg_backend_name) CGH_FN(cg_sync)
     CGH_FN(cg_pool_stats) CGH_FN(cg_program_stats) CGH_FN(cg_pool_trim) CGH_FN(cg_tensor_retain) CGH_FN(cg_tensor_release)
     CGH_FN(cg_tensor_rank) CGH_FN(cg_tensor_shape) CGH_FN(cg_tensor_dtype) CGH_FN(cg_tensor_numel)
-    CGH_FN(cg_tensor_is_contiguous) CGH_FN(cg_zeros) CGH_FN(cg_from_host) CGH_FN(cg_arange) CGH_FN(cg_to_host)
+    CGH_FN(cg_tensor_is_contiguous) CGH_FN(cg_zeros) CGH_FN(cg_from_host) CGH_FN(cg_from_host_bf16_as_f32) CGH_FN(cg_arange) CGH_FN(cg_to_host)
     CGH_FN(cg_to_bool) CGH_FN(cg_compare) CGH_FN(cg_format_tensor) CGH_FN(cg_cast) CGH_FN(cg_unary)
     CGH_FN(cg_binary) CGH_FN(cg_where) CGH_FN(cg_matmul) CGH_FN(cg_sum) CGH_FN(cg_max) CGH_FN(cg_argmax)
     CGH_FN(cg_topk) CGH_FN(cg_broadcast) CGH_FN(cg_reshape) CGH_FN(cg_transpose) CGH_FN(cg_slice)
@@ -53,7 +53,7 @@ struct Abi {
         CGH_LOAD(cg_backend_create) CGH_LOAD(cg_backend_destroy) CGH_LOAD(cg_last_error) CGH_LOAD(cg_backend_name)
         CGH_LOAD(cg_sync) CGH_LOAD(cg_pool_stats) CGH_LOAD(cg_program_stats) CGH_LOAD(cg_pool_trim) CGH_LOAD(cg_tensor_retain)
         CGH_LOAD(cg_tensor_release) CGH_LOAD(cg_tensor_rank) CGH_LOAD(cg_tensor_shape) CGH_LOAD(cg_tensor_dtype)
-        CGH_LOAD(cg_tensor_numel) CGH_LOAD(cg_tensor_is_contiguous) CGH_LOAD(cg_zeros) CGH_LOAD(cg_from_host)
+        CGH_LOAD(cg_tensor_numel) CGH_LOAD(cg_tensor_is_contiguous) CGH_LOAD(cg_zeros) CGH_LOAD(cg_from_host) CGH_LOAD(cg_from_host_bf16_as_f32)
         CGH_LOAD(cg_arange) CGH_LOAD(cg_to_host) CGH_LOAD(cg_to_bool) CGH_LOAD(cg_compare) CGH_LOAD(cg_format_tensor)
         CGH_LOAD(cg_cast) CGH_LOAD(cg_unary) CGH_LOAD(cg_binary) CGH_LOAD(cg_where) CGH_LOAD(cg_matmul) CGH_LOAD(cg_sum)
         CGH_LOAD(cg_max) CGH_LOAD(cg_argmax) CGH_LOAD(cg_topk) CGH_LOAD(cg_broadcast) CGH_LOAD(cg_reshape)
@@ -124,6 +124,12 @@ class Backend {
     }
     Tensor ndarray_from_vec_u32(const uint32_t *data, size_t len, const Shape &shape) {
         return from_vec(CG_U32, data, len, shape);
+    }
+    // Weight ingest (catgrad-llm/src/utils/mod.rs:158-168): f32 tensor from bfloat16 bit patterns.
+    Tensor from_bf16_bits(const uint16_t *bits, size_t len, const Shape &shape) {
+        return out([&](cg_tensor **o) {
+            return abi_.cg_from_host_bf16_as_f32(b_, bits, len, shape.data(), shape.size(), o);
+        });
     }
     Tensor cast(Tensor x, cg_dtype dt) {
         return out([&](cg_tensor **o) { return abi_.cg_cast(b_, x.into_raw(), dt, o); });

@@ -5,6 +5,7 @@
 #include <memory>
 
 #include "models.hpp"
+#include "weights.hpp"
 
 using namespace cgh;
 
@@ -53,6 +54,17 @@ int cgm_set_param(cgm_session *s, const char *path, const float *data, const siz
         size_t n = 1;
         for (size_t d : shape) n *= d;
         s->interp->parameters[path] = s->interp->backend.ndarray_from_vec_f32(data, n, shape);
+    });
+}
+
+int cgm_load_safetensors(cgm_session *s, const char *const *paths, size_t npaths, double *stats4) {
+    return guarded([&] {
+        std::vector<std::string> files(paths, paths + npaths);
+        LoadStats st = load_safetensors(*s->interp, files);
+        stats4[0] = (double)st.tensors;
+        stats4[1] = (double)st.params;
+        stats4[2] = (double)st.bytes;
+        stats4[3] = st.seconds;
     });
 }
 
@@ -128,6 +140,10 @@ int cgm_profile_enable(cgm_session *s, int kernel_class, unsigned sample_every) 
 
 int cgm_profile_read(cgm_session *s, int kernel_class, uint64_t *launches, double *milliseconds, double *work, int reset) {
     return guarded([&] { s->interp->backend.profile_read(kernel_class, launches, milliseconds, work, reset); });
+}
+
+int cgm_sync(cgm_session *s) {
+    return guarded([&] { s->interp->backend.sync(); });
 }
 
 int cgm_pool_stats(cgm_session *s, size_t *in_use, size_t *cached) {

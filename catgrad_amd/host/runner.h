@@ -19,6 +19,10 @@ const char *cgm_backend_name(cgm_session *s);
 /* Parameters::insert(path, interpreter::tensor(backend, shape, data)) */
 int cgm_set_param(cgm_session *s, const char *path, const float *data, const size_t *dims, size_t rank);
 int cgm_clear_params(cgm_session *s);
+/* Parameters from safetensors files (catgrad-llm/src/utils/mod.rs:321-449, dense tensors, f32 target):
+ * F32 and BF16 tensors become f32 parameters named as in the file, I64 tensors are skipped.
+ * stats4: [tensors loaded, parameters, bytes read, seconds]. */
+int cgm_load_safetensors(cgm_session *s, const char *const *paths, size_t npaths, double *stats4);
 
 /* arch: 0 = llama, 1 = qwen3 (dense). */
 int cgm_set_config(cgm_session *s, int arch, size_t hidden_size, size_t num_hidden_layers, size_t num_attention_heads,
@@ -42,6 +46,9 @@ int cgm_mlp(cgm_session *s, const float *x, size_t rows, size_t in_dim, size_t h
 /* Pass-through of the backend's launch-timing hooks (cg_profile_enable / cg_profile_read). */
 int cgm_profile_enable(cgm_session *s, int kernel_class, unsigned sample_every);
 int cgm_profile_read(cgm_session *s, int kernel_class, uint64_t *launches, double *milliseconds, double *work, int reset);
+
+/* Waits for everything queued on the backend's stream (cg_sync). */
+int cgm_sync(cgm_session *s);
 
 /* Bytes the backend's device pool has handed out / holds cached. */
 int cgm_pool_stats(cgm_session *s, size_t *in_use, size_t *cached);

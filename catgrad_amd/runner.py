@@ -34,11 +34,13 @@ def _host():
             "cgm_backend_name": (C.c_char_p, [P]),
             "cgm_set_param": (C.c_int, [P, C.c_char_p, P, SZP, SZ]),
             "cgm_clear_params": (C.c_int, [P]),
+            "cgm_load_safetensors": (C.c_int, [P, C.POINTER(C.c_char_p), SZ, C.POINTER(C.c_double)]),
             "cgm_set_config": (C.c_int, [P, C.c_int] + [SZ] * 7 + [C.c_float, C.c_float, C.c_int]),
             "cgm_generate": (C.c_int, [P, P, SZ, SZ, SZ, SZ, P, C.POINTER(C.c_double)]),
             "cgm_forward": (C.c_int, [P, P, SZ, SZ, SZ, P, P]),
             "cgm_mlp": (C.c_int, [P, P, SZ, SZ, SZ, SZ, P]),
             "cgm_pool_stats": (C.c_int, [P, SZP, SZP]),
+            "cgm_sync": (C.c_int, [P]),
             "cgm_program_stats": (C.c_int, [P, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64), C.c_int]),
             "cgm_profile_enable": (C.c_int, [P, C.c_int, C.c_uint]),
             "cgm_profile_read": (C.c_int, [P, C.c_int, C.POINTER(C.c_uint64), C.POINTER(C.c_double),
@@ -156,6 +158,27 @@ class Session:
     def clear_params(self):
         self._check(self._lib.cgm_clear_params(self._s))
 
+    def set_config(self, config: LlmConfig):
+        self._check(self._lib.cgm_set_config(
+            self._s, 0 if config.arch == "llama" else 1, config.hidden_size, config.num_hidden_layers,
+            config.num_attention_heads, config.num_key_value_heads, config.hd, config.intermediate_size,
+            config.vocab_size, config.rms_norm_eps, config.rope_theta, int(config.tie_word_embeddings)))
+        self.config = config
+
+    def load_safetensors(self, paths, config: LlmConfig = None):
+        """Parameters from safetensors files (F32 and BF16 tensors become f32, I64 is skipped), as
+        `load_model` of the reference does (catgrad-llm/src/utils/mod.rs:321-449).  Returns
+        {tensors, params, bytes, seconds}."""
+        if isinstance(paths, (str, os.PathLike)):
+            paths = [paths]
+        arr = (C.c_char_p * len(paths))(*[os.fspath(p).encode() for p in paths])
+        st = (C.c_double * 4)()
+        self.clear_params()
+        self._check(self._lib.cgm_load_safetensors(self._s, arr, len(paths), st))
+        if config is not None:
+            self.set_config(config)
+        return {"tensors": int(st[0]), "params": int(st[1]), "bytes": int(st[2]), "seconds": float(st[3])}
+
     def load_model(self, config: LlmConfig, params=None, seed: int = 0):
         self.clear_params()
         for name, w in (params if params is not None else random_params(config, seed)):
@@ -203,6 +226,9 @@ class Session:
         n, ms, w = C.c_uint64(), C.c_double(), C.c_double()
         self._check(self._lib.cgm_profile_read(self._s, cls, C.byref(n), C.byref(ms), C.byref(w), int(reset)))
         return int(n.value), float(ms.value), float(w.value)
+
+    def sync(self):
+        self._check(self._lib.cgm_sync(self._s))
 
     def program_stats(self, reset: bool = True):
         """(compiled, interpreted) launches of fused programs since the last reset."""

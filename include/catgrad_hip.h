@@ -156,6 +156,12 @@ int cg_zeros(cg_backend *b, cg_dtype dtype, const size_t *dims, size_t rank, cg_
  * f16/bf16/f8 return CG_ERR_UNSUPPORTED (ndarray.rs:98-120). */
 int cg_from_host(cg_backend *b, cg_dtype dtype, const void *data, size_t len,
                  const size_t *dims, size_t rank, cg_tensor **out);
+/* Weight ingest (catgrad-llm/src/utils/mod.rs:158-168 `decode_bf16_to_f32_into` followed by
+ * `interpreter::tensor`, utils/mod.rs:303-318): an f32 tensor from `len` bfloat16 bit patterns.
+ * The reference widens on the host with rayon and hands the backend f32; here the 2-byte
+ * values cross PCIe and are widened (bits << 16, exact) on the device. */
+int cg_from_host_bf16_as_f32(cg_backend *b, const uint16_t *bits, size_t len, const size_t *dims, size_t rank,
+                             cg_tensor **out);
 /* `Backend::arange` (mod.rs:107; ndarray.rs:134-138): u32 [0, end). */
 int cg_arange(cg_backend *b, size_t end, cg_tensor **out);
 

@@ -476,6 +476,21 @@ int cg_from_host(cg_backend *, cg_dtype dtype, const void *data, size_t len, con
     return CG_OK;
 }
 
+// catgrad-llm/src/utils/mod.rs:158-168 (`decode_bf16_to_f32_into`: bf16::to_f32 is the bit
+// pattern in the high half of an f32) followed by `interpreter::tensor` (mod.rs:23-33).
+int cg_from_host_bf16_as_f32(cg_backend *b, const uint16_t *bits, size_t len, const size_t *dims, size_t rank,
+                             cg_tensor **out) {
+    if (!b || !out || (len && !bits)) return fail(CG_ERR_ARG, "bad arguments");
+    size_t n = 1;
+    for (size_t i = 0; i < rank; i++) n *= dims[i];
+    if (n != len) return fail(CG_ERR_SHAPE, "ShapeError");
+    cg_tensor *t = new_tensor(CG_F32, dims, (int)rank);
+    uint32_t *dst = t->st->data.data();
+    for (size_t i = 0; i < n; i++) dst[i] = (uint32_t)bits[i] << 16;
+    *out = t;
+    return CG_OK;
+}
+
 // ndarray.rs:134-138: `Array::range(0.0, end as f32, 1.0)` then cast to u32.  The f32
 // detour is exact for end <= 2^24; above that the reference itself is inexact.
 int cg_arange(cg_backend *, size_t end, cg_tensor **out) {
