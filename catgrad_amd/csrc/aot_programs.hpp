@@ -14,42 +14,44 @@
 
 #include <utility>
 
-#define CG_PROGRAM(NAME, NLEAF, UNIFORM, ...)                          \
+#define CG_PROGRAM(NAME, NLEAF, UNIFORM, PW, ...)                      \
     struct NAME {                                                      \
         static constexpr int nleaf = NLEAF;                            \
         static constexpr unsigned uniform = UNIFORM; /* bit l: leaf l is a constant */ \
+        static constexpr int pw = PW; /* the piecewise leaf (a deferred last-axis concat), -1: none */ \
         static constexpr uint8_t code[][4] = {__VA_ARGS__};            \
         static constexpr int ninstr = (int)(sizeof(code) / 4);         \
     };
 
-// op codes: 0 neg, 3 exp, 16 add, 17 sub, 18 mul, 19 div, 20 pow, 48 row-sum, 49 row-max;
+// op codes: 0 neg, 3 exp, 16 add, 17 sub, 18 mul, 19 div, 20 pow, 42 copy, 48 row-sum, 49 row-max;
 // +128 = u32 operands (149 = u32 lt, 169 = cast u32 -> f32).  Registers 0..7 are leaves,
 // 8 + i is the result of instruction i.  Which leaves are constants is part of a program's
 // identity: the compiler then sees that whatever depends only on constants and row results
 // (the square root of an RMS norm) does not change along a row and computes it once.
 
 // ---- element-wise ------------------------------------------------------------------------
-// x * cos + rotate_half(x) * sin                         (rotary embedding)
-CG_PROGRAM(MapRope, 4, 0x0, {18, 0, 1, 0}, {18, 2, 3, 2}, {16, 8, 9, 8})
+// cos * x + sin * rotate_half(x), rotate_half(x) = concat(-x2, x1) read in place as the
+// piecewise leaf 3                                        (rotary embedding)
+CG_PROGRAM(MapRope, 4, 0x0, 3, {18, 0, 1, 0}, {42, 3, 3, 3}, {18, 2, 9, 2}, {16, 8, 10, 8})
 // g * (1 / (1 + exp(-g))) * u                            (SiLU gate times up projection)
-CG_PROGRAM(MapSiluMul, 3, 0x2, {0, 0, 0, 0}, {3, 8, 8, 8}, {16, 1, 9, 1}, {19, 1, 10, 1}, {18, 0, 11, 0}, {18, 12, 2, 12})
+CG_PROGRAM(MapSiluMul, 3, 0x2, -1, {0, 0, 0, 0}, {3, 8, 8, 8}, {16, 1, 9, 1}, {19, 1, 10, 1}, {18, 0, 11, 0}, {18, 12, 2, 12})
 // residual stream after three adds, in the two operand orders the layer loop produces
-CG_PROGRAM(MapResidual3a, 4, 0x0, {16, 1, 2, 1}, {16, 0, 8, 0}, {16, 9, 3, 9})
-CG_PROGRAM(MapResidual3b, 4, 0x0, {16, 1, 2, 1}, {16, 8, 3, 8}, {16, 0, 9, 0})
+CG_PROGRAM(MapResidual3a, 4, 0x0, -1, {16, 1, 2, 1}, {16, 0, 8, 0}, {16, 9, 3, 9})
+CG_PROGRAM(MapResidual3b, 4, 0x0, -1, {16, 1, 2, 1}, {16, 8, 3, 8}, {16, 0, 9, 0})
 
 // ---- with row reduces ------------------------------------------------------------------------
 // x / sqrt(sum(x*x)/n + eps) * gamma                     (RMS norm)
-CG_PROGRAM(RowsRmsNorm, 5, 0xE, {18, 0, 0, 0}, {48, 8, 8, 8}, {19, 9, 1, 9}, {16, 10, 2, 10}, {20, 11, 3, 11},
+CG_PROGRAM(RowsRmsNorm, 5, 0xE, -1, {18, 0, 0, 0}, {48, 8, 8, 8}, {19, 9, 1, 9}, {16, 10, 2, 10}, {20, 11, 3, 11},
            {19, 0, 12, 0}, {18, 13, 4, 13})
 // the same on h = a + b, and on h = a + (b + c) / (a + b) + c
-CG_PROGRAM(RowsRmsNormAdd, 6, 0x1C, {16, 0, 1, 0}, {18, 8, 8, 8}, {48, 9, 9, 9}, {19, 10, 2, 10}, {16, 11, 3, 11},
+CG_PROGRAM(RowsRmsNormAdd, 6, 0x1C, -1, {16, 0, 1, 0}, {18, 8, 8, 8}, {48, 9, 9, 9}, {19, 10, 2, 10}, {16, 11, 3, 11},
            {20, 12, 4, 12}, {19, 8, 13, 8}, {18, 14, 5, 14})
-CG_PROGRAM(RowsRmsNormAdd2a, 7, 0x38, {16, 1, 2, 1}, {16, 0, 8, 0}, {18, 9, 9, 9}, {48, 10, 10, 10}, {19, 11, 3, 11},
+CG_PROGRAM(RowsRmsNormAdd2a, 7, 0x38, -1, {16, 1, 2, 1}, {16, 0, 8, 0}, {18, 9, 9, 9}, {48, 10, 10, 10}, {19, 11, 3, 11},
            {16, 12, 4, 12}, {20, 13, 5, 13}, {19, 9, 14, 9}, {18, 15, 6, 15})
-CG_PROGRAM(RowsRmsNormAdd2b, 7, 0x38, {16, 0, 1, 0}, {16, 8, 2, 8}, {18, 9, 9, 9}, {48, 10, 10, 10}, {19, 11, 3, 11},
+CG_PROGRAM(RowsRmsNormAdd2b, 7, 0x38, -1, {16, 0, 1, 0}, {16, 8, 2, 8}, {18, 9, 9, 9}, {48, 10, 10, 10}, {19, 11, 3, 11},
            {16, 12, 4, 12}, {20, 13, 5, 13}, {19, 9, 14, 9}, {18, 15, 6, 15})
 // softmax(s / d + f32(j < i) * m): attention scores, causal mask built from two index vectors
-CG_PROGRAM(RowsSoftmaxCausal, 5, 0x12, {19, 0, 1, 0}, {149, 2, 3, 2}, {169, 9, 9, 9}, {18, 10, 4, 10}, {16, 8, 11, 8},
+CG_PROGRAM(RowsSoftmaxCausal, 5, 0x12, -1, {19, 0, 1, 0}, {149, 2, 3, 2}, {169, 9, 9, 9}, {18, 10, 4, 10}, {16, 8, 11, 8},
            {49, 12, 12, 12}, {17, 12, 13, 12}, {3, 14, 14, 14}, {48, 15, 15, 15}, {19, 15, 16, 15})
 
 template <class... P> struct ProgramList {};
@@ -59,7 +61,7 @@ using RowsPrograms = ProgramList<RowsRmsNorm, RowsRmsNormAdd, RowsRmsNormAdd2a, 
 template <class P> bool program_matches(const Pending &p) {
     if (p.nleaf != P::nleaf || p.ninstr != P::ninstr) return false;
     for (int l = 0; l < P::nleaf; l++)
-        if (p.leaf[l].uniform != (((P::uniform >> l) & 1u) != 0)) return false;
+        if (p.leaf[l].uniform != (((P::uniform >> l) & 1u) != 0) || p.leaf[l].pw != (l == P::pw)) return false;
     for (int i = 0; i < P::ninstr; i++) {
         const Instr &in = p.ins[i];
         if (in.op != P::code[i][0] || in.a != P::code[i][1] || in.b != P::code[i][2] || in.c != P::code[i][3])
@@ -107,17 +109,31 @@ __device__ __forceinline__ void aot_run(Values<P, VEC> &s, const uint32_t (&rs)[
     (aot_step<P, VEC, I>(s, rs, fault), ...);
 }
 
-template <class P, int VEC>
-__device__ __forceinline__ void aot_load(const FusedArgs &a, const int64_t (&off)[P::nleaf], Values<P, VEC> &s) {
+// Leaf l of the work item at position e of its row; off[nleaf] is the offset into the second
+// part of the piecewise leaf (unused when the program has none).
+template <class P, int VEC, int L>
+__device__ __forceinline__ void aot_load_leaf(const FusedArgs &a, const int64_t (&off)[P::nleaf + 1], uint32_t e,
+                                              uint32_t (&t)[VEC]) {
+    if constexpr ((P::uniform >> L) & 1u) {
 #pragma unroll
-    for (int l = 0; l < P::nleaf; l++) {
-        if ((P::uniform >> l) & 1u) {
+        for (int j = 0; j < VEC; j++) t[j] = a.leaf[L].ubits;
+    } else if constexpr (L == P::pw) {
+        const bool second = e >= a.pw_split;
+        if (second) load_words<VEC>(a.leaf2, off[P::nleaf], t);
+        else load_words<VEC>(a.leaf[L], off[L], t);
+        if ((a.pw_neg >> (second ? 1 : 0)) & 1u) {
 #pragma unroll
-            for (int j = 0; j < VEC; j++) s.v[l][j] = a.leaf[l].ubits;
-        } else {
-            load_words<VEC>(a.leaf[l], off[l], s.v[l]);
+            for (int j = 0; j < VEC; j++) t[j] ^= 0x80000000u;
         }
+    } else {
+        load_words<VEC>(a.leaf[L], off[L], t);
     }
+}
+
+template <class P, int VEC, int... L>
+__device__ __forceinline__ void aot_load_all(const FusedArgs &a, const int64_t (&off)[P::nleaf + 1], uint32_t e,
+                                             uint32_t (&v)[P::nleaf][VEC], std::integer_sequence<int, L...>) {
+    (aot_load_leaf<P, VEC, L>(a, off, e, v[L]), ...);
 }
 
 // ---- element-wise kernel: the geometry of fused_kernel, the program compiled in ----------------------
@@ -128,9 +144,10 @@ template <class P, int VEC> __global__ __launch_bounds__(kBlock) void aot_map_ke
     uint32_t row = fastdiv(v, a.g.ipr_div);
     const int64_t e = (int64_t)(v - row * a.g.ipr) * VEC;
     int64_t oo = e * a.out.is;
-    int64_t off[P::nleaf];
+    int64_t off[P::nleaf + 1];
 #pragma unroll
     for (int l = 0; l < P::nleaf; l++) off[l] = e * a.leaf[l].is;
+    off[P::nleaf] = (e - (int64_t)a.pw_split) * a.leaf2.is;
     for (uint32_t d = 0; d < a.g.nouter; d++) {
         const uint32_t q = fastdiv(row, a.g.odiv[d]);
         const int64_t i = (int64_t)(row - q * a.g.od[d]);
@@ -138,9 +155,17 @@ template <class P, int VEC> __global__ __launch_bounds__(kBlock) void aot_map_ke
         oo += i * a.out.os[d];
 #pragma unroll
         for (int l = 0; l < P::nleaf; l++) off[l] += i * a.leaf[l].os[d];
+        if constexpr (P::pw >= 0) off[P::nleaf] += i * a.leaf2.os[d];
     }
     Values<P, VEC> s;
-    aot_load<P, VEC>(a, off, s);
+    {
+        uint32_t lw[P::nleaf][VEC];
+        aot_load_all<P, VEC>(a, off, (uint32_t)e, lw, std::make_integer_sequence<int, P::nleaf>{});
+#pragma unroll
+        for (int l = 0; l < P::nleaf; l++)
+#pragma unroll
+            for (int j = 0; j < VEC; j++) s.v[l][j] = lw[l][j];
+    }
     const uint32_t rs[kMaxRowReduce] = {0, 0, 0};
     aot_run<P, VEC>(s, rs, a.fault, std::make_integer_sequence<int, P::ninstr>{});
     store_words<VEC>(a.out, oo, s.v[kMaxLeaves + P::ninstr - 1]);
@@ -155,17 +180,13 @@ template <class P, int VEC> struct LeafWords {
 };
 
 template <class P, int VEC>
-__device__ __forceinline__ void aot_fetch(const FusedArgs &a, const int64_t (&base)[P::nleaf], uint32_t it,
+__device__ __forceinline__ void aot_fetch(const FusedArgs &a, const int64_t (&base)[P::nleaf + 1], uint32_t it,
                                           LeafWords<P, VEC> &w) {
+    int64_t off[P::nleaf + 1];
 #pragma unroll
-    for (int l = 0; l < P::nleaf; l++) {
-        if ((P::uniform >> l) & 1u) {
-#pragma unroll
-            for (int j = 0; j < VEC; j++) w.v[l][j] = a.leaf[l].ubits;
-        } else {
-            load_words<VEC>(a.leaf[l], base[l] + (int64_t)it * VEC * a.leaf[l].is, w.v[l]);
-        }
-    }
+    for (int l = 0; l < P::nleaf; l++) off[l] = base[l] + (int64_t)it * VEC * a.leaf[l].is;
+    off[P::nleaf] = base[P::nleaf] + ((int64_t)it * VEC - (int64_t)a.pw_split) * a.leaf2.is;
+    aot_load_all<P, VEC>(a, off, it * VEC, w.v, std::make_integer_sequence<int, P::nleaf>{});
 }
 
 // Value of instructions [0, UPTO) on one work item; returns the register file.
@@ -198,7 +219,7 @@ template <bool IS_MAX, bool F, int TPR> __device__ __forceinline__ uint32_t aot_
 }
 
 template <class P, int VEC, int TPR, int CI, int PHASE>
-__device__ __forceinline__ void aot_rows_phase(const FusedArgs &a, const int64_t (&base)[P::nleaf], uint32_t lane, bool live,
+__device__ __forceinline__ void aot_rows_phase(const FusedArgs &a, const int64_t (&base)[P::nleaf + 1], uint32_t lane, bool live,
                                                uint32_t items, const LeafWords<P, VEC> (&cache)[CI > 0 ? CI : 1],
                                                uint32_t (&rs)[kMaxRowReduce]) {
     constexpr int ri = reduce_index<P>(PHASE);
@@ -228,7 +249,7 @@ __device__ __forceinline__ void aot_rows_phase(const FusedArgs &a, const int64_t
 }
 
 template <class P, int VEC, int TPR, int CI, int... PH>
-__device__ __forceinline__ void aot_rows_phases(const FusedArgs &a, const int64_t (&base)[P::nleaf], uint32_t lane, bool live,
+__device__ __forceinline__ void aot_rows_phases(const FusedArgs &a, const int64_t (&base)[P::nleaf + 1], uint32_t lane, bool live,
                                                 uint32_t items, const LeafWords<P, VEC> (&cache)[CI > 0 ? CI : 1],
                                                 uint32_t (&rs)[kMaxRowReduce], std::integer_sequence<int, PH...>) {
     (aot_rows_phase<P, VEC, TPR, CI, PH>(a, base, lane, live, items, cache, rs), ...);
@@ -241,9 +262,9 @@ __global__ __launch_bounds__(kBlock) void aot_rows_kernel(const FusedArgs a, uin
     const uint32_t lane = threadIdx.x % TPR;
     const uint32_t row = blockIdx.x * RPB + threadIdx.x / TPR;
     const bool live = row < a.rows;
-    int64_t base[P::nleaf];
+    int64_t base[P::nleaf + 1];
 #pragma unroll
-    for (int l = 0; l < P::nleaf; l++) base[l] = 0;
+    for (int l = 0; l <= P::nleaf; l++) base[l] = 0;
     int64_t obase = 0;
     if (live) {
         uint32_t rr = row;
@@ -254,6 +275,7 @@ __global__ __launch_bounds__(kBlock) void aot_rows_kernel(const FusedArgs a, uin
             obase += i * a.out.os[d];
 #pragma unroll
             for (int l = 0; l < P::nleaf; l++) base[l] += i * a.leaf[l].os[d];
+            if constexpr (P::pw >= 0) base[P::nleaf] += i * a.leaf2.os[d];
         }
     }
     const uint32_t items = a.n / VEC;

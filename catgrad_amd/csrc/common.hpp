@@ -221,6 +221,16 @@ struct LeafView {
     int64_t offset = 0;
     bool uniform = false;
     uint32_t ubits = 0;
+    // Piecewise leaf (the deferred form of `concat` along the last axis): positions below
+    // `pw_split` of the last axis read the view above, the others read (buf2, strides2,
+    // offset2) at position - pw_split; a part may be negated on load (f32 sign flip), which
+    // is how rotate_half = concat(-x2, x1) of the rotary embedding stays a leaf.
+    bool pw = false;
+    Buffer *buf2 = nullptr; // retained
+    int64_t strides2[kMaxRank] = {0};
+    int64_t offset2 = 0;
+    int64_t pw_split = 0;
+    bool neg1 = false, neg2 = false;
 };
 
 struct Pending {
@@ -243,6 +253,7 @@ struct ViewDesc {
     bool uniform;
     uint32_t ubits;
     const char *ptr; // device address of the view's first element (unused when uniform)
+    int64_t vec_period = 0; // > 0: 16-byte vectors are only allowed if this divides by 4 (a piecewise leaf's split)
 };
 // Collapses the iteration space shared by `n` views of shape `dims` (v[0] is the output)
 // and fills geometry + operands.  keep_last_axis: never merge the last axis into the one

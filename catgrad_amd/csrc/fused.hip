@@ -47,7 +47,30 @@ struct FusedArgs {
     // programs with row-reduce instructions only
     uint32_t nred, reduced;
     uint8_t red_op[4]; // op code of the k-th row reduce
+    // the piecewise leaf, if any (pw_leaf < 0: none): elements of the row at or beyond pw_split come
+    // from `leaf2`, addressed with (position - pw_split); pw_neg bit 0 / 1: negate part 1 / 2
+    int32_t pw_leaf;
+    uint32_t pw_split, pw_neg;
+    Operand leaf2;
 };
+
+// Leaf `l` of the work item that starts at position `e` of its row: `off` is the element offset
+// in the leaf's (first) view, `off2` the offset in the second part of the piecewise leaf.
+template <int VEC>
+__device__ __forceinline__ void load_leaf(const FusedArgs &a, int l, int64_t off, int64_t off2, uint32_t e,
+                                          uint32_t (&t)[VEC]) {
+    if (l != a.pw_leaf) {
+        load_words<VEC>(a.leaf[l], off, t);
+        return;
+    }
+    const bool second = e >= a.pw_split; // a vector never straddles the split (it is a multiple of VEC)
+    if (second) load_words<VEC>(a.leaf2, off2, t);
+    else load_words<VEC>(a.leaf[l], off, t);
+    if ((a.pw_neg >> (second ? 1 : 0)) & 1u) {
+#pragma unroll
+        for (int j = 0; j < VEC; j++) t[j] ^= 0x80000000u;
+    }
+}
 
 // One instruction on the VEC elements of a work item.  op is wave-uniform, so the switch is
 // a scalar branch, and the VEC applications inside a case are independent (they interleave
@@ -86,13 +109,14 @@ __device__ __forceinline__ void apply_rt(uint32_t op, const uint32_t (&x)[VEC], 
 
 // Loads the leaves of one work item and runs the program; result in res[VEC].
 template <int VEC, bool FULL>
-__device__ __forceinline__ void eval_program(const FusedArgs &a, const int64_t (&off)[kMaxLeaves], uint32_t (&res)[VEC]) {
+__device__ __forceinline__ void eval_program(const FusedArgs &a, const int64_t (&off)[kMaxLeaves], int64_t off2, uint32_t e,
+                                             uint32_t (&res)[VEC]) {
     regfile r[VEC];
 #pragma unroll
     for (int l = 0; l < kMaxLeaves; l++) {
         if ((uint32_t)l < a.nleaf) {
             uint32_t t[VEC];
-            load_words<VEC>(a.leaf[l], off[l], t);
+            load_leaf<VEC>(a, l, off[l], off2, e, t);
 #pragma unroll
             for (int j = 0; j < VEC; j++) r[j][l] = t[j];
         }
@@ -127,17 +151,19 @@ template <int VEC, bool FULL> __global__ __launch_bounds__(kBlock) void fused_ke
     int64_t off[kMaxLeaves];
 #pragma unroll
     for (int l = 0; l < kMaxLeaves; l++) off[l] = (uint32_t)l < a.nleaf ? e * a.leaf[l].is : 0;
+    int64_t off2 = (e - (int64_t)a.pw_split) * a.leaf2.is;
     for (uint32_t d = 0; d < a.g.nouter; d++) {
         const uint32_t q = fastdiv(row, a.g.odiv[d]);
         const int64_t i = (int64_t)(row - q * a.g.od[d]);
         row = q;
         oo += i * a.out.os[d];
+        off2 += i * a.leaf2.os[d];
 #pragma unroll
         for (int l = 0; l < kMaxLeaves; l++)
             if ((uint32_t)l < a.nleaf) off[l] += i * a.leaf[l].os[d];
     }
     uint32_t res[VEC];
-    eval_program<VEC, FULL>(a, off, res);
+    eval_program<VEC, FULL>(a, off, off2, (uint32_t)e, res);
     store_words<VEC>(a.out, oo, res);
 }
 
@@ -202,10 +228,12 @@ __global__ __launch_bounds__(kBlock) void fused_reduce_kernel(const FusedArgs a,
 #pragma unroll
         for (int l = 0; l < kMaxLeaves; l++) base[l] = 0;
         uint32_t rr = row;
+        int64_t base2 = 0;
         for (uint32_t d = 0; d < a.g.nouter; d++) {
             const uint32_t q = fastdiv(rr, a.g.odiv[d]);
             const int64_t i = (int64_t)(rr - q * a.g.od[d]);
             rr = q;
+            base2 += i * a.leaf2.os[d];
 #pragma unroll
             for (int l = 0; l < kMaxLeaves; l++)
                 if ((uint32_t)l < a.nleaf) base[l] += i * a.leaf[l].os[d];
@@ -216,8 +244,9 @@ __global__ __launch_bounds__(kBlock) void fused_reduce_kernel(const FusedArgs a,
 #pragma unroll
             for (int l = 0; l < kMaxLeaves; l++)
                 off[l] = (uint32_t)l < a.nleaf ? base[l] + (int64_t)it * VEC * a.leaf[l].is : 0;
+            const int64_t off2 = base2 + ((int64_t)it * VEC - (int64_t)a.pw_split) * a.leaf2.is;
             uint32_t res[VEC];
-            eval_program<VEC, FULL>(a, off, res);
+            eval_program<VEC, FULL>(a, off, off2, it * VEC, res);
 #pragma unroll
             for (int j = 0; j < VEC; j++) acc.take(kind, f, res[j], it * VEC + j);
         }
@@ -252,14 +281,14 @@ __device__ __forceinline__ uint32_t row_merge(bool is_max, bool f, uint32_t c, u
 // their finished row value from rs, the operand of reduce `phase` is returned in res (true),
 // and with phase == nred the whole program runs and res is its value (false).
 template <int VEC, bool FULL>
-__device__ __forceinline__ bool eval_rows(const FusedArgs &a, const int64_t (&off)[kMaxLeaves],
+__device__ __forceinline__ bool eval_rows(const FusedArgs &a, const int64_t (&off)[kMaxLeaves], int64_t off2, uint32_t e,
                                           const uint32_t (&rs)[kMaxRowReduce], uint32_t phase, uint32_t (&res)[VEC]) {
     regfile r[VEC];
 #pragma unroll
     for (int l = 0; l < kMaxLeaves; l++) {
         if ((uint32_t)l < a.nleaf) {
             uint32_t t[VEC];
-            load_words<VEC>(a.leaf[l], off[l], t);
+            load_leaf<VEC>(a, l, off[l], off2, e, t);
 #pragma unroll
             for (int j = 0; j < VEC; j++) r[j][l] = t[j];
         }
@@ -314,7 +343,7 @@ __global__ __launch_bounds__(kBlock) void fused_rows_kernel(const FusedArgs a, u
     int64_t base[kMaxLeaves];
 #pragma unroll
     for (int l = 0; l < kMaxLeaves; l++) base[l] = 0;
-    int64_t obase = 0;
+    int64_t obase = 0, base2 = 0;
     if (live) {
         uint32_t rr = row;
         for (uint32_t d = 0; d < a.g.nouter; d++) {
@@ -322,6 +351,7 @@ __global__ __launch_bounds__(kBlock) void fused_rows_kernel(const FusedArgs a, u
             const int64_t i = (int64_t)(rr - q * a.g.od[d]);
             rr = q;
             obase += i * a.out.os[d];
+            base2 += i * a.leaf2.os[d];
 #pragma unroll
             for (int l = 0; l < kMaxLeaves; l++)
                 if ((uint32_t)l < a.nleaf) base[l] += i * a.leaf[l].os[d];
@@ -339,8 +369,9 @@ __global__ __launch_bounds__(kBlock) void fused_rows_kernel(const FusedArgs a, u
 #pragma unroll
                 for (int l = 0; l < kMaxLeaves; l++)
                     off[l] = (uint32_t)l < a.nleaf ? base[l] + (int64_t)it * VEC * a.leaf[l].is : 0;
+                const int64_t off2 = base2 + ((int64_t)it * VEC - (int64_t)a.pw_split) * a.leaf2.is;
                 uint32_t res[VEC];
-                eval_rows<VEC, FULL>(a, off, rs, phase, res);
+                eval_rows<VEC, FULL>(a, off, off2, it * VEC, rs, phase, res);
 #pragma unroll
                 for (int j = 0; j < VEC; j++) acc = row_merge(is_max, f, acc, res[j]);
             }
@@ -370,7 +401,7 @@ __global__ __launch_bounds__(kBlock) void fused_rows_kernel(const FusedArgs a, u
 #pragma unroll
             for (int l = 0; l < kMaxLeaves; l++) off[l] = base[l];
             uint32_t res[VEC];
-            eval_rows<VEC, FULL>(a, off, rs, a.nred, res);
+            eval_rows<VEC, FULL>(a, off, base2 - (int64_t)a.pw_split * a.leaf2.is, 0, rs, a.nred, res);
             rowout[row] = res[0];
         }
         return;
@@ -380,8 +411,9 @@ __global__ __launch_bounds__(kBlock) void fused_rows_kernel(const FusedArgs a, u
 #pragma unroll
         for (int l = 0; l < kMaxLeaves; l++)
             off[l] = (uint32_t)l < a.nleaf ? base[l] + (int64_t)it * VEC * a.leaf[l].is : 0;
+        const int64_t off2 = base2 + ((int64_t)it * VEC - (int64_t)a.pw_split) * a.leaf2.is;
         uint32_t res[VEC];
-        eval_rows<VEC, FULL>(a, off, rs, a.nred, res);
+        eval_rows<VEC, FULL>(a, off, off2, it * VEC, rs, a.nred, res);
         store_words<VEC>(a.out, obase + (int64_t)it * VEC * a.out.is, res);
     }
 }
@@ -422,7 +454,7 @@ int fill_args(cg_backend *be, const Pending &p, const int64_t *dims, int rank, c
               FusedArgs *a, double *leaf_bytes, bool *full, int ninstr = -1) {
     if (ninstr < 0) ninstr = p.ninstr;
     memset(a, 0, sizeof *a);
-    ViewDesc v[kMaxViews];
+    ViewDesc v[kMaxViews + 1];
     int64_t out_strides[kMaxRank];
     if (out) {
         const void *op;
@@ -444,12 +476,24 @@ int fill_args(cg_backend *be, const Pending &p, const int64_t *dims, int rank, c
         v[0].ptr = nullptr;
     }
     double bytes = 0.0;
+    int pw_leaf = -1;
     for (int l = 0; l < p.nleaf; l++) {
         const LeafView &lv = p.leaf[l];
         v[l + 1].strides = lv.strides;
         v[l + 1].uniform = lv.uniform;
         v[l + 1].ubits = lv.ubits;
         v[l + 1].ptr = lv.uniform ? nullptr : static_cast<const char *>(lv.buf->ptr) + lv.offset * 4;
+        v[l + 1].vec_period = 0;
+        if (lv.pw) { // its second part is planned as one more view, and the row axis stays on its own
+            pw_leaf = l;
+            v[l + 1].vec_period = lv.pw_split;
+            ViewDesc &w = v[p.nleaf + 1];
+            w.strides = lv.strides2;
+            w.uniform = false;
+            w.ubits = 0;
+            w.ptr = static_cast<const char *>(lv.buf2->ptr) + lv.offset2 * 4;
+            w.vec_period = lv.pw_split;
+        }
         if (!lv.uniform) {
             double n = 1.0;
             for (int i = 0; i < rank; i++)
@@ -457,15 +501,24 @@ int fill_args(cg_backend *be, const Pending &p, const int64_t *dims, int rank, c
             bytes += 4.0 * n;
         }
     }
-    Operand ops[kMaxViews];
+    Operand ops[kMaxViews + 1];
     // Small problems are latency-bound: one element per lane keeps each lane's serial chain
     // (operand moves, long routines) four times shorter and still fills the chip.
     int64_t elems = 1;
     for (int i = 0; i < rank; i++) elems *= dims[i];
-    int rc = plan_views(dims, rank, v, p.nleaf + 1, keep_last, &a->g, ops, keep_last || elems > 32768);
+    int rc = plan_views(dims, rank, v, p.nleaf + 1 + (pw_leaf >= 0 ? 1 : 0), keep_last || pw_leaf >= 0, &a->g, ops,
+                        keep_last || elems > 32768);
     if (rc) return rc;
     a->out = ops[0];
     for (int l = 0; l < p.nleaf; l++) a->leaf[l] = ops[l + 1];
+    a->pw_leaf = pw_leaf;
+    if (pw_leaf >= 0) {
+        const LeafView &lv = p.leaf[pw_leaf];
+        if (lv.pw_split > 0xFFFFFFFFll) return fail(CG_ERR_UNSUPPORTED, "concat: last axis above 2^32-1 elements");
+        a->leaf2 = ops[p.nleaf + 1];
+        a->pw_split = (uint32_t)lv.pw_split;
+        a->pw_neg = (lv.neg1 ? 1u : 0u) | (lv.neg2 ? 2u : 0u);
+    }
     a->nleaf = (uint32_t)p.nleaf;
     a->ninstr = (uint32_t)ninstr;
     uint8_t phys[kMaxLeaves + kMaxInstr];
@@ -509,7 +562,7 @@ void trace_program(cg_backend *be, const Pending &p, int ninstr, const char *how
     std::lock_guard<std::mutex> lk(mu);
     if (!seen.insert(key).second) return;
     std::string where = " uniform=";
-    for (int l = 0; l < p.nleaf; l++) where += p.leaf[l].uniform ? '1' : '0';
+    for (int l = 0; l < p.nleaf; l++) where += p.leaf[l].pw ? 'p' : p.leaf[l].uniform ? '1' : '0';
     where += " dims=[";
     for (int i = 0; i < rank; i++) {
         snprintf(buf, sizeof buf, "%s%lld", i ? "," : "", (long long)dims[i]);

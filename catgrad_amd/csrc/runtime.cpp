@@ -124,12 +124,16 @@ Pending::Pending(const Pending &o)
     for (int l = 0; l < nleaf; l++) {
         leaf[l] = o.leaf[l];
         if (leaf[l].buf) leaf[l].buf->rc.fetch_add(1);
+        if (leaf[l].buf2) leaf[l].buf2->rc.fetch_add(1);
     }
     for (int i = 0; i < ninstr; i++) ins[i] = o.ins[i];
 }
 
 Pending::~Pending() {
-    for (int l = 0; l < nleaf; l++) buffer_release(leaf[l].buf);
+    for (int l = 0; l < nleaf; l++) {
+        buffer_release(leaf[l].buf);
+        buffer_release(leaf[l].buf2);
+    }
 }
 
 void release(cg_tensor *t) {
@@ -247,7 +251,7 @@ int plan_views(const int64_t *vdims, int vrank, const ViewDesc *v, int n, bool k
                Operand *ops, bool allow_vec4) {
     int r = 0;
     int64_t dims[kMaxRank];
-    int64_t st[kMaxViews][kMaxRank];
+    int64_t st[kMaxViews + 1][kMaxRank];
     bool last_kept = false;
     for (int i = 0; i < vrank; i++) {
         const bool is_last = i == vrank - 1;
@@ -293,6 +297,7 @@ int plan_views(const int64_t *vdims, int vrank, const ViewDesc *v, int n, bool k
         o.ptr = v[k].uniform ? nullptr : v[k].ptr;
         o.is = st[k][r - 1];
         for (int d = 0; d < r - 1; d++) o.os[d] = st[k][r - 2 - d];
+        if (v[k].vec_period > 0 && v[k].vec_period % 4) vec4 = false;
         if (!o.uniform && o.is == 1) {
             if (reinterpret_cast<uintptr_t>(o.ptr) % 16) vec4 = false;
             for (int d = 0; d < r - 1; d++)
@@ -558,7 +563,9 @@ static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p) {
         }
         return launch_fused_rows(be, dst, p, space.dims, space.rank);
     }
-    if (p.ninstr == 1) {
+    bool piecewise = false;
+    for (int l = 0; l < p.nleaf; l++) piecewise = piecewise || p.leaf[l].pw;
+    if (p.ninstr == 1 && !piecewise) {
         const Instr in = p.ins[0];
         const int op = in.op & ~kInstrU32;
         const cg_dtype dt = (in.op & kInstrU32) ? CG_U32 : CG_F32;
@@ -630,23 +637,32 @@ static int ensure_concrete(cg_tensor *t) {
 }
 
 static bool same_leaf(const LeafView &a, const LeafView &b, const int64_t *dims, int rank) {
-    if (a.uniform != b.uniform) return false;
+    if (a.uniform != b.uniform || a.pw != b.pw) return false;
     if (a.uniform) return a.ubits == b.ubits;
     if (a.buf != b.buf || a.offset != b.offset) return false;
     for (int i = 0; i < rank; i++)
         if (dims[i] > 1 && a.strides[i] != b.strides[i]) return false;
+    if (a.pw) {
+        if (a.buf2 != b.buf2 || a.offset2 != b.offset2 || a.pw_split != b.pw_split || a.neg1 != b.neg1 || a.neg2 != b.neg2)
+            return false;
+        for (int i = 0; i < rank; i++)
+            if (dims[i] > 1 && a.strides2[i] != b.strides2[i]) return false;
+    }
     return true;
 }
 
 static int add_leaf(Pending *p, const LeafView &lv, const int64_t *dims, int rank) {
     for (int l = 0; l < p->nleaf; l++)
         if (same_leaf(p->leaf[l], lv, dims, rank)) return l;
-    if (p->nleaf == kMaxLeaves) {
+    bool second_pw = false; // the kernels address one piecewise leaf per program
+    for (int l = 0; l < p->nleaf; l++) second_pw = second_pw || (lv.pw && p->leaf[l].pw);
+    if (p->nleaf == kMaxLeaves || second_pw) {
         p->overflow = true;
         return 0;
     }
     p->leaf[p->nleaf] = lv;
     if (lv.buf) lv.buf->rc.fetch_add(1);
+    if (lv.buf2) lv.buf2->rc.fetch_add(1);
     return p->nleaf++;
 }
 
@@ -861,6 +877,8 @@ static int pending_view(cg_tensor *x, const int64_t *dims, int rank, F &&fn, cg_
     *handled = false;
     if (!x->pend) return CG_OK;
     if (x->pend->nred > 0) return ensure_concrete(x); // rows do not survive re-striding
+    for (int l = 0; l < x->pend->nleaf; l++)
+        if (x->pend->leaf[l].pw) return ensure_concrete(x); // nor does a split of the last axis
     int64_t n = 1;
     for (int i = 0; i < rank; i++) n *= dims[i];
     const bool grows = n > numel(x);
@@ -1940,6 +1958,52 @@ int cg_concat(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor *
     {
         int arc;
         if (try_row_append(b, x, y, dim, out, &arc)) return arc;
+    }
+    if (b->fuse && dim == (size_t)x->rank - 1 && numel(x) > 0 && numel(y) > 0) {
+        // Along the last axis the result can stay deferred as one piecewise leaf when each
+        // operand is a plain view, or the negation of one (rotate_half of the rotary embedding,
+        // helpers/rope.rs:423-427): its consumer then reads both halves in place.
+        LeafView lv;
+        auto part = [&](cg_tensor *t, Buffer **buf, int64_t *strides, int64_t *offset, bool *neg) {
+            if (t->uniform || t->split >= 0) return false;
+            const int64_t *st;
+            if (!t->pend) {
+                if (!t->buf) return false;
+                *buf = t->buf;
+                st = t->strides;
+                *offset = t->offset;
+                *neg = false;
+            } else {
+                const Pending *p = t->pend;
+                if (p->nleaf != 1 || p->ninstr != 1 || p->nred || p->leaf[0].uniform || p->leaf[0].pw) return false;
+                if (p->ins[0].op != kNeg) return false; // f32 negation only
+                *buf = p->leaf[0].buf;
+                st = p->leaf[0].strides;
+                *offset = p->leaf[0].offset;
+                *neg = true;
+            }
+            memcpy(strides, st, sizeof(int64_t) * kMaxRank);
+            return true;
+        };
+        if (part(x, &lv.buf, lv.strides, &lv.offset, &lv.neg1) && part(y, &lv.buf2, lv.strides2, &lv.offset2, &lv.neg2)) {
+            lv.pw = true;
+            lv.pw_split = x->dims[dim];
+            Pending *p = new Pending;
+            add_leaf(p, lv, od, x->rank);
+            Instr in;
+            in.op = (uint8_t)(kCopy | (x->dt == CG_U32 ? kInstrU32 : 0));
+            in.a = in.b = in.c = 0;
+            emit_instr(p, in);
+            cg_tensor *t = new cg_tensor;
+            t->be = b;
+            t->dt = x->dt;
+            t->rank = x->rank;
+            memcpy(t->dims, od, sizeof t->dims);
+            set_row_major(t);
+            t->pend = p;
+            *out = t;
+            return CG_OK;
+        }
     }
     CG_HIP(hipSetDevice(b->device));
     int64_t nx = numel(x), ny = numel(y);

@@ -831,6 +831,67 @@ def _():
     return run, expect
 
 
+# ---- concat along the last axis stays deferred (piecewise leaf) --------------------------------------------
+def _rot_half(be, t, h):
+    """helpers/rope.rs:423-427: concat(-x[..., h:], x[..., :h])."""
+    nd = len(t.shape) - 1
+    return be.concat(be.neg(be.slice(t, nd, h, h)), be.slice(t, nd, 0, h), nd)
+
+
+for _h, _shape in ((32, (2, 4, 3, 64)), (5, (3, 2, 10)), (8, (4, 16)), (1, (7, 2))):
+    @case(f"concat_last_rotate_half_h{_h}")
+    def _(h=_h, shape=_shape):
+        x = f32(300 + h, shape)
+        c = f32(301 + h, shape)
+        s_ = f32(302 + h, shape)
+
+        def run(be):
+            tx, tc, ts = be.from_numpy(x), be.from_numpy(c), be.from_numpy(s_)
+            rot = _rot_half(be, tx, h)
+            rope = be.add(be.mul(tc, tx), be.mul(ts, _rot_half(be, tx, h)))   # apply_rope_embedding
+            return N(be, rot, rope, be.max(_rot_half(be, tx, h)))
+
+        def expect():
+            r = np.concatenate([-x[..., h:], x[..., :h]], -1)
+            return [r, c * x + s_ * r, r.max(-1, keepdims=True)]
+
+        return run, expect
+
+
+@case("concat_last_deferred_variants")
+def _():
+    """Strided operands, u32, negation on either side, two piecewise operands in one op, views and
+    further concats of a deferred concat, uneven parts."""
+    a = rng(310).integers(-9, 10, size=(3, 6, 4)).astype(np.float32)
+    b = rng(311).integers(-9, 10, size=(3, 6, 7)).astype(np.float32)
+    u = u32(312, (5, 3))
+    v = u32(313, (5, 8))
+
+    def run(be):
+        ta, tb, tu, tv = be.from_numpy(a), be.from_numpy(b), be.from_numpy(u), be.from_numpy(v)
+        at = be.transpose(be.from_numpy(a.transpose(1, 0, 2).copy()), 0, 1)      # strided view equal to a
+        c1 = be.concat(at, be.neg(tb), 2)
+        c2 = be.concat(be.neg(ta), be.neg(tb), 2)
+        two = be.add(be.concat(ta, tb, 2), be.concat(be.neg(ta), tb, 2))         # two piecewise operands
+        cu = be.add(be.concat(tu, tv, 1), be.concat(tu, tv, 1))
+        tr = be.transpose(be.concat(ta, tb, 2), 1, 2)                            # a view ends the deferral
+        cc = be.concat(be.concat(ta, tb, 2), ta, 2)                              # deferred concat as an operand
+        sl = be.slice(be.concat(ta, tb, 2), 2, 2, 6)
+        sm = be.sum(be.mul(be.concat(ta, tb, 2), be.concat(ta, tb, 2)))
+        shared = be.concat(ta, tb, 2)
+        sh = be.sub(be.mul(shared, shared), shared)
+        return N(be, c1, c2, two, cu, tr, cc, sl, sm, sh)
+
+    def expect():
+        ab = np.concatenate([a, b], 2)
+        uv = np.concatenate([u, v], 1)
+        return [np.concatenate([a, -b], 2), np.concatenate([-a, -b], 2), ab + np.concatenate([-a, b], 2), uv + uv,
+                ab.transpose(0, 2, 1), np.concatenate([ab, a], 2), ab[:, :, 2:8], (ab * ab).sum(-1, keepdims=True),
+                ab * ab - ab]
+
+    return run, expect
+
+
 # ---- deferred row programs: sum / max that stay inside a fused expression -----------------------------
 def _const(be, v, shape, dt=np.float32):
     return be.broadcast(be.from_numpy(np.array(v, dt)), shape)
