@@ -32,7 +32,7 @@
 // ---- element-wise ------------------------------------------------------------------------
 // cos * x + sin * rotate_half(x), rotate_half(x) = concat(-x2, x1) read in place as the
 // piecewise leaf 3                                        (rotary embedding)
-CG_PROGRAM(MapRope, 4, 0x0, 3, {18, 0, 1, 0}, {42, 3, 3, 3}, {18, 2, 9, 2}, {16, 8, 10, 8})
+CG_PROGRAM(MapRope, 4, 0x0, 3, {18, 0, 1, 0}, {18, 2, 3, 2}, {16, 8, 9, 8})
 // g * (1 / (1 + exp(-g))) * u                            (SiLU gate times up projection)
 CG_PROGRAM(MapSiluMul, 3, 0x2, -1, {0, 0, 0, 0}, {3, 8, 8, 8}, {16, 1, 9, 1}, {19, 1, 10, 1}, {18, 0, 11, 0}, {18, 12, 2, 12})
 // residual stream after three adds, in the two operand orders the layer loop produces

@@ -1,0 +1,214 @@
+// Decode-time attention in one pass (included by fused.hip after aot_programs.hpp).
+//
+// A decode step issues, per layer, q.K^T (at most 8 query rows per KV head after the GQA
+// group is folded into rows), the soft-max program over the scores, and p.V.  Each of the
+// three reads or writes the [rows, T] score matrix and the two products each stream the
+// cache once from a launch of their own.  When the scores product is still lazy at the
+// moment its soft-max becomes the left operand of p.V (see LazyMm), the three run here
+// instead: a workgroup takes one KV head and one chunk of the T cached positions, computes
+// its scores from K, runs the soft-max program on them with the chunk as the row (local
+// maximum m_c, local sum l_c of exp(x - m_c)), multiplies the un-normalised weights with its
+// chunk of V, and writes (m_c, l_c, o_c).  A second small kernel combines the chunks:
+//     out = sum_c e^(m_c - g) o_c / sum_c e^(m_c - g) l_c,   g = max_c m_c,
+// which is the soft-max-weighted sum written with another grouping of the same terms.
+// The program is the compiled RowsSoftmaxCausal; its instructions before the row maximum
+// (scale, causal mask) and between maximum and sum (subtract, exp) are evaluated by the
+// same template code as in aot_rows_kernel, the final division is replaced by the combine.
+// HBM-bound: K and V once (2 x 4 x T x head_dim bytes per KV head) + the chunk results.
+#pragma once
+
+typedef float float4v __attribute__((ext_vector_type(4)));
+
+// Leaf words of leaves FIRST.. of one work item (leaf 0 of the attention program has no memory).
+template <class P, int VEC, int FIRST, int... L>
+__device__ __forceinline__ void aot_load_from(const FusedArgs &a, const int64_t (&off)[P::nleaf + 1], uint32_t e,
+                                              uint32_t (&v)[P::nleaf][VEC], std::integer_sequence<int, L...>) {
+    (aot_load_leaf<P, VEC, FIRST + L>(a, off, e, v[FIRST + L]), ...);
+}
+template <class P, int FIRST>
+__device__ __forceinline__ void aot_fetch_from(const FusedArgs &a, const int64_t (&base)[P::nleaf + 1], uint32_t it,
+                                               LeafWords<P, 1> &w) {
+    int64_t off[P::nleaf + 1];
+#pragma unroll
+    for (int l = 0; l < P::nleaf; l++) off[l] = base[l] + (int64_t)it * a.leaf[l].is;
+    off[P::nleaf] = 0;
+    aot_load_from<P, 1, FIRST>(a, off, it, w.v, std::make_integer_sequence<int, P::nleaf - FIRST>{});
+}
+
+struct AttnArgs {
+    const uint32_t *Q, *Kc, *V;
+    float *part_o;  // [batch][splits][M][hd]
+    float *part_ml; // [batch][splits][M][2]
+    uint32_t M, T, hd, splits, chunk;
+    uint32_t nb;
+    uint32_t bd[kMaxBatchAxes];
+    FastDiv bdiv[kMaxBatchAxes];
+    int64_t q_bs[kMaxBatchAxes], k_bs[kMaxBatchAxes], v_bs[kMaxBatchAxes], p_bs[kMaxBatchAxes];
+    int64_t q_sm; // stride between the query rows of a group
+    int64_t k_st; // stride between cached positions of K (head_dim contiguous)
+    int64_t v_st; // stride between cached positions of V (head_dim contiguous)
+};
+
+constexpr int kAttnChunk = 256; // most cached positions per workgroup
+constexpr int kAttnRows = 8;    // most query rows per KV head
+
+// LPT lanes share a cached position (head_dim / 4): 16 or 32.
+template <class P, int LPT>
+__global__ __launch_bounds__(kBlock) void decode_attention_kernel(const AttnArgs g, const FusedArgs a) {
+    constexpr int HD = LPT * 4;
+    constexpr int TPB = kBlock / LPT; // positions per pass
+    constexpr int ri0 = reduce_index<P>(0), ri1 = reduce_index<P>(1);
+    constexpr int src0 = P::code[ri0][1], src1 = P::code[ri1][1];
+    __shared__ float sc[kAttnRows][kAttnChunk];
+    __shared__ float red[TPB][kAttnRows * HD / 4 + 1][4];
+    const uint32_t tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+    const uint32_t split = blockIdx.x, b = blockIdx.y;
+    const uint32_t t0 = split * g.chunk, t1 = min(g.T, t0 + g.chunk);
+    // operand offsets of this batch entry
+    int64_t oq = 0, ok = 0, ov = 0, op = 0;
+    {
+        uint32_t bb = b;
+        for (uint32_t d = 0; d < g.nb; d++) {
+            const uint32_t q = fastdiv(bb, g.bdiv[d]);
+            const int64_t i = (int64_t)(bb - q * g.bd[d]);
+            bb = q;
+            oq += i * g.q_bs[d];
+            ok += i * g.k_bs[d];
+            ov += i * g.v_bs[d];
+            op += i * g.p_bs[d];
+        }
+    }
+    const uint32_t row0 = (uint32_t)(op / g.T); // first row of this group in the program's [rows, T] space
+
+    // ---- scores of the chunk: LPT lanes per position, one 16-byte piece of head_dim each
+    {
+        const uint32_t l = tid % LPT, sub = tid / LPT;
+        float4v qf[kAttnRows];
+#pragma unroll
+        for (int m = 0; m < kAttnRows; m++) {
+            qf[m] = (float4v){0.f, 0.f, 0.f, 0.f};
+            if ((uint32_t)m < g.M) qf[m] = *reinterpret_cast<const float4v *>(g.Q + oq + (int64_t)m * g.q_sm + l * 4);
+        }
+        for (uint32_t t = t0 + sub; t < t0 + (t1 - t0 + TPB - 1) / TPB * TPB; t += TPB) {
+            float4v kf = (float4v){0.f, 0.f, 0.f, 0.f};
+            if (t < t1) kf = *reinterpret_cast<const float4v *>(g.Kc + ok + (int64_t)t * g.k_st + l * 4);
+#pragma unroll
+            for (int m = 0; m < kAttnRows; m++) {
+                if ((uint32_t)m < g.M) {
+                    float v = fmaf(qf[m][3], kf[3], fmaf(qf[m][2], kf[2], fmaf(qf[m][1], kf[1], qf[m][0] * kf[0])));
+#pragma unroll
+                    for (int s = LPT / 2; s >= 1; s >>= 1) v += __shfl_xor(v, s);
+                    if (l == 0 && t < t1) sc[m][t - t0] = v;
+                }
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- the soft-max program on the chunk: a wave per query row
+    for (uint32_t m = wave; m < g.M; m += kBlock / 64) {
+        const uint32_t row = row0 + m;
+        int64_t base[P::nleaf + 1];
+#pragma unroll
+        for (int l = 0; l <= P::nleaf; l++) base[l] = 0;
+        {
+            uint32_t rr = row;
+            for (uint32_t d = 0; d < a.g.nouter; d++) {
+                const uint32_t q = fastdiv(rr, a.g.odiv[d]);
+                const int64_t i = (int64_t)(rr - q * a.g.od[d]);
+                rr = q;
+#pragma unroll
+                for (int l = 1; l < P::nleaf; l++) base[l] += i * a.leaf[l].os[d];
+            }
+        }
+        uint32_t rs[kMaxRowReduce] = {0, 0, 0};
+        constexpr bool max0 = (P::code[ri0][0] & ~kInstrU32) == kRowMax;
+        static_assert(max0 && (P::code[ri1][0] & ~kInstrU32) == kRowSum, "a soft-max: row maximum, then row sum");
+        uint32_t acc = row_init(true, true);
+        for (uint32_t i = lane; i < t1 - t0; i += 64) {
+            LeafWords<P, 1> w;
+            aot_fetch_from<P, 1>(a, base, t0 + i, w); // leaf 0 is the score
+            w.v[0][0] = asu(sc[m][i]);
+            const Values<P, 1> s = aot_eval<P, 1, ri0>(w, rs, a.fault);
+            acc = row_merge(true, true, acc, s.v[src0][0]);
+        }
+#pragma unroll
+        for (int sft = 32; sft >= 1; sft >>= 1) acc = row_merge(true, true, acc, (uint32_t)__shfl_xor((int)acc, sft));
+        rs[0] = acc;
+        uint32_t sum = row_init(false, true);
+        for (uint32_t i = lane; i < t1 - t0; i += 64) {
+            LeafWords<P, 1> w;
+            aot_fetch_from<P, 1>(a, base, t0 + i, w);
+            w.v[0][0] = asu(sc[m][i]);
+            const Values<P, 1> s = aot_eval<P, 1, ri1>(w, rs, a.fault);
+            sum = row_merge(false, true, sum, s.v[src1][0]);
+            sc[m][i] = asf(s.v[src1][0]); // the un-normalised weight
+        }
+#pragma unroll
+        for (int sft = 32; sft >= 1; sft >>= 1) sum = row_merge(false, true, sum, (uint32_t)__shfl_xor((int)sum, sft));
+        if (lane == 0) {
+            float *ml = g.part_ml + (((uint64_t)b * g.splits + split) * g.M + m) * 2;
+            ml[0] = asf(acc);
+            ml[1] = asf(sum);
+        }
+    }
+    __syncthreads();
+
+    // ---- weights times V: LPT lanes cover head_dim, TPB groups split the positions
+    {
+        const uint32_t ng = tid % LPT, kg = tid / LPT;
+        float4v o[kAttnRows];
+#pragma unroll
+        for (int m = 0; m < kAttnRows; m++) o[m] = (float4v){0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+        for (uint32_t t = t0 + kg; t < t1; t += TPB) {
+            const float4v vf = *reinterpret_cast<const float4v *>(g.V + ov + (int64_t)t * g.v_st + ng * 4);
+#pragma unroll
+            for (int m = 0; m < kAttnRows; m++) {
+                if ((uint32_t)m < g.M) {
+                    const float w = sc[m][t - t0];
+                    o[m][0] = fmaf(w, vf[0], o[m][0]);
+                    o[m][1] = fmaf(w, vf[1], o[m][1]);
+                    o[m][2] = fmaf(w, vf[2], o[m][2]);
+                    o[m][3] = fmaf(w, vf[3], o[m][3]);
+                }
+            }
+        }
+#pragma unroll
+        for (int m = 0; m < kAttnRows; m++)
+            if ((uint32_t)m < g.M) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) red[kg][m * LPT + ng][j] = o[m][j];
+            }
+        __syncthreads();
+        for (uint32_t e = tid; e < g.M * HD; e += kBlock) {
+            const uint32_t m = e / HD, n = e % HD;
+            float v = 0.0f;
+#pragma unroll
+            for (int k = 0; k < TPB; k++) v += red[k][m * LPT + n / 4][n % 4];
+            g.part_o[(((uint64_t)b * g.splits + split) * g.M + m) * HD + n] = v;
+        }
+    }
+}
+
+// out[b][m][n] = sum_c e^(m_c - g) o_c[n] / sum_c e^(m_c - g) l_c
+__global__ __launch_bounds__(kBlock) void decode_attention_combine_kernel(const float *part_o, const float *part_ml,
+                                                                          uint32_t *out, uint32_t splits, uint32_t M,
+                                                                          uint32_t hd, uint64_t total) {
+    const uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= total) return;
+    const uint32_t n = (uint32_t)(i % hd);
+    const uint64_t bm = i / hd;
+    const uint32_t m = (uint32_t)(bm % M);
+    const uint64_t b = bm / M;
+    float gmax = kF32Min;
+    for (uint32_t c = 0; c < splits; c++) gmax = fmaxf(gmax, part_ml[((b * splits + c) * M + m) * 2]);
+    float num = 0.0f, den = 0.0f;
+    for (uint32_t c = 0; c < splits; c++) {
+        const float *ml = part_ml + ((b * splits + c) * M + m) * 2;
+        const float w = expf(ml[0] - gmax);
+        num = fmaf(w, part_o[((b * splits + c) * M + m) * (uint64_t)hd + n], num);
+        den = fmaf(w, ml[1], den);
+    }
+    out[i] = asu(num / den);
+}

@@ -215,8 +215,24 @@ struct Instr {
 };
 constexpr uint8_t kInstrU32 = 0x80;
 
+// A decode-time attention score product q.K^T (at most 8 rows, K = head_dim) whose execution is
+// put off: if the soft-max over it ends up as the left operand of p.V, the three are run as one
+// fused attention kernel and the scores never exist in memory; any other use computes the
+// product once (`result`) and reads it like any buffer.
+struct LazyMm {
+    std::atomic<long> rc{1};
+    cg_tensor *x = nullptr, *y = nullptr; // retained operands (concrete)
+    Buffer *result = nullptr;             // retained once computed
+    int64_t dims[kMaxRank] = {0};
+    int rank = 0;
+};
+void lazy_mm_release(LazyMm *m);
+// Computes the product if it has not been yet.
+int lazy_mm_force(cg_backend *be, LazyMm *m);
+
 struct LeafView {
-    Buffer *buf = nullptr; // retained; null for uniform leaves
+    Buffer *buf = nullptr; // retained; null for uniform leaves (and for a lazy product not yet computed)
+    LazyMm *lazy = nullptr; // retained: the leaf is the (row-major) result of this product
     int64_t strides[kMaxRank] = {0};
     int64_t offset = 0;
     bool uniform = false;
@@ -322,5 +338,27 @@ int launch_any_positive(cg_backend *be, const cg_tensor *x);
 int launch_any_diff(cg_backend *be, const cg_tensor *x, const cg_tensor *y);
 
 int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_tensor *out);
+
+// The batch structure of x . y after collapsing: batch axes that both operands walk as one run
+// are merged, a split axis contributes its two parts, and the innermost batch axis is folded
+// into M when y ignores it and x walks it as more rows.  Reads shapes and strides only, so x
+// may be a descriptor without memory.
+constexpr int kMaxBatchAxes = 6;
+struct MmFold {
+    int64_t M = 0, N = 0, K = 0, batch = 0;
+    int64_t a_sm = 0, a_sk = 0, b_sk = 0, b_sn = 0;
+    int nb = 0;                                  // collapsed batch axes
+    int64_t bd[kMaxBatchAxes] = {0};             // extents, innermost first
+    int64_t a_bs[kMaxBatchAxes] = {0}, b_bs[kMaxBatchAxes] = {0};
+};
+int fold_matmul(const cg_tensor *x, const cg_tensor *y, MmFold *f);
+
+// Decode-time attention in one pass: out = softmax-program(q . kT) . v, where `p` is the deferred
+// soft-max program whose leaf 0 is the (never computed) lazy product q . kT and (pdims, prank) its
+// shape.  Returns kDeclined when the shapes or the program are not what the kernel handles; the
+// caller then takes the ordinary route.
+constexpr int kDeclined = -1000;
+int launch_decode_attention(cg_backend *be, const Pending &p, const int64_t *pdims, int prank, const cg_tensor *q,
+                            const cg_tensor *kt, const cg_tensor *v, cg_tensor *out);
 
 } // namespace cg

@@ -16,6 +16,7 @@
 #include "common.hpp"
 #include "device_utils.hpp"
 
+#include <algorithm>
 #include <mutex>
 #include <set>
 #include <string>
@@ -451,7 +452,7 @@ bool allocate_registers(const Pending &p, uint8_t *phys) {
 }
 
 int fill_args(cg_backend *be, const Pending &p, const int64_t *dims, int rank, const cg_tensor *out, bool keep_last,
-              FusedArgs *a, double *leaf_bytes, bool *full, int ninstr = -1) {
+              FusedArgs *a, double *leaf_bytes, bool *full, int ninstr = -1, bool skip_lazy = false) {
     if (ninstr < 0) ninstr = p.ninstr;
     memset(a, 0, sizeof *a);
     ViewDesc v[kMaxViews + 1];
@@ -482,7 +483,13 @@ int fill_args(cg_backend *be, const Pending &p, const int64_t *dims, int rank, c
         v[l + 1].strides = lv.strides;
         v[l + 1].uniform = lv.uniform;
         v[l + 1].ubits = lv.ubits;
-        v[l + 1].ptr = lv.uniform ? nullptr : static_cast<const char *>(lv.buf->ptr) + lv.offset * 4;
+        const Buffer *src = lv.buf;
+        if (lv.lazy && !skip_lazy) { // a product that has been put off until now
+            int lrc = lazy_mm_force(be, lv.lazy);
+            if (lrc) return lrc;
+            src = lv.lazy->result;
+        }
+        v[l + 1].ptr = lv.uniform || !src ? nullptr : static_cast<const char *>(src->ptr) + lv.offset * 4;
         v[l + 1].vec_period = 0;
         if (lv.pw) { // its second part is planned as one more view, and the row axis stays on its own
             pw_leaf = l;
@@ -498,7 +505,7 @@ int fill_args(cg_backend *be, const Pending &p, const int64_t *dims, int rank, c
             double n = 1.0;
             for (int i = 0; i < rank; i++)
                 if (lv.strides[i] != 0 || dims[i] <= 1) n *= (double)dims[i];
-            bytes += 4.0 * n;
+            if (!(lv.lazy && skip_lazy)) bytes += 4.0 * n;
         }
     }
     Operand ops[kMaxViews + 1];
@@ -562,7 +569,7 @@ void trace_program(cg_backend *be, const Pending &p, int ninstr, const char *how
     std::lock_guard<std::mutex> lk(mu);
     if (!seen.insert(key).second) return;
     std::string where = " uniform=";
-    for (int l = 0; l < p.nleaf; l++) where += p.leaf[l].pw ? 'p' : p.leaf[l].uniform ? '1' : '0';
+    for (int l = 0; l < p.nleaf; l++) where += p.leaf[l].pw ? 'p' : p.leaf[l].lazy ? 'm' : p.leaf[l].uniform ? '1' : '0';
     where += " dims=[";
     for (int i = 0; i < rank; i++) {
         snprintf(buf, sizeof buf, "%s%lld", i ? "," : "", (long long)dims[i]);
@@ -571,7 +578,107 @@ void trace_program(cg_backend *be, const Pending &p, int ninstr, const char *how
     fprintf(stderr, "[cg program] %s%s]\n", key.c_str(), where.c_str());
 }
 
+#include "attention.hpp"
+
 } // namespace
+
+int launch_decode_attention(cg_backend *be, const Pending &p, const int64_t *pdims, int prank, const cg_tensor *q,
+                            const cg_tensor *kt, const cg_tensor *v, cg_tensor *out) {
+    using P = RowsSoftmaxCausal;
+    if (!be->aot || !program_matches<P>(p) || !p.leaf[0].lazy || p.leaf[0].lazy->result || p.reduced) return kDeclined;
+    cg_tensor pd; // the soft-max result as a dense descriptor: the left operand of p.V
+    pd.rank = prank;
+    int64_t st = 1;
+    for (int i = prank - 1; i >= 0; i--) {
+        pd.dims[i] = pdims[i];
+        pd.strides[i] = st;
+        st *= pdims[i];
+    }
+    if (p.leaf[0].offset != 0) return kDeclined;
+    for (int i = 0; i < prank; i++)
+        if (pdims[i] > 1 && p.leaf[0].strides[i] != pd.strides[i]) return kDeclined;
+    MmFold f1, f2;
+    if (fold_matmul(q, kt, &f1) || fold_matmul(&pd, v, &f2)) return kDeclined;
+    const int64_t T = f1.N, hd = f1.K;
+    if (f1.M != f2.M || f1.M < 1 || f1.M > kAttnRows || f1.nb != f2.nb || f2.K != T || f2.N != hd) return kDeclined;
+    if (hd != 64 && hd != 128) return kDeclined;
+    if (f1.a_sk != 1 || f1.b_sk != 1 || f2.b_sn != 1 || f2.a_sk != 1 || f2.a_sm != T) return kDeclined;
+    if (f1.batch < 1 || f1.batch > 65535 || T < 1 || T > 0x7FFFFFFFll) return kDeclined;
+    for (int d = 0; d < f1.nb; d++)
+        if (f1.bd[d] != f2.bd[d] || f2.a_bs[d] % T || f1.a_bs[d] % 4 || f1.b_bs[d] % 4 || f2.b_bs[d] % 4) return kDeclined;
+    if (f1.a_sm % 4 || f1.b_sn % 4 || f2.b_sk % 4) return kDeclined;
+    const void *pq, *pk, *pv;
+    int rc = device_ptr(q, &pq);
+    if (!rc) rc = device_ptr(kt, &pk);
+    if (!rc) rc = device_ptr(v, &pv);
+    if (rc) return rc;
+    if (reinterpret_cast<uintptr_t>(pq) % 16 || reinterpret_cast<uintptr_t>(pk) % 16 || reinterpret_cast<uintptr_t>(pv) % 16)
+        return kDeclined;
+    FusedArgs a;
+    double leaf_bytes;
+    bool full;
+    rc = fill_args(be, p, pdims, prank, nullptr, true, &a, &leaf_bytes, &full, -1, true);
+    if (rc) return rc;
+    uint64_t rows = 1;
+    for (uint32_t d = 0; d < a.g.nouter; d++) rows *= a.g.od[d];
+    if (a.g.inner != (uint32_t)T || rows != (uint64_t)f1.batch * (uint64_t)f1.M) return kDeclined;
+
+    AttnArgs g;
+    memset(&g, 0, sizeof g);
+    g.Q = static_cast<const uint32_t *>(pq);
+    g.Kc = static_cast<const uint32_t *>(pk);
+    g.V = static_cast<const uint32_t *>(pv);
+    g.M = (uint32_t)f1.M;
+    g.T = (uint32_t)T;
+    g.hd = (uint32_t)hd;
+    // enough workgroups for every CU twice over, chunks of 64..256 positions
+    const int64_t want = std::max<int64_t>(1, 512 / f1.batch);
+    int64_t chunk = std::min<int64_t>(kAttnChunk, std::max<int64_t>(64, (T + want - 1) / want));
+    chunk = (chunk + 15) / 16 * 16;
+    g.chunk = (uint32_t)chunk;
+    g.splits = (uint32_t)((T + chunk - 1) / chunk);
+    g.nb = (uint32_t)f1.nb;
+    for (int d = 0; d < f1.nb; d++) {
+        g.bd[d] = (uint32_t)f1.bd[d];
+        g.bdiv[d] = make_fastdiv(g.bd[d]);
+        g.q_bs[d] = f1.a_bs[d];
+        g.k_bs[d] = f1.b_bs[d];
+        g.v_bs[d] = f2.b_bs[d];
+        g.p_bs[d] = f2.a_bs[d];
+    }
+    g.q_sm = f1.a_sm;
+    g.k_st = f1.b_sn;
+    g.v_st = f2.b_sk;
+    const size_t o_bytes = (size_t)f1.batch * g.splits * g.M * hd * 4, ml_bytes = (size_t)f1.batch * g.splits * g.M * 2 * 4;
+    void *po = nullptr, *pml = nullptr;
+    size_t co = 0, cml = 0;
+    rc = be->pool.alloc(o_bytes, &po, &co);
+    if (rc) return rc;
+    rc = be->pool.alloc(ml_bytes, &pml, &cml);
+    if (rc) {
+        be->pool.free(po, co);
+        return rc;
+    }
+    g.part_o = static_cast<float *>(po);
+    g.part_ml = static_cast<float *>(pml);
+    be->programs_compiled++;
+    {
+        ProfScope prof(be, CG_K_GEMM_SKINNY, distinct_bytes(q) + distinct_bytes(kt) + distinct_bytes(v) + distinct_bytes(out));
+        dim3 grid(g.splits, (uint32_t)f1.batch);
+        if (hd == 64)
+            hipLaunchKernelGGL((decode_attention_kernel<P, 16>), grid, dim3(kBlock), 0, be->stream, g, a);
+        else
+            hipLaunchKernelGGL((decode_attention_kernel<P, 32>), grid, dim3(kBlock), 0, be->stream, g, a);
+        const uint64_t total = (uint64_t)f1.batch * g.M * hd;
+        hipLaunchKernelGGL(decode_attention_combine_kernel, dim3((uint32_t)((total + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+                           be->stream, g.part_o, g.part_ml, static_cast<uint32_t *>(out->buf->ptr), g.splits, g.M,
+                           (uint32_t)hd, total);
+    }
+    be->pool.free(po, co); // stream-ordered: later users queue behind the combine
+    be->pool.free(pml, cml);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CG_OK : hip_fail(e, "decode attention launch");
+}
 
 bool fused_program_fits(const Pending &p) {
     uint8_t phys[kMaxLeaves + kMaxInstr];

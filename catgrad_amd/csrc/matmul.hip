@@ -36,8 +36,6 @@ namespace cg {
 
 namespace {
 
-constexpr int kMaxBatchAxes = 6;
-
 struct MmArgs {
     const uint32_t *A;
     const uint32_t *B;
@@ -580,25 +578,14 @@ template <bool F> __global__ __launch_bounds__(kThreads) void simple_gemm_kernel
 
 } // namespace
 
-int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_tensor *out) {
+int fold_matmul(const cg_tensor *x, const cg_tensor *y, MmFold *f) {
     const int r = x->rank;
-    int64_t M = x->dims[r - 2], K = x->dims[r - 1], N = y->dims[r - 1];
-    MmArgs a;
-    memset(&a, 0, sizeof a);
-    const void *pa, *pb;
-    int rc = device_ptr(x, &pa);
-    if (rc) return rc;
-    rc = device_ptr(y, &pb);
-    if (rc) return rc;
-    a.A = static_cast<const uint32_t *>(pa);
-    a.B = static_cast<const uint32_t *>(pb);
-    a.C = static_cast<uint32_t *>(out->buf->ptr);
+    int64_t M = x->dims[r - 2];
     auto stride = [](const cg_tensor *t, int ax) -> int64_t { return t->uniform ? 0 : t->strides[ax]; };
-    a.a_sm = stride(x, r - 2);
-    a.a_sk = stride(x, r - 1);
-    a.b_sk = stride(y, r - 2);
-    a.b_sn = stride(y, r - 1);
-
+    f->a_sm = stride(x, r - 2);
+    f->a_sk = stride(x, r - 1);
+    f->b_sk = stride(y, r - 2);
+    f->b_sn = stride(y, r - 1);
     // collapse the batch axes of A and B together (C is row-major, so it follows); a split axis of
     // either operand contributes its two parts as separate axes
     int64_t bd[kMaxRank + 1], sa[kMaxRank + 1], sb[kMaxRank + 1];
@@ -628,14 +615,47 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
         }
     }
     // fold the innermost batch axis into M when B ignores it and A walks it as more rows
-    while (w > 0 && sb[w - 1] == 0 && (M == 1 || sa[w - 1] == a.a_sm * M)) {
-        if (M == 1) a.a_sm = sa[w - 1];
+    while (w > 0 && sb[w - 1] == 0 && (M == 1 || sa[w - 1] == f->a_sm * M)) {
+        if (M == 1) f->a_sm = sa[w - 1];
         M *= bd[w - 1];
         w--;
     }
     if (w > kMaxBatchAxes) return fail(CG_ERR_UNSUPPORTED, "matmul: more than %d non-mergeable batch axes", kMaxBatchAxes);
     int64_t batch = 1;
     for (int i = 0; i < w; i++) batch *= bd[i];
+    f->M = M;
+    f->N = y->dims[r - 1];
+    f->K = x->dims[r - 1];
+    f->batch = batch;
+    f->nb = w;
+    for (int d = 0; d < w; d++) {
+        f->bd[d] = bd[w - 1 - d];
+        f->a_bs[d] = sa[w - 1 - d];
+        f->b_bs[d] = sb[w - 1 - d];
+    }
+    return CG_OK;
+}
+
+int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_tensor *out) {
+    MmArgs a;
+    memset(&a, 0, sizeof a);
+    const void *pa, *pb;
+    int rc = device_ptr(x, &pa);
+    if (rc) return rc;
+    rc = device_ptr(y, &pb);
+    if (rc) return rc;
+    a.A = static_cast<const uint32_t *>(pa);
+    a.B = static_cast<const uint32_t *>(pb);
+    a.C = static_cast<uint32_t *>(out->buf->ptr);
+    MmFold f;
+    rc = fold_matmul(x, y, &f);
+    if (rc) return rc;
+    const int64_t M = f.M, N = f.N, K = f.K, batch = f.batch;
+    const int w = f.nb;
+    a.a_sm = f.a_sm;
+    a.a_sk = f.a_sk;
+    a.b_sk = f.b_sk;
+    a.b_sn = f.b_sn;
     if (M > 0x7FFFFFFFll || N > 0x7FFFFFFFll || K > 0x7FFFFFFFll || batch > 65535ll * 1024)
         return fail(CG_ERR_UNSUPPORTED, "matmul: extent above 2^31-1");
     a.M = (uint32_t)M;
@@ -645,10 +665,10 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
     a.batch = (uint32_t)batch;
     bool a_al = reinterpret_cast<uintptr_t>(pa) % 16 == 0, b_al = reinterpret_cast<uintptr_t>(pb) % 16 == 0;
     for (int d = 0; d < w; d++) {
-        a.bd[d] = (uint32_t)bd[w - 1 - d];
+        a.bd[d] = (uint32_t)f.bd[d];
         a.bdiv[d] = make_fastdiv(a.bd[d]);
-        a.a_bs[d] = sa[w - 1 - d];
-        a.b_bs[d] = sb[w - 1 - d];
+        a.a_bs[d] = f.a_bs[d];
+        a.b_bs[d] = f.b_bs[d];
         if (a.a_bs[d] % 4) a_al = false;
         if (a.b_bs[d] % 4) b_al = false;
     }

@@ -125,6 +125,7 @@ Pending::Pending(const Pending &o)
         leaf[l] = o.leaf[l];
         if (leaf[l].buf) leaf[l].buf->rc.fetch_add(1);
         if (leaf[l].buf2) leaf[l].buf2->rc.fetch_add(1);
+        if (leaf[l].lazy) leaf[l].lazy->rc.fetch_add(1);
     }
     for (int i = 0; i < ninstr; i++) ins[i] = o.ins[i];
 }
@@ -133,7 +134,32 @@ Pending::~Pending() {
     for (int l = 0; l < nleaf; l++) {
         buffer_release(leaf[l].buf);
         buffer_release(leaf[l].buf2);
+        lazy_mm_release(leaf[l].lazy);
     }
+}
+
+void lazy_mm_release(LazyMm *m) {
+    if (!m) return;
+    if (m->rc.fetch_sub(1) == 1) {
+        release(m->x);
+        release(m->y);
+        buffer_release(m->result);
+        delete m;
+    }
+}
+
+int lazy_mm_force(cg_backend *be, LazyMm *m) {
+    if (m->result) return CG_OK;
+    cg_tensor *o;
+    int rc = new_dense(be, CG_F32, m->dims, m->rank, &o);
+    if (rc) return rc;
+    rc = launch_matmul(be, m->x, m->y, o);
+    if (!rc) {
+        m->result = o->buf;
+        o->buf = nullptr;
+    }
+    release(o);
+    return rc;
 }
 
 void release(cg_tensor *t) {
@@ -537,7 +563,27 @@ static void leaf_as_tensor(const Pending &p, int l, const cg_tensor *shape_of, c
 
 // Runs the program of `p` into `dst` (a dense or strided view of p's shape).  A single
 // instruction goes to the specialised single-op kernel.
+// Lazy products among the leaves are computed now and become ordinary buffer leaves.
+static int resolve_lazy_leaves(cg_backend *be, const Pending &cp) {
+    Pending &p = const_cast<Pending &>(cp); // a cache fill: the value of the program does not change
+    for (int l = 0; l < p.nleaf; l++) {
+        LeafView &lv = p.leaf[l];
+        if (!lv.lazy) continue;
+        int rc = lazy_mm_force(be, lv.lazy);
+        if (rc) return rc;
+        lv.buf = lv.lazy->result;
+        lv.buf->rc.fetch_add(1);
+        lazy_mm_release(lv.lazy);
+        lv.lazy = nullptr;
+    }
+    return CG_OK;
+}
+
 static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p) {
+    {
+        int lrc = resolve_lazy_leaves(be, p);
+        if (lrc) return lrc;
+    }
     if (p.nred > 0) {
         // the iteration space: dst's shape, with the row restored when dst holds one value per row
         cg_tensor space;
@@ -607,6 +653,29 @@ static int ensure_concrete(cg_tensor *t) {
     cg_backend *be = t->be;
     hipError_t he = hipSetDevice(be->device);
     if (he != hipSuccess) return hip_fail(he, "hipSetDevice");
+    if (t->pend->nleaf == 1 && t->pend->ninstr == 1 && t->pend->leaf[0].lazy && (t->pend->ins[0].op & ~kInstrU32) == kCopy &&
+        t->pend->leaf[0].offset == 0) {
+        // the plain result of a lazy product: compute it and adopt its buffer
+        cg_tensor probe;
+        probe.rank = t->rank;
+        memcpy(probe.dims, t->dims, sizeof probe.dims);
+        set_row_major(&probe);
+        bool dense = true;
+        for (int i = 0; i < t->rank; i++) dense = dense && (t->dims[i] <= 1 || probe.strides[i] == t->pend->leaf[0].strides[i]);
+        if (dense) {
+            LazyMm *m = t->pend->leaf[0].lazy;
+            int rc = lazy_mm_force(be, m);
+            if (rc) return rc;
+            m->result->rc.fetch_add(1);
+            t->buf = m->result;
+            t->offset = 0;
+            set_row_major(t);
+            Pending *old = t->pend;
+            t->pend = nullptr;
+            delete old;
+            return CG_OK;
+        }
+    }
     Buffer *b = new Buffer;
     b->be = be;
     int rc = be->pool.alloc((size_t)numel(t) * 4, &b->ptr, &b->cls);
@@ -637,7 +706,7 @@ static int ensure_concrete(cg_tensor *t) {
 }
 
 static bool same_leaf(const LeafView &a, const LeafView &b, const int64_t *dims, int rank) {
-    if (a.uniform != b.uniform || a.pw != b.pw) return false;
+    if (a.uniform != b.uniform || a.pw != b.pw || a.lazy != b.lazy) return false;
     if (a.uniform) return a.ubits == b.ubits;
     if (a.buf != b.buf || a.offset != b.offset) return false;
     for (int i = 0; i < rank; i++)
@@ -663,6 +732,7 @@ static int add_leaf(Pending *p, const LeafView &lv, const int64_t *dims, int ran
     p->leaf[p->nleaf] = lv;
     if (lv.buf) lv.buf->rc.fetch_add(1);
     if (lv.buf2) lv.buf2->rc.fetch_add(1);
+    if (lv.lazy) lv.lazy->rc.fetch_add(1);
     return p->nleaf++;
 }
 
@@ -708,6 +778,10 @@ static uint8_t splice_program(Pending *p, const Pending *src, const int64_t *dim
         in.a = remap(in.a);
         in.b = n > 1 ? remap(in.b) : in.a;
         in.c = n > 2 ? remap(in.c) : in.a;
+        if ((in.op & ~kInstrU32) == kCopy) { // inside a larger program a copy is just its operand
+            last = rmap[i] = in.a;
+            continue;
+        }
         last = rmap[i] = emit_instr(p, in);
     }
     return last;
@@ -1632,11 +1706,62 @@ int cg_matmul(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **out) {
     // deferred operands are computed now; a split axis may stay if it is a batch axis (the GEMM walks
     // its two parts as separate batch axes) and the two operands do not disagree about it
     int rc = CG_OK;
+    if (b->fuse && x->pend && x->rc.load() == 1 && x->pend->nleaf > 0 && x->pend->leaf[0].lazy &&
+        !x->pend->leaf[0].lazy->result && !y->pend && !y->uniform && (y->split < 0 || y->split < r - 2)) {
+        // soft-max over a lazy q.K^T, times V: one fused attention pass if the kernel takes the shapes
+        LazyMm *m = x->pend->leaf[0].lazy;
+        cg_tensor *o;
+        rc = new_dense(b, x->dt, od, r, &o);
+        if (rc) return rc;
+        rc = numel(o) > 0 ? launch_decode_attention(b, *x->pend, x->dims, x->rank, m->x, m->y, y, o) : kDeclined;
+        if (rc == CG_OK) {
+            *out = o;
+            return CG_OK;
+        }
+        release(o);
+        if (rc != kDeclined) return rc;
+        rc = CG_OK;
+    }
     if (x->pend || x->split >= r - 2) rc = ensure_concrete(x);
     if (!rc && (y->pend || y->split >= r - 2)) rc = ensure_concrete(y);
     if (!rc && x->split >= 0 && y->split >= 0 && (x->split != y->split || x->split_inner != y->split_inner))
         rc = ensure_concrete(y);
     if (rc) return rc;
+    {
+        // decode-time q.K^T: put off, so that soft-max and p.V can absorb it (see LazyMm)
+        int64_t n_out = 1;
+        for (int i = 0; i < r; i++) n_out *= od[i];
+        const int64_t K = x->dims[r - 1];
+        if (b->fuse && x->dt == CG_F32 && r == 4 && n_out > 0 && x->dims[r - 2] <= 8 && K > 0 && K <= 256 &&
+            K % 4 == 0 && !x->uniform && !y->uniform && x->split < 0 && y->strides[r - 2] == 1 && od[r - 1] > 1) {
+            LazyMm *m = new LazyMm;
+            retain(x);
+            retain(y);
+            m->x = x;
+            m->y = y;
+            m->rank = r;
+            memcpy(m->dims, od, sizeof m->dims);
+            cg_tensor *t = new cg_tensor;
+            t->be = b;
+            t->dt = CG_F32;
+            t->rank = r;
+            memcpy(t->dims, od, sizeof t->dims);
+            set_row_major(t);
+            Pending *p = new Pending;
+            LeafView lv;
+            lv.lazy = m;
+            memcpy(lv.strides, t->strides, sizeof lv.strides);
+            add_leaf(p, lv, od, r);
+            lazy_mm_release(m); // the leaf holds it now
+            Instr in;
+            in.op = (uint8_t)kCopy;
+            in.a = in.b = in.c = 0;
+            emit_instr(p, in);
+            t->pend = p;
+            *out = t;
+            return CG_OK;
+        }
+    }
     cg_tensor *o;
     rc = new_dense(b, x->dt, od, r, &o);
     if (rc) return rc;
@@ -1672,7 +1797,8 @@ static int reduce_entry(cg_backend *b, int kind, const char *what, cg_tensor *x,
     if (rc) return rc;
     if (numel(o) > 0) {
         if (x->pend && x->pend->nred == 0 && (x->rc.load() == 1 || cheap(x->pend))) {
-            rc = launch_fused_reduce(b, kind, x->dt == CG_F32, *x->pend, x->pend->ninstr, x->dims, x->rank, o);
+            rc = resolve_lazy_leaves(b, *x->pend);
+            if (!rc) rc = launch_fused_reduce(b, kind, x->dt == CG_F32, *x->pend, x->pend->ninstr, x->dims, x->rank, o);
         } else {
             rc = ensure_concrete(x);
             if (!rc) rc = launch_reduce(b, kind, x, o);
@@ -1975,7 +2101,7 @@ int cg_concat(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor *
                 *neg = false;
             } else {
                 const Pending *p = t->pend;
-                if (p->nleaf != 1 || p->ninstr != 1 || p->nred || p->leaf[0].uniform || p->leaf[0].pw) return false;
+                if (p->nleaf != 1 || p->ninstr != 1 || p->nred || p->leaf[0].uniform || p->leaf[0].pw || p->leaf[0].lazy) return false;
                 if (p->ins[0].op != kNeg) return false; // f32 negation only
                 *buf = p->leaf[0].buf;
                 st = p->leaf[0].strides;

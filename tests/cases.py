@@ -892,6 +892,61 @@ def _():
     return run, expect
 
 
+# ---- decode-time attention: q.K^T -> causal soft-max -> p.V as the model graphs issue it ------------------------
+def decode_attention_ops(be, q, k_cache, v_cache, rep):
+    """One decode step's attention of `LlamaModel` (catgrad-llm-models/src/models/llama.rs:285-345) on a
+    cache of T positions: repeat_kv, scores, 1/sqrt(hd), causal mask row T-1 (helpers/tensors.rs:207-224),
+    soft-max (stdlib/nn/mod.rs:168-179), context.  q [B, kvH*rep, 1, hd]; caches [B, kvH, T, hd]."""
+    B, kvh, T, hd = k_cache.shape
+    H = kvh * rep
+
+    def repeat_kv(t):
+        t = be.reshape(t.move(), (B, kvh, 1, T, hd))
+        t = be.broadcast(t.move(), (B, kvh, rep, T, hd))
+        return be.reshape(t.move(), (B, H, T, hd))
+
+    k, v = repeat_kv(k_cache), repeat_kv(v_cache)
+    attn = be.matmul(q.move(), be.transpose(k.move(), 2, 3).move())
+    sh = (B, H, 1, T)
+    attn = be.div(attn.move(), _const(be, float(np.sqrt(np.float32(hd))), sh).move())
+    ci = be.broadcast(be.arange(T).move(), (T, T))
+    cj = be.broadcast(be.reshape(be.arange(T).move(), (T, 1)).move(), (T, T))
+    mask = be.cast(be.lt(cj.move(), ci.move()).move(), A.F32)
+    mask = be.mul(mask.move(), _const(be, float(F32_MIN), (T, T)).move())
+    mask = be.slice(mask.move(), 0, T - 1, 1)
+    attn = be.add(attn.move(), be.broadcast(mask.move(), sh).move())
+    m = be.max(attn)
+    x = be.sub(attn.move(), be.broadcast(m.move(), sh).move())
+    ex = be.exp(x.move())
+    ssum = be.sum(ex)
+    p = be.div(ex.move(), be.broadcast(ssum.move(), sh).move())
+    return be.matmul(p.move(), v.move())
+
+
+def _np_decode_attention(q, k, v, rep):
+    B, kvh, T, hd = k.shape
+    kk = np.repeat(k.astype(np.float64), rep, axis=1)
+    vv = np.repeat(v.astype(np.float64), rep, axis=1)
+    s = q.astype(np.float64) @ kk.transpose(0, 1, 3, 2) / np.float64(np.sqrt(np.float32(hd)))
+    s = s - s.max(-1, keepdims=True)
+    e = np.exp(s)
+    return (e / e.sum(-1, keepdims=True)) @ vv
+
+
+for _B, _kvh, _rep, _T, _hd in ((2, 2, 4, 300, 64), (1, 3, 1, 1, 64), (2, 1, 8, 63, 64), (1, 2, 2, 65, 128),
+                                (4, 8, 4, 1000, 64), (1, 1, 3, 257, 128), (2, 2, 4, 40, 32)):
+    @case(f"decode_attention_B{_B}_kv{_kvh}_rep{_rep}_T{_T}_hd{_hd}", "ew_abs")
+    def _(B=_B, kvh=_kvh, rep=_rep, T=_T, hd=_hd):
+        q = f32(400 + T, (B, kvh * rep, 1, hd))
+        k = f32(401 + T, (B, kvh, T, hd))
+        v = f32(402 + T, (B, kvh, T, hd))
+
+        def run(be):
+            return N(be, decode_attention_ops(be, be.from_numpy(q), be.from_numpy(k), be.from_numpy(v), rep))
+
+        return run, (lambda: [_np_decode_attention(q, k, v, rep)])
+
+
 # ---- deferred row programs: sum / max that stay inside a fused expression -----------------------------
 def _const(be, v, shape, dt=np.float32):
     return be.broadcast(be.from_numpy(np.array(v, dt)), shape)

@@ -121,6 +121,21 @@ def test_pool_returns_to_baseline(hip):
     assert cached > 0
 
 
+def test_decode_attention_runs_as_one_fused_pass(hip):
+    """The decode-step attention graph (head_dim 64, 4 query heads per KV head) is absorbed by the fused
+    attention kernel: no interpreted program, no separate soft-max launch, and the same values."""
+    from cases import _np_decode_attention, decode_attention_ops, f32
+
+    q, k, v = f32(1, (2, 8, 1, 64)), f32(2, (2, 2, 500, 64)), f32(3, (2, 2, 500, 64))
+    hip.sync()
+    hip.program_stats()
+    out = decode_attention_ops(hip, hip.from_numpy(q), hip.from_numpy(k), hip.from_numpy(v), 4)
+    got = hip.to_numpy(out)
+    compiled, interpreted = hip.program_stats()
+    assert (compiled, interpreted) == (1, 0)
+    np.testing.assert_allclose(got, _np_decode_attention(q, k, v, 4), rtol=1e-4, atol=1e-5)
+
+
 def test_format_tensor(hip):
     s = hip.format_tensor(hip.from_numpy(np.array([[1.5, 2.0]], np.float32)))
     assert "f32[1,2]" in s and "1.5" in s
