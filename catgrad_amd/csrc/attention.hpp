@@ -35,6 +35,16 @@ __device__ __forceinline__ void aot_fetch_from(const FusedArgs &a, const int64_t
     aot_load_from<P, 1, FIRST>(a, off, it, w.v, std::make_integer_sequence<int, P::nleaf - FIRST>{});
 }
 
+// Sum over the 16 lanes of a DPP row (lanes 16i..16i+15), left in every lane of the row: four
+// rotate-and-add steps inside the vector ALU instead of four trips through the LDS crossbar.
+__device__ __forceinline__ float row16_sum(float v) {
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x128, 0xF, 0xF, false)); // row_ror:8
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x124, 0xF, 0xF, false)); // row_ror:4
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x122, 0xF, 0xF, false)); // row_ror:2
+    v += __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x121, 0xF, 0xF, false)); // row_ror:1
+    return v;
+}
+
 struct AttnArgs {
     const uint32_t *Q, *Kc, *V;
     float *part_o;  // [batch][splits][M][hd]
@@ -49,18 +59,26 @@ struct AttnArgs {
     int64_t v_st; // stride between cached positions of V (head_dim contiguous)
 };
 
-constexpr int kAttnChunk = 256; // most cached positions per workgroup
 constexpr int kAttnRows = 8;    // most query rows per KV head
+constexpr int kAttnPasses = 8; // cached positions per lane group and workgroup
+// most cached positions per workgroup: 128 for head_dim 64, 64 for head_dim 128
+constexpr int attn_chunk_cap(int lpt) { return kAttnPasses * (kBlock / lpt); }
 
-// LPT lanes share a cached position (head_dim / 4): 16 or 32.
+// LPT lanes share a cached position (head_dim / 4): 16 or 32.  Every lane first asks for all of
+// its K and V pieces of the chunk (at most 2 x 8 sixteen-byte loads in flight), so the chunk
+// costs one trip to memory; scores, soft-max and the weighted sum then run out of registers and LDS.
 template <class P, int LPT>
 __global__ __launch_bounds__(kBlock) void decode_attention_kernel(const AttnArgs g, const FusedArgs a) {
     constexpr int HD = LPT * 4;
     constexpr int TPB = kBlock / LPT; // positions per pass
+    constexpr int CAP = attn_chunk_cap(LPT);
+    constexpr int IPL = CAP / 64; // chunk positions per lane in the soft-max phase
     constexpr int ri0 = reduce_index<P>(0), ri1 = reduce_index<P>(1);
     constexpr int src0 = P::code[ri0][1], src1 = P::code[ri1][1];
-    __shared__ float sc[kAttnRows][kAttnChunk];
-    __shared__ float red[TPB][kAttnRows * HD / 4 + 1][4];
+    static_assert((P::code[ri0][0] & ~kInstrU32) == kRowMax && (P::code[ri1][0] & ~kInstrU32) == kRowSum,
+                  "a soft-max: row maximum, then row sum");
+    __shared__ float sc[kAttnRows][CAP];
+    __shared__ float red[TPB][kAttnRows * LPT + 1][4];
     const uint32_t tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
     const uint32_t split = blockIdx.x, b = blockIdx.y;
     const uint32_t t0 = split * g.chunk, t1 = min(g.T, t0 + g.chunk);
@@ -79,38 +97,53 @@ __global__ __launch_bounds__(kBlock) void decode_attention_kernel(const AttnArgs
         }
     }
     const uint32_t row0 = (uint32_t)(op / g.T); // first row of this group in the program's [rows, T] space
+    const uint32_t l = tid % LPT, sub = tid / LPT;
+
+    float4v kf[kAttnPasses], vf[kAttnPasses];
+#pragma unroll
+    for (int ps = 0; ps < kAttnPasses; ps++) {
+        const uint32_t t = t0 + sub + ps * TPB;
+        kf[ps] = (float4v){0.f, 0.f, 0.f, 0.f};
+        vf[ps] = (float4v){0.f, 0.f, 0.f, 0.f};
+        if (t < t1) {
+            kf[ps] = *reinterpret_cast<const float4v *>(g.Kc + ok + (int64_t)t * g.k_st + l * 4);
+            vf[ps] = *reinterpret_cast<const float4v *>(g.V + ov + (int64_t)t * g.v_st + l * 4);
+        }
+    }
 
     // ---- scores of the chunk: LPT lanes per position, one 16-byte piece of head_dim each
     {
-        const uint32_t l = tid % LPT, sub = tid / LPT;
         float4v qf[kAttnRows];
 #pragma unroll
         for (int m = 0; m < kAttnRows; m++) {
             qf[m] = (float4v){0.f, 0.f, 0.f, 0.f};
             if ((uint32_t)m < g.M) qf[m] = *reinterpret_cast<const float4v *>(g.Q + oq + (int64_t)m * g.q_sm + l * 4);
         }
-        for (uint32_t t = t0 + sub; t < t0 + (t1 - t0 + TPB - 1) / TPB * TPB; t += TPB) {
-            float4v kf = (float4v){0.f, 0.f, 0.f, 0.f};
-            if (t < t1) kf = *reinterpret_cast<const float4v *>(g.Kc + ok + (int64_t)t * g.k_st + l * 4);
+        const uint32_t passes = (t1 - t0 + TPB - 1) / TPB;
 #pragma unroll
-            for (int m = 0; m < kAttnRows; m++) {
-                if ((uint32_t)m < g.M) {
-                    float v = fmaf(qf[m][3], kf[3], fmaf(qf[m][2], kf[2], fmaf(qf[m][1], kf[1], qf[m][0] * kf[0])));
+        for (int ps = 0; ps < kAttnPasses; ps++) {
+            if ((uint32_t)ps < passes) {
+                const uint32_t t = t0 + sub + ps * TPB;
 #pragma unroll
-                    for (int s = LPT / 2; s >= 1; s >>= 1) v += __shfl_xor(v, s);
-                    if (l == 0 && t < t1) sc[m][t - t0] = v;
+                for (int m = 0; m < kAttnRows; m++) {
+                    if ((uint32_t)m < g.M) {
+                        float v = fmaf(qf[m][3], kf[ps][3], fmaf(qf[m][2], kf[ps][2], fmaf(qf[m][1], kf[ps][1], qf[m][0] * kf[ps][0])));
+                        v = row16_sum(v);
+                        if (LPT == 32) v += __shfl_xor(v, 16);
+                        if (l == 0 && t < t1) sc[m][t - t0] = v;
+                    }
                 }
             }
         }
     }
     __syncthreads();
 
-    // ---- the soft-max program on the chunk: a wave per query row
+    // ---- the soft-max program on the chunk: a wave per query row, IPL positions per lane
     for (uint32_t m = wave; m < g.M; m += kBlock / 64) {
         const uint32_t row = row0 + m;
         int64_t base[P::nleaf + 1];
 #pragma unroll
-        for (int l = 0; l <= P::nleaf; l++) base[l] = 0;
+        for (int i = 0; i <= P::nleaf; i++) base[i] = 0;
         {
             uint32_t rr = row;
             for (uint32_t d = 0; d < a.g.nouter; d++) {
@@ -118,31 +151,39 @@ __global__ __launch_bounds__(kBlock) void decode_attention_kernel(const AttnArgs
                 const int64_t i = (int64_t)(rr - q * a.g.od[d]);
                 rr = q;
 #pragma unroll
-                for (int l = 1; l < P::nleaf; l++) base[l] += i * a.leaf[l].os[d];
+                for (int lf = 1; lf < P::nleaf; lf++) base[lf] += i * a.leaf[lf].os[d];
+            }
+        }
+        LeafWords<P, 1> w[IPL];
+#pragma unroll
+        for (int c = 0; c < IPL; c++) {
+            const uint32_t i = lane + c * 64;
+            if (i < t1 - t0) {
+                aot_fetch_from<P, 1>(a, base, t0 + i, w[c]); // leaf 0 is the score
+                w[c].v[0][0] = asu(sc[m][i]);
             }
         }
         uint32_t rs[kMaxRowReduce] = {0, 0, 0};
-        constexpr bool max0 = (P::code[ri0][0] & ~kInstrU32) == kRowMax;
-        static_assert(max0 && (P::code[ri1][0] & ~kInstrU32) == kRowSum, "a soft-max: row maximum, then row sum");
         uint32_t acc = row_init(true, true);
-        for (uint32_t i = lane; i < t1 - t0; i += 64) {
-            LeafWords<P, 1> w;
-            aot_fetch_from<P, 1>(a, base, t0 + i, w); // leaf 0 is the score
-            w.v[0][0] = asu(sc[m][i]);
-            const Values<P, 1> s = aot_eval<P, 1, ri0>(w, rs, a.fault);
-            acc = row_merge(true, true, acc, s.v[src0][0]);
+#pragma unroll
+        for (int c = 0; c < IPL; c++) {
+            if (lane + c * 64 < t1 - t0) {
+                const Values<P, 1> s = aot_eval<P, 1, ri0>(w[c], rs, a.fault);
+                acc = row_merge(true, true, acc, s.v[src0][0]);
+            }
         }
 #pragma unroll
         for (int sft = 32; sft >= 1; sft >>= 1) acc = row_merge(true, true, acc, (uint32_t)__shfl_xor((int)acc, sft));
         rs[0] = acc;
         uint32_t sum = row_init(false, true);
-        for (uint32_t i = lane; i < t1 - t0; i += 64) {
-            LeafWords<P, 1> w;
-            aot_fetch_from<P, 1>(a, base, t0 + i, w);
-            w.v[0][0] = asu(sc[m][i]);
-            const Values<P, 1> s = aot_eval<P, 1, ri1>(w, rs, a.fault);
-            sum = row_merge(false, true, sum, s.v[src1][0]);
-            sc[m][i] = asf(s.v[src1][0]); // the un-normalised weight
+#pragma unroll
+        for (int c = 0; c < IPL; c++) {
+            const uint32_t i = lane + c * 64;
+            if (i < t1 - t0) {
+                const Values<P, 1> s = aot_eval<P, 1, ri1>(w[c], rs, a.fault);
+                sum = row_merge(false, true, sum, s.v[src1][0]);
+                sc[m][i] = asf(s.v[src1][0]); // the un-normalised weight
+            }
         }
 #pragma unroll
         for (int sft = 32; sft >= 1; sft >>= 1) sum = row_merge(false, true, sum, (uint32_t)__shfl_xor((int)sum, sft));
@@ -154,23 +195,24 @@ __global__ __launch_bounds__(kBlock) void decode_attention_kernel(const AttnArgs
     }
     __syncthreads();
 
-    // ---- weights times V: LPT lanes cover head_dim, TPB groups split the positions
+    // ---- weights times V: the lane's V pieces are those of its positions, head_dim piece l
     {
-        const uint32_t ng = tid % LPT, kg = tid / LPT;
         float4v o[kAttnRows];
 #pragma unroll
         for (int m = 0; m < kAttnRows; m++) o[m] = (float4v){0.f, 0.f, 0.f, 0.f};
-#pragma unroll 4
-        for (uint32_t t = t0 + kg; t < t1; t += TPB) {
-            const float4v vf = *reinterpret_cast<const float4v *>(g.V + ov + (int64_t)t * g.v_st + ng * 4);
 #pragma unroll
-            for (int m = 0; m < kAttnRows; m++) {
-                if ((uint32_t)m < g.M) {
-                    const float w = sc[m][t - t0];
-                    o[m][0] = fmaf(w, vf[0], o[m][0]);
-                    o[m][1] = fmaf(w, vf[1], o[m][1]);
-                    o[m][2] = fmaf(w, vf[2], o[m][2]);
-                    o[m][3] = fmaf(w, vf[3], o[m][3]);
+        for (int ps = 0; ps < kAttnPasses; ps++) {
+            const uint32_t t = t0 + sub + ps * TPB;
+            if (t < t1) {
+#pragma unroll
+                for (int m = 0; m < kAttnRows; m++) {
+                    if ((uint32_t)m < g.M) {
+                        const float wgt = sc[m][t - t0];
+                        o[m][0] = fmaf(wgt, vf[ps][0], o[m][0]);
+                        o[m][1] = fmaf(wgt, vf[ps][1], o[m][1]);
+                        o[m][2] = fmaf(wgt, vf[ps][2], o[m][2]);
+                        o[m][3] = fmaf(wgt, vf[ps][3], o[m][3]);
+                    }
                 }
             }
         }
@@ -178,7 +220,7 @@ __global__ __launch_bounds__(kBlock) void decode_attention_kernel(const AttnArgs
         for (int m = 0; m < kAttnRows; m++)
             if ((uint32_t)m < g.M) {
 #pragma unroll
-                for (int j = 0; j < 4; j++) red[kg][m * LPT + ng][j] = o[m][j];
+                for (int j = 0; j < 4; j++) red[sub][m * LPT + l][j] = o[m][j];
             }
         __syncthreads();
         for (uint32_t e = tid; e < g.M * HD; e += kBlock) {
@@ -202,8 +244,10 @@ __global__ __launch_bounds__(kBlock) void decode_attention_combine_kernel(const 
     const uint32_t m = (uint32_t)(bm % M);
     const uint64_t b = bm / M;
     float gmax = kF32Min;
+#pragma unroll 8
     for (uint32_t c = 0; c < splits; c++) gmax = fmaxf(gmax, part_ml[((b * splits + c) * M + m) * 2]);
     float num = 0.0f, den = 0.0f;
+#pragma unroll 8
     for (uint32_t c = 0; c < splits; c++) {
         const float *ml = part_ml + ((b * splits + c) * M + m) * 2;
         const float w = expf(ml[0] - gmax);

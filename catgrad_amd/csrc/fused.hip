@@ -582,6 +582,11 @@ void trace_program(cg_backend *be, const Pending &p, int ninstr, const char *how
 
 } // namespace
 
+static int64_t attn_blocks() {
+    static const int64_t n = [] { const char *e = getenv("CG_ATTN_BLOCKS"); return e ? atoll(e) : 1024ll; }();
+    return n;
+}
+
 int launch_decode_attention(cg_backend *be, const Pending &p, const int64_t *pdims, int prank, const cg_tensor *q,
                             const cg_tensor *kt, const cg_tensor *v, cg_tensor *out) {
     using P = RowsSoftmaxCausal;
@@ -632,9 +637,10 @@ int launch_decode_attention(cg_backend *be, const Pending &p, const int64_t *pdi
     g.T = (uint32_t)T;
     g.hd = (uint32_t)hd;
     // enough workgroups for every CU twice over, chunks of 64..256 positions
-    const int64_t want = std::max<int64_t>(1, 512 / f1.batch);
-    int64_t chunk = std::min<int64_t>(kAttnChunk, std::max<int64_t>(64, (T + want - 1) / want));
-    chunk = (chunk + 15) / 16 * 16;
+    const int64_t cap = attn_chunk_cap(hd == 64 ? 16 : 32);
+    const int64_t want = std::max<int64_t>(1, attn_blocks() / f1.batch);
+    int64_t chunk = std::min<int64_t>(cap, std::max<int64_t>(32, (T + want - 1) / want));
+    chunk = std::min<int64_t>(cap, (chunk + 15) / 16 * 16);
     g.chunk = (uint32_t)chunk;
     g.splits = (uint32_t)((T + chunk - 1) / chunk);
     g.nb = (uint32_t)f1.nb;
