@@ -62,6 +62,10 @@ struct ProfPending {
 
 } // namespace cg
 
+namespace cg {
+struct LazyMm;
+}
+
 struct cg_backend {
     int device = 0;
     hipStream_t stream = nullptr;
@@ -76,6 +80,7 @@ struct cg_backend {
     bool stage_busy[2] = {false, false};
     unsigned stage_next = 0;
     std::string name;
+    std::vector<cg::LazyMm *> lazy_open; // groupable lazy products not yet computed (not retained)
     bool fuse = true; // defer element-wise ops and fuse them (CG_FUSE=0 switches it off)
     bool aot = true;  // use the compiled kernels for listed programs (CG_AOT=0: interpreter only)
     uint64_t programs_compiled = 0, programs_interpreted = 0; // launches of fused programs, by kernel kind
@@ -225,6 +230,11 @@ struct LazyMm {
     Buffer *result = nullptr;             // retained once computed
     int64_t dims[kMaxRank] = {0};
     int rank = 0;
+    // A decode-time linear layer (few rows times a weight matrix): products of this kind that
+    // share their left operand and are still open when one of them is needed (q / k / v, gate / up)
+    // are computed by one grouped launch.  `be` is set while the product is listed as open.
+    bool groupable = false;
+    cg_backend *be = nullptr;
 };
 void lazy_mm_release(LazyMm *m);
 // Computes the product if it has not been yet.
@@ -343,6 +353,7 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
 // are merged, a split axis contributes its two parts, and the innermost batch axis is folded
 // into M when y ignores it and x walks it as more rows.  Reads shapes and strides only, so x
 // may be a descriptor without memory.
+constexpr int kDeclined = -1000; // "not my case": the caller takes the ordinary route
 constexpr int kMaxBatchAxes = 6;
 struct MmFold {
     int64_t M = 0, N = 0, K = 0, batch = 0;
@@ -352,12 +363,14 @@ struct MmFold {
     int64_t a_bs[kMaxBatchAxes] = {0}, b_bs[kMaxBatchAxes] = {0};
 };
 int fold_matmul(const cg_tensor *x, const cg_tensor *y, MmFold *f);
+// Several skinny products x . ys[i] -> outs[i] (n of them, the same x) in one launch; kDeclined (declared
+// below) when the shapes do not allow it.
+int launch_matmul_group(cg_backend *be, const cg_tensor *x, const cg_tensor *const *ys, cg_tensor *const *outs, int n);
 
 // Decode-time attention in one pass: out = softmax-program(q . kT) . v, where `p` is the deferred
 // soft-max program whose leaf 0 is the (never computed) lazy product q . kT and (pdims, prank) its
 // shape.  Returns kDeclined when the shapes or the program are not what the kernel handles; the
 // caller then takes the ordinary route.
-constexpr int kDeclined = -1000;
 int launch_decode_attention(cg_backend *be, const Pending &p, const int64_t *pdims, int prank, const cg_tensor *q,
                             const cg_tensor *kt, const cg_tensor *v, cg_tensor *out);
 

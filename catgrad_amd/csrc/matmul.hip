@@ -295,13 +295,13 @@ template <int MM> __global__ __launch_bounds__(kThreads) void skinny_kt_kernel(c
 // activation rows stay in L1/L2).  SPLIT: the four waves of the block share the columns
 // and split K, for shapes with too few columns to fill the chip.
 template <int MM, int COLS, bool SPLIT>
-__global__ __launch_bounds__(kThreads) void skinny_kt_wide_kernel(const MmArgs a) {
+__device__ __forceinline__ void skinny_kt_wide_body(const MmArgs &a, const uint32_t block_x, const uint32_t block_y) {
     const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x % 64;
-    const uint32_t group = SPLIT ? blockIdx.x : blockIdx.x * 4 + wave;
+    const uint32_t group = SPLIT ? block_x : block_x * 4 + wave;
     const uint32_t n0 = group * COLS;
     const bool live = n0 < a.N;
     int64_t oa, ob;
-    batch_offsets(a, blockIdx.y, oa, ob);
+    batch_offsets(a, block_y, oa, ob);
     const uint32_t *A = a.A + oa;
     const uint32_t *B = a.B + ob;
     float acc[COLS][MM];
@@ -354,15 +354,40 @@ __global__ __launch_bounds__(kThreads) void skinny_kt_wide_kernel(const MmArgs a
         if (threadIdx.x < COLS * MM) {
             uint32_t c = threadIdx.x / MM, m = threadIdx.x % MM;
             float v = (part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]);
-            if (n0 + c < a.N && m < a.M) a.C[((uint64_t)blockIdx.y * a.M + m) * a.N + n0 + c] = asu(v);
+            if (n0 + c < a.N && m < a.M) a.C[((uint64_t)block_y * a.M + m) * a.N + n0 + c] = asu(v);
         }
     } else if (live && lane == 0) {
 #pragma unroll
         for (int c = 0; c < COLS; c++)
 #pragma unroll
             for (int m = 0; m < MM; m++)
-                if (n0 + c < a.N && (uint32_t)m < a.M) a.C[((uint64_t)blockIdx.y * a.M + m) * a.N + n0 + c] = asu(acc[c][m]);
+                if (n0 + c < a.N && (uint32_t)m < a.M) a.C[((uint64_t)block_y * a.M + m) * a.N + n0 + c] = asu(acc[c][m]);
     }
+}
+
+template <int MM, int COLS, bool SPLIT>
+__global__ __launch_bounds__(kThreads) void skinny_kt_wide_kernel(const MmArgs a) {
+    skinny_kt_wide_body<MM, COLS, SPLIT>(a, blockIdx.x, blockIdx.y);
+}
+
+// Several products that share their left operand (the q / k / v projections of a decode step,
+// gate and up) in one launch: the workgroups are dealt to the problems in order.
+constexpr int kMaxGroup = 4;
+struct MmGroup {
+    MmArgs p[kMaxGroup];
+    uint32_t first[kMaxGroup + 1]; // first workgroup of each problem; first[n] = grid size
+    uint32_t n;
+};
+__device__ __forceinline__ uint32_t group_problem(const MmGroup &g, uint32_t &block_x) {
+    uint32_t p = 0;
+    while (p + 1 < g.n && blockIdx.x >= g.first[p + 1]) p++;
+    block_x = blockIdx.x - g.first[p];
+    return p;
+}
+template <int MM> __global__ __launch_bounds__(kThreads) void skinny_kt_wide_group_kernel(const MmGroup g) {
+    uint32_t bx;
+    const uint32_t p = group_problem(g, bx);
+    skinny_kt_wide_body<MM, 1, false>(g.p[p], bx, 0);
 }
 
 // Skinny kernel on the 4x4x1 matrix instruction (16 independent 4x4 outer products per
@@ -374,13 +399,13 @@ __global__ __launch_bounds__(kThreads) void skinny_kt_wide_kernel(const MmArgs a
 // in registers (8 x 16 bytes per lane and row group) and reuse it for CG groups of four
 // columns, so the activation rows are fetched once per 4 * CG columns.
 template <int MM, int CG>
-__global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_kernel(const MmArgs a) {
+__device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const uint32_t block_x, const uint32_t block_y) {
     constexpr int G = MM / 4;
     const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x % 64;
     const uint32_t j = lane % 4, b = lane / 4;
-    const uint32_t n0 = blockIdx.x * (4 * CG);
+    const uint32_t n0 = block_x * (4 * CG);
     int64_t oa, ob;
-    batch_offsets(a, blockIdx.y, oa, ob);
+    batch_offsets(a, block_y, oa, ob);
     const uint32_t *wrow[CG];
 #pragma unroll
     for (int c = 0; c < CG; c++) wrow[c] = a.B + ob + (int64_t)min(n0 + 4 * c + j, a.N - 1) * a.b_sn;
@@ -440,8 +465,17 @@ __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_kernel(const MmA
     if (threadIdx.x < CG * MM * 4) {
         const uint32_t c = threadIdx.x / (MM * 4), m = threadIdx.x / 4 % MM, col = n0 + 4 * c + threadIdx.x % 4;
         const float v = (part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]);
-        if (col < a.N && m < a.M) a.C[((uint64_t)blockIdx.y * a.M + m) * a.N + col] = asu(v);
+        if (col < a.N && m < a.M) a.C[((uint64_t)block_y * a.M + m) * a.N + col] = asu(v);
     }
+}
+
+template <int MM, int CG> __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_kernel(const MmArgs a) {
+    skinny_kt_mfma_xreg_body<MM, CG>(a, blockIdx.x, blockIdx.y);
+}
+template <int MM, int CG> __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_group_kernel(const MmGroup g) {
+    uint32_t bx;
+    const uint32_t p = group_problem(g, bx);
+    skinny_kt_mfma_xreg_body<MM, CG>(g.p[p], bx, 0);
 }
 
 // Vectorised skinny kernel for short K (K <= 4*LPC, e.g. q.K^T of a decode step with
@@ -636,8 +670,9 @@ int fold_matmul(const cg_tensor *x, const cg_tensor *y, MmFold *f) {
     return CG_OK;
 }
 
-int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_tensor *out) {
-    MmArgs a;
+// Kernel arguments of x . y -> c (row-major); the folded extents come back in *f.
+static int make_mm_args(const cg_tensor *x, const cg_tensor *y, void *c, MmArgs *ap, MmFold *fp) {
+    MmArgs &a = *ap;
     memset(&a, 0, sizeof a);
     const void *pa, *pb;
     int rc = device_ptr(x, &pa);
@@ -646,8 +681,8 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
     if (rc) return rc;
     a.A = static_cast<const uint32_t *>(pa);
     a.B = static_cast<const uint32_t *>(pb);
-    a.C = static_cast<uint32_t *>(out->buf->ptr);
-    MmFold f;
+    a.C = static_cast<uint32_t *>(c);
+    MmFold &f = *fp;
     rc = fold_matmul(x, y, &f);
     if (rc) return rc;
     const int64_t M = f.M, N = f.N, K = f.K, batch = f.batch;
@@ -677,6 +712,55 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
     const bool b_kfast = a.b_sk == 1 || K == 1, b_nfast = !b_kfast && a.b_sn == 1;
     a.a_vec = a_al && ((a.a_sk == 1 && a.a_sm % 4 == 0) || (a_mfast && a.a_sk % 4 == 0));
     a.b_vec = b_al && ((a.b_sk == 1 && a.b_sn % 4 == 0) || (b_nfast && a.b_sk % 4 == 0));
+    return CG_OK;
+}
+
+int launch_matmul_group(cg_backend *be, const cg_tensor *x, const cg_tensor *const *ys, cg_tensor *const *outs, int n) {
+    if (n < 2 || n > kMaxGroup || x->dt != CG_F32) return kDeclined;
+    MmGroup g;
+    memset(&g, 0, sizeof g);
+    double bytes = distinct_bytes(x);
+    bool all_wide = true;
+    for (int i = 0; i < n; i++) {
+        MmFold f;
+        int rc = make_mm_args(x, ys[i], outs[i]->buf->ptr, &g.p[i], &f);
+        if (rc) return rc;
+        const MmArgs &a = g.p[i];
+        const bool vec = a.a_vec && a.b_vec && a.a_sk == 1 && a.K % 4 == 0;
+        if (f.batch != 1 || a.M > 8 || a.b_sk != 1 || !vec || a.K <= 256 || a.N < 4) return kDeclined;
+        if (i > 0 && (a.M != g.p[0].M || a.K != g.p[0].K || a.a_sm != g.p[0].a_sm)) return kDeclined;
+        all_wide = all_wide && a.N >= 8192;
+        bytes += distinct_bytes(ys[i]) + distinct_bytes(outs[i]);
+    }
+    const bool xreg = all_wide && g.p[0].M <= 4;
+    uint32_t blocks = 0;
+    for (int i = 0; i < n; i++) {
+        g.first[i] = blocks;
+        blocks += xreg ? (g.p[i].N + 7) / 8 : (g.p[i].N + 3) / 4;
+    }
+    g.first[n] = blocks;
+    g.n = (uint32_t)n;
+    ProfScope prof(be, CG_K_GEMM_SKINNY, bytes);
+    if (xreg)
+        hipLaunchKernelGGL((skinny_kt_mfma_xreg_group_kernel<4, 2>), dim3(blocks), dim3(kThreads), 0, be->stream, g);
+    else if (g.p[0].M <= 1)
+        hipLaunchKernelGGL((skinny_kt_wide_group_kernel<1>), dim3(blocks), dim3(kThreads), 0, be->stream, g);
+    else if (g.p[0].M <= 4)
+        hipLaunchKernelGGL((skinny_kt_wide_group_kernel<4>), dim3(blocks), dim3(kThreads), 0, be->stream, g);
+    else
+        hipLaunchKernelGGL((skinny_kt_wide_group_kernel<8>), dim3(blocks), dim3(kThreads), 0, be->stream, g);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CG_OK : hip_fail(e, "grouped matmul launch");
+}
+
+int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_tensor *out) {
+    MmArgs a;
+    MmFold f;
+    int rc = make_mm_args(x, y, out->buf->ptr, &a, &f);
+    if (rc) return rc;
+    const int64_t M = f.M, N = f.N, K = f.K, batch = f.batch;
+    const bool a_mfast = !(a.a_sk == 1 || K == 1) && a.a_sm == 1;
+    const bool b_nfast = !(a.b_sk == 1 || K == 1) && a.b_sn == 1;
 
     if (batch > 65535) return fail(CG_ERR_UNSUPPORTED, "matmul: more than 65535 batch entries after folding");
     const bool f32 = x->dt == CG_F32;

@@ -138,9 +138,22 @@ Pending::~Pending() {
     }
 }
 
+static void lazy_mm_close(LazyMm *m) { // no longer open for grouping
+    if (!m->be) return;
+    auto &v = m->be->lazy_open;
+    for (size_t i = 0; i < v.size(); i++)
+        if (v[i] == m) {
+            v[i] = v.back();
+            v.pop_back();
+            break;
+        }
+    m->be = nullptr;
+}
+
 void lazy_mm_release(LazyMm *m) {
     if (!m) return;
     if (m->rc.fetch_sub(1) == 1) {
+        lazy_mm_close(m);
         release(m->x);
         release(m->y);
         buffer_release(m->result);
@@ -150,6 +163,32 @@ void lazy_mm_release(LazyMm *m) {
 
 int lazy_mm_force(cg_backend *be, LazyMm *m) {
     if (m->result) return CG_OK;
+    if (m->groupable && m->be) {
+        // the other open products with the same left operand go along in the same launch
+        LazyMm *grp[4] = {m};
+        int n = 1;
+        for (LazyMm *o : be->lazy_open)
+            if (o != m && !o->result && o->x == m->x && n < 4) grp[n++] = o;
+        if (n > 1) {
+            cg_tensor *outs[4] = {nullptr, nullptr, nullptr, nullptr};
+            const cg_tensor *ys[4];
+            int rc = CG_OK;
+            for (int i = 0; i < n && !rc; i++) {
+                ys[i] = grp[i]->y;
+                rc = new_dense(be, CG_F32, grp[i]->dims, grp[i]->rank, &outs[i]);
+            }
+            if (!rc) rc = launch_matmul_group(be, m->x, ys, outs, n);
+            if (rc == CG_OK)
+                for (int i = 0; i < n; i++) {
+                    grp[i]->result = outs[i]->buf;
+                    outs[i]->buf = nullptr;
+                    lazy_mm_close(grp[i]);
+                }
+            for (int i = 0; i < n; i++) release(outs[i]);
+            if (rc != kDeclined) return rc;
+        }
+    }
+    lazy_mm_close(m);
     cg_tensor *o;
     int rc = new_dense(be, CG_F32, m->dims, m->rank, &o);
     if (rc) return rc;
@@ -653,28 +692,21 @@ static int ensure_concrete(cg_tensor *t) {
     cg_backend *be = t->be;
     hipError_t he = hipSetDevice(be->device);
     if (he != hipSuccess) return hip_fail(he, "hipSetDevice");
-    if (t->pend->nleaf == 1 && t->pend->ninstr == 1 && t->pend->leaf[0].lazy && (t->pend->ins[0].op & ~kInstrU32) == kCopy &&
-        t->pend->leaf[0].offset == 0) {
-        // the plain result of a lazy product: compute it and adopt its buffer
-        cg_tensor probe;
-        probe.rank = t->rank;
-        memcpy(probe.dims, t->dims, sizeof probe.dims);
-        set_row_major(&probe);
-        bool dense = true;
-        for (int i = 0; i < t->rank; i++) dense = dense && (t->dims[i] <= 1 || probe.strides[i] == t->pend->leaf[0].strides[i]);
-        if (dense) {
-            LazyMm *m = t->pend->leaf[0].lazy;
-            int rc = lazy_mm_force(be, m);
-            if (rc) return rc;
-            m->result->rc.fetch_add(1);
-            t->buf = m->result;
-            t->offset = 0;
-            set_row_major(t);
-            Pending *old = t->pend;
-            t->pend = nullptr;
-            delete old;
-            return CG_OK;
-        }
+    if (t->pend->nleaf == 1 && t->pend->ninstr == 1 && (t->pend->ins[0].op & ~kInstrU32) == kCopy && !t->pend->leaf[0].pw &&
+        !t->pend->leaf[0].uniform) {
+        // nothing but a view of one buffer (possibly the result of a lazy product, computed now):
+        // the handle becomes that view
+        int lrc = resolve_lazy_leaves(be, *t->pend);
+        if (lrc) return lrc;
+        const LeafView &lv = t->pend->leaf[0];
+        lv.buf->rc.fetch_add(1);
+        t->buf = lv.buf;
+        t->offset = lv.offset;
+        memcpy(t->strides, lv.strides, sizeof t->strides);
+        Pending *old = t->pend;
+        t->pend = nullptr;
+        delete old;
+        return CG_OK;
     }
     Buffer *b = new Buffer;
     b->be = be;
@@ -1732,9 +1764,18 @@ int cg_matmul(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **out) {
         int64_t n_out = 1;
         for (int i = 0; i < r; i++) n_out *= od[i];
         const int64_t K = x->dims[r - 1];
-        if (b->fuse && x->dt == CG_F32 && r == 4 && n_out > 0 && x->dims[r - 2] <= 8 && K > 0 && K <= 256 &&
-            K % 4 == 0 && !x->uniform && !y->uniform && x->split < 0 && y->strides[r - 2] == 1 && od[r - 1] > 1) {
+        const bool scores = r == 4 && x->dims[r - 2] <= 8 && K > 0 && K <= 256 && od[r - 1] > 1;
+        // a decode-time linear layer: at most 8 rows in all, the weight shared by the batch
+        const bool linear = r == 3 && x->dims[0] * x->dims[1] <= 8 && K > 256 && od[r - 1] >= 64 && y->strides[0] == 0 &&
+                            y->split < 0 && is_contiguous(x);
+        if (b->fuse && x->dt == CG_F32 && n_out > 0 && (scores || linear) && K % 4 == 0 && !x->uniform && !y->uniform &&
+            x->split < 0 && y->strides[r - 2] == 1) {
             LazyMm *m = new LazyMm;
+            if (linear) {
+                m->groupable = true;
+                m->be = b;
+                b->lazy_open.push_back(m);
+            }
             retain(x);
             retain(y);
             m->x = x;
@@ -2090,6 +2131,11 @@ int cg_concat(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor *
         // operand is a plain view, or the negation of one (rotate_half of the rotary embedding,
         // helpers/rope.rs:423-427): its consumer then reads both halves in place.
         LeafView lv;
+        for (cg_tensor *t : {x, y})
+            if (t->pend) {
+                int lrc = resolve_lazy_leaves(b, *t->pend);
+                if (lrc) return lrc;
+            }
         auto part = [&](cg_tensor *t, Buffer **buf, int64_t *strides, int64_t *offset, bool *neg) {
             if (t->uniform || t->split >= 0) return false;
             const int64_t *st;
@@ -2102,11 +2148,12 @@ int cg_concat(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor *
             } else {
                 const Pending *p = t->pend;
                 if (p->nleaf != 1 || p->ninstr != 1 || p->nred || p->leaf[0].uniform || p->leaf[0].pw || p->leaf[0].lazy) return false;
-                if (p->ins[0].op != kNeg) return false; // f32 negation only
+                const int pop = p->ins[0].op & ~kInstrU32;
+                if (p->ins[0].op != kNeg && pop != kCopy) return false; // a view, or the f32 negation of one
                 *buf = p->leaf[0].buf;
                 st = p->leaf[0].strides;
                 *offset = p->leaf[0].offset;
-                *neg = true;
+                *neg = pop != kCopy;
             }
             memcpy(strides, st, sizeof(int64_t) * kMaxRank);
             return true;

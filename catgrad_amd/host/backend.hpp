@@ -13,6 +13,7 @@
 
 #include <cstdint>
 #include <stdexcept>
+#include <chrono>
 #include <string>
 #include <utility>
 #include <vector>
@@ -115,6 +116,8 @@ class Backend {
     }
     std::string name() const { return abi_.cg_backend_name(b_); }
     uint64_t calls = 0; // backend method calls issued (for the launch-count statistics)
+    bool time_calls = false;
+    double seconds_in_backend = 0;
 
     Tensor zeros(const Shape &shape, cg_dtype dt) {
         return out([&](cg_tensor **o) { return abi_.cg_zeros(b_, dt, shape.data(), shape.size(), o); });
@@ -238,7 +241,14 @@ class Backend {
     template <class F> Tensor out(F &&f) {
         calls++;
         cg_tensor *o = nullptr;
-        check(f(&o));
+        if (time_calls) { // diagnostic: how much of a run is spent inside the backend library
+            const auto t0 = std::chrono::steady_clock::now();
+            const int rc = f(&o);
+            seconds_in_backend += std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+            check(rc);
+        } else {
+            check(f(&o));
+        }
         return Tensor(&abi_, o);
     }
     Tensor from_vec(cg_dtype dt, const void *data, size_t len, const Shape &shape) {

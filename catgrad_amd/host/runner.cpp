@@ -1,6 +1,8 @@
 // C entry points of the host driver; see runner.h.
 #include "runner.h"
 
+#include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <memory>
 
@@ -96,7 +98,13 @@ int cgm_generate(cgm_session *s, const uint32_t *prompt, size_t B, size_t S, siz
     return guarded([&] {
         LlmModel m(*s->interp, s->config);
         GenerateStats st;
+        const char *tc = getenv("CGH_TIME_CALLS");
+        s->interp->backend.time_calls = tc && tc[0] == '1';
+        s->interp->backend.seconds_in_backend = 0;
         generate(m, *s->interp, prompt, B, S, steps, max_positions, out_tokens, &st);
+        if (s->interp->backend.time_calls)
+            fprintf(stderr, "[host] generate: %.3f ms inside backend calls (those that return tensors), %.3f ms total\n",
+                    s->interp->backend.seconds_in_backend * 1e3, (st.prefill_s + st.decode_s) * 1e3);
         stats4[0] = st.prefill_s;
         stats4[1] = st.decode_s;
         stats4[2] = (double)st.prefill_calls;

@@ -3,7 +3,7 @@
 //! Drop this file in as `catgrad/src/interpreter/backend/hip.rs`, add
 //! `#[cfg(feature = "hip-backend")] pub mod hip;` next to the other backends in
 //! `catgrad/src/interpreter/backend/mod.rs` (lines 10-14 there) and a `hip-backend`
-//! feature in `catgrad/Cargo.toml`; link with `-lcatgrad_hip`.
+//! feature in `catgrad/Cargo.toml`; link with `-lcatgrad_hip` (a `cargo:rustc-link-lib=dylib=catgrad_hip` line in build.rs).
 //!
 //! The shim is mechanical: every trait method forwards to the C entry point that
 //! include/catgrad_hip.h declares for it.  The C ABI has the trait's own ownership model —
