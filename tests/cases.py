@@ -892,6 +892,58 @@ def _():
     return run, expect
 
 
+# ---- decode-time linear layers: lazy, grouped by their shared left operand ---------------------------------------
+def _linear(be, x, w):
+    """`nn::linear_b_param` without bias (stdlib/nn/mod.rs:182-204): x [B,S,K] times w [N,K] transposed."""
+    B, _, K = x.shape
+    N = w.shape[0]
+    return be.matmul(x, be.broadcast(be.transpose(w, 0, 1), (B, K, N)))
+
+
+for _B, _K, _Ns in ((4, 512, (512, 128, 128)), (1, 1024, (64, 2048)), (8, 388, (300, 8200)), (4, 512, (8192, 8200)),
+                    (2, 2304, (8192, 8192, 96, 100, 104))):
+    @case(f"linear_group_B{_B}_K{_K}_N{'_'.join(map(str, _Ns))}", "red",
+          (lambda B=_B, K=_K, Ns=_Ns: [np.abs(f32(500 + K, (B, 1, K)).astype(np.float64)) @
+                                         np.abs(f32(501 + K + i, (n, K)).astype(np.float64)).T
+                                         for i, n in enumerate(Ns)]))
+    def _(B=_B, K=_K, Ns=_Ns):
+        x = f32(500 + K, (B, 1, K))
+        ws = [f32(501 + K + i, (n, K)) for i, n in enumerate(Ns)]
+
+        def run(be):
+            tx = be.from_numpy(x)
+            ys = [_linear(be, tx, be.from_numpy(w)) for w in ws]     # all issued before any is read
+            return N(be, *reversed(ys))[::-1]                          # ... and read last one first
+
+        return run, (lambda: [x.astype(np.float64) @ w.astype(np.float64).T for w in ws])
+
+
+@case("linear_lazy_consumers", "red")
+def _():
+    """Lazy products consumed through views, element-wise programs, concat and reductions, and one that
+    is never read."""
+    x = np.abs(f32(520, (4, 1, 640)))      # positive data: no cancellation, so 1e-3 of the value itself applies
+    w1, w2, w3 = np.abs(f32(521, (256, 640))), np.abs(f32(522, (256, 640))), np.abs(f32(523, (64, 640)))
+
+    def run(be):
+        tx = be.from_numpy(x)
+        a, b_, c = (_linear(be, tx, be.from_numpy(w)) for w in (w1, w2, w3))
+        _unused = _linear(be, tx, be.from_numpy(w3))
+        heads = be.transpose(be.reshape(a, (4, 1, 4, 64)), 1, 2)          # view of a lazy product
+        gated = be.mul(a, b_)                                             # two lazy leaves in one program
+        cat = be.concat(be.neg(be.slice(c, 2, 32, 32)), be.slice(c, 2, 0, 32), 2)
+        tot = be.sum(b_)
+        return N(be, heads, gated, cat, tot, c)
+
+    def expect():
+        X = x.astype(np.float64)
+        A_, B_, C_ = (X @ w.astype(np.float64).T for w in (w1, w2, w3))
+        return [A_.reshape(4, 1, 4, 64).transpose(0, 2, 1, 3), A_ * B_, np.concatenate([-C_[..., 32:], C_[..., :32]], -1),
+                B_.sum(-1, keepdims=True), C_]
+
+    return run, expect
+
+
 # ---- decode-time attention: q.K^T -> causal soft-max -> p.V as the model graphs issue it ------------------------
 def decode_attention_ops(be, q, k_cache, v_cache, rep):
     """One decode step's attention of `LlamaModel` (catgrad-llm-models/src/models/llama.rs:285-345) on a
