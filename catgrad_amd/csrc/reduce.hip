@@ -17,6 +17,8 @@
 #include "common.hpp"
 #include "device_utils.hpp"
 
+#include <algorithm>
+
 namespace cg {
 
 namespace {
@@ -266,7 +268,66 @@ int fill_rows_args(const cg_tensor *x, RowsArgs *a) {
     return CG_OK;
 }
 
+// Few, long rows (the arg-max over a 128 K vocabulary for a handful of sequences): a row per
+// workgroup would leave most of the chip idle, so every row is cut into segments, a workgroup
+// reduces one segment to a packed accumulator, and a second small kernel merges a row's segments.
+template <int K, bool F>
+__global__ __launch_bounds__(kBlock) void reduce_segments_kernel(const RowsArgs a, long long *part, uint32_t seglen) {
+    const uint32_t row = blockIdx.y, seg = blockIdx.x;
+    const uint32_t lo = seg * seglen, hi = min(a.n, lo + seglen);
+    const uint32_t *p = reinterpret_cast<const uint32_t *>(a.x) + row_offset(row, a.nouter, a.od, a.odiv, a.os);
+    Acc<K, F> acc;
+    if (a.vec == 4) { // seglen is a multiple of 4
+        for (uint32_t i = lo / 4 + threadIdx.x; i < hi / 4; i += kBlock) {
+            const uint4 t = reinterpret_cast<const uint4 *>(p)[i];
+            acc.take(t.x, 4 * i);
+            acc.take(t.y, 4 * i + 1);
+            acc.take(t.z, 4 * i + 2);
+            acc.take(t.w, 4 * i + 3);
+        }
+        for (uint32_t i = hi / 4 * 4 + threadIdx.x; i < hi; i += kBlock) acc.take(p[i], i); // tail of the last segment
+    } else {
+        for (uint32_t i = lo + threadIdx.x; i < hi; i += kBlock) acc.take(p[(int64_t)i * a.sn], i);
+    }
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) acc.merge(acc.shfl(m));
+    __shared__ long long wpart[kBlock / 64];
+    if (threadIdx.x % 64 == 0) wpart[threadIdx.x / 64] = acc.pack();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+#pragma unroll
+        for (int w = 1; w < kBlock / 64; w++) acc.merge(Acc<K, F>::unpack(wpart[w]));
+        part[(uint64_t)row * gridDim.x + seg] = acc.pack();
+    }
+}
+
+template <int K, bool F>
+__global__ __launch_bounds__(64) void reduce_segments_final_kernel(const long long *part, uint32_t *out, uint32_t segs) {
+    const uint32_t row = blockIdx.x;
+    Acc<K, F> acc;
+    for (uint32_t s = threadIdx.x; s < segs; s += 64) acc.merge(Acc<K, F>::unpack(part[(uint64_t)row * segs + s]));
+#pragma unroll
+    for (int m = 32; m >= 1; m >>= 1) acc.merge(acc.shfl(m));
+    if (threadIdx.x == 0) out[row] = acc.result();
+}
+
 template <int K, bool F> int launch_rows(cg_backend *be, const RowsArgs &a) {
+    if (a.rows <= 64 && a.n >= 32768) {
+        uint32_t segs = std::min<uint32_t>(256, (a.n + 1023) / 1024);
+        const uint32_t seglen = ((a.n + segs - 1) / segs + 3) / 4 * 4;
+        segs = (a.n + seglen - 1) / seglen;
+        void *part = nullptr;
+        size_t cls = 0;
+        int rc = be->pool.alloc((size_t)a.rows * segs * sizeof(long long), &part, &cls);
+        if (rc) return rc;
+        hipLaunchKernelGGL((reduce_segments_kernel<K, F>), dim3(segs, a.rows), dim3(kBlock), 0, be->stream, a,
+                           static_cast<long long *>(part), seglen);
+        hipLaunchKernelGGL((reduce_segments_final_kernel<K, F>), dim3(a.rows), dim3(64), 0, be->stream,
+                           static_cast<const long long *>(part), a.out, segs);
+        be->pool.free(part, cls); // stream-ordered: later users queue behind the merge
+        hipError_t e = hipGetLastError();
+        return e == hipSuccess ? CG_OK : hip_fail(e, "segmented reduction launch");
+    }
     // lanes per row: enough that a lane sees about eight elements, within {4,16,64,256}
     uint32_t want = (a.n + 7) / 8;
     int tpr = want <= 4 ? 4 : want <= 16 ? 16 : want <= 64 ? 64 : 256;

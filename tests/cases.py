@@ -892,6 +892,30 @@ def _():
     return run, expect
 
 
+# ---- few long rows: segmented reductions --------------------------------------------------------------------
+for _shape in ((4, 128256), (3, 70001), (1, 1, 32768), (2, 40000)):
+    @case(f"long_rows_argmax_max_sum_{'x'.join(map(str, _shape))}")
+    def _(shape=_shape):
+        n = shape[-1]
+        a = rng(600 + n).integers(-50, 50, size=shape).astype(np.float32)     # integer-valued: sums are exact
+        a[..., 5] = 77.0
+        a[..., n // 2] = 77.0          # equal maxima in different segments: the last one wins
+        a[..., n - 3] = 77.0
+        a[0, ..., n - 3] = -1.0
+        u = u32(601 + n, shape, hi=1000)
+
+        def run(be):
+            t, tu = be.from_numpy(a), be.from_numpy(u)
+            return N(be, be.argmax(t), be.max(t), be.sum(t), be.argmax(tu), be.sum(tu),
+                     be.argmax(be.add(t, t)))      # a deferred program in front of the reduction
+
+        def expect():
+            return [argmax_last(a), a.max(-1, keepdims=True), a.sum(-1, keepdims=True, dtype=np.float64), argmax_last(u),
+                    u.astype(np.uint64).sum(-1, keepdims=True).astype(np.uint32), argmax_last(a + a)]
+
+        return run, expect
+
+
 # ---- decode-time linear layers: lazy, grouped by their shared left operand ---------------------------------------
 def _linear(be, x, w):
     """`nn::linear_b_param` without bias (stdlib/nn/mod.rs:182-204): x [B,S,K] times w [N,K] transposed."""
