@@ -36,7 +36,7 @@ MFMA_F32_PEAK = 157.3e12  # flop/s, MI355X dense f32 matrix
 # HBM bytes per mfma_gemm_kernel launch of this workload's prefill, from rocprofv3 FETCH_SIZE / WRITE_SIZE passes
 # scaled by a copy kernel of known size (profiles/mfma_gemm_llama1b_prefill_pmc.txt); counters cannot be read
 # from inside this process, so the figure is carried here and only reported for the profiled shape.
-MFMA_GEMM_TRAFFIC_PER_LAUNCH = 1.627e9
+MFMA_GEMM_TRAFFIC_PER_LAUNCH = 1.603e9
 
 
 def micro_bench(iters=20):

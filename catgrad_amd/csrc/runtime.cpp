@@ -1837,7 +1837,9 @@ static int reduce_entry(cg_backend *b, int kind, const char *what, cg_tensor *x,
     rc = new_dense(b, kind == kArgmax ? CG_U32 : x->dt, od, x->rank, &o);
     if (rc) return rc;
     if (numel(o) > 0) {
-        if (x->pend && x->pend->nred == 0 && (x->rc.load() == 1 || cheap(x->pend))) {
+        const bool only_a_view = x->pend && x->pend->nleaf == 1 && x->pend->ninstr == 1 &&
+                                 (x->pend->ins[0].op & ~kInstrU32) == kCopy && !x->pend->leaf[0].pw && !x->pend->leaf[0].uniform;
+        if (x->pend && !only_a_view && x->pend->nred == 0 && (x->rc.load() == 1 || cheap(x->pend))) {
             rc = resolve_lazy_leaves(b, *x->pend);
             if (!rc) rc = launch_fused_reduce(b, kind, x->dt == CG_F32, *x->pend, x->pend->ninstr, x->dims, x->rank, o);
         } else {
