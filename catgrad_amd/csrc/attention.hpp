@@ -233,26 +233,42 @@ __global__ __launch_bounds__(kBlock) void decode_attention_kernel(const AttnArgs
     }
 }
 
-// out[b][m][n] = sum_c e^(m_c - g) o_c[n] / sum_c e^(m_c - g) l_c
+// out[b][m][n] = sum_c e^(m_c - g) o_c[n] / sum_c e^(m_c - g) l_c.  A wave per (batch entry, query
+// row): lane c first holds the statistics of chunk c (so each weight e^(m_c - g) is computed once
+// and handed round by lane broadcast), then lane n sums output element n (and n + 64) over the chunks.
 __global__ __launch_bounds__(kBlock) void decode_attention_combine_kernel(const float *part_o, const float *part_ml,
                                                                           uint32_t *out, uint32_t splits, uint32_t M,
-                                                                          uint32_t hd, uint64_t total) {
-    const uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
-    if (i >= total) return;
-    const uint32_t n = (uint32_t)(i % hd);
-    const uint64_t bm = i / hd;
-    const uint32_t m = (uint32_t)(bm % M);
-    const uint64_t b = bm / M;
+                                                                          uint32_t hd, uint64_t rows) {
+    const uint32_t lane = threadIdx.x % 64;
+    const uint64_t r = (uint64_t)blockIdx.x * (kBlock / 64) + threadIdx.x / 64;
+    if (r >= rows) return;
+    const uint32_t m = (uint32_t)(r % M);
+    const uint64_t b = r / M;
+    const float *ml = part_ml + (b * splits * M + m) * 2; // chunk c at + c * M * 2
+    const float *po = part_o + (b * splits * M + m) * (uint64_t)hd; // chunk c at + c * M * hd
     float gmax = kF32Min;
+    for (uint32_t c = lane; c < splits; c += 64) gmax = fmaxf(gmax, ml[(uint64_t)c * M * 2]);
+#pragma unroll
+    for (int sft = 32; sft >= 1; sft >>= 1) gmax = fmaxf(gmax, __shfl_xor(gmax, sft));
+    float num0 = 0.0f, num1 = 0.0f, den = 0.0f;
+    for (uint32_t c0 = 0; c0 < splits; c0 += 64) {
+        const uint32_t c = c0 + lane;
+        float w = 0.0f;
+        if (c < splits) {
+            w = expf(ml[(uint64_t)c * M * 2] - gmax);
+            den = fmaf(w, ml[(uint64_t)c * M * 2 + 1], den);
+        }
+        const uint32_t cnt = min(64u, splits - c0);
 #pragma unroll 8
-    for (uint32_t c = 0; c < splits; c++) gmax = fmaxf(gmax, part_ml[((b * splits + c) * M + m) * 2]);
-    float num = 0.0f, den = 0.0f;
-#pragma unroll 8
-    for (uint32_t c = 0; c < splits; c++) {
-        const float *ml = part_ml + ((b * splits + c) * M + m) * 2;
-        const float w = expf(ml[0] - gmax);
-        num = fmaf(w, part_o[((b * splits + c) * M + m) * (uint64_t)hd + n], num);
-        den = fmaf(w, ml[1], den);
+        for (uint32_t k = 0; k < cnt; k++) {
+            const float wk = __shfl(w, (int)k);
+            const float *o = po + (uint64_t)(c0 + k) * M * hd;
+            num0 = fmaf(wk, o[lane], num0);
+            if (lane + 64 < hd) num1 = fmaf(wk, o[lane + 64], num1);
+        }
     }
-    out[i] = asu(num / den);
+#pragma unroll
+    for (int sft = 32; sft >= 1; sft >>= 1) den += __shfl_xor(den, sft);
+    if (lane < hd) out[r * hd + lane] = asu(num0 / den);
+    if (lane + 64 < hd) out[r * hd + lane + 64] = asu(num1 / den);
 }

@@ -675,10 +675,10 @@ int launch_decode_attention(cg_backend *be, const Pending &p, const int64_t *pdi
             hipLaunchKernelGGL((decode_attention_kernel<P, 16>), grid, dim3(kBlock), 0, be->stream, g, a);
         else
             hipLaunchKernelGGL((decode_attention_kernel<P, 32>), grid, dim3(kBlock), 0, be->stream, g, a);
-        const uint64_t total = (uint64_t)f1.batch * g.M * hd;
-        hipLaunchKernelGGL(decode_attention_combine_kernel, dim3((uint32_t)((total + kBlock - 1) / kBlock)), dim3(kBlock), 0,
+        const uint64_t rows = (uint64_t)f1.batch * g.M, waves = kBlock / 64;
+        hipLaunchKernelGGL(decode_attention_combine_kernel, dim3((uint32_t)((rows + waves - 1) / waves)), dim3(kBlock), 0,
                            be->stream, g.part_o, g.part_ml, static_cast<uint32_t *>(out->buf->ptr), g.splits, g.M,
-                           (uint32_t)hd, total);
+                           (uint32_t)hd, rows);
     }
     be->pool.free(po, co); // stream-ordered: later users queue behind the combine
     be->pool.free(pml, cml);

@@ -398,17 +398,24 @@ template <int MM> __global__ __launch_bounds__(kThreads) void skinny_kt_wide_gro
 // workgroup split each 2048-wide chunk of k, keep their share of the chunk's activations
 // in registers (8 x 16 bytes per lane and row group) and reuse it for CG groups of four
 // columns, so the activation rows are fetched once per 4 * CG columns.
-template <int MM, int CG>
-__device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const uint32_t block_x, const uint32_t block_y) {
+// GATED (CG = 2): the two column groups are the same four columns of two weight matrices, a.B and
+// `second` (same shape and strides), and the block writes g * (1 / (one + exp(-g))) * u for
+// g = x.B^T, u = x.second^T: the SiLU-gated pair of an MLP block without writing g and u.
+template <int MM, int CG, bool GATED = false>
+__device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const uint32_t block_x, const uint32_t block_y,
+                                                         const uint32_t *second = nullptr, const uint32_t one = 0) {
+    static_assert(!GATED || CG == 2, "a gated pair is two column groups");
     constexpr int G = MM / 4;
     const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x % 64;
     const uint32_t j = lane % 4, b = lane / 4;
-    const uint32_t n0 = block_x * (4 * CG);
+    const uint32_t n0 = block_x * (GATED ? 4 : 4 * CG);
     int64_t oa, ob;
     batch_offsets(a, block_y, oa, ob);
     const uint32_t *wrow[CG];
 #pragma unroll
-    for (int c = 0; c < CG; c++) wrow[c] = a.B + ob + (int64_t)min(n0 + 4 * c + j, a.N - 1) * a.b_sn;
+    for (int c = 0; c < CG; c++)
+        wrow[c] = GATED ? (c == 0 ? a.B : second) + ob + (int64_t)min(n0 + j, a.N - 1) * a.b_sn
+                        : a.B + ob + (int64_t)min(n0 + 4 * c + j, a.N - 1) * a.b_sn;
     const uint32_t *xrow[G];
 #pragma unroll
     for (int g = 0; g < G; g++) xrow[g] = a.A + oa + (int64_t)min((uint32_t)(4 * g) + j, a.M - 1) * a.a_sm;
@@ -462,7 +469,18 @@ __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const 
                 if (lane < 4) part[wave][(c * MM + 4 * g + i) * 4 + j] = v;
             }
     __syncthreads();
-    if (threadIdx.x < CG * MM * 4) {
+    if constexpr (GATED) {
+        if (threadIdx.x < MM * 4) {
+            const uint32_t t = threadIdx.x, u_at = MM * 4 + t, m = t / 4, col = n0 + t % 4;
+            const uint32_t gv = asu((part[0][t] + part[1][t]) + (part[2][t] + part[3][t]));
+            const uint32_t uv = asu((part[0][u_at] + part[1][u_at]) + (part[2][u_at] + part[3][u_at]));
+            // the ops of the deferred program, in its order
+            const uint32_t e = apply<kExp, true>(apply<kNeg, true>(gv, 0, 0, nullptr), 0, 0, nullptr);
+            const uint32_t sg = apply<kDiv, true>(one, apply<kAdd, true>(one, e, 0, nullptr), 0, nullptr);
+            const uint32_t r = apply<kMul, true>(apply<kMul, true>(gv, sg, 0, nullptr), uv, 0, nullptr);
+            if (col < a.N && m < a.M) a.C[((uint64_t)block_y * a.M + m) * a.N + col] = r;
+        }
+    } else if (threadIdx.x < CG * MM * 4) {
         const uint32_t c = threadIdx.x / (MM * 4), m = threadIdx.x / 4 % MM, col = n0 + 4 * c + threadIdx.x % 4;
         const float v = (part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]);
         if (col < a.N && m < a.M) a.C[((uint64_t)block_y * a.M + m) * a.N + col] = asu(v);
@@ -471,6 +489,10 @@ __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const 
 
 template <int MM, int CG> __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_kernel(const MmArgs a) {
     skinny_kt_mfma_xreg_body<MM, CG>(a, blockIdx.x, blockIdx.y);
+}
+template <int MM>
+__global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_gated_kernel(const MmArgs a, const uint32_t *second, uint32_t one) {
+    skinny_kt_mfma_xreg_body<MM, 2, true>(a, blockIdx.x, blockIdx.y, second, one);
 }
 template <int MM, int CG> __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_group_kernel(const MmGroup g) {
     uint32_t bx;
@@ -751,6 +773,27 @@ int launch_matmul_group(cg_backend *be, const cg_tensor *x, const cg_tensor *con
         hipLaunchKernelGGL((skinny_kt_wide_group_kernel<8>), dim3(blocks), dim3(kThreads), 0, be->stream, g);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? CG_OK : hip_fail(e, "grouped matmul launch");
+}
+
+// out = g * (1 / (one + exp(-g))) * u with g = x.yg, u = x.yu: two decode-time linear layers and
+// the program between them and the next product in one launch.  Declines unless the 4x4x1
+// kernel takes the shapes.
+int launch_matmul_gated(cg_backend *be, const cg_tensor *x, const cg_tensor *yg, const cg_tensor *yu, uint32_t one,
+                        cg_tensor *out) {
+    if (x->dt != CG_F32) return kDeclined;
+    MmArgs ag, au;
+    MmFold fg, fu;
+    int rc = make_mm_args(x, yg, out->buf->ptr, &ag, &fg);
+    if (!rc) rc = make_mm_args(x, yu, out->buf->ptr, &au, &fu);
+    if (rc) return rc;
+    const bool vec = ag.a_vec && ag.b_vec && au.b_vec && ag.a_sk == 1 && ag.K % 4 == 0;
+    if (fg.batch != 1 || fu.batch != 1 || ag.M > 4 || ag.b_sk != 1 || au.b_sk != 1 || !vec || ag.K <= 256 || ag.N < 4096 ||
+        au.N != ag.N || au.K != ag.K || au.M != ag.M || au.b_sn != ag.b_sn)
+        return kDeclined;
+    ProfScope prof(be, CG_K_GEMM_SKINNY, distinct_bytes(x) + distinct_bytes(yg) + distinct_bytes(yu) + distinct_bytes(out));
+    hipLaunchKernelGGL((skinny_kt_mfma_xreg_gated_kernel<4>), dim3((ag.N + 3) / 4), dim3(kThreads), 0, be->stream, ag, au.B, one);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CG_OK : hip_fail(e, "gated matmul launch");
 }
 
 int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_tensor *out) {

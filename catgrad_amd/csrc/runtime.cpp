@@ -618,7 +618,43 @@ static int resolve_lazy_leaves(cg_backend *be, const Pending &cp) {
     return CG_OK;
 }
 
+// g * (1 / (c + exp(-g))) * u where g and u are open products of the same left operand that nobody
+// else holds (gate and up projection of an MLP block): one launch that never writes g and u.
+static int try_gated_pair(cg_backend *be, const cg_tensor *dst, const Pending &p) {
+    static const uint8_t code[6][3] = {{kNeg, 0, 0}, {kExp, 8, 8}, {kAdd, 1, 9}, {kDiv, 1, 10}, {kMul, 0, 11}, {kMul, 12, 2}};
+    if (p.nleaf != 3 || p.ninstr != 6 || p.nred != 0 || !is_contiguous(dst) || dst->dt != CG_F32) return kDeclined;
+    for (int i = 0; i < 6; i++) {
+        const Instr &in = p.ins[i];
+        if (in.op != code[i][0] || in.a != code[i][1] || (i >= 2 && in.b != code[i][2])) return kDeclined;
+    }
+    const LeafView &lg = p.leaf[0], &lc = p.leaf[1], &lu = p.leaf[2];
+    if (!lc.uniform || lg.uniform || lu.uniform || lg.pw || lu.pw || !lg.lazy || !lu.lazy || lg.lazy == lu.lazy) return kDeclined;
+    LazyMm *mg = lg.lazy, *mu = lu.lazy;
+    if (mg->result || mu->result || !mg->groupable || !mu->groupable || mg->x != mu->x || mg->rc.load() != 1 ||
+        mu->rc.load() != 1 || mg->rank != dst->rank || mu->rank != dst->rank)
+        return kDeclined;
+    // both leaves are the whole products, read in place
+    int64_t st = 1;
+    for (int d = dst->rank - 1; d >= 0; d--) {
+        if (mg->dims[d] != dst->dims[d] || mu->dims[d] != dst->dims[d]) return kDeclined;
+        if (dst->dims[d] != 1 && (lg.strides[d] != st || lu.strides[d] != st)) return kDeclined;
+        st *= dst->dims[d];
+    }
+    if (lg.offset != 0 || lu.offset != 0) return kDeclined;
+    int rc = launch_matmul_gated(be, mg->x, mg->y, mu->y, lc.ubits, const_cast<cg_tensor *>(dst));
+    if (rc == CG_OK) {
+        lazy_mm_close(mg);
+        lazy_mm_close(mu);
+        be->programs_compiled++;
+    }
+    return rc;
+}
+
 static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p) {
+    if (be->aot) {
+        int grc = try_gated_pair(be, dst, p);
+        if (grc != kDeclined) return grc;
+    }
     {
         int lrc = resolve_lazy_leaves(be, p);
         if (lrc) return lrc;

@@ -968,6 +968,35 @@ def _():
     return run, expect
 
 
+# ---- SiLU-gated pair of decode-time linear layers (gate / up of an MLP block) ---------------------------------------
+for _B, _K, _N in ((4, 512, 4096), (1, 2048, 8192), (3, 388, 4100), (8, 512, 4096), (4, 512, 512)):
+    @case(f"linear_gated_B{_B}_K{_K}_N{_N}", "red")
+    def _(B=_B, K=_K, Nn=_N):
+        """`silu(x.Wg) * (x.Wu)` as the MLP of the decoder graphs issues it (llama.rs:262-283 with
+        nn::silu = x * sigmoid(x), stdlib/nn/mod.rs:130-166).  Rows of one sign: no cancellation inside a
+        product, so 1e-3 of the value applies; gate rows alternate in sign to cover both sigmoid tails."""
+        x = np.abs(f32(540 + Nn, (B, 1, K)))
+        wg = np.abs(f32(541 + Nn, (Nn, K))) * np.float32(8.0 / K)
+        wg[::2] *= -1
+        wu = np.abs(f32(542 + Nn, (Nn, K))) * np.float32(8.0 / K)
+
+        def run(be):
+            tx = be.from_numpy(x)
+            g, u = _linear(be, tx, be.from_numpy(wg)), _linear(be, tx, be.from_numpy(wu))
+            del tx
+            sh = (B, 1, Nn)
+            e = be.exp(be.neg(g).move())
+            sg = be.div(_const(be, 1.0, sh).move(), be.add(_const(be, 1.0, sh).move(), e.move()).move())
+            return N(be, be.mul(be.mul(g.move(), sg.move()).move(), u.move()))
+
+        def expect():
+            X = x.astype(np.float64)
+            G, U = X @ wg.astype(np.float64).T, X @ wu.astype(np.float64).T
+            return [G / (1.0 + np.exp(-G)) * U]
+
+        return run, expect
+
+
 # ---- decode-time attention: q.K^T -> causal soft-max -> p.V as the model graphs issue it ------------------------
 def decode_attention_ops(be, q, k_cache, v_cache, rep):
     """One decode step's attention of `LlamaModel` (catgrad-llm-models/src/models/llama.rs:285-345) on a

@@ -136,6 +136,28 @@ def test_decode_attention_runs_as_one_fused_pass(hip):
     np.testing.assert_allclose(got, _np_decode_attention(q, k, v, 4), rtol=1e-4, atol=1e-5)
 
 
+def test_gated_linear_pair_is_one_launch(hip):
+    """gate and up projection of a decode step plus the SiLU program between them and the next product:
+    one skinny-product launch and no element-wise launch; a pair the kernel does not take (8 rows) runs as
+    a grouped product plus the compiled program and gives the same kind of result."""
+    from catgrad_amd import _abi as A
+    from cases import by_name
+
+    for name, launches in (("linear_gated_B4_K512_N4096", (1, 0)), ("linear_gated_B8_K512_N4096", (1, 1))):
+        c = by_name(name)
+        hip.sync()
+        for cls in (A.K_GEMM_SKINNY, A.K_ELEMENTWISE):
+            hip.profile_enable(cls, 1)
+            hip.profile_read(cls, True)
+        got = c.run(hip)
+        counts = tuple(hip.profile_read(cls, True)[0] for cls in (A.K_GEMM_SKINNY, A.K_ELEMENTWISE))
+        for cls in (A.K_GEMM_SKINNY, A.K_ELEMENTWISE):
+            hip.profile_enable(cls, 0)
+        assert counts == launches, (name, counts)
+        for g, e in zip(got, c.expect()):
+            np.testing.assert_allclose(g, e, rtol=1e-3)
+
+
 def test_format_tensor(hip):
     s = hip.format_tensor(hip.from_numpy(np.array([[1.5, 2.0]], np.float32)))
     assert "f32[1,2]" in s and "1.5" in s
