@@ -246,25 +246,43 @@ __global__ __launch_bounds__(kBlock) void decode_attention_combine_kernel(const 
     const uint64_t b = r / M;
     const float *ml = part_ml + (b * splits * M + m) * 2; // chunk c at + c * M * 2
     const float *po = part_o + (b * splits * M + m) * (uint64_t)hd; // chunk c at + c * M * hd
+    constexpr uint32_t kGroup = 32; // chunks per trip to memory
+    const bool wide = lane + 64 < hd;
     float gmax = kF32Min;
-    for (uint32_t c = lane; c < splits; c += 64) gmax = fmaxf(gmax, ml[(uint64_t)c * M * 2]);
-#pragma unroll
-    for (int sft = 32; sft >= 1; sft >>= 1) gmax = fmaxf(gmax, __shfl_xor(gmax, sft));
     float num0 = 0.0f, num1 = 0.0f, den = 0.0f;
-    for (uint32_t c0 = 0; c0 < splits; c0 += 64) {
-        const uint32_t c = c0 + lane;
-        float w = 0.0f;
-        if (c < splits) {
-            w = expf(ml[(uint64_t)c * M * 2] - gmax);
-            den = fmaf(w, ml[(uint64_t)c * M * 2 + 1], den);
+    for (uint32_t c0 = 0; c0 < splits; c0 += kGroup) {
+        // every load of the group is asked for before anything is used
+        float v0[kGroup], v1[kGroup];
+#pragma unroll
+        for (uint32_t k = 0; k < kGroup; k++) {
+            v0[k] = 0.0f;
+            v1[k] = 0.0f;
+            if (c0 + k < splits) {
+                const float *o = po + (uint64_t)(c0 + k) * M * hd;
+                if (lane < hd) v0[k] = o[lane];
+                if (wide) v1[k] = o[lane + 64];
+            }
         }
-        const uint32_t cnt = min(64u, splits - c0);
-#pragma unroll 8
-        for (uint32_t k = 0; k < cnt; k++) {
+        const uint32_t c = c0 + lane;
+        const bool mine = lane < kGroup && c < splits;
+        const float cm = mine ? ml[(uint64_t)c * M * 2] : kF32Min, cl = mine ? ml[(uint64_t)c * M * 2 + 1] : 0.0f;
+        float m2 = fmaxf(gmax, cm);
+#pragma unroll
+        for (int sft = 16; sft >= 1; sft >>= 1) m2 = fmaxf(m2, __shfl_xor(m2, sft));
+        m2 = __shfl(m2, 0);
+        // what was summed so far is relative to the old maximum
+        const float rescale = expf(gmax - m2);
+        num0 *= rescale;
+        num1 *= rescale;
+        den *= rescale;
+        gmax = m2;
+        const float w = mine ? expf(cm - gmax) : 0.0f;
+        den = fmaf(w, cl, den);
+#pragma unroll
+        for (uint32_t k = 0; k < kGroup; k++) {
             const float wk = __shfl(w, (int)k);
-            const float *o = po + (uint64_t)(c0 + k) * M * hd;
-            num0 = fmaf(wk, o[lane], num0);
-            if (lane + 64 < hd) num1 = fmaf(wk, o[lane + 64], num1);
+            num0 = fmaf(wk, v0[k], num0);
+            num1 = fmaf(wk, v1[k], num1);
         }
     }
 #pragma unroll

@@ -367,6 +367,8 @@ int fold_matmul(const cg_tensor *x, const cg_tensor *y, MmFold *f);
 // below) when the shapes do not allow it.
 int launch_matmul_gated(cg_backend *be, const cg_tensor *x, const cg_tensor *yg, const cg_tensor *yu, uint32_t one,
                         cg_tensor *out);
+int launch_matmul_residual(cg_backend *be, const cg_tensor *x, const cg_tensor *y, const uint32_t *const *terms, int slot,
+                           int order, cg_tensor *out);
 int launch_matmul_group(cg_backend *be, const cg_tensor *x, const cg_tensor *const *ys, cg_tensor *const *outs, int n);
 
 // Decode-time attention in one pass: out = softmax-program(q . kT) . v, where `p` is the deferred

@@ -294,8 +294,18 @@ template <int MM> __global__ __launch_bounds__(kThreads) void skinny_kt_kernel(c
 // 16-byte loads (COLS weight loads + M activation loads in flight per lane per trip; the
 // activation rows stay in L1/L2).  SPLIT: the four waves of the block share the columns
 // and split K, for shapes with too few columns to fill the chip.
-template <int MM, int COLS, bool SPLIT>
-__device__ __forceinline__ void skinny_kt_wide_body(const MmArgs &a, const uint32_t block_x, const uint32_t block_y) {
+// A sum of four terms one of which is the product: out = (t0 + (t1 + t2)) + t3 (order 0) or
+// t0 + ((t1 + t2) + t3) (order 1), term[slot] being x.B^T and the others dense tensors of the
+// output's shape.  The residual adds of a decoder layer run in the store of the o / down projection.
+struct MmResidual {
+    const uint32_t *term[4];
+    uint32_t slot, order;
+};
+
+template <int MM, int COLS, bool SPLIT, bool RESIDUAL = false>
+__device__ __forceinline__ void skinny_kt_wide_body(const MmArgs &a, const uint32_t block_x, const uint32_t block_y,
+                                                    const MmResidual *res = nullptr) {
+    static_assert(!RESIDUAL || (COLS == 1 && !SPLIT), "the residual store is written for one column per wave");
     const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x % 64;
     const uint32_t group = SPLIT ? block_x : block_x * 4 + wave;
     const uint32_t n0 = group * COLS;
@@ -304,6 +314,18 @@ __device__ __forceinline__ void skinny_kt_wide_body(const MmArgs &a, const uint3
     batch_offsets(a, block_y, oa, ob);
     const uint32_t *A = a.A + oa;
     const uint32_t *B = a.B + ob;
+    uint32_t term[RESIDUAL ? MM : 1][4] = {};
+    if constexpr (RESIDUAL) {
+        // asked for before the walk along K, used after it
+        if (live && lane == 0) {
+#pragma unroll
+            for (int m = 0; m < MM; m++)
+#pragma unroll
+                for (int t = 0; t < 4; t++)
+                    if ((uint32_t)m < a.M && (uint32_t)t != res->slot)
+                        term[m][t] = res->term[t][((uint64_t)block_y * a.M + m) * a.N + n0];
+        }
+    }
     float acc[COLS][MM];
 #pragma unroll
     for (int c = 0; c < COLS; c++)
@@ -361,13 +383,28 @@ __device__ __forceinline__ void skinny_kt_wide_body(const MmArgs &a, const uint3
         for (int c = 0; c < COLS; c++)
 #pragma unroll
             for (int m = 0; m < MM; m++)
-                if (n0 + c < a.N && (uint32_t)m < a.M) a.C[((uint64_t)block_y * a.M + m) * a.N + n0 + c] = asu(acc[c][m]);
+                if (n0 + c < a.N && (uint32_t)m < a.M) {
+                    uint32_t v = asu(acc[c][m]);
+                    if constexpr (RESIDUAL) {
+                        uint32_t t[4];
+#pragma unroll
+                        for (int i = 0; i < 4; i++) t[i] = (uint32_t)i == res->slot ? v : term[m][i];
+                        const uint32_t inner = apply<kAdd, true>(t[1], t[2], 0, nullptr);
+                        v = res->order == 0 ? apply<kAdd, true>(apply<kAdd, true>(t[0], inner, 0, nullptr), t[3], 0, nullptr)
+                                            : apply<kAdd, true>(t[0], apply<kAdd, true>(inner, t[3], 0, nullptr), 0, nullptr);
+                    }
+                    a.C[((uint64_t)block_y * a.M + m) * a.N + n0 + c] = v;
+                }
     }
 }
 
 template <int MM, int COLS, bool SPLIT>
 __global__ __launch_bounds__(kThreads) void skinny_kt_wide_kernel(const MmArgs a) {
     skinny_kt_wide_body<MM, COLS, SPLIT>(a, blockIdx.x, blockIdx.y);
+}
+
+template <int MM> __global__ __launch_bounds__(kThreads) void skinny_kt_wide_residual_kernel(const MmArgs a, const MmResidual r) {
+    skinny_kt_wide_body<MM, 1, false, true>(a, blockIdx.x, blockIdx.y, &r);
 }
 
 // Several products that share their left operand (the q / k / v projections of a decode step,
@@ -794,6 +831,34 @@ int launch_matmul_gated(cg_backend *be, const cg_tensor *x, const cg_tensor *yg,
     hipLaunchKernelGGL((skinny_kt_mfma_xreg_gated_kernel<4>), dim3((ag.N + 3) / 4), dim3(kThreads), 0, be->stream, ag, au.B, one);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? CG_OK : hip_fail(e, "gated matmul launch");
+}
+
+// out = a sum of four terms, term[slot] = x.y, the other three dense tensors of out's shape
+// (device pointers); `order` as in MmResidual.  Declines unless the one-column-per-wave kernel
+// is what the product would run on anyway.
+int launch_matmul_residual(cg_backend *be, const cg_tensor *x, const cg_tensor *y, const uint32_t *const *terms, int slot,
+                           int order, cg_tensor *out) {
+    if (x->dt != CG_F32) return kDeclined;
+    MmArgs a;
+    MmFold f;
+    int rc = make_mm_args(x, y, out->buf->ptr, &a, &f);
+    if (rc) return rc;
+    const bool vec = a.a_vec && a.b_vec && a.a_sk == 1 && a.K % 4 == 0;
+    if (f.batch != 1 || a.M > 8 || a.b_sk != 1 || !vec || a.K <= 256 || a.N < 2048 || a.N >= 8192) return kDeclined;
+    MmResidual r;
+    for (int t = 0; t < 4; t++) r.term[t] = t == slot ? nullptr : terms[t];
+    r.slot = (uint32_t)slot;
+    r.order = (uint32_t)order;
+    ProfScope prof(be, CG_K_GEMM_SKINNY, distinct_bytes(x) + distinct_bytes(y) + 4.0 * distinct_bytes(out));
+    dim3 grid((uint32_t)((a.N + 3) / 4));
+    if (a.M <= 1)
+        hipLaunchKernelGGL((skinny_kt_wide_residual_kernel<1>), grid, dim3(kThreads), 0, be->stream, a, r);
+    else if (a.M <= 4)
+        hipLaunchKernelGGL((skinny_kt_wide_residual_kernel<4>), grid, dim3(kThreads), 0, be->stream, a, r);
+    else
+        hipLaunchKernelGGL((skinny_kt_wide_residual_kernel<8>), grid, dim3(kThreads), 0, be->stream, a, r);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CG_OK : hip_fail(e, "matmul with residual launch");
 }
 
 int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_tensor *out) {

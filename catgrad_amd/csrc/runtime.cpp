@@ -650,9 +650,56 @@ static int try_gated_pair(cg_backend *be, const cg_tensor *dst, const Pending &p
     return rc;
 }
 
+// A sum of four dense terms, one of them a product nobody has needed yet (the residual stream after the
+// o or down projection): the adds run in the product's store.
+static int try_residual_store(cg_backend *be, const cg_tensor *dst, const Pending &p) {
+    static const uint8_t orders[2][3][2] = {{{1, 2}, {0, 8}, {9, 3}}, {{1, 2}, {8, 3}, {0, 9}}};
+    if (p.nleaf != 4 || p.ninstr != 3 || p.nred != 0 || !is_contiguous(dst) || dst->dt != CG_F32) return kDeclined;
+    int order = -1;
+    for (int o = 0; o < 2 && order < 0; o++) {
+        bool same = true;
+        for (int i = 0; i < 3; i++) same = same && p.ins[i].op == kAdd && p.ins[i].a == orders[o][i][0] && p.ins[i].b == orders[o][i][1];
+        if (same) order = o;
+    }
+    if (order < 0) return kDeclined;
+    int slot = -1;
+    const uint32_t *terms[4] = {nullptr, nullptr, nullptr, nullptr};
+    for (int l = 0; l < 4; l++) {
+        const LeafView &lv = p.leaf[l];
+        if (lv.uniform || lv.pw || lv.offset % 4 != 0) return kDeclined;
+        int64_t st = 1;
+        for (int d = dst->rank - 1; d >= 0; d--) { // the term is read in place, element for element
+            if (dst->dims[d] != 1 && lv.strides[d] != st) return kDeclined;
+            st *= dst->dims[d];
+        }
+        if (lv.lazy && !lv.lazy->result) {
+            LazyMm *m = lv.lazy;
+            if (slot >= 0 || !m->groupable || m->rc.load() != 1 || lv.offset != 0 || m->rank != dst->rank) return kDeclined;
+            for (int d = 0; d < dst->rank; d++)
+                if (m->dims[d] != dst->dims[d]) return kDeclined;
+            for (LazyMm *o : be->lazy_open)
+                if (o != m && !o->result && o->x == m->x) return kDeclined; // it belongs to a group
+            slot = l;
+        } else {
+            const Buffer *b = lv.lazy ? lv.lazy->result : lv.buf;
+            if (!b) return kDeclined;
+            terms[l] = static_cast<const uint32_t *>(b->ptr) + lv.offset;
+        }
+    }
+    if (slot < 0) return kDeclined;
+    LazyMm *m = p.leaf[slot].lazy;
+    int rc = launch_matmul_residual(be, m->x, m->y, terms, slot, order, const_cast<cg_tensor *>(dst));
+    if (rc == CG_OK) {
+        lazy_mm_close(m);
+        be->programs_compiled++;
+    }
+    return rc;
+}
+
 static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p) {
     if (be->aot) {
         int grc = try_gated_pair(be, dst, p);
+        if (grc == kDeclined) grc = try_residual_store(be, dst, p);
         if (grc != kDeclined) return grc;
     }
     {

@@ -997,6 +997,39 @@ for _B, _K, _N in ((4, 512, 4096), (1, 2048, 8192), (3, 388, 4100), (8, 512, 409
         return run, expect
 
 
+# ---- residual adds around a decode-time linear layer (the o / down projection of a decoder layer) -------------------
+for _B, _K, _N in ((4, 512, 2048), (8, 260, 2052), (1, 1024, 4096), (4, 512, 512)):
+    @case(f"linear_residual_B{_B}_K{_K}_N{_N}", "red")
+    def _(B=_B, K=_K, Nn=_N):
+        """Sums of three dense terms and a lazy product in the two association orders and every operand
+        position the layer loop of the decoder graphs produces (llama.rs:347-365: x + attn, then + mlp)."""
+        x = np.abs(f32(560 + Nn, (B, 1, K)))
+        w = np.abs(f32(561 + Nn, (Nn, K)))
+        ts = [np.abs(f32(562 + Nn + i, (B, 1, Nn))) for i in range(3)]
+
+        def run(be):
+            outs = []
+            for order in (0, 1):
+                for slot in range(4):
+                    tx = be.from_numpy(x)
+                    t = [be.from_numpy(a) for a in ts]
+                    t.insert(slot, _linear(be, tx, be.from_numpy(w)))
+                    del tx
+                    inner = be.add(t[1].move(), t[2].move())
+                    if order == 0:
+                        r = be.add(be.add(t[0].move(), inner.move()).move(), t[3].move())
+                    else:
+                        r = be.add(t[0].move(), be.add(inner.move(), t[3].move()).move())
+                    outs.append(r)
+            return N(be, *outs)
+
+        def expect():
+            P = x.astype(np.float64) @ w.astype(np.float64).T
+            return [P + sum(a.astype(np.float64) for a in ts)] * 8
+
+        return run, expect
+
+
 # ---- decode-time attention: q.K^T -> causal soft-max -> p.V as the model graphs issue it ------------------------
 def decode_attention_ops(be, q, k_cache, v_cache, rep):
     """One decode step's attention of `LlamaModel` (catgrad-llm-models/src/models/llama.rs:285-345) on a

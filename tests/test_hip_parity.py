@@ -136,14 +136,16 @@ def test_decode_attention_runs_as_one_fused_pass(hip):
     np.testing.assert_allclose(got, _np_decode_attention(q, k, v, 4), rtol=1e-4, atol=1e-5)
 
 
-def test_gated_linear_pair_is_one_launch(hip):
+def test_programs_absorbed_by_decode_time_products(hip):
     """gate and up projection of a decode step plus the SiLU program between them and the next product:
     one skinny-product launch and no element-wise launch; a pair the kernel does not take (8 rows) runs as
-    a grouped product plus the compiled program and gives the same kind of result."""
+    a grouped product plus the compiled program and gives the same kind of result.  Likewise the residual
+    adds around a product (eight sums per case): absorbed at 2048 columns, separate launches at 512."""
     from catgrad_amd import _abi as A
     from cases import by_name
 
-    for name, launches in (("linear_gated_B4_K512_N4096", (1, 0)), ("linear_gated_B8_K512_N4096", (1, 1))):
+    for name, launches in (("linear_gated_B4_K512_N4096", (1, 0)), ("linear_gated_B8_K512_N4096", (1, 1)),
+                           ("linear_residual_B4_K512_N2048", (8, 0)), ("linear_residual_B4_K512_N512", (8, 8))):
         c = by_name(name)
         hip.sync()
         for cls in (A.K_GEMM_SKINNY, A.K_ELEMENTWISE):
