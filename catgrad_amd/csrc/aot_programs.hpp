@@ -33,6 +33,8 @@
 // cos * x + sin * rotate_half(x), rotate_half(x) = concat(-x2, x1) read in place as the
 // piecewise leaf 3                                        (rotary embedding)
 CG_PROGRAM(MapRope, 4, 0x0, 3, {18, 0, 1, 0}, {18, 2, 3, 2}, {16, 8, 9, 8})
+// a strided copy (only used inside grouped launches; alone it is the single-op copy kernel)
+CG_PROGRAM(MapCopy, 1, 0x0, -1, {42, 0, 0, 0})
 // g * (1 / (1 + exp(-g))) * u                            (SiLU gate times up projection)
 CG_PROGRAM(MapSiluMul, 3, 0x2, -1, {0, 0, 0, 0}, {3, 8, 8, 8}, {16, 1, 9, 1}, {19, 1, 10, 1}, {18, 0, 11, 0}, {18, 12, 2, 12})
 // residual stream after three adds, in the two operand orders the layer loop produces
@@ -137,8 +139,8 @@ __device__ __forceinline__ void aot_load_all(const FusedArgs &a, const int64_t (
 }
 
 // ---- element-wise kernel: the geometry of fused_kernel, the program compiled in ----------------------
-template <class P, int VEC> __global__ __launch_bounds__(kBlock) void aot_map_kernel(const FusedArgs a) {
-    const uint64_t v64 = (uint64_t)blockIdx.x * kBlock + threadIdx.x;
+template <class P, int VEC> __device__ __forceinline__ void aot_map_body(const FusedArgs &a, const uint32_t block) {
+    const uint64_t v64 = (uint64_t)block * kBlock + threadIdx.x;
     if (v64 >= a.g.total) return;
     const uint32_t v = (uint32_t)v64;
     uint32_t row = fastdiv(v, a.g.ipr_div);
@@ -169,6 +171,34 @@ template <class P, int VEC> __global__ __launch_bounds__(kBlock) void aot_map_ke
     const uint32_t rs[kMaxRowReduce] = {0, 0, 0};
     aot_run<P, VEC>(s, rs, a.fault, std::make_integer_sequence<int, P::ninstr>{});
     store_words<VEC>(a.out, oo, s.v[kMaxLeaves + P::ninstr - 1]);
+}
+template <class P, int VEC> __global__ __launch_bounds__(kBlock) void aot_map_kernel(const FusedArgs a) {
+    aot_map_body<P, VEC>(a, blockIdx.x);
+}
+
+// Up to three small element-wise launches in one: the writes of a decode step that nobody reads
+// before the attention does (rotary embedding of k into the cache, v into the cache, rotary
+// embedding of q).  Each workgroup finds its entry from the table of first workgroups.
+constexpr int kMaxMapGroup = 3;
+struct FusedGroup {
+    FusedArgs p[kMaxMapGroup];
+    uint32_t first[kMaxMapGroup + 1]; // first workgroup of each entry; first[n] = grid size
+    uint32_t n;
+    uint32_t prog[kMaxMapGroup]; // 0: MapRope, 1: MapCopy
+};
+static_assert(sizeof(FusedGroup) <= 4096, "kernel arguments are limited to 4 KiB");
+__global__ __launch_bounds__(kBlock) void aot_map_group_kernel(const FusedGroup g) {
+    uint32_t e = 0;
+    while (e + 1 < g.n && blockIdx.x >= g.first[e + 1]) e++;
+    const uint32_t block = blockIdx.x - g.first[e];
+    const FusedArgs &a = g.p[e];
+    if (g.prog[e] == 0) {
+        if (a.g.vec == 4) aot_map_body<MapRope, 4>(a, block);
+        else aot_map_body<MapRope, 1>(a, block);
+    } else {
+        if (a.g.vec == 4) aot_map_body<MapCopy, 4>(a, block);
+        else aot_map_body<MapCopy, 1>(a, block);
+    }
 }
 
 // ---- row kernel: the phases of fused_rows_kernel, unrolled at compile time -----------------------------

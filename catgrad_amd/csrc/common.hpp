@@ -64,6 +64,7 @@ struct ProfPending {
 
 namespace cg {
 struct LazyMm;
+struct DeferredWrite;
 }
 
 struct cg_backend {
@@ -81,6 +82,7 @@ struct cg_backend {
     unsigned stage_next = 0;
     std::string name;
     std::vector<cg::LazyMm *> lazy_open; // groupable lazy products not yet computed (not retained)
+    std::vector<cg::DeferredWrite> deferred; // writes waiting to share a launch (see flush_deferred)
     bool fuse = true; // defer element-wise ops and fuse them (CG_FUSE=0 switches it off)
     bool aot = true;  // use the compiled kernels for listed programs (CG_AOT=0: interpreter only)
     uint64_t programs_compiled = 0, programs_interpreted = 0; // launches of fused programs, by kernel kind
@@ -224,6 +226,14 @@ constexpr uint8_t kInstrU32 = 0x80;
 // put off: if the soft-max over it ends up as the left operand of p.V, the three are run as one
 // fused attention kernel and the scores never exist in memory; any other use computes the
 // product once (`result`) and reads it like any buffer.
+// A small element-wise result whose destination is known but which nobody has read yet: the rows a
+// decode step appends to the KV cache.  Put off until the next launch, which it then shares with
+// its neighbours (at most three per launch).
+struct DeferredWrite {
+    cg_tensor *dst = nullptr; // a view of the destination; its buffer is retained
+    Pending *prog = nullptr;  // owned
+};
+
 struct LazyMm {
     std::atomic<long> rc{1};
     cg_tensor *x = nullptr, *y = nullptr; // retained operands (concrete)
@@ -367,6 +377,10 @@ int fold_matmul(const cg_tensor *x, const cg_tensor *y, MmFold *f);
 // below) when the shapes do not allow it.
 int launch_matmul_gated(cg_backend *be, const cg_tensor *x, const cg_tensor *yg, const cg_tensor *yu, uint32_t one,
                         cg_tensor *out);
+int launch_fused_group(cg_backend *be, const cg_tensor *const *outs, const Pending *const *ps, int n);
+// Writes that were put off so that they can share a launch (see DeferredWrite); every function
+// that launches a kernel or copies device memory calls this first.
+int flush_deferred(cg_backend *be);
 int launch_matmul_residual(cg_backend *be, const cg_tensor *x, const cg_tensor *y, const uint32_t *const *terms, int slot,
                            int order, cg_tensor *out);
 int launch_matmul_group(cg_backend *be, const cg_tensor *x, const cg_tensor *const *ys, cg_tensor *const *outs, int n);

@@ -175,6 +175,7 @@ __global__ __launch_bounds__(kBlock) void gather_kernel(const uint32_t *__restri
 } // namespace
 
 int launch_elementwise(cg_backend *be, int op, cg_dtype dt, const cg_tensor *out, const cg_tensor *const *ins, int nin) {
+    if (int frc = flush_deferred(be)) return frc;
     const cg_tensor *views[4] = {out, nullptr, nullptr, nullptr};
     for (int k = 0; k < nin; k++) views[k + 1] = ins[k];
     EwArgs a;
@@ -235,6 +236,7 @@ int launch_fill_word(cg_backend *be, void *ptr, uint32_t bits) {
 }
 
 int launch_gather(cg_backend *be, const cg_tensor *x, int dim, const cg_tensor *idx, cg_tensor *out) {
+    if (int frc = flush_deferred(be)) return frc;
     int64_t outer = 1, inner = 1;
     for (int i = 0; i < dim; i++) outer *= x->dims[i];
     for (int i = dim + 1; i < x->rank; i++) inner *= x->dims[i];

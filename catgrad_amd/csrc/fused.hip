@@ -589,6 +589,7 @@ static int64_t attn_blocks() {
 
 int launch_decode_attention(cg_backend *be, const Pending &p, const int64_t *pdims, int prank, const cg_tensor *q,
                             const cg_tensor *kt, const cg_tensor *v, cg_tensor *out) {
+    if (int frc = flush_deferred(be)) return frc;
     using P = RowsSoftmaxCausal;
     if (!be->aot || !program_matches<P>(p) || !p.leaf[0].lazy || p.leaf[0].lazy->result || p.reduced) return kDeclined;
     cg_tensor pd; // the soft-max result as a dense descriptor: the left operand of p.V
@@ -692,6 +693,7 @@ bool fused_program_fits(const Pending &p) {
 }
 
 int launch_fused(cg_backend *be, const cg_tensor *out, const Pending &p) {
+    if (int frc = flush_deferred(be)) return frc;
     FusedArgs a;
     double bytes;
     bool full;
@@ -722,8 +724,44 @@ int launch_fused(cg_backend *be, const cg_tensor *out, const Pending &p) {
     return e == hipSuccess ? CG_OK : hip_fail(e, "fused element-wise launch");
 }
 
+// Two or three element-wise results in one launch; declines unless every program is one the
+// grouped kernel holds (rotary embedding, strided copy).
+int launch_fused_group(cg_backend *be, const cg_tensor *const *outs, const Pending *const *ps, int n) {
+    if (!be->aot || n < 2 || n > kMaxMapGroup) return kDeclined;
+    FusedGroup g;
+    double bytes = 0;
+    uint32_t blocks = 0;
+    for (int i = 0; i < n; i++) {
+        const Pending &p = *ps[i];
+        if (program_matches<MapRope>(p))
+            g.prog[i] = 0;
+        else if (p.nleaf == 1 && p.ninstr == 1 && p.nred == 0 && (p.ins[0].op & ~kInstrU32) == kCopy && p.ins[0].a == 0 &&
+                 !p.leaf[0].uniform && !p.leaf[0].pw)
+            g.prog[i] = 1;
+        else
+            return kDeclined;
+        double b;
+        bool full;
+        int rc = fill_args(be, p, outs[i]->dims, outs[i]->rank, outs[i], false, &g.p[i], &b, &full);
+        if (rc) return rc;
+        if (g.p[i].g.total == 0) return kDeclined;
+        bytes += b + distinct_bytes(outs[i]);
+        g.first[i] = blocks;
+        blocks += (uint32_t)((g.p[i].g.total + kBlock - 1) / kBlock);
+    }
+    g.first[n] = blocks;
+    g.n = (uint32_t)n;
+    for (int i = 0; i < n; i++) trace_program(be, *ps[i], ps[i]->ninstr, "map (grouped)", outs[i]->dims, outs[i]->rank);
+    ProfScope prof(be, CG_K_ELEMENTWISE, bytes);
+    hipLaunchKernelGGL(aot_map_group_kernel, dim3(blocks), dim3(kBlock), 0, be->stream, g);
+    be->programs_compiled += n;
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CG_OK : hip_fail(e, "grouped element-wise launch");
+}
+
 int launch_fused_reduce(cg_backend *be, int kind, bool f32, const Pending &p, int ninstr, const int64_t *dims, int rank,
                         cg_tensor *out) {
+    if (int frc = flush_deferred(be)) return frc;
     FusedArgs a;
     double bytes;
     bool full;
@@ -771,6 +809,7 @@ int launch_fused_reduce(cg_backend *be, int kind, bool f32, const Pending &p, in
 }
 
 int launch_fused_rows(cg_backend *be, const cg_tensor *out, const Pending &p, const int64_t *dims, int rank) {
+    if (int frc = flush_deferred(be)) return frc;
     FusedArgs a;
     double bytes;
     bool full;

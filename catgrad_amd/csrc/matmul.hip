@@ -302,10 +302,14 @@ struct MmResidual {
     uint32_t slot, order;
 };
 
+#ifndef CG_WIDE_UNROLL
+#define CG_WIDE_UNROLL 2
+#endif
 template <int MM, int COLS, bool SPLIT, bool RESIDUAL = false>
 __device__ __forceinline__ void skinny_kt_wide_body(const MmArgs &a, const uint32_t block_x, const uint32_t block_y,
                                                     const MmResidual *res = nullptr) {
     static_assert(!RESIDUAL || (COLS == 1 && !SPLIT), "the residual store is written for one column per wave");
+    constexpr int kWideUnroll = COLS == 1 ? CG_WIDE_UNROLL : 2;
     const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x % 64;
     const uint32_t group = SPLIT ? block_x : block_x * 4 + wave;
     const uint32_t n0 = group * COLS;
@@ -333,7 +337,7 @@ __device__ __forceinline__ void skinny_kt_wide_body(const MmArgs &a, const uint3
         for (int m = 0; m < MM; m++) acc[c][m] = 0.0f;
     if (live) {
         const uint32_t kstep = SPLIT ? 1024u : 256u;
-#pragma unroll 2
+#pragma unroll kWideUnroll
         for (uint32_t k = (SPLIT ? wave * 256u : 0u) + lane * 4; k < a.K; k += kstep) {
             float4v w[COLS], x[MM];
 #pragma unroll
@@ -775,6 +779,7 @@ static int make_mm_args(const cg_tensor *x, const cg_tensor *y, void *c, MmArgs 
 }
 
 int launch_matmul_group(cg_backend *be, const cg_tensor *x, const cg_tensor *const *ys, cg_tensor *const *outs, int n) {
+    if (int frc = flush_deferred(be)) return frc;
     if (n < 2 || n > kMaxGroup || x->dt != CG_F32) return kDeclined;
     MmGroup g;
     memset(&g, 0, sizeof g);
@@ -817,6 +822,7 @@ int launch_matmul_group(cg_backend *be, const cg_tensor *x, const cg_tensor *con
 // kernel takes the shapes.
 int launch_matmul_gated(cg_backend *be, const cg_tensor *x, const cg_tensor *yg, const cg_tensor *yu, uint32_t one,
                         cg_tensor *out) {
+    if (int frc = flush_deferred(be)) return frc;
     if (x->dt != CG_F32) return kDeclined;
     MmArgs ag, au;
     MmFold fg, fu;
@@ -838,6 +844,7 @@ int launch_matmul_gated(cg_backend *be, const cg_tensor *x, const cg_tensor *yg,
 // is what the product would run on anyway.
 int launch_matmul_residual(cg_backend *be, const cg_tensor *x, const cg_tensor *y, const uint32_t *const *terms, int slot,
                            int order, cg_tensor *out) {
+    if (int frc = flush_deferred(be)) return frc;
     if (x->dt != CG_F32) return kDeclined;
     MmArgs a;
     MmFold f;
@@ -862,6 +869,7 @@ int launch_matmul_residual(cg_backend *be, const cg_tensor *x, const cg_tensor *
 }
 
 int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_tensor *out) {
+    if (int frc = flush_deferred(be)) return frc;
     MmArgs a;
     MmFold f;
     int rc = make_mm_args(x, y, out->buf->ptr, &a, &f);

@@ -346,6 +346,7 @@ template <int K, bool F> int launch_rows(cg_backend *be, const RowsArgs &a) {
 } // namespace
 
 int launch_reduce(cg_backend *be, int kind, const cg_tensor *x, cg_tensor *out) {
+    if (int frc = flush_deferred(be)) return frc;
     RowsArgs a;
     int rc = fill_rows_args(x, &a);
     if (rc) return rc;
@@ -361,6 +362,7 @@ int launch_reduce(cg_backend *be, int kind, const cg_tensor *x, cg_tensor *out) 
 }
 
 int launch_topk(cg_backend *be, const cg_tensor *x, int64_t k, cg_tensor *vals, cg_tensor *idxs) {
+    if (int frc = flush_deferred(be)) return frc;
     RowsArgs a;
     int rc = fill_rows_args(x, &a);
     if (rc) return rc;
@@ -372,6 +374,7 @@ int launch_topk(cg_backend *be, const cg_tensor *x, int64_t k, cg_tensor *vals, 
 }
 
 static int launch_any(cg_backend *be, int mode, const cg_tensor *x, const cg_tensor *y) {
+    if (int frc = flush_deferred(be)) return frc;
     int rc = launch_fill_word(be, be->flag_dev, 0);
     if (rc) return rc;
     const cg_tensor *views[2] = {x, y ? y : x};

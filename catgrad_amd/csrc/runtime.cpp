@@ -752,6 +752,68 @@ static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p) {
     return launch_fused(be, dst, p);
 }
 
+static void drop_deferred(DeferredWrite &w) {
+    delete w.prog;
+    if (w.dst) {
+        buffer_release(w.dst->buf);
+        w.dst->buf = nullptr;
+        delete w.dst;
+    }
+    w.prog = nullptr;
+    w.dst = nullptr;
+}
+
+int flush_deferred(cg_backend *be) {
+    if (be->deferred.empty()) return CG_OK;
+    std::vector<DeferredWrite> w;
+    w.swap(be->deferred); // the launches below come back here and find nothing to do
+    int rc = CG_OK;
+    const int n = (int)w.size();
+    for (int i = 0; i < n && !rc; i++) rc = resolve_lazy_leaves(be, *w[i].prog);
+    bool done = false;
+    if (!rc && n >= 2) {
+        const cg_tensor *outs[4];
+        const Pending *ps[4];
+        for (int i = 0; i < n && i < 4; i++) {
+            outs[i] = w[i].dst;
+            ps[i] = w[i].prog;
+        }
+        rc = n <= 4 ? launch_fused_group(be, outs, ps, n) : kDeclined;
+        done = rc == CG_OK;
+        if (rc == kDeclined) rc = CG_OK;
+    }
+    for (int i = 0; i < n && !rc && !done; i++) rc = run_pending(be, w[i].dst, *w[i].prog);
+    for (DeferredWrite &d : w) drop_deferred(d);
+    return rc;
+}
+
+// Puts off the write of `prog`'s value (or, prog == null, of a copy of `src`) into the view `dst`.
+// At most three writes wait at a time.
+static int defer_write(cg_backend *be, const cg_tensor *dst, const Pending *prog) {
+    if (be->deferred.size() >= 3) {
+        int rc = flush_deferred(be);
+        if (rc) return rc;
+    }
+    DeferredWrite w;
+    w.dst = new cg_tensor;
+    w.dst->be = be;
+    w.dst->buf = dst->buf;
+    w.dst->buf->rc.fetch_add(1);
+    w.dst->dt = dst->dt;
+    w.dst->rank = dst->rank;
+    memcpy(w.dst->dims, dst->dims, sizeof dst->dims);
+    memcpy(w.dst->strides, dst->strides, sizeof dst->strides);
+    w.dst->offset = dst->offset;
+    w.prog = new Pending(*prog);
+    be->deferred.push_back(w);
+    return CG_OK;
+}
+
+// A program small enough to wait for company: no row reduces, at most 16 K elements.
+static bool may_wait(const cg_backend *be, const cg_tensor *dst, const Pending *p) {
+    return be->fuse && be->aot && p && p->nred == 0 && !p->reduced && numel(dst) > 0 && numel(dst) <= 16384;
+}
+
 // Turns a deferred tensor into a concrete one, in place (every holder of the handle sees it).
 static int ensure_concrete(cg_tensor *t) {
     if (t->split >= 0) { // a split-axis view becomes a plain dense tensor, in place
@@ -805,7 +867,13 @@ static int ensure_concrete(cg_tensor *t) {
     dst.rank = t->rank;
     memcpy(dst.dims, t->dims, sizeof dst.dims);
     set_row_major(&dst);
-    rc = run_pending(be, &dst, *t->pend);
+    if (!be->deferred.empty() && may_wait(be, &dst, t->pend)) {
+        // writes are waiting for a launch: this one goes along
+        rc = defer_write(be, &dst, t->pend);
+        if (!rc) rc = flush_deferred(be);
+    } else {
+        rc = run_pending(be, &dst, *t->pend);
+    }
     dst.buf = nullptr;
     if (rc) {
         buffer_release(b);
@@ -1259,7 +1327,11 @@ static bool try_row_append(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim
         }
         dst.offset = x->offset / (C * R) * (dC * R) + row0 * R;
         const cg_tensor *ins[1] = {src_t};
-        int rc = src_t->pend ? run_pending(b, &dst, *src_t->pend) : launch_elementwise(b, kCopy, x->dt, &dst, ins, 1);
+        int rc;
+        if (src_t->pend && may_wait(b, &dst, src_t->pend))
+            rc = defer_write(b, &dst, src_t->pend); // the rows are written with the next launch
+        else
+            rc = src_t->pend ? run_pending(b, &dst, *src_t->pend) : launch_elementwise(b, kCopy, x->dt, &dst, ins, 1);
         dst.buf = nullptr;
         return rc;
     };
@@ -1365,6 +1437,8 @@ int cg_backend_create(int device, cg_backend **out) {
 void cg_backend_destroy(cg_backend *b) {
     if (!b) return;
     (void)hipSetDevice(b->device);
+    for (DeferredWrite &d : b->deferred) drop_deferred(d); // nobody can read them any more
+    b->deferred.clear();
     (void)hipStreamSynchronize(b->stream);
     prof_drain(b);
     for (auto &ev : b->prof_free) {
@@ -1388,6 +1462,7 @@ const char *cg_backend_name(cg_backend *b) { return b ? b->name.c_str() : ""; }
 
 int cg_sync(cg_backend *b) {
     if (!b) return fail(CG_ERR_ARG, "null backend");
+    if (int frc = flush_deferred(b)) return frc;
     return wait_and_check(b);
 }
 
@@ -1590,6 +1665,7 @@ int cg_arange(cg_backend *b, size_t end, cg_tensor **out) {
 
 // ---- read-back -----------------------------------------------------------------------------
 static int copy_out(cg_backend *b, const cg_tensor *t, void *dst, size_t len) {
+    if (int frc = flush_deferred(b)) return frc;
     if (len == 0) return wait_and_check(b);
     if (t->pend) {
         int rc = ensure_concrete(const_cast<cg_tensor *>(t));

@@ -529,6 +529,51 @@ def _():
     return run, expect
 
 
+@case("kv_deferred_row_writes", "red")
+def _():
+    """Rows appended to a cache from element-wise programs (as the rotary embedding of k is) may be written
+    late, together with their neighbours: every kind of reader that follows must still see them — read-back,
+    a reduction, a gather, a matrix product, another program, a clone taken before the next append — also with
+    more appends in a row than one launch takes, and with a deferred left operand of a product joining them."""
+    B, H, T0, D = 2, 2, 40, 64
+    base = np.abs(f32(700, (B, H, T0, D)))
+    rows = [np.abs(f32(701 + i, (B, H, 1, D))) for i in range(7)]
+    q = np.abs(f32(720, (B, H, 1, D)))
+    ids = np.array([0, T0 + 2, T0 + 6, 5], np.uint32)
+
+    def run(be):
+        two = lambda: _const(be, 2.0, (B, H, 1, D))
+        cache = be.from_numpy(base)
+        outs = []
+        for i, r in enumerate(rows):
+            new = be.mul(be.from_numpy(r).move(), two().move())        # a deferred program
+            cache = be.concat(cache.move(), new.move(), 2)
+            if i == 0:
+                outs.append(be.to_numpy(cache))                          # read-back right after one append
+            if i == 1:
+                outs.append(be.to_numpy(be.sum(be.transpose(cache, 2, 3))))   # reduction over the time axis
+            if i == 2:
+                old = cache.clone()
+        outs.append(be.to_numpy(be.index(cache, 2, be.from_numpy(ids))))      # 4 appends waiting: gather
+        tq = be.mul(be.from_numpy(q).move(), two().move())                   # deferred left operand
+        new = be.add(be.from_numpy(rows[0]).move(), two().move())
+        cache = be.concat(cache.move(), new.move(), 2)
+        scores = be.matmul(tq.move(), be.transpose(cache, 2, 3).move())      # joins the waiting write
+        outs.append(be.to_numpy(scores))
+        outs.append(be.to_numpy(be.exp(be.neg(be.slice(cache, 2, T0, 8)))))
+        outs.append(be.to_numpy(old))
+        outs.append(be.to_numpy(cache))
+        return outs
+
+    def expect():
+        full = np.concatenate([base] + [2 * r for r in rows] + [rows[0] + 2], 2).astype(np.float64)
+        return [full[:, :, :T0 + 1], full[:, :, :T0 + 2].sum(2)[..., None], full[:, :, ids],
+                (2 * q.astype(np.float64)) @ full.transpose(0, 1, 3, 2), np.exp(-full[:, :, T0:T0 + 8]),
+                full[:, :, :T0 + 3], full]
+
+    return run, expect
+
+
 @case("concat_adjacent_views_merge")
 def _():
     a = f32(140, (6, 4, 10))

@@ -160,6 +160,21 @@ def test_programs_absorbed_by_decode_time_products(hip):
             np.testing.assert_allclose(g, e, rtol=1e-3)
 
 
+def test_backend_closes_with_writes_still_waiting():
+    """Rows appended from a program and never read: the write is still waiting when the tensors and the
+    backend go away."""
+    from catgrad_amd import HipBackend
+
+    be = HipBackend(0)
+    cache = be.from_numpy(np.ones((2, 2, 8, 64), np.float32))
+    for _ in range(2):
+        new = be.neg(be.from_numpy(np.ones((2, 2, 1, 64), np.float32)).move())
+        cache = be.concat(cache.move(), new.move(), 2)
+    assert cache.shape == (2, 2, 10, 64)
+    del cache, new
+    be.close()
+
+
 def test_format_tensor(hip):
     s = hip.format_tensor(hip.from_numpy(np.array([[1.5, 2.0]], np.float32)))
     assert "f32[1,2]" in s and "1.5" in s
