@@ -65,6 +65,7 @@ struct ProfPending {
 namespace cg {
 struct LazyMm;
 struct DeferredWrite;
+struct Buffer;
 }
 
 struct cg_backend {
@@ -83,6 +84,14 @@ struct cg_backend {
     std::string name;
     std::vector<cg::LazyMm *> lazy_open; // groupable lazy products not yet computed (not retained)
     std::vector<cg::DeferredWrite> deferred; // writes waiting to share a launch (see flush_deferred)
+    // Results that depend on constants only (the rotary tables every forward pass rebuilds from iota and
+    // scalars) are kept, keyed by the program and its leaves, and handed out again instead of recomputed.
+    // Buffers are retained here; the oldest entries go when the limits are reached.
+    std::map<std::string, cg::Buffer *> const_memo;
+    std::vector<std::string> const_order; // keys, oldest first
+    size_t const_bytes = 0;
+    cg::Buffer *iota = nullptr; // 0, 1, 2, ... : every arange is a view of it
+    int64_t iota_len = 0;
     bool fuse = true; // defer element-wise ops and fuse them (CG_FUSE=0 switches it off)
     bool aot = true;  // use the compiled kernels for listed programs (CG_AOT=0: interpreter only)
     uint64_t programs_compiled = 0, programs_interpreted = 0; // launches of fused programs, by kernel kind
@@ -105,12 +114,19 @@ struct RowStore {
     std::vector<int64_t> fill;
 };
 
+inline uint64_t next_buffer_id() {
+    static std::atomic<uint64_t> n{1};
+    return n.fetch_add(1);
+}
+
 struct Buffer {
     std::atomic<long> rc{1};
+    const uint64_t id = next_buffer_id(); // never reused, unlike the address: what keys of kept results name
     void *ptr = nullptr;
     size_t cls = 0;
     cg_backend *be = nullptr;
     RowStore *rs = nullptr;      // owned
+    bool constant = false;       // the contents depend on constants only (iota, programs over such buffers)
     Buffer *successor = nullptr; // retained: the roomier buffer that blocks of this one migrate to on append
 };
 

@@ -752,6 +752,104 @@ static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p) {
     return launch_fused(be, dst, p);
 }
 
+// ---- results of constant programs -------------------------------------------------------------------------
+constexpr size_t kConstEntryBytes = 64u << 20, kConstTotalBytes = 512u << 20, kConstEntries = 256;
+
+// The identity of a program whose leaves are constants or constant buffers, as a byte string; false
+// when some leaf is neither.
+static bool const_key(const Pending &p, const int64_t *dims, int rank, std::string *key) {
+    if (p.overflow) return false;
+    std::string k;
+    auto put = [&](const void *v, size_t n) { k.append(static_cast<const char *>(v), n); };
+    const int32_t head[5] = {rank, p.nleaf, p.ninstr, p.nred, p.reduced ? 1 : 0};
+    put(head, sizeof head);
+    put(dims, sizeof(int64_t) * (size_t)rank);
+    put(&p.rowlen, sizeof p.rowlen);
+    for (int i = 0; i < p.ninstr; i++) put(&p.ins[i], sizeof(Instr));
+    for (int l = 0; l < p.nleaf; l++) {
+        const LeafView &lv = p.leaf[l];
+        if (lv.lazy) return false;
+        const char kind = lv.uniform ? 'u' : lv.pw ? 'p' : 'v';
+        put(&kind, 1);
+        if (lv.uniform) {
+            put(&lv.ubits, sizeof lv.ubits);
+            continue;
+        }
+        if (!lv.buf || !lv.buf->constant) return false;
+        put(&lv.buf->id, sizeof lv.buf->id);
+        put(&lv.offset, sizeof lv.offset);
+        for (int d = 0; d < rank; d++) {
+            const int64_t st = dims[d] > 1 ? lv.strides[d] : 0;
+            put(&st, sizeof st);
+        }
+        if (lv.pw) {
+            if (!lv.buf2 || !lv.buf2->constant) return false;
+            put(&lv.buf2->id, sizeof lv.buf2->id);
+            put(&lv.offset2, sizeof lv.offset2);
+            put(&lv.pw_split, sizeof lv.pw_split);
+            const char neg[2] = {(char)lv.neg1, (char)lv.neg2};
+            put(neg, 2);
+            for (int d = 0; d < rank; d++) {
+                const int64_t st = dims[d] > 1 ? lv.strides2[d] : 0;
+                put(&st, sizeof st);
+            }
+        }
+    }
+    *key = std::move(k);
+    return true;
+}
+
+// The same for a tensor: deferred (its program), a constant, or a view of a constant buffer.
+static bool const_tensor_key(const cg_tensor *t, std::string *key) {
+    if (t->split >= 0) return false;
+    if (t->pend) return const_key(*t->pend, t->dims, t->rank, key);
+    std::string k(t->uniform ? "U" : "V");
+    auto put = [&](const void *v, size_t n) { k.append(static_cast<const char *>(v), n); };
+    put(&t->rank, sizeof t->rank);
+    put(t->dims, sizeof(int64_t) * (size_t)t->rank);
+    if (t->uniform) {
+        put(&t->ubits, sizeof t->ubits);
+    } else {
+        if (!t->buf || !t->buf->constant) return false;
+        put(&t->buf->id, sizeof t->buf->id);
+        put(&t->offset, sizeof t->offset);
+        for (int d = 0; d < t->rank; d++) {
+            const int64_t st = t->dims[d] > 1 ? t->strides[d] : 0;
+            put(&st, sizeof st);
+        }
+    }
+    *key = std::move(k);
+    return true;
+}
+
+static void const_memo_clear(cg_backend *be) {
+    for (auto &kv : be->const_memo) buffer_release(kv.second);
+    be->const_memo.clear();
+    be->const_order.clear();
+    be->const_bytes = 0;
+    buffer_release(be->iota);
+    be->iota = nullptr;
+    be->iota_len = 0;
+}
+
+static void const_memo_insert(cg_backend *be, const std::string &key, Buffer *b) {
+    if (b->cls > kConstEntryBytes) return;
+    while (!be->const_order.empty() && (be->const_memo.size() >= kConstEntries || be->const_bytes + b->cls > kConstTotalBytes)) {
+        auto it = be->const_memo.find(be->const_order.front());
+        if (it != be->const_memo.end()) {
+            be->const_bytes -= it->second->cls;
+            buffer_release(it->second);
+            be->const_memo.erase(it);
+        }
+        be->const_order.erase(be->const_order.begin());
+    }
+    b->constant = true;
+    b->rc.fetch_add(1);
+    be->const_memo[key] = b;
+    be->const_order.push_back(key);
+    be->const_bytes += b->cls;
+}
+
 static void drop_deferred(DeferredWrite &w) {
     delete w.prog;
     if (w.dst) {
@@ -853,6 +951,21 @@ static int ensure_concrete(cg_tensor *t) {
         delete old;
         return CG_OK;
     }
+    std::string ckey;
+    const bool constant = be->fuse && numel(t) > 0 && const_key(*t->pend, t->dims, t->rank, &ckey);
+    if (constant) {
+        auto hit = be->const_memo.find(ckey);
+        if (hit != be->const_memo.end()) { // computed before from the same constants: the handle takes that buffer
+            hit->second->rc.fetch_add(1);
+            Pending *old = t->pend;
+            t->buf = hit->second;
+            t->offset = 0;
+            set_row_major(t);
+            t->pend = nullptr;
+            delete old;
+            return CG_OK;
+        }
+    }
     Buffer *b = new Buffer;
     b->be = be;
     int rc = be->pool.alloc((size_t)numel(t) * 4, &b->ptr, &b->cls);
@@ -867,6 +980,7 @@ static int ensure_concrete(cg_tensor *t) {
     dst.rank = t->rank;
     memcpy(dst.dims, t->dims, sizeof dst.dims);
     set_row_major(&dst);
+    if (constant) const_memo_insert(be, ckey, b); // before the leaves go away with the program
     if (!be->deferred.empty() && may_wait(be, &dst, t->pend)) {
         // writes are waiting for a launch: this one goes along
         rc = defer_write(be, &dst, t->pend);
@@ -876,6 +990,7 @@ static int ensure_concrete(cg_tensor *t) {
     }
     dst.buf = nullptr;
     if (rc) {
+        if (constant) const_memo_clear(be); // it holds a buffer that was never filled
         buffer_release(b);
         return rc;
     }
@@ -1439,6 +1554,7 @@ void cg_backend_destroy(cg_backend *b) {
     (void)hipSetDevice(b->device);
     for (DeferredWrite &d : b->deferred) drop_deferred(d); // nobody can read them any more
     b->deferred.clear();
+    const_memo_clear(b);
     (void)hipStreamSynchronize(b->stream);
     prof_drain(b);
     for (auto &ev : b->prof_free) {
@@ -1469,12 +1585,17 @@ int cg_sync(cg_backend *b) {
 int cg_pool_stats(cg_backend *b, size_t *bytes_in_use, size_t *bytes_cached) {
     if (!b) return fail(CG_ERR_ARG, "null backend");
     b->pool.stats(bytes_in_use, bytes_cached);
+    // what the backend keeps for itself (iota, results of constant programs) counts as cached
+    size_t kept = b->const_bytes + (b->iota ? b->iota->cls : 0);
+    if (bytes_in_use) *bytes_in_use -= kept < *bytes_in_use ? kept : *bytes_in_use;
+    if (bytes_cached) *bytes_cached += kept;
     return CG_OK;
 }
 
 int cg_pool_trim(cg_backend *b) {
     if (!b) return fail(CG_ERR_ARG, "null backend");
     CG_HIP(hipStreamSynchronize(b->stream));
+    const_memo_clear(b);
     b->pool.trim();
     return CG_OK;
 }
@@ -1650,6 +1771,38 @@ int cg_arange(cg_backend *b, size_t end, cg_tensor **out) {
     if (end > (1u << 24)) return fail(CG_ERR_UNSUPPORTED, "arange: end above 2^24 is inexact in the reference");
     int64_t d[1] = {(int64_t)end};
     cg_tensor *t;
+    if (b->fuse && end > 0) {
+        // a view of the backend's one iota buffer, which grows in powers of two
+        if ((int64_t)end > b->iota_len) {
+            int64_t cap = 4096;
+            while (cap < (int64_t)end) cap *= 2;
+            cg_tensor *full;
+            int64_t fd[1] = {cap};
+            CG_HIP(hipSetDevice(b->device));
+            int rc = new_dense(b, CG_U32, fd, 1, &full);
+            if (!rc) rc = launch_arange(b, full);
+            if (rc) {
+                release(full);
+                return rc;
+            }
+            buffer_release(b->iota);
+            b->iota = full->buf;
+            b->iota->constant = true;
+            b->iota->rc.fetch_add(1);
+            b->iota_len = cap;
+            release(full);
+        }
+        t = new cg_tensor;
+        t->be = b;
+        t->dt = CG_U32;
+        t->rank = 1;
+        t->dims[0] = d[0];
+        t->strides[0] = 1;
+        t->buf = b->iota;
+        t->buf->rc.fetch_add(1);
+        *out = t;
+        return CG_OK;
+    }
     int rc = new_dense(b, CG_U32, d, 1, &t);
     if (rc) return rc;
     if (end) {
@@ -2374,9 +2527,38 @@ int cg_concat(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor *
         return CG_OK;
     }
     cg_tensor *o;
+    // both operands constants (the halves of a rotary table): the result is kept and handed out again
+    std::string ckey;
+    bool constant = false;
+    if (b->fuse && nx > 0 && ny > 0) {
+        std::string kx, ky;
+        if (const_tensor_key(x, &kx) && const_tensor_key(y, &ky)) {
+            constant = true;
+            const int64_t d = (int64_t)dim, lx = (int64_t)kx.size();
+            ckey.assign("concat");
+            ckey.append(reinterpret_cast<const char *>(&d), sizeof d);
+            ckey.append(reinterpret_cast<const char *>(&lx), sizeof lx);
+            ckey += kx;
+            ckey += ky;
+            auto hit = b->const_memo.find(ckey);
+            if (hit != b->const_memo.end()) {
+                o = new cg_tensor;
+                o->be = b;
+                o->dt = x->dt;
+                o->rank = x->rank;
+                memcpy(o->dims, od, sizeof o->dims);
+                set_row_major(o);
+                o->buf = hit->second;
+                o->buf->rc.fetch_add(1);
+                *out = o;
+                return CG_OK;
+            }
+        }
+    }
     // a stack that starts growing gets room for as much again, so later appends stay in place
-    int rc = new_dense(b, x->dt, od, x->rank, &o, outermost ? 2 * (nx + ny) : 0);
+    int rc = new_dense(b, x->dt, od, x->rank, &o, outermost && !constant ? 2 * (nx + ny) : 0);
     if (rc) return rc;
+    if (constant) const_memo_insert(b, ckey, o->buf);
     const cg_tensor *parts[2] = {x, y};
     int64_t at = 0;
     for (int p = 0; p < 2 && !rc; p++) {
@@ -2398,6 +2580,7 @@ int cg_concat(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor *
         at += src->dims[dim];
     }
     if (rc) {
+        if (constant) const_memo_clear(b); // it holds a buffer that was never filled
         release(o);
         return rc;
     }

@@ -574,6 +574,45 @@ def _():
     return run, expect
 
 
+@case("constant_programs_are_kept", "ew_abs")
+def _():
+    """Tables built from iota and scalars (rope.rs:65-104 does this on every forward pass) are computed once
+    and handed out again: the second build must equal the first, a different scalar must give different
+    values, growing a kept table by concat must not change what the next build sees, and every arange is
+    a view of one growing iota.  (Angles up to 100: one ulp of the angle is 8e-6, inside the absolute tolerance.)"""
+    n, h = 100, 16
+
+    def table(be, theta, fn):
+        pos = be.cast(be.arange(n), A.F32)
+        inv = be.pow(_const(be, theta, (h,)), be.neg(be.div(be.cast(be.arange(h), A.F32), _const(be, float(h), (h,)))))
+        ang = be.mul(be.broadcast(be.reshape(pos, (n, 1)), (n, h)), be.broadcast(be.reshape(inv, (1, h)), (n, h)))
+        half = fn(ang)
+        return be.concat(half, half, 1)
+
+    def run(be):
+        outs = [be.to_numpy(be.arange(5)), be.to_numpy(be.arange(5000)), be.to_numpy(be.arange(7))]
+        t1 = table(be, 100.0, be.cos)
+        outs.append(be.to_numpy(t1))
+        grown = be.concat(t1.move(), be.from_numpy(np.ones((2, 2 * h), np.float32)).move(), 0)
+        outs.append(be.to_numpy(grown))
+        outs.append(be.to_numpy(table(be, 100.0, be.cos)))      # kept
+        outs.append(be.to_numpy(table(be, 50.0, be.cos)))       # another constant: not the kept one
+        outs.append(be.to_numpy(table(be, 100.0, be.sin)))
+        return outs
+
+    def expect():
+        def tab(theta, fn):
+            # the angles as f32 computes them (each step rounded), the function itself in float64
+            inv = (np.float64(theta) ** (-(np.arange(h, dtype=np.float32) / np.float32(h)).astype(np.float64))).astype(np.float32)
+            ang = (np.arange(n, dtype=np.float32)[:, None] * inv[None, :]).astype(np.float64)
+            return np.concatenate([fn(ang), fn(ang)], 1)
+        t = tab(100.0, np.cos)
+        return [np.arange(5, dtype=np.uint32), np.arange(5000, dtype=np.uint32), np.arange(7, dtype=np.uint32),
+                t, np.concatenate([t, np.ones((2, 2 * h))], 0), t, tab(50.0, np.cos), tab(100.0, np.sin)]
+
+    return run, expect
+
+
 @case("concat_adjacent_views_merge")
 def _():
     a = f32(140, (6, 4, 10))
