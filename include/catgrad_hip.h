@@ -103,9 +103,10 @@ const char *cg_last_error(void);
 const char *cg_backend_name(cg_backend *b);
 /* Wait for all queued work; reports deferred device-detected faults. */
 int cg_sync(cg_backend *b);
-/* Bytes currently handed out by / cached in the device pool (lifetime tests). */
+/* Bytes currently handed out by / cached in the device pool (lifetime tests).  Memory the backend keeps for
+ * itself (its iota buffer, kept results of constant programs) counts as cached. */
 int cg_pool_stats(cg_backend *b, size_t *bytes_in_use, size_t *bytes_cached);
-/* Return cached blocks to the driver. */
+/* Return cached blocks to the driver; also drops the kept results of constant programs. */
 int cg_pool_trim(cg_backend *b);
 
 /* ---- measurement hooks (no counterpart in the reference; used by the benchmark) ----
