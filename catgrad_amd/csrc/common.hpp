@@ -69,6 +69,7 @@ struct Buffer;
 }
 
 struct cg_backend {
+    std::recursive_mutex mu; // held by every entry point for the duration of the call
     int device = 0;
     hipStream_t stream = nullptr;
     cg::Pool pool;

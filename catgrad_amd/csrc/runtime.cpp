@@ -1514,6 +1514,21 @@ using namespace cg;
 extern "C" {
 
 // ---- backend lifetime ----------------------------------------------------------------
+// Every entry point that touches a backend's state holds the backend's lock for its whole duration
+// (declared first, so the tensor arguments it consumes are released under the lock too): handles may be
+// cloned, moved between threads and used from several threads; calls on one backend then run one at a time.
+struct Enter {
+    explicit Enter(cg_backend *b) : b_(b) {
+        if (b_) b_->mu.lock();
+    }
+    ~Enter() {
+        if (b_) b_->mu.unlock();
+    }
+    Enter(const Enter &) = delete;
+    Enter &operator=(const Enter &) = delete;
+    cg_backend *b_;
+};
+
 int cg_backend_create(int device, cg_backend **out) {
     if (!out) return fail(CG_ERR_ARG, "null out");
     int count = 0;
@@ -1577,12 +1592,14 @@ const char *cg_last_error(void) { return g_err.c_str(); }
 const char *cg_backend_name(cg_backend *b) { return b ? b->name.c_str() : ""; }
 
 int cg_sync(cg_backend *b) {
+    Enter entered(b);
     if (!b) return fail(CG_ERR_ARG, "null backend");
     if (int frc = flush_deferred(b)) return frc;
     return wait_and_check(b);
 }
 
 int cg_pool_stats(cg_backend *b, size_t *bytes_in_use, size_t *bytes_cached) {
+    Enter entered(b);
     if (!b) return fail(CG_ERR_ARG, "null backend");
     b->pool.stats(bytes_in_use, bytes_cached);
     // what the backend keeps for itself (iota, results of constant programs) counts as cached
@@ -1593,6 +1610,7 @@ int cg_pool_stats(cg_backend *b, size_t *bytes_in_use, size_t *bytes_cached) {
 }
 
 int cg_pool_trim(cg_backend *b) {
+    Enter entered(b);
     if (!b) return fail(CG_ERR_ARG, "null backend");
     CG_HIP(hipStreamSynchronize(b->stream));
     const_memo_clear(b);
@@ -1601,12 +1619,14 @@ int cg_pool_trim(cg_backend *b) {
 }
 
 int cg_profile_enable(cg_backend *b, cg_kernel_class cls, unsigned sample_every) {
+    Enter entered(b);
     if (!b || (int)cls < 0 || (int)cls >= CG_K_CLASSES) return fail(CG_ERR_ARG, "bad profile class");
     b->prof[cls].every = sample_every;
     return CG_OK;
 }
 
 int cg_program_stats(cg_backend *b, uint64_t *compiled, uint64_t *interpreted, int reset) {
+    Enter entered(b);
     if (!b) return fail(CG_ERR_ARG, "null backend");
     if (compiled) *compiled = b->programs_compiled;
     if (interpreted) *interpreted = b->programs_interpreted;
@@ -1615,12 +1635,14 @@ int cg_program_stats(cg_backend *b, uint64_t *compiled, uint64_t *interpreted, i
 }
 
 int cg_realize(cg_backend *b, cg_tensor *t) {
+    Enter entered(b);
     if (!b || !t) return fail(CG_ERR_ARG, "null argument");
     return ensure_concrete(t);
 }
 
 int cg_profile_read(cg_backend *b, cg_kernel_class cls, uint64_t *launches, double *milliseconds, double *work,
                     int reset) {
+    Enter entered(b);
     if (!b || (int)cls < 0 || (int)cls >= CG_K_CLASSES) return fail(CG_ERR_ARG, "bad profile class");
     int rc = wait_and_check(b);
     if (rc) return rc;
@@ -1639,7 +1661,11 @@ int cg_profile_read(cg_backend *b, cg_kernel_class cls, uint64_t *launches, doub
 void cg_tensor_retain(cg_tensor *t) {
     if (t) retain(t);
 }
-void cg_tensor_release(cg_tensor *t) { release(t); }
+void cg_tensor_release(cg_tensor *t) {
+    if (!t) return;
+    Enter entered(t->be); // the last holder of a deferred tensor also closes what it had open in the backend
+    release(t);
+}
 size_t cg_tensor_rank(const cg_tensor *t) { return (size_t)t->rank; }
 void cg_tensor_shape(const cg_tensor *t, size_t *dims) {
     for (int i = 0; i < t->rank; i++) dims[i] = (size_t)t->dims[i];
@@ -1647,6 +1673,7 @@ void cg_tensor_shape(const cg_tensor *t, size_t *dims) {
 cg_dtype cg_tensor_dtype(const cg_tensor *t) { return t->dt; }
 size_t cg_tensor_numel(const cg_tensor *t) { return (size_t)numel(t); }
 int cg_tensor_is_contiguous(const cg_tensor *t) {
+    Enter entered(t->be); // a deferred tensor may be being computed, in place, by another thread
     if (t->pend) return 1; // a deferred result is row-major once computed
     return (t->uniform && numel(t) > 1) ? 0 : (is_contiguous(t) ? 1 : 0);
 }
@@ -1661,6 +1688,7 @@ static int check_dims(const size_t *dims, size_t rank, int64_t *d64) {
 
 // ndarray.rs:71-84 — a zero tensor is a uniform constant: no memory, no memset.
 int cg_zeros(cg_backend *b, cg_dtype dtype, const size_t *dims, size_t rank, cg_tensor **out) {
+    Enter entered(b);
     if (!b || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(dtype)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
     int64_t d[kMaxRank];
@@ -1697,6 +1725,7 @@ static int staged_upload(cg_backend *b, void *dst, const void *src, size_t bytes
 
 int cg_from_host(cg_backend *b, cg_dtype dtype, const void *data, size_t len, const size_t *dims, size_t rank,
                  cg_tensor **out) {
+    Enter entered(b);
     if (!b || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(dtype)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
     int64_t d[kMaxRank];
@@ -1729,6 +1758,7 @@ int cg_from_host(cg_backend *b, cg_dtype dtype, const void *data, size_t len, co
 
 int cg_from_host_bf16_as_f32(cg_backend *b, const uint16_t *bits, size_t len, const size_t *dims, size_t rank,
                              cg_tensor **out) {
+    Enter entered(b);
     if (!b || !out) return fail(CG_ERR_ARG, "null argument");
     int64_t d[kMaxRank];
     int rc = check_dims(dims, rank, d);
@@ -1767,6 +1797,7 @@ int cg_from_host_bf16_as_f32(cg_backend *b, const uint16_t *bits, size_t len, co
 // end <= 2^24 that is the integer iota produced here.  Larger ends are rejected
 // rather than reproducing the reference's rounding artefacts.
 int cg_arange(cg_backend *b, size_t end, cg_tensor **out) {
+    Enter entered(b);
     if (!b || !out) return fail(CG_ERR_ARG, "null argument");
     if (end > (1u << 24)) return fail(CG_ERR_UNSUPPORTED, "arange: end above 2^24 is inexact in the reference");
     int64_t d[1] = {(int64_t)end};
@@ -1848,6 +1879,7 @@ static int copy_out(cg_backend *b, const cg_tensor *t, void *dst, size_t len) {
 
 // ndarray.rs:50-58.  Non-contiguous views are materialised first (the reference panics).
 int cg_to_host(cg_backend *b, const cg_tensor *t, void *dst, size_t len) {
+    Enter entered(b);
     if (!b || !t || (!dst && len)) return fail(CG_ERR_ARG, "null argument");
     if ((int64_t)len != numel(t)) return fail(CG_ERR_SHAPE, "to_vec: length mismatch");
     CG_HIP(hipSetDevice(b->device));
@@ -1864,6 +1896,7 @@ static int read_flag(cg_backend *b, int *out) {
 
 // ndarray.rs:140-149
 int cg_to_bool(cg_backend *b, const cg_tensor *t, int *out) {
+    Enter entered(b);
     if (!b || !t || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(t->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
     CG_HIP(hipSetDevice(b->device));
@@ -1884,6 +1917,7 @@ int cg_to_bool(cg_backend *b, const cg_tensor *t, int *out) {
 
 // ndarray.rs:534-541
 int cg_compare(cg_backend *b, const cg_tensor *x, const cg_tensor *y, int *out) {
+    Enter entered(b);
     if (!b || !x || !y || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt) || !supported(y->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
     if (x->dt != y->dt) return fail(CG_ERR_DTYPE, "compare: dtype mismatch");
@@ -1908,6 +1942,7 @@ int cg_compare(cg_backend *b, const cg_tensor *x, const cg_tensor *y, int *out) 
 
 // ndarray.rs:60-69 — free-form debug rendering: dtype, shape and the first 16 elements.
 int cg_format_tensor(cg_backend *b, const cg_tensor *t, char *buf, size_t cap) {
+    Enter entered(b);
     if (!b || !t || !buf || !cap) return fail(CG_ERR_ARG, "null argument");
     CG_HIP(hipSetDevice(b->device));
     size_t n = (size_t)numel(t);
@@ -1955,6 +1990,7 @@ static int ew_result(cg_backend *b, int op, cg_dtype compute_dt, cg_dtype out_dt
 
 // ndarray.rs:151-174
 int cg_cast(cg_backend *b, cg_tensor *x, cg_dtype target, cg_tensor **out) {
+    Enter entered(b);
     Consume cx(x);
     if (!b || !x || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(target) || !supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
@@ -1975,6 +2011,7 @@ int cg_cast(cg_backend *b, cg_tensor *x, cg_dtype target, cg_tensor **out) {
 
 // ndarray.rs:352-407, 630-648
 int cg_unary(cg_backend *b, cg_unary_op op, cg_tensor *x, cg_tensor **out) {
+    Enter entered(b);
     Consume cx(x);
     if (!b || !x || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
@@ -1995,6 +2032,7 @@ int cg_unary(cg_backend *b, cg_unary_op op, cg_tensor *x, cg_tensor **out) {
 
 // ndarray.rs:185-323, 598-654
 int cg_binary(cg_backend *b, cg_binary_op op, cg_tensor *x, cg_tensor *y, cg_tensor **out) {
+    Enter entered(b);
     Consume cx(x), cy(y);
     if (!b || !x || !y || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt) || !supported(y->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
@@ -2017,6 +2055,7 @@ int cg_binary(cg_backend *b, cg_binary_op op, cg_tensor *x, cg_tensor *y, cg_ten
 
 // ndarray.rs:325-350
 int cg_where(cg_backend *b, cg_tensor *mask, cg_tensor *x, cg_tensor *y, cg_tensor **out) {
+    Enter entered(b);
     Consume cm(mask), cx(x), cy(y);
     if (!b || !mask || !x || !y || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
@@ -2030,6 +2069,7 @@ int cg_where(cg_backend *b, cg_tensor *mask, cg_tensor *x, cg_tensor *y, cg_tens
 // ---- contraction / reductions ---------------------------------------------------------------------
 // ndarray.rs:176-183, 750-816
 int cg_matmul(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **out) {
+    Enter entered(b);
     Consume cx(x), cy(y);
     if (!b || !x || !y || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt) || !supported(y->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
@@ -2130,6 +2170,7 @@ int cg_matmul(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **out) {
 }
 
 static int reduce_entry(cg_backend *b, int kind, const char *what, cg_tensor *x, cg_tensor **out) {
+    Enter entered(b);
     Consume cx(x);
     if (!b || !x || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
@@ -2176,6 +2217,7 @@ int cg_argmax(cg_backend *b, cg_tensor *x, cg_tensor **out) { return reduce_entr
 
 // ndarray.rs:436-446, 696-721
 int cg_topk(cg_backend *b, cg_tensor *x, size_t k, cg_tensor **values, cg_tensor **indices) {
+    Enter entered(b);
     Consume cx(x);
     if (!b || !x || !values || !indices) return fail(CG_ERR_ARG, "null argument");
     if (x->dt == CG_U32) return fail(CG_ERR_DTYPE, "Unsupported type for topk");
@@ -2214,6 +2256,7 @@ int cg_topk(cg_backend *b, cg_tensor *x, size_t k, cg_tensor **values, cg_tensor
 // ---- shape and indexing ---------------------------------------------------------------------------
 // ndarray.rs:448-455, 553-559 — a stride-0 view; the reference materialises.
 int cg_broadcast(cg_backend *b, cg_tensor *x, const size_t *dims, size_t rank, cg_tensor **out) {
+    Enter entered(b);
     Consume cx(x);
     if (!b || !x || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
@@ -2271,6 +2314,7 @@ int cg_broadcast(cg_backend *b, cg_tensor *x, const size_t *dims, size_t rank, c
 
 // ndarray.rs:504-511, 545-551 — a view when the strides allow it, else one row-major copy.
 int cg_reshape(cg_backend *b, cg_tensor *x, const size_t *dims, size_t rank, cg_tensor **out) {
+    Enter entered(b);
     Consume cx(x);
     if (!b || !x || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
@@ -2352,6 +2396,7 @@ int cg_reshape(cg_backend *b, cg_tensor *x, const size_t *dims, size_t rank, cg_
 
 // ndarray.rs:457-464, 561-569
 int cg_transpose(cg_backend *b, cg_tensor *x, size_t dim0, size_t dim1, cg_tensor **out) {
+    Enter entered(b);
     Consume cx(x);
     if (!b || !x || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
@@ -2378,6 +2423,7 @@ int cg_transpose(cg_backend *b, cg_tensor *x, size_t dim0, size_t dim1, cg_tenso
 
 // ndarray.rs:489-502, 581-588
 int cg_slice(cg_backend *b, cg_tensor *x, size_t dim, size_t start, size_t len, cg_tensor **out) {
+    Enter entered(b);
     Consume cx(x);
     if (!b || !x || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
@@ -2408,6 +2454,7 @@ int cg_slice(cg_backend *b, cg_tensor *x, size_t dim, size_t start, size_t len, 
 
 // ndarray.rs:513-532, 590-596 — two strided copies into the halves of a fresh tensor.
 int cg_concat(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor **out) {
+    Enter entered(b);
     Consume cx(x), cy(y);
     if (!b || !x || !y || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt) || !supported(y->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
@@ -2591,6 +2638,7 @@ int cg_concat(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor *
 // ndarray.rs:466-487, 571-579 — gather; out-of-range indices are detected by the kernel
 // and reported by the next call that waits for the device.
 int cg_index(cg_backend *b, cg_tensor *x, size_t dim, cg_tensor *indices, cg_tensor **out) {
+    Enter entered(b);
     Consume cx(x), ci(indices);
     if (!b || !x || !indices || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);

@@ -29,6 +29,11 @@
  *    cg_to_host, cg_to_bool, cg_compare, cg_format_tensor and cg_sync wait
  *    for the device.  Device-detected faults (gather index out of range,
  *    u32 division by zero) are reported by the next waiting call.
+ *  - Threads: handles may be cloned, sent to and used from any thread
+ *    (`BackendTensorOps: Send + Sync`, mod.rs:124); calls on one backend are
+ *    serialised by a lock inside the library, so concurrent callers are
+ *    safe but do not overlap.  cg_backend_destroy must not race with
+ *    anything.
  *  - dims/shape arrays are row-major extents as size_t; rank 0 and zero
  *    extents are legal.  Maximum rank: CG_MAX_RANK.
  */

@@ -175,6 +175,44 @@ def test_backend_closes_with_writes_still_waiting():
     be.close()
 
 
+def test_one_backend_from_several_threads(hip):
+    """Handles are `Send + Sync` in the reference (backend/mod.rs:124): several threads use one backend and
+    shared input tensors at once — deferred programs, lazy products, appended rows, read-backs — and each gets
+    the values it would get alone."""
+    import threading
+
+    rng = np.random.default_rng(11)
+    w = (rng.standard_normal((4096, 512)) * 0.02).astype(np.float32)
+    tw = hip.from_numpy(w)
+    errors = []
+
+    def work(seed):
+        try:
+            r = np.random.default_rng(seed)
+            for it in range(12):
+                x = np.abs(r.standard_normal((4, 1, 512)).astype(np.float32))
+                tx = hip.from_numpy(x)
+                y = hip.matmul(tx, hip.broadcast(hip.transpose(tw, 0, 1), (4, 512, 4096)))
+                z = hip.exp(hip.neg(hip.mul(y, y)))
+                cache = hip.from_numpy(np.zeros((2, 2, 300, 64), np.float32))
+                rows = hip.add(hip.from_numpy(np.full((2, 2, 1, 64), float(seed), np.float32)),
+                               hip.from_numpy(np.full((2, 2, 1, 64), float(it), np.float32)))
+                cache = hip.concat(cache.move(), rows.move(), 2)
+                got_z, got_c = hip.to_numpy(z), hip.to_numpy(cache)
+                yy = x.astype(np.float64) @ w.astype(np.float64).T
+                np.testing.assert_allclose(got_z, np.exp(-(yy * yy)), rtol=2e-3, atol=1e-6)
+                assert got_c.shape == (2, 2, 301, 64) and np.all(got_c[:, :, 300] == seed + it) and not got_c[:, :, :300].any()
+        except Exception as e:  # noqa: BLE001 - reported by the main thread
+            errors.append(repr(e))
+
+    threads = [threading.Thread(target=work, args=(s,)) for s in range(1, 5)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert not errors, errors
+
+
 def test_format_tensor(hip):
     s = hip.format_tensor(hip.from_numpy(np.array([[1.5, 2.0]], np.float32)))
     assert "f32[1,2]" in s and "1.5" in s
