@@ -203,7 +203,9 @@ class Backend:
             return self.ndarray_from_vec_f32(arr, arr.shape)
         if arr.dtype == np.uint32:
             return self.ndarray_from_vec_u32(arr, arr.shape)
-        raise TypeError(f"unsupported dtype {arr.dtype}")
+        if arr.dtype == np.float16:
+            return self.ndarray_from_vec_f16(arr, arr.shape)
+        raise TypeError(f"unsupported dtype {arr.dtype} (bfloat16: ndarray_from_vec_bf16 with uint16 bit patterns)")
 
     def arange(self, end: int) -> Tensor:
         return self._op(lambda b, o: self._lib.cg_arange(b, end, o))
@@ -212,7 +214,8 @@ class Backend:
     def to_vec(self, x: Tensor) -> np.ndarray:
         """`Backend::to_vec`: flat row-major contents."""
         n = int(self._lib.cg_tensor_numel(x._h))
-        out = np.empty(n, dtype=np.float32 if x.dtype == A.F32 else np.uint32)
+        # f16 as numpy float16; bf16 as its uint16 bit patterns (numpy has no bfloat16): `bits << 16` is the f32 value
+        out = np.empty(n, dtype={A.F32: np.float32, A.F16: np.float16, A.BF16: np.uint16}.get(x.dtype, np.uint32))
         self._check(self._lib.cg_to_host(self._b, x._h, out.ctypes.data_as(C.c_void_p), n))
         return out
 

@@ -167,6 +167,11 @@ struct cg_tensor {
 
 namespace cg {
 
+// Floating-point dtypes: the arithmetic is f32 on 32-bit words; CG_F16 / CG_BF16 results are rounded
+// to their 16-bit format after every op (the words always hold exactly representable values).
+inline bool is_f(cg_dtype d) { return d == CG_F32 || d == CG_F16 || d == CG_BF16; }
+inline bool is_half(cg_dtype d) { return d == CG_F16 || d == CG_BF16; }
+
 inline int64_t numel(const cg_tensor *t) {
     int64_t n = 1;
     for (int i = 0; i < t->rank; i++) n *= t->dims[i];
@@ -338,6 +343,9 @@ void prof_drain(cg_backend *be);
 enum EwOp : int {
     // unary (CG_NEG.. order of cg_unary_op)
     kNeg = 0, kSin, kCos, kExp, kLog, kFloor, kRound,
+    // f32 -> nearest bfloat16 / binary16 value (ties to even), still held as f32: how results of the
+    // 16-bit float dtypes are rounded (every tensor is stored as 32-bit words)
+    kRoundBF16, kRoundF16,
     // binary (order of cg_binary_op) offset by 16
     kAdd = 16, kSub, kMul, kDiv, kPow, kLt, kGt, kGte, kLte, kEq,
     kWhere = 32,
@@ -364,6 +372,10 @@ int launch_arange(cg_backend *be, cg_tensor *out);
 int launch_fill_word(cg_backend *be, void *ptr, uint32_t bits);
 // dst[i] = (uint32_t)src[i] << 16 : bfloat16 bit patterns widened to f32
 int launch_bf16_widen(cg_backend *be, const void *src, void *dst, uint64_t n);
+// binary16 bit patterns widened to f32
+int launch_f16_widen(cg_backend *be, const void *src, void *dst, uint64_t n);
+// f32 words holding bfloat16 / binary16 values -> their 16-bit patterns (exact)
+int launch_narrow16(cg_backend *be, cg_dtype dt, const void *src, void *dst, uint64_t n);
 // out[outer, j, inner] = x[outer, idx[j], inner]
 int launch_gather(cg_backend *be, const cg_tensor *x, int dim, const cg_tensor *idx, cg_tensor *out);
 

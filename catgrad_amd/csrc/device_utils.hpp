@@ -1,5 +1,6 @@
 // Device-side helpers shared by the kernel files.
 #pragma once
+#include <hip/hip_fp16.h>
 #include "common.hpp"
 
 namespace cg {
@@ -74,6 +75,12 @@ __device__ __forceinline__ uint32_t wrapping_pow(uint32_t a, uint32_t e) {
     return acc;
 }
 
+// f32 bits -> bits of the nearest bfloat16 value (ties to even), as f32; NaNs stay NaNs (quiet)
+__host__ __device__ __forceinline__ uint32_t round_bf16_bits(uint32_t u) {
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (u | 0x00400000u) & 0xFFFF0000u;
+    return (u + 0x7FFFu + ((u >> 16) & 1u)) & 0xFFFF0000u;
+}
+
 // One scalar application of OP on raw 32-bit words.  F = operands are f32.
 template <int OP, bool F>
 __device__ __forceinline__ uint32_t apply(uint32_t a, uint32_t b, uint32_t c, uint32_t *fault) {
@@ -93,6 +100,8 @@ __device__ __forceinline__ uint32_t apply(uint32_t a, uint32_t b, uint32_t c, ui
         if constexpr (OP == kLog) return asu(logf(x));
         if constexpr (OP == kFloor) return asu(floorf(x));
         if constexpr (OP == kRound) return asu(rintf(x)); // ties to even (ndarray.rs:646-648)
+        if constexpr (OP == kRoundBF16) return round_bf16_bits(a);
+        if constexpr (OP == kRoundF16) return asu(__half2float(__float2half_rn(x))); // v_cvt_f16_f32: nearest even, overflow -> inf
         if constexpr (OP == kAdd) return asu(x + y);
         if constexpr (OP == kSub) return asu(x - y);
         if constexpr (OP == kMul) return asu(x * y);

@@ -114,7 +114,7 @@ template <int OP, bool F, int NIN> int launch_variants(cg_backend *be, const EwA
 }
 
 template <int OP, int NIN> int launch_by_dtype(cg_backend *be, cg_dtype dt, const EwArgs &a) {
-    return dt == CG_F32 ? launch_variants<OP, true, NIN>(be, a) : launch_variants<OP, false, NIN>(be, a);
+    return is_f(dt) ? launch_variants<OP, true, NIN>(be, a) : launch_variants<OP, false, NIN>(be, a);
 }
 
 __global__ void arange_kernel(uint32_t *out, uint32_t n) {
@@ -199,6 +199,8 @@ int launch_elementwise(cg_backend *be, int op, cg_dtype dt, const cg_tensor *out
     case kLog: return launch_variants<kLog, true, 1>(be, a);
     case kFloor: return launch_variants<kFloor, true, 1>(be, a);
     case kRound: return launch_variants<kRound, true, 1>(be, a);
+    case kRoundBF16: return launch_variants<kRoundBF16, true, 1>(be, a);
+    case kRoundF16: return launch_variants<kRoundF16, true, 1>(be, a);
     CG_EW2(kAdd) CG_EW2(kSub) CG_EW2(kMul) CG_EW2(kDiv) CG_EW2(kPow)
     CG_EW2(kLt) CG_EW2(kGt) CG_EW2(kGte) CG_EW2(kLte) CG_EW2(kEq)
     case kWhere: return launch_by_dtype<kWhere, 3>(be, dt, a);
@@ -227,6 +229,39 @@ int launch_bf16_widen(cg_backend *be, const void *src, void *dst, uint64_t n) {
                        static_cast<uint32_t *>(dst), n);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? CG_OK : hip_fail(e, "bf16 widen launch");
+}
+
+__global__ __launch_bounds__(kBlock) void f16_widen_kernel(const uint16_t *src, uint32_t *dst, uint64_t n) {
+    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (uint64_t)gridDim.x * kBlock)
+        dst[i] = asu(__half2float(__ushort_as_half(src[i])));
+}
+// BF16: the upper halves; else binary16 conversion (exact: the words hold representable values)
+template <bool BF16> __global__ __launch_bounds__(kBlock) void narrow16_kernel(const uint32_t *src, uint16_t *dst, uint64_t n) {
+    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (uint64_t)gridDim.x * kBlock)
+        dst[i] = BF16 ? (uint16_t)(src[i] >> 16) : __half_as_ushort(__float2half_rn(asf(src[i])));
+}
+
+int launch_f16_widen(cg_backend *be, const void *src, void *dst, uint64_t n) {
+    if (n == 0) return CG_OK;
+    const uint32_t blocks = (uint32_t)std::min<uint64_t>((n + kBlock - 1) / kBlock, 16384);
+    hipLaunchKernelGGL(f16_widen_kernel, dim3(blocks), dim3(kBlock), 0, be->stream, static_cast<const uint16_t *>(src),
+                       static_cast<uint32_t *>(dst), n);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CG_OK : hip_fail(e, "f16 widen launch");
+}
+
+int launch_narrow16(cg_backend *be, cg_dtype dt, const void *src, void *dst, uint64_t n) {
+    if (n == 0) return CG_OK;
+    if (int frc = flush_deferred(be)) return frc;
+    const uint32_t blocks = (uint32_t)std::min<uint64_t>((n + kBlock - 1) / kBlock, 16384);
+    if (dt == CG_BF16)
+        hipLaunchKernelGGL((narrow16_kernel<true>), dim3(blocks), dim3(kBlock), 0, be->stream, static_cast<const uint32_t *>(src),
+                           static_cast<uint16_t *>(dst), n);
+    else
+        hipLaunchKernelGGL((narrow16_kernel<false>), dim3(blocks), dim3(kBlock), 0, be->stream, static_cast<const uint32_t *>(src),
+                           static_cast<uint16_t *>(dst), n);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CG_OK : hip_fail(e, "16-bit narrowing launch");
 }
 
 int launch_fill_word(cg_backend *be, void *ptr, uint32_t bits) {

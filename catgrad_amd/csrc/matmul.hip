@@ -879,7 +879,7 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
     const bool b_nfast = !(a.b_sk == 1 || K == 1) && a.b_sn == 1;
 
     if (batch > 65535) return fail(CG_ERR_UNSUPPORTED, "matmul: more than 65535 batch entries after folding");
-    const bool f32 = x->dt == CG_F32;
+    const bool f32 = is_f(x->dt);
     hipStream_t s = be->stream;
     const double flop = 2.0 * (double)M * (double)N * (double)K * (double)batch;
     const double bytes = distinct_bytes(x) + distinct_bytes(y) + distinct_bytes(out);

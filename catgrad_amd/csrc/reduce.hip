@@ -351,7 +351,7 @@ int launch_reduce(cg_backend *be, int kind, const cg_tensor *x, cg_tensor *out) 
     int rc = fill_rows_args(x, &a);
     if (rc) return rc;
     a.out = static_cast<uint32_t *>(out->buf->ptr);
-    bool f = x->dt == CG_F32;
+    bool f = is_f(x->dt);
     ProfScope prof(be, CG_K_REDUCE, distinct_bytes(x) + distinct_bytes(out));
     switch (kind) {
     case kSum: return f ? launch_rows<kSum, true>(be, a) : launch_rows<kSum, false>(be, a);
@@ -387,7 +387,7 @@ static int launch_any(cg_backend *be, int mode, const cg_tensor *x, const cg_ten
     a.y = ops[1];
     a.flag = be->flag_dev;
     dim3 grid((uint32_t)((a.g.total + kBlock - 1) / kBlock)), block(kBlock);
-    bool f = x->dt == CG_F32;
+    bool f = is_f(x->dt);
 #define CG_ANY(MODE, F, VEC) hipLaunchKernelGGL((any_kernel<MODE, F, VEC>), grid, block, 0, be->stream, a)
     if (mode == 0) {
         if (a.g.vec == 4) { if (f) CG_ANY(0, true, 4); else CG_ANY(0, false, 4); }

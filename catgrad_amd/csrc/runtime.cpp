@@ -465,8 +465,40 @@ struct Consume { // the consumed reference of a tensor argument (move semantics 
     ~Consume() { release(t); }
 };
 
-static const char *kTodo = "f16, bf16, and fp8 are not supported (todo!() in the reference NdArrayBackend)";
-static bool supported(cg_dtype d) { return d == CG_F32 || d == CG_U32; }
+static const char *kTodo = "fp8 is not supported (todo!() in the reference NdArrayBackend)";
+static bool supported(cg_dtype d) { return d == CG_F32 || d == CG_U32 || d == CG_F16 || d == CG_BF16; }
+
+// The 16-bit float dtypes on the host (constants that never reach the device): widening of a bit pattern
+// and rounding of an f32 to the nearest representable value (ties to even), both as f32 bits.
+static uint32_t widen16_host(cg_dtype dt, uint16_t h) {
+    if (dt == CG_BF16) return (uint32_t)h << 16;
+    _Float16 v;
+    memcpy(&v, &h, 2);
+    float f = (float)v;
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    return u;
+}
+static uint32_t round16_host(cg_dtype dt, uint32_t u) {
+    if (dt == CG_BF16) {
+        if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (u | 0x00400000u) & 0xFFFF0000u;
+        return (u + 0x7FFFu + ((u >> 16) & 1u)) & 0xFFFF0000u;
+    }
+    float f;
+    memcpy(&f, &u, 4);
+    f = (float)(_Float16)f;
+    memcpy(&u, &f, 4);
+    return u;
+}
+static uint16_t narrow16_host(cg_dtype dt, uint32_t u) {
+    if (dt == CG_BF16) return (uint16_t)(u >> 16);
+    float f;
+    memcpy(&f, &u, 4);
+    _Float16 v = (_Float16)f;
+    uint16_t h;
+    memcpy(&h, &v, 2);
+    return h;
+}
 
 static bool same_shape(const cg_tensor *a, const cg_tensor *b) {
     if (a->rank != b->rank) return false;
@@ -1296,7 +1328,7 @@ static uint32_t f_bits(float f) {
 // Exactly-rounded scalar ops are folded on the host when every operand is uniform
 // (IEEE add/sub/mul/div and comparisons give the same bits on host and device).
 static bool fold_binary(int op, cg_dtype dt, uint32_t a, uint32_t b, uint32_t *r, bool *divzero) {
-    if (dt == CG_F32) {
+    if (is_f(dt)) {
         float x = bits_f(a), y = bits_f(b);
         switch (op) {
         case CG_ADD: *r = f_bits(x + y); return true;
@@ -1737,7 +1769,13 @@ int cg_from_host(cg_backend *b, cg_dtype dtype, const void *data, size_t len, co
     if (n && !data) return fail(CG_ERR_ARG, "null data");
     if (n == 1) {
         uint32_t bits;
-        memcpy(&bits, data, 4);
+        if (is_half(dtype)) {
+            uint16_t h;
+            memcpy(&h, data, 2);
+            bits = widen16_host(dtype, h);
+        } else {
+            memcpy(&bits, data, 4);
+        }
         *out = new_uniform(b, dtype, d, (int)rank, bits);
         return CG_OK;
     }
@@ -1746,7 +1784,18 @@ int cg_from_host(cg_backend *b, cg_dtype dtype, const void *data, size_t len, co
     if (rc) return rc;
     if (n) {
         CG_HIP(hipSetDevice(b->device));
-        rc = staged_upload(b, t->buf->ptr, data, n * 4);
+        if (is_half(dtype)) { // 2-byte elements: uploaded as they are, widened to 32-bit words on the device
+            void *tmp = nullptr;
+            size_t cls = 0;
+            rc = b->pool.alloc(n * 2, &tmp, &cls);
+            if (!rc) {
+                rc = staged_upload(b, tmp, data, n * 2);
+                if (!rc) rc = dtype == CG_BF16 ? launch_bf16_widen(b, tmp, t->buf->ptr, n) : launch_f16_widen(b, tmp, t->buf->ptr, n);
+                b->pool.free(tmp, cls); // stream-ordered: later users queue behind the widening kernel
+            }
+        } else {
+            rc = staged_upload(b, t->buf->ptr, data, n * 4);
+        }
         if (rc) {
             release(t);
             return rc;
@@ -1883,6 +1932,39 @@ int cg_to_host(cg_backend *b, const cg_tensor *t, void *dst, size_t len) {
     if (!b || !t || (!dst && len)) return fail(CG_ERR_ARG, "null argument");
     if ((int64_t)len != numel(t)) return fail(CG_ERR_SHAPE, "to_vec: length mismatch");
     CG_HIP(hipSetDevice(b->device));
+    if (is_half(t->dt) && len > 0) {
+        // 2-byte elements out: the words are narrowed on the device (exact), then copied
+        uint16_t *d16 = static_cast<uint16_t *>(dst);
+        if (t->uniform) {
+            const uint16_t h = narrow16_host(t->dt, t->ubits);
+            for (size_t i = 0; i < len; i++) d16[i] = h;
+            return wait_and_check(b);
+        }
+        int rc = ensure_concrete(const_cast<cg_tensor *>(t));
+        if (rc) return rc;
+        cg_tensor *tmp = nullptr;
+        const cg_tensor *src = t;
+        if (!is_contiguous(t)) {
+            rc = materialize(b, t, &tmp);
+            if (rc) return rc;
+            src = tmp;
+        }
+        const void *p;
+        void *half = nullptr;
+        size_t cls = 0;
+        rc = device_ptr(src, &p);
+        if (!rc) rc = b->pool.alloc(len * 2, &half, &cls);
+        if (!rc) {
+            rc = launch_narrow16(b, t->dt, p, half, len);
+            if (!rc) {
+                hipError_t e = hipMemcpyAsync(dst, half, len * 2, hipMemcpyDeviceToHost, b->stream);
+                rc = e == hipSuccess ? wait_and_check(b) : hip_fail(e, "device to host copy");
+            }
+            b->pool.free(half, cls);
+        }
+        release(tmp);
+        return rc;
+    }
     return copy_out(b, t, dst, len);
 }
 
@@ -1905,7 +1987,7 @@ int cg_to_bool(cg_backend *b, const cg_tensor *t, int *out) {
         return wait_and_check(b);
     }
     if (t->uniform) {
-        *out = t->dt == CG_F32 ? bits_f(t->ubits) > 0.0f : t->ubits != 0;
+        *out = is_f(t->dt) ? bits_f(t->ubits) > 0.0f : t->ubits != 0;
         return wait_and_check(b);
     }
     int rc = ensure_concrete(const_cast<cg_tensor *>(t));
@@ -1947,15 +2029,15 @@ int cg_format_tensor(cg_backend *b, const cg_tensor *t, char *buf, size_t cap) {
     CG_HIP(hipSetDevice(b->device));
     size_t n = (size_t)numel(t);
     std::vector<uint32_t> host(n);
-    int rc = copy_out(b, t, host.data(), n);
+    int rc = copy_out(b, t, host.data(), n); // the 32-bit words, whatever the dtype
     if (rc) return rc;
-    std::string s = t->dt == CG_F32 ? "f32[" : "u32[";
+    std::string s = t->dt == CG_F32 ? "f32[" : t->dt == CG_F16 ? "f16[" : t->dt == CG_BF16 ? "bf16[" : "u32[";
     for (int i = 0; i < t->rank; i++) s += (i ? "," : "") + std::to_string(t->dims[i]);
     s += "] [";
     size_t shown = std::min<size_t>(n, 16);
     char tmp[48];
     for (size_t i = 0; i < shown; i++) {
-        if (t->dt == CG_F32)
+        if (is_f(t->dt))
             snprintf(tmp, sizeof tmp, "%s%.9g", i ? ", " : "", bits_f(host[i]));
         else
             snprintf(tmp, sizeof tmp, "%s%u", i ? ", " : "", host[i]);
@@ -1988,7 +2070,35 @@ static int ew_result(cg_backend *b, int op, cg_dtype compute_dt, cg_dtype out_dt
     return CG_OK;
 }
 
-// ndarray.rs:151-174
+// Results of the 16-bit float dtypes: the f32 value just computed is rounded to the dtype (one more
+// deferred instruction, or on the host for a constant).  Takes over the reference in *io.
+static int round_result(cg_backend *b, cg_dtype dt, cg_tensor **io) {
+    if (!is_half(dt)) return CG_OK;
+    cg_tensor *x = *io;
+    *io = nullptr;
+    int rc = CG_OK;
+    if (x->uniform) {
+        *io = new_uniform(b, dt, x->dims, x->rank, round16_host(dt, x->ubits));
+    } else {
+        const cg_tensor *ins[1] = {x};
+        rc = ew_result(b, dt == CG_BF16 ? kRoundBF16 : kRoundF16, dt, dt, x, ins, 1, io);
+    }
+    release(x);
+    return rc;
+}
+
+// The same tensor under another floating-point dtype tag (its words already hold values of that dtype).
+static int retag(cg_backend *b, cg_tensor *x, cg_dtype target, cg_tensor **out) {
+    if (x->uniform) {
+        *out = new_uniform(b, target, x->dims, x->rank, x->ubits);
+        return CG_OK;
+    }
+    const cg_tensor *ins[1] = {x};
+    return ew_result(b, kCopy, CG_F32, target, x, ins, 1, out); // deferred: a view once it is needed
+}
+
+// ndarray.rs:151-174; the 16-bit float dtypes as candle.rs:575-599 (`to_dtype`): widening is exact,
+// narrowing rounds to nearest even, u32 goes through f32 on the way.
 int cg_cast(cg_backend *b, cg_tensor *x, cg_dtype target, cg_tensor **out) {
     Enter entered(b);
     Consume cx(x);
@@ -1999,14 +2109,21 @@ int cg_cast(cg_backend *b, cg_tensor *x, cg_dtype target, cg_tensor **out) {
         *out = x;
         return CG_OK;
     }
+    CG_HIP(hipSetDevice(b->device));
+    if (is_f(x->dt) && is_f(target)) {
+        // between floating-point dtypes: the words stay, a narrower target rounds them
+        int rc = retag(b, x, target, out);
+        const bool exact = target == CG_F32; // f16 <-> bf16 round too: neither contains the other
+        return rc || exact ? rc : round_result(b, target, out);
+    }
     if (x->uniform) {
         uint32_t r = target == CG_U32 ? f32_as_u32_host(bits_f(x->ubits)) : f_bits((float)x->ubits);
         *out = new_uniform(b, target, x->dims, x->rank, r);
-        return CG_OK;
+        return round_result(b, target, out);
     }
-    CG_HIP(hipSetDevice(b->device));
     const cg_tensor *ins[1] = {x};
-    return ew_result(b, target == CG_U32 ? kCastF2U : kCastU2F, x->dt, target, x, ins, 1, out);
+    int rc = ew_result(b, target == CG_U32 ? kCastF2U : kCastU2F, x->dt, target, x, ins, 1, out);
+    return rc ? rc : round_result(b, target, out);
 }
 
 // ndarray.rs:352-407, 630-648
@@ -2021,13 +2138,17 @@ int cg_unary(cg_backend *b, cg_unary_op op, cg_tensor *x, cg_tensor **out) {
         return fail(CG_ERR_DTYPE, "Invalid input types for %s", names[op]);
     }
     if (x->uniform && op == CG_NEG) {
-        uint32_t r = x->dt == CG_F32 ? (x->ubits ^ 0x80000000u) : (0u - x->ubits);
+        uint32_t r = is_f(x->dt) ? (x->ubits ^ 0x80000000u) : (0u - x->ubits);
         *out = new_uniform(b, x->dt, x->dims, x->rank, r);
         return CG_OK;
     }
     CG_HIP(hipSetDevice(b->device));
     const cg_tensor *ins[1] = {x};
-    return ew_result(b, kNeg + (int)op, x->dt, x->dt, x, ins, 1, out);
+    const cg_dtype dt = x->dt;
+    int rc = ew_result(b, kNeg + (int)op, dt, dt, x, ins, 1, out);
+    // neg, floor and round of a representable value are representable; the others round
+    const bool exact = op == CG_NEG || op == CG_FLOOR || op == CG_ROUND;
+    return rc || exact ? rc : round_result(b, dt, out);
 }
 
 // ndarray.rs:185-323, 598-654
@@ -2044,13 +2165,16 @@ int cg_binary(cg_backend *b, cg_binary_op op, cg_tensor *x, cg_tensor *y, cg_ten
         bool divzero = false;
         if (fold_binary(op, x->dt, x->ubits, y->ubits, &r, &divzero)) {
             if (divzero) return fail(CG_ERR_RANGE, "attempt to divide by zero");
-            *out = new_uniform(b, x->dt, x->dims, x->rank, r);
+            *out = new_uniform(b, x->dt, x->dims, x->rank, is_half(x->dt) ? round16_host(x->dt, r) : r);
             return CG_OK;
         }
     }
     CG_HIP(hipSetDevice(b->device));
     const cg_tensor *ins[2] = {x, y};
-    return ew_result(b, kAdd + (int)op, x->dt, x->dt, x, ins, 2, out);
+    const cg_dtype dt = x->dt;
+    int rc = ew_result(b, kAdd + (int)op, dt, dt, x, ins, 2, out);
+    const bool exact = op >= CG_LT; // comparisons give 0 or 1
+    return rc || exact ? rc : round_result(b, dt, out);
 }
 
 // ndarray.rs:325-350
@@ -2068,8 +2192,15 @@ int cg_where(cg_backend *b, cg_tensor *mask, cg_tensor *x, cg_tensor *y, cg_tens
 
 // ---- contraction / reductions ---------------------------------------------------------------------
 // ndarray.rs:176-183, 750-816
+static int matmul_entry(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **out);
+// The 16-bit float dtypes: products of exactly held values, summed in f32, rounded once.
 int cg_matmul(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **out) {
     Enter entered(b);
+    const cg_dtype dt = x ? x->dt : CG_F32;
+    int rc = matmul_entry(b, x, y, out);
+    return rc ? rc : round_result(b, dt, out);
+}
+static int matmul_entry(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **out) {
     Consume cx(x), cy(y);
     if (!b || !x || !y || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt) || !supported(y->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
@@ -2194,7 +2325,7 @@ static int reduce_entry(cg_backend *b, int kind, const char *what, cg_tensor *x,
                                  (x->pend->ins[0].op & ~kInstrU32) == kCopy && !x->pend->leaf[0].pw && !x->pend->leaf[0].uniform;
         if (x->pend && !only_a_view && x->pend->nred == 0 && (x->rc.load() == 1 || cheap(x->pend))) {
             rc = resolve_lazy_leaves(b, *x->pend);
-            if (!rc) rc = launch_fused_reduce(b, kind, x->dt == CG_F32, *x->pend, x->pend->ninstr, x->dims, x->rank, o);
+            if (!rc) rc = launch_fused_reduce(b, kind, is_f(x->dt), *x->pend, x->pend->ninstr, x->dims, x->rank, o);
         } else {
             rc = ensure_concrete(x);
             if (!rc) rc = launch_reduce(b, kind, x, o);
@@ -2208,10 +2339,21 @@ static int reduce_entry(cg_backend *b, int kind, const char *what, cg_tensor *x,
     return CG_OK;
 }
 
-// ndarray.rs:418-425, 723-730
-int cg_sum(cg_backend *b, cg_tensor *x, cg_tensor **out) { return reduce_entry(b, kSum, "sum", x, out); }
+// ndarray.rs:418-425, 723-730.  The 16-bit float dtypes: summed in f32, rounded once.
+int cg_sum(cg_backend *b, cg_tensor *x, cg_tensor **out) {
+    Enter entered(b);
+    const cg_dtype dt = x ? x->dt : CG_F32;
+    int rc = reduce_entry(b, kSum, "sum", x, out);
+    return rc ? rc : round_result(b, dt, out);
+}
 // ndarray.rs:409-416, 656-668
-int cg_max(cg_backend *b, cg_tensor *x, cg_tensor **out) { return reduce_entry(b, kMax, "max", x, out); }
+int cg_max(cg_backend *b, cg_tensor *x, cg_tensor **out) {
+    Enter entered(b);
+    const cg_dtype dt = x ? x->dt : CG_F32;
+    int rc = reduce_entry(b, kMax, "max", x, out);
+    // exact, except that the seed f32::MIN of an empty or all-NaN row is not a value of the 16-bit dtypes
+    return rc ? rc : round_result(b, dt, out);
+}
 // ndarray.rs:427-434, 670-694
 int cg_argmax(cg_backend *b, cg_tensor *x, cg_tensor **out) { return reduce_entry(b, kArgmax, "argmax", x, out); }
 
@@ -2221,7 +2363,7 @@ int cg_topk(cg_backend *b, cg_tensor *x, size_t k, cg_tensor **values, cg_tensor
     Consume cx(x);
     if (!b || !x || !values || !indices) return fail(CG_ERR_ARG, "null argument");
     if (x->dt == CG_U32) return fail(CG_ERR_DTYPE, "Unsupported type for topk");
-    if (x->dt != CG_F32) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
+    if (!is_f(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
     if (x->rank == 0) return fail(CG_ERR_SHAPE, "topk: rank-0 tensor has no last axis");
     int64_t n = x->dims[x->rank - 1];
     if (n == 0) return fail(CG_ERR_SHAPE, "topk: attempt to divide by zero (empty last axis)");
@@ -2233,7 +2375,7 @@ int cg_topk(cg_backend *b, cg_tensor *x, size_t k, cg_tensor **values, cg_tensor
     cg_tensor *v, *i;
     int rc = ensure_concrete(x);
     if (rc) return rc;
-    rc = new_dense(b, CG_F32, od, x->rank, &v);
+    rc = new_dense(b, x->dt, od, x->rank, &v);
     if (rc) return rc;
     rc = new_dense(b, CG_U32, od, x->rank, &i);
     if (rc) {

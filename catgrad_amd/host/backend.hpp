@@ -128,6 +128,13 @@ class Backend {
     Tensor ndarray_from_vec_u32(const uint32_t *data, size_t len, const Shape &shape) {
         return from_vec(CG_U32, data, len, shape);
     }
+    // mod.rs:36-46: the 16-bit floats cross the boundary as their bit patterns (2 bytes per element).
+    Tensor ndarray_from_vec_f16(const uint16_t *bits, size_t len, const Shape &shape) {
+        return from_vec(CG_F16, bits, len, shape);
+    }
+    Tensor ndarray_from_vec_bf16(const uint16_t *bits, size_t len, const Shape &shape) {
+        return from_vec(CG_BF16, bits, len, shape);
+    }
     // Weight ingest (catgrad-llm/src/utils/mod.rs:158-168): f32 tensor from bfloat16 bit patterns.
     Tensor from_bf16_bits(const uint16_t *bits, size_t len, const Shape &shape) {
         return out([&](cg_tensor **o) {
@@ -218,6 +225,13 @@ class Backend {
     std::vector<uint32_t> to_vec_bits(Tensor x) {
         calls++;
         std::vector<uint32_t> v(x.numel());
+        check(abi_.cg_to_host(b_, x.get(), v.data(), v.size()));
+        return v;
+    }
+    // `to_vec` of an f16 / bf16 tensor: its 16-bit patterns.
+    std::vector<uint16_t> to_vec_bits16(Tensor x) {
+        calls++;
+        std::vector<uint16_t> v(x.numel());
         check(abi_.cg_to_host(b_, x.get(), v.data(), v.size()));
         return v;
     }

@@ -238,7 +238,7 @@ impl HipBackend {
         if st == CG_ERR_SHAPE {
             return Err(BackendError::ShapeError);
         }
-        check(st); // reduced-precision floats: the same todo!() as NdArrayBackend
+        check(st); // fp8: the same todo!() as NdArrayBackend
         Ok(tag_for(&dt, HipTensor(out)))
     }
 }
@@ -387,7 +387,18 @@ impl Backend for HipBackend {
                 check(unsafe { cg_to_host(self.raw(), t.0, v.as_mut_ptr() as *mut c_void, n) });
                 TaggedVec::U32(v)
             }
-            _ => todo!("f16, bf16, and fp8 are not supported by the hip backend"),
+            Dtype::F16 => {
+                // 2-byte elements: half::f16 is repr(transparent) over its u16 bit pattern
+                let mut v = vec![half::f16::ZERO; n];
+                check(unsafe { cg_to_host(self.raw(), t.0, v.as_mut_ptr() as *mut c_void, n) });
+                TaggedVec::F16(v)
+            }
+            Dtype::BF16 => {
+                let mut v = vec![half::bf16::ZERO; n];
+                check(unsafe { cg_to_host(self.raw(), t.0, v.as_mut_ptr() as *mut c_void, n) });
+                TaggedVec::BF16(v)
+            }
+            _ => todo!("fp8 is not supported by the hip backend"),
         }
     }
 

@@ -120,6 +120,13 @@ cg_tensor *new_tensor(cg_dtype dt, const size_t *dims, int rank) {
     return t;
 }
 
+// A freshly computed (standard-layout, unshared) result of a 16-bit float dtype: every word rounded to the dtype.
+uint32_t round_to(cg_dtype dt, uint32_t u);
+void round_tensor(cg_tensor *t) {
+    if (t->dt != CG_F16 && t->dt != CG_BF16) return;
+    for (uint32_t &w : t->st->data) w = round_to(t->dt, w);
+}
+
 void release(cg_tensor *t) {
     if (!t) return;
     if (t->rc.fetch_sub(1) == 1) {
@@ -219,7 +226,66 @@ bool same_shape(const cg_tensor *a, const cg_tensor *b) {
     return true;
 }
 
-bool supported(cg_dtype d) { return d == CG_F32 || d == CG_U32; }
+bool supported(cg_dtype d) { return d == CG_F32 || d == CG_U32 || d == CG_F16 || d == CG_BF16; }
+
+// ---- the 16-bit float dtypes ------------------------------------------------------------------
+// NdArrayBackend has `todo!()` for them (ndarray.rs:7-9, 98-120); what is restated here is the model of
+// the `half` crate that CandleBackend's CPU path builds on (candle.rs:530-551, 575-599, 605-718): a value
+// is widened to f32 exactly, the op runs in f32, the result is rounded to the dtype (nearest, ties to even;
+// overflow to infinity; NaN stays NaN).  Sums and matrix products accumulate in f32 and round once: Candle's
+// own accumulation order and width are NOT restated (PARITY UNPINNED for those two; conversions and
+// element-wise results are pinned by numpy's float16 and by the closed form of bfloat16 rounding).
+// Tensors of these dtypes hold 32-bit words whose values are exactly representable in the dtype.
+bool isf(cg_dtype d) { return d == CG_F32 || d == CG_F16 || d == CG_BF16; }
+bool is_half(cg_dtype d) { return d == CG_F16 || d == CG_BF16; }
+
+uint32_t bits_of(float f) {
+    uint32_t u;
+    memcpy(&u, &f, 4);
+    return u;
+}
+float float_of(uint32_t u) {
+    float f;
+    memcpy(&f, &u, 4);
+    return f;
+}
+
+uint16_t f32_to_bf16_bits(uint32_t u) {
+    if ((u & 0x7FFFFFFFu) > 0x7F800000u) return (uint16_t)((u >> 16) | 0x0040u); // NaN, made quiet
+    return (uint16_t)((u + 0x7FFFu + ((u >> 16) & 1u)) >> 16);
+}
+
+// IEEE binary32 -> binary16, round to nearest even, written out on the bit patterns.
+uint16_t f32_to_f16_bits(uint32_t u) {
+    const uint16_t sign = (uint16_t)((u >> 16) & 0x8000u);
+    const uint32_t a = u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return sign | 0x7E00u;  // NaN
+    if (a >= 0x477FF000u) return sign | 0x7C00u; // >= 65520 rounds to infinity (and infinity itself)
+    if (a >= 0x38800000u) {                      // normal in binary16: >= 2^-14
+        uint32_t h = (((a >> 23) - 112u) << 10) | ((a & 0x7FFFFFu) >> 13);
+        const uint32_t rest = a & 0x1FFFu;
+        if (rest > 0x1000u || (rest == 0x1000u && (h & 1u))) h++; // a carry runs into the exponent, as it should
+        return sign | (uint16_t)h;
+    }
+    // subnormal in binary16: the value in units of 2^-24, rounded to nearest even
+    const float units = float_of(a) * 16777216.0f; // exact: a power of two
+    return sign | (uint16_t)(uint32_t)nearbyintf(units);
+}
+
+uint32_t f16_bits_to_f32(uint16_t h) {
+    const uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    const uint32_t e = (h >> 10) & 0x1Fu, m = h & 0x3FFu;
+    if (e == 0x1F) return sign | 0x7F800000u | (m << 13);
+    if (e != 0) return sign | ((e + 112u) << 23) | (m << 13);
+    return sign | bits_of((float)m * (1.0f / 16777216.0f)); // subnormal or zero: m * 2^-24, exact in f32
+}
+
+uint32_t round_to(cg_dtype dt, uint32_t u) {
+    if (dt == CG_BF16) return (uint32_t)f32_to_bf16_bits(u) << 16;
+    if (dt == CG_F16) return f16_bits_to_f32(f32_to_f16_bits(u));
+    return u;
+}
+
 
 // Rust `f32 as u32`: truncate toward zero, saturating, NaN -> 0 (ndarray.rs:155).
 inline uint32_t f32_as_u32(float v) {
@@ -404,9 +470,9 @@ const T *as_batch3(cg_tensor *t, size_t batch, std::vector<T> &tmp, ptrdiff_t &s
 }
 
 template <typename F> int for_each_dtype(cg_dtype dt, F &&f) {
-    if (dt == CG_F32) return f(float{});
+    if (isf(dt)) return f(float{});
     if (dt == CG_U32) return f(uint32_t{});
-    return fail(CG_ERR_UNSUPPORTED, "f16, bf16, and fp8 are not supported by the ndarray backend");
+    return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
 }
 
 } // namespace
@@ -457,7 +523,7 @@ int cg_tensor_is_contiguous(const cg_tensor *t) { return is_standard(t) ? 1 : 0;
 // ndarray.rs:71-84
 int cg_zeros(cg_backend *, cg_dtype dtype, const size_t *dims, size_t rank, cg_tensor **out) {
     if (!out || rank > CG_MAX_RANK) return fail(CG_ERR_ARG, "bad arguments");
-    if (!supported(dtype)) return fail(CG_ERR_UNSUPPORTED, "f16, bf16, and fp8 are not supported by the ndarray backend");
+    if (!supported(dtype)) return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
     *out = new_tensor(dtype, dims, (int)rank); // vector::resize zero-fills
     return CG_OK;
 }
@@ -466,12 +532,18 @@ int cg_zeros(cg_backend *, cg_dtype dtype, const size_t *dims, size_t rank, cg_t
 int cg_from_host(cg_backend *, cg_dtype dtype, const void *data, size_t len, const size_t *dims, size_t rank,
                  cg_tensor **out) {
     if (!out || rank > CG_MAX_RANK) return fail(CG_ERR_ARG, "bad arguments");
-    if (!supported(dtype)) return fail(CG_ERR_UNSUPPORTED, "f16, bf16, and fp8 are not supported by the ndarray backend");
+    if (!supported(dtype)) return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
     size_t n = 1;
     for (size_t i = 0; i < rank; i++) n *= dims[i];
     if (n != len) return fail(CG_ERR_SHAPE, "ShapeError");
     cg_tensor *t = new_tensor(dtype, dims, (int)rank);
-    if (n) memcpy(t->st->data.data(), data, n * 4);
+    if (n && is_half(dtype)) { // 2-byte elements, widened exactly (candle.rs:530-551)
+        const uint16_t *h = static_cast<const uint16_t *>(data);
+        uint32_t *d = t->st->data.data();
+        for (size_t i = 0; i < n; i++) d[i] = dtype == CG_BF16 ? (uint32_t)h[i] << 16 : f16_bits_to_f32(h[i]);
+    } else if (n) {
+        memcpy(t->st->data.data(), data, n * 4);
+    }
     *out = t;
     return CG_OK;
 }
@@ -510,7 +582,13 @@ int cg_to_host(cg_backend *, const cg_tensor *t, void *dst, size_t len) {
     if (!t || (!dst && len)) return fail(CG_ERR_ARG, "null argument");
     if (len != numel(t)) return fail(CG_ERR_SHAPE, "to_vec: length mismatch");
     if (!is_standard(t)) return fail(CG_ERR_SHAPE, "to_vec: called `Option::unwrap()` on a `None` value (non-contiguous)");
-    if (len) memcpy(dst, reinterpret_cast<const uint32_t *>(t->st->data.data()) + t->offset, len * 4);
+    const uint32_t *src = reinterpret_cast<const uint32_t *>(t->st->data.data()) + t->offset;
+    if (is_half(t->dt)) { // 2-byte elements out (candle.rs:463-470); exact, the words hold representable values
+        uint16_t *h = static_cast<uint16_t *>(dst);
+        for (size_t i = 0; i < len; i++) h[i] = t->dt == CG_BF16 ? (uint16_t)(src[i] >> 16) : f32_to_f16_bits(src[i]);
+    } else if (len) {
+        memcpy(dst, src, len * 4);
+    }
     return CG_OK;
 }
 
@@ -518,7 +596,7 @@ int cg_to_host(cg_backend *, const cg_tensor *t, void *dst, size_t len) {
 int cg_to_bool(cg_backend *, const cg_tensor *t, int *out) {
     if (!t || !out) return fail(CG_ERR_ARG, "null argument");
     bool any = false;
-    if (t->dt == CG_F32) {
+    if (isf(t->dt)) {
         for (float v : dense<float>(t)) any |= v > 0.0f;
     } else {
         for (uint32_t v : dense<uint32_t>(t)) any |= v != 0;
@@ -533,7 +611,7 @@ int cg_compare(cg_backend *, const cg_tensor *x, const cg_tensor *y, int *out) {
     if (x->dt != y->dt) return fail(CG_ERR_DTYPE, "compare: dtype mismatch");
     bool eq = same_shape(x, y);
     if (eq) {
-        if (x->dt == CG_F32) {
+        if (isf(x->dt)) {
             auto a = dense<float>(x), b = dense<float>(y);
             for (size_t i = 0; i < a.size() && eq; i++) eq = a[i] == b[i];
         } else {
@@ -547,12 +625,12 @@ int cg_compare(cg_backend *, const cg_tensor *x, const cg_tensor *y, int *out) {
 // ndarray.rs:60-69
 int cg_format_tensor(cg_backend *, const cg_tensor *t, char *buf, size_t cap) {
     if (!t || !buf || !cap) return fail(CG_ERR_ARG, "null argument");
-    std::string s = t->dt == CG_F32 ? "f32[" : "u32[";
+    std::string s = t->dt == CG_F32 ? "f32[" : t->dt == CG_F16 ? "f16[" : t->dt == CG_BF16 ? "bf16[" : "u32[";
     for (int i = 0; i < t->rank; i++) s += (i ? "," : "") + std::to_string(t->dims[i]);
     s += "] [";
     size_t n = numel(t), shown = std::min<size_t>(n, 16);
     char tmp[48];
-    if (t->dt == CG_F32) {
+    if (isf(t->dt)) {
         auto v = dense<float>(t);
         for (size_t i = 0; i < shown; i++) {
             snprintf(tmp, sizeof tmp, "%s%.9g", i ? ", " : "", v[i]);
@@ -575,7 +653,7 @@ int cg_cast(cg_backend *, cg_tensor *x, cg_dtype target, cg_tensor **out) {
     Consume cx(x);
     if (!x || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(target) || !supported(x->dt))
-        return fail(CG_ERR_UNSUPPORTED, "f16, bf16, and fp8 are not supported by the ndarray backend");
+        return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
     if (target == x->dt) { // (x @ F32, F32) => x
         x->rc.fetch_add(1);
         *out = x;
@@ -588,11 +666,16 @@ int cg_cast(cg_backend *, cg_tensor *x, cg_dtype target, cg_tensor **out) {
         auto v = dense<float>(o);
         uint32_t *d = data_of<uint32_t>(r);
         for (size_t i = 0; i < n; i++) d[i] = f32_as_u32(v[i]);
-    } else {
+    } else if (o->dt == CG_U32) {
         auto v = dense<uint32_t>(o);
         float *d = data_of<float>(r);
         for (size_t i = 0; i < n; i++) d[i] = (float)v[i]; // round to nearest even
+    } else { // between floating-point dtypes (candle.rs:575-599): the value, rounded below if the target is narrower
+        auto v = dense<uint32_t>(o);
+        uint32_t *d = data_of<uint32_t>(r);
+        for (size_t i = 0; i < n; i++) d[i] = v[i];
     }
+    round_tensor(r);
     release(o);
     *out = r;
     return CG_OK;
@@ -602,7 +685,7 @@ int cg_cast(cg_backend *, cg_tensor *x, cg_dtype target, cg_tensor **out) {
 int cg_unary(cg_backend *, cg_unary_op op, cg_tensor *x, cg_tensor **out) {
     Consume cx(x);
     if (!x || !out) return fail(CG_ERR_ARG, "null argument");
-    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "f16, bf16, and fp8 are not supported by the ndarray backend");
+    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
     if (x->dt == CG_U32 && op != CG_NEG) {
         static const char *names[] = {"neg", "sin", "cos", "exp", "log", "floor", "round"};
         return fail(CG_ERR_DTYPE, "Invalid input types for %s", names[op]);
@@ -628,6 +711,7 @@ int cg_unary(cg_backend *, cg_unary_op op, cg_tensor *x, cg_tensor **out) {
         default: release(o); release(r); return fail(CG_ERR_ARG, "unknown unary op");
         }
     }
+    round_tensor(r);
     release(o);
     *out = r;
     return CG_OK;
@@ -648,14 +732,14 @@ int cg_binary(cg_backend *, cg_binary_op op, cg_tensor *x, cg_tensor *y, cg_tens
     Consume cx(x), cy(y);
     if (!x || !y || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt) || !supported(y->dt))
-        return fail(CG_ERR_UNSUPPORTED, "f16, bf16, and fp8 are not supported by the ndarray backend");
+        return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
     if (x->dt != y->dt) return fail(CG_ERR_DTYPE, "TypeError: mixed dtypes in a binary operation");
     if (!same_shape(x, y)) return fail(CG_ERR_SHAPE, "Shape mismatch in operation");
     cg_tensor *ox = unwrap_owned(x), *oy = unwrap_owned(y);
     cg_tensor *r = new_tensor(ox->dt, ox->dims, ox->rank);
     size_t n = numel(ox);
     int rc = CG_OK;
-    if (ox->dt == CG_F32) {
+    if (isf(ox->dt)) {
         auto a = dense<float>(ox), b = dense<float>(oy);
         float *d = data_of<float>(r);
         switch (op) {
@@ -702,6 +786,7 @@ int cg_binary(cg_backend *, cg_binary_op op, cg_tensor *x, cg_tensor *y, cg_tens
         release(r);
         return rc;
     }
+    round_tensor(r);
     *out = r;
     return CG_OK;
 }
@@ -710,13 +795,13 @@ int cg_binary(cg_backend *, cg_binary_op op, cg_tensor *x, cg_tensor *y, cg_tens
 int cg_where(cg_backend *, cg_tensor *mask, cg_tensor *x, cg_tensor *y, cg_tensor **out) {
     Consume cm(mask), cx(x), cy(y);
     if (!mask || !x || !y || !out) return fail(CG_ERR_ARG, "null argument");
-    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "f16, bf16, and fp8 are not supported by the ndarray backend");
+    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
     if (mask->dt != x->dt || y->dt != x->dt) return fail(CG_ERR_DTYPE, "TypeError: mixed dtypes in where");
     if (!same_shape(mask, x) || !same_shape(x, y)) return fail(CG_ERR_SHAPE, "Shape mismatch in operation");
     cg_tensor *om = unwrap_owned(mask), *ox = unwrap_owned(x), *oy = unwrap_owned(y);
     cg_tensor *r = new_tensor(ox->dt, ox->dims, ox->rank);
     size_t n = numel(ox);
-    if (ox->dt == CG_F32) {
+    if (isf(ox->dt)) {
         auto m = dense<float>(om), a = dense<float>(ox), b = dense<float>(oy);
         float *d = data_of<float>(r);
         for (size_t i = 0; i < n; i++) d[i] = m[i] > 0.0f ? a[i] : b[i];
@@ -737,7 +822,7 @@ int cg_matmul(cg_backend *, cg_tensor *x, cg_tensor *y, cg_tensor **out) {
     Consume cx(x), cy(y);
     if (!x || !y || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt) || !supported(y->dt))
-        return fail(CG_ERR_UNSUPPORTED, "f16, bf16, and fp8 are not supported by the ndarray backend");
+        return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
     if (x->dt != y->dt) return fail(CG_ERR_DTYPE, "TypeError: mixed dtypes in matmul");
     if (x->rank < 2) return fail(CG_ERR_SHAPE, "batched_matmul: lhs must be at least rank 2");
     if (y->rank < 2) return fail(CG_ERR_SHAPE, "batched_matmul: rhs must be at least rank 2");
@@ -755,7 +840,7 @@ int cg_matmul(cg_backend *, cg_tensor *x, cg_tensor *y, cg_tensor **out) {
     odims[rx - 2] = M;
     odims[rx - 1] = N;
     cg_tensor *r = new_tensor(ox->dt, odims, rx);
-    if (ox->dt == CG_F32) {
+    if (isf(ox->dt)) {
         std::vector<float> ta, tb;
         ptrdiff_t sba, sra, sca, sbb, srb, scb;
         const float *a = as_batch3<float>(ox, batch, ta, sba, sra, sca);
@@ -773,6 +858,7 @@ int cg_matmul(cg_backend *, cg_tensor *x, cg_tensor *y, cg_tensor **out) {
         for (size_t bi = 0; bi < batch; bi++)
             ugemm(M, K, N, a + (ptrdiff_t)bi * sba, sra, sca, b + (ptrdiff_t)bi * sbb, srb, scb, c + bi * M * N);
     }
+    round_tensor(r);
     release(ox);
     release(oy);
     *out = r;
@@ -784,7 +870,7 @@ namespace {
 // underflows on rank 0, ndarray.rs:658,672,728).
 int reduce_frame(cg_tensor *x, cg_tensor **out, const char *what, cg_tensor **owned, size_t *rows, size_t *n) {
     if (!x || !out) return fail(CG_ERR_ARG, "null argument");
-    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "f16, bf16, and fp8 are not supported by the ndarray backend");
+    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
     if (x->rank == 0) return fail(CG_ERR_SHAPE, "%s: rank-0 tensor has no last axis", what);
     *owned = unwrap_owned(x);
     *n = x->dims[x->rank - 1];
@@ -844,6 +930,7 @@ int cg_sum(cg_backend *, cg_tensor *x, cg_tensor **out) {
         }
         return CG_OK;
     });
+    round_tensor(res);
     release(o);
     *out = res;
     return CG_OK;
@@ -861,7 +948,7 @@ int cg_max(cg_backend *, cg_tensor *x, cg_tensor **out) {
     memcpy(odims, o->dims, sizeof odims);
     odims[r - 1] = 1;
     cg_tensor *res = new_tensor(o->dt, odims, r);
-    if (o->dt == CG_F32) {
+    if (isf(o->dt)) {
         auto v = dense<float>(o);
         float *d = data_of<float>(res);
         for (size_t i = 0; i < rows; i++) {
@@ -878,6 +965,7 @@ int cg_max(cg_backend *, cg_tensor *x, cg_tensor **out) {
             d[i] = acc;
         }
     }
+    round_tensor(res); // the seed f32::MIN of an empty or all-NaN row is not a value of the 16-bit dtypes
     release(o);
     *out = res;
     return CG_OK;
@@ -900,7 +988,7 @@ int cg_argmax(cg_backend *, cg_tensor *x, cg_tensor **out) {
     odims[r - 1] = 1;
     cg_tensor *res = new_tensor(CG_U32, odims, r);
     uint32_t *d = data_of<uint32_t>(res);
-    if (o->dt == CG_F32) {
+    if (isf(o->dt)) {
         auto v = dense<float>(o);
         for (size_t i = 0; i < rows; i++) {
             size_t best = 0;
@@ -933,7 +1021,7 @@ int cg_topk(cg_backend *, cg_tensor *x, size_t k, cg_tensor **values, cg_tensor 
     Consume cx(x);
     if (!x || !values || !indices) return fail(CG_ERR_ARG, "null argument");
     if (x->dt == CG_U32) return fail(CG_ERR_DTYPE, "Unsupported type for topk");
-    if (x->dt != CG_F32) return fail(CG_ERR_UNSUPPORTED, "f16, bf16, and fp8 are not supported by the ndarray backend");
+    if (!isf(x->dt)) return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
     if (x->rank == 0) return fail(CG_ERR_SHAPE, "topk: rank-0 tensor has no last axis");
     size_t n = x->dims[x->rank - 1];
     if (n == 0) return fail(CG_ERR_SHAPE, "topk: attempt to divide by zero (empty last axis)");
@@ -948,7 +1036,7 @@ int cg_topk(cg_backend *, cg_tensor *x, size_t k, cg_tensor **values, cg_tensor 
     size_t odims[CG_MAX_RANK];
     memcpy(odims, o->dims, sizeof odims);
     odims[o->rank - 1] = k;
-    cg_tensor *vals = new_tensor(CG_F32, odims, o->rank);
+    cg_tensor *vals = new_tensor(o->dt, odims, o->rank);
     cg_tensor *idxs = new_tensor(CG_U32, odims, o->rank);
     auto v = dense<float>(o);
     float *dv = data_of<float>(vals);
@@ -974,7 +1062,7 @@ int cg_topk(cg_backend *, cg_tensor *x, size_t k, cg_tensor **values, cg_tensor 
 int cg_broadcast(cg_backend *, cg_tensor *x, const size_t *dims, size_t rank, cg_tensor **out) {
     Consume cx(x);
     if (!x || !out || rank > CG_MAX_RANK) return fail(CG_ERR_ARG, "bad arguments");
-    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "f16, bf16, and fp8 are not supported by the ndarray backend");
+    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
     if ((size_t)x->rank > rank) return fail(CG_ERR_SHAPE, "broadcast: called `Option::unwrap()` on a `None` value");
     int shift = (int)rank - x->rank;
     for (int i = 0; i < x->rank; i++)
@@ -1003,7 +1091,7 @@ int cg_broadcast(cg_backend *, cg_tensor *x, const size_t *dims, size_t rank, cg
 int cg_reshape(cg_backend *, cg_tensor *x, const size_t *dims, size_t rank, cg_tensor **out) {
     Consume cx(x);
     if (!x || !out || rank > CG_MAX_RANK) return fail(CG_ERR_ARG, "bad arguments");
-    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "f16, bf16, and fp8 are not supported by the ndarray backend");
+    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
     size_t n = 1;
     for (size_t i = 0; i < rank; i++) n *= dims[i];
     if (n != numel(x)) return fail(CG_ERR_SHAPE, "reshape: ShapeError/IncompatibleShape");
@@ -1019,7 +1107,7 @@ int cg_reshape(cg_backend *, cg_tensor *x, const size_t *dims, size_t rank, cg_t
 int cg_transpose(cg_backend *, cg_tensor *x, size_t dim0, size_t dim1, cg_tensor **out) {
     Consume cx(x);
     if (!x || !out) return fail(CG_ERR_ARG, "null argument");
-    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "f16, bf16, and fp8 are not supported by the ndarray backend");
+    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
     if (dim0 >= (size_t)x->rank || dim1 >= (size_t)x->rank) return fail(CG_ERR_RANGE, "transpose: axis out of range");
     cg_tensor *o = unwrap_owned(x);
     cg_tensor *v = view_of(o);
@@ -1034,7 +1122,7 @@ int cg_transpose(cg_backend *, cg_tensor *x, size_t dim0, size_t dim1, cg_tensor
 int cg_slice(cg_backend *, cg_tensor *x, size_t dim, size_t start, size_t len, cg_tensor **out) {
     Consume cx(x);
     if (!x || !out) return fail(CG_ERR_ARG, "null argument");
-    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "f16, bf16, and fp8 are not supported by the ndarray backend");
+    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
     if (dim >= (size_t)x->rank) return fail(CG_ERR_RANGE, "slice: axis out of range");
     if (start > x->dims[dim] || len > x->dims[dim] - start) return fail(CG_ERR_RANGE, "slice: range out of bounds");
     cg_tensor *o = unwrap_owned(x);
@@ -1051,7 +1139,7 @@ int cg_concat(cg_backend *, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor **
     Consume cx(x), cy(y);
     if (!x || !y || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt) || !supported(y->dt))
-        return fail(CG_ERR_UNSUPPORTED, "f16, bf16, and fp8 are not supported by the ndarray backend");
+        return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
     if (x->dt != y->dt) return fail(CG_ERR_DTYPE, "Incompatible types for concatenation");
     if (x->rank != y->rank || dim >= (size_t)x->rank) return fail(CG_ERR_SHAPE, "concat: IncompatibleShape");
     for (int i = 0; i < x->rank; i++)
@@ -1081,7 +1169,7 @@ int cg_concat(cg_backend *, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor **
 int cg_index(cg_backend *, cg_tensor *x, size_t dim, cg_tensor *indices, cg_tensor **out) {
     Consume cx(x), ci(indices);
     if (!x || !indices || !out) return fail(CG_ERR_ARG, "null argument");
-    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "f16, bf16, and fp8 are not supported by the ndarray backend");
+    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
     if (indices->dt != CG_U32) return fail(CG_ERR_DTYPE, "Invalid input types for indexing");
     if (dim >= (size_t)x->rank) return fail(CG_ERR_RANGE, "index: axis out of range");
     cg_tensor *ox = unwrap_owned(x), *oi = unwrap_owned(indices);

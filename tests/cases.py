@@ -1388,6 +1388,11 @@ def assert_close(kind, got, exp, scale=None, name=""):
         np.testing.assert_allclose(got.astype(np.float64), exp.astype(np.float64), rtol=1e-4, atol=1e-6, err_msg=name)
     elif kind == "ew_abs":  # element-wise math downstream of a row sum: the sum's rounding shows as absolute error
         np.testing.assert_allclose(got.astype(np.float64), exp.astype(np.float64), rtol=1e-4, atol=1e-5, err_msg=name)
+    elif kind in ("ulp_f16", "ulp_bf16"):
+        # one unit in the last place of the 16-bit dtype: 2^-10 (f16, 11-bit significand) resp. 2^-7 (bf16, 8-bit)
+        # of the value at most, plus the spacing of f16 subnormals
+        rtol, atol = (2.0 ** -10, 2.0 ** -24) if kind == "ulp_f16" else (2.0 ** -7, 1e-38)
+        np.testing.assert_allclose(got.astype(np.float64), exp.astype(np.float64), rtol=rtol, atol=atol, err_msg=name)
     elif kind == "red":
         s = np.asarray(scale, dtype=np.float64) if scale is not None else np.abs(exp.astype(np.float64))
         err = np.abs(got.astype(np.float64) - exp.astype(np.float64))
@@ -1395,3 +1400,6 @@ def assert_close(kind, got, exp, scale=None, name=""):
         assert (err <= bound).all(), f"{name}: max err/scale {np.max(err / np.maximum(s, 1e-30)):.3e} > 1e-3"
     else:
         raise ValueError(kind)
+
+
+import cases_half  # noqa: E402,F401  (appends the 16-bit float cases to CASES)
