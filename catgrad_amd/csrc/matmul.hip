@@ -201,6 +201,10 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
             load_tile<B_NFAST>(rb, B, a.b_sn, a.b_sk, n0, (kt + 1) * BK, a.N, a.K, a.b_vec);
         }
         const float *la = lds_a(cur), *lb = lds_b(cur);
+        // While a wave is in its burst of matrix instructions it wins issue arbitration against the other
+        // wave of its SIMD (which is loading or storing a tile): the two stop advancing in lock-step and
+        // their stalls at the barrier no longer coincide.
+        __builtin_amdgcn_s_setprio(1);
 #pragma unroll
         for (int kc = 0; kc < BK / 8; kc++) {
             // lane group g supplies k = 8*kc + 4*g + t to the t-th MFMA of this chunk, for
@@ -220,6 +224,7 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
                     for (int j = 0; j < NT; j++)
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][t], fb[j][t], acc[i][j], 0, 0, 0);
         }
+        __builtin_amdgcn_s_setprio(0);
         if (kt + 1 < nk) {
             store_tile<A_MFAST>(ra, lds_a(cur ^ 1));
             store_tile<B_NFAST>(rb, lds_b(cur ^ 1));
