@@ -67,7 +67,7 @@ __device__ __forceinline__ void batch_offsets(const MmArgs &a, uint32_t b, int64
 // ------------------------------------------------------------------------------------------
 constexpr int BM = 128, BN = 128, BK = 32; // BN = 64 in the narrow variant
 constexpr int PITCH = BK + 4; // words per LDS row: row r starts at bank 4r mod 32
-constexpr size_t gemm_lds_bytes(int bn) { return 2 * (size_t)(BM + bn) * PITCH * sizeof(float); }
+constexpr size_t gemm_lds_bytes(int bn, int bm = BM) { return 2 * (size_t)(bm + bn) * PITCH * sizeof(float); }
 constexpr int kThreads = 256;
 constexpr uint32_t kXcds = 8, kGroupM = 8;
 
@@ -139,11 +139,14 @@ template <bool ROWS_FAST, int TR> __device__ __forceinline__ void store_tile(con
     }
 }
 
-// NT: 32-column MFMA tiles per wave.  2: the 128 x 128 macro tile; 1: 128 x 64 (each wave a
-// 64 x 32 strip) for products whose N is a small multiple of 64, such as p.V with head_dim 64.
-template <bool A_MFAST, bool B_NFAST, int NT>
+// NT / MT: 32-wide MFMA tiles per wave along N / M (the block is 2 x 2 waves).  NT = 2, MT = 2: the
+// 128 x 128 macro tile; NT = 1: 128 x 64 (each wave a 64 x 32 strip) for products whose N is a small
+// multiple of 64, such as p.V with head_dim 64; NT = MT = 4: 256 x 256, each wave a 128 x 128 block in
+// 256 accumulation registers, one wave per SIMD: four times the matrix instructions between two
+// barriers and half the LDS traffic per flop, for products with enough tiles to fill the chip.
+template <bool A_MFAST, bool B_NFAST, int NT, int MT = 2>
 __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
-    constexpr int BN = 64 * NT; // shadows the wide default
+    constexpr int BN = 64 * NT, BM = 64 * MT; // shadow the defaults
     extern __shared__ float lds_dyn[]; // [2][BM][PITCH] for A, then [2][BN][PITCH] for B
     auto lds_a = [&](uint32_t buf) { return lds_dyn + buf * (BM * PITCH); };
     auto lds_b = [&](uint32_t buf) { return lds_dyn + 2 * BM * PITCH + buf * (BN * PITCH); };
@@ -174,12 +177,12 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
     uint32_t *C = a.C + (uint64_t)blockIdx.y * a.M * a.N;
 
     const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x % 64;
-    const uint32_t wm = (wave / 2) * 64, wn = (wave % 2) * (32 * NT); // wave quadrant
+    const uint32_t wm = (wave / 2) * (32 * MT), wn = (wave % 2) * (32 * NT); // wave quadrant
     const uint32_t li = lane % 32, lg = lane / 32;
 
-    float16v acc[2][NT];
+    float16v acc[MT][NT];
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < MT; i++)
 #pragma unroll
         for (int j = 0; j < NT; j++)
 #pragma unroll
@@ -196,22 +199,14 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
 
     for (uint32_t kt = 0; kt < nk; kt++) {
         const uint32_t cur = kt & 1;
-        if (kt + 1 < nk) {
-            load_tile<A_MFAST>(ra, A, a.a_sm, a.a_sk, m0, (kt + 1) * BK, a.M, a.K, a.a_vec);
-            load_tile<B_NFAST>(rb, B, a.b_sn, a.b_sk, n0, (kt + 1) * BK, a.N, a.K, a.b_vec);
-        }
+        const bool more = kt + 1 < nk;
         const float *la = lds_a(cur), *lb = lds_b(cur);
-        // While a wave is in its burst of matrix instructions it wins issue arbitration against the other
-        // wave of its SIMD (which is loading or storing a tile): the two stop advancing in lock-step and
-        // their stalls at the barrier no longer coincide.
-        __builtin_amdgcn_s_setprio(1);
+        // One 8-deep chunk of the tile: lane group g supplies k = 8*kc + 4*g + t to the t-th MFMA,
+        // for A and B alike, so one 128-bit LDS read feeds four MFMAs.
+        auto chunk = [&](const int kc) {
+            float4v fa[MT], fb[NT];
 #pragma unroll
-        for (int kc = 0; kc < BK / 8; kc++) {
-            // lane group g supplies k = 8*kc + 4*g + t to the t-th MFMA of this chunk, for
-            // A and B alike, so one 128-bit LDS read feeds four MFMAs.
-            float4v fa[2], fb[NT];
-#pragma unroll
-            for (int i = 0; i < 2; i++)
+            for (int i = 0; i < MT; i++)
                 fa[i] = *reinterpret_cast<const float4v *>(la + (wm + i * 32 + li) * PITCH + kc * 8 + lg * 4);
 #pragma unroll
             for (int j = 0; j < NT; j++)
@@ -219,13 +214,23 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
 #pragma unroll
             for (int t = 0; t < 4; t++)
 #pragma unroll
-                for (int i = 0; i < 2; i++)
+                for (int i = 0; i < MT; i++)
 #pragma unroll
                     for (int j = 0; j < NT; j++)
                         acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][t], fb[j][t], acc[i][j], 0, 0, 0);
+        };
+        // While a wave is in its burst of matrix instructions it wins issue arbitration against the other
+        // wave of its SIMD (which is loading or storing a tile): the two stop advancing in lock-step and
+        // their stalls at the barrier no longer coincide.
+        if (more) {
+            load_tile<A_MFAST>(ra, A, a.a_sm, a.a_sk, m0, (kt + 1) * BK, a.M, a.K, a.a_vec);
+            load_tile<B_NFAST>(rb, B, a.b_sn, a.b_sk, n0, (kt + 1) * BK, a.N, a.K, a.b_vec);
         }
+        __builtin_amdgcn_s_setprio(1);
+#pragma unroll
+        for (int kc = 0; kc < BK / 8; kc++) chunk(kc);
         __builtin_amdgcn_s_setprio(0);
-        if (kt + 1 < nk) {
+        if (more) {
             store_tile<A_MFAST>(ra, lds_a(cur ^ 1));
             store_tile<B_NFAST>(rb, lds_b(cur ^ 1));
         }
@@ -234,7 +239,7 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
 
     // D layout of v_mfma_f32_32x32x2_f32: lane (li, lg), register v -> row 8*(v/4) + 4*lg + v%4, col li
 #pragma unroll
-    for (int i = 0; i < 2; i++)
+    for (int i = 0; i < MT; i++)
 #pragma unroll
         for (int j = 0; j < NT; j++) {
             uint32_t col = n0 + wn + j * 32 + li;
@@ -973,7 +978,14 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
         const int64_t cols128 = (N + 127) / 128 * 128, cols64 = (N + 63) / 64 * 64;
         const bool narrow = cols128 * 7 > cols64 * 8;
         const int bn = narrow ? 64 : 128;
-        uint64_t tiles = (uint64_t)((M + BM - 1) / BM) * ((N + bn - 1) / bn);
+        // the 256 x 256 tile when it covers the chip at least once (env CG_GEMM_BIG=0 switches it off)
+        const uint64_t tiles_big = (uint64_t)((M + 255) / 256) * ((N + 255) / 256) * batch;
+        static const bool big_allowed = [] {
+            const char *e = getenv("CG_GEMM_BIG");
+            return !(e && e[0] == '0');
+        }();
+        const bool big = big_allowed && !narrow && tiles_big >= 256 && M >= 256 && N >= 256;
+        uint64_t tiles = big ? tiles_big / batch : (uint64_t)((M + BM - 1) / BM) * ((N + bn - 1) / bn);
         if (tiles > 0x7FFFFFFFull) return fail(CG_ERR_UNSUPPORTED, "matmul: too many tiles");
         dim3 grid((uint32_t)tiles, (uint32_t)batch);
         static const bool lds_ok = [] { // the tiles need more than the default 64 KiB of dynamic LDS
@@ -982,7 +994,9 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
     ok &= hipFuncSetAttribute(reinterpret_cast<const void *>(&mfma_gemm_kernel<AF, BF, 2>),                           \
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds_bytes(128)) == hipSuccess;    \
     ok &= hipFuncSetAttribute(reinterpret_cast<const void *>(&mfma_gemm_kernel<AF, BF, 1>),                           \
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds_bytes(64)) == hipSuccess;
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds_bytes(64)) == hipSuccess;     \
+    ok &= hipFuncSetAttribute(reinterpret_cast<const void *>(&mfma_gemm_kernel<AF, BF, 4, 4>),                        \
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds_bytes(256, 256)) == hipSuccess;
             CG_LDS(true, true) CG_LDS(true, false) CG_LDS(false, true) CG_LDS(false, false)
 #undef CG_LDS
             return ok;
@@ -990,7 +1004,9 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
         if (!lds_ok) return fail(CG_ERR_DEVICE, "matmul: cannot reserve %zu bytes of LDS", gemm_lds_bytes(128));
 #define CG_GEMM(AF, BF)                                                                                            \
     do {                                                                                                           \
-        if (narrow)                                                                                                \
+        if (big)                                                                                                   \
+            hipLaunchKernelGGL((mfma_gemm_kernel<AF, BF, 4, 4>), grid, dim3(kThreads), gemm_lds_bytes(256, 256), s, a); \
+        else if (narrow)                                                                                           \
             hipLaunchKernelGGL((mfma_gemm_kernel<AF, BF, 1>), grid, dim3(kThreads), gemm_lds_bytes(64), s, a);     \
         else                                                                                                       \
             hipLaunchKernelGGL((mfma_gemm_kernel<AF, BF, 2>), grid, dim3(kThreads), gemm_lds_bytes(128), s, a);    \

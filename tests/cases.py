@@ -844,6 +844,15 @@ _mm_case("mm_sliced_operands", (2, 50, 80), (2, 80, 70),
 _mm_case("mm_k_over_256", (2, 16, 700), (2, 700, 24))
 _mm_case("mm_tile_edges", (1, 129, 67), (1, 67, 131))
 _mm_case("mm_big_tile", (2, 256, 128), (2, 128, 384))
+# enough 256 x 256 tiles to cover the chip: the one-wave-per-SIMD tile, in all four operand layouts, full and ragged
+_mm_case("mm_256_tiles_full", (64, 512, 40), (64, 40, 512), seed=96)
+_mm_case("mm_256_tiles_ragged", (43, 300, 70), (43, 70, 520), seed=97)
+_mm_case("mm_256_tiles_lhs_transposed", (43, 70, 300), (43, 70, 520),
+         lambda be, a, b: (be.transpose(a, 1, 2), b, None, None), seed=98)
+_mm_case("mm_256_tiles_rhs_transposed", (43, 300, 70), (43, 520, 70),
+         lambda be, a, b: (a, be.transpose(b, 1, 2), None, None), seed=99)
+_mm_case("mm_256_tiles_both_transposed_linear", (300, 16, 68), (5000, 68),
+         lambda be, a, b: (be.transpose(a, 0, 1), be.broadcast(be.transpose(b, 0, 1), (16, 68, 5000)), None, None), seed=100)
 
 
 @case("mm_u32_wrapping")
