@@ -36,7 +36,7 @@ MFMA_F32_PEAK = 157.3e12  # flop/s, MI355X dense f32 matrix
 # HBM bytes per mfma_gemm_kernel launch of this workload's prefill, from rocprofv3 FETCH_SIZE / WRITE_SIZE passes
 # scaled by a copy kernel of known size (profiles/mfma_gemm_llama1b_prefill_pmc.txt); counters cannot be read
 # from inside this process, so the figure is carried here and only reported for the profiled shape.
-MFMA_GEMM_TRAFFIC_PER_LAUNCH = 1.603e9
+MFMA_GEMM_TRAFFIC_PER_LAUNCH = 1.055e9
 
 
 def micro_bench(iters=20):
@@ -230,7 +230,7 @@ def main():
         "backend_calls": {"prefill": calls[0], "per_decode_step": round(calls[1] / max(T, 1), 1)},
         "backend": sess.backend_name,
         "roofline": {
-            "kernel": "mfma_gemm_kernel (f32 v_mfma_f32_32x32x2, 128x128x32 tiles)",
+            "kernel": "mfma_gemm_kernel (f32 v_mfma_f32_32x32x2; 256x256x32 tiles, 128x128 and 128x64 for small N)",
             "bound": "mfma", "achieved": round(mfma_rate / 1e12, 3), "peak": MFMA_F32_PEAK / 1e12, "unit": "TFLOP/s",
             "frac": round(mfma_rate / MFMA_F32_PEAK, 4),
             "traffic": MFMA_GEMM_TRAFFIC_PER_LAUNCH if (B, S) == (4, 2048) else None,
