@@ -21,7 +21,7 @@ NEG, SIN, COS, EXP, LOG, FLOOR, ROUND = range(7)
 ADD, SUB, MUL, DIV, POW, LT, GT, GTE, LTE, EQ = range(10)
 
 # enum cg_kernel_class
-K_GEMM_MFMA, K_GEMM_SKINNY, K_GEMM_SIMPLE, K_ELEMENTWISE, K_REDUCE, K_GATHER = range(6)
+K_GEMM_MFMA, K_GEMM_SKINNY, K_GEMM_SIMPLE, K_ELEMENTWISE, K_REDUCE, K_GATHER, K_ATTENTION = range(7)
 
 _P = C.c_void_p
 _PP = C.POINTER(C.c_void_p)

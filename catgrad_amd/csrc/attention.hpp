@@ -57,6 +57,10 @@ struct AttnArgs {
     int64_t q_sm; // stride between the query rows of a group
     int64_t k_st; // stride between cached positions of K (head_dim contiguous)
     int64_t v_st; // stride between cached positions of V (head_dim contiguous)
+    // prefill only: the batch axes as p.V collapsed them (same number of entries, possibly another split)
+    uint32_t nbv;
+    uint32_t vbd[kMaxBatchAxes];
+    FastDiv vbdiv[kMaxBatchAxes];
 };
 
 constexpr int kAttnRows = 8;    // most query rows per KV head
@@ -289,4 +293,194 @@ __global__ __launch_bounds__(kBlock) void decode_attention_combine_kernel(const 
     for (int sft = 32; sft >= 1; sft >>= 1) den += __shfl_xor(den, sft);
     if (lane < hd) out[r * hd + lane] = asu(num0 / den);
     if (lane + 64 < hd) out[r * hd + lane + 64] = asu(num1 / den);
+}
+
+// ---- prefill: causal attention of many query rows in one pass ---------------------------------------------------
+// The same three ops as above with thousands of query rows per KV head: unfused they write and re-read the
+// [rows, T] score matrix four times (2 GiB per layer of the 1B-shape prefill).  Here a workgroup takes 128
+// query rows of one KV head (a wave 32 of them) and walks the cached positions in tiles of 64, never going
+// beyond the last position its rows may see.  Everything is computed TRANSPOSED, so that a query is a lane:
+//     S^T[t][m] = K[t] . Q[m]          first MFMA operand K (from LDS), second Q (registers, loaded once)
+//     running maximum / sum per query  = per lane: in-register over its 32 values + one exchange with lane ^ 32
+//     O^T[d][m] += V^T[d][t] P^T[t][m] first operand V^T (from LDS), second P^T — which, in the accumulator
+//                                      layout of v_mfma_f32_32x32x2 (column = lane % 32, rows 8*(v/4) + 4*(lane/32)
+//                                      + v%4), already is the operand layout: no trip through LDS, no transposition
+// The scores are divided by the scale and masked exactly as the soft-max program does (x / d + f32(i < j) * m with
+// i the query's position, j the key's); masked keys get weight zero, which is what exp(x - max) rounds to for them.
+// out = O / l at the end (the program divides the weights first: same value up to rounding).
+// MFMA-bound: 2 x 2 x 32 x 64 x 64 flop per wave and tile over ~half of the [rows, T] rectangle.
+struct PrefillArgs {
+    uint32_t *out;      // [batch][M][hd], dense
+    uint32_t S;         // query positions per head: row m of a group is position m % S
+    uint32_t pos0;      // position of the first query row (length of the cache before this chunk)
+    uint32_t scale;     // f32 bits of the divisor of the scores
+    uint32_t mask_mul;  // f32 bits of the multiplier of the 0/1 mask
+};
+
+constexpr int kPfRows = 128, kPfKeys = 64, kPfPitch = 68;
+constexpr size_t prefill_lds_bytes(int hd) { return 2 * (size_t)(kPfKeys + hd) * kPfPitch * sizeof(float); }
+
+template <int HD>
+__global__ __launch_bounds__(kBlock) void prefill_attention_kernel(const AttnArgs g, const PrefillArgs e) {
+    static_assert(HD == 64, "written for head_dim 64");
+    typedef float float16v __attribute__((ext_vector_type(16)));
+    extern __shared__ float pf_lds[]; // 68 KiB: above the static limit
+    float (*Ks)[kPfKeys][kPfPitch] = reinterpret_cast<float (*)[kPfKeys][kPfPitch]>(pf_lds);                       // [2][t][d]
+    float (*Vt)[HD][kPfPitch] = reinterpret_cast<float (*)[HD][kPfPitch]>(pf_lds + 2 * kPfKeys * kPfPitch);        // [2][d][t]
+    const uint32_t tid = threadIdx.x, lane = tid % 64, wave = tid / 64, li = lane % 32, lg = lane / 32;
+    const uint32_t ntile_rows = (g.M + kPfRows - 1) / kPfRows;
+    const uint32_t rt = ntile_rows - 1 - blockIdx.x; // the longest rows first
+    const uint32_t b = blockIdx.y;
+    int64_t oq = 0, ok = 0, ov = 0;
+    {
+        uint32_t bb = b;
+        for (uint32_t d = 0; d < g.nb; d++) {
+            const uint32_t q = fastdiv(bb, g.bdiv[d]);
+            const int64_t i = (int64_t)(bb - q * g.bd[d]);
+            bb = q;
+            oq += i * g.q_bs[d];
+            ok += i * g.k_bs[d];
+        }
+        bb = b;
+        for (uint32_t d = 0; d < g.nbv; d++) {
+            const uint32_t q = fastdiv(bb, g.vbdiv[d]);
+            const int64_t i = (int64_t)(bb - q * g.vbd[d]);
+            bb = q;
+            ov += i * g.v_bs[d];
+        }
+    }
+    const uint32_t m0 = rt * kPfRows;
+    const uint32_t m = m0 + wave * 32 + li; // this lane's query row (both halves of the wave hold the same 32 queries)
+    const bool live = m < g.M;
+    const uint32_t iq = e.pos0 + (live ? m % e.S : 0); // position of the query: keys up to iq are visible
+    // last key any row of the workgroup may see
+    uint32_t kmax;
+    {
+        const uint32_t s0 = m0 % e.S, last = min(m0 + kPfRows, g.M) - 1 - m0; // rows m0 .. m0 + last
+        const uint32_t smax = s0 + last < e.S ? s0 + last : e.S - 1;            // the tile may run into the next head
+        kmax = min(g.T - 1, e.pos0 + smax);
+    }
+    const uint32_t ntiles = kmax / kPfKeys + 1;
+
+    // the query rows, as second MFMA operands: chunk c covers d = 8c .. 8c+7, this lane holds 4*lg .. 4*lg+3 of them
+    float4v qf[HD / 8];
+#pragma unroll
+    for (int c = 0; c < HD / 8; c++) {
+        qf[c] = (float4v){0.f, 0.f, 0.f, 0.f};
+        if (live) qf[c] = *reinterpret_cast<const float4v *>(g.Q + oq + (int64_t)m * g.q_sm + c * 8 + lg * 4);
+    }
+    float16v acc_o[HD / 32];
+#pragma unroll
+    for (int db = 0; db < HD / 32; db++)
+#pragma unroll
+        for (int v = 0; v < 16; v++) acc_o[db][v] = 0.0f;
+    float run_max = -INFINITY, run_sum = 0.0f;
+    const float scale = asf(e.scale);
+
+    // K / V tile: 64 positions x 64 floats each = 1024 float4 per operand, 4 per thread
+    float4v kr[4], vr[4];
+    auto load_kv = [&](uint32_t t0) {
+#pragma unroll
+        for (int h = 0; h < 4; h++) {
+            const uint32_t slot = tid + h * kBlock, t = t0 + slot / 16, dq = slot % 16;
+            kr[h] = (float4v){0.f, 0.f, 0.f, 0.f};
+            vr[h] = (float4v){0.f, 0.f, 0.f, 0.f};
+            if (t < g.T) {
+                kr[h] = *reinterpret_cast<const float4v *>(g.Kc + ok + (int64_t)t * g.k_st + dq * 4);
+                vr[h] = *reinterpret_cast<const float4v *>(g.V + ov + (int64_t)t * g.v_st + dq * 4);
+            }
+        }
+    };
+    auto store_kv = [&](uint32_t buf) {
+#pragma unroll
+        for (int h = 0; h < 4; h++) {
+            const uint32_t slot = tid + h * kBlock, t = slot / 16, dq = slot % 16;
+            *reinterpret_cast<float4v *>(&Ks[buf][t][dq * 4]) = kr[h];
+            Vt[buf][dq * 4 + 0][t] = vr[h][0];
+            Vt[buf][dq * 4 + 1][t] = vr[h][1];
+            Vt[buf][dq * 4 + 2][t] = vr[h][2];
+            Vt[buf][dq * 4 + 3][t] = vr[h][3];
+        }
+    };
+    load_kv(0);
+    store_kv(0);
+    __syncthreads();
+
+    for (uint32_t it = 0; it < ntiles; it++) {
+        const uint32_t cur = it & 1, t0 = it * kPfKeys;
+        const bool more = it + 1 < ntiles;
+        if (more) load_kv(t0 + kPfKeys);
+        // ---- S^T = K Q^T for the tile: two blocks of 32 keys x this wave's 32 queries
+        float16v acc_s[kPfKeys / 32];
+#pragma unroll
+        for (int tb = 0; tb < kPfKeys / 32; tb++) {
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc_s[tb][v] = 0.0f;
+#pragma unroll
+            for (int c = 0; c < HD / 8; c++) {
+                const float4v kf = *reinterpret_cast<const float4v *>(&Ks[cur][tb * 32 + li][c * 8 + lg * 4]);
+#pragma unroll
+                for (int r = 0; r < 4; r++) acc_s[tb] = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[r], qf[c][r], acc_s[tb], 0, 0, 0);
+            }
+        }
+        // ---- scale, mask, running soft-max statistics of this lane's query
+        float tile_max = -INFINITY;
+#pragma unroll
+        for (int tb = 0; tb < kPfKeys / 32; tb++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const uint32_t t = t0 + tb * 32 + 8 * (v / 4) + 4 * lg + (v % 4);
+                // the program's x / d + f32(i < j) * m: nothing is added to a visible key, and an invisible one
+                // (m is hugely negative: the host checks) ends with weight exp(-huge) = 0, so it is left out
+                const float x = acc_s[tb][v] / scale;
+                const bool seen = t <= iq && t < g.T && live;
+                acc_s[tb][v] = seen ? x : -INFINITY;
+                tile_max = fmaxf(tile_max, acc_s[tb][v]);
+            }
+        tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32));
+        const float new_max = fmaxf(run_max, tile_max);
+        const float alpha = new_max == -INFINITY ? 1.0f : expf(run_max - new_max);
+        float tile_sum = 0.0f;
+#pragma unroll
+        for (int tb = 0; tb < kPfKeys / 32; tb++)
+#pragma unroll
+            for (int v = 0; v < 16; v++) {
+                const float p = acc_s[tb][v] == -INFINITY ? 0.0f : expf(acc_s[tb][v] - new_max);
+                acc_s[tb][v] = p;
+                tile_sum += p;
+            }
+        tile_sum += __shfl_xor(tile_sum, 32);
+        run_sum = run_sum * alpha + tile_sum;
+        run_max = new_max;
+        // ---- O^T = alpha O^T + V^T P^T
+#pragma unroll
+        for (int db = 0; db < HD / 32; db++) {
+#pragma unroll
+            for (int v = 0; v < 16; v++) acc_o[db][v] *= alpha;
+#pragma unroll
+            for (int tb = 0; tb < kPfKeys / 32; tb++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) {
+                    const float4v vf = *reinterpret_cast<const float4v *>(&Vt[cur][db * 32 + li][tb * 32 + q * 8 + lg * 4]);
+#pragma unroll
+                    for (int r = 0; r < 4; r++)
+                        acc_o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(vf[r], acc_s[tb][q * 4 + r], acc_o[db], 0, 0, 0);
+                }
+        }
+        if (more) store_kv(cur ^ 1);
+        __syncthreads();
+    }
+    // ---- out[m][d] = O^T[d][m] / l[m]
+    if (live) {
+        uint32_t *orow = e.out + ((uint64_t)b * g.M + m) * HD;
+#pragma unroll
+        for (int db = 0; db < HD / 32; db++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                float4v o;
+#pragma unroll
+                for (int r = 0; r < 4; r++) o[r] = acc_o[db][j * 4 + r] / run_sum;
+                *reinterpret_cast<float4v *>(orow + db * 32 + j * 8 + lg * 4) = o;
+            }
+    }
 }

@@ -406,6 +406,8 @@ int fold_matmul(const cg_tensor *x, const cg_tensor *y, MmFold *f);
 // below) when the shapes do not allow it.
 int launch_matmul_gated(cg_backend *be, const cg_tensor *x, const cg_tensor *yg, const cg_tensor *yu, uint32_t one,
                         cg_tensor *out);
+int launch_prefill_attention(cg_backend *be, const Pending &p, const int64_t *pdims, int prank, const cg_tensor *q,
+                             const cg_tensor *kt, const cg_tensor *v, cg_tensor *out);
 int launch_fused_group(cg_backend *be, const cg_tensor *const *outs, const Pending *const *ps, int n);
 // Writes that were put off so that they can share a launch (see DeferredWrite); every function
 // that launches a kernel or copies device memory calls this first.

@@ -687,6 +687,116 @@ int launch_decode_attention(cg_backend *be, const Pending &p, const int64_t *pdi
     return e == hipSuccess ? CG_OK : hip_fail(e, "decode attention launch");
 }
 
+// q.K^T -> causal soft-max -> p.V for many query rows per KV head (a prefill), in one pass: see
+// prefill_attention_kernel.  Declines unless the program is the listed soft-max with a causal mask built
+// from the backend's iota (query position against key position), head_dim is 64 and the operands are laid
+// out as the decoder graphs lay them out.
+// With CG_TRACE_PROGRAMS=1: which check made the one-pass prefill attention decline (the number counts the
+// checks of launch_prefill_attention from the top).
+static int pf_declined(const cg_backend *be, int check) {
+    if (be->trace_programs) fprintf(stderr, "[cg program] prefill attention declined at check %d\n", check);
+    return kDeclined;
+}
+
+int launch_prefill_attention(cg_backend *be, const Pending &p, const int64_t *pdims, int prank, const cg_tensor *q,
+                             const cg_tensor *kt, const cg_tensor *v, cg_tensor *out) {
+    if (int frc = flush_deferred(be)) return frc;
+    using P = RowsSoftmaxCausal;
+    if (!be->aot || prank != 4 || !program_matches<P>(p) || !p.leaf[0].lazy || p.leaf[0].lazy->result || p.reduced) return pf_declined(be, 1);
+    cg_tensor pd; // the soft-max result as a dense descriptor: the left operand of p.V
+    pd.rank = prank;
+    int64_t st = 1;
+    for (int i = prank - 1; i >= 0; i--) {
+        pd.dims[i] = pdims[i];
+        pd.strides[i] = st;
+        st *= pdims[i];
+    }
+    if (p.leaf[0].offset != 0) return pf_declined(be, 2);
+    for (int i = 0; i < prank; i++)
+        if (pdims[i] > 1 && p.leaf[0].strides[i] != pd.strides[i]) return pf_declined(be, 3);
+    // the mask: f32(l2 < l3) * l4 with l2 = position of the query (iota along axis 2, from some offset) and
+    // l3 = position of the key (iota along axis 3, from 0); l4 hugely negative
+    const LeafView &lq = p.leaf[2], &lk = p.leaf[3];
+    const int64_t S = pdims[2], T = pdims[3];
+    if (!be->iota || lq.buf != be->iota || lk.buf != be->iota || lk.offset != 0 || lq.offset < 0 || lq.offset + S > be->iota_len ||
+        T > be->iota_len)
+        return pf_declined(be, 4);
+    for (int i = 0; i < 4; i++) {
+        const int64_t want_q = i == 2 ? 1 : 0, want_k = i == 3 ? 1 : 0;
+        if (pdims[i] > 1 && (lq.strides[i] != want_q || lk.strides[i] != want_k)) return pf_declined(be, 5);
+    }
+    float mask_mul;
+    memcpy(&mask_mul, &p.leaf[4].ubits, 4);
+    if (!(mask_mul <= -1e30f)) return pf_declined(be, 6);
+    MmFold f1, f2;
+    if (fold_matmul(q, kt, &f1) || fold_matmul(&pd, v, &f2)) return pf_declined(be, 7);
+    const int64_t hd = f1.K;
+    if (be->trace_programs)
+        fprintf(stderr, "[cg program] prefill attention: q.K^T M %lld N %lld K %lld batch %lld nb %d; p.V M %lld N %lld K %lld batch %lld nb %d; S %lld T %lld\n",
+                (long long)f1.M, (long long)f1.N, (long long)f1.K, (long long)f1.batch, f1.nb, (long long)f2.M, (long long)f2.N,
+                (long long)f2.K, (long long)f2.batch, f2.nb, (long long)S, (long long)T);
+    if (f1.N != T || f1.M != f2.M || f1.M <= kAttnRows || f1.M % S != 0 || f1.batch != f2.batch || f2.K != T || f2.N != hd) return pf_declined(be, 8);
+    if (hd != 64) return pf_declined(be, 9);
+    if (f1.a_sk != 1 || f1.b_sk != 1 || f2.b_sn != 1 || f2.a_sk != 1 || f2.a_sm != T) return pf_declined(be, 10);
+    if (f1.batch < 1 || f1.batch > 65535 || T < 1 || T > 0x7FFFFFFFll || f1.M > 0x7FFFFFFFll) return pf_declined(be, 11);
+    for (int d = 0; d < f1.nb; d++)
+        if (f1.a_bs[d] % 4 || f1.b_bs[d] % 4) return pf_declined(be, 12);
+    for (int d = 0; d < f2.nb; d++)
+        if (f2.b_bs[d] % 4) return pf_declined(be, 12);
+    if (f1.a_sm % 4 || f1.b_sn % 4 || f2.b_sk % 4) return pf_declined(be, 13);
+    // rows of the folded group must land in `out` in order: out is [batch][M][hd]
+    if ((int64_t)f1.batch * f1.M * hd != numel(out) || !is_contiguous(out)) return pf_declined(be, 14);
+    const void *pq, *pk, *pv;
+    int rc = device_ptr(q, &pq);
+    if (!rc) rc = device_ptr(kt, &pk);
+    if (!rc) rc = device_ptr(v, &pv);
+    if (rc) return rc;
+    if (reinterpret_cast<uintptr_t>(pq) % 16 || reinterpret_cast<uintptr_t>(pk) % 16 || reinterpret_cast<uintptr_t>(pv) % 16)
+        return pf_declined(be, 15);
+    static const bool lds_ok = hipFuncSetAttribute(reinterpret_cast<const void *>(&prefill_attention_kernel<64>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                   (int)prefill_lds_bytes(64)) == hipSuccess;
+    if (!lds_ok) return pf_declined(be, 16);
+    AttnArgs g;
+    memset(&g, 0, sizeof g);
+    g.Q = static_cast<const uint32_t *>(pq);
+    g.Kc = static_cast<const uint32_t *>(pk);
+    g.V = static_cast<const uint32_t *>(pv);
+    g.M = (uint32_t)f1.M;
+    g.T = (uint32_t)T;
+    g.hd = (uint32_t)hd;
+    g.nb = (uint32_t)f1.nb;
+    for (int d = 0; d < f1.nb; d++) {
+        g.bd[d] = (uint32_t)f1.bd[d];
+        g.bdiv[d] = make_fastdiv(g.bd[d]);
+        g.q_bs[d] = f1.a_bs[d];
+        g.k_bs[d] = f1.b_bs[d];
+    }
+    g.nbv = (uint32_t)f2.nb;
+    for (int d = 0; d < f2.nb; d++) {
+        g.vbd[d] = (uint32_t)f2.bd[d];
+        g.vbdiv[d] = make_fastdiv(g.vbd[d]);
+        g.v_bs[d] = f2.b_bs[d];
+    }
+    g.q_sm = f1.a_sm;
+    g.k_st = f1.b_sn;
+    g.v_st = f2.b_sk;
+    PrefillArgs e;
+    e.out = static_cast<uint32_t *>(out->buf->ptr);
+    e.S = (uint32_t)S;
+    e.pos0 = (uint32_t)lq.offset;
+    e.scale = p.leaf[1].ubits;
+    e.mask_mul = p.leaf[4].ubits;
+    be->programs_compiled++;
+    // flop: the visible half of the [rows, T] rectangle, twice (scores and weighted sum)
+    const double flop = 2.0 * 2.0 * (double)f1.batch * (double)f1.M * (double)hd * ((double)e.pos0 + 0.5 * (double)S);
+    ProfScope prof(be, CG_K_ATTENTION, flop);
+    dim3 grid((uint32_t)((f1.M + kPfRows - 1) / kPfRows), (uint32_t)f1.batch);
+    hipLaunchKernelGGL((prefill_attention_kernel<64>), grid, dim3(kBlock), prefill_lds_bytes(64), be->stream, g, e);
+    hipError_t err = hipGetLastError();
+    return err == hipSuccess ? CG_OK : hip_fail(err, "prefill attention launch");
+}
+
 bool fused_program_fits(const Pending &p) {
     uint8_t phys[kMaxLeaves + kMaxInstr];
     return allocate_registers(p, phys);

@@ -129,7 +129,8 @@ typedef enum cg_kernel_class {
     CG_K_ELEMENTWISE = 3, /* work = bytes of distinct operand elements + output */
     CG_K_REDUCE = 4,      /* work = bytes of the input + output */
     CG_K_GATHER = 5,      /* work = bytes gathered + written */
-    CG_K_CLASSES = 6
+    CG_K_ATTENTION = 6,   /* one-pass causal attention of a prefill; work = flop of the visible scores and sums */
+    CG_K_CLASSES = 7
 } cg_kernel_class;
 int cg_profile_enable(cg_backend *b, cg_kernel_class cls, unsigned sample_every);
 /* Element-wise results are computed lazily (fused into their consumer); cg_realize queues

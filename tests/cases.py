@@ -1130,6 +1130,7 @@ def decode_attention_ops(be, q, k_cache, v_cache, rep):
     soft-max (stdlib/nn/mod.rs:168-179), context.  q [B, kvH*rep, 1, hd]; caches [B, kvH, T, hd]."""
     B, kvh, T, hd = k_cache.shape
     H = kvh * rep
+    S = q.shape[2]          # 1: a decode step; more: a prefill chunk whose last position is T - 1
 
     def repeat_kv(t):
         t = be.reshape(t.move(), (B, kvh, 1, T, hd))
@@ -1138,13 +1139,13 @@ def decode_attention_ops(be, q, k_cache, v_cache, rep):
 
     k, v = repeat_kv(k_cache), repeat_kv(v_cache)
     attn = be.matmul(q.move(), be.transpose(k.move(), 2, 3).move())
-    sh = (B, H, 1, T)
+    sh = (B, H, S, T)
     attn = be.div(attn.move(), _const(be, float(np.sqrt(np.float32(hd))), sh).move())
     ci = be.broadcast(be.arange(T).move(), (T, T))
     cj = be.broadcast(be.reshape(be.arange(T).move(), (T, 1)).move(), (T, T))
     mask = be.cast(be.lt(cj.move(), ci.move()).move(), A.F32)
     mask = be.mul(mask.move(), _const(be, float(F32_MIN), (T, T)).move())
-    mask = be.slice(mask.move(), 0, T - 1, 1)
+    mask = be.slice(mask.move(), 0, T - S, S)
     attn = be.add(attn.move(), be.broadcast(mask.move(), sh).move())
     m = be.max(attn)
     x = be.sub(attn.move(), be.broadcast(m.move(), sh).move())
@@ -1156,9 +1157,12 @@ def decode_attention_ops(be, q, k_cache, v_cache, rep):
 
 def _np_decode_attention(q, k, v, rep):
     B, kvh, T, hd = k.shape
+    S = q.shape[2]
     kk = np.repeat(k.astype(np.float64), rep, axis=1)
     vv = np.repeat(v.astype(np.float64), rep, axis=1)
     s = q.astype(np.float64) @ kk.transpose(0, 1, 3, 2) / np.float64(np.sqrt(np.float32(hd)))
+    visible = np.arange(T)[None, :] <= (T - S + np.arange(S))[:, None]      # query at position T - S + i sees keys 0 .. T - S + i
+    s = np.where(visible, s, -np.inf)
     s = s - s.max(-1, keepdims=True)
     e = np.exp(s)
     return (e / e.sum(-1, keepdims=True)) @ vv
@@ -1171,6 +1175,24 @@ for _B, _kvh, _rep, _T, _hd in ((2, 2, 4, 300, 64), (1, 3, 1, 1, 64), (2, 1, 8, 
         q = f32(400 + T, (B, kvh * rep, 1, hd))
         k = f32(401 + T, (B, kvh, T, hd))
         v = f32(402 + T, (B, kvh, T, hd))
+
+        def run(be):
+            return N(be, decode_attention_ops(be, be.from_numpy(q), be.from_numpy(k), be.from_numpy(v), rep))
+
+        return run, (lambda: [_np_decode_attention(q, k, v, rep)])
+
+
+# ---- prefill attention: many query positions per head, causal ---------------------------------------------------------
+for _B, _kvh, _rep, _S, _T, _hd in ((1, 2, 4, 48, 48, 64), (2, 1, 1, 128, 128, 64), (1, 2, 2, 200, 333, 64), (2, 2, 4, 96, 96, 64),
+                                     (1, 1, 3, 70, 70, 64), (1, 1, 1, 9, 500, 64), (1, 2, 2, 64, 64, 128), (1, 2, 2, 40, 40, 32)):
+    @case(f"prefill_attention_B{_B}_kv{_kvh}_rep{_rep}_S{_S}_T{_T}_hd{_hd}", "ew_abs")
+    def _(B=_B, kvh=_kvh, rep=_rep, S=_S, T=_T, hd=_hd):
+        """q [B, H, S, hd] against caches of T >= S positions (the last S of them are the queries' own): row tiles
+        that end inside a head or span two heads, a cache longer than the chunk, key tiles cut by the diagonal,
+        head sizes the one-pass kernel declines."""
+        q = f32(450 + S + T, (B, kvh * rep, S, hd))
+        k = f32(451 + S + T, (B, kvh, T, hd))
+        v = f32(452 + S + T, (B, kvh, T, hd))
 
         def run(be):
             return N(be, decode_attention_ops(be, be.from_numpy(q), be.from_numpy(k), be.from_numpy(v), rep))

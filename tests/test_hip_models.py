@@ -136,7 +136,7 @@ def test_pool_returns_to_baseline_after_runs(hip_session):
 def test_decoder_programs_are_compiled_and_match_the_interpreter(hip_session, interp_session, arch):
     """The fused programs that the decoder graphs produce per layer are the ones compiled ahead of
     time: the number of interpreted launches does not grow with the layer count, and the compiled
-    kernels give bit-identical logits to the interpreter."""
+    kernels give the interpreter's logits (bit-identical programs; the one-pass attention to rounding)."""
     interpreted = []
     for layers in (2, 5):
         cfg = LlmConfig(arch, 256, layers, 8, 4, 512, 384, head_dim=64, rope_theta=500000.0, tie_word_embeddings=True)
@@ -157,7 +157,8 @@ def test_decoder_programs_are_compiled_and_match_the_interpreter(hip_session, in
         assert comp_i == 0 and interp_i == comp + interp
         assert comp >= 7 * layers * 5  # at least five programs per layer and run
         interpreted.append(interp)
-        np.testing.assert_array_equal(l_h, l_i)
+        # bit-identical where the same arithmetic runs; the one-pass attention sums in another order
+        np.testing.assert_allclose(l_h, l_i, rtol=1e-4, atol=1e-5)
         np.testing.assert_array_equal(g_h, g_i)
     # what is interpreted does not depend on the depth (the rotary tables: built once, then kept by the backend)
     assert interpreted[1] <= interpreted[0] <= 4

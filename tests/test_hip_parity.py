@@ -137,6 +137,12 @@ def test_decode_attention_runs_as_one_fused_pass(hip):
     compiled, interpreted = hip.program_stats()
     assert (compiled, interpreted) == (1, 0)
     np.testing.assert_allclose(got, _np_decode_attention(q, k, v, 4), rtol=1e-4, atol=1e-5)
+    # the same graph with 200 query positions per head: the one-pass prefill kernel
+    q = f32(4, (2, 8, 200, 64))
+    out = decode_attention_ops(hip, hip.from_numpy(q), hip.from_numpy(k), hip.from_numpy(v), 4)
+    got = hip.to_numpy(out)
+    assert hip.program_stats() == (1, 0)
+    np.testing.assert_allclose(got, _np_decode_attention(q, k, v, 4), rtol=1e-4, atol=1e-5)
 
 
 def test_programs_absorbed_by_decode_time_products(hip):
