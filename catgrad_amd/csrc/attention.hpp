@@ -300,9 +300,9 @@ __global__ __launch_bounds__(kBlock) void decode_attention_combine_kernel(const 
 // [rows, T] score matrix four times (2 GiB per layer of the 1B-shape prefill).  Here a workgroup takes 128
 // query rows of one KV head (a wave 32 of them) and walks the cached positions in tiles of 64, never going
 // beyond the last position its rows may see.  Everything is computed TRANSPOSED, so that a query is a lane:
-//     S^T[t][m] = K[t] . Q[m]          first MFMA operand K (from LDS), second Q (registers, loaded once)
+//     S^T[t][m] = K[t] . Q[m] / scale  first MFMA operand K (from LDS), second Q / scale (registers, loaded once)
 //     running maximum / sum per query  = per lane: in-register over its 32 values + one exchange with lane ^ 32
-//     O^T[d][m] += V^T[d][t] P^T[t][m] first operand V^T (from LDS), second P^T — which, in the accumulator
+//     O^T[d][m] += V^T[d][t] P^T[t][m] first operand V^T (columns of the LDS tile), second P^T — which, in the accumulator
 //                                      layout of v_mfma_f32_32x32x2 (column = lane % 32, rows 8*(v/4) + 4*(lane/32)
 //                                      + v%4), already is the operand layout: no trip through LDS, no transposition
 // The scores are divided by the scale and masked exactly as the soft-max program does (x / d + f32(i < j) * m with
@@ -315,6 +315,8 @@ struct PrefillArgs {
     uint32_t pos0;      // position of the first query row (length of the cache before this chunk)
     uint32_t scale;     // f32 bits of the divisor of the scores
     uint32_t mask_mul;  // f32 bits of the multiplier of the 0/1 mask
+    uint32_t batch;     // folded batch entries (KV heads)
+    uint32_t tiles_per_head; // S / 128 when that is whole and heads are whole in M, else 0
 };
 
 constexpr int kPfRows = 128, kPfKeys = 64, kPfPitch = 68;
@@ -326,11 +328,21 @@ __global__ __launch_bounds__(kBlock) void prefill_attention_kernel(const AttnArg
     typedef float float16v __attribute__((ext_vector_type(16)));
     extern __shared__ float pf_lds[]; // 68 KiB: above the static limit
     float (*Ks)[kPfKeys][kPfPitch] = reinterpret_cast<float (*)[kPfKeys][kPfPitch]>(pf_lds);                       // [2][t][d]
-    float (*Vt)[HD][kPfPitch] = reinterpret_cast<float (*)[HD][kPfPitch]>(pf_lds + 2 * kPfKeys * kPfPitch);        // [2][d][t]
+    float (*Vs)[kPfKeys][kPfPitch] = reinterpret_cast<float (*)[kPfKeys][kPfPitch]>(pf_lds + 2 * kPfKeys * kPfPitch); // [2][t][d]
     const uint32_t tid = threadIdx.x, lane = tid % 64, wave = tid / 64, li = lane % 32, lg = lane / 32;
+    // Work per workgroup grows with the position of its rows inside their head (more visible keys), so the grid
+    // is walked longest first over ALL batch entries and heads: the tail of the launch is made of short ones.
     const uint32_t ntile_rows = (g.M + kPfRows - 1) / kPfRows;
-    const uint32_t rt = ntile_rows - 1 - blockIdx.x; // the longest rows first
-    const uint32_t b = blockIdx.y;
+    uint32_t rt, b;
+    if (e.tiles_per_head) {
+        const uint32_t per_step = e.batch * (ntile_rows / e.tiles_per_head); // workgroups with the same row position
+        const uint32_t step = blockIdx.x / per_step, rest = blockIdx.x % per_step;
+        rt = (rest / e.batch) * e.tiles_per_head + (e.tiles_per_head - 1 - step);
+        b = rest % e.batch;
+    } else { // heads are not whole numbers of row tiles
+        rt = ntile_rows - 1 - blockIdx.x / e.batch;
+        b = blockIdx.x % e.batch;
+    }
     int64_t oq = 0, ok = 0, ov = 0;
     {
         uint32_t bb = b;
@@ -362,12 +374,17 @@ __global__ __launch_bounds__(kBlock) void prefill_attention_kernel(const AttnArg
     }
     const uint32_t ntiles = kmax / kPfKeys + 1;
 
-    // the query rows, as second MFMA operands: chunk c covers d = 8c .. 8c+7, this lane holds 4*lg .. 4*lg+3 of them
+    // the query rows, as second MFMA operands: chunk c covers d = 8c .. 8c+7, this lane holds 4*lg .. 4*lg+3 of them.
+    // The program divides every score by the scale; dividing the query once instead is the same value up to
+    // rounding and takes the division out of the loop.
+    const float scale = asf(e.scale);
     float4v qf[HD / 8];
 #pragma unroll
     for (int c = 0; c < HD / 8; c++) {
         qf[c] = (float4v){0.f, 0.f, 0.f, 0.f};
         if (live) qf[c] = *reinterpret_cast<const float4v *>(g.Q + oq + (int64_t)m * g.q_sm + c * 8 + lg * 4);
+#pragma unroll
+        for (int r = 0; r < 4; r++) qf[c][r] = qf[c][r] / scale;
     }
     float16v acc_o[HD / 32];
 #pragma unroll
@@ -375,7 +392,7 @@ __global__ __launch_bounds__(kBlock) void prefill_attention_kernel(const AttnArg
 #pragma unroll
         for (int v = 0; v < 16; v++) acc_o[db][v] = 0.0f;
     float run_max = -INFINITY, run_sum = 0.0f;
-    const float scale = asf(e.scale);
+    constexpr float kLog2e = 1.4426950408889634f;
 
     // K / V tile: 64 positions x 64 floats each = 1024 float4 per operand, 4 per thread
     float4v kr[4], vr[4];
@@ -396,10 +413,7 @@ __global__ __launch_bounds__(kBlock) void prefill_attention_kernel(const AttnArg
         for (int h = 0; h < 4; h++) {
             const uint32_t slot = tid + h * kBlock, t = slot / 16, dq = slot % 16;
             *reinterpret_cast<float4v *>(&Ks[buf][t][dq * 4]) = kr[h];
-            Vt[buf][dq * 4 + 0][t] = vr[h][0];
-            Vt[buf][dq * 4 + 1][t] = vr[h][1];
-            Vt[buf][dq * 4 + 2][t] = vr[h][2];
-            Vt[buf][dq * 4 + 3][t] = vr[h][3];
+            *reinterpret_cast<float4v *>(&Vs[buf][t][dq * 4]) = vr[h];
         }
     };
     load_kv(0);
@@ -423,36 +437,46 @@ __global__ __launch_bounds__(kBlock) void prefill_attention_kernel(const AttnArg
                 for (int r = 0; r < 4; r++) acc_s[tb] = __builtin_amdgcn_mfma_f32_32x32x2f32(kf[r], qf[c][r], acc_s[tb], 0, 0, 0);
             }
         }
-        // ---- scale, mask, running soft-max statistics of this lane's query
+        // ---- mask, running soft-max statistics of this lane's query.  Weights are 2^((x - max) log2 e) on the
+        // hardware's exp2 (relative error ~1e-6 for the arguments that matter: inside the 1e-4 of element-wise math).
+        // A tile that every query of the wave sees whole (the common case below the diagonal) needs no per-key test.
+        const bool whole = __all((int)(live && t0 + kPfKeys - 1 <= iq && t0 + kPfKeys <= g.T));
         float tile_max = -INFINITY;
+        if (whole) {
 #pragma unroll
-        for (int tb = 0; tb < kPfKeys / 32; tb++)
+            for (int tb = 0; tb < kPfKeys / 32; tb++)
 #pragma unroll
-            for (int v = 0; v < 16; v++) {
-                const uint32_t t = t0 + tb * 32 + 8 * (v / 4) + 4 * lg + (v % 4);
-                // the program's x / d + f32(i < j) * m: nothing is added to a visible key, and an invisible one
-                // (m is hugely negative: the host checks) ends with weight exp(-huge) = 0, so it is left out
-                const float x = acc_s[tb][v] / scale;
-                const bool seen = t <= iq && t < g.T && live;
-                acc_s[tb][v] = seen ? x : -INFINITY;
-                tile_max = fmaxf(tile_max, acc_s[tb][v]);
-            }
+                for (int v = 0; v < 16; v++) tile_max = fmaxf(tile_max, acc_s[tb][v]);
+        } else {
+#pragma unroll
+            for (int tb = 0; tb < kPfKeys / 32; tb++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) {
+                    // the program's x / d + f32(i < j) * m: nothing is added to a visible key, and an invisible one
+                    // (m is hugely negative: the host checks) ends with weight exp(-huge) = 0, so it is left out
+                    const uint32_t t = t0 + tb * 32 + 8 * (v / 4) + 4 * lg + (v % 4);
+                    const bool seen = t <= iq && t < g.T && live;
+                    acc_s[tb][v] = seen ? acc_s[tb][v] : -INFINITY;
+                    tile_max = fmaxf(tile_max, acc_s[tb][v]);
+                }
+        }
         tile_max = fmaxf(tile_max, __shfl_xor(tile_max, 32));
         const float new_max = fmaxf(run_max, tile_max);
-        const float alpha = new_max == -INFINITY ? 1.0f : expf(run_max - new_max);
+        const float base = new_max == -INFINITY ? 0.0f : new_max; // a lane without a live query: keep NaN out
+        const float alpha = __builtin_amdgcn_exp2f((run_max - base) * kLog2e);
         float tile_sum = 0.0f;
 #pragma unroll
         for (int tb = 0; tb < kPfKeys / 32; tb++)
 #pragma unroll
             for (int v = 0; v < 16; v++) {
-                const float p = acc_s[tb][v] == -INFINITY ? 0.0f : expf(acc_s[tb][v] - new_max);
+                const float p = __builtin_amdgcn_exp2f((acc_s[tb][v] - base) * kLog2e); // 2^-inf = 0 for a hidden key
                 acc_s[tb][v] = p;
                 tile_sum += p;
             }
         tile_sum += __shfl_xor(tile_sum, 32);
         run_sum = run_sum * alpha + tile_sum;
         run_max = new_max;
-        // ---- O^T = alpha O^T + V^T P^T
+        // ---- O^T = alpha O^T + V^T P^T: the V operand is read column-wise from the [t][d] tile (32 lanes, 32 banks)
 #pragma unroll
         for (int db = 0; db < HD / 32; db++) {
 #pragma unroll
@@ -461,10 +485,11 @@ __global__ __launch_bounds__(kBlock) void prefill_attention_kernel(const AttnArg
             for (int tb = 0; tb < kPfKeys / 32; tb++)
 #pragma unroll
                 for (int q = 0; q < 4; q++) {
-                    const float4v vf = *reinterpret_cast<const float4v *>(&Vt[cur][db * 32 + li][tb * 32 + q * 8 + lg * 4]);
 #pragma unroll
-                    for (int r = 0; r < 4; r++)
-                        acc_o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(vf[r], acc_s[tb][q * 4 + r], acc_o[db], 0, 0, 0);
+                    for (int r = 0; r < 4; r++) {
+                        const float vf = Vs[cur][tb * 32 + q * 8 + lg * 4 + r][db * 32 + li];
+                        acc_o[db] = __builtin_amdgcn_mfma_f32_32x32x2f32(vf, acc_s[tb][q * 4 + r], acc_o[db], 0, 0, 0);
+                    }
                 }
         }
         if (more) store_kv(cur ^ 1);

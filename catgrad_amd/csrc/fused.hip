@@ -787,11 +787,15 @@ int launch_prefill_attention(cg_backend *be, const Pending &p, const int64_t *pd
     e.pos0 = (uint32_t)lq.offset;
     e.scale = p.leaf[1].ubits;
     e.mask_mul = p.leaf[4].ubits;
+    e.batch = (uint32_t)f1.batch;
+    e.tiles_per_head = S % kPfRows == 0 ? (uint32_t)(S / kPfRows) : 0;
+    const uint64_t nblocks = (uint64_t)((f1.M + kPfRows - 1) / kPfRows) * (uint64_t)f1.batch;
+    if (nblocks > 0x7FFFFFFFull) return pf_declined(be, 17);
     be->programs_compiled++;
     // flop: the visible half of the [rows, T] rectangle, twice (scores and weighted sum)
     const double flop = 2.0 * 2.0 * (double)f1.batch * (double)f1.M * (double)hd * ((double)e.pos0 + 0.5 * (double)S);
     ProfScope prof(be, CG_K_ATTENTION, flop);
-    dim3 grid((uint32_t)((f1.M + kPfRows - 1) / kPfRows), (uint32_t)f1.batch);
+    dim3 grid((uint32_t)nblocks);
     hipLaunchKernelGGL((prefill_attention_kernel<64>), grid, dim3(kBlock), prefill_lds_bytes(64), be->stream, g, e);
     hipError_t err = hipGetLastError();
     return err == hipSuccess ? CG_OK : hip_fail(err, "prefill attention launch");
