@@ -36,7 +36,7 @@ MFMA_F32_PEAK = 157.3e12  # flop/s, MI355X dense f32 matrix
 # HBM bytes per mfma_gemm_kernel launch of this workload's prefill, from rocprofv3 FETCH_SIZE / WRITE_SIZE passes
 # scaled by a copy kernel of known size (profiles/mfma_gemm_llama1b_prefill_pmc.txt); counters cannot be read
 # from inside this process, so the figure is carried here and only reported for the profiled shape.
-MFMA_GEMM_TRAFFIC_PER_LAUNCH = 1.055e9
+MFMA_GEMM_TRAFFIC_PER_LAUNCH = 0.691e9
 
 
 def micro_bench(iters=20):
@@ -170,8 +170,10 @@ def main():
         sess.generate(prompt, steps=T, max_positions=S + T)
     sess.profile_enable(A.K_GEMM_MFMA, 1)
     sess.profile_enable(A.K_GEMM_SKINNY, 8)
+    sess.profile_enable(A.K_ATTENTION, 1)
     sess.profile_read(A.K_GEMM_MFMA, reset=True)
     sess.profile_read(A.K_GEMM_SKINNY, reset=True)
+    sess.profile_read(A.K_ATTENTION, reset=True)
 
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -188,8 +190,11 @@ def main():
 
     n_m, ms_m, flop_m = sess.profile_read(A.K_GEMM_MFMA)
     n_s, ms_s, bytes_s = sess.profile_read(A.K_GEMM_SKINNY)
+    n_a, ms_a, flop_a = sess.profile_read(A.K_ATTENTION)
     sess.profile_enable(A.K_GEMM_MFMA, 0)
     sess.profile_enable(A.K_GEMM_SKINNY, 0)
+    sess.profile_enable(A.K_ATTENTION, 0)
+    attn_rate = flop_a / (ms_a * 1e-3) if ms_a else 0.0
     mfma_rate = flop_m / (ms_m * 1e-3) if ms_m else 0.0
     skinny_rate = bytes_s / (ms_s * 1e-3) if ms_s else 0.0
 
@@ -236,6 +241,13 @@ def main():
             "traffic": MFMA_GEMM_TRAFFIC_PER_LAUNCH if (B, S) == (4, 2048) else None,
             "launches_timed": n_m, "avg_launch_ms": round(ms_m / max(n_m, 1), 4),
             "flop_per_launch_avg": flop_m / max(n_m, 1),
+        },
+        # the one-pass causal attention of the prefill (q.K^T, soft-max, p.V): flop of the visible half only
+        "prefill_attention": {
+            "kernel": "prefill_attention_kernel (f32 v_mfma_f32_32x32x2, 128 query rows x 64 keys per step)",
+            "bound": "mfma", "achieved": round(attn_rate / 1e12, 3), "peak": MFMA_F32_PEAK / 1e12, "unit": "TFLOP/s",
+            "frac": round(attn_rate / MFMA_F32_PEAK, 4), "launches_timed": n_a,
+            "avg_launch_ms": round(ms_a / max(n_a, 1), 4),
         },
         "decode_roofline": {
             "scope": "one decode step, all kernels: every weight matrix and the KV cache are read once",
