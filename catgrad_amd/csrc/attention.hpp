@@ -319,14 +319,17 @@ struct PrefillArgs {
     uint32_t tiles_per_head; // S / 128 when that is whole and heads are whole in M, else 0
 };
 
-constexpr int kPfRows = 128, kPfKeys = 64, kPfPitch = 68;
-constexpr size_t prefill_lds_bytes(int hd) { return 2 * (size_t)(kPfKeys + hd) * kPfPitch * sizeof(float); }
+constexpr int kPfRows = 128, kPfKeys = 64;
+// K and V tiles, [64 keys][head_dim + 4] each (a row starts 4 banks after the one before), double buffered:
+// 68 KiB for head_dim 64 (two workgroups per CU), 132 KiB for 128 (one)
+constexpr size_t prefill_lds_bytes(int hd) { return 2 * 2 * (size_t)kPfKeys * (hd + 4) * sizeof(float); }
 
 template <int HD>
 __global__ __launch_bounds__(kBlock) void prefill_attention_kernel(const AttnArgs g, const PrefillArgs e) {
-    static_assert(HD == 64, "written for head_dim 64");
+    static_assert(HD == 64 || HD == 128, "head_dim 64 or 128");
+    constexpr int kPfPitch = HD + 4;
     typedef float float16v __attribute__((ext_vector_type(16)));
-    extern __shared__ float pf_lds[]; // 68 KiB: above the static limit
+    extern __shared__ float pf_lds[]; // above the static limit
     float (*Ks)[kPfKeys][kPfPitch] = reinterpret_cast<float (*)[kPfKeys][kPfPitch]>(pf_lds);                       // [2][t][d]
     float (*Vs)[kPfKeys][kPfPitch] = reinterpret_cast<float (*)[kPfKeys][kPfPitch]>(pf_lds + 2 * kPfKeys * kPfPitch); // [2][t][d]
     const uint32_t tid = threadIdx.x, lane = tid % 64, wave = tid / 64, li = lane % 32, lg = lane / 32;
@@ -394,12 +397,13 @@ __global__ __launch_bounds__(kBlock) void prefill_attention_kernel(const AttnArg
     float run_max = -INFINITY, run_sum = 0.0f;
     constexpr float kLog2e = 1.4426950408889634f;
 
-    // K / V tile: 64 positions x 64 floats each = 1024 float4 per operand, 4 per thread
-    float4v kr[4], vr[4];
+    // K / V tile: 64 positions x HD floats each = 16 * HD float4 per operand, HD / 16 per thread
+    constexpr int kSlots = kPfKeys * (HD / 4) / kBlock, kQpr = HD / 4;
+    float4v kr[kSlots], vr[kSlots];
     auto load_kv = [&](uint32_t t0) {
 #pragma unroll
-        for (int h = 0; h < 4; h++) {
-            const uint32_t slot = tid + h * kBlock, t = t0 + slot / 16, dq = slot % 16;
+        for (int h = 0; h < kSlots; h++) {
+            const uint32_t slot = tid + h * kBlock, t = t0 + slot / kQpr, dq = slot % kQpr;
             kr[h] = (float4v){0.f, 0.f, 0.f, 0.f};
             vr[h] = (float4v){0.f, 0.f, 0.f, 0.f};
             if (t < g.T) {
@@ -410,8 +414,8 @@ __global__ __launch_bounds__(kBlock) void prefill_attention_kernel(const AttnArg
     };
     auto store_kv = [&](uint32_t buf) {
 #pragma unroll
-        for (int h = 0; h < 4; h++) {
-            const uint32_t slot = tid + h * kBlock, t = slot / 16, dq = slot % 16;
+        for (int h = 0; h < kSlots; h++) {
+            const uint32_t slot = tid + h * kBlock, t = slot / kQpr, dq = slot % kQpr;
             *reinterpret_cast<float4v *>(&Ks[buf][t][dq * 4]) = kr[h];
             *reinterpret_cast<float4v *>(&Vs[buf][t][dq * 4]) = vr[h];
         }

@@ -736,7 +736,7 @@ int launch_prefill_attention(cg_backend *be, const Pending &p, const int64_t *pd
                 (long long)f1.M, (long long)f1.N, (long long)f1.K, (long long)f1.batch, f1.nb, (long long)f2.M, (long long)f2.N,
                 (long long)f2.K, (long long)f2.batch, f2.nb, (long long)S, (long long)T);
     if (f1.N != T || f1.M != f2.M || f1.M <= kAttnRows || f1.M % S != 0 || f1.batch != f2.batch || f2.K != T || f2.N != hd) return pf_declined(be, 8);
-    if (hd != 64) return pf_declined(be, 9);
+    if (hd != 64 && hd != 128) return pf_declined(be, 9);
     if (f1.a_sk != 1 || f1.b_sk != 1 || f2.b_sn != 1 || f2.a_sk != 1 || f2.a_sm != T) return pf_declined(be, 10);
     if (f1.batch < 1 || f1.batch > 65535 || T < 1 || T > 0x7FFFFFFFll || f1.M > 0x7FFFFFFFll) return pf_declined(be, 11);
     for (int d = 0; d < f1.nb; d++)
@@ -755,7 +755,10 @@ int launch_prefill_attention(cg_backend *be, const Pending &p, const int64_t *pd
         return pf_declined(be, 15);
     static const bool lds_ok = hipFuncSetAttribute(reinterpret_cast<const void *>(&prefill_attention_kernel<64>),
                                                    hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                   (int)prefill_lds_bytes(64)) == hipSuccess;
+                                                   (int)prefill_lds_bytes(64)) == hipSuccess &&
+                               hipFuncSetAttribute(reinterpret_cast<const void *>(&prefill_attention_kernel<128>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                   (int)prefill_lds_bytes(128)) == hipSuccess;
     if (!lds_ok) return pf_declined(be, 16);
     AttnArgs g;
     memset(&g, 0, sizeof g);
@@ -796,7 +799,10 @@ int launch_prefill_attention(cg_backend *be, const Pending &p, const int64_t *pd
     const double flop = 2.0 * 2.0 * (double)f1.batch * (double)f1.M * (double)hd * ((double)e.pos0 + 0.5 * (double)S);
     ProfScope prof(be, CG_K_ATTENTION, flop);
     dim3 grid((uint32_t)nblocks);
-    hipLaunchKernelGGL((prefill_attention_kernel<64>), grid, dim3(kBlock), prefill_lds_bytes(64), be->stream, g, e);
+    if (hd == 64)
+        hipLaunchKernelGGL((prefill_attention_kernel<64>), grid, dim3(kBlock), prefill_lds_bytes(64), be->stream, g, e);
+    else
+        hipLaunchKernelGGL((prefill_attention_kernel<128>), grid, dim3(kBlock), prefill_lds_bytes(128), be->stream, g, e);
     hipError_t err = hipGetLastError();
     return err == hipSuccess ? CG_OK : hip_fail(err, "prefill attention launch");
 }

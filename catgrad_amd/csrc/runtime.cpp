@@ -2248,8 +2248,8 @@ static int matmul_entry(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **o
         int64_t n_out = 1;
         for (int i = 0; i < r; i++) n_out *= od[i];
         const int64_t K = x->dims[r - 1];
-        // (few rows: a decode step; many rows: a prefill, whose one-pass kernel takes head_dim 64 only)
-        const bool scores = r == 4 && K > 0 && K <= 256 && od[r - 1] > 1 && (x->dims[r - 2] <= 8 || (K == 64 && b->aot));
+        // (few rows: a decode step; many rows: a prefill, whose one-pass kernel takes head_dim 64 and 128)
+        const bool scores = r == 4 && K > 0 && K <= 256 && od[r - 1] > 1 && (x->dims[r - 2] <= 8 || ((K == 64 || K == 128) && b->aot));
         // a decode-time linear layer: at most 8 rows in all, the weight shared by the batch
         const bool linear = r == 3 && x->dims[0] * x->dims[1] <= 8 && K > 256 && od[r - 1] >= 64 && y->strides[0] == 0 &&
                             y->split < 0 && is_contiguous(x);

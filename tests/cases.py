@@ -1184,7 +1184,8 @@ for _B, _kvh, _rep, _T, _hd in ((2, 2, 4, 300, 64), (1, 3, 1, 1, 64), (2, 1, 8, 
 
 # ---- prefill attention: many query positions per head, causal ---------------------------------------------------------
 for _B, _kvh, _rep, _S, _T, _hd in ((1, 2, 4, 48, 48, 64), (2, 1, 1, 128, 128, 64), (1, 2, 2, 200, 333, 64), (2, 2, 4, 96, 96, 64),
-                                     (1, 1, 3, 70, 70, 64), (1, 1, 1, 9, 500, 64), (1, 2, 2, 64, 64, 128), (1, 2, 2, 40, 40, 32)):
+                                     (1, 1, 3, 70, 70, 64), (1, 1, 1, 9, 500, 64), (1, 2, 2, 64, 64, 128), (2, 1, 4, 200, 333, 128),
+                                     (1, 2, 2, 40, 40, 32)):
     @case(f"prefill_attention_B{_B}_kv{_kvh}_rep{_rep}_S{_S}_T{_T}_hd{_hd}", "ew_abs")
     def _(B=_B, kvh=_kvh, rep=_rep, S=_S, T=_T, hd=_hd):
         """q [B, H, S, hd] against caches of T >= S positions (the last S of them are the queries' own): row tiles

@@ -143,6 +143,11 @@ def test_decode_attention_runs_as_one_fused_pass(hip):
     got = hip.to_numpy(out)
     assert hip.program_stats() == (1, 0)
     np.testing.assert_allclose(got, _np_decode_attention(q, k, v, 4), rtol=1e-4, atol=1e-5)
+    # head_dim 128, a cache longer than the chunk
+    q, k, v = f32(5, (1, 4, 100, 128)), f32(6, (1, 2, 150, 128)), f32(7, (1, 2, 150, 128))
+    got = hip.to_numpy(decode_attention_ops(hip, hip.from_numpy(q), hip.from_numpy(k), hip.from_numpy(v), 2))
+    assert hip.program_stats() == (1, 0)
+    np.testing.assert_allclose(got, _np_decode_attention(q, k, v, 2), rtol=1e-4, atol=1e-5)
 
 
 def test_programs_absorbed_by_decode_time_products(hip):
