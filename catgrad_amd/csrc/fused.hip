@@ -731,10 +731,6 @@ int launch_prefill_attention(cg_backend *be, const Pending &p, const int64_t *pd
     MmFold f1, f2;
     if (fold_matmul(q, kt, &f1) || fold_matmul(&pd, v, &f2)) return pf_declined(be, 7);
     const int64_t hd = f1.K;
-    if (be->trace_programs)
-        fprintf(stderr, "[cg program] prefill attention: q.K^T M %lld N %lld K %lld batch %lld nb %d; p.V M %lld N %lld K %lld batch %lld nb %d; S %lld T %lld\n",
-                (long long)f1.M, (long long)f1.N, (long long)f1.K, (long long)f1.batch, f1.nb, (long long)f2.M, (long long)f2.N,
-                (long long)f2.K, (long long)f2.batch, f2.nb, (long long)S, (long long)T);
     if (f1.N != T || f1.M != f2.M || f1.M <= kAttnRows || f1.M % S != 0 || f1.batch != f2.batch || f2.K != T || f2.N != hd) return pf_declined(be, 8);
     if (hd != 64 && hd != 128) return pf_declined(be, 9);
     if (f1.a_sk != 1 || f1.b_sk != 1 || f2.b_sn != 1 || f2.a_sk != 1 || f2.a_sm != T) return pf_declined(be, 10);
