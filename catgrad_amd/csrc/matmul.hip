@@ -67,7 +67,9 @@ __device__ __forceinline__ void batch_offsets(const MmArgs &a, uint32_t b, int64
 // ------------------------------------------------------------------------------------------
 constexpr int BM = 128, BN = 128, BK = 32; // BN = 64 in the narrow variant
 constexpr int PITCH = BK + 4; // words per LDS row: row r starts at bank 4r mod 32
-constexpr size_t gemm_lds_bytes(int bn, int bm = BM) { return 2 * (size_t)(bm + bn) * PITCH * sizeof(float); }
+constexpr size_t gemm_lds_bytes(int bn, int bm = BM, bool half = false) {
+    return 2 * (size_t)(bm + bn) * (half ? BK / 2 + 4 : PITCH) * sizeof(float);
+}
 constexpr int kThreads = 256;
 constexpr uint32_t kXcds = 8, kGroupM = 8;
 
@@ -139,17 +141,68 @@ template <bool ROWS_FAST, int TR> __device__ __forceinline__ void store_tile(con
     }
 }
 
+// ---- the 16-bit float dtypes on their own matrix instructions ------------------------------------------------
+// Tensors of these dtypes hold f32 words with exactly representable values, so a tile is narrowed to its 16-bit
+// patterns on the way into LDS (exact: the upper half of the word for bfloat16, v_cvt_f16_f32 for binary16) and the
+// products run on v_mfma_f32_32x32x16_{bf16,f16}: 16 k per instruction instead of 2, f32 accumulation as before.
+// LDS rows hold BK/2 words + 4 of padding (a row starts 20 banks after the one before: 8 lanes of a 128-bit
+// read cover all 32 banks); a lane's 128-bit read is its 8 consecutive k of one 16-deep chunk.
+constexpr int PITCH_H = BK / 2 + 4;
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+
+// HALF: 1 bfloat16, 2 binary16
+template <int HALF> __device__ __forceinline__ uint32_t pack_halves(float lo, float hi) {
+    if constexpr (HALF == 1) return (asu(lo) >> 16) | (asu(hi) & 0xFFFF0000u);
+    return (uint32_t)__half_as_ushort(__float2half_rn(lo)) | ((uint32_t)__half_as_ushort(__float2half_rn(hi)) << 16);
+}
+template <int HALF> __device__ __forceinline__ uint16_t narrow_half(float v) {
+    if constexpr (HALF == 1) return (uint16_t)(asu(v) >> 16);
+    return __half_as_ushort(__float2half_rn(v));
+}
+
+// Stores the registers K-fastest into an LDS tile [TR][PITCH_H] of 16-bit patterns.
+template <bool ROWS_FAST, int HALF, int TR> __device__ __forceinline__ void store_tile_half(const TileRegs<TR> &t, uint32_t *lds) {
+#pragma unroll
+    for (int h = 0; h < TileRegs<TR>::slots; h++) {
+        uint32_t slot = threadIdx.x + h * kThreads;
+        if (!ROWS_FAST) {
+            uint32_t row = slot / (BK / 4), k = (slot % (BK / 4)) * 4;
+            uint2 w;
+            w.x = pack_halves<HALF>(t.v[h][0], t.v[h][1]);
+            w.y = pack_halves<HALF>(t.v[h][2], t.v[h][3]);
+            *reinterpret_cast<uint2 *>(lds + row * PITCH_H + k / 2) = w;
+        } else {
+            uint32_t k = slot / (TR / 4), row = (slot % (TR / 4)) * 4;
+            uint16_t *l16 = reinterpret_cast<uint16_t *>(lds);
+#pragma unroll
+            for (int i = 0; i < 4; i++) l16[(row + i) * (PITCH_H * 2) + k] = narrow_half<HALF>(t.v[h][i]);
+        }
+    }
+}
+
 // NT / MT: 32-wide MFMA tiles per wave along N / M (the block is 2 x 2 waves).  NT = 2, MT = 2: the
 // 128 x 128 macro tile; NT = 1: 128 x 64 (each wave a 64 x 32 strip) for products whose N is a small
 // multiple of 64, such as p.V with head_dim 64; NT = MT = 4: 256 x 256, each wave a 128 x 128 block in
 // 256 accumulation registers, one wave per SIMD: four times the matrix instructions between two
 // barriers and half the LDS traffic per flop, for products with enough tiles to fill the chip.
-template <bool A_MFAST, bool B_NFAST, int NT, int MT = 2>
+// HALF: 0 f32 operands (v_mfma_f32_32x32x2_f32); 1 / 2: bfloat16 / binary16 operands (see above).
+template <bool A_MFAST, bool B_NFAST, int NT, int MT = 2, int HALF = 0>
 __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
     constexpr int BN = 64 * NT, BM = 64 * MT; // shadow the defaults
-    extern __shared__ float lds_dyn[]; // [2][BM][PITCH] for A, then [2][BN][PITCH] for B
-    auto lds_a = [&](uint32_t buf) { return lds_dyn + buf * (BM * PITCH); };
-    auto lds_b = [&](uint32_t buf) { return lds_dyn + 2 * BM * PITCH + buf * (BN * PITCH); };
+    constexpr int LP = HALF ? PITCH_H : PITCH; // words per LDS row
+    extern __shared__ float lds_dyn[]; // [2][BM][LP] for A, then [2][BN][LP] for B
+    auto lds_a = [&](uint32_t buf) { return lds_dyn + buf * (BM * LP); };
+    auto lds_b = [&](uint32_t buf) { return lds_dyn + 2 * BM * LP + buf * (BN * LP); };
+    auto stage = [&](const TileRegs<BM> &ta, const TileRegs<BN> &tb, uint32_t buf) {
+        if constexpr (HALF) {
+            store_tile_half<A_MFAST, HALF>(ta, reinterpret_cast<uint32_t *>(lds_a(buf)));
+            store_tile_half<B_NFAST, HALF>(tb, reinterpret_cast<uint32_t *>(lds_b(buf)));
+        } else {
+            store_tile<A_MFAST>(ta, lds_a(buf));
+            store_tile<B_NFAST>(tb, lds_b(buf));
+        }
+    };
 
     // Tile order.  Workgroups are dealt round-robin to the 8 XCDs, each with its own L2, so
     // the linear id is first regrouped to give every XCD one contiguous run of tiles; inside
@@ -193,8 +246,7 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
     const uint32_t nk = (a.K + BK - 1) / BK;
     load_tile<A_MFAST>(ra, A, a.a_sm, a.a_sk, m0, 0, a.M, a.K, a.a_vec);
     load_tile<B_NFAST>(rb, B, a.b_sn, a.b_sk, n0, 0, a.N, a.K, a.b_vec);
-    store_tile<A_MFAST>(ra, lds_a(0));
-    store_tile<B_NFAST>(rb, lds_b(0));
+    stage(ra, rb, 0);
     __syncthreads();
 
     for (uint32_t kt = 0; kt < nk; kt++) {
@@ -227,13 +279,35 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
             load_tile<B_NFAST>(rb, B, a.b_sn, a.b_sk, n0, (kt + 1) * BK, a.N, a.K, a.b_vec);
         }
         __builtin_amdgcn_s_setprio(1);
+        if constexpr (HALF) {
+            // 16-deep chunks: lane group g supplies k = 16*kc + 8*g .. + 7, one 128-bit LDS read per operand block
 #pragma unroll
-        for (int kc = 0; kc < BK / 8; kc++) chunk(kc);
-        __builtin_amdgcn_s_setprio(0);
-        if (more) {
-            store_tile<A_MFAST>(ra, lds_a(cur ^ 1));
-            store_tile<B_NFAST>(rb, lds_b(cur ^ 1));
+            for (int kc = 0; kc < BK / 16; kc++) {
+                float4v fa[MT], fb[NT];
+#pragma unroll
+                for (int i = 0; i < MT; i++)
+                    fa[i] = *reinterpret_cast<const float4v *>(la + (wm + i * 32 + li) * PITCH_H + kc * 8 + lg * 4);
+#pragma unroll
+                for (int j = 0; j < NT; j++)
+                    fb[j] = *reinterpret_cast<const float4v *>(lb + (wn + j * 32 + li) * PITCH_H + kc * 8 + lg * 4);
+#pragma unroll
+                for (int i = 0; i < MT; i++)
+#pragma unroll
+                    for (int j = 0; j < NT; j++) {
+                        if constexpr (HALF == 1)
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fa[i]),
+                                                                                __builtin_bit_cast(bf16x8, fb[j]), acc[i][j], 0, 0, 0);
+                        else
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, fa[i]),
+                                                                               __builtin_bit_cast(f16x8, fb[j]), acc[i][j], 0, 0, 0);
+                    }
+            }
+        } else {
+#pragma unroll
+            for (int kc = 0; kc < BK / 8; kc++) chunk(kc);
         }
+        __builtin_amdgcn_s_setprio(0);
+        if (more) stage(ra, rb, cur ^ 1);
         __syncthreads();
     }
 
@@ -890,6 +964,7 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
 
     if (batch > 65535) return fail(CG_ERR_UNSUPPORTED, "matmul: more than 65535 batch entries after folding");
     const bool f32 = is_f(x->dt);
+    const int half = x->dt == CG_BF16 ? 1 : x->dt == CG_F16 ? 2 : 0; // operands of the 16-bit matrix instructions
     hipStream_t s = be->stream;
     const double flop = 2.0 * (double)M * (double)N * (double)K * (double)batch;
     const double bytes = distinct_bytes(x) + distinct_bytes(y) + distinct_bytes(out);
@@ -976,7 +1051,7 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
     } else {
         // the narrow tile when the wide one would leave over a seventh of its columns empty
         const int64_t cols128 = (N + 127) / 128 * 128, cols64 = (N + 63) / 64 * 64;
-        const bool narrow = cols128 * 7 > cols64 * 8;
+        const bool narrow = cols128 * 7 > cols64 * 8 && !half; // (the 16-bit kernels come in the two square tiles)
         const int bn = narrow ? 64 : 128;
         // the 256 x 256 tile when it covers the chip at least once (env CG_GEMM_BIG=0 switches it off)
         const uint64_t tiles_big = (uint64_t)((M + 255) / 256) * ((N + 255) / 256) * batch;
@@ -996,15 +1071,30 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
     ok &= hipFuncSetAttribute(reinterpret_cast<const void *>(&mfma_gemm_kernel<AF, BF, 1>),                           \
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds_bytes(64)) == hipSuccess;     \
     ok &= hipFuncSetAttribute(reinterpret_cast<const void *>(&mfma_gemm_kernel<AF, BF, 4, 4>),                        \
-                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds_bytes(256, 256)) == hipSuccess;
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds_bytes(256, 256)) == hipSuccess; \
+    ok &= hipFuncSetAttribute(reinterpret_cast<const void *>(&mfma_gemm_kernel<AF, BF, 4, 4, 1>),                     \
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds_bytes(256, 256, true)) == hipSuccess; \
+    ok &= hipFuncSetAttribute(reinterpret_cast<const void *>(&mfma_gemm_kernel<AF, BF, 4, 4, 2>),                     \
+                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds_bytes(256, 256, true)) == hipSuccess;
             CG_LDS(true, true) CG_LDS(true, false) CG_LDS(false, true) CG_LDS(false, false)
 #undef CG_LDS
             return ok;
         }();
         if (!lds_ok) return fail(CG_ERR_DEVICE, "matmul: cannot reserve %zu bytes of LDS", gemm_lds_bytes(128));
-#define CG_GEMM(AF, BF)                                                                                            \
+#define CG_GEMM_HALF(AF, BF, H)                                                                                    \
     do {                                                                                                           \
         if (big)                                                                                                   \
+            hipLaunchKernelGGL((mfma_gemm_kernel<AF, BF, 4, 4, H>), grid, dim3(kThreads), gemm_lds_bytes(256, 256, true), s, a); \
+        else                                                                                                       \
+            hipLaunchKernelGGL((mfma_gemm_kernel<AF, BF, 2, 2, H>), grid, dim3(kThreads), gemm_lds_bytes(128, 128, true), s, a); \
+    } while (0)
+#define CG_GEMM(AF, BF)                                                                                            \
+    do {                                                                                                           \
+        if (half == 1) {                                                                                           \
+            CG_GEMM_HALF(AF, BF, 1);                                                                               \
+        } else if (half == 2) {                                                                                    \
+            CG_GEMM_HALF(AF, BF, 2);                                                                               \
+        } else if (big)                                                                                            \
             hipLaunchKernelGGL((mfma_gemm_kernel<AF, BF, 4, 4>), grid, dim3(kThreads), gemm_lds_bytes(256, 256), s, a); \
         else if (narrow)                                                                                           \
             hipLaunchKernelGGL((mfma_gemm_kernel<AF, BF, 1>), grid, dim3(kThreads), gemm_lds_bytes(64), s, a);     \
@@ -1019,6 +1109,7 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
             else CG_GEMM(false, false);
         }
 #undef CG_GEMM
+#undef CG_GEMM_HALF
     }
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? CG_OK : hip_fail(e, "matmul launch");

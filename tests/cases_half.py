@@ -273,6 +273,35 @@ for _dt in (A.F16, A.BF16):
         return run, expect
 
 
+for _dt in (A.F16, A.BF16):
+    @case(f"half_{NAMES[_dt]}_matmul_mfma_tiles", "ulp_" + NAMES[_dt])
+    def _(dt=_dt):
+        """Products large enough for the 16-bit matrix instructions in both macro tiles (256 x 256 needs 256 of them),
+        all four operand layouts, ragged edges and a k tail that is not a multiple of the tile depth."""
+        ux, x = half_inputs(dt, 850, (64, 512, 40), 1.0)
+        uw, w = half_inputs(dt, 851, (64, 40, 512), 1.0)
+        ux, uw = round_to(dt, np.abs(x)), round_to(dt, np.abs(w))
+        x, w = as_f32(dt, ux), as_f32(dt, uw)
+        ur, r = half_inputs(dt, 852, (43, 300, 70), 1.0)
+        us, s_ = half_inputs(dt, 853, (43, 70, 520), 1.0)
+        ur, us = round_to(dt, np.abs(r)), round_to(dt, np.abs(s_))
+        r, s_ = as_f32(dt, ur), as_f32(dt, us)
+
+        def run(be):
+            tx, tw, tr, ts = (from_half(be, dt, u) for u in (ux, uw, ur, us))
+            outs = [be.matmul(tx, tw), be.matmul(tr, ts),
+                    be.matmul(be.transpose(ts, 1, 2), be.transpose(tr, 1, 2)),                       # both operands transposed
+                    be.matmul(be.slice(tr, 1, 0, 150), ts)]                                          # 128 x 128 tiles
+            assert all(o.dtype == dt for o in outs)
+            return [as_f32(dt, read(be, o)) for o in outs]
+
+        def expect():
+            x64, w64, r64, s64 = (a.astype(np.float64) for a in (x, w, r, s_))
+            return [x64 @ w64, r64 @ s64, (r64 @ s64).transpose(0, 2, 1), r64[:, :150] @ s64]
+
+        return run, expect
+
+
 # ---- shape and index ops carry the dtype --------------------------------------------------------------------------
 for _dt in (A.F16, A.BF16):
     @case(f"half_{NAMES[_dt]}_views_concat_index")
