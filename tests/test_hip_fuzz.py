@@ -1,0 +1,215 @@
+"""Seeded random op graphs, HipBackend against the CPU oracle.
+
+Each graph is a short random program over a few small f32 tensors: element-wise ops, row reductions broadcast
+back over their rows, views (transpose / slice / reshape / broadcast), last- and inner-axis concats, casts and a
+gather — the mix that exercises the deferred-program engine (splicing, shared sub-expressions, row programs,
+piecewise leaves, views of deferred results) in combinations the hand-written cases do not enumerate.  Every
+node carries a bound on its magnitude, graphs stay below 1e6, and the comparison is the element-wise tolerance of
+the contract (rtol 1e-4) plus an absolute term of 1e-5 of the node's bound, which covers differences that a
+subtraction of nearly equal values amplifies."""
+import numpy as np
+import pytest
+
+from catgrad_amd import _abi as A
+
+pytestmark = pytest.mark.gpu
+
+LIMIT = 1e6
+
+
+class Node:
+    """`fn(be, *parent tensors)` builds this node; `hi` bounds |values|; `exact` says that every op on the way
+    here rounds identically on any IEEE f32 implementation (no exp / sin / cos, no sum whose order may differ), so
+    a discontinuous op (floor, round, a comparison, a mask, a truncating cast) may follow it."""
+
+    def __init__(self, fn, parents, shape, hi, exact):
+        self.fn, self.parents, self.shape, self.hi, self.exact = fn, parents, tuple(shape), hi, exact
+
+
+def const(be, v, shape):
+    return be.broadcast(be.from_numpy(np.array(v, np.float32)), shape)
+
+
+def random_graph(rng):
+    """Returns (inputs, nodes, outputs): numpy inputs, all nodes in build order, and the nodes to read back."""
+    depth = int(rng.integers(6, 30))
+    base = (int(rng.integers(1, 4)), int(rng.integers(1, 7)), int(rng.choice([1, 3, 8, 16, 33, 64, 130, 256, 1000, 2048])))
+    inputs = [rng.uniform(0.25, 2.0, size=base).astype(np.float32) for _ in range(3)]
+    nodes = [Node(None, (), base, 2.0, True) for _ in range(3)]
+
+    def pick(shape=None):
+        c = [n for n in nodes if shape is None or n.shape == tuple(shape)]
+        return c[int(rng.integers(0, len(c)))]
+
+    def add(fn, parents, shape, hi, inexact=False, needs_exact=()):
+        if hi <= LIMIT and all(s > 0 for s in shape) and all(p.exact for p in needs_exact):
+            nodes.append(Node(fn, parents, shape, hi, not inexact and all(p.exact for p in parents)))
+
+    kinds = ["unary", "binary", "binary", "binary", "where", "rowsum", "rowmax", "transpose", "slice", "reshape",
+             "rotate_half", "concat_last", "concat_inner", "cast", "index", "scalar"]
+    for _ in range(depth):
+        kind = str(rng.choice(kinds))
+        x = pick()
+        last = len(x.shape) - 1
+        if kind == "unary":
+            op = str(rng.choice(["neg", "gauss", "floor", "round", "sin", "cos", "square"]))
+            if op == "gauss":      # exp(-x^2), in (0, 1]
+                add(lambda be, a: be.exp(be.neg(be.mul(a, a))), (x,), x.shape, 1.0, inexact=True)
+            elif op == "square":
+                add(lambda be, a: be.mul(a, a), (x,), x.shape, x.hi * x.hi)
+            elif op in ("sin", "cos"):
+                if x.hi <= 64.0:   # the contract's tolerance for sin / cos holds for moderate arguments
+                    add(lambda be, a, op=op: getattr(be, op)(a), (x,), x.shape, 1.0, inexact=True)
+            else:
+                add(lambda be, a, op=op: getattr(be, op)(a), (x,), x.shape, x.hi + 1.0, needs_exact=() if op == "neg" else (x,))
+        elif kind == "binary":
+            y = pick(x.shape)
+            op = str(rng.choice(["add", "mul", "sub", "ratio", "lt", "gte"]))
+            if op == "ratio":      # x / (y^2 + 0.5)
+                add(lambda be, a, b, s=x.shape: be.div(a, be.add(be.mul(b, b), const(be, 0.5, s))), (x, y), x.shape, 2 * x.hi)
+            else:
+                hi = {"add": x.hi + y.hi, "sub": x.hi + y.hi, "mul": x.hi * y.hi}.get(op, 1.0)
+                add(lambda be, a, b, op=op: getattr(be, op)(a, b), (x, y), x.shape, hi, needs_exact=(x, y) if op in ("lt", "gte") else ())
+        elif kind == "where":
+            y, m = pick(x.shape), pick(x.shape)
+            add(lambda be, a, b, c, s=x.shape: be.where_cond(be.sub(c, const(be, 1.0, s)), a, b), (x, y, m), x.shape, max(x.hi, y.hi),
+                needs_exact=(m,))
+        elif kind == "rowsum":     # x / (1 + sum x^2): positive terms, no cancellation inside the sum
+            add(lambda be, a, s=x.shape: be.div(a, be.add(be.broadcast(be.sum(be.mul(a, a)), s), const(be, 1.0, s))), (x,), x.shape, x.hi,
+                inexact=True)
+        elif kind == "rowmax":     # x - max x, the softmax shift
+            add(lambda be, a, s=x.shape: be.sub(a, be.broadcast(be.max(a), s)), (x,), x.shape, 2 * x.hi)
+        elif kind == "transpose" and len(x.shape) >= 2:
+            i, j = sorted(rng.choice(len(x.shape), size=2, replace=False).tolist())
+            shp = list(x.shape)
+            shp[i], shp[j] = shp[j], shp[i]
+            add(lambda be, a, i=i, j=j: be.transpose(a, i, j), (x,), shp, x.hi)
+        elif kind == "slice":
+            d = int(rng.integers(0, len(x.shape)))
+            if x.shape[d] >= 2:
+                start = int(rng.integers(0, x.shape[d] - 1))
+                ln = int(rng.integers(1, x.shape[d] - start + 1))
+                shp = list(x.shape)
+                shp[d] = ln
+                add(lambda be, a, d=d, start=start, ln=ln: be.slice(a, d, start, ln), (x,), shp, x.hi)
+        elif kind == "reshape":
+            n = int(np.prod(x.shape))
+            shp = (n,) if rng.random() < 0.3 else (n // x.shape[-1], x.shape[-1])
+            add(lambda be, a, shp=shp: be.reshape(a, shp), (x,), shp, x.hi)
+        elif kind == "rotate_half":    # concat(-x[.., h:], x[.., :h]): one tensor read piecewise
+            h = x.shape[-1] // 2
+            if h >= 1:
+                w = x.shape[-1]
+                add(lambda be, a, h=h, w=w, last=last: be.concat(be.neg(be.slice(a, last, h, w - h)), be.slice(a, last, 0, h), last),
+                    (x,), x.shape, x.hi)
+        elif kind == "concat_last":
+            y = pick(x.shape)
+            add(lambda be, a, b, last=last: be.concat(a, b, last), (x, y), x.shape[:-1] + (2 * x.shape[-1],), max(x.hi, y.hi))
+        elif kind == "concat_inner":
+            y = pick(x.shape)
+            d = int(rng.integers(0, len(x.shape)))
+            shp = list(x.shape)
+            shp[d] *= 2
+            add(lambda be, a, b, d=d: be.concat(a, b, d), (x, y), shp, max(x.hi, y.hi))
+        elif kind == "cast":           # f32 -> u32 -> f32 of a non-negative value: truncation
+            add(lambda be, a, s=x.shape: be.cast(be.cast(be.mul(be.mul(a, a), const(be, 7.0, s)), A.U32), A.F32), (x,), x.shape,
+                7 * x.hi * x.hi, needs_exact=(x,))
+        elif kind == "index":
+            d = int(rng.integers(0, len(x.shape)))
+            ids = rng.integers(0, x.shape[d], size=int(rng.integers(1, 6))).astype(np.uint32)
+            shp = list(x.shape)
+            shp[d] = len(ids)
+            add(lambda be, a, d=d, ids=ids: be.index(a, d, be.from_numpy(ids)), (x,), shp, x.hi)
+        elif kind == "scalar":
+            c = float(rng.uniform(0.5, 1.5))
+            add(lambda be, a, c=c, s=x.shape: be.mul(a, const(be, c, s)), (x,), x.shape, 1.5 * x.hi)
+    cand = np.arange(3, len(nodes))
+    outs = [nodes[int(i)] for i in rng.choice(cand, size=min(4, len(cand)), replace=False)] if len(cand) else [nodes[0]]
+    return inputs, nodes, outs
+
+
+def evaluate(be, inputs, nodes, outs):
+    """Builds every node once, in order (so a node used twice is one shared tensor), then reads the outputs
+    back last-built first: a read of a late node must not disturb the deferred state of an earlier one."""
+    val = {}
+    for i, n in enumerate(nodes):
+        val[id(n)] = be.from_numpy(inputs[i]) if n.fn is None else n.fn(be, *[val[id(p)] for p in n.parents])
+    got = {id(n): be.to_numpy(val[id(n)]) for n in reversed(outs)}
+    return [got[id(n)] for n in outs]
+
+
+@pytest.mark.parametrize("seed", range(400))
+def test_random_graph_matches_oracle(hip, oracle, seed):
+    rng = np.random.default_rng(1000 + seed)
+    inputs, nodes, outs = random_graph(rng)
+    got = evaluate(hip, inputs, nodes, outs)
+    ref = evaluate(oracle, inputs, nodes, outs)
+    for i, (n, g, e) in enumerate(zip(outs, got, ref)):
+        assert g.shape == e.shape == n.shape and g.dtype == e.dtype
+        assert np.isfinite(e).all() and np.abs(e).max(initial=0.0) <= n.hi * 1.001, f"seed {seed}: bound of output {i} is wrong"
+        np.testing.assert_allclose(g, e, rtol=1e-4, atol=1e-5 * max(1.0, n.hi), err_msg=f"seed {seed} output {i}")
+
+
+@pytest.mark.parametrize("seed", range(200))
+def test_random_matmul_shapes_match_oracle(hip, oracle, seed):
+    """[.., M, K] x [.., K, N] at random extents, either operand possibly a transposed or sliced view, the
+    result possibly consumed by an element-wise op first.  Tolerance: 1e-3 of the result's largest magnitude."""
+    rng = np.random.default_rng(5000 + seed)
+    big = rng.random() < 0.25
+    M, K, N = (int(rng.integers(1, 700 if big else 70)) for _ in range(3))
+    if rng.random() < 0.3:
+        M = int(rng.integers(1, 9))          # the decode-time row counts
+    if rng.random() < 0.3:
+        K = int(rng.choice([64, 128, 256, 512]))
+    batch = tuple(int(b) for b in rng.integers(1, 4, size=int(rng.integers(0, 3))))
+    xt, yt = rng.random() < 0.4, rng.random() < 0.5
+    pad = int(rng.integers(0, 5)) if rng.random() < 0.3 else 0
+    x = rng.standard_normal(batch + ((K, M) if xt else (M, K + pad))).astype(np.float32)
+    y = rng.standard_normal(batch + ((N, K) if yt else (K, N))).astype(np.float32)
+    post = str(rng.choice(["none", "scale", "add"]))
+    r = len(batch) + 2
+
+    def run(be):
+        a, b = be.from_numpy(x), be.from_numpy(y)
+        if xt:
+            a = be.transpose(a, r - 2, r - 1)
+        elif pad:
+            a = be.slice(a, r - 1, pad // 2, K)
+        if yt:
+            b = be.transpose(b, r - 2, r - 1)
+        o = be.matmul(a, b)
+        if post == "scale":
+            o = be.mul(o, const(be, 0.125, o.shape))
+        elif post == "add":
+            o = be.add(o, o)
+        return be.to_numpy(o)
+
+    got, ref = run(hip), run(oracle)
+    assert got.shape == ref.shape == batch + (M, N)
+    scale = max(1.0, float(np.abs(ref).max()))
+    assert float(np.abs(got - ref).max()) <= 1e-3 * scale, f"seed {seed}: M={M} K={K} N={N} batch={batch} xt={xt} yt={yt} pad={pad}"
+
+
+@pytest.mark.parametrize("seed", range(120))
+def test_random_attention_shapes_match_oracle(hip, oracle, seed):
+    """The model graphs' attention (repeat_kv, scores, scale, causal mask rows, soft-max, context) at random
+    batch / head / query / cache extents: decode steps (one query), speculative-width chunks and prefill chunks
+    that start anywhere in the cache, head widths with and without a one-pass kernel."""
+    import cases
+
+    rng = np.random.default_rng(9000 + seed)
+    B, kvh, rep = int(rng.integers(1, 3)), int(rng.integers(1, 4)), int(rng.choice([1, 2, 4, 8]))
+    hd = int(rng.choice([64, 64, 128, 128, 32, 80]))
+    T = int(rng.integers(1, 600))
+    S = int(rng.choice([1, 1, int(rng.integers(1, 10)), int(rng.integers(1, T + 1)), T]))
+    S = min(S, T)
+    q = rng.standard_normal((B, kvh * rep, S, hd)).astype(np.float32)
+    k = rng.standard_normal((B, kvh, T, hd)).astype(np.float32)
+    v = rng.standard_normal((B, kvh, T, hd)).astype(np.float32)
+
+    def run(be):
+        return be.to_numpy(cases.decode_attention_ops(be, be.from_numpy(q), be.from_numpy(k), be.from_numpy(v), rep))
+
+    got, ref = run(hip), run(oracle)
+    assert got.shape == ref.shape == (B, kvh * rep, S, hd)
+    np.testing.assert_allclose(got, ref, rtol=1e-4, atol=2e-5, err_msg=f"seed {seed}: B={B} kvh={kvh} rep={rep} hd={hd} S={S} T={T}")
