@@ -1006,7 +1006,7 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
 #define CG_CALL(MMV) hipLaunchKernelGGL((skinny_kt_wide_kernel<MMV, 4, false>), grid, dim3(kThreads), 0, s, a);
                 CG_MM_SWITCH(CG_CALL)
 #undef CG_CALL
-            } else if (cols >= 8192 && M <= 4) { // gate / up projections of a decode step
+            } else if (cols >= 4096 && M <= 4) { // the wider projections of a decode step: activations are fetched once per 8 columns
                 dim3 grid((uint32_t)((N + 7) / 8), (uint32_t)batch);
                 hipLaunchKernelGGL((skinny_kt_mfma_xreg_kernel<4, 2>), grid, dim3(kThreads), 0, s, a);
             } else if (cols >= 2048) {
