@@ -497,6 +497,9 @@ template <int MM> __global__ __launch_bounds__(kThreads) void skinny_kt_wide_res
 
 // Several products that share their left operand (the q / k / v projections of a decode step,
 // gate and up) in one launch: the workgroups are dealt to the problems in order.
+// Products too narrow for eight columns per workgroup still gain from the matrix-instruction kernel at four
+// columns per workgroup (one activation load per lane and trip instead of M) when its 2048-wide chunks of k are full.
+static inline bool xreg_narrow(uint32_t M, uint32_t K) { return M > 1 && M <= 4 && K % 2048 == 0; }
 constexpr int kMaxGroup = 4;
 struct MmGroup {
     MmArgs p[kMaxGroup];
@@ -520,16 +523,21 @@ template <int MM> __global__ __launch_bounds__(kThreads) void skinny_kt_wide_gro
 // X[j][k] for the k values of block b, so one 16-byte weight load per lane drives four
 // instructions that update all 4 (rows) x 4 (columns) partial sums of the block.  Against
 // the FMA kernels this needs a quarter of the vector issue slots.  The four waves of a
-// workgroup split each 2048-wide chunk of k, keep their share of the chunk's activations
-// in registers (8 x 16 bytes per lane and row group) and reuse it for CG groups of four
-// columns, so the activation rows are fetched once per 4 * CG columns.
+// workgroup split each 2048-wide chunk of k into runs of 512 (a wave reads 2 KiB in a row of
+// each weight row: measured 12 % faster on the gate / up pair than interleaving the waves
+// every 256 bytes), keep their share of the chunk's activations in registers (8 x 16 bytes
+// per lane and row group) and reuse it for CG groups of four columns, so the activation rows
+// are fetched once per 4 * CG columns.
+// RESIDUAL (CG = 1): the store adds the other terms of a four-term sum, as skinny_kt_wide_residual_kernel does.
 // GATED (CG = 2): the two column groups are the same four columns of two weight matrices, a.B and
 // `second` (same shape and strides), and the block writes g * (1 / (one + exp(-g))) * u for
 // g = x.B^T, u = x.second^T: the SiLU-gated pair of an MLP block without writing g and u.
-template <int MM, int CG, bool GATED = false>
+template <int MM, int CG, bool GATED = false, bool RESIDUAL = false>
 __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const uint32_t block_x, const uint32_t block_y,
-                                                         const uint32_t *second = nullptr, const uint32_t one = 0) {
+                                                         const uint32_t *second = nullptr, const uint32_t one = 0,
+                                                         const MmResidual *res = nullptr) {
     static_assert(!GATED || CG == 2, "a gated pair is two column groups");
+    static_assert(!(GATED && RESIDUAL), "one epilogue at a time");
     constexpr int G = MM / 4;
     const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x % 64;
     const uint32_t j = lane % 4, b = lane / 4;
@@ -549,12 +557,25 @@ __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const 
     for (int c = 0; c < CG; c++)
 #pragma unroll
         for (int g = 0; g < G; g++) acc[c][g] = (float4v){0.f, 0.f, 0.f, 0.f};
-    const uint32_t kb = (wave * 16 + b) * 4;
+    // the sum's other terms for the value this thread will store: asked for before the walk along K
+    uint32_t term[4] = {};
+    if constexpr (RESIDUAL) {
+        if (threadIdx.x < CG * MM * 4) {
+            const uint32_t c = threadIdx.x / (MM * 4), m = threadIdx.x / 4 % MM, col = n0 + 4 * c + threadIdx.x % 4;
+            if (col < a.N && m < a.M) {
+#pragma unroll
+                for (int t = 0; t < 4; t++)
+                    if ((uint32_t)t != res->slot) term[t] = res->term[t][((uint64_t)block_y * a.M + m) * a.N + col];
+            }
+        }
+    }
+    // of every 2048 values of k a wave takes 512 in a row (8 trips of 64): 2 KiB of each weight row
+    const uint32_t kb = wave * 512 + b * 4;
     for (uint32_t k0 = 0; k0 < a.K; k0 += 2048) {
         float4v xr[G][8];
 #pragma unroll
         for (int t = 0; t < 8; t++) {
-            const uint32_t k = k0 + kb + 256 * t;
+            const uint32_t k = k0 + kb + 64 * t;
 #pragma unroll
             for (int g = 0; g < G; g++) {
                 xr[g][t] = (float4v){0.f, 0.f, 0.f, 0.f};
@@ -566,7 +587,7 @@ __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const 
             float4v w[8];
 #pragma unroll
             for (int t = 0; t < 8; t++) {
-                const uint32_t k = k0 + kb + 256 * t;
+                const uint32_t k = k0 + kb + 64 * t;
                 w[t] = (float4v){0.f, 0.f, 0.f, 0.f};
                 if (k < a.K) w[t] = *reinterpret_cast<const float4v *>(wrow[c] + k);
             }
@@ -607,8 +628,15 @@ __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const 
         }
     } else if (threadIdx.x < CG * MM * 4) {
         const uint32_t c = threadIdx.x / (MM * 4), m = threadIdx.x / 4 % MM, col = n0 + 4 * c + threadIdx.x % 4;
-        const float v = (part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]);
-        if (col < a.N && m < a.M) a.C[((uint64_t)block_y * a.M + m) * a.N + col] = asu(v);
+        uint32_t v = asu((part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]));
+        if constexpr (RESIDUAL) {
+#pragma unroll
+            for (int t = 0; t < 4; t++) term[t] = (uint32_t)t == res->slot ? v : term[t];
+            const uint32_t inner = apply<kAdd, true>(term[1], term[2], 0, nullptr);
+            v = res->order == 0 ? apply<kAdd, true>(apply<kAdd, true>(term[0], inner, 0, nullptr), term[3], 0, nullptr)
+                                : apply<kAdd, true>(term[0], apply<kAdd, true>(inner, term[3], 0, nullptr), 0, nullptr);
+        }
+        if (col < a.N && m < a.M) a.C[((uint64_t)block_y * a.M + m) * a.N + col] = v;
     }
 }
 
@@ -618,6 +646,10 @@ template <int MM, int CG> __global__ __launch_bounds__(kThreads) void skinny_kt_
 template <int MM>
 __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_gated_kernel(const MmArgs a, const uint32_t *second, uint32_t one) {
     skinny_kt_mfma_xreg_body<MM, 2, true>(a, blockIdx.x, blockIdx.y, second, one);
+}
+template <int MM>
+__global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_residual_kernel(const MmArgs a, const MmResidual r) {
+    skinny_kt_mfma_xreg_body<MM, 1, false, true>(a, blockIdx.x, blockIdx.y, nullptr, 0, &r);
 }
 template <int MM, int CG> __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_group_kernel(const MmGroup g) {
     uint32_t bx;
@@ -881,6 +913,7 @@ int launch_matmul_group(cg_backend *be, const cg_tensor *x, const cg_tensor *con
         bytes += distinct_bytes(ys[i]) + distinct_bytes(outs[i]);
     }
     const bool xreg = all_wide && g.p[0].M <= 4;
+    const bool xreg1 = !xreg && xreg_narrow(g.p[0].M, g.p[0].K);
     uint32_t blocks = 0;
     for (int i = 0; i < n; i++) {
         g.first[i] = blocks;
@@ -891,6 +924,8 @@ int launch_matmul_group(cg_backend *be, const cg_tensor *x, const cg_tensor *con
     ProfScope prof(be, CG_K_GEMM_SKINNY, bytes);
     if (xreg)
         hipLaunchKernelGGL((skinny_kt_mfma_xreg_group_kernel<4, 2>), dim3(blocks), dim3(kThreads), 0, be->stream, g);
+    else if (xreg1)
+        hipLaunchKernelGGL((skinny_kt_mfma_xreg_group_kernel<4, 1>), dim3(blocks), dim3(kThreads), 0, be->stream, g);
     else if (g.p[0].M <= 1)
         hipLaunchKernelGGL((skinny_kt_wide_group_kernel<1>), dim3(blocks), dim3(kThreads), 0, be->stream, g);
     else if (g.p[0].M <= 4)
@@ -942,7 +977,9 @@ int launch_matmul_residual(cg_backend *be, const cg_tensor *x, const cg_tensor *
     r.order = (uint32_t)order;
     ProfScope prof(be, CG_K_GEMM_SKINNY, distinct_bytes(x) + distinct_bytes(y) + 4.0 * distinct_bytes(out));
     dim3 grid((uint32_t)((a.N + 3) / 4));
-    if (a.M <= 1)
+    if (xreg_narrow(a.M, a.K))
+        hipLaunchKernelGGL((skinny_kt_mfma_xreg_residual_kernel<4>), grid, dim3(kThreads), 0, be->stream, a, r);
+    else if (a.M <= 1)
         hipLaunchKernelGGL((skinny_kt_wide_residual_kernel<1>), grid, dim3(kThreads), 0, be->stream, a, r);
     else if (a.M <= 4)
         hipLaunchKernelGGL((skinny_kt_wide_residual_kernel<4>), grid, dim3(kThreads), 0, be->stream, a, r);
@@ -1009,6 +1046,9 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
             } else if (cols >= 4096 && M <= 4) { // the wider projections of a decode step: activations are fetched once per 8 columns
                 dim3 grid((uint32_t)((N + 7) / 8), (uint32_t)batch);
                 hipLaunchKernelGGL((skinny_kt_mfma_xreg_kernel<4, 2>), grid, dim3(kThreads), 0, s, a);
+            } else if (cols >= 2048 && xreg_narrow((uint32_t)M, (uint32_t)K)) {
+                dim3 grid((uint32_t)((N + 3) / 4), (uint32_t)batch);
+                hipLaunchKernelGGL((skinny_kt_mfma_xreg_kernel<4, 1>), grid, dim3(kThreads), 0, s, a);
             } else if (cols >= 2048) {
                 dim3 grid((uint32_t)((N + 3) / 4), (uint32_t)batch);
 #define CG_CALL(MMV) hipLaunchKernelGGL((skinny_kt_wide_kernel<MMV, 1, false>), grid, dim3(kThreads), 0, s, a);

@@ -1018,7 +1018,7 @@ def _linear(be, x, w):
 
 
 for _B, _K, _Ns in ((4, 512, (512, 128, 128)), (1, 1024, (64, 2048)), (8, 388, (300, 8200)), (4, 512, (8192, 8200)),
-                    (2, 2304, (8192, 8192, 96, 100, 104))):
+                    (2, 2304, (8192, 8192, 96, 100, 104)), (4, 2048, (2048, 512, 516)), (3, 4096, (300, 2052)), (2, 2048, (2500,))):
     @case(f"linear_group_B{_B}_K{_K}_N{'_'.join(map(str, _Ns))}", "red",
           (lambda B=_B, K=_K, Ns=_Ns: [np.abs(f32(500 + K, (B, 1, K)).astype(np.float64)) @
                                          np.abs(f32(501 + K + i, (n, K)).astype(np.float64)).T
@@ -1091,7 +1091,7 @@ for _B, _K, _N in ((4, 512, 4096), (1, 2048, 8192), (3, 388, 4100), (8, 512, 409
 
 
 # ---- residual adds around a decode-time linear layer (the o / down projection of a decoder layer) -------------------
-for _B, _K, _N in ((4, 512, 2048), (8, 260, 2052), (1, 1024, 4096), (4, 512, 512)):
+for _B, _K, _N in ((4, 512, 2048), (8, 260, 2052), (1, 1024, 4096), (4, 512, 512), (4, 2048, 2048), (3, 4096, 2052), (2, 2048, 4100)):
     @case(f"linear_residual_B{_B}_K{_K}_N{_N}", "red")
     def _(B=_B, K=_K, Nn=_N):
         """Sums of three dense terms and a lazy product in the two association orders and every operand
