@@ -214,8 +214,9 @@ class Backend:
     def to_vec(self, x: Tensor) -> np.ndarray:
         """`Backend::to_vec`: flat row-major contents."""
         n = int(self._lib.cg_tensor_numel(x._h))
-        # f16 as numpy float16; bf16 as its uint16 bit patterns (numpy has no bfloat16): `bits << 16` is the f32 value
-        out = np.empty(n, dtype={A.F32: np.float32, A.F16: np.float16, A.BF16: np.uint16}.get(x.dtype, np.uint32))
+        # f16 as numpy float16; bf16 as its uint16 bit patterns (numpy has no bfloat16): `bits << 16` is the f32 value;
+        # fp8 (E4M3) as its uint8 bit patterns
+        out = np.empty(n, dtype={A.F32: np.float32, A.F16: np.float16, A.BF16: np.uint16, A.F8: np.uint8}.get(x.dtype, np.uint32))
         self._check(self._lib.cg_to_host(self._b, x._h, out.ctypes.data_as(C.c_void_p), n))
         return out
 

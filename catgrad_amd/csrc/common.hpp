@@ -167,10 +167,12 @@ struct cg_tensor {
 
 namespace cg {
 
-// Floating-point dtypes: the arithmetic is f32 on 32-bit words; CG_F16 / CG_BF16 results are rounded
-// to their 16-bit format after every op (the words always hold exactly representable values).
-inline bool is_f(cg_dtype d) { return d == CG_F32 || d == CG_F16 || d == CG_BF16; }
+// Floating-point dtypes: the arithmetic is f32 on 32-bit words; CG_F16 / CG_BF16 / CG_F8 results are rounded
+// to their format after every op (the words always hold exactly representable values).
+inline bool is_f(cg_dtype d) { return d == CG_F32 || d == CG_F16 || d == CG_BF16 || d == CG_F8; }
 inline bool is_half(cg_dtype d) { return d == CG_F16 || d == CG_BF16; }
+// dtypes narrower than their 32-bit words: results are rounded after every op
+inline bool is_narrow(cg_dtype d) { return is_half(d) || d == CG_F8; }
 
 inline int64_t numel(const cg_tensor *t) {
     int64_t n = 1;
@@ -346,6 +348,8 @@ enum EwOp : int {
     // f32 -> nearest bfloat16 / binary16 value (ties to even), still held as f32: how results of the
     // 16-bit float dtypes are rounded (every tensor is stored as 32-bit words)
     kRoundBF16, kRoundF16,
+    // f32 -> nearest fp8 (E4M3) value, ties to even, +-448 beyond the largest finite value; still held as f32
+    kRoundF8,
     // binary (order of cg_binary_op) offset by 16
     kAdd = 16, kSub, kMul, kDiv, kPow, kLt, kGt, kGte, kLte, kEq,
     kWhere = 32,
@@ -376,6 +380,9 @@ int launch_bf16_widen(cg_backend *be, const void *src, void *dst, uint64_t n);
 int launch_f16_widen(cg_backend *be, const void *src, void *dst, uint64_t n);
 // f32 words holding bfloat16 / binary16 values -> their 16-bit patterns (exact)
 int launch_narrow16(cg_backend *be, cg_dtype dt, const void *src, void *dst, uint64_t n);
+// fp8 (E4M3) bytes <-> 32-bit words holding the same values
+int launch_f8_widen(cg_backend *be, const void *src, void *dst, uint64_t n);
+int launch_narrow8(cg_backend *be, const void *src, void *dst, uint64_t n);
 // out[outer, j, inner] = x[outer, idx[j], inner]
 int launch_gather(cg_backend *be, const cg_tensor *x, int dim, const cg_tensor *idx, cg_tensor *out);
 

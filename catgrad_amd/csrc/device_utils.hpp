@@ -81,6 +81,35 @@ __host__ __device__ __forceinline__ uint32_t round_bf16_bits(uint32_t u) {
     return (u + 0x7FFFu + ((u >> 16) & 1u)) & 0xFFFF0000u;
 }
 
+// fp8 = E4M3 (float8::F8E4M3): 4 exponent bits with bias 7, 3 mantissa bits, no infinities, 0x7F the NaN, largest
+// finite value 448, subnormals m * 2^-9.  f32 bits -> f32 bits of the nearest such value (ties to even); 448 and
+// beyond, infinities included, give +-448 (the crate's saturating conversion); NaN stays NaN.
+__host__ __device__ __forceinline__ uint32_t round_f8_bits(uint32_t u) {
+    const uint32_t sign = u & 0x80000000u, a = u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return sign | 0x7FC00000u;
+    if (a >= 0x43E00000u) return sign | 0x43E00000u; // 448
+    if (a < 0x3C800000u) {                           // below 2^-6: whole multiples of 2^-9
+        const float units = rintf(__builtin_bit_cast(float, a) * 512.0f);
+        return sign | __builtin_bit_cast(uint32_t, units * (1.0f / 512.0f));
+    }
+    const uint32_t r = (a + 0x7FFFFu + ((a >> 20) & 1u)) & 0xFFF00000u; // a carry runs into the exponent
+    return sign | (r > 0x43E00000u ? 0x43E00000u : r);
+}
+// the byte of a representable value, and back
+__host__ __device__ __forceinline__ uint8_t f8_byte_of(uint32_t u) {
+    const uint8_t sign = (uint8_t)((u >> 24) & 0x80u);
+    const uint32_t a = u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return sign | 0x7Fu;
+    if (a >= 0x3C800000u) return sign | (uint8_t)((((a >> 23) - 120u) << 3) | ((a >> 20) & 7u));
+    return sign | (uint8_t)(uint32_t)(__builtin_bit_cast(float, a) * 512.0f);
+}
+__host__ __device__ __forceinline__ uint32_t f8_word_of(uint8_t b) {
+    const uint32_t sign = (uint32_t)(b & 0x80u) << 24, e = (b >> 3) & 0xFu, m = b & 7u;
+    if (e == 0xFu && m == 7u) return sign | 0x7FC00000u;
+    if (e != 0) return sign | ((e + 120u) << 23) | (m << 20);
+    return sign | __builtin_bit_cast(uint32_t, (float)m * (1.0f / 512.0f));
+}
+
 // One scalar application of OP on raw 32-bit words.  F = operands are f32.
 template <int OP, bool F>
 __device__ __forceinline__ uint32_t apply(uint32_t a, uint32_t b, uint32_t c, uint32_t *fault) {
@@ -102,6 +131,7 @@ __device__ __forceinline__ uint32_t apply(uint32_t a, uint32_t b, uint32_t c, ui
         if constexpr (OP == kRound) return asu(rintf(x)); // ties to even (ndarray.rs:646-648)
         if constexpr (OP == kRoundBF16) return round_bf16_bits(a);
         if constexpr (OP == kRoundF16) return asu(__half2float(__float2half_rn(x))); // v_cvt_f16_f32: nearest even, overflow -> inf
+        if constexpr (OP == kRoundF8) return round_f8_bits(a);
         if constexpr (OP == kAdd) return asu(x + y);
         if constexpr (OP == kSub) return asu(x - y);
         if constexpr (OP == kMul) return asu(x * y);

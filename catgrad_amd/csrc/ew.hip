@@ -201,6 +201,7 @@ int launch_elementwise(cg_backend *be, int op, cg_dtype dt, const cg_tensor *out
     case kRound: return launch_variants<kRound, true, 1>(be, a);
     case kRoundBF16: return launch_variants<kRoundBF16, true, 1>(be, a);
     case kRoundF16: return launch_variants<kRoundF16, true, 1>(be, a);
+    case kRoundF8: return launch_variants<kRoundF8, true, 1>(be, a);
     CG_EW2(kAdd) CG_EW2(kSub) CG_EW2(kMul) CG_EW2(kDiv) CG_EW2(kPow)
     CG_EW2(kLt) CG_EW2(kGt) CG_EW2(kGte) CG_EW2(kLte) CG_EW2(kEq)
     case kWhere: return launch_by_dtype<kWhere, 3>(be, dt, a);
@@ -262,6 +263,30 @@ int launch_narrow16(cg_backend *be, cg_dtype dt, const void *src, void *dst, uin
                            static_cast<uint16_t *>(dst), n);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? CG_OK : hip_fail(e, "16-bit narrowing launch");
+}
+
+__global__ __launch_bounds__(kBlock) void f8_widen_kernel(const uint8_t *src, uint32_t *dst, uint64_t n) {
+    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (uint64_t)gridDim.x * kBlock) dst[i] = f8_word_of(src[i]);
+}
+__global__ __launch_bounds__(kBlock) void narrow8_kernel(const uint32_t *src, uint8_t *dst, uint64_t n) {
+    for (uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (uint64_t)gridDim.x * kBlock) dst[i] = f8_byte_of(src[i]);
+}
+int launch_f8_widen(cg_backend *be, const void *src, void *dst, uint64_t n) {
+    if (n == 0) return CG_OK;
+    const uint32_t blocks = (uint32_t)std::min<uint64_t>((n + kBlock - 1) / kBlock, 16384);
+    hipLaunchKernelGGL(f8_widen_kernel, dim3(blocks), dim3(kBlock), 0, be->stream, static_cast<const uint8_t *>(src),
+                       static_cast<uint32_t *>(dst), n);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CG_OK : hip_fail(e, "fp8 widen launch");
+}
+int launch_narrow8(cg_backend *be, const void *src, void *dst, uint64_t n) {
+    if (n == 0) return CG_OK;
+    if (int frc = flush_deferred(be)) return frc;
+    const uint32_t blocks = (uint32_t)std::min<uint64_t>((n + kBlock - 1) / kBlock, 16384);
+    hipLaunchKernelGGL(narrow8_kernel, dim3(blocks), dim3(kBlock), 0, be->stream, static_cast<const uint32_t *>(src),
+                       static_cast<uint8_t *>(dst), n);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CG_OK : hip_fail(e, "fp8 narrowing launch");
 }
 
 int launch_fill_word(cg_backend *be, void *ptr, uint32_t bits) {

@@ -93,7 +93,7 @@ __device__ __forceinline__ void apply_rt(uint32_t op, const uint32_t (&x)[VEC], 
         }
     }
     switch (op) {
-        CG_F(kNeg) CG_F(kExp) CG_F(kFloor) CG_F(kRound) CG_F(kRoundBF16) CG_F(kRoundF16)
+        CG_F(kNeg) CG_F(kExp) CG_F(kFloor) CG_F(kRound) CG_F(kRoundBF16) CG_F(kRoundF16) CG_F(kRoundF8)
         CG_F(kAdd) CG_F(kSub) CG_F(kMul) CG_F(kDiv)
         CG_F(kLt) CG_F(kGt) CG_F(kGte) CG_F(kLte) CG_F(kEq) CG_F(kWhere) CG_F(kCastF2U)
         CG_U(kNeg) CG_U(kAdd) CG_U(kSub) CG_U(kMul) CG_U(kDiv)

@@ -465,8 +465,10 @@ struct Consume { // the consumed reference of a tensor argument (move semantics 
     ~Consume() { release(t); }
 };
 
-static const char *kTodo = "fp8 is not supported (todo!() in the reference NdArrayBackend)";
-static bool supported(cg_dtype d) { return d == CG_F32 || d == CG_U32 || d == CG_F16 || d == CG_BF16; }
+static const char *kTodo = "unknown dtype";
+static bool supported(cg_dtype d) { return d == CG_F32 || d == CG_U32 || d == CG_F16 || d == CG_BF16 || d == CG_F8; }
+// bytes of one element at the boundary (from_vec / to_vec)
+static size_t host_bytes(cg_dtype d) { return d == CG_F8 ? 1 : is_half(d) ? 2 : 4; }
 
 // The 16-bit float dtypes on the host (constants that never reach the device): widening of a bit pattern
 // and rounding of an f32 to the nearest representable value (ties to even), both as f32 bits.
@@ -499,6 +501,43 @@ static uint16_t narrow16_host(cg_dtype dt, uint32_t u) {
     memcpy(&h, &v, 2);
     return h;
 }
+
+// fp8 = E4M3 on the host, as round_f8_bits / f8_byte_of / f8_word_of do it on the device
+static uint32_t round8_host(uint32_t u) {
+    const uint32_t sign = u & 0x80000000u, a = u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return sign | 0x7FC00000u;
+    if (a >= 0x43E00000u) return sign | 0x43E00000u;
+    if (a < 0x3C800000u) {
+        float f;
+        memcpy(&f, &a, 4);
+        f = nearbyintf(f * 512.0f) * (1.0f / 512.0f);
+        uint32_t r;
+        memcpy(&r, &f, 4);
+        return sign | r;
+    }
+    const uint32_t r = (a + 0x7FFFFu + ((a >> 20) & 1u)) & 0xFFF00000u;
+    return sign | (r > 0x43E00000u ? 0x43E00000u : r);
+}
+static uint32_t widen8_host(uint8_t b) {
+    const uint32_t sign = (uint32_t)(b & 0x80u) << 24, e = (b >> 3) & 0xFu, m = b & 7u;
+    if (e == 0xFu && m == 7u) return sign | 0x7FC00000u;
+    if (e != 0) return sign | ((e + 120u) << 23) | (m << 20);
+    const float f = (float)m * (1.0f / 512.0f);
+    uint32_t r;
+    memcpy(&r, &f, 4);
+    return sign | r;
+}
+static uint8_t narrow8_host(uint32_t u) {
+    const uint8_t sign = (uint8_t)((u >> 24) & 0x80u);
+    const uint32_t a = u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return sign | 0x7Fu;
+    if (a >= 0x3C800000u) return sign | (uint8_t)((((a >> 23) - 120u) << 3) | ((a >> 20) & 7u));
+    float f;
+    memcpy(&f, &a, 4);
+    return sign | (uint8_t)(uint32_t)(f * 512.0f);
+}
+// a constant's value rounded to a narrow dtype
+static uint32_t round_host(cg_dtype dt, uint32_t u) { return dt == CG_F8 ? round8_host(u) : is_half(dt) ? round16_host(dt, u) : u; }
 
 static bool same_shape(const cg_tensor *a, const cg_tensor *b) {
     if (a->rank != b->rank) return false;
@@ -1773,6 +1812,8 @@ int cg_from_host(cg_backend *b, cg_dtype dtype, const void *data, size_t len, co
             uint16_t h;
             memcpy(&h, data, 2);
             bits = widen16_host(dtype, h);
+        } else if (dtype == CG_F8) {
+            bits = widen8_host(*static_cast<const uint8_t *>(data));
         } else {
             memcpy(&bits, data, 4);
         }
@@ -1784,13 +1825,17 @@ int cg_from_host(cg_backend *b, cg_dtype dtype, const void *data, size_t len, co
     if (rc) return rc;
     if (n) {
         CG_HIP(hipSetDevice(b->device));
-        if (is_half(dtype)) { // 2-byte elements: uploaded as they are, widened to 32-bit words on the device
+        if (is_narrow(dtype)) { // 2- or 1-byte elements: uploaded as they are, widened to 32-bit words on the device
             void *tmp = nullptr;
             size_t cls = 0;
-            rc = b->pool.alloc(n * 2, &tmp, &cls);
+            const size_t eb = host_bytes(dtype);
+            rc = b->pool.alloc(n * eb, &tmp, &cls);
             if (!rc) {
-                rc = staged_upload(b, tmp, data, n * 2);
-                if (!rc) rc = dtype == CG_BF16 ? launch_bf16_widen(b, tmp, t->buf->ptr, n) : launch_f16_widen(b, tmp, t->buf->ptr, n);
+                rc = staged_upload(b, tmp, data, n * eb);
+                if (!rc)
+                    rc = dtype == CG_BF16  ? launch_bf16_widen(b, tmp, t->buf->ptr, n)
+                         : dtype == CG_F16 ? launch_f16_widen(b, tmp, t->buf->ptr, n)
+                                           : launch_f8_widen(b, tmp, t->buf->ptr, n);
                 b->pool.free(tmp, cls); // stream-ordered: later users queue behind the widening kernel
             }
         } else {
@@ -1932,12 +1977,17 @@ int cg_to_host(cg_backend *b, const cg_tensor *t, void *dst, size_t len) {
     if (!b || !t || (!dst && len)) return fail(CG_ERR_ARG, "null argument");
     if ((int64_t)len != numel(t)) return fail(CG_ERR_SHAPE, "to_vec: length mismatch");
     CG_HIP(hipSetDevice(b->device));
-    if (is_half(t->dt) && len > 0) {
-        // 2-byte elements out: the words are narrowed on the device (exact), then copied
-        uint16_t *d16 = static_cast<uint16_t *>(dst);
+    if (is_narrow(t->dt) && len > 0) {
+        // 2- or 1-byte elements out: the words are narrowed on the device (exact), then copied
+        const size_t eb = host_bytes(t->dt);
         if (t->uniform) {
-            const uint16_t h = narrow16_host(t->dt, t->ubits);
-            for (size_t i = 0; i < len; i++) d16[i] = h;
+            if (t->dt == CG_F8) {
+                memset(dst, narrow8_host(t->ubits), len);
+            } else {
+                uint16_t *d16 = static_cast<uint16_t *>(dst);
+                const uint16_t h = narrow16_host(t->dt, t->ubits);
+                for (size_t i = 0; i < len; i++) d16[i] = h;
+            }
             return wait_and_check(b);
         }
         int rc = ensure_concrete(const_cast<cg_tensor *>(t));
@@ -1953,11 +2003,11 @@ int cg_to_host(cg_backend *b, const cg_tensor *t, void *dst, size_t len) {
         void *half = nullptr;
         size_t cls = 0;
         rc = device_ptr(src, &p);
-        if (!rc) rc = b->pool.alloc(len * 2, &half, &cls);
+        if (!rc) rc = b->pool.alloc(len * eb, &half, &cls);
         if (!rc) {
-            rc = launch_narrow16(b, t->dt, p, half, len);
+            rc = t->dt == CG_F8 ? launch_narrow8(b, p, half, len) : launch_narrow16(b, t->dt, p, half, len);
             if (!rc) {
-                hipError_t e = hipMemcpyAsync(dst, half, len * 2, hipMemcpyDeviceToHost, b->stream);
+                hipError_t e = hipMemcpyAsync(dst, half, len * eb, hipMemcpyDeviceToHost, b->stream);
                 rc = e == hipSuccess ? wait_and_check(b) : hip_fail(e, "device to host copy");
             }
             b->pool.free(half, cls);
@@ -2031,7 +2081,7 @@ int cg_format_tensor(cg_backend *b, const cg_tensor *t, char *buf, size_t cap) {
     std::vector<uint32_t> host(n);
     int rc = copy_out(b, t, host.data(), n); // the 32-bit words, whatever the dtype
     if (rc) return rc;
-    std::string s = t->dt == CG_F32 ? "f32[" : t->dt == CG_F16 ? "f16[" : t->dt == CG_BF16 ? "bf16[" : "u32[";
+    std::string s = t->dt == CG_F32 ? "f32[" : t->dt == CG_F16 ? "f16[" : t->dt == CG_BF16 ? "bf16[" : t->dt == CG_F8 ? "fp8[" : "u32[";
     for (int i = 0; i < t->rank; i++) s += (i ? "," : "") + std::to_string(t->dims[i]);
     s += "] [";
     size_t shown = std::min<size_t>(n, 16);
@@ -2070,18 +2120,18 @@ static int ew_result(cg_backend *b, int op, cg_dtype compute_dt, cg_dtype out_dt
     return CG_OK;
 }
 
-// Results of the 16-bit float dtypes: the f32 value just computed is rounded to the dtype (one more
+// Results of the 16-bit float dtypes and of fp8: the f32 value just computed is rounded to the dtype (one more
 // deferred instruction, or on the host for a constant).  Takes over the reference in *io.
 static int round_result(cg_backend *b, cg_dtype dt, cg_tensor **io) {
-    if (!is_half(dt)) return CG_OK;
+    if (!is_narrow(dt)) return CG_OK;
     cg_tensor *x = *io;
     *io = nullptr;
     int rc = CG_OK;
     if (x->uniform) {
-        *io = new_uniform(b, dt, x->dims, x->rank, round16_host(dt, x->ubits));
+        *io = new_uniform(b, dt, x->dims, x->rank, round_host(dt, x->ubits));
     } else {
         const cg_tensor *ins[1] = {x};
-        rc = ew_result(b, dt == CG_BF16 ? kRoundBF16 : kRoundF16, dt, dt, x, ins, 1, io);
+        rc = ew_result(b, dt == CG_BF16 ? kRoundBF16 : dt == CG_F16 ? kRoundF16 : kRoundF8, dt, dt, x, ins, 1, io);
     }
     release(x);
     return rc;
@@ -2165,7 +2215,7 @@ int cg_binary(cg_backend *b, cg_binary_op op, cg_tensor *x, cg_tensor *y, cg_ten
         bool divzero = false;
         if (fold_binary(op, x->dt, x->ubits, y->ubits, &r, &divzero)) {
             if (divzero) return fail(CG_ERR_RANGE, "attempt to divide by zero");
-            *out = new_uniform(b, x->dt, x->dims, x->rank, is_half(x->dt) ? round16_host(x->dt, r) : r);
+            *out = new_uniform(b, x->dt, x->dims, x->rank, round_host(x->dt, r));
             return CG_OK;
         }
     }

@@ -135,6 +135,10 @@ class Backend {
     Tensor ndarray_from_vec_bf16(const uint16_t *bits, size_t len, const Shape &shape) {
         return from_vec(CG_BF16, bits, len, shape);
     }
+    // mod.rs:48-52: fp8 (float8::F8E4M3) as its bit patterns, one byte per element.
+    Tensor ndarray_from_vec_fp8(const uint8_t *bits, size_t len, const Shape &shape) {
+        return from_vec(CG_F8, bits, len, shape);
+    }
     // Weight ingest (catgrad-llm/src/utils/mod.rs:158-168): f32 tensor from bfloat16 bit patterns.
     Tensor from_bf16_bits(const uint16_t *bits, size_t len, const Shape &shape) {
         return out([&](cg_tensor **o) {
@@ -232,6 +236,13 @@ class Backend {
     std::vector<uint16_t> to_vec_bits16(Tensor x) {
         calls++;
         std::vector<uint16_t> v(x.numel());
+        check(abi_.cg_to_host(b_, x.get(), v.data(), v.size()));
+        return v;
+    }
+    // `to_vec` of an fp8 tensor: its 8-bit patterns.
+    std::vector<uint8_t> to_vec_bits8(Tensor x) {
+        calls++;
+        std::vector<uint8_t> v(x.numel());
         check(abi_.cg_to_host(b_, x.get(), v.data(), v.size()));
         return v;
     }

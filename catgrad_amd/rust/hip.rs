@@ -238,7 +238,7 @@ impl HipBackend {
         if st == CG_ERR_SHAPE {
             return Err(BackendError::ShapeError);
         }
-        check(st); // fp8: the same todo!() as NdArrayBackend
+        check(st);
         Ok(tag_for(&dt, HipTensor(out)))
     }
 }
@@ -398,7 +398,12 @@ impl Backend for HipBackend {
                 check(unsafe { cg_to_host(self.raw(), t.0, v.as_mut_ptr() as *mut c_void, n) });
                 TaggedVec::BF16(v)
             }
-            _ => todo!("fp8 is not supported by the hip backend"),
+            Dtype::F8 => {
+                // 1-byte elements: float8::F8E4M3 is repr(transparent) over its u8 bit pattern
+                let mut v = vec![float8::F8E4M3::ZERO; n];
+                check(unsafe { cg_to_host(self.raw(), t.0, v.as_mut_ptr() as *mut c_void, n) });
+                TaggedVec::FP8(v)
+            }
         }
     }
 

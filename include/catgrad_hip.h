@@ -59,7 +59,9 @@ typedef enum cg_dtype {
     CG_BF16 = 2, /* bfloat16; idem.  Both: 2-byte elements at the boundary (cg_from_host / cg_to_host), held as
                     32-bit words inside; every op computes in f32 on exactly held values and rounds its result
                     to the dtype (nearest, ties to even); sums and products accumulate in f32 and round once */
-    CG_F8 = 3,   /* declared by the trait; unsupported here exactly as in NdArrayBackend (ndarray.rs:7-9) */
+    CG_F8 = 3,   /* float8::F8E4M3 (candle.rs:9,382): 4 exponent bits (bias 7), 3 mantissa bits, no infinities, largest
+                    finite value 448; same model: 1-byte elements at the boundary, 32-bit words inside, every result
+                    rounded to nearest even and saturated to +-448.  NdArrayBackend has todo!() here too */
     CG_U32 = 4
 } cg_dtype;
 
@@ -160,10 +162,9 @@ int cg_tensor_is_contiguous(const cg_tensor *t);
 /* ---- creation --------------------------------------------------------------*/
 /* `Backend::zeros` (mod.rs:28; ndarray.rs:71-84). */
 int cg_zeros(cg_backend *b, cg_dtype dtype, const size_t *dims, size_t rank, cg_tensor **out);
-/* `Backend::ndarray_from_vec_{f32,f16,bf16,u32}` (mod.rs:30-58; ndarray.rs:86-96,122-132;
- * candle.rs:530-551 for the 16-bit floats): row-major host data of `len` elements, 4 bytes each
- * for f32/u32 and 2 bytes each for f16/bf16; CG_ERR_SHAPE iff len != prod(dims).
- * f8 returns CG_ERR_UNSUPPORTED (ndarray.rs:98-120). */
+/* `Backend::ndarray_from_vec_{f32,f16,bf16,fp8,u32}` (mod.rs:30-58; ndarray.rs:86-96,122-132;
+ * candle.rs:530-562 for the 16-bit floats and fp8): row-major host data of `len` elements, 4 bytes each
+ * for f32/u32, 2 bytes each for f16/bf16, 1 byte each for fp8; CG_ERR_SHAPE iff len != prod(dims). */
 int cg_from_host(cg_backend *b, cg_dtype dtype, const void *data, size_t len,
                  const size_t *dims, size_t rank, cg_tensor **out);
 /* Weight ingest (catgrad-llm/src/utils/mod.rs:158-168 `decode_bf16_to_f32_into` followed by
@@ -178,7 +179,7 @@ int cg_arange(cg_backend *b, size_t end, cg_tensor **out);
 /* ---- read-back (borrowing) --------------------------------------------------*/
 /* `Backend::to_vec` (mod.rs:111; ndarray.rs:50-58; candle.rs:463-470): row-major copy of the
  * logical contents into `dst` (capacity `len` elements of the tensor's dtype, 2 bytes each for
- * f16/bf16; must equal numel). */
+ * f16/bf16, 1 byte each for fp8; must equal numel). */
 int cg_to_host(cg_backend *b, const cg_tensor *t, void *dst, size_t len);
 /* `Backend::to_bool` (mod.rs:109; ndarray.rs:140-149): any element > 0 (f32) / != 0 (u32). */
 int cg_to_bool(cg_backend *b, const cg_tensor *t, int *out);

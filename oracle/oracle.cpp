@@ -21,7 +21,10 @@
 // evaluation for f32 math.  PARITY UNPINNED at bit level (only to 1e-3 / 1e-4
 // relative): the exact f32 accumulation order of sgemm and sum_axis and the last
 // ulp of libm's expf/logf/sinf/cosf/powf — those could only be pinned by
-// building the Rust reference, for which this image has no toolchain.
+// building the Rust reference, for which this image has no toolchain.  For the
+// f16 / bf16 / fp8 dtypes (restated from CandleBackend's CPU path, further down):
+// PARITY UNPINNED for Candle's accumulation in sum / matmul and for fp8 values
+// beyond 464 (saturation per the float8 crate's documentation).
 //
 // Deliberate, documented differences from NdArrayBackend:
 //   * element-wise operands of different shape are rejected ("Shape mismatch in
@@ -123,7 +126,7 @@ cg_tensor *new_tensor(cg_dtype dt, const size_t *dims, int rank) {
 // A freshly computed (standard-layout, unshared) result of a 16-bit float dtype: every word rounded to the dtype.
 uint32_t round_to(cg_dtype dt, uint32_t u);
 void round_tensor(cg_tensor *t) {
-    if (t->dt != CG_F16 && t->dt != CG_BF16) return;
+    if (t->dt != CG_F16 && t->dt != CG_BF16 && t->dt != CG_F8) return;
     for (uint32_t &w : t->st->data) w = round_to(t->dt, w);
 }
 
@@ -226,7 +229,7 @@ bool same_shape(const cg_tensor *a, const cg_tensor *b) {
     return true;
 }
 
-bool supported(cg_dtype d) { return d == CG_F32 || d == CG_U32 || d == CG_F16 || d == CG_BF16; }
+bool supported(cg_dtype d) { return d == CG_F32 || d == CG_U32 || d == CG_F16 || d == CG_BF16 || d == CG_F8; }
 
 // ---- the 16-bit float dtypes ------------------------------------------------------------------
 // NdArrayBackend has `todo!()` for them (ndarray.rs:7-9, 98-120); what is restated here is the model of
@@ -236,7 +239,7 @@ bool supported(cg_dtype d) { return d == CG_F32 || d == CG_U32 || d == CG_F16 ||
 // own accumulation order and width are NOT restated (PARITY UNPINNED for those two; conversions and
 // element-wise results are pinned by numpy's float16 and by the closed form of bfloat16 rounding).
 // Tensors of these dtypes hold 32-bit words whose values are exactly representable in the dtype.
-bool isf(cg_dtype d) { return d == CG_F32 || d == CG_F16 || d == CG_BF16; }
+bool isf(cg_dtype d) { return d == CG_F32 || d == CG_F16 || d == CG_BF16 || d == CG_F8; }
 bool is_half(cg_dtype d) { return d == CG_F16 || d == CG_BF16; }
 
 uint32_t bits_of(float f) {
@@ -280,9 +283,43 @@ uint32_t f16_bits_to_f32(uint16_t h) {
     return sign | bits_of((float)m * (1.0f / 16777216.0f)); // subnormal or zero: m * 2^-24, exact in f32
 }
 
+// ---- fp8 --------------------------------------------------------------------------------------
+// `Dtype::F8` is `float8::F8E4M3` (candle.rs:9, 382; crate float8 0.7.0 per Cargo.lock, not vendored): sign,
+// 4 exponent bits (bias 7), 3 mantissa bits, no infinities, 0x7F / 0xFF the only NaNs, largest finite value
+// 448 = 0x7E, subnormals m * 2^-9.  The crate documents its conversions as those of CUDA's cuda_fp8.hpp with
+// saturation to the largest finite value (`__NV_SATFINITE`): round to nearest even; anything beyond 448,
+// infinities included, becomes +-448; NaN stays NaN.  Element-wise ops are f32 ops on the widened values,
+// narrowed again (the crate's operator impls), which is the same model as for the 16-bit dtypes above.
+// Pinned: all 256 decodings and in-range rounding (ties, subnormals, the carry into 2^-6 and up to 448)
+// against torch.float8_e4m3fn.  PARITY UNPINNED: what happens beyond 448 (torch makes NaN there, the crate's
+// documentation says saturate; only the latter is restated), and the accumulation of sums and products.
+uint8_t f32_to_f8e4m3_bits(uint32_t u) {
+    const uint8_t sign = (uint8_t)((u >> 24) & 0x80u);
+    const uint32_t a = u & 0x7FFFFFFFu;
+    if (a > 0x7F800000u) return sign | 0x7Fu;   // NaN
+    if (a >= 0x43E00000u) return sign | 0x7Eu;  // >= 448, infinity too: the largest finite value
+    if (a >= 0x3C800000u) {                     // normal in e4m3: >= 2^-6
+        uint32_t h = (((a >> 23) - 120u) << 3) | ((a & 0x7FFFFFu) >> 20);
+        const uint32_t rest = a & 0xFFFFFu;
+        if (rest > 0x80000u || (rest == 0x80000u && (h & 1u))) h++; // a carry runs into the exponent
+        return sign | (uint8_t)(h > 0x7Eu ? 0x7Eu : h);             // 464 and up would be 0x7F: saturate
+    }
+    const float units = float_of(a) * 512.0f; // subnormal: the value in units of 2^-9, nearest even
+    return sign | (uint8_t)(uint32_t)nearbyintf(units);
+}
+
+uint32_t f8e4m3_bits_to_f32(uint8_t b) {
+    const uint32_t sign = (uint32_t)(b & 0x80u) << 24;
+    const uint32_t e = (b >> 3) & 0xFu, m = b & 7u;
+    if (e == 0xF && m == 7) return sign | 0x7FC00000u;
+    if (e != 0) return sign | ((e + 120u) << 23) | (m << 20);
+    return sign | bits_of((float)m * (1.0f / 512.0f));
+}
+
 uint32_t round_to(cg_dtype dt, uint32_t u) {
     if (dt == CG_BF16) return (uint32_t)f32_to_bf16_bits(u) << 16;
     if (dt == CG_F16) return f16_bits_to_f32(f32_to_f16_bits(u));
+    if (dt == CG_F8) return f8e4m3_bits_to_f32(f32_to_f8e4m3_bits(u));
     return u;
 }
 
@@ -472,7 +509,7 @@ const T *as_batch3(cg_tensor *t, size_t batch, std::vector<T> &tmp, ptrdiff_t &s
 template <typename F> int for_each_dtype(cg_dtype dt, F &&f) {
     if (isf(dt)) return f(float{});
     if (dt == CG_U32) return f(uint32_t{});
-    return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
+    return fail(CG_ERR_UNSUPPORTED, "unknown dtype");
 }
 
 } // namespace
@@ -523,7 +560,7 @@ int cg_tensor_is_contiguous(const cg_tensor *t) { return is_standard(t) ? 1 : 0;
 // ndarray.rs:71-84
 int cg_zeros(cg_backend *, cg_dtype dtype, const size_t *dims, size_t rank, cg_tensor **out) {
     if (!out || rank > CG_MAX_RANK) return fail(CG_ERR_ARG, "bad arguments");
-    if (!supported(dtype)) return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
+    if (!supported(dtype)) return fail(CG_ERR_UNSUPPORTED, "unknown dtype");
     *out = new_tensor(dtype, dims, (int)rank); // vector::resize zero-fills
     return CG_OK;
 }
@@ -532,7 +569,7 @@ int cg_zeros(cg_backend *, cg_dtype dtype, const size_t *dims, size_t rank, cg_t
 int cg_from_host(cg_backend *, cg_dtype dtype, const void *data, size_t len, const size_t *dims, size_t rank,
                  cg_tensor **out) {
     if (!out || rank > CG_MAX_RANK) return fail(CG_ERR_ARG, "bad arguments");
-    if (!supported(dtype)) return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
+    if (!supported(dtype)) return fail(CG_ERR_UNSUPPORTED, "unknown dtype");
     size_t n = 1;
     for (size_t i = 0; i < rank; i++) n *= dims[i];
     if (n != len) return fail(CG_ERR_SHAPE, "ShapeError");
@@ -541,6 +578,10 @@ int cg_from_host(cg_backend *, cg_dtype dtype, const void *data, size_t len, con
         const uint16_t *h = static_cast<const uint16_t *>(data);
         uint32_t *d = t->st->data.data();
         for (size_t i = 0; i < n; i++) d[i] = dtype == CG_BF16 ? (uint32_t)h[i] << 16 : f16_bits_to_f32(h[i]);
+    } else if (n && dtype == CG_F8) { // 1-byte elements (candle.rs:553-562)
+        const uint8_t *h = static_cast<const uint8_t *>(data);
+        uint32_t *d = t->st->data.data();
+        for (size_t i = 0; i < n; i++) d[i] = f8e4m3_bits_to_f32(h[i]);
     } else if (n) {
         memcpy(t->st->data.data(), data, n * 4);
     }
@@ -586,6 +627,9 @@ int cg_to_host(cg_backend *, const cg_tensor *t, void *dst, size_t len) {
     if (is_half(t->dt)) { // 2-byte elements out (candle.rs:463-470); exact, the words hold representable values
         uint16_t *h = static_cast<uint16_t *>(dst);
         for (size_t i = 0; i < len; i++) h[i] = t->dt == CG_BF16 ? (uint16_t)(src[i] >> 16) : f32_to_f16_bits(src[i]);
+    } else if (t->dt == CG_F8) {
+        uint8_t *h = static_cast<uint8_t *>(dst);
+        for (size_t i = 0; i < len; i++) h[i] = f32_to_f8e4m3_bits(src[i]);
     } else if (len) {
         memcpy(dst, src, len * 4);
     }
@@ -625,7 +669,7 @@ int cg_compare(cg_backend *, const cg_tensor *x, const cg_tensor *y, int *out) {
 // ndarray.rs:60-69
 int cg_format_tensor(cg_backend *, const cg_tensor *t, char *buf, size_t cap) {
     if (!t || !buf || !cap) return fail(CG_ERR_ARG, "null argument");
-    std::string s = t->dt == CG_F32 ? "f32[" : t->dt == CG_F16 ? "f16[" : t->dt == CG_BF16 ? "bf16[" : "u32[";
+    std::string s = t->dt == CG_F32 ? "f32[" : t->dt == CG_F16 ? "f16[" : t->dt == CG_BF16 ? "bf16[" : t->dt == CG_F8 ? "fp8[" : "u32[";
     for (int i = 0; i < t->rank; i++) s += (i ? "," : "") + std::to_string(t->dims[i]);
     s += "] [";
     size_t n = numel(t), shown = std::min<size_t>(n, 16);
@@ -653,7 +697,7 @@ int cg_cast(cg_backend *, cg_tensor *x, cg_dtype target, cg_tensor **out) {
     Consume cx(x);
     if (!x || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(target) || !supported(x->dt))
-        return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
+        return fail(CG_ERR_UNSUPPORTED, "unknown dtype");
     if (target == x->dt) { // (x @ F32, F32) => x
         x->rc.fetch_add(1);
         *out = x;
@@ -685,7 +729,7 @@ int cg_cast(cg_backend *, cg_tensor *x, cg_dtype target, cg_tensor **out) {
 int cg_unary(cg_backend *, cg_unary_op op, cg_tensor *x, cg_tensor **out) {
     Consume cx(x);
     if (!x || !out) return fail(CG_ERR_ARG, "null argument");
-    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
+    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "unknown dtype");
     if (x->dt == CG_U32 && op != CG_NEG) {
         static const char *names[] = {"neg", "sin", "cos", "exp", "log", "floor", "round"};
         return fail(CG_ERR_DTYPE, "Invalid input types for %s", names[op]);
@@ -732,7 +776,7 @@ int cg_binary(cg_backend *, cg_binary_op op, cg_tensor *x, cg_tensor *y, cg_tens
     Consume cx(x), cy(y);
     if (!x || !y || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt) || !supported(y->dt))
-        return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
+        return fail(CG_ERR_UNSUPPORTED, "unknown dtype");
     if (x->dt != y->dt) return fail(CG_ERR_DTYPE, "TypeError: mixed dtypes in a binary operation");
     if (!same_shape(x, y)) return fail(CG_ERR_SHAPE, "Shape mismatch in operation");
     cg_tensor *ox = unwrap_owned(x), *oy = unwrap_owned(y);
@@ -795,7 +839,7 @@ int cg_binary(cg_backend *, cg_binary_op op, cg_tensor *x, cg_tensor *y, cg_tens
 int cg_where(cg_backend *, cg_tensor *mask, cg_tensor *x, cg_tensor *y, cg_tensor **out) {
     Consume cm(mask), cx(x), cy(y);
     if (!mask || !x || !y || !out) return fail(CG_ERR_ARG, "null argument");
-    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
+    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "unknown dtype");
     if (mask->dt != x->dt || y->dt != x->dt) return fail(CG_ERR_DTYPE, "TypeError: mixed dtypes in where");
     if (!same_shape(mask, x) || !same_shape(x, y)) return fail(CG_ERR_SHAPE, "Shape mismatch in operation");
     cg_tensor *om = unwrap_owned(mask), *ox = unwrap_owned(x), *oy = unwrap_owned(y);
@@ -822,7 +866,7 @@ int cg_matmul(cg_backend *, cg_tensor *x, cg_tensor *y, cg_tensor **out) {
     Consume cx(x), cy(y);
     if (!x || !y || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt) || !supported(y->dt))
-        return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
+        return fail(CG_ERR_UNSUPPORTED, "unknown dtype");
     if (x->dt != y->dt) return fail(CG_ERR_DTYPE, "TypeError: mixed dtypes in matmul");
     if (x->rank < 2) return fail(CG_ERR_SHAPE, "batched_matmul: lhs must be at least rank 2");
     if (y->rank < 2) return fail(CG_ERR_SHAPE, "batched_matmul: rhs must be at least rank 2");
@@ -870,7 +914,7 @@ namespace {
 // underflows on rank 0, ndarray.rs:658,672,728).
 int reduce_frame(cg_tensor *x, cg_tensor **out, const char *what, cg_tensor **owned, size_t *rows, size_t *n) {
     if (!x || !out) return fail(CG_ERR_ARG, "null argument");
-    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
+    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "unknown dtype");
     if (x->rank == 0) return fail(CG_ERR_SHAPE, "%s: rank-0 tensor has no last axis", what);
     *owned = unwrap_owned(x);
     *n = x->dims[x->rank - 1];
@@ -1021,7 +1065,7 @@ int cg_topk(cg_backend *, cg_tensor *x, size_t k, cg_tensor **values, cg_tensor 
     Consume cx(x);
     if (!x || !values || !indices) return fail(CG_ERR_ARG, "null argument");
     if (x->dt == CG_U32) return fail(CG_ERR_DTYPE, "Unsupported type for topk");
-    if (!isf(x->dt)) return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
+    if (!isf(x->dt)) return fail(CG_ERR_UNSUPPORTED, "unknown dtype");
     if (x->rank == 0) return fail(CG_ERR_SHAPE, "topk: rank-0 tensor has no last axis");
     size_t n = x->dims[x->rank - 1];
     if (n == 0) return fail(CG_ERR_SHAPE, "topk: attempt to divide by zero (empty last axis)");
@@ -1062,7 +1106,7 @@ int cg_topk(cg_backend *, cg_tensor *x, size_t k, cg_tensor **values, cg_tensor 
 int cg_broadcast(cg_backend *, cg_tensor *x, const size_t *dims, size_t rank, cg_tensor **out) {
     Consume cx(x);
     if (!x || !out || rank > CG_MAX_RANK) return fail(CG_ERR_ARG, "bad arguments");
-    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
+    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "unknown dtype");
     if ((size_t)x->rank > rank) return fail(CG_ERR_SHAPE, "broadcast: called `Option::unwrap()` on a `None` value");
     int shift = (int)rank - x->rank;
     for (int i = 0; i < x->rank; i++)
@@ -1091,7 +1135,7 @@ int cg_broadcast(cg_backend *, cg_tensor *x, const size_t *dims, size_t rank, cg
 int cg_reshape(cg_backend *, cg_tensor *x, const size_t *dims, size_t rank, cg_tensor **out) {
     Consume cx(x);
     if (!x || !out || rank > CG_MAX_RANK) return fail(CG_ERR_ARG, "bad arguments");
-    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
+    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "unknown dtype");
     size_t n = 1;
     for (size_t i = 0; i < rank; i++) n *= dims[i];
     if (n != numel(x)) return fail(CG_ERR_SHAPE, "reshape: ShapeError/IncompatibleShape");
@@ -1107,7 +1151,7 @@ int cg_reshape(cg_backend *, cg_tensor *x, const size_t *dims, size_t rank, cg_t
 int cg_transpose(cg_backend *, cg_tensor *x, size_t dim0, size_t dim1, cg_tensor **out) {
     Consume cx(x);
     if (!x || !out) return fail(CG_ERR_ARG, "null argument");
-    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
+    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "unknown dtype");
     if (dim0 >= (size_t)x->rank || dim1 >= (size_t)x->rank) return fail(CG_ERR_RANGE, "transpose: axis out of range");
     cg_tensor *o = unwrap_owned(x);
     cg_tensor *v = view_of(o);
@@ -1122,7 +1166,7 @@ int cg_transpose(cg_backend *, cg_tensor *x, size_t dim0, size_t dim1, cg_tensor
 int cg_slice(cg_backend *, cg_tensor *x, size_t dim, size_t start, size_t len, cg_tensor **out) {
     Consume cx(x);
     if (!x || !out) return fail(CG_ERR_ARG, "null argument");
-    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
+    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "unknown dtype");
     if (dim >= (size_t)x->rank) return fail(CG_ERR_RANGE, "slice: axis out of range");
     if (start > x->dims[dim] || len > x->dims[dim] - start) return fail(CG_ERR_RANGE, "slice: range out of bounds");
     cg_tensor *o = unwrap_owned(x);
@@ -1139,7 +1183,7 @@ int cg_concat(cg_backend *, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor **
     Consume cx(x), cy(y);
     if (!x || !y || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt) || !supported(y->dt))
-        return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
+        return fail(CG_ERR_UNSUPPORTED, "unknown dtype");
     if (x->dt != y->dt) return fail(CG_ERR_DTYPE, "Incompatible types for concatenation");
     if (x->rank != y->rank || dim >= (size_t)x->rank) return fail(CG_ERR_SHAPE, "concat: IncompatibleShape");
     for (int i = 0; i < x->rank; i++)
@@ -1169,7 +1213,7 @@ int cg_concat(cg_backend *, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor **
 int cg_index(cg_backend *, cg_tensor *x, size_t dim, cg_tensor *indices, cg_tensor **out) {
     Consume cx(x), ci(indices);
     if (!x || !indices || !out) return fail(CG_ERR_ARG, "null argument");
-    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "fp8 is not supported by the ndarray backend");
+    if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "unknown dtype");
     if (indices->dt != CG_U32) return fail(CG_ERR_DTYPE, "Invalid input types for indexing");
     if (dim >= (size_t)x->rank) return fail(CG_ERR_RANGE, "index: axis out of range");
     cg_tensor *ox = unwrap_owned(x), *oi = unwrap_owned(indices);

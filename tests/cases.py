@@ -1425,6 +1425,8 @@ def assert_close(kind, got, exp, scale=None, name=""):
         # of the value at most, plus the spacing of f16 subnormals
         rtol, atol = (2.0 ** -10, 2.0 ** -24) if kind == "ulp_f16" else (2.0 ** -7, 1e-38)
         np.testing.assert_allclose(got.astype(np.float64), exp.astype(np.float64), rtol=rtol, atol=atol, err_msg=name)
+    elif kind == "ulp_f8":  # one unit in the last place of E4M3 (4-bit significand), plus the spacing of its subnormals
+        np.testing.assert_allclose(got.astype(np.float64), exp.astype(np.float64), rtol=2.0 ** -3, atol=2.0 ** -9, err_msg=name)
     elif kind == "red":
         s = np.asarray(scale, dtype=np.float64) if scale is not None else np.abs(exp.astype(np.float64))
         err = np.abs(got.astype(np.float64) - exp.astype(np.float64))
@@ -1435,3 +1437,4 @@ def assert_close(kind, got, exp, scale=None, name=""):
 
 
 import cases_half  # noqa: E402,F401  (appends the 16-bit float cases to CASES)
+import cases_fp8  # noqa: E402,F401  (appends the fp8 cases to CASES)

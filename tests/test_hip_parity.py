@@ -75,9 +75,9 @@ def test_error_paths(hip):
         lambda: hip.index(x, 0, x),
         lambda: hip.max(hip.from_numpy(np.float32(1).reshape(()))),
         lambda: hip.argmax(hip.zeros((3, 0), A.F32)),
-        lambda: hip.zeros((2, 2), A.F8),
-        lambda: hip.cast(x, A.F8),
-        lambda: hip.ndarray_from_vec_fp8(np.zeros(4, np.uint8), (4,)),
+        lambda: hip.zeros((2, 2), 9),            # not a dtype
+        lambda: hip.cast(x, 9),
+        lambda: hip.add(hip.cast(x, A.F8), hip.cast(x, A.BF16)),
         lambda: hip.add(hip.cast(x, A.F16), hip.cast(x, A.BF16)),
         lambda: hip.matmul(hip.cast(x, A.F16), hip.transpose(x, 0, 1)),
         lambda: hip.div(hip.broadcast(hip.from_numpy(np.uint32(3).reshape(())), (2,)),

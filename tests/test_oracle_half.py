@@ -78,7 +78,7 @@ def test_dtype_rules(oracle):
     assert (h.dtype, bh.dtype) == (A.F16, A.BF16)
     assert oracle.cast(h, A.F16).dtype == A.F16
     for bad in (lambda: oracle.add(h, bh), lambda: oracle.mul(h, x), lambda: oracle.matmul(h, oracle.transpose(x, 0, 1)),
-                lambda: oracle.zeros((2,), A.F8), lambda: oracle.cast(x, A.F8),
+                lambda: oracle.zeros((2,), 9), lambda: oracle.cast(x, 9), lambda: oracle.add(h, oracle.cast(x, A.F8)),
                 lambda: oracle.sin(oracle.cast(h, A.U32))):
         with pytest.raises(BackendPanic):
             bad()
