@@ -129,6 +129,12 @@ struct Buffer {
     RowStore *rs = nullptr;      // owned
     bool constant = false;       // the contents depend on constants only (iota, programs over such buffers)
     Buffer *successor = nullptr; // retained: the roomier buffer that blocks of this one migrate to on append
+    // Set by the product kernels that store a residual stream [rows <= 4, N]: per workgroup (4 columns) and row
+    // the sum of squares of what it stored, [side_blocks][4] floats.  An RMS norm over these rows that feeds
+    // decode-time products needs no pass of its own then (see NormFuse).  Owned (pool memory).
+    void *side = nullptr;
+    size_t side_cls = 0;
+    uint32_t side_blocks = 0;
 };
 
 } // namespace cg
@@ -258,9 +264,20 @@ struct DeferredWrite {
     Pending *prog = nullptr;  // owned
 };
 
+// x / pow(sum(x*x) / n + eps, e) * gamma applied to the left operand while a decode-time product loads it:
+// the row sums come from the per-workgroup partial sums that the kernel which stored x left behind.
+struct NormFuse {
+    const float *partials; // [blocks][4]
+    uint32_t blocks;
+    const uint32_t *gamma; // [K]
+    uint32_t n_bits, eps_bits, exp_bits;
+};
+
 struct LazyMm {
     std::atomic<long> rc{1};
-    cg_tensor *x = nullptr, *y = nullptr; // retained operands (concrete)
+    // retained operands; y is concrete, x is concrete or (groupable products only) still the deferred RMS norm
+    // of a residual stream with partial sums, see norm_fuse_of
+    cg_tensor *x = nullptr, *y = nullptr;
     Buffer *result = nullptr;             // retained once computed
     int64_t dims[kMaxRank] = {0};
     int rank = 0;
@@ -411,17 +428,21 @@ struct MmFold {
 int fold_matmul(const cg_tensor *x, const cg_tensor *y, MmFold *f);
 // Several skinny products x . ys[i] -> outs[i] (n of them, the same x) in one launch; kDeclined (declared
 // below) when the shapes do not allow it.
+// nf != null: x is the residual stream and the kernel applies the RMS norm to it on load (needs M in 2..4 and K a
+// multiple of 2048; kDeclined otherwise, before anything is launched).
 int launch_matmul_gated(cg_backend *be, const cg_tensor *x, const cg_tensor *yg, const cg_tensor *yu, uint32_t one,
-                        cg_tensor *out);
+                        cg_tensor *out, const NormFuse *nf = nullptr);
 int launch_prefill_attention(cg_backend *be, const Pending &p, const int64_t *pdims, int prank, const cg_tensor *q,
                              const cg_tensor *kt, const cg_tensor *v, cg_tensor *out);
 int launch_fused_group(cg_backend *be, const cg_tensor *const *outs, const Pending *const *ps, int n);
 // Writes that were put off so that they can share a launch (see DeferredWrite); every function
 // that launches a kernel or copies device memory calls this first.
 int flush_deferred(cg_backend *be);
-int launch_matmul_residual(cg_backend *be, const cg_tensor *x, const cg_tensor *y, const uint32_t *const *terms, int slot,
-                           int order, cg_tensor *out);
-int launch_matmul_group(cg_backend *be, const cg_tensor *x, const cg_tensor *const *ys, cg_tensor *const *outs, int n);
+// nterms: 2 (out = t0 + t1) or 4.  On success out->buf may have received the partial sums of squares (Buffer::side).
+int launch_matmul_residual(cg_backend *be, const cg_tensor *x, const cg_tensor *y, const uint32_t *const *terms, int nterms,
+                           int slot, int order, cg_tensor *out);
+int launch_matmul_group(cg_backend *be, const cg_tensor *x, const cg_tensor *const *ys, cg_tensor *const *outs, int n,
+                        const NormFuse *nf = nullptr);
 
 // Decode-time attention in one pass: out = softmax-program(q . kT) . v, where `p` is the deferred
 // soft-max program whose leaf 0 is the (never computed) lazy product q . kT and (pdims, prank) its

@@ -384,7 +384,16 @@ template <int MM> __global__ __launch_bounds__(kThreads) void skinny_kt_kernel(c
 struct MmResidual {
     const uint32_t *term[4];
     uint32_t slot, order;
+    uint32_t nterms;  // 4, or 2: out = t0 + t1
+    float *partials;  // null, or [workgroups][4]: per row the sum of squares of the four columns stored
 };
+// the sum, given all its terms
+__device__ __forceinline__ uint32_t residual_sum(const MmResidual &r, const uint32_t (&t)[4]) {
+    if (r.nterms == 2) return apply<kAdd, true>(t[0], t[1], 0, nullptr);
+    const uint32_t inner = apply<kAdd, true>(t[1], t[2], 0, nullptr);
+    return r.order == 0 ? apply<kAdd, true>(apply<kAdd, true>(t[0], inner, 0, nullptr), t[3], 0, nullptr)
+                        : apply<kAdd, true>(t[0], apply<kAdd, true>(inner, t[3], 0, nullptr), 0, nullptr);
+}
 
 #ifndef CG_WIDE_UNROLL
 #define CG_WIDE_UNROLL 2
@@ -410,7 +419,7 @@ __device__ __forceinline__ void skinny_kt_wide_body(const MmArgs &a, const uint3
             for (int m = 0; m < MM; m++)
 #pragma unroll
                 for (int t = 0; t < 4; t++)
-                    if ((uint32_t)m < a.M && (uint32_t)t != res->slot)
+                    if ((uint32_t)m < a.M && (uint32_t)t != res->slot && (uint32_t)t < res->nterms)
                         term[m][t] = res->term[t][((uint64_t)block_y * a.M + m) * a.N + n0];
         }
     }
@@ -477,9 +486,7 @@ __device__ __forceinline__ void skinny_kt_wide_body(const MmArgs &a, const uint3
                         uint32_t t[4];
 #pragma unroll
                         for (int i = 0; i < 4; i++) t[i] = (uint32_t)i == res->slot ? v : term[m][i];
-                        const uint32_t inner = apply<kAdd, true>(t[1], t[2], 0, nullptr);
-                        v = res->order == 0 ? apply<kAdd, true>(apply<kAdd, true>(t[0], inner, 0, nullptr), t[3], 0, nullptr)
-                                            : apply<kAdd, true>(t[0], apply<kAdd, true>(inner, t[3], 0, nullptr), 0, nullptr);
+                        v = residual_sum(*res, t);
                     }
                     a.C[((uint64_t)block_y * a.M + m) * a.N + n0 + c] = v;
                 }
@@ -532,10 +539,16 @@ template <int MM> __global__ __launch_bounds__(kThreads) void skinny_kt_wide_gro
 // GATED (CG = 2): the two column groups are the same four columns of two weight matrices, a.B and
 // `second` (same shape and strides), and the block writes g * (1 / (one + exp(-g))) * u for
 // g = x.B^T, u = x.second^T: the SiLU-gated pair of an MLP block without writing g and u.
-template <int MM, int CG, bool GATED = false, bool RESIDUAL = false>
+// pow(sum / n + eps, e): the divisor of an RMS norm from its row's sum of squares, in the program's own ops
+__device__ __forceinline__ uint32_t norm_divisor(const NormFuse &nf, float sum) {
+    const uint32_t mean = apply<kDiv, true>(asu(sum), nf.n_bits, 0, nullptr);
+    return apply<kPow, true>(apply<kAdd, true>(mean, nf.eps_bits, 0, nullptr), nf.exp_bits, 0, nullptr);
+}
+template <int MM, int CG, bool GATED = false, bool RESIDUAL = false, bool NORM = false>
 __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const uint32_t block_x, const uint32_t block_y,
                                                          const uint32_t *second = nullptr, const uint32_t one = 0,
-                                                         const MmResidual *res = nullptr) {
+                                                         const MmResidual *res = nullptr, const NormFuse *nf = nullptr) {
+    static_assert(!NORM || MM == 4, "the norm's row sums are kept for four rows");
     static_assert(!GATED || CG == 2, "a gated pair is two column groups");
     static_assert(!(GATED && RESIDUAL), "one epilogue at a time");
     constexpr int G = MM / 4;
@@ -565,8 +578,21 @@ __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const 
             if (col < a.N && m < a.M) {
 #pragma unroll
                 for (int t = 0; t < 4; t++)
-                    if ((uint32_t)t != res->slot) term[t] = res->term[t][((uint64_t)block_y * a.M + m) * a.N + col];
+                    if ((uint32_t)t != res->slot && (uint32_t)t < res->nterms)
+                        term[t] = res->term[t][((uint64_t)block_y * a.M + m) * a.N + col];
             }
+        }
+    }
+    // NORM: the products are taken of x * gamma and divided by d_m = pow(sum(x[m]^2) / n + eps, e) where they are stored:
+    // (x / d * gamma) . w = ((x * gamma) . w) / d.  The row sums are put together from the partial sums that the kernel
+    // which stored x left (always in the same order); thread t takes entries t, t + 256, ... of [blocks][4], all of row
+    // t % 4.  The first eight per thread are asked for here and added up after the walk along K: nothing waits for them.
+    float pv[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if constexpr (NORM) {
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const uint32_t i = threadIdx.x + u * kThreads;
+            if (i < nf->blocks * 4) pv[u] = nf->partials[i];
         }
     }
     // of every 2048 values of k a wave takes 512 in a row (8 trips of 64): 2 KiB of each weight row
@@ -580,6 +606,13 @@ __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const 
             for (int g = 0; g < G; g++) {
                 xr[g][t] = (float4v){0.f, 0.f, 0.f, 0.f};
                 if (k < a.K) xr[g][t] = *reinterpret_cast<const float4v *>(xrow[g] + k);
+                if constexpr (NORM) {
+                    if (k < a.K) {
+                        const float4v gm = *reinterpret_cast<const float4v *>(nf->gamma + k);
+#pragma unroll
+                        for (int e = 0; e < 4; e++) xr[g][t][e] = asf(apply<kMul, true>(asu(xr[g][t][e]), asu(gm[e]), 0, nullptr));
+                    }
+                }
             }
         }
 #pragma unroll
@@ -603,6 +636,16 @@ __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const 
         }
     }
     __shared__ float part[4][CG * MM * 4];
+    __shared__ float nsum[4][4];
+    if constexpr (NORM) {
+        float s = 0.0f;
+#pragma unroll
+        for (int u = 0; u < 8; u++) s += pv[u];
+        for (uint32_t i = threadIdx.x + 8 * kThreads; i < nf->blocks * 4; i += kThreads) s += nf->partials[i];
+#pragma unroll
+        for (int sh = 32; sh >= 4; sh >>= 1) s += __shfl_xor(s, sh);
+        if (lane < 4) nsum[wave][lane] = s;
+    }
 #pragma unroll
     for (int c = 0; c < CG; c++)
 #pragma unroll
@@ -618,8 +661,13 @@ __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const 
     if constexpr (GATED) {
         if (threadIdx.x < MM * 4) {
             const uint32_t t = threadIdx.x, u_at = MM * 4 + t, m = t / 4, col = n0 + t % 4;
-            const uint32_t gv = asu((part[0][t] + part[1][t]) + (part[2][t] + part[3][t]));
-            const uint32_t uv = asu((part[0][u_at] + part[1][u_at]) + (part[2][u_at] + part[3][u_at]));
+            uint32_t gv = asu((part[0][t] + part[1][t]) + (part[2][t] + part[3][t]));
+            uint32_t uv = asu((part[0][u_at] + part[1][u_at]) + (part[2][u_at] + part[3][u_at]));
+            if constexpr (NORM) {
+                const uint32_t d = norm_divisor(*nf, (nsum[0][m % 4] + nsum[1][m % 4]) + (nsum[2][m % 4] + nsum[3][m % 4]));
+                gv = apply<kDiv, true>(gv, d, 0, nullptr);
+                uv = apply<kDiv, true>(uv, d, 0, nullptr);
+            }
             // the ops of the deferred program, in its order
             const uint32_t e = apply<kExp, true>(apply<kNeg, true>(gv, 0, 0, nullptr), 0, 0, nullptr);
             const uint32_t sg = apply<kDiv, true>(one, apply<kAdd, true>(one, e, 0, nullptr), 0, nullptr);
@@ -629,14 +677,24 @@ __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const 
     } else if (threadIdx.x < CG * MM * 4) {
         const uint32_t c = threadIdx.x / (MM * 4), m = threadIdx.x / 4 % MM, col = n0 + 4 * c + threadIdx.x % 4;
         uint32_t v = asu((part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]));
+        if constexpr (NORM)
+            v = apply<kDiv, true>(v, norm_divisor(*nf, (nsum[0][m % 4] + nsum[1][m % 4]) + (nsum[2][m % 4] + nsum[3][m % 4])), 0, nullptr);
         if constexpr (RESIDUAL) {
 #pragma unroll
             for (int t = 0; t < 4; t++) term[t] = (uint32_t)t == res->slot ? v : term[t];
-            const uint32_t inner = apply<kAdd, true>(term[1], term[2], 0, nullptr);
-            v = res->order == 0 ? apply<kAdd, true>(apply<kAdd, true>(term[0], inner, 0, nullptr), term[3], 0, nullptr)
-                                : apply<kAdd, true>(term[0], apply<kAdd, true>(inner, term[3], 0, nullptr), 0, nullptr);
+            v = residual_sum(*res, term);
         }
-        if (col < a.N && m < a.M) a.C[((uint64_t)block_y * a.M + m) * a.N + col] = v;
+        const bool stored = col < a.N && m < a.M;
+        if (stored) a.C[((uint64_t)block_y * a.M + m) * a.N + col] = v;
+        if constexpr (RESIDUAL) {
+            // threads 0..15 = (row m, column n0 + t % 4): the row's sum of squares over the block's four columns
+            if (res->partials) {
+                float q = stored ? asf(v) * asf(v) : 0.0f;
+                q += __shfl_xor(q, 1);
+                q += __shfl_xor(q, 2);
+                if (threadIdx.x % 4 == 0) res->partials[(uint64_t)block_x * 4 + m] = q;
+            }
+        }
     }
 }
 
@@ -651,10 +709,21 @@ template <int MM>
 __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_residual_kernel(const MmArgs a, const MmResidual r) {
     skinny_kt_mfma_xreg_body<MM, 1, false, true>(a, blockIdx.x, blockIdx.y, nullptr, 0, &r);
 }
+// the same with the RMS norm of the left operand applied on load
+__global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_gated_norm_kernel(const MmArgs a, const uint32_t *second, uint32_t one,
+                                                                                  const NormFuse nf) {
+    skinny_kt_mfma_xreg_body<4, 2, true, false, true>(a, blockIdx.x, blockIdx.y, second, one, nullptr, &nf);
+}
 template <int MM, int CG> __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_group_kernel(const MmGroup g) {
     uint32_t bx;
     const uint32_t p = group_problem(g, bx);
     skinny_kt_mfma_xreg_body<MM, CG>(g.p[p], bx, 0);
+}
+
+__global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_group_norm_kernel(const MmGroup g, const NormFuse nf) {
+    uint32_t bx;
+    const uint32_t p = group_problem(g, bx);
+    skinny_kt_mfma_xreg_body<4, 1, false, false, true>(g.p[p], bx, 0, nullptr, 0, nullptr, &nf);
 }
 
 // Vectorised skinny kernel for short K (K <= 4*LPC, e.g. q.K^T of a decode step with
@@ -894,9 +963,10 @@ static int make_mm_args(const cg_tensor *x, const cg_tensor *y, void *c, MmArgs 
     return CG_OK;
 }
 
-int launch_matmul_group(cg_backend *be, const cg_tensor *x, const cg_tensor *const *ys, cg_tensor *const *outs, int n) {
+int launch_matmul_group(cg_backend *be, const cg_tensor *x, const cg_tensor *const *ys, cg_tensor *const *outs, int n,
+                        const NormFuse *nf) {
     if (int frc = flush_deferred(be)) return frc;
-    if (n < 2 || n > kMaxGroup || x->dt != CG_F32) return kDeclined;
+    if (n < (nf ? 1 : 2) || n > kMaxGroup || x->dt != CG_F32) return kDeclined;
     MmGroup g;
     memset(&g, 0, sizeof g);
     double bytes = distinct_bytes(x);
@@ -912,8 +982,11 @@ int launch_matmul_group(cg_backend *be, const cg_tensor *x, const cg_tensor *con
         all_wide = all_wide && a.N >= 8192;
         bytes += distinct_bytes(ys[i]) + distinct_bytes(outs[i]);
     }
-    const bool xreg = all_wide && g.p[0].M <= 4;
+    const bool xreg = !nf && all_wide && g.p[0].M <= 4;
     const bool xreg1 = !xreg && xreg_narrow(g.p[0].M, g.p[0].K);
+    if (nf && !xreg1) return kDeclined;
+    for (int i = 0; i < n && nf; i++)
+        if (g.p[i].N >= 8192) return kDeclined; // a vocabulary-sized product: the kernel with more columns per wave, the norm on its own
     uint32_t blocks = 0;
     for (int i = 0; i < n; i++) {
         g.first[i] = blocks;
@@ -924,6 +997,8 @@ int launch_matmul_group(cg_backend *be, const cg_tensor *x, const cg_tensor *con
     ProfScope prof(be, CG_K_GEMM_SKINNY, bytes);
     if (xreg)
         hipLaunchKernelGGL((skinny_kt_mfma_xreg_group_kernel<4, 2>), dim3(blocks), dim3(kThreads), 0, be->stream, g);
+    else if (nf)
+        hipLaunchKernelGGL(skinny_kt_mfma_xreg_group_norm_kernel, dim3(blocks), dim3(kThreads), 0, be->stream, g, *nf);
     else if (xreg1)
         hipLaunchKernelGGL((skinny_kt_mfma_xreg_group_kernel<4, 1>), dim3(blocks), dim3(kThreads), 0, be->stream, g);
     else if (g.p[0].M <= 1)
@@ -940,7 +1015,7 @@ int launch_matmul_group(cg_backend *be, const cg_tensor *x, const cg_tensor *con
 // the program between them and the next product in one launch.  Declines unless the 4x4x1
 // kernel takes the shapes.
 int launch_matmul_gated(cg_backend *be, const cg_tensor *x, const cg_tensor *yg, const cg_tensor *yu, uint32_t one,
-                        cg_tensor *out) {
+                        cg_tensor *out, const NormFuse *nf) {
     if (int frc = flush_deferred(be)) return frc;
     if (x->dt != CG_F32) return kDeclined;
     MmArgs ag, au;
@@ -952,8 +1027,12 @@ int launch_matmul_gated(cg_backend *be, const cg_tensor *x, const cg_tensor *yg,
     if (fg.batch != 1 || fu.batch != 1 || ag.M > 4 || ag.b_sk != 1 || au.b_sk != 1 || !vec || ag.K <= 256 || ag.N < 4096 ||
         au.N != ag.N || au.K != ag.K || au.M != ag.M || au.b_sn != ag.b_sn)
         return kDeclined;
+    if (nf && ag.K % 2048 != 0) return kDeclined;
     ProfScope prof(be, CG_K_GEMM_SKINNY, distinct_bytes(x) + distinct_bytes(yg) + distinct_bytes(yu) + distinct_bytes(out));
-    hipLaunchKernelGGL((skinny_kt_mfma_xreg_gated_kernel<4>), dim3((ag.N + 3) / 4), dim3(kThreads), 0, be->stream, ag, au.B, one);
+    if (nf)
+        hipLaunchKernelGGL(skinny_kt_mfma_xreg_gated_norm_kernel, dim3((ag.N + 3) / 4), dim3(kThreads), 0, be->stream, ag, au.B, one, *nf);
+    else
+        hipLaunchKernelGGL((skinny_kt_mfma_xreg_gated_kernel<4>), dim3((ag.N + 3) / 4), dim3(kThreads), 0, be->stream, ag, au.B, one);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? CG_OK : hip_fail(e, "gated matmul launch");
 }
@@ -961,8 +1040,8 @@ int launch_matmul_gated(cg_backend *be, const cg_tensor *x, const cg_tensor *yg,
 // out = a sum of four terms, term[slot] = x.y, the other three dense tensors of out's shape
 // (device pointers); `order` as in MmResidual.  Declines unless the one-column-per-wave kernel
 // is what the product would run on anyway.
-int launch_matmul_residual(cg_backend *be, const cg_tensor *x, const cg_tensor *y, const uint32_t *const *terms, int slot,
-                           int order, cg_tensor *out) {
+int launch_matmul_residual(cg_backend *be, const cg_tensor *x, const cg_tensor *y, const uint32_t *const *terms, int nterms,
+                           int slot, int order, cg_tensor *out) {
     if (int frc = flush_deferred(be)) return frc;
     if (x->dt != CG_F32) return kDeclined;
     MmArgs a;
@@ -972,9 +1051,22 @@ int launch_matmul_residual(cg_backend *be, const cg_tensor *x, const cg_tensor *
     const bool vec = a.a_vec && a.b_vec && a.a_sk == 1 && a.K % 4 == 0;
     if (f.batch != 1 || a.M > 8 || a.b_sk != 1 || !vec || a.K <= 256 || a.N < 2048 || a.N >= 8192) return kDeclined;
     MmResidual r;
-    for (int t = 0; t < 4; t++) r.term[t] = t == slot ? nullptr : terms[t];
+    for (int t = 0; t < 4; t++) r.term[t] = t == slot || t >= nterms ? nullptr : terms[t];
     r.slot = (uint32_t)slot;
     r.order = (uint32_t)order;
+    r.nterms = (uint32_t)nterms;
+    r.partials = nullptr;
+    const uint32_t blocks = (uint32_t)((a.N + 3) / 4);
+    if (xreg_narrow(a.M, a.K) && !out->buf->side) {
+        // the stored rows' sums of squares per workgroup, for an RMS norm that may follow (Buffer::side)
+        Buffer *ob = out->buf;
+        if (be->pool.alloc((size_t)blocks * 4 * sizeof(float), &ob->side, &ob->side_cls) == CG_OK) {
+            ob->side_blocks = blocks;
+            r.partials = static_cast<float *>(ob->side);
+        } else {
+            ob->side = nullptr;
+        }
+    }
     ProfScope prof(be, CG_K_GEMM_SKINNY, distinct_bytes(x) + distinct_bytes(y) + 4.0 * distinct_bytes(out));
     dim3 grid((uint32_t)((a.N + 3) / 4));
     if (xreg_narrow(a.M, a.K))

@@ -19,7 +19,8 @@
 namespace cg {
 
 static thread_local std::string g_err;
-static std::mutex g_lazy_mu; // guards lazy backing of uniform tensors
+static std::recursive_mutex g_lazy_mu; // guards lazy backing of uniform tensors and of deferred ones (computing one may compute another)
+static int ensure_concrete(cg_tensor *t);
 
 int fail(int code, const char *fmt, ...) {
     char buf[512];
@@ -112,6 +113,7 @@ bool is_contiguous(const cg_tensor *t) {
 static void buffer_release(Buffer *b) {
     while (b && b->rc.fetch_sub(1) == 1) {
         if (b->ptr) b->be->pool.free(b->ptr, b->cls);
+        if (b->side) b->be->pool.free(b->side, b->side_cls);
         Buffer *next = b->successor;
         delete b->rs;
         delete b;
@@ -136,6 +138,74 @@ Pending::~Pending() {
         buffer_release(leaf[l].buf2);
         lazy_mm_release(leaf[l].lazy);
     }
+}
+
+// Is x (still) the deferred program  h / pow(sum(h * h) / n + eps, e) * gamma  over the rows of a residual stream h
+// [rows <= 4, K] whose kernel left the partial sums of squares (Buffer::side)?  Then a decode-time product can apply
+// the norm while it loads h (K a multiple of 2048) and the norm needs no launch.  Fills nf and the stand-in tensor
+// h (a borrowed view of the leaf's buffer: set h->buf to null before it goes out of scope).
+static bool norm_fuse_of(const cg_tensor *x, NormFuse *nf, cg_tensor *h) {
+    static const uint8_t code[7][4] = {{kMul, 0, 0, 0},   {kRowSum, 8, 8, 8}, {kDiv, 9, 1, 9},  {kAdd, 10, 2, 10},
+                                       {kPow, 11, 3, 11}, {kDiv, 0, 12, 0},   {kMul, 13, 4, 13}};
+    const Pending *p = x->pend;
+    if (!p || !x->be->aot || x->dt != CG_F32 || x->rank < 2 || x->split >= 0) return false;
+    if (p->nleaf != 5 || p->ninstr != 7 || p->nred != 1 || p->reduced) return false;
+    for (int i = 0; i < 7; i++)
+        if (p->ins[i].op != code[i][0] || p->ins[i].a != code[i][1] || p->ins[i].b != code[i][2] || p->ins[i].c != code[i][3]) return false;
+    const int r = x->rank;
+    const int64_t K = x->dims[r - 1], rows = K > 0 ? numel(x) / K : 0;
+    if (K <= 0 || K % 2048 != 0 || rows < 2 || rows > 4 || p->rowlen != K) return false;
+    const LeafView &lh = p->leaf[0], &lg = p->leaf[4];
+    if (lh.uniform || lh.pw || lh.lazy || !lh.buf || !lh.buf->side || lh.offset != 0 || (int64_t)lh.buf->side_blocks * 4 != K) return false;
+    if (!p->leaf[1].uniform || !p->leaf[2].uniform || !p->leaf[3].uniform) return false;
+    if (lg.uniform || lg.pw || lg.lazy || !lg.buf || lg.offset % 4 != 0) return false;
+    int64_t st = 1;
+    for (int d = r - 1; d >= 0; d--) { // h dense in the program's space, gamma along the last axis only
+        if (x->dims[d] != 1 && lh.strides[d] != st) return false;
+        if (x->dims[d] != 1 && lg.strides[d] != (d == r - 1 ? 1 : 0)) return false;
+        st *= x->dims[d];
+    }
+    nf->partials = static_cast<const float *>(lh.buf->side);
+    nf->blocks = lh.buf->side_blocks;
+    nf->gamma = static_cast<const uint32_t *>(lg.buf->ptr) + lg.offset;
+    nf->n_bits = p->leaf[1].ubits;
+    nf->eps_bits = p->leaf[2].ubits;
+    nf->exp_bits = p->leaf[3].ubits;
+    h->be = x->be;
+    h->buf = lh.buf;
+    h->dt = CG_F32;
+    h->rank = r;
+    memcpy(h->dims, x->dims, sizeof h->dims);
+    int64_t s2 = 1;
+    for (int d = r - 1; d >= 0; d--) {
+        h->strides[d] = s2;
+        s2 *= x->dims[d];
+    }
+    h->offset = 0;
+    return true;
+}
+
+// t0 + t1 with one term a decode-time product nobody has needed yet and of the extent that the products' residual
+// store takes (the residual stream after an o or down projection): worth computing where it stands — the add runs
+// in the product's store and the row sums of squares come with it — rather than carrying it into a longer program.
+static bool residual_sum_open(const cg_tensor *x) {
+    const Pending *p = x->pend;
+    if (!p || !x->be->aot || x->dt != CG_F32 || p->nleaf != 2 || p->ninstr != 1 || p->nred != 0) return false;
+    if (p->ins[0].op != kAdd || p->ins[0].a + p->ins[0].b != 1) return false;
+    int open = 0;
+    for (int l = 0; l < 2; l++) {
+        const LeafView &lv = p->leaf[l];
+        if (lv.uniform || lv.pw) return false;
+        if (lv.lazy && !lv.lazy->result) {
+            const LazyMm *m = lv.lazy;
+            const int64_t N = m->rank > 0 ? m->dims[m->rank - 1] : 0;
+            if (!m->groupable || m->rc.load() != 1 || m->rank != x->rank || N < 2048 || N >= 8192) return false;
+            open++;
+        } else if (!lv.lazy && !lv.buf) {
+            return false;
+        }
+    }
+    return open == 1;
 }
 
 static void lazy_mm_close(LazyMm *m) { // no longer open for grouping
@@ -169,7 +239,10 @@ int lazy_mm_force(cg_backend *be, LazyMm *m) {
         int n = 1;
         for (LazyMm *o : be->lazy_open)
             if (o != m && !o->result && o->x == m->x && n < 4) grp[n++] = o;
-        if (n > 1) {
+        NormFuse nf;
+        cg_tensor h;
+        const bool normed = m->x->pend && norm_fuse_of(m->x, &nf, &h);
+        if (n > 1 || normed) {
             cg_tensor *outs[4] = {nullptr, nullptr, nullptr, nullptr};
             const cg_tensor *ys[4];
             int rc = CG_OK;
@@ -177,7 +250,13 @@ int lazy_mm_force(cg_backend *be, LazyMm *m) {
                 ys[i] = grp[i]->y;
                 rc = new_dense(be, CG_F32, grp[i]->dims, grp[i]->rank, &outs[i]);
             }
-            if (!rc) rc = launch_matmul_group(be, m->x, ys, outs, n);
+            if (!rc && normed) rc = launch_matmul_group(be, &h, ys, outs, n, &nf); // the norm runs in the products' loads
+            h.buf = nullptr;
+            if (!rc && normed) be->programs_compiled++;
+            if ((!rc && !normed) || (normed && rc == kDeclined)) {
+                rc = m->x->pend ? ensure_concrete(m->x) : CG_OK;
+                if (!rc) rc = n > 1 ? launch_matmul_group(be, m->x, ys, outs, n) : kDeclined;
+            }
             if (rc == CG_OK)
                 for (int i = 0; i < n; i++) {
                     grp[i]->result = outs[i]->buf;
@@ -189,6 +268,10 @@ int lazy_mm_force(cg_backend *be, LazyMm *m) {
         }
     }
     lazy_mm_close(m);
+    if (m->x->pend) { // a left operand still deferred (see norm_fuse_of): this launch takes it from memory
+        int xrc = ensure_concrete(m->x);
+        if (xrc) return xrc;
+    }
     cg_tensor *o;
     int rc = new_dense(be, CG_F32, m->dims, m->rank, &o);
     if (rc) return rc;
@@ -280,7 +363,7 @@ int device_ptr(const cg_tensor *t, const void **ptr) {
             *ptr = nullptr;
             return CG_OK;
         }
-        std::lock_guard<std::mutex> lk(g_lazy_mu);
+        std::lock_guard<std::recursive_mutex> lk(g_lazy_mu);
         if (!t->buf) {
             Buffer *b = new Buffer;
             b->be = t->be;
@@ -712,7 +795,23 @@ static int try_gated_pair(cg_backend *be, const cg_tensor *dst, const Pending &p
         st *= dst->dims[d];
     }
     if (lg.offset != 0 || lu.offset != 0) return kDeclined;
-    int rc = launch_matmul_gated(be, mg->x, mg->y, mu->y, lc.ubits, const_cast<cg_tensor *>(dst));
+    int rc = kDeclined;
+    {
+        NormFuse nf;
+        cg_tensor h;
+        if (mg->x->pend && norm_fuse_of(mg->x, &nf, &h)) { // the norm runs in the products' loads
+            rc = launch_matmul_gated(be, &h, mg->y, mu->y, lc.ubits, const_cast<cg_tensor *>(dst), &nf);
+            if (rc == CG_OK) be->programs_compiled++;
+        }
+        h.buf = nullptr;
+    }
+    if (rc == kDeclined) {
+        if (mg->x->pend) {
+            int xrc = ensure_concrete(mg->x);
+            if (xrc) return xrc;
+        }
+        rc = launch_matmul_gated(be, mg->x, mg->y, mu->y, lc.ubits, const_cast<cg_tensor *>(dst));
+    }
     if (rc == CG_OK) {
         lazy_mm_close(mg);
         lazy_mm_close(mu);
@@ -725,17 +824,23 @@ static int try_gated_pair(cg_backend *be, const cg_tensor *dst, const Pending &p
 // o or down projection): the adds run in the product's store.
 static int try_residual_store(cg_backend *be, const cg_tensor *dst, const Pending &p) {
     static const uint8_t orders[2][3][2] = {{{1, 2}, {0, 8}, {9, 3}}, {{1, 2}, {8, 3}, {0, 9}}};
-    if (p.nleaf != 4 || p.ninstr != 3 || p.nred != 0 || !is_contiguous(dst) || dst->dt != CG_F32) return kDeclined;
+    if (p.nred != 0 || !is_contiguous(dst) || dst->dt != CG_F32) return kDeclined;
     int order = -1;
-    for (int o = 0; o < 2 && order < 0; o++) {
-        bool same = true;
-        for (int i = 0; i < 3; i++) same = same && p.ins[i].op == kAdd && p.ins[i].a == orders[o][i][0] && p.ins[i].b == orders[o][i][1];
-        if (same) order = o;
+    const int nterms = p.nleaf;
+    if (p.nleaf == 2 && p.ninstr == 1) { // t0 + t1, either way round
+        if (p.ins[0].op != kAdd || p.ins[0].a + p.ins[0].b != 1) return kDeclined;
+        order = 0;
+    } else if (p.nleaf == 4 && p.ninstr == 3) {
+        for (int o = 0; o < 2 && order < 0; o++) {
+            bool same = true;
+            for (int i = 0; i < 3; i++) same = same && p.ins[i].op == kAdd && p.ins[i].a == orders[o][i][0] && p.ins[i].b == orders[o][i][1];
+            if (same) order = o;
+        }
     }
     if (order < 0) return kDeclined;
     int slot = -1;
     const uint32_t *terms[4] = {nullptr, nullptr, nullptr, nullptr};
-    for (int l = 0; l < 4; l++) {
+    for (int l = 0; l < nterms; l++) {
         const LeafView &lv = p.leaf[l];
         if (lv.uniform || lv.pw || lv.offset % 4 != 0) return kDeclined;
         int64_t st = 1;
@@ -759,7 +864,11 @@ static int try_residual_store(cg_backend *be, const cg_tensor *dst, const Pendin
     }
     if (slot < 0) return kDeclined;
     LazyMm *m = p.leaf[slot].lazy;
-    int rc = launch_matmul_residual(be, m->x, m->y, terms, slot, order, const_cast<cg_tensor *>(dst));
+    if (m->x->pend) { // a left operand still deferred (see norm_fuse_of): this launch takes it from memory
+        int xrc = ensure_concrete(m->x);
+        if (xrc) return xrc;
+    }
+    int rc = launch_matmul_residual(be, m->x, m->y, terms, nterms, slot, order, const_cast<cg_tensor *>(dst));
     if (rc == CG_OK) {
         lazy_mm_close(m);
         be->programs_compiled++;
@@ -986,7 +1095,7 @@ static bool may_wait(const cg_backend *be, const cg_tensor *dst, const Pending *
 // Turns a deferred tensor into a concrete one, in place (every holder of the handle sees it).
 static int ensure_concrete(cg_tensor *t) {
     if (t->split >= 0) { // a split-axis view becomes a plain dense tensor, in place
-        std::lock_guard<std::mutex> lk(g_lazy_mu);
+        std::lock_guard<std::recursive_mutex> lk(g_lazy_mu);
         if (t->split < 0) return CG_OK;
         cg_tensor *m;
         int rc = materialize(t->be, t, &m);
@@ -1001,7 +1110,7 @@ static int ensure_concrete(cg_tensor *t) {
         return CG_OK;
     }
     if (!t->pend) return CG_OK;
-    std::lock_guard<std::mutex> lk(g_lazy_mu);
+    std::lock_guard<std::recursive_mutex> lk(g_lazy_mu);
     if (!t->pend) return CG_OK;
     cg_backend *be = t->be;
     hipError_t he = hipSetDevice(be->device);
@@ -1169,6 +1278,10 @@ static int defer_elementwise(cg_backend *be, int op, cg_dtype in_dt, cg_dtype ou
     for (int k = 0; k < nin; k++) {
         cg_tensor *x = ins[k];
         if (x->split >= 0) {
+            int rc = ensure_concrete(x);
+            if (rc) return rc;
+        }
+        if (op != kAdd && x->pend && residual_sum_open(x)) { // see there; a further add may still join the sum
             int rc = ensure_concrete(x);
             if (rc) return rc;
         }
@@ -2288,7 +2401,15 @@ static int matmul_entry(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **o
         if (rc != kDeclined) return rc;
         rc = CG_OK;
     }
-    if (x->pend || x->split >= r - 2) rc = ensure_concrete(x);
+    // the RMS norm of a residual stream stays deferred when decode-time products can apply it on load (norm_fuse_of)
+    bool norm_x = false;
+    if (b->fuse && x->pend && r == 3) {
+        NormFuse nfx;
+        cg_tensor hx;
+        norm_x = norm_fuse_of(x, &nfx, &hx);
+        hx.buf = nullptr;
+    }
+    if (!norm_x && (x->pend || x->split >= r - 2)) rc = ensure_concrete(x);
     if (!rc && (y->pend || y->split >= r - 2)) rc = ensure_concrete(y);
     if (!rc && x->split >= 0 && y->split >= 0 && (x->split != y->split || x->split_inner != y->split_inner))
         rc = ensure_concrete(y);
@@ -2303,8 +2424,13 @@ static int matmul_entry(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **o
         // a decode-time linear layer: at most 8 rows in all, the weight shared by the batch
         const bool linear = r == 3 && x->dims[0] * x->dims[1] <= 8 && K > 256 && od[r - 1] >= 64 && y->strides[0] == 0 &&
                             y->split < 0 && is_contiguous(x);
-        if (b->fuse && x->dt == CG_F32 && n_out > 0 && (scores || linear) && K % 4 == 0 && !x->uniform && !y->uniform &&
-            x->split < 0 && y->strides[r - 2] == 1) {
+        const bool lazy = b->fuse && x->dt == CG_F32 && n_out > 0 && (scores || linear) && K % 4 == 0 && !x->uniform && !y->uniform &&
+                          x->split < 0 && y->strides[r - 2] == 1;
+        if (norm_x && !(lazy && linear)) { // not a product that could apply the norm: the norm runs now
+            rc = ensure_concrete(x);
+            if (rc) return rc;
+        }
+        if (lazy) {
             LazyMm *m = new LazyMm;
             if (linear) {
                 m->groupable = true;

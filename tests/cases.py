@@ -1260,6 +1260,70 @@ for _n in (64, 576, 2048):
         return run, expect
 
 
+def _rmsnorm_ops(be, h, gamma, n, shp):
+    """`rmsnorm` of the decoder graphs (stdlib/nn/mod.rs:208-232): x / sqrt(mean(x^2) + eps) * gamma."""
+    one = shp[:-1] + (1,)
+    s = be.sum(be.mul(h, h))
+    mean = be.div(s, _const(be, float(n), one))
+    rms = be.pow(be.add(mean, _const(be, 1e-5, one)), _const(be, 0.5, one))
+    return be.mul(be.div(h, be.broadcast(rms, shp)), be.broadcast(gamma, shp))
+
+
+for _B, _H, _F, _read_norms in ((4, 2048, 4096, False), (2, 2048, 4096, True), (3, 4096, 8192, False), (4, 512, 4096, False), (1, 2048, 4096, False)):
+    @case(f"decoder_block_B{_B}_H{_H}_F{_F}{'_norms_read' if _read_norms else ''}", "red",
+          (lambda n=5 + 2 * _read_norms: [np.float64(4.0)] * n))   # every output is of order one: 1e-3 of 4
+    def _(B=_B, H=_H, F=_F, read_norms=_read_norms):
+        """The dense part of a decoder layer at decode time (llama.rs:347-365): residual add of the o projection,
+        RMS norm, gate / up / SiLU, down projection, residual add, RMS norm, q / k / v projections.  Where the
+        extents allow it the residual adds run in the stores of the o / down products and the norms in the loads of
+        the products behind them; with `norms_read` the norms are also read back, which makes them run on their own."""
+        rng_ = np.random.default_rng(700 + B + H)
+        sc = np.float32(1.0 / np.sqrt(H))
+        x0 = rng_.standard_normal((B, 1, H)).astype(np.float32)
+        a0 = rng_.standard_normal((B, 1, H)).astype(np.float32)
+        wo = rng_.standard_normal((H, H)).astype(np.float32) * sc
+        wg = rng_.standard_normal((F, H)).astype(np.float32) * sc
+        wu = rng_.standard_normal((F, H)).astype(np.float32) * sc
+        wd = rng_.standard_normal((H, F)).astype(np.float32) * np.float32(1.0 / np.sqrt(F))
+        wq = rng_.standard_normal((H, H)).astype(np.float32) * sc
+        wk = rng_.standard_normal((H // 4, H)).astype(np.float32) * sc
+        wv = rng_.standard_normal((H // 4, H)).astype(np.float32) * sc
+        g1 = (1.0 + 0.1 * rng_.standard_normal(H)).astype(np.float32)
+        g2 = (1.0 + 0.1 * rng_.standard_normal(H)).astype(np.float32)
+
+        def run(be):
+            shp, fs = (B, 1, H), (B, 1, F)
+            h1 = be.add(be.from_numpy(x0), _linear(be, be.from_numpy(a0), be.from_numpy(wo)))
+            n1 = _rmsnorm_ops(be, h1, be.from_numpy(g1), H, shp)
+            g, u = _linear(be, n1, be.from_numpy(wg)), _linear(be, n1, be.from_numpy(wu))
+            e = be.exp(be.neg(g))
+            act = be.mul(be.mul(g, be.div(_const(be, 1.0, fs), be.add(_const(be, 1.0, fs), e))), u)
+            h2 = be.add(h1, _linear(be, act, be.from_numpy(wd)))
+            n2 = _rmsnorm_ops(be, h2, be.from_numpy(g2), H, shp)
+            q, k, v = (_linear(be, n2, be.from_numpy(w)) for w in (wq, wk, wv))
+            outs = [q, k, v, h2, h1]
+            if read_norms:
+                outs += [n1, n2]
+            return N(be, *outs)
+
+        def expect():
+            f8 = np.float64
+
+            def norm(h, gm):
+                return h / np.sqrt((h * h).mean(-1, keepdims=True) + f8(np.float32(1e-5))) * gm.astype(f8)
+
+            h1 = x0.astype(f8) + a0.astype(f8) @ wo.astype(f8).T
+            n1 = norm(h1, g1)
+            G, U = n1 @ wg.astype(f8).T, n1 @ wu.astype(f8).T
+            act = G / (1.0 + np.exp(-G)) * U
+            h2 = h1 + act @ wd.astype(f8).T
+            n2 = norm(h2, g2)
+            outs = [n2 @ wq.astype(f8).T, n2 @ wk.astype(f8).T, n2 @ wv.astype(f8).T, h2, h1]
+            return outs + ([n1, n2] if read_norms else [])
+
+        return run, expect
+
+
 @case("rows_reduced_results_alone", "red")
 def _():
     """Row results that are read back without being broadcast: a lone reduce, ops then reduce,
