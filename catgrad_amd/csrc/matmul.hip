@@ -606,13 +606,15 @@ __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const 
             for (int g = 0; g < G; g++) {
                 xr[g][t] = (float4v){0.f, 0.f, 0.f, 0.f};
                 if (k < a.K) xr[g][t] = *reinterpret_cast<const float4v *>(xrow[g] + k);
-                if constexpr (NORM) {
-                    if (k < a.K) {
-                        const float4v gm = *reinterpret_cast<const float4v *>(nf->gamma + k);
+            }
+        }
+        float4v gm[NORM ? 8 : 1]; // asked for with the activations, multiplied in once the first weights are on their way
+        if constexpr (NORM) {
 #pragma unroll
-                        for (int e = 0; e < 4; e++) xr[g][t][e] = asf(apply<kMul, true>(asu(xr[g][t][e]), asu(gm[e]), 0, nullptr));
-                    }
-                }
+            for (int t = 0; t < 8; t++) {
+                const uint32_t k = k0 + kb + 64 * t;
+                gm[t] = (float4v){0.f, 0.f, 0.f, 0.f};
+                if (k < a.K) gm[t] = *reinterpret_cast<const float4v *>(nf->gamma + k);
             }
         }
 #pragma unroll
@@ -623,6 +625,16 @@ __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const 
                 const uint32_t k = k0 + kb + 64 * t;
                 w[t] = (float4v){0.f, 0.f, 0.f, 0.f};
                 if (k < a.K) w[t] = *reinterpret_cast<const float4v *>(wrow[c] + k);
+            }
+            if constexpr (NORM) {
+                if (c == 0) {
+#pragma unroll
+                    for (int t = 0; t < 8; t++)
+#pragma unroll
+                        for (int g = 0; g < G; g++)
+#pragma unroll
+                            for (int e = 0; e < 4; e++) xr[g][t][e] = asf(apply<kMul, true>(asu(xr[g][t][e]), asu(gm[t][e]), 0, nullptr));
+                }
             }
 #pragma unroll
             for (int t = 0; t < 8; t++)

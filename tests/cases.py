@@ -1263,10 +1263,11 @@ for _n in (64, 576, 2048):
 def _rmsnorm_ops(be, h, gamma, n, shp):
     """`rmsnorm` of the decoder graphs (stdlib/nn/mod.rs:208-232): x / sqrt(mean(x^2) + eps) * gamma."""
     one = shp[:-1] + (1,)
-    s = be.sum(be.mul(h, h))
-    mean = be.div(s, _const(be, float(n), one))
-    rms = be.pow(be.add(mean, _const(be, 1e-5, one)), _const(be, 0.5, one))
-    return be.mul(be.div(h, be.broadcast(rms, shp)), be.broadcast(gamma, shp))
+    # every intermediate handle is given away at its last use, as the graph interpreter does
+    s = be.sum(be.mul(h, h).move())
+    mean = be.div(s.move(), _const(be, float(n), one).move())
+    rms = be.pow(be.add(mean.move(), _const(be, 1e-5, one).move()).move(), _const(be, 0.5, one).move())
+    return be.mul(be.div(h, be.broadcast(rms.move(), shp).move()).move(), be.broadcast(gamma.move(), shp).move())
 
 
 for _B, _H, _F, _read_norms in ((4, 2048, 4096, False), (2, 2048, 4096, True), (3, 4096, 8192, False), (4, 512, 4096, False), (1, 2048, 4096, False)):
@@ -1293,17 +1294,21 @@ for _B, _H, _F, _read_norms in ((4, 2048, 4096, False), (2, 2048, 4096, True), (
 
         def run(be):
             shp, fs = (B, 1, H), (B, 1, F)
-            h1 = be.add(be.from_numpy(x0), _linear(be, be.from_numpy(a0), be.from_numpy(wo)))
+            h1 = be.add(be.from_numpy(x0).move(), _linear(be, be.from_numpy(a0), be.from_numpy(wo)).move())
             n1 = _rmsnorm_ops(be, h1, be.from_numpy(g1), H, shp)
             g, u = _linear(be, n1, be.from_numpy(wg)), _linear(be, n1, be.from_numpy(wu))
-            e = be.exp(be.neg(g))
-            act = be.mul(be.mul(g, be.div(_const(be, 1.0, fs), be.add(_const(be, 1.0, fs), e))), u)
-            h2 = be.add(h1, _linear(be, act, be.from_numpy(wd)))
+            e = be.exp(be.neg(g).move())
+            sg = be.div(_const(be, 1.0, fs).move(), be.add(_const(be, 1.0, fs).move(), e.move()).move())
+            act = be.mul(be.mul(g.move(), sg.move()).move(), u.move())
+            h2 = be.add(h1, _linear(be, act, be.from_numpy(wd)).move())
+            del act
             n2 = _rmsnorm_ops(be, h2, be.from_numpy(g2), H, shp)
             q, k, v = (_linear(be, n2, be.from_numpy(w)) for w in (wq, wk, wv))
             outs = [q, k, v, h2, h1]
             if read_norms:
                 outs += [n1, n2]
+            else:
+                del n1, n2
             return N(be, *outs)
 
         def expect():

@@ -150,6 +150,33 @@ def test_decode_attention_runs_as_one_fused_pass(hip):
     np.testing.assert_allclose(got, _np_decode_attention(q, k, v, 2), rtol=1e-4, atol=1e-5)
 
 
+def test_norms_run_in_the_products_behind_them(hip):
+    """The dense part of a decoder layer at decode time (hidden 2048, 4 rows): four skinny-product launches — o
+    projection + residual add, gate / up / SiLU with the first norm in its loads, down projection + residual add,
+    q / k / v with the second norm in their loads — and no launch for the norms or the adds.  With hidden 512
+    the products' kernels do not take the norms, which then run on their own: same values either way."""
+    from catgrad_amd import _abi as A
+    from cases import by_name
+
+    classes = (A.K_GEMM_SKINNY, A.K_ELEMENTWISE, A.K_REDUCE)
+    for name, fused in (("decoder_block_B4_H2048_F4096", True), ("decoder_block_B4_H512_F4096", False)):
+        c = by_name(name)
+        hip.sync()
+        for cls in classes:
+            hip.profile_enable(cls, 1)
+            hip.profile_read(cls, True)
+        got = c.run(hip)
+        counts = tuple(hip.profile_read(cls, True)[0] for cls in classes)
+        for cls in classes:
+            hip.profile_enable(cls, 0)
+        if fused:
+            assert counts == (4, 0, 0), (name, counts)
+        else:
+            assert counts[0] == 4 and counts[1] + counts[2] >= 2, (name, counts)
+        for g, e in zip(got, c.expect()):
+            np.testing.assert_allclose(g, e, rtol=1e-3, atol=4e-3)
+
+
 def test_programs_absorbed_by_decode_time_products(hip):
     """gate and up projection of a decode step plus the SiLU program between them and the next product:
     one skinny-product launch and no element-wise launch; a pair the kernel does not take (8 rows) runs as
