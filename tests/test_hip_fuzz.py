@@ -213,3 +213,56 @@ def test_random_attention_shapes_match_oracle(hip, oracle, seed):
     got, ref = run(hip), run(oracle)
     assert got.shape == ref.shape == (B, kvh * rep, S, hd)
     np.testing.assert_allclose(got, ref, rtol=1e-4, atol=2e-5, err_msg=f"seed {seed}: B={B} kvh={kvh} rep={rep} hd={hd} S={S} T={T}")
+
+
+@pytest.mark.parametrize("seed", range(12))
+def test_random_decoder_blocks_match_oracle(hip, oracle, seed):
+    """The dense part of a decoder layer at decode time (residual add in the store of the o / down product, RMS norm in
+    the loads of the products behind it, gated pair) with random row counts and widths, and with the results — norms and
+    raw products included or not — read back in a random order, which decides what is still deferred when each
+    product runs.  1e-3 of the values' scale (they are of order one)."""
+    import cases
+
+    rng = np.random.default_rng(7000 + seed)
+    B = int(rng.integers(1, 6))
+    H = int(rng.choice([2048, 2048, 4096, 1024]))
+    F = int(rng.choice([4096, 6144, 8192]))
+    kv = int(rng.choice([256, 512, 2048]))
+    sc = np.float32(1.0 / np.sqrt(H))
+    r = lambda *s: rng.standard_normal(s).astype(np.float32)  # noqa: E731
+    x0, a0 = r(B, 1, H), r(B, 1, H)
+    wo, wg, wu, wd = r(H, H) * sc, r(F, H) * sc, r(F, H) * sc, r(H, F) * np.float32(1.0 / np.sqrt(F))
+    wq, wk, wv = r(H, H) * sc, r(kv, H) * sc, r(kv, H) * sc
+    g1, g2 = 1 + 0.1 * r(H), 1 + 0.1 * r(H)
+    wanted = ["q", "k", "v", "h1", "h2"] + [n for n in ("n1", "n2", "g", "u", "act") if rng.random() < 0.35]
+    order = [wanted[i] for i in rng.permutation(len(wanted))]
+    two_norm_uses = rng.random() < 0.5      # the second norm also feeds an element-wise op
+
+    def run(be):
+        shp, fs = (B, 1, H), (B, 1, F)
+        L, C = cases._linear, cases._const
+        t = {}
+        t["h1"] = be.add(be.from_numpy(x0).move(), L(be, be.from_numpy(a0), be.from_numpy(wo)).move())
+        t["n1"] = cases._rmsnorm_ops(be, t["h1"], be.from_numpy(g1), H, shp)
+        t["g"], t["u"] = L(be, t["n1"], be.from_numpy(wg)), L(be, t["n1"], be.from_numpy(wu))
+        e = be.exp(be.neg(t["g"]).move())
+        sg = be.div(C(be, 1.0, fs).move(), be.add(C(be, 1.0, fs).move(), e.move()).move())
+        t["act"] = be.mul(be.mul(t["g"], sg.move()).move(), t["u"])
+        t["h2"] = be.add(t["h1"], L(be, t["act"], be.from_numpy(wd)).move())
+        t["n2"] = cases._rmsnorm_ops(be, t["h2"], be.from_numpy(g2), H, shp)
+        t["q"], t["k"], t["v"] = (L(be, t["n2"], be.from_numpy(w)) for w in (wq, wk, wv))
+        extra = be.to_numpy(be.add(t["n2"], t["n2"])) if two_norm_uses else None
+        for name in list(t):
+            if name not in order:
+                del t[name]
+        outs = {name: be.to_numpy(t[name]) for name in order}
+        return outs, extra
+
+    got, gx = run(hip)
+    ref, rx = run(oracle)
+    for name in order:
+        assert got[name].shape == ref[name].shape
+        err = float(np.abs(got[name].astype(np.float64) - ref[name]).max())
+        assert err <= 1e-3 * max(4.0, float(np.abs(ref[name]).max())), f"seed {seed} B={B} H={H} F={F} kv={kv} {name} order={order}: {err}"
+    if two_norm_uses:
+        np.testing.assert_allclose(gx, rx, rtol=1e-4, atol=1e-4)
