@@ -124,7 +124,7 @@ def main():
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-micro", action="store_true")
-    ap.add_argument("--cpu-sample", type=int, nargs=3, default=[1, 8, 1], metavar=("BATCH", "PREFILL", "DECODE"))
+    ap.add_argument("--cpu-sample", type=int, nargs=3, default=[1, 4, 1], metavar=("BATCH", "PREFILL", "DECODE"))
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a strided copy of known size (268435456 B read + 268435456 B written per launch), "
                          "the yardstick for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE")
