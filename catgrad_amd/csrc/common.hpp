@@ -428,7 +428,7 @@ struct MmFold {
 int fold_matmul(const cg_tensor *x, const cg_tensor *y, MmFold *f);
 // Several skinny products x . ys[i] -> outs[i] (n of them, the same x) in one launch; kDeclined (declared
 // below) when the shapes do not allow it.
-// nf != null: x is the residual stream and the kernel applies the RMS norm to it on load (needs M in 2..4 and K a
+// nf != null: x is the residual stream and the kernel applies the RMS norm to it on load (needs M <= 4 and K a
 // multiple of 2048; kDeclined otherwise, before anything is launched).
 int launch_matmul_gated(cg_backend *be, const cg_tensor *x, const cg_tensor *yg, const cg_tensor *yu, uint32_t one,
                         cg_tensor *out, const NormFuse *nf = nullptr);
