@@ -508,7 +508,9 @@ template <int MM> __global__ __launch_bounds__(kThreads) void skinny_kt_wide_res
 // columns per workgroup (one activation load per lane and trip instead of M) when its 2048-wide chunks of k are full.
 // With a single row it is 0.7 us behind the one-column-per-wave kernel at K = 2048 and level with it at K = 8192;
 // it is used all the same, because its residual store and its norm-applying loads save two launches per layer.
-static inline bool xreg_narrow(uint32_t M, uint32_t K) { return M >= 1 && M <= 4 && K % 2048 == 0; }
+// Chunks of 2048 values of k when K is a multiple of that, of 1024 when of that (hidden sizes like 1024 or 3072).
+static inline int xreg_trips(uint32_t K) { return K % 2048 == 0 ? 8 : K % 1024 == 0 ? 4 : 0; }
+static inline bool xreg_narrow(uint32_t M, uint32_t K) { return M >= 1 && M <= 4 && xreg_trips(K) != 0; }
 constexpr int kMaxGroup = 4;
 struct MmGroup {
     MmArgs p[kMaxGroup];
@@ -546,7 +548,7 @@ __device__ __forceinline__ uint32_t norm_divisor(const NormFuse &nf, float sum) 
     const uint32_t mean = apply<kDiv, true>(asu(sum), nf.n_bits, 0, nullptr);
     return apply<kPow, true>(apply<kAdd, true>(mean, nf.eps_bits, 0, nullptr), nf.exp_bits, 0, nullptr);
 }
-template <int MM, int CG, bool GATED = false, bool RESIDUAL = false, bool NORM = false>
+template <int MM, int CG, bool GATED = false, bool RESIDUAL = false, bool NORM = false, int TRIPS = 8>
 __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const uint32_t block_x, const uint32_t block_y,
                                                          const uint32_t *second = nullptr, const uint32_t one = 0,
                                                          const MmResidual *res = nullptr, const NormFuse *nf = nullptr) {
@@ -597,12 +599,13 @@ __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const 
             if (i < nf->blocks * 4) pv[u] = nf->partials[i];
         }
     }
-    // of every 2048 values of k a wave takes 512 in a row (8 trips of 64): 2 KiB of each weight row
-    const uint32_t kb = wave * 512 + b * 4;
-    for (uint32_t k0 = 0; k0 < a.K; k0 += 2048) {
-        float4v xr[G][8];
+    // of every chunk of TRIPS * 256 values of k (2048 or 1024) a wave takes a quarter in a row (TRIPS trips of 64)
+    static_assert(TRIPS == 8 || TRIPS == 4, "chunks of 2048 or 1024");
+    const uint32_t kb = wave * (TRIPS * 64) + b * 4;
+    for (uint32_t k0 = 0; k0 < a.K; k0 += TRIPS * 256) {
+        float4v xr[G][TRIPS];
 #pragma unroll
-        for (int t = 0; t < 8; t++) {
+        for (int t = 0; t < TRIPS; t++) {
             const uint32_t k = k0 + kb + 64 * t;
 #pragma unroll
             for (int g = 0; g < G; g++) {
@@ -610,10 +613,10 @@ __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const 
                 if (k < a.K) xr[g][t] = *reinterpret_cast<const float4v *>(xrow[g] + k);
             }
         }
-        float4v gm[NORM ? 8 : 1]; // asked for with the activations, multiplied in once the first weights are on their way
+        float4v gm[NORM ? TRIPS : 1]; // asked for with the activations, multiplied in once the first weights are on their way
         if constexpr (NORM) {
 #pragma unroll
-            for (int t = 0; t < 8; t++) {
+            for (int t = 0; t < TRIPS; t++) {
                 const uint32_t k = k0 + kb + 64 * t;
                 gm[t] = (float4v){0.f, 0.f, 0.f, 0.f};
                 if (k < a.K) gm[t] = *reinterpret_cast<const float4v *>(nf->gamma + k);
@@ -621,9 +624,9 @@ __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const 
         }
 #pragma unroll
         for (int c = 0; c < CG; c++) {
-            float4v w[8];
+            float4v w[TRIPS];
 #pragma unroll
-            for (int t = 0; t < 8; t++) {
+            for (int t = 0; t < TRIPS; t++) {
                 const uint32_t k = k0 + kb + 64 * t;
                 w[t] = (float4v){0.f, 0.f, 0.f, 0.f};
                 if (k < a.K) w[t] = *reinterpret_cast<const float4v *>(wrow[c] + k);
@@ -631,7 +634,7 @@ __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const 
             if constexpr (NORM) {
                 if (c == 0) {
 #pragma unroll
-                    for (int t = 0; t < 8; t++)
+                    for (int t = 0; t < TRIPS; t++)
 #pragma unroll
                         for (int g = 0; g < G; g++)
 #pragma unroll
@@ -639,7 +642,7 @@ __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const 
                 }
             }
 #pragma unroll
-            for (int t = 0; t < 8; t++)
+            for (int t = 0; t < TRIPS; t++)
 #pragma unroll
                 for (int g = 0; g < G; g++) {
                     acc[c][g] = __builtin_amdgcn_mfma_f32_4x4x1f32(xr[g][t][0], w[t][0], acc[c][g], 0, 0, 0);
@@ -712,32 +715,33 @@ __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const 
     }
 }
 
-template <int MM, int CG> __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_kernel(const MmArgs a) {
-    skinny_kt_mfma_xreg_body<MM, CG>(a, blockIdx.x, blockIdx.y);
+template <int MM, int CG, int TRIPS = 8> __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_kernel(const MmArgs a) {
+    skinny_kt_mfma_xreg_body<MM, CG, false, false, false, TRIPS>(a, blockIdx.x, blockIdx.y);
 }
-template <int MM>
+template <int MM, int TRIPS = 8>
 __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_gated_kernel(const MmArgs a, const uint32_t *second, uint32_t one) {
-    skinny_kt_mfma_xreg_body<MM, 2, true>(a, blockIdx.x, blockIdx.y, second, one);
+    skinny_kt_mfma_xreg_body<MM, 2, true, false, false, TRIPS>(a, blockIdx.x, blockIdx.y, second, one);
 }
-template <int MM>
+template <int MM, int TRIPS = 8>
 __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_residual_kernel(const MmArgs a, const MmResidual r) {
-    skinny_kt_mfma_xreg_body<MM, 1, false, true>(a, blockIdx.x, blockIdx.y, nullptr, 0, &r);
+    skinny_kt_mfma_xreg_body<MM, 1, false, true, false, TRIPS>(a, blockIdx.x, blockIdx.y, nullptr, 0, &r);
 }
 // the same with the RMS norm of the left operand applied on load
+template <int TRIPS = 8>
 __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_gated_norm_kernel(const MmArgs a, const uint32_t *second, uint32_t one,
                                                                                   const NormFuse nf) {
-    skinny_kt_mfma_xreg_body<4, 2, true, false, true>(a, blockIdx.x, blockIdx.y, second, one, nullptr, &nf);
+    skinny_kt_mfma_xreg_body<4, 2, true, false, true, TRIPS>(a, blockIdx.x, blockIdx.y, second, one, nullptr, &nf);
 }
-template <int MM, int CG> __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_group_kernel(const MmGroup g) {
+template <int MM, int CG, int TRIPS = 8> __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_group_kernel(const MmGroup g) {
     uint32_t bx;
     const uint32_t p = group_problem(g, bx);
-    skinny_kt_mfma_xreg_body<MM, CG>(g.p[p], bx, 0);
+    skinny_kt_mfma_xreg_body<MM, CG, false, false, false, TRIPS>(g.p[p], bx, 0);
 }
-
+template <int TRIPS = 8>
 __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_group_norm_kernel(const MmGroup g, const NormFuse nf) {
     uint32_t bx;
     const uint32_t p = group_problem(g, bx);
-    skinny_kt_mfma_xreg_body<4, 1, false, false, true>(g.p[p], bx, 0, nullptr, 0, nullptr, &nf);
+    skinny_kt_mfma_xreg_body<4, 1, false, false, true, TRIPS>(g.p[p], bx, 0, nullptr, 0, nullptr, &nf);
 }
 
 // Vectorised skinny kernel for short K (K <= 4*LPC, e.g. q.K^T of a decode step with
@@ -1010,11 +1014,15 @@ int launch_matmul_group(cg_backend *be, const cg_tensor *x, const cg_tensor *con
     g.n = (uint32_t)n;
     ProfScope prof(be, CG_K_GEMM_SKINNY, bytes);
     if (xreg)
-        hipLaunchKernelGGL((skinny_kt_mfma_xreg_group_kernel<4, 2>), dim3(blocks), dim3(kThreads), 0, be->stream, g);
+        hipLaunchKernelGGL((skinny_kt_mfma_xreg_group_kernel<4, 2, 8>), dim3(blocks), dim3(kThreads), 0, be->stream, g);
+    else if (nf && xreg_trips(g.p[0].K) == 8)
+        hipLaunchKernelGGL(skinny_kt_mfma_xreg_group_norm_kernel<8>, dim3(blocks), dim3(kThreads), 0, be->stream, g, *nf);
     else if (nf)
-        hipLaunchKernelGGL(skinny_kt_mfma_xreg_group_norm_kernel, dim3(blocks), dim3(kThreads), 0, be->stream, g, *nf);
+        hipLaunchKernelGGL(skinny_kt_mfma_xreg_group_norm_kernel<4>, dim3(blocks), dim3(kThreads), 0, be->stream, g, *nf);
+    else if (xreg1 && xreg_trips(g.p[0].K) == 8)
+        hipLaunchKernelGGL((skinny_kt_mfma_xreg_group_kernel<4, 1, 8>), dim3(blocks), dim3(kThreads), 0, be->stream, g);
     else if (xreg1)
-        hipLaunchKernelGGL((skinny_kt_mfma_xreg_group_kernel<4, 1>), dim3(blocks), dim3(kThreads), 0, be->stream, g);
+        hipLaunchKernelGGL((skinny_kt_mfma_xreg_group_kernel<4, 1, 4>), dim3(blocks), dim3(kThreads), 0, be->stream, g);
     else if (g.p[0].M <= 1)
         hipLaunchKernelGGL((skinny_kt_wide_group_kernel<1>), dim3(blocks), dim3(kThreads), 0, be->stream, g);
     else if (g.p[0].M <= 4)
@@ -1038,15 +1046,21 @@ int launch_matmul_gated(cg_backend *be, const cg_tensor *x, const cg_tensor *yg,
     if (!rc) rc = make_mm_args(x, yu, out->buf->ptr, &au, &fu);
     if (rc) return rc;
     const bool vec = ag.a_vec && ag.b_vec && au.b_vec && ag.a_sk == 1 && ag.K % 4 == 0;
-    if (fg.batch != 1 || fu.batch != 1 || ag.M > 4 || ag.b_sk != 1 || au.b_sk != 1 || !vec || ag.K <= 256 || ag.N < 4096 ||
+    if (fg.batch != 1 || fu.batch != 1 || ag.M > 4 || ag.b_sk != 1 || au.b_sk != 1 || !vec || ag.K <= 256 || ag.N < 2048 ||
         au.N != ag.N || au.K != ag.K || au.M != ag.M || au.b_sn != ag.b_sn)
         return kDeclined;
-    if (nf && ag.K % 2048 != 0) return kDeclined;
+    if (nf && xreg_trips(ag.K) == 0) return kDeclined;
+    const bool short_chunks = xreg_trips(ag.K) == 4; // K a multiple of 1024 but not of 2048
     ProfScope prof(be, CG_K_GEMM_SKINNY, distinct_bytes(x) + distinct_bytes(yg) + distinct_bytes(yu) + distinct_bytes(out));
-    if (nf)
-        hipLaunchKernelGGL(skinny_kt_mfma_xreg_gated_norm_kernel, dim3((ag.N + 3) / 4), dim3(kThreads), 0, be->stream, ag, au.B, one, *nf);
+    const dim3 ggrid((ag.N + 3) / 4);
+    if (nf && short_chunks)
+        hipLaunchKernelGGL(skinny_kt_mfma_xreg_gated_norm_kernel<4>, ggrid, dim3(kThreads), 0, be->stream, ag, au.B, one, *nf);
+    else if (nf)
+        hipLaunchKernelGGL(skinny_kt_mfma_xreg_gated_norm_kernel<8>, ggrid, dim3(kThreads), 0, be->stream, ag, au.B, one, *nf);
+    else if (short_chunks)
+        hipLaunchKernelGGL((skinny_kt_mfma_xreg_gated_kernel<4, 4>), ggrid, dim3(kThreads), 0, be->stream, ag, au.B, one);
     else
-        hipLaunchKernelGGL((skinny_kt_mfma_xreg_gated_kernel<4>), dim3((ag.N + 3) / 4), dim3(kThreads), 0, be->stream, ag, au.B, one);
+        hipLaunchKernelGGL((skinny_kt_mfma_xreg_gated_kernel<4, 8>), ggrid, dim3(kThreads), 0, be->stream, ag, au.B, one);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? CG_OK : hip_fail(e, "gated matmul launch");
 }
@@ -1063,7 +1077,7 @@ int launch_matmul_residual(cg_backend *be, const cg_tensor *x, const cg_tensor *
     int rc = make_mm_args(x, y, out->buf->ptr, &a, &f);
     if (rc) return rc;
     const bool vec = a.a_vec && a.b_vec && a.a_sk == 1 && a.K % 4 == 0;
-    if (f.batch != 1 || a.M > 8 || a.b_sk != 1 || !vec || a.K <= 256 || a.N < 2048 || a.N >= 8192) return kDeclined;
+    if (f.batch != 1 || a.M > 8 || a.b_sk != 1 || !vec || a.K <= 256 || a.N < 1024 || a.N >= 8192) return kDeclined;
     MmResidual r;
     for (int t = 0; t < 4; t++) r.term[t] = t == slot || t >= nterms ? nullptr : terms[t];
     r.slot = (uint32_t)slot;
@@ -1083,9 +1097,12 @@ int launch_matmul_residual(cg_backend *be, const cg_tensor *x, const cg_tensor *
     }
     ProfScope prof(be, CG_K_GEMM_SKINNY, distinct_bytes(x) + distinct_bytes(y) + 4.0 * distinct_bytes(out));
     dim3 grid((uint32_t)((a.N + 3) / 4));
-    if (xreg_narrow(a.M, a.K))
-        hipLaunchKernelGGL((skinny_kt_mfma_xreg_residual_kernel<4>), grid, dim3(kThreads), 0, be->stream, a, r);
-    else if (a.M <= 1)
+    if (xreg_narrow(a.M, a.K)) {
+        if (xreg_trips(a.K) == 8)
+            hipLaunchKernelGGL((skinny_kt_mfma_xreg_residual_kernel<4, 8>), grid, dim3(kThreads), 0, be->stream, a, r);
+        else
+            hipLaunchKernelGGL((skinny_kt_mfma_xreg_residual_kernel<4, 4>), grid, dim3(kThreads), 0, be->stream, a, r);
+    } else if (a.M <= 1)
         hipLaunchKernelGGL((skinny_kt_wide_residual_kernel<1>), grid, dim3(kThreads), 0, be->stream, a, r);
     else if (a.M <= 4)
         hipLaunchKernelGGL((skinny_kt_wide_residual_kernel<4>), grid, dim3(kThreads), 0, be->stream, a, r);
@@ -1151,10 +1168,16 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
 #undef CG_CALL
             } else if (cols >= 4096 && M <= 4) { // the wider projections of a decode step: activations are fetched once per 8 columns
                 dim3 grid((uint32_t)((N + 7) / 8), (uint32_t)batch);
-                hipLaunchKernelGGL((skinny_kt_mfma_xreg_kernel<4, 2>), grid, dim3(kThreads), 0, s, a);
+                if (xreg_trips((uint32_t)K) == 4)
+                    hipLaunchKernelGGL((skinny_kt_mfma_xreg_kernel<4, 2, 4>), grid, dim3(kThreads), 0, s, a);
+                else
+                    hipLaunchKernelGGL((skinny_kt_mfma_xreg_kernel<4, 2, 8>), grid, dim3(kThreads), 0, s, a);
             } else if (cols >= 2048 && xreg_narrow((uint32_t)M, (uint32_t)K)) {
                 dim3 grid((uint32_t)((N + 3) / 4), (uint32_t)batch);
-                hipLaunchKernelGGL((skinny_kt_mfma_xreg_kernel<4, 1>), grid, dim3(kThreads), 0, s, a);
+                if (xreg_trips((uint32_t)K) == 4)
+                    hipLaunchKernelGGL((skinny_kt_mfma_xreg_kernel<4, 1, 4>), grid, dim3(kThreads), 0, s, a);
+                else
+                    hipLaunchKernelGGL((skinny_kt_mfma_xreg_kernel<4, 1, 8>), grid, dim3(kThreads), 0, s, a);
             } else if (cols >= 2048) {
                 dim3 grid((uint32_t)((N + 3) / 4), (uint32_t)batch);
 #define CG_CALL(MMV) hipLaunchKernelGGL((skinny_kt_wide_kernel<MMV, 1, false>), grid, dim3(kThreads), 0, s, a);

@@ -142,7 +142,7 @@ Pending::~Pending() {
 
 // Is x (still) the deferred program  h / pow(sum(h * h) / n + eps, e) * gamma  over the rows of a residual stream h
 // [1..4 rows, K] whose kernel left the partial sums of squares (Buffer::side)?  Then a decode-time product can apply
-// the norm while it loads h (K a multiple of 2048) and the norm needs no launch.  Fills nf and the stand-in tensor
+// the norm while it loads h (K a multiple of 1024) and the norm needs no launch.  Fills nf and the stand-in tensor
 // h (a borrowed view of the leaf's buffer: set h->buf to null before it goes out of scope).
 static bool norm_fuse_of(const cg_tensor *x, NormFuse *nf, cg_tensor *h) {
     static const uint8_t code[7][4] = {{kMul, 0, 0, 0},   {kRowSum, 8, 8, 8}, {kDiv, 9, 1, 9},  {kAdd, 10, 2, 10},
@@ -154,7 +154,7 @@ static bool norm_fuse_of(const cg_tensor *x, NormFuse *nf, cg_tensor *h) {
         if (p->ins[i].op != code[i][0] || p->ins[i].a != code[i][1] || p->ins[i].b != code[i][2] || p->ins[i].c != code[i][3]) return false;
     const int r = x->rank;
     const int64_t K = x->dims[r - 1], rows = K > 0 ? numel(x) / K : 0;
-    if (K <= 0 || K % 2048 != 0 || rows < 1 || rows > 4 || p->rowlen != K) return false;
+    if (K <= 0 || K % 1024 != 0 || rows < 1 || rows > 4 || p->rowlen != K) return false;
     const LeafView &lh = p->leaf[0], &lg = p->leaf[4];
     if (lh.uniform || lh.pw || lh.lazy || !lh.buf || !lh.buf->side || lh.offset != 0 || (int64_t)lh.buf->side_blocks * 4 != K) return false;
     if (!p->leaf[1].uniform || !p->leaf[2].uniform || !p->leaf[3].uniform) return false;
@@ -199,7 +199,7 @@ static bool residual_sum_open(const cg_tensor *x) {
         if (lv.lazy && !lv.lazy->result) {
             const LazyMm *m = lv.lazy;
             const int64_t N = m->rank > 0 ? m->dims[m->rank - 1] : 0;
-            if (!m->groupable || m->rc.load() != 1 || m->rank != x->rank || N < 2048 || N >= 8192) return false;
+            if (!m->groupable || m->rc.load() != 1 || m->rank != x->rank || N < 1024 || N >= 8192) return false;
             open++;
         } else if (!lv.lazy && !lv.buf) {
             return false;

@@ -1018,7 +1018,8 @@ def _linear(be, x, w):
 
 
 for _B, _K, _Ns in ((4, 512, (512, 128, 128)), (1, 1024, (64, 2048)), (8, 388, (300, 8200)), (4, 512, (8192, 8200)),
-                    (2, 2304, (8192, 8192, 96, 100, 104)), (4, 2048, (2048, 512, 516)), (3, 4096, (300, 2052)), (2, 2048, (2500,))):
+                    (2, 2304, (8192, 8192, 96, 100, 104)), (4, 2048, (2048, 512, 516)), (3, 4096, (300, 2052)), (2, 2048, (2500,)),
+                    (1, 1024, (2048, 1024, 1024)), (4, 3072, (300, 2052))):
     @case(f"linear_group_B{_B}_K{_K}_N{'_'.join(map(str, _Ns))}", "red",
           (lambda B=_B, K=_K, Ns=_Ns: [np.abs(f32(500 + K, (B, 1, K)).astype(np.float64)) @
                                          np.abs(f32(501 + K + i, (n, K)).astype(np.float64)).T
@@ -1062,7 +1063,7 @@ def _():
 
 
 # ---- SiLU-gated pair of decode-time linear layers (gate / up of an MLP block) ---------------------------------------
-for _B, _K, _N in ((4, 512, 4096), (1, 2048, 8192), (3, 388, 4100), (8, 512, 4096), (4, 512, 512)):
+for _B, _K, _N in ((4, 512, 4096), (1, 2048, 8192), (3, 388, 4100), (8, 512, 4096), (4, 512, 512), (1, 1024, 4096), (4, 3072, 4100)):
     @case(f"linear_gated_B{_B}_K{_K}_N{_N}", "red")
     def _(B=_B, K=_K, Nn=_N):
         """`silu(x.Wg) * (x.Wu)` as the MLP of the decoder graphs issues it (llama.rs:262-283 with
@@ -1091,7 +1092,7 @@ for _B, _K, _N in ((4, 512, 4096), (1, 2048, 8192), (3, 388, 4100), (8, 512, 409
 
 
 # ---- residual adds around a decode-time linear layer (the o / down projection of a decoder layer) -------------------
-for _B, _K, _N in ((4, 512, 2048), (8, 260, 2052), (1, 1024, 4096), (4, 512, 512), (4, 2048, 2048), (3, 4096, 2052), (2, 2048, 4100)):
+for _B, _K, _N in ((4, 512, 2048), (8, 260, 2052), (1, 1024, 4096), (4, 512, 512), (4, 2048, 2048), (3, 4096, 2052), (2, 2048, 4100), (1, 3072, 2048), (4, 1024, 2052)):
     @case(f"linear_residual_B{_B}_K{_K}_N{_N}", "red")
     def _(B=_B, K=_K, Nn=_N):
         """Sums of three dense terms and a lazy product in the two association orders and every operand
@@ -1270,7 +1271,8 @@ def _rmsnorm_ops(be, h, gamma, n, shp):
     return be.mul(be.div(h, be.broadcast(rms.move(), shp).move()).move(), be.broadcast(gamma.move(), shp).move())
 
 
-for _B, _H, _F, _read_norms in ((4, 2048, 4096, False), (2, 2048, 4096, True), (3, 4096, 8192, False), (4, 512, 4096, False), (1, 2048, 4096, False)):
+for _B, _H, _F, _read_norms in ((4, 2048, 4096, False), (2, 2048, 4096, True), (3, 4096, 8192, False), (4, 512, 4096, False), (1, 2048, 4096, False),
+                                 (1, 1024, 3072, False), (4, 3072, 4096, False)):
     @case(f"decoder_block_B{_B}_H{_H}_F{_F}{'_norms_read' if _read_norms else ''}", "red",
           (lambda n=5 + 2 * _read_norms: [np.float64(4.0)] * n))   # every output is of order one: 1e-3 of 4
     def _(B=_B, H=_H, F=_F, read_norms=_read_norms):

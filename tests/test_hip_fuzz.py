@@ -225,7 +225,7 @@ def test_random_decoder_blocks_match_oracle(hip, oracle, seed):
 
     rng = np.random.default_rng(7000 + seed)
     B = int(rng.integers(1, 6))
-    H = int(rng.choice([2048, 2048, 4096, 1024]))
+    H = int(rng.choice([2048, 2048, 4096, 1024, 3072, 512]))
     F = int(rng.choice([4096, 6144, 8192]))
     kv = int(rng.choice([256, 512, 2048]))
     sc = np.float32(1.0 / np.sqrt(H))

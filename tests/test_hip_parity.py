@@ -159,7 +159,7 @@ def test_norms_run_in_the_products_behind_them(hip):
     from cases import by_name
 
     classes = (A.K_GEMM_SKINNY, A.K_ELEMENTWISE, A.K_REDUCE)
-    for name, fused in (("decoder_block_B4_H2048_F4096", True), ("decoder_block_B4_H512_F4096", False)):
+    for name, fused in (("decoder_block_B4_H2048_F4096", True), ("decoder_block_B1_H1024_F3072", True), ("decoder_block_B4_H512_F4096", False)):
         c = by_name(name)
         hip.sync()
         for cls in classes:
