@@ -112,6 +112,7 @@ constexpr size_t kStageBytes = 16u << 20; // size of each pinned host-to-device 
 // in place at that frontier.
 struct RowStore {
     int64_t R = 0, C = 0, nblocks = 0;
+    int64_t src_C = 0; // block capacity of the buffer whose blocks migrate here: block ids are numbered in its units
     std::vector<int64_t> fill;
 };
 
@@ -125,6 +126,7 @@ struct Buffer {
     const uint64_t id = next_buffer_id(); // never reused, unlike the address: what keys of kept results name
     void *ptr = nullptr;
     size_t cls = 0;
+    int64_t elems = 0;           // elements in use from the start of the buffer (grows with in-place appends); <= cls / 4
     cg_backend *be = nullptr;
     RowStore *rs = nullptr;      // owned
     bool constant = false;       // the contents depend on constants only (iota, programs over such buffers)
@@ -438,9 +440,10 @@ int launch_fused_group(cg_backend *be, const cg_tensor *const *outs, const Pendi
 // Writes that were put off so that they can share a launch (see DeferredWrite); every function
 // that launches a kernel or copies device memory calls this first.
 int flush_deferred(cg_backend *be);
-// nterms: 2 (out = t0 + t1) or 4.  On success out->buf may have received the partial sums of squares (Buffer::side).
+// nterms: 2 (out = t0 + t1) or 4.  out is a contiguous view (any offset).  keep_sums: out is the whole of its buffer, which
+// may then receive the partial sums of squares of the stored rows (Buffer::side).
 int launch_matmul_residual(cg_backend *be, const cg_tensor *x, const cg_tensor *y, const uint32_t *const *terms, int nterms,
-                           int slot, int order, cg_tensor *out);
+                           int slot, int order, cg_tensor *out, bool keep_sums);
 int launch_matmul_group(cg_backend *be, const cg_tensor *x, const cg_tensor *const *ys, cg_tensor *const *outs, int n,
                         const NormFuse *nf = nullptr);
 

@@ -1042,8 +1042,9 @@ int launch_matmul_gated(cg_backend *be, const cg_tensor *x, const cg_tensor *yg,
     if (x->dt != CG_F32) return kDeclined;
     MmArgs ag, au;
     MmFold fg, fu;
-    int rc = make_mm_args(x, yg, out->buf->ptr, &ag, &fg);
-    if (!rc) rc = make_mm_args(x, yu, out->buf->ptr, &au, &fu);
+    uint32_t *const c = static_cast<uint32_t *>(out->buf->ptr) + out->offset; // out: a contiguous view, not always at element 0
+    int rc = make_mm_args(x, yg, c, &ag, &fg);
+    if (!rc) rc = make_mm_args(x, yu, c, &au, &fu);
     if (rc) return rc;
     const bool vec = ag.a_vec && ag.b_vec && au.b_vec && ag.a_sk == 1 && ag.K % 4 == 0;
     if (fg.batch != 1 || fu.batch != 1 || ag.M > 4 || ag.b_sk != 1 || au.b_sk != 1 || !vec || ag.K <= 256 || ag.N < 2048 ||
@@ -1069,12 +1070,12 @@ int launch_matmul_gated(cg_backend *be, const cg_tensor *x, const cg_tensor *yg,
 // (device pointers); `order` as in MmResidual.  Declines unless the one-column-per-wave kernel
 // is what the product would run on anyway.
 int launch_matmul_residual(cg_backend *be, const cg_tensor *x, const cg_tensor *y, const uint32_t *const *terms, int nterms,
-                           int slot, int order, cg_tensor *out) {
+                           int slot, int order, cg_tensor *out, bool keep_sums) {
     if (int frc = flush_deferred(be)) return frc;
     if (x->dt != CG_F32) return kDeclined;
     MmArgs a;
     MmFold f;
-    int rc = make_mm_args(x, y, out->buf->ptr, &a, &f);
+    int rc = make_mm_args(x, y, static_cast<uint32_t *>(out->buf->ptr) + out->offset, &a, &f);
     if (rc) return rc;
     const bool vec = a.a_vec && a.b_vec && a.a_sk == 1 && a.K % 4 == 0;
     if (f.batch != 1 || a.M > 8 || a.b_sk != 1 || !vec || a.K <= 256 || a.N < 1024 || a.N >= 8192) return kDeclined;
@@ -1085,7 +1086,7 @@ int launch_matmul_residual(cg_backend *be, const cg_tensor *x, const cg_tensor *
     r.nterms = (uint32_t)nterms;
     r.partials = nullptr;
     const uint32_t blocks = (uint32_t)((a.N + 3) / 4);
-    if (xreg_narrow(a.M, a.K) && !out->buf->side) {
+    if (keep_sums && out->offset == 0 && xreg_narrow(a.M, a.K) && !out->buf->side) {
         // the stored rows' sums of squares per workgroup, for an RMS norm that may follow (Buffer::side)
         Buffer *ob = out->buf;
         if (be->pool.alloc((size_t)blocks * 4 * sizeof(float), &ob->side, &ob->side_cls) == CG_OK) {

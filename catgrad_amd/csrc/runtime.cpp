@@ -318,6 +318,7 @@ int new_dense(cg_backend *be, cg_dtype dt, const int64_t *dims, int rank, cg_ten
             delete t;
             return rc;
         }
+        b->elems = n;
         t->buf = b;
     }
     *out = t;
@@ -641,7 +642,8 @@ static int wait_and_check(cg_backend *be) {
     return CG_OK;
 }
 
-static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p);
+// fresh: dst is the whole of a buffer allocated for this very result (nothing else lives in it).
+static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p, bool fresh = false);
 
 // Row-major copy of a view (the materialising half of reshape / to_vec).
 static int materialize(cg_backend *be, const cg_tensor *x, cg_tensor **out) {
@@ -684,7 +686,7 @@ static int materialize(cg_backend *be, const cg_tensor *x, cg_tensor **out) {
         }
     } else if (numel(x) > 0) {
         const cg_tensor *ins[1] = {x};
-        rc = x->pend ? run_pending(be, o, *x->pend) : launch_elementwise(be, kCopy, x->dt, o, ins, 1);
+        rc = x->pend ? run_pending(be, o, *x->pend, true) : launch_elementwise(be, kCopy, x->dt, o, ins, 1);
         if (rc) {
             release(o);
             return rc;
@@ -822,7 +824,8 @@ static int try_gated_pair(cg_backend *be, const cg_tensor *dst, const Pending &p
 
 // A sum of four dense terms, one of them a product nobody has needed yet (the residual stream after the
 // o or down projection): the adds run in the product's store.
-static int try_residual_store(cg_backend *be, const cg_tensor *dst, const Pending &p) {
+// fresh: dst is a whole new buffer, so the row sums of squares of what is stored may be kept with it.
+static int try_residual_store(cg_backend *be, const cg_tensor *dst, const Pending &p, bool fresh) {
     static const uint8_t orders[2][3][2] = {{{1, 2}, {0, 8}, {9, 3}}, {{1, 2}, {8, 3}, {0, 9}}};
     if (p.nred != 0 || !is_contiguous(dst) || dst->dt != CG_F32) return kDeclined;
     int order = -1;
@@ -868,7 +871,7 @@ static int try_residual_store(cg_backend *be, const cg_tensor *dst, const Pendin
         int xrc = ensure_concrete(m->x);
         if (xrc) return xrc;
     }
-    int rc = launch_matmul_residual(be, m->x, m->y, terms, nterms, slot, order, const_cast<cg_tensor *>(dst));
+    int rc = launch_matmul_residual(be, m->x, m->y, terms, nterms, slot, order, const_cast<cg_tensor *>(dst), fresh && dst->offset == 0);
     if (rc == CG_OK) {
         lazy_mm_close(m);
         be->programs_compiled++;
@@ -876,10 +879,10 @@ static int try_residual_store(cg_backend *be, const cg_tensor *dst, const Pendin
     return rc;
 }
 
-static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p) {
+static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p, bool fresh) {
     if (be->aot) {
         int grc = try_gated_pair(be, dst, p);
-        if (grc == kDeclined) grc = try_residual_store(be, dst, p);
+        if (grc == kDeclined) grc = try_residual_store(be, dst, p, fresh);
         if (grc != kDeclined) return grc;
     }
     {
@@ -1153,6 +1156,7 @@ static int ensure_concrete(cg_tensor *t) {
         delete b;
         return rc;
     }
+    b->elems = numel(t);
     cg_tensor dst;
     dst.be = be;
     dst.buf = b;
@@ -1166,7 +1170,7 @@ static int ensure_concrete(cg_tensor *t) {
         rc = defer_write(be, &dst, t->pend);
         if (!rc) rc = flush_deferred(be);
     } else {
-        rc = run_pending(be, &dst, *t->pend);
+        rc = run_pending(be, &dst, *t->pend, true);
     }
     dst.buf = nullptr;
     if (rc) {
@@ -1586,7 +1590,9 @@ static bool try_row_append(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim
     for (int i = 0; i < (int)dim; i++)
         if (x->dims[i] > 1 && x->strides[i] % (C * R)) return false;
     if (!rs && xd != C) return false; // a partial view of a plain buffer: its "slack" is someone's data
-    const int64_t src_blocks = (int64_t)(src->cls / 4) / (C * R);
+    // blocks of a plain buffer: what has been written of it, not the size class it was rounded up to
+    const int64_t src_elems = src->elems > 0 ? src->elems : (int64_t)(src->cls / 4);
+    const int64_t src_blocks = (src_elems + C * R - 1) / (C * R);
     // blocks touched, in row-major order of the outer index
     std::vector<int64_t> blocks((size_t)outer);
     {
@@ -1652,6 +1658,7 @@ static bool try_row_append(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim
             nbuf->rs = new RowStore;
             nbuf->rs->R = R;
             nbuf->rs->C = xd + yd + grow;
+            nbuf->rs->src_C = C;
             nbuf->rs->nblocks = nb;
             nbuf->rs->fill.assign((size_t)nb, 0);
             int rc = b->pool.alloc((size_t)(nb * nbuf->rs->C * R) * 4, &nbuf->ptr, &nbuf->cls);
@@ -1661,13 +1668,17 @@ static bool try_row_append(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim
                 *status = rc;
                 return true;
             }
+            nbuf->elems = nb * nbuf->rs->C * R;
             src->successor = nbuf;
         }
         dstbuf = src->successor;
         RowStore *ds = dstbuf->rs;
-        if (ds->R != R || ds->C < xd + yd) return false;
-        for (int64_t o = 0; o < outer; o++)
+        // the successor numbers its blocks as the view that created it saw this buffer: another blocking does not fit
+        if (ds->R != R || ds->src_C != C || ds->C < xd + yd) return false;
+        for (int64_t o = 0; o < outer; o++) {
+            if (blocks[(size_t)o] >= ds->nblocks) return false;
             if (ds->fill[(size_t)blocks[(size_t)o]] != 0) return false; // somebody already migrated these blocks
+        }
         dC = ds->C;
         *status = write_rows(dstbuf, dC, 0, x);
         if (!*status) *status = write_rows(dstbuf, dC, xd, y);
@@ -2887,6 +2898,12 @@ int cg_concat(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor *
         if (!rc) rc = y->pend ? run_pending(b, &tail, *y->pend) : launch_elementwise(b, kCopy, x->dt, &tail, ins, 1);
         tail.buf = nullptr;
         if (rc) return rc;
+        x->buf->elems = nx + ny;
+        if (x->buf->side) { // row sums kept for the rows this buffer held so far do not describe the grown tensor
+            b->pool.free(x->buf->side, x->buf->side_cls);
+            x->buf->side = nullptr;
+            x->buf->side_blocks = 0;
+        }
         x->dims[dim] = od[dim];
         set_row_major(x);
         retain(x);

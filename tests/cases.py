@@ -1124,6 +1124,84 @@ for _B, _K, _N in ((4, 512, 2048), (8, 260, 2052), (1, 1024, 4096), (4, 512, 512
         return run, expect
 
 
+# ---- products with a fused store whose destination is a part of a larger buffer --------------------------------------
+for _axis, _B, _K, _N in ((0, 2, 512, 2048), (1, 1, 1024, 2048), (0, 4, 2048, 2048), (1, 1, 512, 4096)):
+    @case(f"linear_fused_store_into_concat_dim{_axis}_B{_B}_K{_K}_N{_N}", "red",
+          (lambda: [None] * 6 + [np.float64(8.0)] * 2))   # positive data: 1e-3 of the value; the normed products: of 8
+    def _(axis=_axis, B=_B, K=_K, Nn=_N):
+        """`concat(prev, h + x.W)`, `concat(prev, t0 + (t1 + t2) + x.W)` and `concat(prev, silu(x.Wg) * x.Wu)` along the
+        outermost axis: the open product is computed straight into the second part of the result (a view with an
+        offset), both into a fresh buffer and appended in place to a stack this call holds alone; then an RMS norm over
+        rows of the stack feeds further products (row sums kept for a part must not be taken for the whole)."""
+        r_ = np.random.default_rng(580 + axis + Nn)
+        x = np.abs(r_.standard_normal((B, 1, K))).astype(np.float32)
+        w, wg, wu = (np.abs(r_.standard_normal((Nn, K))).astype(np.float32) for _ in range(3))
+        wg *= np.float32(8.0 / K)
+        wu *= np.float32(8.0 / K)
+        wg[::2] *= -1
+        ts = [np.abs(r_.standard_normal((B, 1, Nn))).astype(np.float32) for _ in range(3)]
+        pshape = (3, 1, Nn) if axis == 0 else (1, 3, Nn)
+        prev = np.abs(r_.standard_normal(pshape)).astype(np.float32)
+        gm = (1.0 + 0.1 * r_.standard_normal(Nn)).astype(np.float32)
+        w2 = r_.standard_normal((64, Nn)).astype(np.float32) * np.float32(1.0 / np.sqrt(Nn))
+
+        def run(be):
+            def two():
+                return be.add(be.from_numpy(ts[0]).move(), _linear(be, be.from_numpy(x), be.from_numpy(w)).move())
+
+            def four():
+                inner = be.add(be.from_numpy(ts[1]).move(), be.from_numpy(ts[2]).move())
+                return be.add(be.add(be.from_numpy(ts[0]).move(), inner.move()).move(),
+                              _linear(be, be.from_numpy(x), be.from_numpy(w)).move())
+
+            def gated():
+                tx = be.from_numpy(x)
+                g, u = _linear(be, tx, be.from_numpy(wg)), _linear(be, tx, be.from_numpy(wu))
+                del tx
+                sh = (B, 1, Nn)
+                e = be.exp(be.neg(g).move())
+                sg = be.div(_const(be, 1.0, sh).move(), be.add(_const(be, 1.0, sh).move(), e.move()).move())
+                return be.mul(be.mul(g.move(), sg.move()).move(), u.move())
+
+            outs = []
+            for make in (two, four, gated):
+                # into the second part of a fresh result
+                outs.append(be.concat(be.from_numpy(prev), make().move(), axis))
+                # appended in place: the stack is held by this call alone and has room behind it
+                stack = be.concat(be.from_numpy(prev[:1] if axis == 0 else prev[:, :1]),
+                                  be.from_numpy(prev[1:] if axis == 0 else prev[:, 1:]), axis)
+                outs.append(be.concat(stack.move(), make().move(), axis))
+            # an RMS norm over the rows of a stack whose last rows came from a fused store, then a product
+            for cat in (outs[0], outs[1]):
+                rows = int(np.prod(pshape[:2])) + B
+                h = be.reshape(cat, (1, rows, Nn)) if rows <= 4 else be.slice(be.reshape(cat, (1, rows, Nn)), 1, rows - 4, 4)
+                shp = (1, min(rows, 4), Nn)
+                n1 = _rmsnorm_ops(be, h, be.from_numpy(gm), Nn, shp)
+                outs.append(_linear(be, n1, be.from_numpy(w2)))
+            return N(be, *outs)
+
+        def expect():
+            f8 = np.float64
+            X = x.astype(f8)
+            P = X @ w.astype(f8).T
+            G, U = X @ wg.astype(f8).T, X @ wu.astype(f8).T
+            vals = [ts[0].astype(f8) + P, sum(t.astype(f8) for t in ts) + P, G / (1.0 + np.exp(-G)) * U]
+            if axis == 1:
+                vals = [v.reshape(1, B, Nn) for v in vals]
+            cats = []
+            for v in vals:
+                c = np.concatenate([prev.astype(f8), v], axis)
+                cats += [c, c]
+            outs = list(cats)
+            for c in cats[:2]:
+                h = c.reshape(1, -1, Nn)[:, -4:]
+                n1 = h / np.sqrt((h * h).mean(-1, keepdims=True) + f8(np.float32(1e-5))) * gm.astype(f8)
+                outs.append(n1 @ w2.astype(f8).T)
+            return outs
+
+        return run, expect
+
+
 # ---- decode-time attention: q.K^T -> causal soft-max -> p.V as the model graphs issue it ------------------------
 def decode_attention_ops(be, q, k_cache, v_cache, rep):
     """One decode step's attention of `LlamaModel` (catgrad-llm-models/src/models/llama.rs:285-345) on a
