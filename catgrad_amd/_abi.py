@@ -65,6 +65,7 @@ SIGNATURES = {
     "cg_sum": (_I, [_P, _P, _PP]),
     "cg_max": (_I, [_P, _P, _PP]),
     "cg_argmax": (_I, [_P, _P, _PP]),
+    "cg_argmax_rows_noalloc": (_I, [_I, _I, _P, _SZ, _SZ, _P, _P]),
     "cg_topk": (_I, [_P, _P, _SZ, _PP, _PP]),
     "cg_broadcast": (_I, [_P, _P, _SZP, _SZ, _PP]),
     "cg_reshape": (_I, [_P, _P, _SZP, _SZ, _PP]),

@@ -407,6 +407,8 @@ int launch_gather(cg_backend *be, const cg_tensor *x, int dim, const cg_tensor *
 
 enum ReduceKind : int { kSum = 0, kMax = 1, kArgmax = 2 };
 int launch_reduce(cg_backend *be, int kind, const cg_tensor *x, cg_tensor *out);
+// Asks for the device address of the fixed scratch array of cg_argmax_rows_noalloc on `device` (once per device).
+int noalloc_setup(int device);
 int launch_topk(cg_backend *be, const cg_tensor *x, int64_t k, cg_tensor *vals, cg_tensor *idxs);
 // *flag_dev = any(x > 0) / any(x != y)
 int launch_any_positive(cg_backend *be, const cg_tensor *x);

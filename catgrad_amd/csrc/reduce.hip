@@ -18,6 +18,7 @@
 #include "device_utils.hpp"
 
 #include <algorithm>
+#include <mutex>
 
 namespace cg {
 
@@ -345,6 +346,30 @@ template <int K, bool F> int launch_rows(cg_backend *be, const RowsArgs &a) {
 
 } // namespace
 
+// ---- arg-max for callers that cannot allocate -------------------------------------------------------------------
+// The segmented arg-max above takes its per-segment results from the pool.  This variant keeps them in a fixed array
+// in device memory instead, so that the call allocates nothing: every GPU the library runs on holds one copy of the
+// array (128 KiB) until the process ends.  In host code the array's name stands for no device address; the address
+// on a given device comes from hipGetSymbolAddress, asked once per device with that device current.
+constexpr uint32_t kNoAllocMaxParts = 16384; // rows x segments
+static __device__ __align__(256) long long scratch[kNoAllocMaxParts];
+
+constexpr int kNoAllocMaxDevices = 64;
+static std::mutex g_scratch_mu;
+static long long *g_scratch_ptr[kNoAllocMaxDevices] = {};
+
+int noalloc_setup(int device) {
+    if (device < 0 || device >= kNoAllocMaxDevices) return fail(CG_ERR_ARG, "device %d out of range", device);
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (g_scratch_ptr[device]) return CG_OK;
+    CG_HIP(hipSetDevice(device));
+    long long *ptr = nullptr;
+    CG_HIP(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
+    if (!ptr) return fail(CG_ERR_DEVICE, "no device address for the scratch array on device %d", device);
+    g_scratch_ptr[device] = ptr;
+    return CG_OK;
+}
+
 int launch_reduce(cg_backend *be, int kind, const cg_tensor *x, cg_tensor *out) {
     if (int frc = flush_deferred(be)) return frc;
     RowsArgs a;
@@ -405,3 +430,52 @@ int launch_any_positive(cg_backend *be, const cg_tensor *x) { return launch_any(
 int launch_any_diff(cg_backend *be, const cg_tensor *x, const cg_tensor *y) { return launch_any(be, 1, x, y); }
 
 } // namespace cg
+
+// Arg-max over the rows of a dense [rows, n] array of 32-bit words at `x` (device memory) into out[rows] (device
+// memory), queued on `stream`; nothing is allocated and nothing waits.  Same kernels as the segmented arg-max behind
+// cg_argmax, with the per-segment results in the library's fixed scratch array.
+extern "C" int cg_argmax_rows_noalloc(int device, cg_dtype dtype, const void *x, size_t rows, size_t n, uint32_t *out,
+                                      void *stream) {
+    using namespace cg;
+    if (dtype != CG_F32 && dtype != CG_U32 && dtype != CG_F16 && dtype != CG_BF16 && dtype != CG_F8)
+        return fail(CG_ERR_UNSUPPORTED, "unknown dtype");
+    if (n == 0) return fail(CG_ERR_SHAPE, "argmax: called `Option::unwrap()` on a `None` value (empty axis)");
+    if (rows == 0) return CG_OK;
+    if (!x || !out) return fail(CG_ERR_ARG, "null argument");
+    if (n > 0x3FFFFFFFull) return fail(CG_ERR_UNSUPPORTED, "argmax without allocation: rows longer than 2^30-1 elements");
+    uint32_t segs = std::min<uint32_t>(256, (uint32_t)((n + 1023) / 1024));
+    const uint32_t seglen = (uint32_t)(((n + segs - 1) / segs + 3) / 4 * 4);
+    segs = (uint32_t)((n + seglen - 1) / seglen);
+    if (rows > 65535 || rows * segs > kNoAllocMaxParts)
+        return fail(CG_ERR_UNSUPPORTED,
+                    "argmax without allocation: %zu rows x %u segments exceed the fixed scratch of %u partial results "
+                    "(rows x ceil(n / 1024), segments capped at 256)",
+                    rows, segs, kNoAllocMaxParts);
+    int rc = noalloc_setup(device); // the first call on a device asks for the array's address there
+    if (rc) return rc;
+    CG_HIP(hipSetDevice(device));
+    long long *part = g_scratch_ptr[device];
+    RowsArgs a;
+    memset(&a, 0, sizeof a);
+    a.x = static_cast<const char *>(x);
+    a.out = out;
+    a.rows = (uint32_t)rows;
+    a.n = (uint32_t)n;
+    a.sn = 1;
+    a.nouter = 1;
+    a.od[0] = (uint32_t)rows;
+    a.odiv[0] = make_fastdiv(a.od[0]);
+    a.os[0] = (int64_t)n;
+    a.vec = (n % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0) ? 4 : 1;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // every partial result the second kernel reads is written by the first: nothing has to start at zero
+    if (dtype == CG_U32) {
+        hipLaunchKernelGGL((reduce_segments_kernel<kArgmax, false>), dim3(segs, a.rows), dim3(kBlock), 0, s, a, part, seglen);
+        hipLaunchKernelGGL((reduce_segments_final_kernel<kArgmax, false>), dim3(a.rows), dim3(64), 0, s, part, out, segs);
+    } else {
+        hipLaunchKernelGGL((reduce_segments_kernel<kArgmax, true>), dim3(segs, a.rows), dim3(kBlock), 0, s, a, part, seglen);
+        hipLaunchKernelGGL((reduce_segments_final_kernel<kArgmax, true>), dim3(a.rows), dim3(64), 0, s, part, out, segs);
+    }
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CG_OK : hip_fail(e, "argmax without allocation: launch");
+}

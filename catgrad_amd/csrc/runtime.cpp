@@ -1737,6 +1737,7 @@ int cg_backend_create(int device, cg_backend **out) {
     CG_HIP(hipSetDevice(device));
     hipDeviceProp_t prop;
     CG_HIP(hipGetDeviceProperties(&prop, device));
+    if (int nrc = noalloc_setup(device)) return nrc; // set-up of the entry point that may not allocate later
     cg_backend *b = new cg_backend;
     b->device = device;
     CG_HIP(hipStreamCreateWithFlags(&b->stream, hipStreamNonBlocking));

@@ -207,6 +207,16 @@ int cg_matmul(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **out);
 int cg_sum(cg_backend *b, cg_tensor *x, cg_tensor **out);
 int cg_max(cg_backend *b, cg_tensor *x, cg_tensor **out);
 int cg_argmax(cg_backend *b, cg_tensor *x, cg_tensor **out);
+/* No counterpart in the reference.  For callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): the arg-max of cg_argmax over the rows of a dense
+ * [rows, n] array of `dtype` words (4 bytes each, also for the narrow float dtypes) that already lies in device
+ * memory at `x`, written as u32 to `out` (device memory, `rows` entries).  The two kernels are queued on `stream`
+ * (a hipStream_t; null = the default stream) of `device`; the call allocates nothing, frees nothing and does not
+ * wait.  Per-segment partial results go to a fixed 128 KiB array that each GPU holds until the process ends:
+ * rows * min(256, ceil(n / 1024)) must not exceed 16384 (and rows 65535), else CG_ERR_UNSUPPORTED.  All calls on one
+ * GPU share that array: calls that overlap in time on one GPU race; order them on one stream or with events. */
+int cg_argmax_rows_noalloc(int device, cg_dtype dtype, const void *x, size_t rows, size_t n, uint32_t *out,
+                           void *stream);
 /* `Backend::topk` (mod.rs:86; ndarray.rs:436-446,696-721). */
 int cg_topk(cg_backend *b, cg_tensor *x, size_t k, cg_tensor **values, cg_tensor **indices);
 

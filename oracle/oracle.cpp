@@ -1060,6 +1060,34 @@ int cg_argmax(cg_backend *, cg_tensor *x, cg_tensor **out) {
     return CG_OK;
 }
 
+// The same rule on a dense [rows, n] array in plain memory (the checker's side of the entry point that the GPU
+// library offers to callers that cannot allocate; `device` and `stream` mean nothing here).
+int cg_argmax_rows_noalloc(int, cg_dtype dtype, const void *x, size_t rows, size_t n, uint32_t *out, void *) {
+    if (n == 0) return fail(CG_ERR_SHAPE, "argmax: called `Option::unwrap()` on a `None` value (empty axis)");
+    if (rows == 0) return CG_OK;
+    if (!x || !out) return fail(CG_ERR_ARG, "null argument");
+    for (size_t i = 0; i < rows; i++) {
+        size_t best = 0;
+        if (dtype == CG_U32) {
+            const uint32_t *v = static_cast<const uint32_t *>(x) + i * n;
+            for (size_t j = 1; j < n; j++)
+                if (v[j] >= v[best]) best = j;
+        } else {
+            const float *v = static_cast<const float *>(x) + i * n;
+            int32_t bk = total_key(v[0]);
+            for (size_t j = 1; j < n; j++) {
+                const int32_t k = total_key(v[j]);
+                if (k >= bk) {
+                    bk = k;
+                    best = j;
+                }
+            }
+        }
+        out[i] = (uint32_t)best;
+    }
+    return CG_OK;
+}
+
 // ndarray.rs:436-446, 696-721 — stable sort, descending by total_cmp, first k.
 int cg_topk(cg_backend *, cg_tensor *x, size_t k, cg_tensor **values, cg_tensor **indices) {
     Consume cx(x);
