@@ -70,6 +70,8 @@ struct Buffer;
 
 struct cg_backend {
     std::recursive_mutex mu; // held by every entry point for the duration of the call
+    std::atomic<long> live_tensors{0}; // heap handles that name this backend (see alloc_tensor)
+    bool owner_gone = false;           // cg_backend_destroy has been called; the last handle released tears down
     int device = 0;
     hipStream_t stream = nullptr;
     cg::Pool pool;

@@ -284,12 +284,23 @@ int lazy_mm_force(cg_backend *be, LazyMm *m) {
     return rc;
 }
 
+// Every handle that can leave the library is counted in its backend: the backend's memory pool, stream and lock
+// outlive cg_backend_destroy for as long as such a handle exists (see there).
+static cg_tensor *alloc_tensor(cg_backend *be) {
+    cg_tensor *t = new cg_tensor;
+    t->be = be;
+    be->live_tensors.fetch_add(1, std::memory_order_relaxed);
+    return t;
+}
+
 void release(cg_tensor *t) {
     if (!t) return;
     if (t->rc.fetch_sub(1) == 1) {
+        cg_backend *be = t->be;
         buffer_release(t->buf);
         delete t->pend;
         delete t;
+        be->live_tensors.fetch_sub(1, std::memory_order_relaxed);
     }
 }
 
@@ -302,7 +313,7 @@ static void set_row_major(cg_tensor *t) {
 }
 
 int new_dense(cg_backend *be, cg_dtype dt, const int64_t *dims, int rank, cg_tensor **out, int64_t reserve_elems) {
-    cg_tensor *t = new cg_tensor;
+    cg_tensor *t = alloc_tensor(be);
     t->be = be;
     t->dt = dt;
     t->rank = rank;
@@ -316,6 +327,7 @@ int new_dense(cg_backend *be, cg_dtype dt, const int64_t *dims, int rank, cg_ten
         if (rc) {
             delete b;
             delete t;
+            be->live_tensors.fetch_sub(1, std::memory_order_relaxed);
             return rc;
         }
         b->elems = n;
@@ -326,7 +338,7 @@ int new_dense(cg_backend *be, cg_dtype dt, const int64_t *dims, int rank, cg_ten
 }
 
 cg_tensor *new_uniform(cg_backend *be, cg_dtype dt, const int64_t *dims, int rank, uint32_t bits) {
-    cg_tensor *t = new cg_tensor;
+    cg_tensor *t = alloc_tensor(be);
     t->be = be;
     t->dt = dt;
     t->rank = rank;
@@ -340,7 +352,7 @@ cg_tensor *new_uniform(cg_backend *be, cg_dtype dt, const int64_t *dims, int ran
 }
 
 cg_tensor *new_view(const cg_tensor *t) {
-    cg_tensor *v = new cg_tensor;
+    cg_tensor *v = alloc_tensor(t->be);
     v->be = t->be;
     v->buf = t->buf;
     if (v->buf) v->buf->rc.fetch_add(1);
@@ -1370,7 +1382,7 @@ static int defer_elementwise(cg_backend *be, int op, cg_dtype in_dt, cg_dtype ou
         for (int k = 0; k < nin; k++)
             if (ins[k] == w) splice[k] = false;
     }
-    cg_tensor *t = new cg_tensor;
+    cg_tensor *t = alloc_tensor(be);
     t->be = be;
     t->dt = out_dt;
     t->rank = rank;
@@ -1418,7 +1430,7 @@ static int defer_reduce(cg_backend *be, int kind, cg_tensor *x, const int64_t *o
         delete p;
         return CG_OK;
     }
-    cg_tensor *t = new cg_tensor;
+    cg_tensor *t = alloc_tensor(be);
     t->be = be;
     t->dt = x->dt;
     t->rank = rank;
@@ -1453,7 +1465,7 @@ static int pending_view(cg_tensor *x, const int64_t *dims, int rank, F &&fn, cg_
             return ensure_concrete(x);
         }
     }
-    cg_tensor *t = new cg_tensor;
+    cg_tensor *t = alloc_tensor(x->be);
     t->be = x->be;
     t->dt = x->dt;
     t->rank = rank;
@@ -1685,7 +1697,7 @@ static bool try_row_append(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim
         if (*status) return true;
         for (int64_t o = 0; o < outer; o++) ds->fill[(size_t)blocks[(size_t)o]] = xd + yd;
     }
-    cg_tensor *v = new cg_tensor;
+    cg_tensor *v = alloc_tensor(b);
     v->be = b;
     v->buf = dstbuf;
     dstbuf->rc.fetch_add(1);
@@ -1760,18 +1772,10 @@ int cg_backend_create(int device, cg_backend **out) {
     return CG_OK;
 }
 
-void cg_backend_destroy(cg_backend *b) {
-    if (!b) return;
+// What is left of a backend once nothing refers to it any more.
+static void backend_teardown(cg_backend *b) {
     (void)hipSetDevice(b->device);
-    for (DeferredWrite &d : b->deferred) drop_deferred(d); // nobody can read them any more
-    b->deferred.clear();
-    const_memo_clear(b);
     (void)hipStreamSynchronize(b->stream);
-    prof_drain(b);
-    for (auto &ev : b->prof_free) {
-        (void)hipEventDestroy(ev.first);
-        (void)hipEventDestroy(ev.second);
-    }
     b->pool.trim();
     (void)hipFree(b->flag_dev);
     for (int i = 0; i < 2; i++) {
@@ -1782,6 +1786,34 @@ void cg_backend_destroy(cg_backend *b) {
     (void)hipHostFree(b->fault_host);
     (void)hipStreamDestroy(b->stream);
     delete b;
+}
+
+// The reference's tensors own their data and may outlive the backend value that made them
+// (`BackendTensorOps: Send + Sync + Clone`, backend/mod.rs:124-126, no lifetime ties them to a `Backend`).  So
+// destroying a backend only gives up the owner's hold on it: everything that needs no tensor goes now, and the pool,
+// the stream and the lock stay until the last tensor handle has been released (cg_tensor_release then finishes the
+// job).  Such surviving handles can be cloned, queried for their shape and released, nothing else.
+void cg_backend_destroy(cg_backend *b) {
+    if (!b) return;
+    bool last;
+    {
+        Enter entered(b);
+        (void)hipSetDevice(b->device);
+        for (DeferredWrite &d : b->deferred) drop_deferred(d); // nobody can read them any more
+        b->deferred.clear();
+        const_memo_clear(b);
+        (void)hipStreamSynchronize(b->stream);
+        prof_drain(b);
+        for (auto &ev : b->prof_free) {
+            (void)hipEventDestroy(ev.first);
+            (void)hipEventDestroy(ev.second);
+        }
+        b->prof_free.clear();
+        b->pool.trim();
+        b->owner_gone = true;
+        last = b->live_tensors.load() == 0;
+    }
+    if (last) backend_teardown(b);
 }
 
 const char *cg_last_error(void) { return g_err.c_str(); }
@@ -1859,8 +1891,14 @@ void cg_tensor_retain(cg_tensor *t) {
 }
 void cg_tensor_release(cg_tensor *t) {
     if (!t) return;
-    Enter entered(t->be); // the last holder of a deferred tensor also closes what it had open in the backend
-    release(t);
+    cg_backend *be = t->be;
+    bool last;
+    {
+        Enter entered(be); // the last holder of a deferred tensor also closes what it had open in the backend
+        release(t);
+        last = be->owner_gone && be->live_tensors.load() == 0;
+    }
+    if (last) backend_teardown(be); // the backend was destroyed while handles were still out: this was the last one
 }
 size_t cg_tensor_rank(const cg_tensor *t) { return (size_t)t->rank; }
 void cg_tensor_shape(const cg_tensor *t, size_t *dims) {
@@ -2042,7 +2080,7 @@ int cg_arange(cg_backend *b, size_t end, cg_tensor **out) {
             b->iota_len = cap;
             release(full);
         }
-        t = new cg_tensor;
+        t = alloc_tensor(b);
         t->be = b;
         t->dt = CG_U32;
         t->rank = 1;
@@ -2455,7 +2493,7 @@ static int matmul_entry(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **o
             m->y = y;
             m->rank = r;
             memcpy(m->dims, od, sizeof m->dims);
-            cg_tensor *t = new cg_tensor;
+            cg_tensor *t = alloc_tensor(b);
             t->be = b;
             t->dt = CG_F32;
             t->rank = r;
@@ -2608,7 +2646,7 @@ int cg_broadcast(cg_backend *b, cg_tensor *x, const size_t *dims, size_t rank, c
         if (same) {
             Pending *p = new Pending(*x->pend);
             p->reduced = false;
-            cg_tensor *t = new cg_tensor;
+            cg_tensor *t = alloc_tensor(b);
             t->be = b;
             t->dt = x->dt;
             t->rank = (int)rank;
@@ -2860,7 +2898,7 @@ int cg_concat(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor *
             in.op = (uint8_t)(kCopy | (x->dt == CG_U32 ? kInstrU32 : 0));
             in.a = in.b = in.c = 0;
             emit_instr(p, in);
-            cg_tensor *t = new cg_tensor;
+            cg_tensor *t = alloc_tensor(b);
             t->be = b;
             t->dt = x->dt;
             t->rank = x->rank;
@@ -2927,7 +2965,7 @@ int cg_concat(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor *
             ckey += ky;
             auto hit = b->const_memo.find(ckey);
             if (hit != b->const_memo.end()) {
-                o = new cg_tensor;
+                o = alloc_tensor(b);
                 o->be = b;
                 o->dt = x->dt;
                 o->rank = x->rank;

@@ -152,8 +152,10 @@ struct GenerateStats {
 // is the next input (main.rs:1031-1037 generalised from batch 1 to B rows).
 // out_tokens receives (steps + 1) x B ids: the token produced by the prefill, then one
 // per decode run.  Prefill time includes the first read-back, as in main.rs:914-917.
+// prefill_logits, when given, receives the lm_head output [B, S, vocab] of the prefill run (read back after the
+// timed part of that run; for parity checks).
 inline void generate(LlmModel &m, Interpreter &i, const uint32_t *prompt, size_t B, size_t S, size_t steps,
-                     size_t max_positions, uint32_t *out_tokens, GenerateStats *st) {
+                     size_t max_positions, uint32_t *out_tokens, GenerateStats *st, std::vector<uint32_t> *prefill_logits = nullptr) {
     const LlmConfig &c = m.config();
     // empty_state_cache (utils/mod.rs:570-583) with the batch axis set to B
     Shape kv{c.num_hidden_layers, B, c.num_key_value_heads, 0, c.head_dim};
@@ -165,7 +167,8 @@ inline void generate(LlmModel &m, Interpreter &i, const uint32_t *prompt, size_t
     for (size_t it = 0; it <= steps; it++) {
         Tensor x = i.backend.ndarray_from_vec_u32(ids.data(), ids.size(), Shape{B, cur});
         // the run's inputs are clones of the caller's state (main.rs:1007)
-        ForwardOut o = m.forward(std::move(x), state_k, state_v, max_positions);
+        Tensor logits;
+        ForwardOut o = m.forward(std::move(x), state_k, state_v, max_positions, it == 0 && prefill_logits ? &logits : nullptr);
         std::vector<uint32_t> tok = i.backend.to_vec_bits(std::move(o.tokens));
         ids.resize(B);
         for (size_t b = 0; b < B; b++) {
@@ -179,8 +182,9 @@ inline void generate(LlmModel &m, Interpreter &i, const uint32_t *prompt, size_t
             auto t1 = std::chrono::steady_clock::now();
             st->prefill_s = std::chrono::duration<double>(t1 - t0).count();
             st->prefill_calls = i.backend.calls - calls0;
+            if (prefill_logits) *prefill_logits = i.backend.to_vec_bits(std::move(logits));
             calls0 = i.backend.calls;
-            t0 = t1;
+            t0 = std::chrono::steady_clock::now();
         }
     }
     st->decode_s = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();

@@ -112,6 +112,21 @@ int cgm_generate(cgm_session *s, const uint32_t *prompt, size_t B, size_t S, siz
     });
 }
 
+int cgm_generate_with_logits(cgm_session *s, const uint32_t *prompt, size_t B, size_t S, size_t steps, size_t max_positions,
+                             uint32_t *out_tokens, double *stats4, float *prefill_logits) {
+    return guarded([&] {
+        LlmModel m(*s->interp, s->config);
+        GenerateStats st;
+        std::vector<uint32_t> lg;
+        generate(m, *s->interp, prompt, B, S, steps, max_positions, out_tokens, &st, &lg);
+        memcpy(prefill_logits, lg.data(), lg.size() * 4);
+        stats4[0] = st.prefill_s;
+        stats4[1] = st.decode_s;
+        stats4[2] = (double)st.prefill_calls;
+        stats4[3] = (double)st.decode_calls;
+    });
+}
+
 int cgm_forward(cgm_session *s, const uint32_t *tokens, size_t B, size_t S, size_t max_positions, uint32_t *out_tokens,
                 float *out_logits) {
     return guarded([&] {
@@ -129,6 +144,26 @@ int cgm_forward(cgm_session *s, const uint32_t *tokens, size_t B, size_t S, size
             std::vector<uint32_t> lg = i.backend.to_vec_bits(std::move(logits));
             memcpy(out_logits, lg.data(), lg.size() * 4);
         }
+    });
+}
+
+int cgm_forward_rows(cgm_session *s, const uint32_t *tokens, size_t B, size_t S, size_t max_positions, uint32_t *out_tokens,
+                     const uint32_t *rows, size_t nrows, float *out_logits) {
+    return guarded([&] {
+        Interpreter &i = *s->interp;
+        LlmModel m(i, s->config);
+        const LlmConfig &c = s->config;
+        Shape kv{c.num_hidden_layers, B, c.num_key_value_heads, 0, c.head_dim};
+        Tensor x = i.backend.ndarray_from_vec_u32(tokens, B * S, Shape{B, S});
+        Tensor logits;
+        ForwardOut o = m.forward(std::move(x), i.backend.zeros(kv, CG_F32), i.backend.zeros(kv, CG_F32), max_positions, &logits);
+        std::vector<uint32_t> tok = i.backend.to_vec_bits(std::move(o.tokens));
+        memcpy(out_tokens, tok.data(), tok.size() * 4);
+        Tensor flat = i.backend.reshape(std::move(logits), Shape{B * S, c.vocab_size});
+        Tensor idx = i.backend.ndarray_from_vec_u32(rows, nrows, Shape{nrows});
+        Tensor picked = i.backend.index(std::move(flat), 0, std::move(idx));
+        std::vector<uint32_t> lg = i.backend.to_vec_bits(std::move(picked));
+        memcpy(out_logits, lg.data(), lg.size() * 4);
     });
 }
 

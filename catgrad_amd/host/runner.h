@@ -33,11 +33,20 @@ int cgm_set_config(cgm_session *s, int arch, size_t hidden_size, size_t num_hidd
  * [prefill_s, decode_s, backend calls in prefill, backend calls in decode]. */
 int cgm_generate(cgm_session *s, const uint32_t *prompt, size_t B, size_t S, size_t steps, size_t max_positions,
                  uint32_t *out_tokens, double *stats4);
+/* The same, also returning the prefill run's logits [B, S, vocab] (read back outside the timed parts). */
+int cgm_generate_with_logits(cgm_session *s, const uint32_t *prompt, size_t B, size_t S, size_t steps, size_t max_positions,
+                             uint32_t *out_tokens, double *stats4, float *prefill_logits);
 
 /* One run on an empty cache.  out_tokens: B x S argmax ids.  out_logits (may be null):
  * B x S x vocab logits, read from the same run just before `argmax`. */
 int cgm_forward(cgm_session *s, const uint32_t *tokens, size_t B, size_t S, size_t max_positions, uint32_t *out_tokens,
                 float *out_logits);
+
+/* As cgm_forward, but only the logits of `nrows` chosen positions are read back: rows[i] = b * S + s selects
+ * sequence b, position s; out_logits: nrows x vocab.  (The [B, S, vocab] logits of a full-size run are gigabytes;
+ * the rows are gathered on the device with `index` before `to_vec`.) */
+int cgm_forward_rows(cgm_session *s, const uint32_t *tokens, size_t B, size_t S, size_t max_positions, uint32_t *out_tokens,
+                     const uint32_t *rows, size_t nrows, float *out_logits);
 
 /* Config-1 MLP: x f32[1, rows, in] -> Linear(in, hidden)+b -> Sigmoid -> Linear(hidden, out)+b.
  * Parameters: mlp.l1.weight [hidden,in], mlp.l1.bias [hidden], mlp.l2.weight [out,hidden], mlp.l2.bias [out]. */

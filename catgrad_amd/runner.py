@@ -37,7 +37,9 @@ def _host():
             "cgm_load_safetensors": (C.c_int, [P, C.POINTER(C.c_char_p), SZ, C.POINTER(C.c_double)]),
             "cgm_set_config": (C.c_int, [P, C.c_int] + [SZ] * 7 + [C.c_float, C.c_float, C.c_int]),
             "cgm_generate": (C.c_int, [P, P, SZ, SZ, SZ, SZ, P, C.POINTER(C.c_double)]),
+            "cgm_generate_with_logits": (C.c_int, [P, P, SZ, SZ, SZ, SZ, P, C.POINTER(C.c_double), P]),
             "cgm_forward": (C.c_int, [P, P, SZ, SZ, SZ, P, P]),
+            "cgm_forward_rows": (C.c_int, [P, P, SZ, SZ, SZ, P, P, SZ, P]),
             "cgm_mlp": (C.c_int, [P, P, SZ, SZ, SZ, SZ, P]),
             "cgm_pool_stats": (C.c_int, [P, SZP, SZP]),
             "cgm_sync": (C.c_int, [P]),
@@ -189,17 +191,25 @@ class Session:
             config.vocab_size, config.rms_norm_eps, config.rope_theta, int(config.tie_word_embeddings)))
         self.config = config
 
-    def generate(self, prompt: np.ndarray, steps: int, max_positions: int | None = None):
-        """Prefill + `steps` greedy decode runs.  Returns (tokens [(steps+1), B], stats dict)."""
+    def generate(self, prompt: np.ndarray, steps: int, max_positions: int | None = None, want_logits: bool = False):
+        """Prefill + `steps` greedy decode runs.  Returns (tokens [(steps+1), B], stats dict); with `want_logits`
+        also the prefill run's logits [B, S, vocab] as a third value."""
         prompt = np.ascontiguousarray(prompt, dtype=np.uint32)
         B, S = prompt.shape
         max_positions = max_positions or (S + steps)
         out = np.zeros((steps + 1, B), dtype=np.uint32)
         stats = (C.c_double * 4)()
-        self._check(self._lib.cgm_generate(self._s, prompt.ctypes.data_as(C.c_void_p), B, S, steps, max_positions,
-                                           out.ctypes.data_as(C.c_void_p), stats))
-        return out, {"prefill_s": stats[0], "decode_s": stats[1], "prefill_calls": int(stats[2]),
-                     "decode_calls": int(stats[3])}
+        logits = None
+        if want_logits:
+            logits = np.zeros((B, S, self.config.vocab_size), dtype=np.float32)
+            self._check(self._lib.cgm_generate_with_logits(self._s, prompt.ctypes.data_as(C.c_void_p), B, S, steps,
+                                                           max_positions, out.ctypes.data_as(C.c_void_p), stats,
+                                                           logits.ctypes.data_as(C.c_void_p)))
+        else:
+            self._check(self._lib.cgm_generate(self._s, prompt.ctypes.data_as(C.c_void_p), B, S, steps, max_positions,
+                                               out.ctypes.data_as(C.c_void_p), stats))
+        st = {"prefill_s": stats[0], "decode_s": stats[1], "prefill_calls": int(stats[2]), "decode_calls": int(stats[3])}
+        return (out, st, logits) if want_logits else (out, st)
 
     def forward(self, tokens: np.ndarray, max_positions: int | None = None, want_logits: bool = True):
         tokens = np.ascontiguousarray(tokens, dtype=np.uint32)
@@ -209,6 +219,19 @@ class Session:
         self._check(self._lib.cgm_forward(self._s, tokens.ctypes.data_as(C.c_void_p), B, S, max_positions or S,
                                           out.ctypes.data_as(C.c_void_p),
                                           logits.ctypes.data_as(C.c_void_p) if want_logits else None))
+        return out, logits
+
+    def forward_rows(self, tokens: np.ndarray, rows, max_positions: int | None = None):
+        """One run on an empty cache; returns the argmax ids [B, S] and the logits [len(rows), vocab] of the chosen
+        positions only (rows[i] = b * S + s), gathered on the device."""
+        tokens = np.ascontiguousarray(tokens, dtype=np.uint32)
+        rows = np.ascontiguousarray(rows, dtype=np.uint32)
+        B, S = tokens.shape
+        out = np.zeros((B, S), dtype=np.uint32)
+        logits = np.zeros((rows.size, self.config.vocab_size), dtype=np.float32)
+        self._check(self._lib.cgm_forward_rows(self._s, tokens.ctypes.data_as(C.c_void_p), B, S, max_positions or S,
+                                               out.ctypes.data_as(C.c_void_p), rows.ctypes.data_as(C.c_void_p), rows.size,
+                                               logits.ctypes.data_as(C.c_void_p)))
         return out, logits
 
     def mlp(self, x: np.ndarray, hidden: int, out_dim: int) -> np.ndarray:

@@ -131,6 +131,10 @@ impl HipBackend {
 }
 
 /// A reference-counted handle to a strided device view.  `Clone` is a refcount bump.
+/// A tensor may outlive every `HipBackend` value (a `Parameters<HipBackend>` map dropped after the backend, a result
+/// kept by the caller): the C library counts the live handles of a backend and `cg_backend_destroy` only gives up the
+/// owner's hold, so `Drop` and `Clone` here stay valid in any drop order, as for the reference's tensors
+/// (`BackendTensorOps`, mod.rs:124-126, has no lifetime tied to a backend).
 pub struct HipTensor(*mut CgTensor);
 unsafe impl Send for HipTensor {}
 unsafe impl Sync for HipTensor {}
@@ -325,10 +329,11 @@ impl Backend for HipBackend {
         self.one(x, Some(Dtype::U32), |b, t, o| unsafe { cg_argmax(b, t, o) })
     }
     fn topk(&self, x: TaggedTensor<Self>, k: usize) -> (TaggedTensor<Self>, TaggedTensor<Self>) {
+        let dt = x.dtype(); // the values keep the input's dtype (cg_topk takes every floating-point dtype)
         let [t] = untag(x);
         let (mut v, mut i) = (std::ptr::null_mut(), std::ptr::null_mut());
         check(unsafe { cg_topk(self.raw(), t.into_raw(), k, &mut v, &mut i) });
-        (TaggedTensor::F32([HipTensor(v)]), TaggedTensor::U32([HipTensor(i)]))
+        (tag_for(&dt, HipTensor(v)), TaggedTensor::U32([HipTensor(i)]))
     }
     fn compare(&self, x: TaggedTensorTuple<Self, 2>) -> bool {
         let [a, b] = untag(x);

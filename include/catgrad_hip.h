@@ -33,7 +33,14 @@
  *    (`BackendTensorOps: Send + Sync`, mod.rs:124); calls on one backend are
  *    serialised by a lock inside the library, so concurrent callers are
  *    safe but do not overlap.  cg_backend_destroy must not race with
- *    anything.
+ *    another call on the same backend.
+ *  - Lifetime: a tensor handle may outlive its backend, as the reference's
+ *    tensors may (they own their data; nothing in mod.rs:124-126 ties a
+ *    tensor to a `Backend` value).  cg_backend_destroy gives up the owner's
+ *    hold: work in flight is waited for and cached memory freed at once, and
+ *    the pool, stream and lock go with the last cg_tensor_release.  After
+ *    cg_backend_destroy a surviving handle may only be retained, queried
+ *    (cg_tensor_rank / shape / dtype / numel) and released.
  *  - dims/shape arrays are row-major extents as size_t; rank 0 and zero
  *    extents are legal.  Maximum rank: CG_MAX_RANK.
  */

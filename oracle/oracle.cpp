@@ -45,6 +45,8 @@
 #include <cstdlib>
 #include <cstring>
 #include <limits>
+#include <map>
+#include <mutex>
 #include <numeric>
 #include <string>
 #include <vector>
@@ -64,9 +66,59 @@ int fail(int code, const char *fmt, ...) {
 }
 
 // ArcArray's shared allocation (ndarray.rs:19-20).
+// Large blocks are kept and handed out again instead of going back to the operating system: a model-sized run
+// allocates and drops gigabytes per op (every op of the reference makes a fresh array), and first-touch page faults
+// on fresh mappings cost several times the arithmetic.  Values are unaffected (vectors still zero-fill).
+struct BlockCache {
+    std::mutex mu;
+    std::multimap<size_t, void *> free_;
+    size_t cached = 0;
+    static constexpr size_t kMin = 1u << 20, kMaxCached = (size_t)24 << 30;
+    void *take(size_t bytes) {
+        if (bytes >= kMin) {
+            std::lock_guard<std::mutex> lk(mu);
+            auto it = free_.lower_bound(bytes);
+            if (it != free_.end() && it->first <= bytes + bytes / 4) {
+                void *p = it->second;
+                cached -= it->first;
+                free_.erase(it);
+                return p;
+            }
+        }
+        void *p = malloc(bytes);
+        if (!p) throw std::bad_alloc();
+        return p;
+    }
+    void give(void *p, size_t bytes) {
+        if (bytes >= kMin) {
+            std::lock_guard<std::mutex> lk(mu);
+            if (cached + bytes <= kMaxCached) {
+                free_.emplace(bytes, p);
+                cached += bytes;
+                return;
+            }
+        }
+        free(p);
+    }
+};
+inline BlockCache &block_cache() {
+    static BlockCache *c = new BlockCache; // never destroyed: vectors with static lifetime may outlive any order
+    return *c;
+}
+template <class T> struct CachedAlloc {
+    using value_type = T;
+    CachedAlloc() = default;
+    template <class U> CachedAlloc(const CachedAlloc<U> &) {}
+    T *allocate(size_t n) { return static_cast<T *>(block_cache().take(n * sizeof(T))); }
+    void deallocate(T *p, size_t n) { block_cache().give(p, n * sizeof(T)); }
+    template <class U> bool operator==(const CachedAlloc<U> &) const { return true; }
+    template <class U> bool operator!=(const CachedAlloc<U> &) const { return false; }
+};
+template <class T> using Vec = std::vector<T, CachedAlloc<T>>;
+
 struct Storage {
     std::atomic<long> rc{1};
-    std::vector<uint32_t> data; // f32 and u32 are both stored as 4-byte words
+    Vec<uint32_t> data; // f32 and u32 are both stored as 4-byte words
 };
 
 } // namespace
@@ -192,6 +244,51 @@ template <typename T> void gather_logical(const cg_tensor *t, T *dst) {
         dst[0] = base[0];
         return;
     }
+    // Same values, fewer cache misses (this is a checker, not a timing model of the reference): an outermost
+    // stride-0 axis is gathered once and repeated, and a view whose unit stride sits on the second-to-last axis (a
+    // transposed matrix, or a stack of them) is gathered in 32 x 32 tiles.
+    if (r >= 2 && t->dims[0] > 1 && t->strides[0] == 0) {
+        cg_tensor sub;
+        sub.st = t->st;
+        sub.dt = t->dt;
+        sub.offset = t->offset;
+        sub.rank = r - 1;
+        for (int d = 1; d < r; d++) {
+            sub.dims[d - 1] = t->dims[d];
+            sub.strides[d - 1] = t->strides[d];
+        }
+        const size_t slab = n / t->dims[0];
+        gather_logical<T>(&sub, dst);
+        sub.st = nullptr;
+        for (size_t i = 1; i < t->dims[0]; i++) memcpy(dst + i * slab, dst, slab * sizeof(T));
+        return;
+    }
+    if (r >= 2 && t->strides[r - 2] == 1 && t->strides[r - 1] != 1 && t->dims[r - 1] >= 32 && t->dims[r - 2] >= 32) {
+        const size_t R = t->dims[r - 2], Cn = t->dims[r - 1], mats = n / (R * Cn);
+        const ptrdiff_t cs = t->strides[r - 1];
+        size_t midx[CG_MAX_RANK] = {0};
+        ptrdiff_t moff = 0;
+        for (size_t m = 0; m < mats; m++) {
+            const T *src = base + moff;
+            T *out = dst + m * R * Cn;
+            for (size_t i0 = 0; i0 < R; i0 += 32)
+                for (size_t j0 = 0; j0 < Cn; j0 += 32) {
+                    const size_t i1 = std::min(R, i0 + 32), j1 = std::min(Cn, j0 + 32);
+                    for (size_t j = j0; j < j1; j++) {
+                        const T *col = src + (ptrdiff_t)j * cs;
+                        for (size_t i = i0; i < i1; i++) out[i * Cn + j] = col[i];
+                    }
+                }
+            for (int d = r - 3; d >= 0; d--) { // odometer over the matrices
+                midx[d]++;
+                moff += t->strides[d];
+                if (midx[d] < t->dims[d]) break;
+                moff -= (ptrdiff_t)midx[d] * t->strides[d];
+                midx[d] = 0;
+            }
+        }
+        return;
+    }
     size_t idx[CG_MAX_RANK] = {0};
     size_t inner = t->dims[r - 1];
     ptrdiff_t is = t->strides[r - 1];
@@ -214,8 +311,8 @@ template <typename T> void gather_logical(const cg_tensor *t, T *dst) {
     }
 }
 
-template <typename T> std::vector<T> dense(const cg_tensor *t) {
-    std::vector<T> v(numel(t));
+template <typename T> Vec<T> dense(const cg_tensor *t) {
+    Vec<T> v(numel(t));
     gather_logical<T>(t, v.data());
     return v;
 }
@@ -474,7 +571,7 @@ void ugemm(size_t m, size_t k, size_t n, const uint32_t *a, ptrdiff_t rsa, ptrdi
 // memory layout allows merging the leading axes, else a row-major copy.  Returns base
 // pointer and the three strides; `tmp` holds the copy if one was needed.
 template <typename T>
-const T *as_batch3(cg_tensor *t, size_t batch, std::vector<T> &tmp, ptrdiff_t &sb, ptrdiff_t &sr, ptrdiff_t &sc) {
+const T *as_batch3(cg_tensor *t, size_t batch, Vec<T> &tmp, ptrdiff_t &sb, ptrdiff_t &sr, ptrdiff_t &sc) {
     int r = t->rank;
     size_t R = t->dims[r - 2], C = t->dims[r - 1];
     // leading axes mergeable iff they are mutually row-major nested
@@ -885,7 +982,7 @@ int cg_matmul(cg_backend *, cg_tensor *x, cg_tensor *y, cg_tensor **out) {
     odims[rx - 1] = N;
     cg_tensor *r = new_tensor(ox->dt, odims, rx);
     if (isf(ox->dt)) {
-        std::vector<float> ta, tb;
+        Vec<float> ta, tb;
         ptrdiff_t sba, sra, sca, sbb, srb, scb;
         const float *a = as_batch3<float>(ox, batch, ta, sba, sra, sca);
         const float *b = as_batch3<float>(oy, batch, tb, sbb, srb, scb);
@@ -894,7 +991,7 @@ int cg_matmul(cg_backend *, cg_tensor *x, cg_tensor *y, cg_tensor **out) {
             sgemm(M, K, N, a + (ptrdiff_t)bi * sba, sra, sca, b + (ptrdiff_t)bi * sbb, srb, scb, c + bi * M * N,
                   (ptrdiff_t)N, 1);
     } else {
-        std::vector<uint32_t> ta, tb;
+        Vec<uint32_t> ta, tb;
         ptrdiff_t sba, sra, sca, sbb, srb, scb;
         const uint32_t *a = as_batch3<uint32_t>(ox, batch, ta, sba, sra, sca);
         const uint32_t *b = as_batch3<uint32_t>(oy, batch, tb, sbb, srb, scb);

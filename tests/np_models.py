@@ -21,9 +21,20 @@ def rope(x, theta, positions):
     return x * cos + rot * sin
 
 
-def llm_logits(cfg, params, tokens):
-    """Logits [B, S, V] for token ids [B, S] (no cache: full causal recomputation)."""
-    P = {k: v.astype(np.float64) for k, v in params.items()}
+class _Wide:
+    """Parameters widened to float64 one at a time, on use (the full-size models do not fit twice)."""
+
+    def __init__(self, params):
+        self.p = params
+
+    def __getitem__(self, k):
+        return self.p[k].astype(np.float64)
+
+
+def llm_logits(cfg, params, tokens, positions=None):
+    """Logits [B, S, V] for token ids [B, S] (no cache: full causal recomputation); with `positions`
+    (indices along S) only those rows go through the vocabulary projection: [B, len(positions), V]."""
+    P = _Wide(params)
     r = cfg.arch
     B, S = tokens.shape
     h, kv, hd = cfg.num_attention_heads, cfg.num_key_value_heads, cfg.hd
@@ -51,6 +62,8 @@ def llm_logits(cfg, params, tokens):
         g = hn @ P[f"{p}.mlp.gate_proj.weight"].T
         u = hn @ P[f"{p}.mlp.up_proj.weight"].T
         x = x + ((g / (1.0 + np.exp(-g))) * u) @ P[f"{p}.mlp.down_proj.weight"].T
+    if positions is not None:
+        x = x[:, list(positions), :]
     x = rmsnorm(x, P[f"{r}.model.norm.weight"], cfg.rms_norm_eps)
     head = f"{r}.model.embed_tokens.weight" if cfg.tie_word_embeddings else f"{r}.lm_head.weight"
     return x @ P[head].T

@@ -113,11 +113,13 @@ def test_reduced_qwen3_prefill_and_decode(hip_session, cpu_session):
     print(f"qwen3-reduced: max |dlogit| {err:.3e} (scale {scale:.3e}); calls/decode step {st['decode_calls'] / 16:.0f}",
           flush=True)
     assert err <= 1e-3 * scale
-    bad = np.argwhere(g_h != g_c)
-    if bad.size:
-        # after a near-tie flip the sequences legitimately diverge; require agreement up to there
-        print(f"first divergence at step {bad[0][0]}", flush=True)
-        assert bad[0][0] > 0
+    # tokens: identical up to a choice whose float64 top1-top2 gap is within twice the logit error; float64 gaps of
+    # the oracle's own sequence, teacher-forced (after such a near-tie the sequences legitimately diverge)
+    seq = np.concatenate([prompt, g_c[:-1].T], axis=1)
+    l64 = np_models.llm_logits(cfg, dict(params), seq, positions=range(127, 144))
+    srt = np.sort(l64, -1)
+    gaps = (srt[..., -1] - srt[..., -2]).T
+    assert_tokens_match(g_h, g_c, gaps, 2 * err)
 
 
 def test_pool_returns_to_baseline_after_runs(hip_session):

@@ -284,9 +284,23 @@ def test_microbench_shapes_properties(hip):
     d = hip.to_numpy(hip.max(hip.reshape(hip.div(hip.sub(lhs.clone(), rhs), lhs), (1, n * n))))
     assert float(d[0, 0]) < 1e-5
     # bmm [16,1024,1024]: (A B) 1 == A (B 1)
-    A_ = hip.from_numpy(rng.standard_normal((16, 1024, 1024)).astype(np.float32))
-    B_ = hip.from_numpy(rng.standard_normal((16, 1024, 1024)).astype(np.float32))
+    a_np = rng.standard_normal((16, 1024, 1024)).astype(np.float32)
+    b_np = rng.standard_normal((16, 1024, 1024)).astype(np.float32)
+    A_, B_ = hip.from_numpy(a_np), hip.from_numpy(b_np)
     ones = hip.broadcast(hip.from_numpy(np.float32(1).reshape(())), (16, 1024, 1))
-    left = hip.to_numpy(hip.matmul(hip.matmul(A_, B_), ones))
+    prod = hip.matmul(A_, B_)
+    left = hip.to_numpy(hip.matmul(prod, ones))
     right = hip.to_numpy(hip.matmul(A_, hip.matmul(B_, ones)))
-    np.testing.assert_allclose(left, right, rtol=0, atol=1e-3 * 1024 * 32)
+    # both sides against float64, 1e-3 of the scale of the terms summed (sum_k |a| * |sum_n b|, resp. sum_n |(ab)|)
+    a64, b64 = a_np.astype(np.float64), b_np.astype(np.float64)
+    b1 = b64.sum(-1, keepdims=True)
+    exact = a64 @ b1
+    scale_r = np.abs(a64) @ np.abs(b1)
+    assert (np.abs(right - exact) <= 1e-3 * scale_r).all()
+    assert (np.abs(left - exact) <= 1e-3 * scale_r).all()
+    # sampled rows of the product itself in float64: 1e-3 of sum_k |a| |b|
+    full = hip.to_numpy(prod)
+    for bi, r in ((0, 0), (5, 1023), (15, 517), (9, 64)):
+        ex = a64[bi, r] @ b64[bi]
+        sc = np.abs(a64[bi, r]) @ np.abs(b64[bi])
+        assert (np.abs(full[bi, r] - ex) <= 1e-3 * sc).all()
