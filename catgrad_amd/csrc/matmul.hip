@@ -510,6 +510,17 @@ template <int MM> __global__ __launch_bounds__(kThreads) void skinny_kt_wide_res
 // it is used all the same, because its residual store and its norm-applying loads save two launches per layer.
 // Chunks of 2048 values of k when K is a multiple of that, of 1024 when of that (hidden sizes like 1024 or 3072).
 static inline int xreg_trips(uint32_t K) { return K % 2048 == 0 ? 8 : K % 1024 == 0 ? 4 : 0; }
+// Column groups per workgroup of the one-chunk gated kernel: as many as leave about two workgroups per compute unit
+// (env CG_XREG_ITERS=n forces n, for measurements).
+static inline uint32_t xreg_cols_iters(uint64_t groups) {
+    static const int forced = [] {
+        const char *e = getenv("CG_XREG_ITERS");
+        return e ? atoi(e) : 0;
+    }();
+    if (forced > 0) return (uint32_t)forced;
+    const uint64_t it = groups / 512;
+    return (uint32_t)(it < 1 ? 1 : it > 4 ? 4 : it);
+}
 static inline bool xreg_narrow(uint32_t M, uint32_t K) { return M >= 1 && M <= 4 && xreg_trips(K) != 0; }
 constexpr int kMaxGroup = 4;
 struct MmGroup {
@@ -742,6 +753,116 @@ __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_group_norm_kerne
     uint32_t bx;
     const uint32_t p = group_problem(g, bx);
     skinny_kt_mfma_xreg_body<4, 1, false, false, true, TRIPS>(g.p[p], bx, 0, nullptr, 0, nullptr, &nf);
+}
+
+// The gated pair when K is exactly one chunk (TRIPS * 256: the hidden size of the model): the workgroup asks for its
+// share of the activations (and of gamma, and of the row sums of an RMS norm) ONCE and walks `iters` consecutive
+// groups of four columns with them, the next group's weights always on their way while the current group is
+// multiplied, reduced and stored.  Measured on the 1B-shape decode step: the activation, gamma and partial-sum loads
+// of a workgroup that owns a single column group cost a fifth of the kernel's time although they all hit in L2 (they
+// are three quarters as many bytes again as the weights); four groups per workgroup take 29.5 instead of 34.3 us for
+// the 128 MiB of gate + up, more leave too few workgroups in flight.  For q / k / v and o (a quarter of the columns)
+// one group per workgroup stays the fastest.  Weights are read with the non-temporal hint.
+// M <= 4, batch folded away (one batch entry).  Epilogues as in skinny_kt_mfma_xreg_body.
+template <bool NORM, int TRIPS>
+__global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_cols_gated_kernel(const MmArgs a, const uint32_t *second, uint32_t one,
+                                                                                  uint32_t iters, const NormFuse nf) {
+    static_assert(TRIPS == 8 || TRIPS == 4, "chunks of 2048 or 1024");
+    const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    const uint32_t j = lane % 4, b = lane / 4;
+    const uint32_t kb = wave * (TRIPS * 64) + b * 4; // this lane's k: kb + 64 t
+    const uint32_t *xrow = a.A + (int64_t)min(j, a.M - 1) * a.a_sm;
+    float4v xr[TRIPS];
+#pragma unroll
+    for (int t = 0; t < TRIPS; t++) xr[t] = *reinterpret_cast<const float4v *>(xrow + kb + 64 * t);
+    float pv[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    float4v gm[NORM ? TRIPS : 1];
+    if constexpr (NORM) {
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const uint32_t i = threadIdx.x + u * kThreads;
+            if (i < nf.blocks * 4) pv[u] = nf.partials[i];
+        }
+#pragma unroll
+        for (int t = 0; t < TRIPS; t++) gm[t] = *reinterpret_cast<const float4v *>(nf.gamma + kb + 64 * t);
+    }
+    __shared__ float part[2][4][32];
+    __shared__ float nsum[4][4];
+    const uint32_t groups = (a.N + 3) / 4;
+    float4v wg[TRIPS], wu[TRIPS]; // the group's four columns of the two weight matrices
+    auto ask = [&](float4v (&w)[TRIPS], const uint32_t *base, uint32_t n0) {
+        const uint32_t *row = base + (int64_t)min(n0 + j, a.N - 1) * a.b_sn + kb;
+#pragma unroll
+        for (int t = 0; t < TRIPS; t++) w[t] = __builtin_nontemporal_load(reinterpret_cast<const float4v *>(row + 64 * t));
+    };
+    auto multiply = [&](float4v &sum, const float4v (&w)[TRIPS]) {
+#pragma unroll
+        for (int t = 0; t < TRIPS; t++) {
+            sum = __builtin_amdgcn_mfma_f32_4x4x1f32(xr[t][0], w[t][0], sum, 0, 0, 0);
+            sum = __builtin_amdgcn_mfma_f32_4x4x1f32(xr[t][1], w[t][1], sum, 0, 0, 0);
+            sum = __builtin_amdgcn_mfma_f32_4x4x1f32(xr[t][2], w[t][2], sum, 0, 0, 0);
+            sum = __builtin_amdgcn_mfma_f32_4x4x1f32(xr[t][3], w[t][3], sum, 0, 0, 0);
+        }
+    };
+    const uint32_t first_grp = blockIdx.x * iters;
+    if (first_grp >= groups) return; // the same for every thread of the workgroup
+    ask(wg, a.B, first_grp * 4);
+    if constexpr (NORM) {
+        // (x / d * gamma) . w = ((x * gamma) . w) / d: gamma goes in once, while the first weights are on their way; the row
+        // sums of squares are put together from the partial sums, always in the same order
+#pragma unroll
+        for (int t = 0; t < TRIPS; t++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) xr[t][e] = asf(apply<kMul, true>(asu(xr[t][e]), asu(gm[t][e]), 0, nullptr));
+        float s = 0.0f;
+#pragma unroll
+        for (int u = 0; u < 8; u++) s += pv[u];
+        for (uint32_t i = threadIdx.x + 8 * kThreads; i < nf.blocks * 4; i += kThreads) s += nf.partials[i];
+#pragma unroll
+        for (int sh = 32; sh >= 4; sh >>= 1) s += __shfl_xor(s, sh);
+        if (lane < 4) nsum[wave][lane] = s;
+    }
+    uint32_t divisor = 0;
+    for (uint32_t it = 0; it < iters; it++) {
+        const uint32_t grp = first_grp + it;
+        if (grp >= groups) break;
+        const uint32_t n0 = grp * 4;
+        float4v acc_g = {0.f, 0.f, 0.f, 0.f}, acc_u = {0.f, 0.f, 0.f, 0.f};
+        ask(wu, second, n0);
+        multiply(acc_g, wg);
+        if (it + 1 < iters && grp + 1 < groups) ask(wg, a.B, n0 + 4); // on its way through the rest of this group
+        multiply(acc_u, wu);
+        float (*pt)[32] = part[it & 1];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float vg = acc_g[i], vu = acc_u[i];
+#pragma unroll
+            for (int s = 32; s >= 4; s >>= 1) {
+                vg += __shfl_xor(vg, s);
+                vu += __shfl_xor(vu, s);
+            }
+            if (lane < 4) {
+                pt[wave][i * 4 + j] = vg;
+                pt[wave][16 + i * 4 + j] = vu;
+            }
+        }
+        __syncthreads(); // (the buffer written two groups ago was read before the barrier of the group in between)
+        if (threadIdx.x < 16) {
+            const uint32_t t = threadIdx.x, m = t / 4, col = n0 + t % 4;
+            uint32_t gv = asu((pt[0][t] + pt[1][t]) + (pt[2][t] + pt[3][t]));
+            uint32_t uv = asu((pt[0][16 + t] + pt[1][16 + t]) + (pt[2][16 + t] + pt[3][16 + t]));
+            if constexpr (NORM) {
+                if (it == 0) divisor = norm_divisor(nf, (nsum[0][m] + nsum[1][m]) + (nsum[2][m] + nsum[3][m]));
+                gv = apply<kDiv, true>(gv, divisor, 0, nullptr);
+                uv = apply<kDiv, true>(uv, divisor, 0, nullptr);
+            }
+            // the ops of the deferred program, in its order
+            const uint32_t e = apply<kExp, true>(apply<kNeg, true>(gv, 0, 0, nullptr), 0, 0, nullptr);
+            const uint32_t sg = apply<kDiv, true>(one, apply<kAdd, true>(one, e, 0, nullptr), 0, nullptr);
+            const uint32_t r = apply<kMul, true>(apply<kMul, true>(gv, sg, 0, nullptr), uv, 0, nullptr);
+            if (col < a.N && m < a.M) a.C[(uint64_t)m * a.N + col] = r;
+        }
+    }
 }
 
 // Vectorised skinny kernel for short K (K <= 4*LPC, e.g. q.K^T of a decode step with
@@ -1054,7 +1175,16 @@ int launch_matmul_gated(cg_backend *be, const cg_tensor *x, const cg_tensor *yg,
     const bool short_chunks = xreg_trips(ag.K) == 4; // K a multiple of 1024 but not of 2048
     ProfScope prof(be, CG_K_GEMM_SKINNY, distinct_bytes(x) + distinct_bytes(yg) + distinct_bytes(yu) + distinct_bytes(out));
     const dim3 ggrid((ag.N + 3) / 4);
-    if (nf && short_chunks)
+    if ((int)ag.K == xreg_trips(ag.K) * 256) { // one chunk of k: see skinny_kt_mfma_xreg_cols_body
+        NormFuse none;
+        memset(&none, 0, sizeof none);
+        const uint32_t groups = (ag.N + 3) / 4, iters = xreg_cols_iters(groups);
+        const dim3 cgrid((groups + iters - 1) / iters);
+        if (nf && short_chunks) hipLaunchKernelGGL((skinny_kt_mfma_xreg_cols_gated_kernel<true, 4>), cgrid, dim3(kThreads), 0, be->stream, ag, au.B, one, iters, *nf);
+        else if (nf) hipLaunchKernelGGL((skinny_kt_mfma_xreg_cols_gated_kernel<true, 8>), cgrid, dim3(kThreads), 0, be->stream, ag, au.B, one, iters, *nf);
+        else if (short_chunks) hipLaunchKernelGGL((skinny_kt_mfma_xreg_cols_gated_kernel<false, 4>), cgrid, dim3(kThreads), 0, be->stream, ag, au.B, one, iters, none);
+        else hipLaunchKernelGGL((skinny_kt_mfma_xreg_cols_gated_kernel<false, 8>), cgrid, dim3(kThreads), 0, be->stream, ag, au.B, one, iters, none);
+    } else if (nf && short_chunks)
         hipLaunchKernelGGL(skinny_kt_mfma_xreg_gated_norm_kernel<4>, ggrid, dim3(kThreads), 0, be->stream, ag, au.B, one, *nf);
     else if (nf)
         hipLaunchKernelGGL(skinny_kt_mfma_xreg_gated_norm_kernel<8>, ggrid, dim3(kThreads), 0, be->stream, ag, au.B, one, *nf);
