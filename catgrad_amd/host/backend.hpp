@@ -68,41 +68,79 @@ struct Abi {
     }
 };
 
-// `Backend::BackendTensor`: Clone = retain, Drop = release.
+// What a `Tensor` needs from a term that is being recorded (graph.hpp): a tensor that stands for a wire of such a
+// term has no handle, only the wire's number.
+struct WireTable {
+    virtual ~WireTable() = default;
+    // `x.clone()` in the DSL: a Copy operation with one source and two targets (the numbers of the two new wires)
+    virtual std::pair<int, int> copy(int wire) = 0;
+    virtual Shape shape_of(int wire) const = 0;
+    virtual cg_dtype dtype_of(int wire) const = 0;
+};
+
+// `Backend::BackendTensor`: Clone = retain, Drop = release.  While a term is being recorded (graph.hpp) a Tensor can
+// also stand for a wire of that term: copying it then records a Copy operation, as `Var::clone` does in the DSL.
 class Tensor {
   public:
     Tensor() = default;
     Tensor(const Abi *abi, cg_tensor *h) : abi_(abi), h_(h) {}
-    Tensor(const Tensor &o) : abi_(o.abi_), h_(o.h_) {
+    Tensor(WireTable *wires, int wire) : wires_(wires), wire_(wire) {}
+    Tensor(const Tensor &o) : abi_(o.abi_), h_(o.h_), wires_(o.wires_) {
         if (h_) abi_->cg_tensor_retain(h_);
+        if (wires_ && o.wire_ >= 0) {
+            const std::pair<int, int> two = wires_->copy(o.wire_);
+            o.wire_ = two.first;
+            wire_ = two.second;
+        }
     }
-    Tensor(Tensor &&o) noexcept : abi_(o.abi_), h_(o.h_) { o.h_ = nullptr; }
+    Tensor(Tensor &&o) noexcept : abi_(o.abi_), h_(o.h_), wires_(o.wires_), wire_(o.wire_) {
+        o.h_ = nullptr;
+        o.wire_ = -1;
+    }
     Tensor &operator=(Tensor o) noexcept {
         std::swap(abi_, o.abi_);
         std::swap(h_, o.h_);
+        std::swap(wires_, o.wires_);
+        std::swap(wire_, o.wire_);
         return *this;
     }
     ~Tensor() {
         if (h_) abi_->cg_tensor_release(h_);
     }
-    explicit operator bool() const { return h_ != nullptr; }
+    explicit operator bool() const { return h_ != nullptr || wire_ >= 0; }
     cg_tensor *get() const { return h_; }
     cg_tensor *into_raw() { // hands the reference to a consuming ABI call
         cg_tensor *h = h_;
         h_ = nullptr;
         return h;
     }
+    bool is_wire() const { return wire_ >= 0; }
+    int take_wire() { // the wire is consumed by the operation being recorded
+        const int w = wire_;
+        wire_ = -1;
+        return w;
+    }
     Shape shape() const { // BackendTensorOps::shape
+        if (wire_ >= 0) return wires_->shape_of(wire_);
         Shape s(abi_->cg_tensor_rank(h_));
         if (!s.empty()) abi_->cg_tensor_shape(h_, s.data());
         return s;
     }
-    cg_dtype dtype() const { return abi_->cg_tensor_dtype(h_); }
-    size_t numel() const { return abi_->cg_tensor_numel(h_); }
+    cg_dtype dtype() const { return wire_ >= 0 ? wires_->dtype_of(wire_) : abi_->cg_tensor_dtype(h_); }
+    size_t numel() const {
+        if (wire_ >= 0) {
+            size_t n = 1;
+            for (size_t d : wires_->shape_of(wire_)) n *= d;
+            return n;
+        }
+        return abi_->cg_tensor_numel(h_);
+    }
 
   private:
     const Abi *abi_ = nullptr;
     cg_tensor *h_ = nullptr;
+    WireTable *wires_ = nullptr;
+    mutable int wire_ = -1;
 };
 
 class Backend {

@@ -181,21 +181,37 @@ inline std::vector<Value> tensor_op(Backend &b, const Op &op, std::vector<Value>
     throw InterpreterError("unknown tensor op");
 }
 
+// What the interpreter hands operations to while a term is being recorded instead of run (graph.hpp).
+struct OpRecorder {
+    virtual ~OpRecorder() = default;
+    virtual std::vector<Value> record_op(const Op &op, std::vector<Value> args) = 0;
+    virtual Tensor record_param(const std::string &path, const Tensor &stored) = 0;
+};
+
 // `Interpreter<B>` (interpreter/interpreter.rs:13-59): backend + parameters.
 class Interpreter {
   public:
     Interpreter(const std::string &library, int device) : backend(library, device) {}
     Backend backend;
     std::map<std::string, Tensor> parameters; // `Parameters<B>`
+    OpRecorder *recorder = nullptr; // set: operations are recorded as a term, not run
+    // 0: operations run as the DSL issues them; 1: a forward pass is recorded and run in the layers of the reference's
+    // evaluator (graph.hpp); 2: recorded, then run in the order of recording (the lifetime model of 1, the order of 0)
+    int schedule = 0;
 
     // `Load`: parameters.get(path).clone()
     Tensor param(const std::string &path) {
         auto it = parameters.find(path);
         if (it == parameters.end()) throw InterpreterError("MissingParameter: " + path);
+        if (recorder) return recorder->record_param(path, it->second);
         return it->second;
     }
+    std::vector<Value> run(const Op &op, std::vector<Value> args) {
+        if (recorder) return recorder->record_op(op, std::move(args));
+        return tensor_op(backend, op, std::move(args));
+    }
     Tensor run1(const Op &op, std::vector<Value> args) {
-        auto r = tensor_op(backend, op, std::move(args));
+        auto r = run(op, std::move(args));
         return std::move(r[0].tensor);
     }
 };

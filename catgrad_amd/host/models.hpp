@@ -8,6 +8,7 @@
 
 #include <chrono>
 
+#include "graph.hpp"
 #include "nn.hpp"
 
 namespace cgh {
@@ -30,9 +31,42 @@ class LlmModel {
     const LlmConfig &config() const { return c_; }
     std::string root() const { return c_.arch == 0 ? "llama" : "qwen3"; }
 
+    // `Interpreter::run(term, inputs)` for the model's term.  With Interpreter::schedule 0 the operations run as the
+    // graph builder issues them; with 1 the pass is first recorded as a term and then evaluated in the layers of the
+    // reference's evaluator, with its value map (graph.hpp); with 2 recorded and evaluated in the order of recording.
+    ForwardOut forward(Tensor x, Tensor in_k, Tensor in_v, size_t max_positions, Tensor *logits = nullptr) {
+        if (i_.schedule == 0 || i_.recorder) return def(std::move(x), std::move(in_k), std::move(in_v), max_positions, logits);
+        Term term;
+        Tensor sx = term.source(x.shape(), x.dtype()), sk = term.source(in_k.shape(), in_k.dtype()),
+               sv = term.source(in_v.shape(), in_v.dtype());
+        ForwardOut o;
+        Tensor lg;
+        i_.recorder = &term;
+        try {
+            o = def(std::move(sx), std::move(sk), std::move(sv), max_positions, logits ? &lg : nullptr);
+        } catch (...) {
+            i_.recorder = nullptr;
+            throw;
+        }
+        i_.recorder = nullptr;
+        std::vector<Tensor> outs;
+        outs.push_back(std::move(o.tokens));
+        outs.push_back(std::move(o.out_k));
+        outs.push_back(std::move(o.out_v));
+        if (logits) outs.push_back(std::move(lg));
+        term.finish(std::move(outs));
+        std::vector<Tensor> in;
+        in.push_back(std::move(x));
+        in.push_back(std::move(in_k));
+        in.push_back(std::move(in_v));
+        std::vector<Tensor> r = term.run(i_, std::move(in), i_.schedule == 2);
+        if (logits) *logits = std::move(r[3]);
+        return {std::move(r[0]), std::move(r[1]), std::move(r[2])};
+    }
+
     // `DynModule::def` for inputs [x u32[B,S], in_k, in_v f32[L,B,kvH,P,hd], Nat(max_positions)]
     // `logits`, when given, receives a clone of the lm_head output (for parity checks).
-    ForwardOut forward(Tensor x, Tensor in_k, Tensor in_v, size_t max_positions, Tensor *logits = nullptr) {
+    ForwardOut def(Tensor x, Tensor in_k, Tensor in_v, size_t max_positions, Tensor *logits = nullptr) {
         using namespace nn;
         I &i = i_;
         const std::string model = root() + ".model";

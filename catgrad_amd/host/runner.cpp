@@ -93,6 +93,52 @@ int cgm_set_config(cgm_session *s, int arch, size_t hidden_size, size_t num_hidd
     });
 }
 
+int cgm_set_schedule(cgm_session *s, int schedule) {
+    return guarded([&] {
+        if (schedule < 0 || schedule > 2) throw InterpreterError("unknown schedule");
+        s->interp->schedule = schedule;
+    });
+}
+
+int cgm_cond_kat(cgm_session *s, float x, float c, float *out) {
+    return guarded([&] {
+        Interpreter &i = *s->interp;
+        auto body = [&](Tensor tx, Tensor tc) {
+            Tensor keep = tx; // `x.clone()`: the term also returns x itself in the reference's test
+            (void)keep;
+            return ops::cond(
+                i, std::move(tc),
+                [&](std::vector<Tensor> a) { return std::vector<Tensor>{ops::add(i, a[0], a[0])}; },
+                [&](std::vector<Tensor> a) { return std::vector<Tensor>{std::move(a[0])}; },
+                std::vector<Tensor>{std::move(tx)});
+        };
+        Tensor tx = i.backend.ndarray_from_vec_f32(&x, 1, Shape{}), tc = i.backend.ndarray_from_vec_f32(&c, 1, Shape{});
+        Tensor res;
+        if (i.schedule == 0) {
+            res = std::move(body(std::move(tx), std::move(tc))[0]);
+        } else {
+            Term term;
+            Tensor sx = term.source(Shape{}, CG_F32), sc = term.source(Shape{}, CG_F32);
+            i.recorder = &term;
+            std::vector<Tensor> r;
+            try {
+                r = body(std::move(sx), std::move(sc));
+            } catch (...) {
+                i.recorder = nullptr;
+                throw;
+            }
+            i.recorder = nullptr;
+            term.finish(std::move(r));
+            std::vector<Tensor> in;
+            in.push_back(std::move(tx));
+            in.push_back(std::move(tc));
+            res = std::move(term.run(i, std::move(in), i.schedule == 2)[0]);
+        }
+        std::vector<uint32_t> v = i.backend.to_vec_bits(std::move(res));
+        memcpy(out, v.data(), 4);
+    });
+}
+
 int cgm_generate(cgm_session *s, const uint32_t *prompt, size_t B, size_t S, size_t steps, size_t max_positions,
                  uint32_t *out_tokens, double *stats4) {
     return guarded([&] {

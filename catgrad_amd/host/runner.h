@@ -29,6 +29,16 @@ int cgm_set_config(cgm_session *s, int arch, size_t hidden_size, size_t num_hidd
                    size_t num_key_value_heads, size_t head_dim, size_t intermediate_size, size_t vocab_size,
                    float rms_norm_eps, float rope_theta, int tie_word_embeddings);
 
+/* Order of evaluation of the model runs and of cgm_cond_kat: 0 = the operations run as the graph builder issues
+ * them; 1 = every run is first recorded as a term and evaluated in the layers of the reference's evaluator
+ * (catgrad/src/abstract_interpreter/eval.rs:38-66, catgrad/src/ssa/mod.rs:24-76) with its move / clone value map;
+ * 2 = recorded and evaluated in the order of recording. */
+int cgm_set_schedule(cgm_session *s, int schedule);
+
+/* The term of catgrad/tests/test_if.rs: cond(c, then: x + x, else: x, [x]) on rank-0 f32 tensors; *out receives
+ * the result's value. */
+int cgm_cond_kat(cgm_session *s, float x, float c, float *out);
+
 /* Prefill + `steps` greedy decode runs.  out_tokens: (steps+1) x B ids.  stats:
  * [prefill_s, decode_s, backend calls in prefill, backend calls in decode]. */
 int cgm_generate(cgm_session *s, const uint32_t *prompt, size_t B, size_t S, size_t steps, size_t max_positions,

@@ -36,6 +36,8 @@ def _host():
             "cgm_clear_params": (C.c_int, [P]),
             "cgm_load_safetensors": (C.c_int, [P, C.POINTER(C.c_char_p), SZ, C.POINTER(C.c_double)]),
             "cgm_set_config": (C.c_int, [P, C.c_int] + [SZ] * 7 + [C.c_float, C.c_float, C.c_int]),
+            "cgm_set_schedule": (C.c_int, [P, C.c_int]),
+            "cgm_cond_kat": (C.c_int, [P, C.c_float, C.c_float, C.POINTER(C.c_float)]),
             "cgm_generate": (C.c_int, [P, P, SZ, SZ, SZ, SZ, P, C.POINTER(C.c_double)]),
             "cgm_generate_with_logits": (C.c_int, [P, P, SZ, SZ, SZ, SZ, P, C.POINTER(C.c_double), P]),
             "cgm_forward": (C.c_int, [P, P, SZ, SZ, SZ, P, P]),
@@ -190,6 +192,18 @@ class Session:
             config.num_attention_heads, config.num_key_value_heads, config.hd, config.intermediate_size,
             config.vocab_size, config.rms_norm_eps, config.rope_theta, int(config.tie_word_embeddings)))
         self.config = config
+
+    def set_schedule(self, schedule: int):
+        """0: operations run as the graph builder issues them (default); 1: every model run is recorded as a term and
+        evaluated in the layers of the reference's evaluator (eval.rs:38-66, ssa/mod.rs:24-76) with its move / clone
+        value map; 2: recorded, evaluated in the order of recording."""
+        self._check(self._lib.cgm_set_schedule(self._s, schedule))
+
+    def cond_kat(self, x: float, c: float) -> float:
+        """cond(c, then: x + x, else: x, [x]) on rank-0 tensors (catgrad/tests/test_if.rs)."""
+        out = C.c_float()
+        self._check(self._lib.cgm_cond_kat(self._s, x, c, C.byref(out)))
+        return float(out.value)
 
     def generate(self, prompt: np.ndarray, steps: int, max_positions: int | None = None, want_logits: bool = False):
         """Prefill + `steps` greedy decode runs.  Returns (tokens [(steps+1), B], stats dict); with `want_logits`
