@@ -33,10 +33,18 @@ HBM_PEAK = 8.0e12       # B/s, MI355X HBM3E
 MFMA_F32_PEAK = 157.3e12  # flop/s, MI355X dense f32 matrix
 
 
-# HBM bytes per mfma_gemm_kernel launch of this workload's prefill, from rocprofv3 FETCH_SIZE / WRITE_SIZE passes
-# scaled by a copy kernel of known size (profiles/mfma_gemm_llama1b_prefill_pmc.txt); counters cannot be read
-# from inside this process, so the figure is carried here and only reported for the profiled shape.
-MFMA_GEMM_TRAFFIC_PER_LAUNCH = 0.691e9
+def profiled_traffic():
+    """HBM bytes per launch of the dominant kernel (mfma_gemm_kernel) on the config-5 prefill, as the rocprofv3
+    FETCH_SIZE / WRITE_SIZE passes measured them: read from the committed summary (its line
+    `traffic_bytes_per_launch: <n>`), not measured by this process (counters need the profiler)."""
+    path = os.path.join(ROOT, "profiles", "mfma_gemm_llama1b_prefill_pmc.txt")
+    try:
+        for line in open(path):
+            if line.startswith("traffic_bytes_per_launch:"):
+                return float(line.split(":", 1)[1].split()[0])
+    except OSError:
+        pass
+    return None
 
 
 def micro_bench(iters=20):
@@ -47,7 +55,7 @@ def micro_bench(iters=20):
     rng = np.random.default_rng(0)
     out = {}
 
-    def run(name, cls, fn, unit):
+    def run(name, cls, fn, unit, launches_per_call=1):
         for _ in range(3):
             fn()
         be.sync()
@@ -57,6 +65,7 @@ def micro_bench(iters=20):
             fn()
         n, ms, work = be.profile_read(cls, reset=True)
         be.profile_enable(cls, 0)
+        n = n / launches_per_call      # an op of several launches (the two halves of a concat): time and bytes of all
         per = max(ms / max(n, 1) * 1e-3, 1e-12)
         rate = work / max(n, 1) / per
         peak = MFMA_F32_PEAK if unit == "TFLOP/s" else HBM_PEAK
@@ -81,16 +90,35 @@ def micro_bench(iters=20):
     y = be.from_numpy(rng.standard_normal((16, 1024, 1024), dtype=np.float32))
     run("bmm_f32_16x1024x1024x1024", A.K_GEMM_MFMA, lambda: be.matmul(x, y), "TFLOP/s")
     del x, y
+    # the strided / indexing kernels of the path: a materialised transpose, concat along the outermost and the innermost
+    # axis, the embedding gather of the 1B-shape prefill and a sum over a non-last axis (8 bytes per element moved,
+    # 4 per element reduced)
+    a = be.from_numpy(rng.standard_normal((n, n), dtype=np.float32))
+    run("transpose_8192x8192_materialised", A.K_ELEMENTWISE,
+        lambda: be.realize(be.reshape(be.transpose(a, 0, 1), (n * n,))), "GB/s")
+    run("sum_axis0_8192x8192", A.K_REDUCE, lambda: be.realize(be.sum(be.transpose(a, 0, 1))), "GB/s")
+    h = be.from_numpy(rng.standard_normal((n // 2, n), dtype=np.float32))
+    g = be.from_numpy(rng.standard_normal((n // 2, n), dtype=np.float32))
+    hv, gv = be.slice(h, 1, 0, n // 2), be.slice(g, 1, 0, n // 2)     # [4096, 4096] views of row pitch 8192
+    run("concat_dim0_2x4096x8192", A.K_ELEMENTWISE, lambda: be.concat(h, g, 0), "GB/s", launches_per_call=2)
+    # along the last axis the result stays a deferred two-part view until something needs memory; then two strided copies
+    run("concat_dim1_2x4096x4096", A.K_ELEMENTWISE, lambda: be.realize(be.concat(hv, gv, 1)), "GB/s", launches_per_call=2)
+    del a, h, g, hv, gv
+    wte = be.from_numpy(rng.standard_normal((128256, 2048), dtype=np.float32))
+    ids = be.from_numpy(rng.integers(0, 128256, size=(8192,), dtype=np.uint32))
+    run("index_embedding_128256x2048_8192ids", A.K_GATHER, lambda: be.index(wte, 0, ids), "GB/s")
+    del wte, ids
     be.pool_trim()
     return out
 
 
-def cpu_baseline(cfg, params, B, sample_prefill, sample_decode, seed):
-    """The oracle on this box's host cores (it is single-threaded, like NdArrayBackend) on a
-    bounded sample of the workload: same model, a short prompt and few steps, at the
-    batch size the reference's own CLI uses (1; catgrad-llm/examples/llama/main.rs:947-951).
-    With batch 4 one forward pass alone takes about a minute of CPU time, most of it
-    materialising the batch-broadcast weight views."""
+def cpu_baseline(cfg, params, B, sample_prefill, sample_decode, seed, gpu_tokens=None):
+    """The oracle on this box's host cores (it is single-threaded, like NdArrayBackend) on a bounded sample of the
+    workload: the same model at the measured batch size, a short prompt and few steps.  A forward pass of the oracle
+    costs about the same whatever its token count (most of it is materialising the batch-broadcast weight views, as
+    ndarray.rs:553-559 does), so the per-token rates of the sample overstate what the full 2048 + 256 run would
+    reach per token of prefill and understate nothing: they are reported as measured, with the sample named.
+    gpu_tokens: what HipBackend generated for the same sample prompt; compared token for token."""
     from catgrad_amd.runner import Session
 
     lib = os.path.join(ROOT, "oracle", "liboracle.so")
@@ -98,19 +126,28 @@ def cpu_baseline(cfg, params, B, sample_prefill, sample_decode, seed):
         return None
     s = Session(lib)
     s.load_model(cfg, params=params)
-    prompt = np.random.default_rng(seed).integers(0, cfg.vocab_size, size=(B, sample_prefill), dtype=np.uint32)
+    prompt = sample_prompt(cfg, B, sample_prefill, seed)
     t0 = time.perf_counter()
-    _, st = s.generate(prompt, steps=sample_decode, max_positions=sample_prefill + sample_decode)
+    toks, st = s.generate(prompt, steps=sample_decode, max_positions=sample_prefill + sample_decode)
     wall = time.perf_counter() - t0
     s.close()
     tokens = B * (sample_prefill + sample_decode)
-    return {
+    out = {
         "value": round(tokens / (st["prefill_s"] + st["decode_s"]), 3), "unit": "tok/s", "cores": 1,
         "host_cores": os.cpu_count(), "kind": "port",
         "sample": f"same model, batch {B}; prefill {sample_prefill} tokens/seq + {sample_decode} decode steps "
                   f"({wall:.1f} s of CPU work); prefill {B * sample_prefill / st['prefill_s']:.2f} tok/s, "
-                  f"decode {B * sample_decode / max(st['decode_s'], 1e-9):.3f} tok/s",
+                  f"decode {B * sample_decode / max(st['decode_s'], 1e-9):.3f} tok/s; a pass costs about the same for any "
+                  f"token count, so the full-size run would be about {st['prefill_s']:.0f} s of prefill per "
+                  f"{B * sample_prefill} tokens scaled by the GEMM work, and {st['decode_s'] / max(sample_decode, 1):.0f} s per decode step",
     }
+    if gpu_tokens is not None:
+        out["tokens_equal_gpu"] = bool((toks == gpu_tokens).all())
+    return out
+
+
+def sample_prompt(cfg, B, S, seed):
+    return np.random.default_rng(seed + 1).integers(0, cfg.vocab_size, size=(B, S), dtype=np.uint32)
 
 
 def main():
@@ -118,13 +155,19 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=3)
     ap.add_argument("--warmup", type=int, default=1)
-    ap.add_argument("--batch", type=int, default=4)
-    ap.add_argument("--prefill", type=int, default=2048)
-    ap.add_argument("--decode", type=int, default=256)
+    ap.add_argument("--config", type=int, default=5, choices=[3, 4, 5],
+                    help="BASELINE.json configs index + 1: 5 = Llama-3.2-1B shape, batch 4, 2048 + 256 (the metric's "
+                         "configuration, default); 4 = Qwen3-0.6B shape, batch 1, 1024 + 128; 3 = SmolLM2-135M shape, "
+                         "batch 1, prefill 512 (+ 16 decode steps so that the decode figures exist)")
+    ap.add_argument("--batch", type=int, default=None)
+    ap.add_argument("--prefill", type=int, default=None)
+    ap.add_argument("--decode", type=int, default=None)
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-micro", action="store_true")
-    ap.add_argument("--cpu-sample", type=int, nargs=3, default=[1, 4, 1], metavar=("BATCH", "PREFILL", "DECODE"))
+    ap.add_argument("--cpu-sample", type=int, nargs=3, default=None, metavar=("BATCH", "PREFILL", "DECODE"),
+                    help="the CPU baseline's sample (default: the measured batch, prefill 8, 1 decode step)")
+    ap.add_argument("--micro-only", action="store_true", help="only the op micro-benchmarks (one JSON line of their own)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="only run a strided copy of known size (268435456 B read + 268435456 B written per launch), "
                          "the yardstick for scaling rocprofv3 FETCH_SIZE / WRITE_SIZE")
@@ -146,17 +189,30 @@ def main():
                           "write_bytes": 8192 * 8192 * 4}))
         return
 
+    if args.micro_only:
+        print(json.dumps({"micro": micro_bench()}))
+        return
+
     import torch  # device-wide synchronisation around the timed region
 
     from catgrad_amd import _abi as A
-    from catgrad_amd.runner import LLAMA_3_2_1B, Session, random_params
+    from catgrad_amd.runner import LLAMA_3_2_1B, QWEN3_0_6B, SMOLLM2_135M, Session, random_params
 
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; HipBackend has no CPU fallback.", file=sys.stderr)
         sys.exit(1)
 
-    cfg = LLAMA_3_2_1B
-    B, S, T = args.batch, args.prefill, args.decode
+    cfg, dB, dS, dT, cfg_name = {
+        5: (LLAMA_3_2_1B, 4, 2048, 256, "Llama-3.2-1B-shape decoder (hidden 2048, 16 layers, 32/8 heads, MLP 8192, vocab 128256, "
+                                        "rope theta 500000, tied lm_head)"),
+        4: (QWEN3_0_6B, 1, 1024, 128, "Qwen3-0.6B-shape decoder (hidden 1024, 28 layers, 16/8 heads of 128, QK-norm, MLP 3072, "
+                                      "vocab 151936, tied lm_head)"),
+        3: (SMOLLM2_135M, 1, 512, 16, "SmolLM2-135M-shape decoder (hidden 576, 30 layers, 9/3 heads, MLP 1536, vocab 49152, "
+                                      "tied lm_head)"),
+    }[args.config]
+    B = args.batch if args.batch is not None else dB
+    S = args.prefill if args.prefill is not None else dS
+    T = args.decode if args.decode is not None else dT
     params = list(random_params(cfg, args.seed))
     sess = Session()
     t_up = time.perf_counter()
@@ -223,9 +279,9 @@ def main():
         "dtype": "f32",
         "data": "synthetic",
         "config": {
-            "workload": f"Llama-3.2-1B-shape decoder (hidden 2048, 16 layers, 32/8 heads, MLP 8192, vocab 128256, "
-                        f"rope theta 500000, tied lm_head), random-init f32, batch {B}, prefill {S} random tokens, "
+            "workload": f"{cfg_name}, random-init f32, batch {B}, prefill {S} random tokens, "
                         f"{T} greedy decode steps with KV cache",
+            "baseline_config": args.config,
             "global_batch": B, "seq_len": S, "decode_steps": T, "parallelism": "single GPU",
         },
         "prefill_tok_s": round(K * B * S / pp_s, 2),
@@ -238,7 +294,9 @@ def main():
             "kernel": "mfma_gemm_kernel (f32 v_mfma_f32_32x32x2; 256x256x32 tiles, 128x128 and 128x64 for small N)",
             "bound": "mfma", "achieved": round(mfma_rate / 1e12, 3), "peak": MFMA_F32_PEAK / 1e12, "unit": "TFLOP/s",
             "frac": round(mfma_rate / MFMA_F32_PEAK, 4),
-            "traffic": MFMA_GEMM_TRAFFIC_PER_LAUNCH if (B, S) == (4, 2048) else None,
+            # from the committed rocprofv3 counter summary of this very workload (null for any other)
+            "traffic": profiled_traffic() if (args.config, B, S) == (5, 4, 2048) else None,
+            "traffic_source": "profiles/mfma_gemm_llama1b_prefill_pmc.txt" if (args.config, B, S) == (5, 4, 2048) else None,
             "launches_timed": n_m, "avg_launch_ms": round(ms_m / max(n_m, 1), 4),
             "flop_per_launch_avg": flop_m / max(n_m, 1),
         },
@@ -259,16 +317,23 @@ def main():
                 "launches_timed": n_s, "avg_launch_us": round(ms_s / max(n_s, 1) * 1e3, 3),
             },
         },
+        # the first decoded tokens of the timed run, for eyeballing across builds; what checks tokens is the CPU sample
+        # below (cpu_baseline.tokens_equal_gpu) and the full-size parity tests (tests/test_hip_config5.py)
         "first_tokens": tokens[:2].tolist() if tokens is not None else None,
         # not part of `value`: the one-off upload of the weights from pageable host memory through the
         # backend's pinned staging buffers (the PCIe-inclusive cost of a cold start)
         "weights_upload": {"bytes": weight_bytes, "seconds": round(t_up, 3), "GB_per_s": round(weight_bytes / t_up / 1e9, 2)},
     }
+    cpu_sample = args.cpu_sample or [B, 8, 1]
+    gpu_sample_tokens = None
+    if not args.no_cpu_baseline:   # the CPU sample's prompt through the GPU path too: its tokens are compared below
+        gpu_sample_tokens, _ = sess.generate(sample_prompt(cfg, cpu_sample[0], cpu_sample[1], args.seed), steps=cpu_sample[2],
+                                             max_positions=cpu_sample[1] + cpu_sample[2])
     sess.close()
     if not args.no_micro:
         result["micro"] = micro_bench()
     if not args.no_cpu_baseline:
-        result["cpu_baseline"] = cpu_baseline(cfg, params, *args.cpu_sample, args.seed)
+        result["cpu_baseline"] = cpu_baseline(cfg, params, *cpu_sample, args.seed, gpu_tokens=gpu_sample_tokens)
     print(json.dumps(result))
 
 

@@ -174,6 +174,116 @@ __global__ __launch_bounds__(kBlock) void gather_kernel(const uint32_t *__restri
 
 } // namespace
 
+// ---- copies that transpose ------------------------------------------------------------------------------------------
+// A strided copy whose source is unit-stride along another axis than its destination (the row-major copy of a
+// transposed view: `reshape` of [B, h, S, hd] seen as [B, S, h, hd], ndarray.rs:545-569) would read 4 bytes per 128-byte
+// line with one of the two.  Here a workgroup moves a 64 x 64 tile through LDS: 16-byte loads along the source's
+// unit-stride axis, 16-byte stores along the destination's.  HBM-bound: 8 bytes per element.
+struct TransposeArgs {
+    const uint32_t *src;
+    uint32_t *dst;
+    uint32_t I, T;            // extents of the destination's fast axis (i) and of the source's fast axis (t)
+    int64_t src_is, dst_ts;   // source stride along i, destination stride along t (the other two are 1)
+    uint32_t tiles_i, tiles_t;
+    uint32_t nrest;           // further axes, innermost first
+    uint32_t rd[kMaxOuter];
+    FastDiv rdiv[kMaxOuter];
+    int64_t src_rs[kMaxOuter], dst_rs[kMaxOuter];
+    uint32_t vec;             // 1: every 16-byte access of a whole tile is aligned
+};
+
+__global__ __launch_bounds__(kBlock) void transpose_copy_kernel(const TransposeArgs a) {
+    constexpr int TS = 64, PITCH = TS + 1;
+    __shared__ uint32_t tile[TS][PITCH]; // [i][t]
+    // tiles are walked along diagonals: neighbouring workgroups then differ in BOTH their source rows and their
+    // destination rows, which spreads the strided side of the copy over the memory channels
+    uint32_t blk = blockIdx.x;
+    const uint32_t tt = blk % a.tiles_t;
+    blk /= a.tiles_t;
+    const uint32_t ti = (blk % a.tiles_i + tt) % a.tiles_i;
+    uint32_t rest = blk / a.tiles_i;
+    int64_t so = 0, dofs = 0;
+    for (uint32_t d = 0; d < a.nrest; d++) {
+        const uint32_t q = fastdiv(rest, a.rdiv[d]);
+        const int64_t i = (int64_t)(rest - q * a.rd[d]);
+        rest = q;
+        so += i * a.src_rs[d];
+        dofs += i * a.dst_rs[d];
+    }
+    const uint32_t i0 = ti * TS, t0 = tt * TS;
+    const bool whole = a.vec && i0 + TS <= a.I && t0 + TS <= a.T;
+    const uint32_t q = threadIdx.x % 16, r = threadIdx.x / 16; // a quarter-row of 16-byte pieces, 16 rows per pass
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    if (whole) {
+        u4 v[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) // row i0 + r + 16k of the source, pieces t0 + 4q .. + 3
+            v[k] = __builtin_nontemporal_load(reinterpret_cast<const u4 *>(a.src + so + (int64_t)(i0 + r + 16 * k) * a.src_is + t0 + 4 * q));
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            uint32_t *row = tile[r + 16 * k];
+            row[4 * q] = v[k][0];
+            row[4 * q + 1] = v[k][1];
+            row[4 * q + 2] = v[k][2];
+            row[4 * q + 3] = v[k][3];
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < 4; k++) { // row t0 + r + 16k of the destination, pieces i0 + 4q .. + 3
+            const uint32_t t = r + 16 * k;
+            const u4 o = {tile[4 * q][t], tile[4 * q + 1][t], tile[4 * q + 2][t], tile[4 * q + 3][t]};
+            __builtin_nontemporal_store(o, reinterpret_cast<u4 *>(a.dst + dofs + (int64_t)(t0 + t) * a.dst_ts + i0 + 4 * q));
+        }
+        return;
+    }
+    // ragged or unaligned tile: element by element, still along the fast axis of each side
+    const uint32_t c = threadIdx.x % 64, w = threadIdx.x / 64;
+    for (uint32_t k = w; k < TS; k += 4)
+        if (i0 + k < a.I && t0 + c < a.T) tile[k][c] = a.src[so + (int64_t)(i0 + k) * a.src_is + t0 + c];
+    __syncthreads();
+    for (uint32_t k = w; k < TS; k += 4)
+        if (t0 + k < a.T && i0 + c < a.I) a.dst[dofs + (int64_t)(t0 + k) * a.dst_ts + i0 + c] = tile[c][k];
+}
+
+// Takes a planned copy (a.out, a.in[0]) when it is a transposition worth tiling; kDeclined otherwise.
+static int try_transpose_copy(cg_backend *be, const EwArgs &a) {
+    const EwGeom &g = a.g;
+    if (a.in[0].uniform || a.out.is != 1 || a.in[0].is == 1 || a.in[0].is == 0 || g.nouter < 1) return kDeclined;
+    int td = -1; // the outer axis along which the source is unit-stride
+    for (uint32_t d = 0; d < g.nouter; d++)
+        if (a.in[0].os[d] == 1 && g.od[d] >= 16) td = (int)d;
+    if (td < 0 || g.inner < 16) return kDeclined;
+    TransposeArgs t;
+    memset(&t, 0, sizeof t);
+    t.src = reinterpret_cast<const uint32_t *>(a.in[0].ptr);
+    t.dst = reinterpret_cast<uint32_t *>(const_cast<char *>(a.out.ptr));
+    t.I = g.inner;
+    t.T = g.od[td];
+    t.src_is = a.in[0].is;
+    t.dst_ts = a.out.os[td];
+    if (t.src_is < 0 || t.dst_ts <= 0) return kDeclined;
+    t.tiles_i = (t.I + 63) / 64;
+    t.tiles_t = (t.T + 63) / 64;
+    uint64_t blocks = (uint64_t)t.tiles_i * t.tiles_t;
+    bool vec = reinterpret_cast<uintptr_t>(t.src) % 16 == 0 && reinterpret_cast<uintptr_t>(t.dst) % 16 == 0 && t.src_is % 4 == 0 &&
+               t.dst_ts % 4 == 0;
+    for (uint32_t d = 0; d < g.nouter; d++) {
+        if ((int)d == td) continue;
+        t.rd[t.nrest] = g.od[d];
+        t.rdiv[t.nrest] = make_fastdiv(g.od[d]);
+        t.src_rs[t.nrest] = a.in[0].os[d];
+        t.dst_rs[t.nrest] = a.out.os[d];
+        if (a.in[0].os[d] % 4 || a.out.os[d] % 4) vec = false;
+        blocks *= g.od[d];
+        t.nrest++;
+    }
+    if (blocks == 0 || blocks > 0x7FFFFFFFull) return kDeclined;
+    t.vec = vec ? 1u : 0u;
+    hipLaunchKernelGGL(transpose_copy_kernel, dim3((uint32_t)blocks), dim3(kBlock), 0, be->stream, t);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CG_OK : hip_fail(e, "transposing copy launch");
+}
+
 int launch_elementwise(cg_backend *be, int op, cg_dtype dt, const cg_tensor *out, const cg_tensor *const *ins, int nin) {
     if (int frc = flush_deferred(be)) return frc;
     const cg_tensor *views[4] = {out, nullptr, nullptr, nullptr};
@@ -189,6 +299,10 @@ int launch_elementwise(cg_backend *be, int op, cg_dtype dt, const cg_tensor *out
     double work = distinct_bytes(out);
     for (int k = 0; k < nin; k++) work += distinct_bytes(ins[k]);
     ProfScope prof(be, CG_K_ELEMENTWISE, work);
+    if (op == kCopy && nin == 1) {
+        const int trc = try_transpose_copy(be, a);
+        if (trc != kDeclined) return trc;
+    }
     switch (op) {
 #define CG_EW1(OP) case OP: return launch_by_dtype<OP, 1>(be, dt, a);
 #define CG_EW2(OP) case OP: return launch_by_dtype<OP, 2>(be, dt, a);

@@ -312,7 +312,121 @@ __global__ __launch_bounds__(64) void reduce_segments_final_kernel(const long lo
     if (threadIdx.x == 0) out[row] = acc.result();
 }
 
+// The reduced axis is not the unit-stride one, the innermost of the other axes is (the last axis of a transposed view:
+// a sum over the rows of a row-major matrix).  A lane per output would read 4 bytes per 128-byte line; here the lanes of a
+// wave sit on neighbouring OUTPUTS (16 bytes each when aligned) and every lane walks the reduced axis, so each step of a
+// wave reads one contiguous kilobyte.  The four waves of a workgroup split the steps and meet in LDS; few outputs with a
+// long axis are also cut into segments over grid.y, merged by a second small kernel.  HBM-bound: 4 bytes per element.
+template <int K, bool F, int VEC>
+__global__ __launch_bounds__(kBlock) void reduce_cols_kernel(const RowsArgs a, uint32_t tiles0, uint32_t seglen, uint32_t segs,
+                                                             long long *part) {
+    constexpr uint32_t CH = 64 * VEC; // outputs per workgroup
+    const uint32_t lx = threadIdx.x % 64, ly = threadIdx.x / 64;
+    const uint32_t tile = blockIdx.x % tiles0;
+    uint32_t rest = blockIdx.x / tiles0;
+    const uint32_t rest_index = rest;
+    int64_t base = 0;
+    for (uint32_t d = 1; d < a.nouter; d++) {
+        const uint32_t q = fastdiv(rest, a.odiv[d]);
+        base += (int64_t)(rest - q * a.od[d]) * a.os[d];
+        rest = q;
+    }
+    const uint32_t r0 = tile * CH + lx * VEC;
+    const uint32_t lo = blockIdx.y * seglen, hi = min(a.n, lo + seglen);
+    const uint32_t *p = reinterpret_cast<const uint32_t *>(a.x) + base + r0;
+    Acc<K, F> acc[VEC];
+    if (r0 < a.od[0]) {
+        if constexpr (VEC == 4) {
+            typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+            uint32_t i = lo + ly;
+            for (; i + 28 < hi; i += 32) { // eight loads in flight per lane
+                u4 t[8];
+#pragma unroll
+                for (int u = 0; u < 8; u++) t[u] = __builtin_nontemporal_load(reinterpret_cast<const u4 *>(p + (int64_t)(i + 4 * u) * a.sn));
+#pragma unroll
+                for (int u = 0; u < 8; u++)
+#pragma unroll
+                    for (int v = 0; v < 4; v++) acc[v].take(t[u][v], i + 4 * u);
+            }
+            for (; i < hi; i += 4) {
+                const u4 t = __builtin_nontemporal_load(reinterpret_cast<const u4 *>(p + (int64_t)i * a.sn));
+#pragma unroll
+                for (int v = 0; v < 4; v++) acc[v].take(t[v], i);
+            }
+        } else {
+            for (uint32_t i = lo + ly; i < hi; i += 4) acc[0].take(p[(int64_t)i * a.sn], i);
+        }
+    }
+    __shared__ long long meet[3][CH];
+    if (ly > 0) {
+#pragma unroll
+        for (int v = 0; v < VEC; v++) meet[ly - 1][lx * VEC + v] = acc[v].pack();
+    }
+    __syncthreads();
+    if (ly == 0 && r0 < a.od[0]) {
+#pragma unroll
+        for (int v = 0; v < VEC; v++) {
+            for (int w = 0; w < 3; w++) acc[v].merge(Acc<K, F>::unpack(meet[w][lx * VEC + v]));
+            if (r0 + v < a.od[0]) {
+                const uint64_t row = (uint64_t)rest_index * a.od[0] + r0 + v;
+                if (segs == 1) a.out[row] = acc[v].result();
+                else part[(uint64_t)blockIdx.y * a.rows + row] = acc[v].pack();
+            }
+        }
+    }
+}
+
+template <int K, bool F>
+__global__ __launch_bounds__(kBlock) void reduce_cols_final_kernel(const long long *part, uint32_t *out, uint32_t segs, uint32_t rows) {
+    // 64 neighbouring outputs per workgroup; the four waves split the segments (independent loads) and meet in LDS
+    const uint32_t lx = threadIdx.x % 64, ly = threadIdx.x / 64;
+    const uint32_t row = blockIdx.x * 64 + lx;
+    Acc<K, F> acc;
+    if (row < rows)
+        for (uint32_t s = ly; s < segs; s += 4) acc.merge(Acc<K, F>::unpack(part[(uint64_t)s * rows + row]));
+    __shared__ long long meet[3][64];
+    if (ly > 0) meet[ly - 1][lx] = acc.pack();
+    __syncthreads();
+    if (ly == 0 && row < rows) {
+        for (int w = 0; w < 3; w++) acc.merge(Acc<K, F>::unpack(meet[w][lx]));
+        out[row] = acc.result();
+    }
+}
+
+template <int K, bool F> int launch_cols(cg_backend *be, const RowsArgs &a) {
+    const uint32_t R0 = a.od[0];
+    bool vec = R0 % 4 == 0 && reinterpret_cast<uintptr_t>(a.x) % 16 == 0 && a.sn % 4 == 0;
+    for (uint32_t d = 1; d < a.nouter; d++) vec = vec && a.os[d] % 4 == 0;
+    const uint32_t ch = vec ? 256 : 64, tiles0 = (R0 + ch - 1) / ch;
+    const uint64_t blocks = (uint64_t)tiles0 * (a.rows / R0);
+    if (blocks > 0x7FFFFFFFull) return fail(CG_ERR_UNSUPPORTED, "reduction extents above 2^31-1 workgroups");
+    // segments along the reduced axis until about 2048 workgroups are in flight, at least 64 steps each
+    uint32_t segs = (uint32_t)std::min<uint64_t>(std::min<uint64_t>((2048 + blocks - 1) / blocks, (a.n + 63) / 64), 64);
+    if (segs < 1) segs = 1;
+    const uint32_t seglen = ((a.n + segs - 1) / segs + 3) / 4 * 4;
+    segs = (a.n + seglen - 1) / seglen;
+    void *part = nullptr;
+    size_t cls = 0;
+    if (segs > 1) {
+        int rc = be->pool.alloc((size_t)segs * a.rows * sizeof(long long), &part, &cls);
+        if (rc) return rc;
+    }
+    const dim3 grid((uint32_t)blocks, segs);
+    if (vec)
+        hipLaunchKernelGGL((reduce_cols_kernel<K, F, 4>), grid, dim3(kBlock), 0, be->stream, a, tiles0, seglen, segs, static_cast<long long *>(part));
+    else
+        hipLaunchKernelGGL((reduce_cols_kernel<K, F, 1>), grid, dim3(kBlock), 0, be->stream, a, tiles0, seglen, segs, static_cast<long long *>(part));
+    if (segs > 1) {
+        hipLaunchKernelGGL((reduce_cols_final_kernel<K, F>), dim3((a.rows + 63) / 64), dim3(kBlock), 0, be->stream,
+                           static_cast<const long long *>(part), a.out, segs, a.rows);
+        be->pool.free(part, cls); // stream-ordered: later users queue behind the merge
+    }
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CG_OK : hip_fail(e, "column reduction launch");
+}
+
 template <int K, bool F> int launch_rows(cg_backend *be, const RowsArgs &a) {
+    if (a.sn != 1 && a.nouter >= 1 && a.os[0] == 1 && a.od[0] >= 16 && a.n >= 8) return launch_cols<K, F>(be, a);
     if (a.rows <= 64 && a.n >= 32768) {
         uint32_t segs = std::min<uint32_t>(256, (a.n + 1023) / 1024);
         const uint32_t seglen = ((a.n + segs - 1) / segs + 3) / 4 * 4;

@@ -928,6 +928,33 @@ static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p, b
     }
     bool piecewise = false;
     for (int l = 0; l < p.nleaf; l++) piecewise = piecewise || p.leaf[l].pw;
+    if (p.ninstr == 1 && p.nleaf == 1 && piecewise && (p.ins[0].op & ~kInstrU32) == kCopy && !p.leaf[0].neg1 && !p.leaf[0].neg2 &&
+        numel(dst) >= (1 << 20)) {
+        // a large concat along the last axis that somebody wants in memory after all: two strided copies at streaming
+        // speed (the program kernels walk a two-part leaf element by element)
+        const LeafView &lv = p.leaf[0];
+        const int last = dst->rank - 1;
+        int rc = CG_OK;
+        for (int part = 0; part < 2 && !rc; part++) {
+            cg_tensor src, half;
+            src.be = half.be = be;
+            src.buf = part ? lv.buf2 : lv.buf;
+            half.buf = dst->buf;
+            src.dt = half.dt = dst->dt;
+            src.rank = half.rank = dst->rank;
+            memcpy(src.dims, dst->dims, sizeof src.dims);
+            src.dims[last] = part ? dst->dims[last] - lv.pw_split : lv.pw_split;
+            memcpy(half.dims, src.dims, sizeof half.dims);
+            memcpy(src.strides, part ? lv.strides2 : lv.strides, sizeof src.strides);
+            memcpy(half.strides, dst->strides, sizeof half.strides);
+            src.offset = part ? lv.offset2 : lv.offset;
+            half.offset = dst->offset + (part ? lv.pw_split * dst->strides[last] : 0);
+            const cg_tensor *ins[1] = {&src};
+            if (numel(&src) > 0) rc = launch_elementwise(be, kCopy, dst->dt, &half, ins, 1);
+            src.buf = half.buf = nullptr;
+        }
+        return rc;
+    }
     if (p.ninstr == 1 && !piecewise) {
         const Instr in = p.ins[0];
         const int op = in.op & ~kInstrU32;

@@ -1009,6 +1009,78 @@ for _shape in ((4, 128256), (3, 70001), (1, 1, 32768), (2, 40000)):
         return run, expect
 
 
+# ---- copies that transpose, reductions over an axis that is not the unit-stride one ------------------------------------
+@case("transpose_copies_tiled")
+def _():
+    """Row-major copies of transposed views (`reshape` after `transpose`, ndarray.rs:545-569): whole 64 x 64 tiles with
+    16-byte accesses, ragged edges, further axes, an unaligned (sliced) source, u32, the head merge of attention."""
+    a = f32(600, (130, 70))
+    b = u32(601, (256, 512))
+    c = f32(602, (257, 513))
+    d = f32(603, (4, 6, 64, 128))
+    e = f32(604, (3, 200, 96))
+    g = f32(605, (128, 260))
+
+    def run(be):
+        outs = [be.reshape(be.transpose(be.from_numpy(a), 0, 1), (70 * 130,)),
+                be.reshape(be.transpose(be.from_numpy(b), 0, 1), (512, 256, 1)),
+                be.reshape(be.transpose(be.from_numpy(c), 0, 1), (513 * 257,)),
+                be.reshape(be.transpose(be.from_numpy(d), 1, 2), (4, 64, 6 * 128)),
+                be.reshape(be.transpose(be.from_numpy(e), 0, 2), (96 * 200 * 3,)),
+                be.reshape(be.transpose(be.slice(be.from_numpy(g), 1, 3, 192), 0, 1), (192 * 128,)),
+                be.concat(be.transpose(be.from_numpy(a), 0, 1), be.transpose(be.from_numpy(a), 0, 1), 0)]
+        return N(be, *outs)
+
+    def expect():
+        return [a.T.reshape(-1), b.T.reshape(512, 256, 1), c.T.reshape(-1), d.transpose(0, 2, 1, 3).reshape(4, 64, 768),
+                e.transpose(2, 1, 0).reshape(-1), g[:, 3:195].T.reshape(-1), np.concatenate([a.T, a.T], 0)]
+
+    return run, expect
+
+
+_COLS_IN = [f32(610, (1000, 300)), f32(611, (8192, 64)), f32(612, (64, 4096)), f32(613, (70000, 16)), f32(614, (3, 500, 130))]
+
+
+@case("reduce_over_strided_axis_sum", "red",
+      (lambda: [np.abs(x.astype(np.float64)).sum(-2)[..., None] if x.ndim == 2 else np.abs(x.astype(np.float64)).sum(1)[..., None]
+                for x in _COLS_IN]))
+def _():
+    """`sum` over the last axis of transposed views: the reduced axis has a stride, the outputs are contiguous."""
+    def run(be):
+        return N(be, *[be.sum(be.transpose(be.from_numpy(x), x.ndim - 2, x.ndim - 1)) for x in _COLS_IN])
+
+    return run, (lambda: [x.astype(np.float64).sum(-2)[..., None] for x in _COLS_IN])
+
+
+@case("reduce_over_strided_axis_max_argmax_u32")
+def _():
+    xs = [x.copy() for x in _COLS_IN]
+    xs[0][::7] = np.float32(9.5)            # equal maxima down a column: the last one wins
+    xs[1][5, :] = np.float32(np.nan)
+    xs[3][69999, 3] = np.float32(np.inf)
+    u = u32(615, (300, 130))
+    us = u32(616, (2000, 260), hi=50)       # many ties
+
+    def run(be):
+        outs = []
+        for x in xs:
+            t = be.transpose(be.from_numpy(x), x.ndim - 2, x.ndim - 1)
+            outs += [be.max(t), be.argmax(t)]
+        tu = be.transpose(be.from_numpy(u), 0, 1)
+        outs += [be.sum(tu), be.max(tu), be.argmax(be.transpose(be.from_numpy(us), 0, 1))]
+        return N(be, *outs)
+
+    def expect():
+        outs = []
+        for x in xs:
+            t = np.swapaxes(x, -1, -2)
+            outs += [max_last_f32(t), argmax_last(t)]
+        outs += [(u.astype(np.uint64).sum(0) & 0xFFFFFFFF).astype(np.uint32)[:, None], u.max(0)[:, None], argmax_last(us.T)]
+        return outs
+
+    return run, expect
+
+
 # ---- decode-time linear layers: lazy, grouped by their shared left operand ---------------------------------------
 def _linear(be, x, w):
     """`nn::linear_b_param` without bias (stdlib/nn/mod.rs:182-204): x [B,S,K] times w [N,K] transposed."""
