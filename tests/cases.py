@@ -1618,6 +1618,63 @@ def _():
     return run, expect
 
 
+# ---- mixture-of-experts routing as Qwen3's MoE layer issues it (qwen3.rs:125-194) ------------------------------------
+for _S, _E, _k, _H, _I in ((1, 8, 2, 256, 512), (16, 8, 2, 256, 512), (5, 4, 3, 128, 320)):
+    @case(f"moe_topk_index_grouped_matmul_S{_S}_E{_E}_k{_k}", "red", (lambda: [np.float64(1.0)]))
+    def _(S=_S, E=_E, k=_k, H=_H, I=_I):
+        """soft-max router -> `topk` -> per chosen expert `index` on the [E, I, H] stacks -> batched matmul with one
+        row per token ([S, 1, H] x [S, H, I]) -> SiLU * up -> down -> weighted sum (norm_topk_prob).  Outputs are of
+        order 0.1: 1e-3 of 1 is the bound."""
+        for seed in range(640, 740):     # the first seed whose router probabilities leave every top-k choice clear
+            r_ = np.random.default_rng(seed + S + E)
+            x = r_.standard_normal((1, S, H)).astype(np.float32)
+            wr = r_.standard_normal((E, H)).astype(np.float32) * np.float32(4.0 / np.sqrt(H))     # spread router logits
+            pr = _np_softmax((x.astype(np.float64) @ wr.astype(np.float64).T)[0])
+            srt = np.sort(pr, -1)[:, ::-1]
+            if (srt[:, :k] - srt[:, 1:k + 1]).min() > 2e-3:
+                break
+        wg = r_.standard_normal((E, I, H)).astype(np.float32) * np.float32(1.0 / np.sqrt(H))
+        wu = r_.standard_normal((E, I, H)).astype(np.float32) * np.float32(1.0 / np.sqrt(H))
+        wd = r_.standard_normal((E, H, I)).astype(np.float32) * np.float32(1.0 / np.sqrt(I))
+        assert (srt[:, :k] - srt[:, 1:k + 1]).min() > 2e-3, "router probabilities too close for a stable top-k"
+
+        def run(be):
+            tx = be.from_numpy(x)
+            routed = softmax_ops(be, _linear(be, tx, be.from_numpy(wr)))
+            vals, idxs = be.topk(routed, k)
+            sh = (S, k)
+            idxs, vals = be.reshape(idxs, sh), be.reshape(vals, sh)
+            vals = be.div(vals, be.broadcast(be.sum(vals), sh))
+            fullx = be.transpose(tx, 0, 1)                                  # [S, 1, H]
+            sumk = _const(be, 0.0, (S, 1, H))
+            ga, ua, da = be.from_numpy(wg), be.from_numpy(wu), be.from_numpy(wd)
+            for i in range(k):
+                idx = be.slice(idxs, 1, i, 1)
+                val = be.slice(vals, 1, i, 1)
+                g = be.matmul(fullx, be.transpose(be.index(ga, 0, idx), 1, 2))
+                u = be.matmul(fullx, be.transpose(be.index(ua, 0, idx), 1, 2))
+                one = _const(be, 1.0, (S, 1, I))
+                act = be.mul(be.mul(g, be.div(one, be.add(one, be.exp(be.neg(g))))), u)
+                y = be.matmul(act, be.transpose(be.index(da, 0, idx), 1, 2))
+                v = be.broadcast(be.reshape(val, (S, 1, 1)), (S, 1, H))
+                sumk = be.add(sumk, be.mul(y, v))
+            return N(be, be.transpose(sumk, 0, 1))
+
+        def expect():
+            f8 = np.float64
+            out = np.zeros((S, H))
+            for t in range(S):
+                order = np.argsort(-pr[t], kind="stable")[:k]
+                w = pr[t][order] / pr[t][order].sum()
+                for e, wt in zip(order, w):
+                    g = wg[e].astype(f8) @ x[0, t].astype(f8)
+                    u = wu[e].astype(f8) @ x[0, t].astype(f8)
+                    out[t] += wt * (wd[e].astype(f8) @ (g / (1.0 + np.exp(-g)) * u))
+            return [out[None]]
+
+        return run, expect
+
+
 def by_name(name):
     for c in CASES:
         if c.name == name:
