@@ -65,13 +65,19 @@ class Tensor:
 
     @property
     def dtype(self) -> int:
+        if self._h is None:
+            raise ValueError("use of a moved tensor")
         return int(self._be._lib.cg_tensor_dtype(self._h))
 
     @property
     def is_contiguous(self) -> bool:
+        if self._h is None:
+            raise ValueError("use of a moved tensor")
         return bool(self._be._lib.cg_tensor_is_contiguous(self._h))
 
     def clone(self) -> "Tensor":
+        if self._h is None:
+            raise ValueError("use of a moved tensor")
         self._be._lib.cg_tensor_retain(self._h)
         return Tensor(self._be, self._h)
 
@@ -88,6 +94,8 @@ class Tensor:
             self._be._lib.cg_tensor_release(h)
 
     def __repr__(self):
+        if self._h is None:
+            return "Tensor(<moved>)"
         return f"Tensor({A.DTYPE_NAMES[self.dtype]}{list(self.shape)})"
 
 

@@ -308,6 +308,7 @@ struct LeafView {
     // is how rotate_half = concat(-x2, x1) of the rotary embedding stays a leaf.
     bool pw = false;
     Buffer *buf2 = nullptr; // retained
+    LazyMm *lazy2 = nullptr; // retained: the second part is a view of this product's result (buf2 null until it is computed)
     int64_t strides2[kMaxRank] = {0};
     int64_t offset2 = 0;
     int64_t pw_split = 0;
@@ -443,13 +444,26 @@ int launch_prefill_attention(cg_backend *be, const Pending &p, const int64_t *pd
 int launch_fused_group(cg_backend *be, const cg_tensor *const *outs, const Pending *const *ps, int n);
 // Writes that were put off so that they can share a launch (see DeferredWrite); every function
 // that launches a kernel or copies device memory calls this first.
-int flush_deferred(cg_backend *be);
+int flush_deferred(cg_backend *be, const Pending *also = nullptr);
 // nterms: 2 (out = t0 + t1) or 4.  out is a contiguous view (any offset).  keep_sums: out is the whole of its buffer, which
 // may then receive the partial sums of squares of the stored rows (Buffer::side).
 int launch_matmul_residual(cg_backend *be, const cg_tensor *x, const cg_tensor *y, const uint32_t *const *terms, int nterms,
                            int slot, int order, cg_tensor *out, bool keep_sums);
 int launch_matmul_group(cg_backend *be, const cg_tensor *x, const cg_tensor *const *ys, cg_tensor *const *outs, int n,
                         const NormFuse *nf = nullptr);
+// Where the columns of a decode-time product go when the rotary embedding and the write into a KV cache (or into q's own
+// buffer) run in the product's store: column n = head * hd + d of row b goes to dst[b * sb + head * sh + d], after
+// out[d] = cos[d] * x[d] + sin[d] * rot[d], rot = concat(-x[hd/2..], x[..hd/2]) when `rope` (cos, sin: hd words each).
+struct RopeStore {
+    uint32_t *dst;
+    int64_t sb, sh;
+    const uint32_t *cos, *sin;
+    uint32_t hd, rope;
+};
+// The products x . ys[i] (one row per batch entry, the same x) with such a store each; kDeclined when the shapes are not
+// the grouped kernel's.  nf as in launch_matmul_group.
+int launch_matmul_group_rope(cg_backend *be, const cg_tensor *x, const cg_tensor *const *ys, const RopeStore *stores, int n,
+                             const NormFuse *nf);
 
 // Decode-time attention in one pass: out = softmax-program(q . kT) . v, where `p` is the deferred
 // soft-max program whose leaf 0 is the (never computed) lazy product q . kT and (pdims, prank) its

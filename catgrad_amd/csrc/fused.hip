@@ -498,7 +498,13 @@ int fill_args(cg_backend *be, const Pending &p, const int64_t *dims, int rank, c
             w.strides = lv.strides2;
             w.uniform = false;
             w.ubits = 0;
-            w.ptr = static_cast<const char *>(lv.buf2->ptr) + lv.offset2 * 4;
+            const Buffer *src2 = lv.buf2;
+            if (lv.lazy2) { // the second part is a view of a product that has been put off until now
+                int lrc = lazy_mm_force(be, lv.lazy2);
+                if (lrc) return lrc;
+                src2 = lv.lazy2->result;
+            }
+            w.ptr = static_cast<const char *>(src2->ptr) + lv.offset2 * 4;
             w.vec_period = lv.pw_split;
         }
         if (!lv.uniform) {

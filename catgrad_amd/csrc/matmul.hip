@@ -755,6 +755,114 @@ __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_group_norm_kerne
     skinny_kt_mfma_xreg_body<4, 1, false, false, true, TRIPS>(g.p[p], bx, 0, nullptr, 0, nullptr, &nf);
 }
 
+// The grouped products of an attention block's decode step (q, k, v: a few rows, the same left operand) with the
+// rotary embedding and the move into the KV cache done where they are stored: a workgroup owns two groups of four
+// columns half a head apart (the pair the embedding mixes; next to each other for a product stored as it is) and
+// writes column n = head * hd + d of row m to dst[m * sb + head * sh + d] (see RopeStore).  The embedding's ops are
+// those of the deferred program cos * x + sin * concat(-x2, x1), in its order.  M <= 4, K a multiple of TRIPS * 256,
+// N a multiple of hd (of 8 without the embedding).
+struct RopeGroup {
+    RopeStore s[kMaxGroup];
+};
+template <bool NORM, int TRIPS>
+__global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_group_rope_kernel(const MmGroup g, const RopeGroup rg, const NormFuse nf) {
+    static_assert(TRIPS == 8 || TRIPS == 4, "chunks of 2048 or 1024");
+    uint32_t bx;
+    const uint32_t p = group_problem(g, bx);
+    const MmArgs &a = g.p[p];
+    const RopeStore &rs = rg.s[p];
+    const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    const uint32_t j = lane % 4, b = lane / 4;
+    const uint32_t span = rs.rope ? rs.hd : 8, per = span / 8;
+    const uint32_t n0 = bx / per * span + bx % per * 4;
+    const uint32_t nc[2] = {n0, n0 + span / 2};
+    const uint32_t *wrow[2];
+#pragma unroll
+    for (int c = 0; c < 2; c++) wrow[c] = a.B + (int64_t)min(nc[c] + j, a.N - 1) * a.b_sn;
+    const uint32_t *xrow = a.A + (int64_t)min(j, a.M - 1) * a.a_sm;
+    float4v acc[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    // the embedding's factors for the value this thread will store: asked for before the walk along K
+    uint32_t cs = 0, sn = 0;
+    if (rs.rope && threadIdx.x < 32) {
+        const uint32_t d = (nc[threadIdx.x / 16] + threadIdx.x % 4) % rs.hd;
+        cs = rs.cos[d];
+        sn = rs.sin[d];
+    }
+    float pv[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    if constexpr (NORM) {
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const uint32_t i = threadIdx.x + u * kThreads;
+            if (i < nf.blocks * 4) pv[u] = nf.partials[i];
+        }
+    }
+    const uint32_t kb = wave * (TRIPS * 64) + b * 4;
+    for (uint32_t k0 = 0; k0 < a.K; k0 += TRIPS * 256) {
+        float4v xr[TRIPS];
+#pragma unroll
+        for (int t = 0; t < TRIPS; t++) xr[t] = *reinterpret_cast<const float4v *>(xrow + k0 + kb + 64 * t);
+        float4v gm[NORM ? TRIPS : 1];
+        if constexpr (NORM) {
+#pragma unroll
+            for (int t = 0; t < TRIPS; t++) gm[t] = *reinterpret_cast<const float4v *>(nf.gamma + k0 + kb + 64 * t);
+        }
+#pragma unroll
+        for (int c = 0; c < 2; c++) {
+            float4v w[TRIPS];
+#pragma unroll
+            for (int t = 0; t < TRIPS; t++) w[t] = *reinterpret_cast<const float4v *>(wrow[c] + k0 + kb + 64 * t);
+            if constexpr (NORM) {
+                if (c == 0) {
+#pragma unroll
+                    for (int t = 0; t < TRIPS; t++)
+#pragma unroll
+                        for (int e = 0; e < 4; e++) xr[t][e] = asf(apply<kMul, true>(asu(xr[t][e]), asu(gm[t][e]), 0, nullptr));
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < TRIPS; t++) {
+                acc[c] = __builtin_amdgcn_mfma_f32_4x4x1f32(xr[t][0], w[t][0], acc[c], 0, 0, 0);
+                acc[c] = __builtin_amdgcn_mfma_f32_4x4x1f32(xr[t][1], w[t][1], acc[c], 0, 0, 0);
+                acc[c] = __builtin_amdgcn_mfma_f32_4x4x1f32(xr[t][2], w[t][2], acc[c], 0, 0, 0);
+                acc[c] = __builtin_amdgcn_mfma_f32_4x4x1f32(xr[t][3], w[t][3], acc[c], 0, 0, 0);
+            }
+        }
+    }
+    __shared__ float part[4][32];
+    __shared__ float nsum[4][4];
+    if constexpr (NORM) {
+        float s = 0.0f;
+#pragma unroll
+        for (int u = 0; u < 8; u++) s += pv[u];
+        for (uint32_t i = threadIdx.x + 8 * kThreads; i < nf.blocks * 4; i += kThreads) s += nf.partials[i];
+#pragma unroll
+        for (int sh = 32; sh >= 4; sh >>= 1) s += __shfl_xor(s, sh);
+        if (lane < 4) nsum[wave][lane] = s;
+    }
+#pragma unroll
+    for (int c = 0; c < 2; c++)
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float v = acc[c][i];
+#pragma unroll
+            for (int s = 32; s >= 4; s >>= 1) v += __shfl_xor(v, s);
+            if (lane < 4) part[wave][(c * 4 + i) * 4 + j] = v;
+        }
+    __syncthreads();
+    if (threadIdx.x < 64) { // the first wave: lanes 0..31 hold (column group, row, column), the others idle along
+        const uint32_t t = threadIdx.x % 32, c = t / 16, m = t / 4 % 4, col = nc[c] + t % 4;
+        uint32_t v = asu((part[0][t] + part[1][t]) + (part[2][t] + part[3][t]));
+        if constexpr (NORM) v = apply<kDiv, true>(v, norm_divisor(nf, (nsum[0][m] + nsum[1][m]) + (nsum[2][m] + nsum[3][m])), 0, nullptr);
+        const uint32_t other = __shfl_xor(v, 16); // the same row's column half a head away
+        if (rs.rope) {
+            // lower half: rotate_half reads -x[d + hd / 2]; upper half: x[d - hd / 2]
+            const uint32_t rot = c == 0 ? apply<kNeg, true>(other, 0, 0, nullptr) : other;
+            v = apply<kAdd, true>(apply<kMul, true>(cs, v, 0, nullptr), apply<kMul, true>(sn, rot, 0, nullptr), 0, nullptr);
+        }
+        if (threadIdx.x < 32 && col < a.N && m < a.M) rs.dst[(int64_t)m * rs.sb + (int64_t)(col / rs.hd) * rs.sh + col % rs.hd] = v;
+    }
+}
+
 // The gated pair when K is exactly one chunk (TRIPS * 256: the hidden size of the model): the workgroup asks for its
 // share of the activations (and of gamma, and of the row sums of an RMS norm) ONCE and walks `iters` consecutive
 // groups of four columns with them, the next group's weights always on their way while the current group is
@@ -1152,6 +1260,44 @@ int launch_matmul_group(cg_backend *be, const cg_tensor *x, const cg_tensor *con
         hipLaunchKernelGGL((skinny_kt_wide_group_kernel<8>), dim3(blocks), dim3(kThreads), 0, be->stream, g);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? CG_OK : hip_fail(e, "grouped matmul launch");
+}
+
+int launch_matmul_group_rope(cg_backend *be, const cg_tensor *x, const cg_tensor *const *ys, const RopeStore *stores, int n,
+                             const NormFuse *nf) {
+    if (n < 1 || n > kMaxGroup || x->dt != CG_F32) return kDeclined;
+    MmGroup g;
+    RopeGroup rg;
+    memset(&g, 0, sizeof g);
+    memset(&rg, 0, sizeof rg);
+    double bytes = distinct_bytes(x);
+    uint32_t blocks = 0;
+    for (int i = 0; i < n; i++) {
+        MmFold f;
+        int rc = make_mm_args(x, ys[i], stores[i].dst, &g.p[i], &f);
+        if (rc) return rc;
+        const MmArgs &a = g.p[i];
+        const RopeStore &st = stores[i];
+        const bool vec = a.a_vec && a.b_vec && a.a_sk == 1 && a.K % 4 == 0;
+        if (f.batch != 1 || !xreg_narrow(a.M, a.K) || a.b_sk != 1 || !vec || a.N >= 8192) return kDeclined;
+        if (i > 0 && (a.M != g.p[0].M || a.K != g.p[0].K || a.a_sm != g.p[0].a_sm)) return kDeclined;
+        if (st.hd < 8 || st.hd % 8 || a.N % st.hd || !st.dst || (st.rope && (!st.cos || !st.sin))) return kDeclined;
+        rg.s[i] = st;
+        g.first[i] = blocks;
+        blocks += a.N / 8;
+        bytes += distinct_bytes(ys[i]) + 4.0 * (double)a.M * a.N;
+    }
+    g.first[n] = blocks;
+    g.n = (uint32_t)n;
+    NormFuse none;
+    memset(&none, 0, sizeof none);
+    const bool wide = xreg_trips(g.p[0].K) == 8;
+    ProfScope prof(be, CG_K_GEMM_SKINNY, bytes);
+    if (nf && wide) hipLaunchKernelGGL((skinny_kt_mfma_xreg_group_rope_kernel<true, 8>), dim3(blocks), dim3(kThreads), 0, be->stream, g, rg, *nf);
+    else if (nf) hipLaunchKernelGGL((skinny_kt_mfma_xreg_group_rope_kernel<true, 4>), dim3(blocks), dim3(kThreads), 0, be->stream, g, rg, *nf);
+    else if (wide) hipLaunchKernelGGL((skinny_kt_mfma_xreg_group_rope_kernel<false, 8>), dim3(blocks), dim3(kThreads), 0, be->stream, g, rg, none);
+    else hipLaunchKernelGGL((skinny_kt_mfma_xreg_group_rope_kernel<false, 4>), dim3(blocks), dim3(kThreads), 0, be->stream, g, rg, none);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CG_OK : hip_fail(e, "grouped matmul with rotary store launch");
 }
 
 // out = g * (1 / (one + exp(-g))) * u with g = x.yg, u = x.yu: two decode-time linear layers and

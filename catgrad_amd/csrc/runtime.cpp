@@ -128,6 +128,7 @@ Pending::Pending(const Pending &o)
         if (leaf[l].buf) leaf[l].buf->rc.fetch_add(1);
         if (leaf[l].buf2) leaf[l].buf2->rc.fetch_add(1);
         if (leaf[l].lazy) leaf[l].lazy->rc.fetch_add(1);
+        if (leaf[l].lazy2) leaf[l].lazy2->rc.fetch_add(1);
     }
     for (int i = 0; i < ninstr; i++) ins[i] = o.ins[i];
 }
@@ -137,6 +138,7 @@ Pending::~Pending() {
         buffer_release(leaf[l].buf);
         buffer_release(leaf[l].buf2);
         lazy_mm_release(leaf[l].lazy);
+        lazy_mm_release(leaf[l].lazy2);
     }
 }
 
@@ -775,13 +777,22 @@ static int resolve_lazy_leaves(cg_backend *be, const Pending &cp) {
     Pending &p = const_cast<Pending &>(cp); // a cache fill: the value of the program does not change
     for (int l = 0; l < p.nleaf; l++) {
         LeafView &lv = p.leaf[l];
-        if (!lv.lazy) continue;
-        int rc = lazy_mm_force(be, lv.lazy);
-        if (rc) return rc;
-        lv.buf = lv.lazy->result;
-        lv.buf->rc.fetch_add(1);
-        lazy_mm_release(lv.lazy);
-        lv.lazy = nullptr;
+        if (lv.lazy) {
+            int rc = lazy_mm_force(be, lv.lazy);
+            if (rc) return rc;
+            lv.buf = lv.lazy->result;
+            lv.buf->rc.fetch_add(1);
+            lazy_mm_release(lv.lazy);
+            lv.lazy = nullptr;
+        }
+        if (lv.lazy2) {
+            int rc = lazy_mm_force(be, lv.lazy2);
+            if (rc) return rc;
+            lv.buf2 = lv.lazy2->result;
+            lv.buf2->rc.fetch_add(1);
+            lazy_mm_release(lv.lazy2);
+            lv.lazy2 = nullptr;
+        }
     }
     return CG_OK;
 }
@@ -990,7 +1001,7 @@ static bool const_key(const Pending &p, const int64_t *dims, int rank, std::stri
     for (int i = 0; i < p.ninstr; i++) put(&p.ins[i], sizeof(Instr));
     for (int l = 0; l < p.nleaf; l++) {
         const LeafView &lv = p.leaf[l];
-        if (lv.lazy) return false;
+        if (lv.lazy || lv.lazy2) return false;
         const char kind = lv.uniform ? 'u' : lv.pw ? 'p' : 'v';
         put(&kind, 1);
         if (lv.uniform) {
@@ -1083,11 +1094,106 @@ static void drop_deferred(DeferredWrite &w) {
     w.dst = nullptr;
 }
 
-int flush_deferred(cg_backend *be) {
+// The waiting writes of a decode step's attention block: the rotary embedding of q and of k (k's destination the
+// new row of the KV cache, helpers/rope.rs:423-447 and helpers/cache.rs:64-74) and the copy of v into its cache row,
+// each over a product that nobody has computed yet (q / k / v share their left operand).  Then the products
+// themselves store roped values straight to those destinations, in one launch: the three products never reach
+// memory un-roped and the launch that would read them back goes away.  `also`: a program that refers to the same
+// products and goes away with the caller (the handle that is being made concrete).  kDeclined: not that shape.
+static int try_rope_stores(cg_backend *be, std::vector<DeferredWrite> &w, const Pending *also) {
+    const int n = (int)w.size();
+    if (!be->aot || !be->fuse || n < 1 || n > 4) return kDeclined;
+    LazyMm *ms[4];
+    RopeStore st[4];
+    for (int i = 0; i < n; i++) {
+        const Pending &p = *w[i].prog;
+        const cg_tensor *dst = w[i].dst;
+        if (p.reduced || p.nred || p.overflow || dst->dt != CG_F32 || dst->rank != 4 || dst->dims[2] != 1 || dst->split >= 0) return kDeclined;
+        const int64_t B = dst->dims[0], H = dst->dims[1], hd = dst->dims[3];
+        if (hd < 8 || hd % 8 || dst->strides[3] != 1) return kDeclined;
+        const LeafView *lx = nullptr, *lc = nullptr, *ls = nullptr, *lr = nullptr;
+        if (p.nleaf == 1 && p.ninstr == 1 && p.ins[0].op == kCopy) {
+            lx = &p.leaf[0];
+        } else if (p.nleaf == 4 && p.ninstr == 3 && p.ins[0].op == kMul && p.ins[1].op == kMul && p.ins[2].op == kAdd &&
+                   p.ins[0].a + p.ins[0].b == 1 && p.ins[1].a + p.ins[1].b == 5 && p.ins[2].a + p.ins[2].b == 2 * kMaxLeaves + 1) {
+            // cos * x + sin * rotate_half(x), the factors of each product in either order
+            const bool x_first = p.leaf[0].lazy != nullptr, r_first = p.leaf[2].pw;
+            lx = &p.leaf[x_first ? 0 : 1];
+            lc = &p.leaf[x_first ? 1 : 0];
+            lr = &p.leaf[r_first ? 2 : 3];
+            ls = &p.leaf[r_first ? 3 : 2];
+        } else {
+            return kDeclined;
+        }
+        LazyMm *m = lx->lazy;
+        if (lx->uniform || lx->pw || !m || m->result || !m->groupable || !m->be || m->rank < 1) return kDeclined;
+        const int64_t N = m->dims[m->rank - 1];
+        int64_t rows = 1;
+        for (int d = 0; d + 1 < m->rank; d++) rows *= m->dims[d];
+        if (H * hd != N || rows != B || B > 4) return kDeclined;
+        auto whole = [&](const int64_t *s, int64_t off, int64_t want_off) { // the view [B, H, 1, hd] of the product's rows, from `want_off`
+            return (B == 1 || s[0] == N) && (H == 1 || s[1] == hd) && s[3] == 1 && off == want_off;
+        };
+        auto row_table = [&](const LeafView *l) { // one row of hd factors, the same for every batch entry and head
+            return l->buf && !l->uniform && !l->pw && !l->lazy && (B == 1 || l->strides[0] == 0) && (H == 1 || l->strides[1] == 0) &&
+                   l->strides[3] == 1;
+        };
+        if (!whole(lx->strides, lx->offset, 0)) return kDeclined;
+        memset(&st[i], 0, sizeof st[i]);
+        if (lr) {
+            if (!lr->pw || lr->uniform || lr->lazy != m || lr->lazy2 != m || !lr->neg1 || lr->neg2 || lr->pw_split * 2 != hd) return kDeclined;
+            if (!whole(lr->strides, lr->offset, hd / 2) || !whole(lr->strides2, lr->offset2, 0)) return kDeclined;
+            if (!row_table(lc) || !row_table(ls)) return kDeclined;
+            st[i].cos = static_cast<const uint32_t *>(lc->buf->ptr) + lc->offset;
+            st[i].sin = static_cast<const uint32_t *>(ls->buf->ptr) + ls->offset;
+            st[i].rope = 1;
+        }
+        st[i].dst = static_cast<uint32_t *>(dst->buf->ptr) + dst->offset;
+        st[i].sb = B > 1 ? dst->strides[0] : 0;
+        st[i].sh = H > 1 ? dst->strides[1] : 0;
+        st[i].hd = (uint32_t)hd;
+        if (st[i].sb < 0 || st[i].sh < 0) return kDeclined;
+        for (int k = 0; k < i; k++)
+            if (ms[k] == m) return kDeclined; // one destination per product
+        if (i > 0 && m->x != ms[0]->x) return kDeclined;
+        ms[i] = m;
+    }
+    // nobody else may want the products as they are: every reference to them is held by these programs
+    for (int i = 0; i < n; i++) {
+        long held = 0;
+        auto count = [&](const Pending *p) {
+            for (int l = 0; p && l < p->nleaf; l++) held += (p->leaf[l].lazy == ms[i]) + (p->leaf[l].lazy2 == ms[i]);
+        };
+        for (int k = 0; k < n; k++) count(w[k].prog);
+        count(also);
+        if (ms[i]->rc.load() != held) return kDeclined;
+    }
+    cg_tensor *x = ms[0]->x;
+    NormFuse nf;
+    cg_tensor h;
+    const bool normed = x->pend && norm_fuse_of(x, &nf, &h);
+    const cg_tensor *ys[4];
+    for (int i = 0; i < n; i++) ys[i] = ms[i]->y;
+    int rc = CG_OK;
+    if (x->pend && !normed) rc = ensure_concrete(x);
+    if (!rc) rc = launch_matmul_group_rope(be, normed ? &h : x, ys, st, n, normed ? &nf : nullptr);
+    h.buf = nullptr;
+    if (rc) return rc;
+    be->programs_compiled++;
+    for (int i = 0; i < n; i++) lazy_mm_close(ms[i]); // they go away with the programs, never computed on their own
+    return CG_OK;
+}
+
+int flush_deferred(cg_backend *be, const Pending *also) {
     if (be->deferred.empty()) return CG_OK;
     std::vector<DeferredWrite> w;
     w.swap(be->deferred); // the launches below come back here and find nothing to do
-    int rc = CG_OK;
+    int rc = try_rope_stores(be, w, also);
+    if (rc != kDeclined) {
+        for (DeferredWrite &d : w) drop_deferred(d);
+        return rc;
+    }
+    rc = CG_OK;
     const int n = (int)w.size();
     for (int i = 0; i < n && !rc; i++) rc = resolve_lazy_leaves(be, *w[i].prog);
     bool done = false;
@@ -1207,7 +1313,7 @@ static int ensure_concrete(cg_tensor *t) {
     if (!be->deferred.empty() && may_wait(be, &dst, t->pend)) {
         // writes are waiting for a launch: this one goes along
         rc = defer_write(be, &dst, t->pend);
-        if (!rc) rc = flush_deferred(be);
+        if (!rc) rc = flush_deferred(be, t->pend);
     } else {
         rc = run_pending(be, &dst, *t->pend, true);
     }
@@ -1227,7 +1333,7 @@ static int ensure_concrete(cg_tensor *t) {
 }
 
 static bool same_leaf(const LeafView &a, const LeafView &b, const int64_t *dims, int rank) {
-    if (a.uniform != b.uniform || a.pw != b.pw || a.lazy != b.lazy) return false;
+    if (a.uniform != b.uniform || a.pw != b.pw || a.lazy != b.lazy || a.lazy2 != b.lazy2) return false;
     if (a.uniform) return a.ubits == b.ubits;
     if (a.buf != b.buf || a.offset != b.offset) return false;
     for (int i = 0; i < rank; i++)
@@ -1254,6 +1360,7 @@ static int add_leaf(Pending *p, const LeafView &lv, const int64_t *dims, int ran
     if (lv.buf) lv.buf->rc.fetch_add(1);
     if (lv.buf2) lv.buf2->rc.fetch_add(1);
     if (lv.lazy) lv.lazy->rc.fetch_add(1);
+    if (lv.lazy2) lv.lazy2->rc.fetch_add(1);
     return p->nleaf++;
 }
 
@@ -2889,12 +2996,9 @@ int cg_concat(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor *
         // operand is a plain view, or the negation of one (rotate_half of the rotary embedding,
         // helpers/rope.rs:423-427): its consumer then reads both halves in place.
         LeafView lv;
-        for (cg_tensor *t : {x, y})
-            if (t->pend) {
-                int lrc = resolve_lazy_leaves(b, *t->pend);
-                if (lrc) return lrc;
-            }
-        auto part = [&](cg_tensor *t, Buffer **buf, int64_t *strides, int64_t *offset, bool *neg) {
+        // a part may also be a view of a decode-time product that has not been computed yet: it stays open, so that a
+        // rotary embedding over it can still run in the product's own store (see try_rope_stores)
+        auto part = [&](cg_tensor *t, Buffer **buf, LazyMm **lazy, int64_t *strides, int64_t *offset, bool *neg) {
             if (t->uniform || t->split >= 0) return false;
             const int64_t *st;
             if (!t->pend) {
@@ -2905,18 +3009,24 @@ int cg_concat(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor *
                 *neg = false;
             } else {
                 const Pending *p = t->pend;
-                if (p->nleaf != 1 || p->ninstr != 1 || p->nred || p->leaf[0].uniform || p->leaf[0].pw || p->leaf[0].lazy) return false;
+                if (p->nleaf != 1 || p->ninstr != 1 || p->nred || p->leaf[0].uniform || p->leaf[0].pw) return false;
                 const int pop = p->ins[0].op & ~kInstrU32;
                 if (p->ins[0].op != kNeg && pop != kCopy) return false; // a view, or the f32 negation of one
-                *buf = p->leaf[0].buf;
-                st = p->leaf[0].strides;
-                *offset = p->leaf[0].offset;
+                const LeafView &src = p->leaf[0];
+                if (src.lazy && src.lazy->result) { // computed in the meantime: an ordinary buffer
+                    *buf = src.lazy->result;
+                } else {
+                    *buf = src.buf;
+                    *lazy = src.lazy;
+                }
+                st = src.strides;
+                *offset = src.offset;
                 *neg = pop != kCopy;
             }
             memcpy(strides, st, sizeof(int64_t) * kMaxRank);
             return true;
         };
-        if (part(x, &lv.buf, lv.strides, &lv.offset, &lv.neg1) && part(y, &lv.buf2, lv.strides2, &lv.offset2, &lv.neg2)) {
+        if (part(x, &lv.buf, &lv.lazy, lv.strides, &lv.offset, &lv.neg1) && part(y, &lv.buf2, &lv.lazy2, lv.strides2, &lv.offset2, &lv.neg2)) {
             lv.pw = true;
             lv.pw_split = x->dims[dim];
             Pending *p = new Pending;

@@ -1333,6 +1333,94 @@ for _B, _kvh, _rep, _T, _hd in ((2, 2, 4, 300, 64), (1, 3, 1, 1, 64), (2, 1, 8, 
         return run, (lambda: [_np_decode_attention(q, k, v, rep)])
 
 
+# ---- a decode step's attention block: q / k / v projections, rotary embedding, cache append, attention ------------------
+def _np_rope(x, cos, sin):
+    h = x.shape[-1] // 2
+    return cos * x + sin * np.concatenate([-x[..., h:], x[..., :h]], -1)
+
+
+for _B, _K, _kvh, _rep, _T, _hd, _normed in ((4, 2048, 8, 4, 300, 64, True), (1, 1024, 2, 2, 256, 128, False), (2, 2048, 4, 1, 131, 64, True),
+                                              (3, 512, 4, 2, 200, 64, False), (4, 2048, 2, 4, 512, 32, False)):
+    @case(f"decode_qkv_rope_append_B{_B}_K{_K}_kv{_kvh}_rep{_rep}_T{_T}_hd{_hd}{'_normed' if _normed else ''}", "red",
+          (lambda n=2 * 3: [np.float64(4.0)] * n))   # projections of order one, rows of the caches likewise: 1e-3 of 4
+    def _(B=_B, K=_K, kvh=_kvh, rep=_rep, T=_T, hd=_hd, normed=_normed):
+        """Two decode steps of an attention block (llama.rs:285-345): the q / k / v projections of one activation row
+        per batch entry (with `normed` the RMS norm of a residual stream that an o projection's store produced),
+        heads split off, rotary embedding at the new position (helpers/rope.rs:423-447), k and v appended to caches of
+        T rows (helpers/cache.rs:64-74; the first append moves the cache into a buffer with room, the second lands
+        behind it), attention over the grown caches.  Where the extents allow it the embedding and the append run in
+        the stores of the three products."""
+        H = kvh * rep
+        r_ = np.random.default_rng(4400 + K + T)
+        sc = np.float32(1.0 / np.sqrt(K))
+        xs = [r_.standard_normal((B, 1, K)).astype(np.float32) for _ in range(2)]
+        res = [r_.standard_normal((B, 1, K)).astype(np.float32) for _ in range(2)]
+        wo = r_.standard_normal((K, K)).astype(np.float32) * sc
+        gm = (1.0 + 0.1 * r_.standard_normal(K)).astype(np.float32)
+        wq = r_.standard_normal((H * hd, K)).astype(np.float32) * sc
+        wk = r_.standard_normal((kvh * hd, K)).astype(np.float32) * sc
+        wv = r_.standard_normal((kvh * hd, K)).astype(np.float32) * sc
+        ck = r_.standard_normal((B, kvh, T, hd)).astype(np.float32)
+        cv = r_.standard_normal((B, kvh, T, hd)).astype(np.float32)
+        ang = r_.uniform(0, 6.28, (T + 2, hd)).astype(np.float32)
+        cos_t, sin_t = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+
+        def run(be):
+            k_cache, v_cache = be.from_numpy(ck), be.from_numpy(cv)
+            tcos, tsin = be.from_numpy(cos_t), be.from_numpy(sin_t)
+            weights = [be.from_numpy(w) for w in (wq, wk, wv)]
+            outs = []
+            for step in range(2):
+                pos = T + step
+                if normed:
+                    h = be.add(be.from_numpy(res[step]).move(), _linear(be, be.from_numpy(xs[step]), be.from_numpy(wo)).move())
+                    xn = _rmsnorm_ops(be, h, be.from_numpy(gm), K, (B, 1, K))
+                    del h
+                else:
+                    xn = be.from_numpy(xs[step])
+                q, k, v = (_linear(be, xn, w) for w in weights)
+                del xn
+
+                def heads(t, n):
+                    return be.transpose(be.reshape(t.move(), (B, 1, n, hd)).move(), 1, 2)
+
+                def rope(t, n):
+                    sh = (B, n, 1, hd)
+                    c = be.broadcast(be.reshape(be.slice(tcos, 0, pos, 1).move(), (1, 1, 1, hd)).move(), sh)
+                    s_ = be.broadcast(be.reshape(be.slice(tsin, 0, pos, 1).move(), (1, 1, 1, hd)).move(), sh)
+                    rot = _rot_half(be, t, hd // 2)
+                    return be.add(be.mul(c.move(), t.move()).move(), be.mul(s_.move(), rot.move()).move())
+
+                q, k, v = heads(q, H), heads(k, kvh), heads(v, kvh)
+                q, k = rope(q, H), rope(k, kvh)
+                k_cache = be.concat(k_cache.move(), k.move(), 2)
+                v_cache = be.concat(v_cache.move(), v.move(), 2)
+                outs.append(decode_attention_ops(be, q, k_cache.clone(), v_cache.clone(), rep))
+                outs += [be.slice(k_cache, 2, pos, 1), be.slice(v_cache, 2, pos, 1)]
+            return N(be, *outs)
+
+        def expect():
+            f8 = np.float64
+            K_, V_ = ck.astype(f8), cv.astype(f8)
+            outs = []
+            for step in range(2):
+                pos = T + step
+                x = xs[step].astype(f8)
+                if normed:
+                    h = res[step].astype(f8) + x @ wo.astype(f8).T
+                    x = h / np.sqrt((h * h).mean(-1, keepdims=True) + 1e-5) * gm.astype(f8)
+                q = (x @ wq.astype(f8).T).reshape(B, 1, H, hd).transpose(0, 2, 1, 3)
+                k = (x @ wk.astype(f8).T).reshape(B, 1, kvh, hd).transpose(0, 2, 1, 3)
+                v = (x @ wv.astype(f8).T).reshape(B, 1, kvh, hd).transpose(0, 2, 1, 3)
+                c, s_ = cos_t[pos].astype(f8), sin_t[pos].astype(f8)
+                q, k = _np_rope(q, c, s_), _np_rope(k, c, s_)
+                K_, V_ = np.concatenate([K_, k], 2), np.concatenate([V_, v], 2)
+                outs += [_np_decode_attention(q, K_, V_, rep), k, v]
+            return outs
+
+        return run, expect
+
+
 # ---- prefill attention: many query positions per head, causal ---------------------------------------------------------
 for _B, _kvh, _rep, _S, _T, _hd in ((1, 2, 4, 48, 48, 64), (2, 1, 1, 128, 128, 64), (1, 2, 2, 200, 333, 64), (2, 2, 4, 96, 96, 64),
                                      (1, 1, 3, 70, 70, 64), (1, 1, 1, 9, 500, 64), (1, 2, 2, 64, 64, 128), (2, 1, 4, 200, 333, 128),

@@ -201,6 +201,32 @@ def test_programs_absorbed_by_decode_time_products(hip):
             np.testing.assert_allclose(g, e, rtol=1e-3)
 
 
+def test_rotary_embedding_and_cache_append_run_in_the_products_store(hip):
+    """Two decode steps of an attention block (hidden 2048, 4 rows; hidden 1024, 1 row): the element-wise launches
+    that remain are the two moves of the caches into buffers with room (first append) and the four read-backs of
+    cache rows the case asks for; the rotary embedding of q and k and the writes of the new k / v rows cost none.
+    With hidden 512 the products' kernel does not take the store and they run as a launch of their own per step."""
+    from catgrad_amd import _abi as A
+    from cases import by_name
+
+    for name, ew in (("decode_qkv_rope_append_B4_K2048_kv8_rep4_T300_hd64_normed", 6),
+                     ("decode_qkv_rope_append_B1_K1024_kv2_rep2_T256_hd128", 6),
+                     ("decode_qkv_rope_append_B3_K512_kv4_rep2_T200_hd64", None)):
+        c = by_name(name)
+        hip.sync()
+        hip.profile_enable(A.K_ELEMENTWISE, 1)
+        hip.profile_read(A.K_ELEMENTWISE, True)
+        got = c.run(hip)
+        count = hip.profile_read(A.K_ELEMENTWISE, True)[0]
+        hip.profile_enable(A.K_ELEMENTWISE, 0)
+        if ew is None:
+            assert count > 6, (name, count)
+        else:
+            assert count == ew, (name, count)
+        for g, e in zip(got, c.expect()):
+            np.testing.assert_allclose(g, e, rtol=1e-3, atol=4e-3)
+
+
 def test_backend_closes_with_writes_still_waiting():
     """Rows appended from a program and never read: the write is still waiting when the tensors and the
     backend go away."""
