@@ -17,6 +17,8 @@
 // HBM-bound: K and V once (2 x 4 x T x head_dim bytes per KV head) + the chunk results.
 #pragma once
 
+#include <type_traits>
+
 typedef float float4v __attribute__((ext_vector_type(4)));
 
 // Leaf words of leaves FIRST.. of one work item (leaf 0 of the attention program has no memory).
@@ -234,6 +236,255 @@ __global__ __launch_bounds__(kBlock) void decode_attention_kernel(const AttnArgs
             for (int k = 0; k < TPB; k++) v += red[k][m * LPT + n / 4][n % 4];
             g.part_o[(((uint64_t)b * g.splits + split) * g.M + m) * HD + n] = v;
         }
+    }
+}
+
+// The same attention with ONE workgroup of 1024 threads per query row (and per half of head_dim, see VS) walking all
+// T cached positions: no chunk results, no second launch.  At decode time a KV head's cache is a few hundred KiB to
+// a few MiB, and the chunked pair of kernels spends most of its 20 us waiting (launch, operand offsets, a trip to
+// memory, the hand-over to the combine, its trip).  Here the loads of K are asked for as far ahead as registers
+// allow, the scores of the row wait in LDS, the soft-max program runs once over all of them (the row's maximum and
+// sum cross the waves through LDS), V is on its way while that happens, and the weighted sum is divided by the
+// row's sum where it is stored.  The workgroups of a batch entry (its query rows read the same K and V) get block
+// indices a multiple of eight apart, which lands them on the same XCD: the second to last read hit in its L2.
+// What bounds a workgroup is its compute unit's path to L2, 64 bytes a clock (K and V of 530 positions take
+// 1.8 us through it), and T x head_dim x 4 multiply-adds on one compute unit: taken up to T = 4096, longer caches go
+// to the chunked kernels, which spread a KV head over many workgroups.
+// PASSES x (1024 / LPT) positions per trip to memory.  LOOP: several trips, the next always asked for before the
+// current one is used (PASSES registers twice); else one trip covers T, the soft-max program's other leaves are
+// asked for before K, and with at most ten passes V right behind K (the registers hold both).
+// VS = 2: the workgroup computes all scores but only one half of head_dim of the output, so that twice as many compute
+// units pull on V (used when the launch would otherwise leave half of them idle).
+constexpr int kRowBlock = 1024;
+constexpr int kRowMaxT = 4096;
+template <class P, int LPT, int PASSES, bool LOOP, int VS>
+__global__ __launch_bounds__(kRowBlock) void decode_attention_row_kernel(const AttnArgs g, const FusedArgs a, uint32_t *out) {
+    constexpr int HD = LPT * 4;
+    constexpr int TPB = kRowBlock / LPT; // positions per pass
+    constexpr int SPAN = TPB * PASSES;    // positions per trip to memory
+    constexpr int LPV = LPT / VS;         // lanes per position in the V phase
+    constexpr int TPV = kRowBlock / LPV, PASSES_V = (PASSES + VS - 1) / VS, SPAN_V = TPV * PASSES_V;
+    constexpr int WAVES = kRowBlock / 64;
+    constexpr int IPL = LOOP ? kRowMaxT / kRowBlock : 1; // positions per thread in the soft-max phase
+    constexpr bool V_EARLY = !LOOP && PASSES + PASSES_V <= 20;
+    constexpr int ri0 = reduce_index<P>(0), ri1 = reduce_index<P>(1);
+    constexpr int src0 = P::code[ri0][1], src1 = P::code[ri1][1];
+    static_assert((P::code[ri0][0] & ~kInstrU32) == kRowMax && (P::code[ri1][0] & ~kInstrU32) == kRowSum,
+                  "a soft-max: row maximum, then row sum");
+    static_assert(LOOP || SPAN <= kRowBlock, "one position per thread in the soft-max phase");
+    __shared__ float sc[LOOP ? kRowMaxT : kRowBlock];
+    __shared__ float red[WAVES][HD / VS];
+    __shared__ uint32_t cross[2][WAVES];
+    const uint32_t tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+    const uint32_t T = g.T;
+    // block -> (batch entry, query row, half): the workgroups of an entry eight blocks apart
+    const uint32_t rest = blockIdx.x / 8, inner = rest % (g.M * VS), m = inner / VS, part = inner % VS;
+    const uint32_t b = rest / (g.M * VS) * 8 + blockIdx.x % 8;
+    if (b >= g.splits) return; // (the number of batch entries; the same for the whole workgroup)
+    int64_t oq = 0, ok = 0, ov = 0, op = 0;
+    {
+        uint32_t bb = b;
+        // (every axis slot is visited, so that the fields are read from the argument block up front and at once
+        // instead of one dependent scalar load after the other)
+#pragma unroll
+        for (uint32_t d = 0; d < (uint32_t)kMaxBatchAxes; d++) {
+            if (d >= g.nb) break;
+            const uint32_t q = fastdiv(bb, g.bdiv[d]);
+            const int64_t i = (int64_t)(bb - q * g.bd[d]);
+            bb = q;
+            oq += i * g.q_bs[d];
+            ok += i * g.k_bs[d];
+            ov += i * g.v_bs[d];
+            op += i * g.p_bs[d];
+        }
+    }
+    const uint32_t l = tid % LPT, sub = tid / LPT, lv = tid % LPV, subv = tid / LPV;
+    const uint32_t *kbase = g.Kc + ok + l * 4, *vbase = g.V + ov + (part * LPV + lv) * 4;
+    // FULL (a tag type): the trip lies inside the T positions, nothing is checked
+    const int64_t k_step = (int64_t)TPB * g.k_st, v_step = (int64_t)TPV * g.v_st;
+    auto ask_k = [&](float4v (&f)[PASSES], uint32_t first, auto full) {
+        const uint32_t *p = kbase + (int64_t)(first + sub) * g.k_st;
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ps++) {
+            if constexpr (decltype(full)::value) {
+                f[ps] = *reinterpret_cast<const float4v *>(p);
+            } else {
+                f[ps] = (float4v){0.f, 0.f, 0.f, 0.f};
+                if (first + sub + ps * TPB < T) f[ps] = *reinterpret_cast<const float4v *>(p);
+            }
+            p += k_step;
+        }
+    };
+    auto ask_v = [&](float4v (&f)[PASSES_V], uint32_t first, auto full) {
+        const uint32_t *p = vbase + (int64_t)(first + subv) * g.v_st;
+#pragma unroll
+        for (int ps = 0; ps < PASSES_V; ps++) {
+            if constexpr (decltype(full)::value) {
+                f[ps] = *reinterpret_cast<const float4v *>(p);
+            } else {
+                f[ps] = (float4v){0.f, 0.f, 0.f, 0.f};
+                if (first + subv + ps * TPV < T) f[ps] = *reinterpret_cast<const float4v *>(p);
+            }
+            p += v_step;
+        }
+    };
+    constexpr std::true_type whole_trip{};
+    constexpr std::false_type ragged{};
+    // the trip that starts at `first`, checked only when it reaches beyond T
+    auto ask_k_at = [&](float4v (&f)[PASSES], uint32_t first) {
+        if (first + SPAN <= T) ask_k(f, first, whole_trip);
+        else ask_k(f, first, ragged);
+    };
+    auto ask_v_at = [&](float4v (&f)[PASSES_V], uint32_t first) {
+        if (first + SPAN_V <= T) ask_v(f, first, whole_trip);
+        else ask_v(f, first, ragged);
+    };
+    float4v ka[PASSES], kb[LOOP ? PASSES : 1];
+    float4v va[PASSES_V], vb[LOOP ? PASSES_V : 1];
+    ask_k_at(ka, 0);
+    if constexpr (V_EARLY) ask_v_at(va, 0);
+    const float4v qf = *reinterpret_cast<const float4v *>(g.Q + oq + (int64_t)m * g.q_sm + l * 4);
+    // the soft-max program's other leaves at this thread's positions (tid, tid + 1024, ...)
+    LeafWords<P, 1> w[IPL];
+    int64_t base[P::nleaf + 1];
+    {
+#pragma unroll
+        for (int i = 0; i <= P::nleaf; i++) base[i] = 0;
+        uint32_t rr = (uint32_t)(op / T) + m; // the row in the program's [rows, T] space
+#pragma unroll
+        for (uint32_t d = 0; d < (uint32_t)kMaxOuter; d++) {
+            if (d >= a.g.nouter) break;
+            const uint32_t q = fastdiv(rr, a.g.odiv[d]);
+            const int64_t i = (int64_t)(rr - q * a.g.od[d]);
+            rr = q;
+#pragma unroll
+            for (int lf = 1; lf < P::nleaf; lf++) base[lf] += i * a.leaf[lf].os[d];
+        }
+    }
+    auto fetch_leaves = [&]() {
+#pragma unroll
+        for (int c = 0; c < IPL; c++)
+            if (tid + c * kRowBlock < T) aot_fetch_from<P, 1>(a, base, tid + c * kRowBlock, w[c]);
+    };
+    if constexpr (!LOOP) fetch_leaves(); // nothing waits for them yet
+
+    // ---- scores of the whole row
+    auto score = [&](const float4v (&f)[PASSES], uint32_t first, auto full) {
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ps++) {
+            const uint32_t t = first + sub + ps * TPB;
+            if (decltype(full)::value || first + ps * TPB < T) { // the same for the whole workgroup
+                float v = fmaf(qf[3], f[ps][3], fmaf(qf[2], f[ps][2], fmaf(qf[1], f[ps][1], qf[0] * f[ps][0])));
+                v = row16_sum(v);
+                if (LPT == 32) v += __shfl_xor(v, 16);
+                if (l == 0 && (decltype(full)::value || t < T)) sc[t] = v;
+            }
+        }
+    };
+    auto score_at = [&](const float4v (&f)[PASSES], uint32_t first) {
+        if (first + SPAN <= T) score(f, first, whole_trip);
+        else score(f, first, ragged);
+    };
+    if constexpr (LOOP) {
+        for (uint32_t first = 0; first < T; first += 2 * SPAN) {
+            if (first + SPAN < T) ask_k_at(kb, first + SPAN);
+            score_at(ka, first);
+            if (first + 2 * SPAN < T) ask_k_at(ka, first + 2 * SPAN);
+            if (first + SPAN < T) score_at(kb, first + SPAN);
+        }
+    } else {
+        score_at(ka, 0);
+    }
+    if constexpr (!V_EARLY) ask_v_at(va, 0); // on its way through the soft-max
+    if constexpr (LOOP) fetch_leaves();
+    __syncthreads();
+
+    // ---- the soft-max program over the row
+    float total;
+    {
+        uint32_t rs[kMaxRowReduce] = {0, 0, 0};
+        uint32_t acc = row_init(true, true);
+#pragma unroll
+        for (int c = 0; c < IPL; c++) {
+            const uint32_t i = tid + c * kRowBlock;
+            if (i < T) {
+                w[c].v[0][0] = asu(sc[i]); // leaf 0 is the score
+                const Values<P, 1> s = aot_eval<P, 1, ri0>(w[c], rs, a.fault);
+                acc = row_merge(true, true, acc, s.v[src0][0]);
+            }
+        }
+#pragma unroll
+        for (int sft = 32; sft >= 1; sft >>= 1) acc = row_merge(true, true, acc, (uint32_t)__shfl_xor((int)acc, sft));
+        if (lane == 0) cross[0][wave] = acc;
+        __syncthreads();
+        acc = cross[0][0];
+#pragma unroll
+        for (int k = 1; k < WAVES; k++) acc = row_merge(true, true, acc, cross[0][k]);
+        rs[0] = acc;
+        uint32_t sum = row_init(false, true);
+#pragma unroll
+        for (int c = 0; c < IPL; c++) {
+            const uint32_t i = tid + c * kRowBlock;
+            if (i < T) {
+                const Values<P, 1> s = aot_eval<P, 1, ri1>(w[c], rs, a.fault);
+                sum = row_merge(false, true, sum, s.v[src1][0]);
+                sc[i] = asf(s.v[src1][0]); // the un-normalised weight
+            }
+        }
+#pragma unroll
+        for (int sft = 32; sft >= 1; sft >>= 1) sum = row_merge(false, true, sum, (uint32_t)__shfl_xor((int)sum, sft));
+        if (lane == 0) cross[1][wave] = sum;
+        __syncthreads();
+        sum = cross[1][0];
+#pragma unroll
+        for (int k = 1; k < WAVES; k++) sum = row_merge(false, true, sum, cross[1][k]);
+        total = asf(sum);
+    }
+
+    // ---- weights times V (this workgroup's columns)
+    float4v o = {0.f, 0.f, 0.f, 0.f};
+    auto weigh = [&](const float4v (&f)[PASSES_V], uint32_t first, auto full) {
+#pragma unroll
+        for (int ps = 0; ps < PASSES_V; ps++) {
+            const uint32_t t = first + subv + ps * TPV;
+            if (decltype(full)::value || t < T) {
+                const float wgt = sc[t];
+                o[0] = fmaf(wgt, f[ps][0], o[0]);
+                o[1] = fmaf(wgt, f[ps][1], o[1]);
+                o[2] = fmaf(wgt, f[ps][2], o[2]);
+                o[3] = fmaf(wgt, f[ps][3], o[3]);
+            }
+        }
+    };
+    auto weigh_at = [&](const float4v (&f)[PASSES_V], uint32_t first) {
+        if (first + SPAN_V <= T) weigh(f, first, whole_trip);
+        else weigh(f, first, ragged);
+    };
+    if constexpr (LOOP) {
+        for (uint32_t first = 0; first < T; first += 2 * SPAN_V) {
+            if (first + SPAN_V < T) ask_v_at(vb, first + SPAN_V);
+            weigh_at(va, first);
+            if (first + 2 * SPAN_V < T) ask_v_at(va, first + 2 * SPAN_V);
+            if (first + SPAN_V < T) weigh_at(vb, first + SPAN_V);
+        }
+    } else {
+        weigh_at(va, 0);
+    }
+    // the wave's position groups (lanes lv, lv + LPV, ...) first, then the waves through LDS
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        float v = o[j];
+#pragma unroll
+        for (int sft = LPV; sft < 64; sft <<= 1) v += __shfl_xor(v, sft);
+        o[j] = v;
+    }
+    if (lane < LPV) *reinterpret_cast<float4v *>(&red[wave][lv * 4]) = o;
+    __syncthreads();
+    if (tid < HD / VS) {
+        float v = 0.0f;
+#pragma unroll
+        for (int k = 0; k < WAVES; k++) v += red[k][tid];
+        out[((uint64_t)b * g.M + m) * HD + part * (HD / VS) + tid] = asu(v / total);
     }
 }
 

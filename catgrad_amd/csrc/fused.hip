@@ -593,6 +593,19 @@ static int64_t attn_blocks() {
     return n;
 }
 
+// Longest cache that the one-workgroup-per-KV-head attention kernel takes (env CG_ATTN_WHOLE_T, for measurements).
+static int64_t attn_whole_limit() {
+    static const int64_t n = [] { const char *e = getenv("CG_ATTN_WHOLE_T"); return e ? atoll(e) : 4096ll; }();
+    return n;
+}
+
+// Launches of the one-workgroup-per-row attention kernel with fewer workgroups than this split each row's output in
+// two halves (env CG_ATTN_HALVES_BELOW, for measurements; 0: never).
+static int64_t attn_row_halves_below() {
+    static const int64_t n = [] { const char *e = getenv("CG_ATTN_HALVES_BELOW"); return e ? atoll(e) : 256ll; }();
+    return n;
+}
+
 int launch_decode_attention(cg_backend *be, const Pending &p, const int64_t *pdims, int prank, const cg_tensor *q,
                             const cg_tensor *kt, const cg_tensor *v, cg_tensor *out) {
     if (int frc = flush_deferred(be)) return frc;
@@ -662,6 +675,31 @@ int launch_decode_attention(cg_backend *be, const Pending &p, const int64_t *pdi
     g.q_sm = f1.a_sm;
     g.k_st = f1.b_sn;
     g.v_st = f2.b_sk;
+    // a cache short enough for one workgroup per query row: one launch, nothing to combine
+    if (T <= std::min<int64_t>(attn_whole_limit(), kRowMaxT)) {
+        be->programs_compiled++;
+        ProfScope prof(be, CG_K_GEMM_SKINNY, distinct_bytes(q) + distinct_bytes(kt) + distinct_bytes(v) + distinct_bytes(out));
+        uint32_t *const po = static_cast<uint32_t *>(out->buf->ptr);
+        g.splits = (uint32_t)f1.batch; // (this kernel has no chunks: the field carries the number of batch entries)
+        const int64_t per_pass = hd == 64 ? kRowBlock / 16 : kRowBlock / 32;
+        const int passes = T <= 5 * per_pass ? 5 : T <= 10 * per_pass ? 10 : T <= 16 * per_pass ? 16 : 0;
+        const bool halves = f1.batch * g.M * 2 <= attn_row_halves_below(); // two workgroups per row still leave compute units idle
+        const dim3 grid((uint32_t)((f1.batch + 7) / 8 * 8 * g.M * (halves ? 2 : 1))), block(kRowBlock);
+#define CG_ROW_KERNEL(LPT, VS)                                                                                                     \
+    do {                                                                                                                           \
+        if (passes == 5) hipLaunchKernelGGL((decode_attention_row_kernel<P, LPT, 5, false, VS>), grid, block, 0, be->stream, g, a, po);   \
+        else if (passes == 10) hipLaunchKernelGGL((decode_attention_row_kernel<P, LPT, 10, false, VS>), grid, block, 0, be->stream, g, a, po); \
+        else if (passes == 16) hipLaunchKernelGGL((decode_attention_row_kernel<P, LPT, 16, false, VS>), grid, block, 0, be->stream, g, a, po); \
+        else hipLaunchKernelGGL((decode_attention_row_kernel<P, LPT, 6, true, VS>), grid, block, 0, be->stream, g, a, po);          \
+    } while (0)
+        if (hd == 64 && halves) CG_ROW_KERNEL(16, 2);
+        else if (hd == 64) CG_ROW_KERNEL(16, 1);
+        else if (halves) CG_ROW_KERNEL(32, 2);
+        else CG_ROW_KERNEL(32, 1);
+#undef CG_ROW_KERNEL
+        hipError_t e = hipGetLastError();
+        return e == hipSuccess ? CG_OK : hip_fail(e, "decode attention launch");
+    }
     const size_t o_bytes = (size_t)f1.batch * g.splits * g.M * hd * 4, ml_bytes = (size_t)f1.batch * g.splits * g.M * 2 * 4;
     void *po = nullptr, *pml = nullptr;
     size_t co = 0, cml = 0;
