@@ -676,7 +676,9 @@ int launch_decode_attention(cg_backend *be, const Pending &p, const int64_t *pdi
     g.k_st = f1.b_sn;
     g.v_st = f2.b_sk;
     // a cache short enough for one workgroup per query row: one launch, nothing to combine
-    if (T <= std::min<int64_t>(attn_whole_limit(), kRowMaxT)) {
+    // (beyond 1024 positions only while its workgroups fit the compute units in one round: a row costs its compute
+    // unit T x head_dim x 4 multiply-adds, the chunked kernels spread that over as many workgroups as they like)
+    if (T <= std::min<int64_t>(attn_whole_limit(), kRowMaxT) && (T <= 1024 || f1.batch * f1.M <= 256)) {
         be->programs_compiled++;
         ProfScope prof(be, CG_K_GEMM_SKINNY, distinct_bytes(q) + distinct_bytes(kt) + distinct_bytes(v) + distinct_bytes(out));
         uint32_t *const po = static_cast<uint32_t *>(out->buf->ptr);
