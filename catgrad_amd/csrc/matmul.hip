@@ -9,17 +9,28 @@
 // axes form one run, the batch is folded into M (one tall GEMM instead of B small ones).
 //
 // Kernels
-//   mfma_gemm_kernel   128x128x32 macro tile, 256 threads = 2x2 waves, each wave a 64x64
-//                      quadrant as 2x2 v_mfma_f32_32x32x2_f32 accumulators (64 VGPRs).
-//                      A and B tiles are staged K-fastest in LDS (pitch 36 words: 128-bit
-//                      fragment reads and tile stores are both free of bank conflicts),
-//                      two LDS buffers (72 KiB, dynamic), next tile's global loads in
-//                      flight during the MFMAs.  MFMA-bound: 2*M*N*K flop.
-//   skinny_kt_*        M <= 8 with K-contiguous B rows (decode-time linear layers and
-//                      q.K^T): a wave per output column (or per 4 columns, or a column per
-//                      16/32 lanes for short K), 16-byte loads along K, wave shuffle
-//                      reduction; skinny_kt_mfma_xreg_kernel does the gate/up-sized
-//                      products on the 4x4x1 matrix instruction.  HBM-bound: 4*K*N bytes of B.
+//   mfma_gemm_kernel   256 threads = 2x2 waves, one template for three macro tiles: 256x256x32 (each
+//                      wave a 128x128 block as 4x4 v_mfma_f32_32x32x2_f32 accumulators, all 256
+//                      accumulation registers, 144 KiB of LDS) whenever the product has at least
+//                      one such tile per compute unit, 128x128x32 (2x2 accumulators per wave) for
+//                      smaller products, 128x64x32 when N is a small multiple of 64; a HALF variant
+//                      narrows the tiles to bf16 / f16 on their way into LDS and issues
+//                      v_mfma_f32_32x32x16_{bf16,f16}.  A and B tiles are staged K-fastest in LDS
+//                      (pitch 36 words: 128-bit fragment reads and tile stores are both free of
+//                      bank conflicts), two LDS buffers, next tile's global loads in flight during
+//                      the MFMAs, XCD-aware tile order.  MFMA-bound: 2*M*N*K flop.
+//   skinny_kt_*        M <= 8 with K-contiguous B rows (decode-time linear layers and q.K^T),
+//                      HBM-bound streams of B (4*K*N bytes):
+//                      skinny_kt_wide / _narrow: a wave per output column (or per 4 columns, or a
+//                      column per 16/32 lanes for short K), 16-byte loads along K, wave shuffle
+//                      reduction;
+//                      skinny_kt_mfma_xreg_*: M <= 4 on the 4x4x1 matrix instruction with the
+//                      activations held in registers, in the variants the decode step needs:
+//                      _group (products that share their left operand in one launch), _group_rope
+//                      (the same with the rotary embedding and the KV-cache row writes in the
+//                      store), _gated / _cols_gated (two products and SiLU(g)*u in one launch),
+//                      _residual (the residual adds in the store, row sums of squares left
+//                      behind), _norm (an RMS norm applied to the left operand while it loads).
 //   skinny_nn_kernel   M <= 8 with N-contiguous B rows (p.V of a decode step), split over K
 //                      with a second pass that adds the partial sums.
 //   simple_gemm_kernel u32 (wrapping) and any shape the others decline.
