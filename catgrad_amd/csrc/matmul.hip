@@ -91,7 +91,8 @@ typedef float float16v __attribute__((ext_vector_type(16)));
 // registers: TR*BK/4/256 float4 slots per thread.  Layout of the float4 slots of a tile:
 //   K-contiguous source (s_k == 1): slot = row*(BK/4) + kq  (float4 along k; 8 lanes read
 //                                                            128 contiguous bytes of a row)
-//   R-contiguous source (s_r == 1): slot = k*(TR/4) + rq    (float4 along rows)
+//   R-contiguous source (s_r == 1): float4 along rows; a wave's 64 slots are 16 row-quads x 4 values of k
+//                                   (rows_fast_slot), so that its LDS stores spread over all banks
 //   otherwise                      : as K-contiguous, element by element
 template <int TR> struct TileRegs {
     static constexpr int slots = TR * BK / 4 / 256;
@@ -99,6 +100,19 @@ template <int TR> struct TileRegs {
 };
 
 __device__ __forceinline__ float ld_guard(const uint32_t *p, bool ok) { return ok ? asf(*p) : 0.0f; }
+
+// Slot -> (first of four rows, k) of a tile whose rows are the unit-stride axis in memory.  The tile is staged K-fastest
+// in LDS, so a lane's four values go to four different LDS rows, one 4-byte store each.  With a whole wave on one k (64
+// row-quads) those stores hit 2 of the 32 banks; with 16 row-quads x 4 consecutive k per wave, and each lane writing its
+// four rows in an order rotated by its row-quad (rows_fast_order), a wave's store covers all 32 banks twice, which is the
+// best 64 lanes can do.  Global loads stay 256 contiguous bytes per k.
+template <int TR> __device__ __forceinline__ void rows_fast_slot(uint32_t slot, uint32_t &row, uint32_t &k) {
+    const uint32_t group = slot / 64, in = slot % 64;
+    row = (group % (TR / 64)) * 64 + (in % 16) * 4;
+    k = (group / (TR / 64)) * 4 + in / 16;
+}
+__device__ __forceinline__ uint32_t rows_fast_order(uint32_t slot, int i) { return ((uint32_t)i + ((slot % 16) >> 1)) & 3u; }
+__device__ __forceinline__ float pick4(const float4v &v, uint32_t j) { return j == 0 ? v[0] : j == 1 ? v[1] : j == 2 ? v[2] : v[3]; }
 
 template <bool ROWS_FAST, int TR>
 __device__ __forceinline__ void load_tile(TileRegs<TR> &t, const uint32_t *base, int64_t s_r, int64_t s_k, uint32_t r0,
@@ -119,7 +133,10 @@ __device__ __forceinline__ void load_tile(TileRegs<TR> &t, const uint32_t *base,
                 t.v[h][3] = ld_guard(p + 3 * s_k, rok && k + 3 < K);
             }
         } else {
-            uint32_t k = k0 + slot / (TR / 4), row = r0 + (slot % (TR / 4)) * 4;
+            uint32_t row, k;
+            rows_fast_slot<TR>(slot, row, k);
+            row += r0;
+            k += k0;
             const uint32_t *p = base + (int64_t)row * s_r + (int64_t)k * s_k;
             if (vec_ok && k < K && row + 3 < R) {
                 t.v[h] = *reinterpret_cast<const float4v *>(p);
@@ -143,11 +160,13 @@ template <bool ROWS_FAST, int TR> __device__ __forceinline__ void store_tile(con
             uint32_t row = slot / (BK / 4), k = (slot % (BK / 4)) * 4;
             *reinterpret_cast<float4v *>(lds + row * PITCH + k) = t.v[h];
         } else {
-            uint32_t k = slot / (TR / 4), row = (slot % (TR / 4)) * 4;
-            lds[(row + 0) * PITCH + k] = t.v[h][0];
-            lds[(row + 1) * PITCH + k] = t.v[h][1];
-            lds[(row + 2) * PITCH + k] = t.v[h][2];
-            lds[(row + 3) * PITCH + k] = t.v[h][3];
+            uint32_t row, k;
+            rows_fast_slot<TR>(slot, row, k);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const uint32_t j = rows_fast_order(slot, i);
+                lds[(row + j) * PITCH + k] = pick4(t.v[h], j);
+            }
         }
     }
 }
@@ -184,10 +203,14 @@ template <bool ROWS_FAST, int HALF, int TR> __device__ __forceinline__ void stor
             w.y = pack_halves<HALF>(t.v[h][2], t.v[h][3]);
             *reinterpret_cast<uint2 *>(lds + row * PITCH_H + k / 2) = w;
         } else {
-            uint32_t k = slot / (TR / 4), row = (slot % (TR / 4)) * 4;
+            uint32_t row, k;
+            rows_fast_slot<TR>(slot, row, k);
             uint16_t *l16 = reinterpret_cast<uint16_t *>(lds);
 #pragma unroll
-            for (int i = 0; i < 4; i++) l16[(row + i) * (PITCH_H * 2) + k] = narrow_half<HALF>(t.v[h][i]);
+            for (int i = 0; i < 4; i++) {
+                const uint32_t j = rows_fast_order(slot, i);
+                l16[(row + j) * (PITCH_H * 2) + k] = narrow_half<HALF>(pick4(t.v[h], j));
+            }
         }
     }
 }
@@ -313,12 +336,21 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
                                                                                __builtin_bit_cast(f16x8, fb[j]), acc[i][j], 0, 0, 0);
                     }
             }
+        } else if constexpr (MT == 4) {
+            // one wave per SIMD: nobody else fills the time the staging of the next tile takes (for a row-contiguous
+            // operand 4-byte LDS stores and their addresses), so it goes between the two halves of the burst, by when
+            // the tile's global loads have long arrived; the other LDS buffer is written, the current one read
+#pragma unroll
+            for (int kc = 0; kc < BK / 16; kc++) chunk(kc);
+            if (more) stage(ra, rb, cur ^ 1);
+#pragma unroll
+            for (int kc = BK / 16; kc < BK / 8; kc++) chunk(kc);
         } else {
 #pragma unroll
             for (int kc = 0; kc < BK / 8; kc++) chunk(kc);
         }
         __builtin_amdgcn_s_setprio(0);
-        if (more) stage(ra, rb, cur ^ 1);
+        if (more && (HALF || MT != 4)) stage(ra, rb, cur ^ 1);
         __syncthreads();
     }
 
