@@ -266,3 +266,87 @@ def test_random_decoder_blocks_match_oracle(hip, oracle, seed):
         assert err <= 1e-3 * max(4.0, float(np.abs(ref[name]).max())), f"seed {seed} B={B} H={H} F={F} kv={kv} {name} order={order}: {err}"
     if two_norm_uses:
         np.testing.assert_allclose(gx, rx, rtol=1e-4, atol=1e-4)
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_random_attention_block_steps_match_oracle(hip, oracle, seed):
+    """Decode steps of a whole attention block (q / k / v projections, heads split off, rotary embedding, cache append,
+    attention) at random row counts, widths, head counts and sizes and cache lengths, with or without an RMS norm of a
+    residual stream in front, and with random extra holders of the intermediate handles (a clone of a projection or of
+    a roped tensor that is read later, the roped q read back before the attention): who else holds a product decides
+    whether the embedding and the append may run in the products' store.  1e-3 of the values' scale (order one)."""
+    import cases
+
+    rng = np.random.default_rng(11000 + seed)
+    B = int(rng.integers(1, 6))
+    K = int(rng.choice([1024, 2048, 2048, 3072, 512]))
+    hd = int(rng.choice([64, 64, 128, 32]))
+    kvh, rep = int(rng.integers(1, 5)), int(rng.choice([1, 2, 4]))
+    H = kvh * rep
+    T = int(rng.choice([int(rng.integers(1, 40)), int(rng.integers(200, 700)), int(rng.integers(1000, 2300))]))
+    steps = int(rng.integers(1, 4))
+    normed = bool(rng.random() < 0.5)
+    keep = {n: bool(rng.random() < 0.2) for n in ("q_raw", "k_raw", "v_raw", "q_rope", "k_rope")}
+    read_q_first = bool(rng.random() < 0.25)
+    sc = np.float32(1.0 / np.sqrt(K))
+    r = lambda *s: rng.standard_normal(s).astype(np.float32)  # noqa: E731
+    xs, res = [r(B, 1, K) for _ in range(steps)], [r(B, 1, K) for _ in range(steps)]
+    wo, gm = r(K, K) * sc, (1 + 0.1 * r(K)).astype(np.float32)
+    wq, wk, wv = r(H * hd, K) * sc, r(kvh * hd, K) * sc, r(kvh * hd, K) * sc
+    ck, cv = r(B, kvh, T, hd), r(B, kvh, T, hd)
+    ang = rng.uniform(0, 6.28, (T + steps, hd)).astype(np.float32)
+    cos_t, sin_t = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+
+    def run(be):
+        k_cache, v_cache = be.from_numpy(ck), be.from_numpy(cv)
+        tcos, tsin = be.from_numpy(cos_t), be.from_numpy(sin_t)
+        weights = [be.from_numpy(w) for w in (wq, wk, wv)]
+        outs = []
+        for step in range(steps):
+            pos = T + step
+            held = {}
+            if normed:
+                h = be.add(be.from_numpy(res[step]).move(), cases._linear(be, be.from_numpy(xs[step]), be.from_numpy(wo)).move())
+                xn = cases._rmsnorm_ops(be, h, be.from_numpy(gm), K, (B, 1, K))
+                del h
+            else:
+                xn = be.from_numpy(xs[step])
+            q, k, v = (cases._linear(be, xn, w) for w in weights)
+            del xn
+            for name, t in (("q_raw", q), ("k_raw", k), ("v_raw", v)):
+                if keep[name]:
+                    held[name] = t.clone()
+
+            def heads(t, n):
+                return be.transpose(be.reshape(t.move(), (B, 1, n, hd)).move(), 1, 2)
+
+            def rope(t, n):
+                sh = (B, n, 1, hd)
+                c = be.broadcast(be.reshape(be.slice(tcos, 0, pos, 1).move(), (1, 1, 1, hd)).move(), sh)
+                s_ = be.broadcast(be.reshape(be.slice(tsin, 0, pos, 1).move(), (1, 1, 1, hd)).move(), sh)
+                rot = cases._rot_half(be, t, hd // 2)
+                return be.add(be.mul(c.move(), t.move()).move(), be.mul(s_.move(), rot.move()).move())
+
+            q, k, v = heads(q, H), heads(k, kvh), heads(v, kvh)
+            q, k = rope(q, H), rope(k, kvh)
+            if keep["q_rope"]:
+                held["q_rope"] = q.clone()
+            if keep["k_rope"]:
+                held["k_rope"] = k.clone()
+            k_cache = be.concat(k_cache.move(), k.move(), 2)
+            v_cache = be.concat(v_cache.move(), v.move(), 2)
+            if read_q_first:
+                outs.append(be.to_numpy(q))
+            outs.append(be.to_numpy(cases.decode_attention_ops(be, q, k_cache.clone(), v_cache.clone(), rep)))
+            outs += [be.to_numpy(be.slice(k_cache, 2, pos, 1)), be.to_numpy(be.slice(v_cache, 2, pos, 1))]
+            outs += [be.to_numpy(held[n]) for n in sorted(held)]
+        outs.append(be.to_numpy(k_cache))
+        return outs
+
+    got, ref = run(hip), run(oracle)
+    assert len(got) == len(ref)
+    what = f"seed {seed}: B={B} K={K} hd={hd} kvh={kvh} rep={rep} T={T} steps={steps} normed={normed} keep={keep} read_q_first={read_q_first}"
+    for i, (g, e) in enumerate(zip(got, ref)):
+        assert g.shape == e.shape, what
+        err = float(np.abs(g.astype(np.float64) - e).max())
+        assert err <= 1e-3 * max(4.0, float(np.abs(e).max())), f"{what} output {i}: {err}"
