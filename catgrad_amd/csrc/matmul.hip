@@ -572,8 +572,11 @@ struct MmGroup {
     uint32_t n;
 };
 __device__ __forceinline__ uint32_t group_problem(const MmGroup &g, uint32_t &block_x) {
+    // every slot of the prefix table is compared (the problems are in increasing order of their first workgroup), so the
+    // table is read from the argument block at once instead of one dependent scalar load per problem
     uint32_t p = 0;
-    while (p + 1 < g.n && blockIdx.x >= g.first[p + 1]) p++;
+#pragma unroll
+    for (int i = 1; i < kMaxGroup; i++) p += (uint32_t)i < g.n && blockIdx.x >= g.first[i] ? 1u : 0u;
     block_x = blockIdx.x - g.first[p];
     return p;
 }
