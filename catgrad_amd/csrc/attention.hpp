@@ -92,7 +92,11 @@ __global__ __launch_bounds__(kBlock) void decode_attention_kernel(const AttnArgs
     int64_t oq = 0, ok = 0, ov = 0, op = 0;
     {
         uint32_t bb = b;
-        for (uint32_t d = 0; d < g.nb; d++) {
+        // (every axis slot is visited, so that the fields are read from the argument block at once instead of one
+        // dependent scalar load after the other)
+#pragma unroll
+        for (uint32_t d = 0; d < (uint32_t)kMaxBatchAxes; d++) {
+            if (d >= g.nb) break;
             const uint32_t q = fastdiv(bb, g.bdiv[d]);
             const int64_t i = (int64_t)(bb - q * g.bd[d]);
             bb = q;
@@ -152,7 +156,9 @@ __global__ __launch_bounds__(kBlock) void decode_attention_kernel(const AttnArgs
         for (int i = 0; i <= P::nleaf; i++) base[i] = 0;
         {
             uint32_t rr = row;
-            for (uint32_t d = 0; d < a.g.nouter; d++) {
+#pragma unroll
+            for (uint32_t d = 0; d < (uint32_t)kMaxOuter; d++) {
+                if (d >= a.g.nouter) break;
                 const uint32_t q = fastdiv(rr, a.g.odiv[d]);
                 const int64_t i = (int64_t)(rr - q * a.g.od[d]);
                 rr = q;
