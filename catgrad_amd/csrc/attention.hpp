@@ -254,8 +254,9 @@ __global__ __launch_bounds__(kBlock) void decode_attention_kernel(const AttnArgs
 // row's sum where it is stored.  The workgroups of a batch entry (its query rows read the same K and V) get block
 // indices a multiple of eight apart, which lands them on the same XCD: the second to last read hit in its L2.
 // What bounds a workgroup is its compute unit's path to L2, 64 bytes a clock (K and V of 530 positions take
-// 1.8 us through it), and T x head_dim x 4 multiply-adds on one compute unit: taken up to T = 4096, longer caches go
-// to the chunked kernels, which spread a KV head over many workgroups.
+// 1.8 us through it), and T x head_dim x 4 multiply-adds on one compute unit: taken up to T = 4096 in one launch and, in
+// two segments per row whose results decode_attention_combine_kernel merges, up to 8192; longer caches go to the chunked
+// kernels, which spread a KV head over many workgroups.
 // PASSES x (1024 / LPT) positions per trip to memory.  LOOP: several trips, the next always asked for before the
 // current one is used (PASSES registers twice); else one trip covers T, the soft-max program's other leaves are
 // asked for before K, and with at most ten passes V right behind K (the registers hold both).
@@ -282,7 +283,10 @@ __global__ __launch_bounds__(kRowBlock) void decode_attention_row_kernel(const A
     __shared__ float red[WAVES][HD / VS];
     __shared__ uint32_t cross[2][WAVES];
     const uint32_t tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
-    const uint32_t T = g.T;
+    // a cache beyond kRowMaxT positions is cut into segments over grid.y: a workgroup then leaves its segment's maximum,
+    // sum and un-normalised weighted sum for decode_attention_combine_kernel
+    const uint32_t seg = blockIdx.y, t_first = seg * g.chunk;
+    const uint32_t T = min(g.T, t_first + g.chunk) - t_first; // positions of this workgroup
     // block -> (batch entry, query row, half): the workgroups of an entry eight blocks apart
     const uint32_t rest = blockIdx.x / 8, inner = rest % (g.M * VS), m = inner / VS, part = inner % VS;
     const uint32_t b = rest / (g.M * VS) * 8 + blockIdx.x % 8;
@@ -305,7 +309,8 @@ __global__ __launch_bounds__(kRowBlock) void decode_attention_row_kernel(const A
         }
     }
     const uint32_t l = tid % LPT, sub = tid / LPT, lv = tid % LPV, subv = tid / LPV;
-    const uint32_t *kbase = g.Kc + ok + l * 4, *vbase = g.V + ov + (part * LPV + lv) * 4;
+    const uint32_t *kbase = g.Kc + ok + (int64_t)t_first * g.k_st + l * 4;
+    const uint32_t *vbase = g.V + ov + (int64_t)t_first * g.v_st + (part * LPV + lv) * 4;
     // FULL (a tag type): the trip lies inside the T positions, nothing is checked
     const int64_t k_step = (int64_t)TPB * g.k_st, v_step = (int64_t)TPV * g.v_st;
     auto ask_k = [&](float4v (&f)[PASSES], uint32_t first, auto full) {
@@ -356,7 +361,7 @@ __global__ __launch_bounds__(kRowBlock) void decode_attention_row_kernel(const A
     {
 #pragma unroll
         for (int i = 0; i <= P::nleaf; i++) base[i] = 0;
-        uint32_t rr = (uint32_t)(op / T) + m; // the row in the program's [rows, T] space
+        uint32_t rr = (uint32_t)(op / g.T) + m; // the row in the program's [rows, T] space
 #pragma unroll
         for (uint32_t d = 0; d < (uint32_t)kMaxOuter; d++) {
             if (d >= a.g.nouter) break;
@@ -370,7 +375,7 @@ __global__ __launch_bounds__(kRowBlock) void decode_attention_row_kernel(const A
     auto fetch_leaves = [&]() {
 #pragma unroll
         for (int c = 0; c < IPL; c++)
-            if (tid + c * kRowBlock < T) aot_fetch_from<P, 1>(a, base, tid + c * kRowBlock, w[c]);
+            if (tid + c * kRowBlock < T) aot_fetch_from<P, 1>(a, base, t_first + tid + c * kRowBlock, w[c]);
     };
     if constexpr (!LOOP) fetch_leaves(); // nothing waits for them yet
 
@@ -406,7 +411,7 @@ __global__ __launch_bounds__(kRowBlock) void decode_attention_row_kernel(const A
     __syncthreads();
 
     // ---- the soft-max program over the row
-    float total;
+    float total, row_max;
     {
         uint32_t rs[kMaxRowReduce] = {0, 0, 0};
         uint32_t acc = row_init(true, true);
@@ -427,6 +432,7 @@ __global__ __launch_bounds__(kRowBlock) void decode_attention_row_kernel(const A
 #pragma unroll
         for (int k = 1; k < WAVES; k++) acc = row_merge(true, true, acc, cross[0][k]);
         rs[0] = acc;
+        row_max = asf(acc);
         uint32_t sum = row_init(false, true);
 #pragma unroll
         for (int c = 0; c < IPL; c++) {
@@ -490,7 +496,16 @@ __global__ __launch_bounds__(kRowBlock) void decode_attention_row_kernel(const A
         float v = 0.0f;
 #pragma unroll
         for (int k = 0; k < WAVES; k++) v += red[k][tid];
-        out[((uint64_t)b * g.M + m) * HD + part * (HD / VS) + tid] = asu(v / total);
+        if (g.part_o) {
+            const uint64_t at = ((uint64_t)b * gridDim.y + seg) * g.M + m;
+            g.part_o[at * HD + part * (HD / VS) + tid] = v;
+            if (tid == 0 && part == 0) {
+                g.part_ml[at * 2] = row_max;
+                g.part_ml[at * 2 + 1] = total;
+            }
+        } else {
+            out[((uint64_t)b * g.M + m) * HD + part * (HD / VS) + tid] = asu(v / total);
+        }
     }
 }
 

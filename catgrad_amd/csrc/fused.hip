@@ -599,6 +599,14 @@ static int64_t attn_whole_limit() {
     return n;
 }
 
+// Longest cache that the one-workgroup-per-row attention kernel takes in segments (env CG_ATTN_SEGMENT_T, for measurements).
+// Measured at 128 query rows: 6000 positions in 25.9 + 4.1 us against 33.0 + 7.6 for the chunked pair, 12000 positions (three
+// segments, one and a half rounds of workgroups) in 56 + 4 against 47 + 11.
+static int64_t attn_segment_limit() {
+    static const int64_t n = [] { const char *e = getenv("CG_ATTN_SEGMENT_T"); return e ? atoll(e) : 8192ll; }();
+    return n;
+}
+
 // Launches of the one-workgroup-per-row attention kernel with fewer workgroups than this split each row's output in
 // two halves (env CG_ATTN_HALVES_BELOW, for measurements; 0: never).
 static int64_t attn_row_halves_below() {
@@ -675,18 +683,38 @@ int launch_decode_attention(cg_backend *be, const Pending &p, const int64_t *pdi
     g.q_sm = f1.a_sm;
     g.k_st = f1.b_sn;
     g.v_st = f2.b_sk;
-    // a cache short enough for one workgroup per query row: one launch, nothing to combine
-    // (beyond 1024 positions only while its workgroups fit the compute units in one round: a row costs its compute
-    // unit T x head_dim x 4 multiply-adds, the chunked kernels spread that over as many workgroups as they like)
-    if (T <= std::min<int64_t>(attn_whole_limit(), kRowMaxT) && (T <= 1024 || f1.batch * f1.M <= 256)) {
+    // One workgroup per query row: a cache of up to kRowMaxT positions in one launch with nothing to combine (beyond
+    // 1024 positions only while the workgroups fit the compute units in one round: a row costs its compute unit
+    // T x head_dim x 4 multiply-adds); longer caches in segments of at most kRowMaxT positions per workgroup, merged by the
+    // combine kernel.  Everything else goes to the chunked kernel below, which spreads a KV head over many workgroups.
+    const int64_t qrows = f1.batch * f1.M;
+    const bool one_launch = T <= std::min<int64_t>(attn_whole_limit(), kRowMaxT) && (T <= 1024 || qrows <= 256);
+    const bool segmented = !one_launch && attn_whole_limit() > 0 && T > kRowMaxT && T <= attn_segment_limit() && qrows <= 256;
+    if (one_launch || segmented) {
         be->programs_compiled++;
         ProfScope prof(be, CG_K_GEMM_SKINNY, distinct_bytes(q) + distinct_bytes(kt) + distinct_bytes(v) + distinct_bytes(out));
         uint32_t *const po = static_cast<uint32_t *>(out->buf->ptr);
+        const uint32_t nseg = segmented ? (uint32_t)((T + kRowMaxT - 1) / kRowMaxT) : 1u;
+        const int64_t seglen = segmented ? ((T + nseg - 1) / nseg + 63) / 64 * 64 : T;
+        g.chunk = (uint32_t)seglen;
         g.splits = (uint32_t)f1.batch; // (this kernel has no chunks: the field carries the number of batch entries)
+        void *part_o = nullptr, *part_ml = nullptr;
+        size_t co = 0, cml = 0;
+        if (segmented) {
+            rc = be->pool.alloc((size_t)f1.batch * nseg * g.M * hd * 4, &part_o, &co);
+            if (rc) return rc;
+            rc = be->pool.alloc((size_t)f1.batch * nseg * g.M * 2 * 4, &part_ml, &cml);
+            if (rc) {
+                be->pool.free(part_o, co);
+                return rc;
+            }
+        }
+        g.part_o = static_cast<float *>(part_o);
+        g.part_ml = static_cast<float *>(part_ml);
         const int64_t per_pass = hd == 64 ? kRowBlock / 16 : kRowBlock / 32;
-        const int passes = T <= 5 * per_pass ? 5 : T <= 10 * per_pass ? 10 : T <= 16 * per_pass ? 16 : 0;
-        const bool halves = f1.batch * g.M * 2 <= attn_row_halves_below(); // two workgroups per row still leave compute units idle
-        const dim3 grid((uint32_t)((f1.batch + 7) / 8 * 8 * g.M * (halves ? 2 : 1))), block(kRowBlock);
+        const int passes = seglen <= 5 * per_pass ? 5 : seglen <= 10 * per_pass ? 10 : seglen <= 16 * per_pass ? 16 : 0;
+        const bool halves = qrows * nseg * 2 <= attn_row_halves_below(); // two workgroups per row still leave compute units idle
+        const dim3 grid((uint32_t)((f1.batch + 7) / 8 * 8 * g.M * (halves ? 2 : 1)), nseg), block(kRowBlock);
 #define CG_ROW_KERNEL(LPT, VS)                                                                                                     \
     do {                                                                                                                           \
         if (passes == 5) hipLaunchKernelGGL((decode_attention_row_kernel<P, LPT, 5, false, VS>), grid, block, 0, be->stream, g, a, po);   \
@@ -699,6 +727,13 @@ int launch_decode_attention(cg_backend *be, const Pending &p, const int64_t *pdi
         else if (halves) CG_ROW_KERNEL(32, 2);
         else CG_ROW_KERNEL(32, 1);
 #undef CG_ROW_KERNEL
+        if (segmented) {
+            const uint64_t nrows = (uint64_t)f1.batch * g.M, waves = kBlock / 64;
+            hipLaunchKernelGGL(decode_attention_combine_kernel, dim3((uint32_t)((nrows + waves - 1) / waves)), dim3(kBlock), 0,
+                               be->stream, g.part_o, g.part_ml, po, nseg, g.M, (uint32_t)hd, nrows);
+            be->pool.free(part_o, co); // stream-ordered: later users queue behind the combine
+            be->pool.free(part_ml, cml);
+        }
         hipError_t e = hipGetLastError();
         return e == hipSuccess ? CG_OK : hip_fail(e, "decode attention launch");
     }

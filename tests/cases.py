@@ -1322,9 +1322,10 @@ def _np_decode_attention(q, k, v, rep):
 for _B, _kvh, _rep, _T, _hd in ((2, 2, 4, 300, 64), (1, 3, 1, 1, 64), (2, 1, 8, 63, 64), (1, 2, 2, 65, 128),
                                 (4, 8, 4, 1000, 64), (1, 1, 3, 257, 128), (2, 2, 4, 40, 32),
                                 # one workgroup per query row in several trips, with and without the split of head_dim, a
-                                # batch that does not fill the last eight block indices, a cache beyond that kernel's reach
+                                # batch that does not fill the last eight block indices, caches it takes in two segments and one
+                                # beyond its reach
                                 (4, 8, 4, 2100, 64), (1, 2, 2, 3000, 128), (5, 8, 4, 700, 64), (9, 1, 8, 1100, 128),
-                                (1, 2, 4, 4500, 64)):
+                                (1, 2, 4, 4500, 64), (2, 2, 4, 9000, 64), (1, 1, 2, 5000, 128), (1, 2, 4, 7000, 64)):
     @case(f"decode_attention_B{_B}_kv{_kvh}_rep{_rep}_T{_T}_hd{_hd}", "ew_abs")
     def _(B=_B, kvh=_kvh, rep=_rep, T=_T, hd=_hd):
         q = f32(400 + T, (B, kvh * rep, 1, hd))
