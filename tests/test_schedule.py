@@ -8,6 +8,7 @@ import numpy as np
 import pytest
 
 import np_models
+from catgrad_amd import _abi as A
 from catgrad_amd.runner import LlmConfig, Session, random_params
 from model_cases import TINY, params_of, prompt_of
 from oracle_loader import ORACLE_LIB, oracle_library
@@ -88,14 +89,17 @@ def test_hip_under_the_reference_schedule(name, cfg, scale, B):
     srt = np.sort(l64, -1)
     gaps = (srt[..., -1] - srt[..., -2]).T
     scale_l = float(np.abs(l_c).max())
-    stats = {}
+    stats, launches = {}, {}
     for schedule in (0, 1, 2):
         hip = Session()
         hip.set_schedule(schedule)
         hip.load_model(cfg, params=params.items())
         hip.program_stats()
+        hip.profile_enable(A.K_ELEMENTWISE, 1)
+        hip.profile_read(A.K_ELEMENTWISE, True)
         g_h, st, l_h = hip.generate(prompt, steps=steps, max_positions=32, want_logits=True)
         stats[schedule] = hip.program_stats()
+        launches[schedule] = hip.profile_read(A.K_ELEMENTWISE, True)[0]
         hip.close()
         err = float(np.abs(l_h - l_c).max())
         print(f"{name} schedule {schedule}: max |dlogit| {err:.3e} (scale {scale_l:.3e}); fused programs compiled / "
@@ -109,3 +113,6 @@ def test_hip_under_the_reference_schedule(name, cfg, scale, B):
     for schedule in (1, 2):
         assert stats[schedule][1] <= stats[0][1]
         assert stats[schedule][0] <= stats[0][0] * 1.02 + 2
+        # nor more element-wise launches: the rotary embedding and the cache rows still go into the q / k / v store
+        assert launches[schedule] <= launches[0] + 2, (launches, name)
+    print(f"{name}: element-wise launches per schedule {launches}", flush=True)
