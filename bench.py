@@ -55,7 +55,7 @@ def micro_bench(iters=20):
     rng = np.random.default_rng(0)
     out = {}
 
-    def run(name, cls, fn, unit, launches_per_call=1):
+    def run(name, cls, fn, unit, launches_per_call=1, mfma_peak=MFMA_F32_PEAK):
         for _ in range(3):
             fn()
         be.sync()
@@ -68,7 +68,7 @@ def micro_bench(iters=20):
         n = n / launches_per_call      # an op of several launches (the two halves of a concat): time and bytes of all
         per = max(ms / max(n, 1) * 1e-3, 1e-12)
         rate = work / max(n, 1) / per
-        peak = MFMA_F32_PEAK if unit == "TFLOP/s" else HBM_PEAK
+        peak = mfma_peak if unit == "TFLOP/s" else HBM_PEAK
         out[name] = {"us": round(per * 1e6, 2), "achieved": round(rate / (1e12 if unit == "TFLOP/s" else 1e9), 2),
                      "unit": unit, "frac": round(rate / peak, 4)}
 
@@ -90,6 +90,19 @@ def micro_bench(iters=20):
     y = be.from_numpy(rng.standard_normal((16, 1024, 1024), dtype=np.float32))
     run("bmm_f32_16x1024x1024x1024", A.K_GEMM_MFMA, lambda: be.matmul(x, y), "TFLOP/s")
     del x, y
+    # a linear layer of the 1B-shape prefill on the narrow dtypes (the reduced-precision row of the path): operands narrowed
+    # to 2-byte / 1-byte patterns in memory (the weight once, the activations inside the timed launch), then the 16-bit /
+    # fp8 matrix instructions; against their dense peaks
+    x32 = be.from_numpy(rng.standard_normal((1, 8192, 2048), dtype=np.float32) * np.float32(0.25))
+    w32 = be.from_numpy(rng.standard_normal((8192, 2048), dtype=np.float32) * np.float32(0.25))
+    for dt, tag, peak in ((A.BF16, "bf16", 2.5e15), (A.F8, "fp8", 5.0e15)):
+        xn, wn = be.cast(x32, dt), be.cast(w32, dt)
+        be.realize(xn)
+        be.realize(wn)
+        wv = be.broadcast(be.transpose(wn, 0, 1), (1, 2048, 8192))
+        run(f"linear_{tag}_8192x2048x8192", A.K_GEMM_MFMA, lambda: be.matmul(xn, wv), "TFLOP/s", mfma_peak=peak)
+        del xn, wn, wv
+    del x32, w32
     # the strided / indexing kernels of the path: a materialised transpose, concat along the outermost and the innermost
     # axis, the embedding gather of the 1B-shape prefill and a sum over a non-last axis (8 bytes per element moved,
     # 4 per element reduced)

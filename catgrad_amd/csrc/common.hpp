@@ -139,6 +139,14 @@ struct Buffer {
     void *side = nullptr;
     size_t side_cls = 0;
     uint32_t side_blocks = 0;
+    // A narrow copy of one 2-D view of this buffer for the matrix instructions of its dtype (launch_matmul): [rows][k] of
+    // 2-byte (f16 / bf16) or 1-byte (fp8) patterns, k contiguous.  A weight matrix is narrowed once and the copy kept while
+    // the buffer lives; what a view shows never changes (in-place appends write behind it), so the copy stays valid.
+    // Owned (pool memory).
+    void *packed = nullptr;
+    size_t packed_cls = 0;
+    int packed_kind = 0; // 1 bf16, 2 f16, 3 fp8
+    int64_t packed_off = 0, packed_rows = 0, packed_k = 0, packed_sr = 0, packed_sk = 0;
 };
 
 } // namespace cg

@@ -13,9 +13,10 @@
 //                      wave a 128x128 block as 4x4 v_mfma_f32_32x32x2_f32 accumulators, all 256
 //                      accumulation registers, 144 KiB of LDS) whenever the product has at least
 //                      one such tile per compute unit, 128x128x32 (2x2 accumulators per wave) for
-//                      smaller products, 128x64x32 when N is a small multiple of 64; a HALF variant
-//                      narrows the tiles to bf16 / f16 on their way into LDS and issues
-//                      v_mfma_f32_32x32x16_{bf16,f16}.  A and B tiles are staged K-fastest in LDS
+//                      smaller products, 128x64x32 when N is a small multiple of 64; HALF variants
+//                      narrow the tiles to bf16 / f16 on their way into LDS, or read operands that
+//                      pack_operand_kernel narrowed in memory (bf16 / f16 / fp8), and issue
+//                      v_mfma_f32_32x32x16_{bf16,f16,fp8_fp8}.  A and B tiles are staged K-fastest in LDS
 //                      (pitch 36 words: 128-bit fragment reads and tile stores are both free of
 //                      bank conflicts), two LDS buffers, next tile's global loads in flight during
 //                      the MFMAs, XCD-aware tile order.  MFMA-bound: 2*M*N*K flop.
@@ -180,6 +181,7 @@ template <bool ROWS_FAST, int TR> __device__ __forceinline__ void store_tile(con
 constexpr int PITCH_H = BK / 2 + 4;
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef long long2v __attribute__((ext_vector_type(2)));
 
 // HALF: 1 bfloat16, 2 binary16
 template <int HALF> __device__ __forceinline__ uint32_t pack_halves(float lo, float hi) {
@@ -221,15 +223,23 @@ template <bool ROWS_FAST, int HALF, int TR> __device__ __forceinline__ void stor
 // 256 accumulation registers, one wave per SIMD: four times the matrix instructions between two
 // barriers and half the LDS traffic per flop, for products with enough tiles to fill the chip.
 // HALF: 0 f32 operands (v_mfma_f32_32x32x2_f32); 1 / 2: bfloat16 / binary16 operands (see above).
+// 3 / 4 / 5: operands that are ALREADY narrow in memory — bfloat16 / binary16 / fp8 (E4M3) patterns, k contiguous,
+// addressed as 32-bit words of 2 or 4 values (a.K counts words; see pack_operand).  The tile pipeline is the f32 one
+// word for word (16-byte global loads, K-fastest LDS rows of 32 words + 4, one 128-bit LDS read per fragment); a
+// fragment then is 8 (16) consecutive k of a row and feeds one v_mfma_f32_32x32x16_{bf16,f16} (two
+// v_mfma_f32_32x32x16_fp8_fp8): a tile is 64 (128) deep in k, and half (a quarter) of the bytes move per flop.
 template <bool A_MFAST, bool B_NFAST, int NT, int MT = 2, int HALF = 0>
 __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
     constexpr int BN = 64 * NT, BM = 64 * MT; // shadow the defaults
-    constexpr int LP = HALF ? PITCH_H : PITCH; // words per LDS row
+    constexpr bool WIDEN = HALF == 1 || HALF == 2; // f32 words narrowed on their way into LDS
+    constexpr bool PACKED = HALF >= 3;             // narrow in memory already
+    static_assert(!PACKED || (!A_MFAST && !B_NFAST), "packed operands are k-contiguous");
+    constexpr int LP = WIDEN ? PITCH_H : PITCH; // words per LDS row
     extern __shared__ float lds_dyn[]; // [2][BM][LP] for A, then [2][BN][LP] for B
     auto lds_a = [&](uint32_t buf) { return lds_dyn + buf * (BM * LP); };
     auto lds_b = [&](uint32_t buf) { return lds_dyn + 2 * BM * LP + buf * (BN * LP); };
     auto stage = [&](const TileRegs<BM> &ta, const TileRegs<BN> &tb, uint32_t buf) {
-        if constexpr (HALF) {
+        if constexpr (WIDEN) {
             store_tile_half<A_MFAST, HALF>(ta, reinterpret_cast<uint32_t *>(lds_a(buf)));
             store_tile_half<B_NFAST, HALF>(tb, reinterpret_cast<uint32_t *>(lds_b(buf)));
         } else {
@@ -283,7 +293,69 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
     stage(ra, rb, 0);
     __syncthreads();
 
-    for (uint32_t kt = 0; kt < nk; kt++) {
+    if constexpr (PACKED) {
+        // A tile's burst of matrix instructions is an eighth (a sixteenth) as long as the f32 tile's, about as long as a
+        // trip to memory: the next tile is staged into the other LDS buffer in the middle of the burst and the loads of
+        // the tile after it are asked for right there, a whole burst before they are needed (two sets of tile registers
+        // for loads two tiles ahead spill: the accumulators take every accumulation register).
+        // a 128-bit fragment is the lane's 8 (fp8: 16) consecutive k of its row: lane group g supplies the second half
+        // of each 16-deep step (fp8: bytes 0..7 of both groups form one step, bytes 8..15 the next — A and B agree)
+        float4v fa[2][MT], fb[2][NT]; // the fragments of the next 16-deep step are read while the current one multiplies
+        auto fragments = [&](const float *la, const float *lb, const int set, const int kc) {
+#pragma unroll
+            for (int i = 0; i < MT; i++)
+                fa[set][i] = *reinterpret_cast<const float4v *>(la + (wm + i * 32 + li) * PITCH + kc * 8 + lg * 4);
+#pragma unroll
+            for (int j = 0; j < NT; j++)
+                fb[set][j] = *reinterpret_cast<const float4v *>(lb + (wn + j * 32 + li) * PITCH + kc * 8 + lg * 4);
+        };
+        auto multiply = [&](const int set) {
+#pragma unroll
+            for (int i = 0; i < MT; i++)
+#pragma unroll
+                for (int j = 0; j < NT; j++) {
+                    if constexpr (HALF == 3) {
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fa[set][i]),
+                                                                            __builtin_bit_cast(bf16x8, fb[set][j]), acc[i][j], 0, 0, 0);
+                    } else if constexpr (HALF == 4) {
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, fa[set][i]),
+                                                                           __builtin_bit_cast(f16x8, fb[set][j]), acc[i][j], 0, 0, 0);
+                    } else {
+                        const long2v pa = __builtin_bit_cast(long2v, fa[set][i]), pb = __builtin_bit_cast(long2v, fb[set][j]);
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(pa[0], pb[0], acc[i][j], 0, 0, 0);
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(pa[1], pb[1], acc[i][j], 0, 0, 0);
+                    }
+                }
+        };
+        // steps [first, last) of the tile; the fragments of step `first` are in set first & 1 already
+        auto steps = [&](const float *la, const float *lb, const int first, const int last) {
+#pragma unroll
+            for (int kc = first; kc < last; kc++) {
+                if (kc + 1 < BK / 8) fragments(la, lb, (kc + 1) & 1, kc + 1);
+                multiply(kc & 1);
+            }
+        };
+        auto ask = [&](TileRegs<BM> &ta, TileRegs<BN> &tb, uint32_t kt) {
+            load_tile<false>(ta, A, a.a_sm, a.a_sk, m0, kt * BK, a.M, a.K, a.a_vec);
+            load_tile<false>(tb, B, a.b_sn, a.b_sk, n0, kt * BK, a.N, a.K, a.b_vec);
+        };
+        if (nk > 1) ask(ra, rb, 1); // (tile 0 is in LDS buffer 0 by now)
+        for (uint32_t kt = 0; kt < nk; kt++) {
+            // tile kt in buffer kt & 1, tile kt + 1 in ra / rb (asked for in the middle of the previous burst)
+            const uint32_t cur = kt & 1;
+            fragments(lds_a(cur), lds_b(cur), 0, 0);
+            __builtin_amdgcn_s_setprio(1);
+            steps(lds_a(cur), lds_b(cur), 0, BK / 16);
+            if (kt + 1 < nk) {
+                stage(ra, rb, cur ^ 1);
+                if (kt + 2 < nk) ask(ra, rb, kt + 2);
+            }
+            steps(lds_a(cur), lds_b(cur), BK / 16, BK / 8);
+            __builtin_amdgcn_s_setprio(0);
+            __syncthreads();
+        }
+    }
+    for (uint32_t kt = 0; kt < (PACKED ? 0u : nk); kt++) {
         const uint32_t cur = kt & 1;
         const bool more = kt + 1 < nk;
         const float *la = lds_a(cur), *lb = lds_b(cur);
@@ -313,7 +385,7 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
             load_tile<B_NFAST>(rb, B, a.b_sn, a.b_sk, n0, (kt + 1) * BK, a.N, a.K, a.b_vec);
         }
         __builtin_amdgcn_s_setprio(1);
-        if constexpr (HALF) {
+        if constexpr (WIDEN) {
             // 16-deep chunks: lane group g supplies k = 16*kc + 8*g .. + 7, one 128-bit LDS read per operand block
 #pragma unroll
             for (int kc = 0; kc < BK / 16; kc++) {
@@ -1435,6 +1507,73 @@ int launch_matmul_residual(cg_backend *be, const cg_tensor *x, const cg_tensor *
     return e == hipSuccess ? CG_OK : hip_fail(e, "matmul with residual launch");
 }
 
+// ---- narrow operands for the 16-bit and 8-bit matrix instructions ---------------------------------------------------
+// A [rows, k] view of f32 words that hold values of a narrow dtype (exactly) is written as its 2-byte (bf16 / f16) or
+// 1-byte (fp8) patterns, k contiguous: half or a quarter of the bytes for the product that follows, and a tile of the
+// same 32 words is 64 or 128 deep in k.  KIND 1 bf16, 2 f16, 3 fp8.  A thread narrows four consecutive k of a row.
+template <int KIND>
+__global__ __launch_bounds__(kThreads) void pack_operand_kernel(const uint32_t *src, int64_t s_r, int64_t s_k, uint32_t rows, uint32_t K,
+                                                                void *dst) {
+    const uint64_t quads = (uint64_t)rows * (K / 4);
+    const uint64_t i = (uint64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (i >= quads) return;
+    const uint32_t r = (uint32_t)(i / (K / 4)), k = (uint32_t)(i % (K / 4)) * 4;
+    const uint32_t *p = src + (int64_t)r * s_r + (int64_t)k * s_k;
+    uint32_t w[4];
+    if (s_k == 1 && ((reinterpret_cast<uintptr_t>(p) & 15) == 0)) {
+        const uint4 v = *reinterpret_cast<const uint4 *>(p);
+        w[0] = v.x, w[1] = v.y, w[2] = v.z, w[3] = v.w;
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; e++) w[e] = p[(int64_t)e * s_k];
+    }
+    if constexpr (KIND == 3) {
+        static_cast<uint32_t *>(dst)[i] = (uint32_t)f8_byte_of(w[0]) | ((uint32_t)f8_byte_of(w[1]) << 8) | ((uint32_t)f8_byte_of(w[2]) << 16) |
+                                          ((uint32_t)f8_byte_of(w[3]) << 24);
+    } else {
+        uint2 o;
+        o.x = pack_halves<KIND>(asf(w[0]), asf(w[1]));
+        o.y = pack_halves<KIND>(asf(w[2]), asf(w[3]));
+        static_cast<uint2 *>(dst)[i] = o;
+    }
+}
+
+// The narrow copy of the [rows, K] view (row stride s_r, k stride s_k, in words) at `ptr` inside `buf`; kept with the buffer
+// when `keep` (the right operand: a weight matrix is narrowed once), else the caller frees *tmp after its launch.
+static int pack_operand(cg_backend *be, Buffer *buf, const uint32_t *ptr, int64_t s_r, int64_t s_k, int64_t rows, int64_t K, int kind,
+                        bool keep, const void **packed, void **tmp, size_t *tmp_cls) {
+    const int64_t off = ptr - static_cast<const uint32_t *>(buf->ptr);
+    if (buf->packed && buf->packed_kind == kind && buf->packed_off == off && buf->packed_rows == rows && buf->packed_k == K &&
+        buf->packed_sr == s_r && buf->packed_sk == s_k) {
+        *packed = buf->packed;
+        return CG_OK;
+    }
+    void *dst = nullptr;
+    size_t cls = 0;
+    int rc = be->pool.alloc((size_t)rows * (size_t)K * (kind == 3 ? 1 : 2), &dst, &cls);
+    if (rc) return rc;
+    const uint64_t quads = (uint64_t)rows * (uint64_t)(K / 4);
+    const dim3 grid((uint32_t)((quads + kThreads - 1) / kThreads));
+    if (kind == 1) hipLaunchKernelGGL(pack_operand_kernel<1>, grid, dim3(kThreads), 0, be->stream, ptr, s_r, s_k, (uint32_t)rows, (uint32_t)K, dst);
+    else if (kind == 2) hipLaunchKernelGGL(pack_operand_kernel<2>, grid, dim3(kThreads), 0, be->stream, ptr, s_r, s_k, (uint32_t)rows, (uint32_t)K, dst);
+    else hipLaunchKernelGGL(pack_operand_kernel<3>, grid, dim3(kThreads), 0, be->stream, ptr, s_r, s_k, (uint32_t)rows, (uint32_t)K, dst);
+    if (keep && !buf->packed) {
+        buf->packed = dst;
+        buf->packed_cls = cls;
+        buf->packed_kind = kind;
+        buf->packed_off = off;
+        buf->packed_rows = rows;
+        buf->packed_k = K;
+        buf->packed_sr = s_r;
+        buf->packed_sk = s_k;
+    } else {
+        *tmp = dst;
+        *tmp_cls = cls;
+    }
+    *packed = dst;
+    return CG_OK;
+}
+
 int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_tensor *out) {
     if (int frc = flush_deferred(be)) return frc;
     MmArgs a;
@@ -1570,9 +1709,47 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds_bytes(256, 256, true)) == hipSuccess;
             CG_LDS(true, true) CG_LDS(true, false) CG_LDS(false, true) CG_LDS(false, false)
 #undef CG_LDS
+            ok &= hipFuncSetAttribute(reinterpret_cast<const void *>(&mfma_gemm_kernel<false, false, 4, 4, 3>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds_bytes(256, 256)) == hipSuccess;
+            ok &= hipFuncSetAttribute(reinterpret_cast<const void *>(&mfma_gemm_kernel<false, false, 4, 4, 4>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds_bytes(256, 256)) == hipSuccess;
+            ok &= hipFuncSetAttribute(reinterpret_cast<const void *>(&mfma_gemm_kernel<false, false, 4, 4, 5>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)gemm_lds_bytes(256, 256)) == hipSuccess;
             return ok;
         }();
         if (!lds_ok) return fail(CG_ERR_DEVICE, "matmul: cannot reserve %zu bytes of LDS", gemm_lds_bytes(128));
+        // Operands of a narrow dtype in a product big enough for the 256 x 256 tile: narrowed in memory first (the right
+        // operand once per buffer), then multiplied from 2-byte / 1-byte patterns (env CG_GEMM_PACKED=0 switches it off).
+        static const bool packed_allowed = [] {
+            const char *e = getenv("CG_GEMM_PACKED");
+            return !(e && e[0] == '0');
+        }();
+        const int kind = half ? half : x->dt == CG_F8 ? 3 : 0;
+        if (kind && packed_allowed && big && batch == 1 && K % (kind == 3 ? 16 : 8) == 0 && x->buf && y->buf) {
+            const void *pa = nullptr, *pb = nullptr;
+            void *ta = nullptr, *tb = nullptr;
+            size_t ca = 0, cb = 0;
+            int prc = pack_operand(be, x->buf, a.A, a.a_sm, a.a_sk, M, K, kind, false, &pa, &ta, &ca);
+            if (!prc) prc = pack_operand(be, y->buf, a.B, a.b_sn, a.b_sk, N, K, kind, true, &pb, &tb, &cb);
+            if (!prc) {
+                MmArgs p = a;
+                const int64_t kw = K / (kind == 3 ? 4 : 2); // words per row
+                p.A = static_cast<const uint32_t *>(pa);
+                p.B = static_cast<const uint32_t *>(pb);
+                p.K = (uint32_t)kw;
+                p.a_sm = p.b_sn = kw;
+                p.a_sk = p.b_sk = 1;
+                p.a_vec = p.b_vec = 1;
+                if (kind == 1) hipLaunchKernelGGL((mfma_gemm_kernel<false, false, 4, 4, 3>), grid, dim3(kThreads), gemm_lds_bytes(256, 256), s, p);
+                else if (kind == 2) hipLaunchKernelGGL((mfma_gemm_kernel<false, false, 4, 4, 4>), grid, dim3(kThreads), gemm_lds_bytes(256, 256), s, p);
+                else hipLaunchKernelGGL((mfma_gemm_kernel<false, false, 4, 4, 5>), grid, dim3(kThreads), gemm_lds_bytes(256, 256), s, p);
+            }
+            if (ta) be->pool.free(ta, ca); // stream-ordered: later users queue behind the product
+            if (tb) be->pool.free(tb, cb);
+            if (prc) return prc;
+            hipError_t pe = hipGetLastError();
+            return pe == hipSuccess ? CG_OK : hip_fail(pe, "matmul launch");
+        }
 #define CG_GEMM_HALF(AF, BF, H)                                                                                    \
     do {                                                                                                           \
         if (big)                                                                                                   \

@@ -114,6 +114,7 @@ static void buffer_release(Buffer *b) {
     while (b && b->rc.fetch_sub(1) == 1) {
         if (b->ptr) b->be->pool.free(b->ptr, b->cls);
         if (b->side) b->be->pool.free(b->side, b->side_cls);
+        if (b->packed) b->be->pool.free(b->packed, b->packed_cls);
         Buffer *next = b->successor;
         delete b->rs;
         delete b;

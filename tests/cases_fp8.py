@@ -178,3 +178,21 @@ def _():
         return [f8_round(av.astype(np.float64) @ bv.astype(np.float64)), f8_round(sv.astype(np.float64).sum(-1, keepdims=True))]
 
     return run, expect
+
+
+@case("fp8_matmul_narrow_operands", "ulp_f8")
+def _():
+    """A product big enough for the 256 x 256 tile and without a batch axis: the operands are narrowed to their bytes in
+    memory and multiplied on the fp8 matrix instructions (k a multiple of 16 but not of the tile depth, ragged edges)."""
+    ab, av = f8_inputs(950, (4000, 48), 0.5)
+    bb, bv = f8_inputs(951, (4100, 48), 0.5)
+
+    def run(be):
+        a, b = be.ndarray_from_vec_fp8(ab, ab.shape), be.ndarray_from_vec_fp8(bb, bb.shape)
+        return [read(be, be.matmul(a, be.transpose(b, 0, 1)))]
+
+    def expect():
+        p = av.astype(np.float64) @ bv.astype(np.float64).T
+        return [f8_round(p)]
+
+    return run, expect

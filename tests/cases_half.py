@@ -302,6 +302,34 @@ for _dt in (A.F16, A.BF16):
         return run, expect
 
 
+for _dt in (A.F16, A.BF16):
+    @case(f"half_{NAMES[_dt]}_matmul_narrow_operands", "ulp_" + NAMES[_dt])
+    def _(dt=_dt):
+        """Products without a batch axis (or with it folded into the rows, as a linear layer's) and enough 256 x 256 tiles
+        for a whole device: the operands are narrowed to 2-byte patterns in memory first and multiplied from those.
+        Ragged edges, k a multiple of 8 but not of the tile depth, the right operand k-contiguous (a weight matrix
+        [out, in] transposed), row-contiguous, and shared by a batch that folds into the rows (the same weight again)."""
+        ux, x = half_inputs(dt, 860, (4000, 40), 1.0)
+        uw, w = half_inputs(dt, 861, (4100, 40), 1.0)
+        ux, uw = round_to(dt, np.abs(x)), round_to(dt, np.abs(w))
+        x, w = as_f32(dt, ux), as_f32(dt, uw)
+        uy = np.ascontiguousarray(uw.T)
+
+        def run(be):
+            tx, tw, ty = (from_half(be, dt, u) for u in (ux, uw, uy))
+            x3 = be.reshape(be.slice(tx, 0, 0, 3840), (2, 1920, 40))
+            outs = [be.matmul(tx, be.transpose(tw, 0, 1)), be.matmul(tx, ty),
+                    be.matmul(x3, be.broadcast(be.transpose(tw, 0, 1), (2, 40, 4100)))]   # the narrowed weight is found again
+            assert all(o.dtype == dt for o in outs)
+            return [as_f32(dt, read(be, o)) for o in outs]
+
+        def expect():
+            p = x.astype(np.float64) @ w.astype(np.float64).T
+            return [p, p, p[:3840].reshape(2, 1920, 4100)]
+
+        return run, expect
+
+
 # ---- shape and index ops carry the dtype --------------------------------------------------------------------------
 for _dt in (A.F16, A.BF16):
     @case(f"half_{NAMES[_dt]}_views_concat_index")
