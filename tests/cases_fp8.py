@@ -196,3 +196,27 @@ def _():
         return [f8_round(p)]
 
     return run, expect
+
+
+@case("fp8_linear_few_rows_narrow_weights", "ulp_f8")
+def _():
+    """Decode-time linear layers of fp8 tensors (1 and 4 rows): the weight matrix is narrowed to its bytes in memory once
+    and read at one byte a weight."""
+    shapes = ((1, 512, 300), (4, 2048, 1024))
+    data = []
+    for i, (B, K, Nn) in enumerate(shapes):
+        ab, av = f8_inputs(960 + i, (B, 1, K), 0.25)
+        wb, wv = f8_inputs(970 + i, (Nn, K), 0.25)
+        data.append((ab, wb, av, wv))
+
+    def run(be):
+        outs = []
+        for (B, K, Nn), (ab, wb, _, _) in zip(shapes, data):
+            a, w = be.ndarray_from_vec_fp8(ab, ab.shape), be.ndarray_from_vec_fp8(wb, wb.shape)
+            outs.append(read(be, be.matmul(a, be.broadcast(be.transpose(w, 0, 1), (B, K, Nn)))))
+        return outs
+
+    def expect():
+        return [f8_round(av.astype(np.float64) @ wv.astype(np.float64).T) for (_, _, av, wv) in data]
+
+    return run, expect

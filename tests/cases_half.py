@@ -330,6 +330,38 @@ for _dt in (A.F16, A.BF16):
         return run, expect
 
 
+for _dt in (A.F16, A.BF16):
+    @case(f"half_{NAMES[_dt]}_linear_few_rows_narrow_weights", "ulp_" + NAMES[_dt])
+    def _(dt=_dt):
+        """Decode-time linear layers of a 16-bit dtype (1, 4 and 8 rows; the batch folds into the rows): the weight matrix
+        is narrowed to 2-byte patterns in memory once and read at 2 bytes a weight; the same weight used twice."""
+        shapes = ((1, 512, 300), (4, 2048, 1024), (8, 1024, 640))
+        data = []
+        for i, (B, K, Nn) in enumerate(shapes):
+            ux, x = half_inputs(dt, 870 + i, (B, 1, K), 1.0)
+            uw, w = half_inputs(dt, 880 + i, (Nn, K), 1.0)
+            ux, uw = round_to(dt, np.abs(x)), round_to(dt, np.abs(w))
+            data.append((ux, uw, as_f32(dt, ux), as_f32(dt, uw)))
+
+        def run(be):
+            outs = []
+            for (B, K, Nn), (ux, uw, _, _) in zip(shapes, data):
+                tx, tw = from_half(be, dt, ux), from_half(be, dt, uw)
+                wv = be.broadcast(be.transpose(tw, 0, 1), (B, K, Nn))
+                outs += [be.matmul(tx, wv), be.matmul(be.add(tx, tx), wv)]
+            assert all(o.dtype == dt for o in outs)
+            return [as_f32(dt, read(be, o)) for o in outs]
+
+        def expect():
+            outs = []
+            for (_, _, x, w) in data:
+                p = x.astype(np.float64) @ w.astype(np.float64).T
+                outs += [p, 2.0 * p]
+            return outs
+
+        return run, expect
+
+
 # ---- shape and index ops carry the dtype --------------------------------------------------------------------------
 for _dt in (A.F16, A.BF16):
     @case(f"half_{NAMES[_dt]}_views_concat_index")
