@@ -1548,6 +1548,15 @@ static bool packed_narrow_ok() {
     return ok;
 }
 
+// (env CG_PACKED_MFMA=0 keeps few-row products of the 16-bit dtypes on the wave-per-column kernel, for measurements)
+static bool packed_mfma_ok() {
+    static const bool ok = [] {
+        const char *e = getenv("CG_PACKED_MFMA");
+        return !(e && e[0] == '0');
+    }();
+    return ok;
+}
+
 // The narrow copy of the [rows, K] view (row stride s_r, k stride s_k, in words) at `ptr` inside `buf`; kept with the buffer
 // when `keep` (the right operand: a weight matrix is narrowed once), else the caller frees *tmp after its launch.
 static int pack_operand(cg_backend *be, Buffer *buf, const uint32_t *ptr, int64_t s_r, int64_t s_k, int64_t rows, int64_t K, int kind,
@@ -1609,6 +1618,79 @@ template <int KIND> __device__ __forceinline__ void widen_weights(const uint4v &
             for (int b = 0; b < 4; b++) w[4 * i + b] = asf(f8_word_of((uint8_t)(r[i] >> (8 * b))));
     }
 }
+// The same for at most four rows of the 16-bit dtypes on the matrix instruction v_mfma_f32_4x4x4_{bf16_1k,f16}: the layout
+// of skinny_kt_mfma_xreg_body (lane (b, j) = (lane / 4, lane % 4) feeds weight row n0 + j and activation row j for the k of
+// block b) with 8 k per lane and trip instead of 4: one 16-byte load of narrow weights drives two instructions.  The
+// activations, which are f32 words in memory, are narrowed (exact) into registers ONCE per workgroup — all of K, 16
+// registers per 2048 — and the workgroup walks `iters` consecutive groups of four columns with them, the next group's
+// weights on their way while the current group is reduced: the activation traffic out of L2, twice the weights' bytes per
+// column group, is paid once.  K = KCH x 1024.  KIND 1 bf16, 2 f16.
+typedef short short4v __attribute__((ext_vector_type(4)));
+typedef _Float16 half4v __attribute__((ext_vector_type(4)));
+template <int KIND, int KCH>
+__global__ __launch_bounds__(kThreads) void skinny_kt_packed_mfma_kernel(const MmArgs a, const void *weights, uint32_t iters) {
+    constexpr int TRIPS = 2 * KCH; // a wave takes 128 k per trip, four waves 512: two trips per 1024
+    const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x % 64;
+    const uint32_t j = lane % 4, b = lane / 4;
+    const uint32_t kb = wave * 128 + b * 8; // this lane's k: kb + 512 t .. + 7
+    const uint32_t groups = (a.N + 3) / 4;
+    const uint32_t first_grp = blockIdx.x * iters;
+    if (first_grp >= groups) return; // the same for every thread of the workgroup
+    uint4v wq[TRIPS];
+    auto ask = [&](uint32_t grp) {
+        const uint16_t *row = static_cast<const uint16_t *>(weights) + (size_t)min(grp * 4 + j, a.N - 1) * a.K + kb;
+#pragma unroll
+        for (int t = 0; t < TRIPS; t++) wq[t] = __builtin_nontemporal_load(reinterpret_cast<const uint4v *>(row + 512 * t));
+    };
+    ask(first_grp);
+    // the activations of row j, narrowed: xq[t] = its 8 values at kb + 512 t as four words of two
+    uint4v xq[TRIPS];
+    {
+        const uint32_t *xrow = a.A + (int64_t)min(j, a.M - 1) * a.a_sm + kb;
+#pragma unroll
+        for (int t = 0; t < TRIPS; t++) {
+            const float4v lo = *reinterpret_cast<const float4v *>(xrow + 512 * t), hi = *reinterpret_cast<const float4v *>(xrow + 512 * t + 4);
+            xq[t][0] = pack_halves<KIND>(lo[0], lo[1]);
+            xq[t][1] = pack_halves<KIND>(lo[2], lo[3]);
+            xq[t][2] = pack_halves<KIND>(hi[0], hi[1]);
+            xq[t][3] = pack_halves<KIND>(hi[2], hi[3]);
+        }
+    }
+    __shared__ float part[2][4][16];
+    for (uint32_t it = 0; it < iters; it++) {
+        const uint32_t grp = first_grp + it;
+        if (grp >= groups) break;
+        float4v acc = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int t = 0; t < TRIPS; t++) {
+            typedef uint32_t uint2v __attribute__((ext_vector_type(2)));
+            const uint2v x0 = {xq[t][0], xq[t][1]}, x1 = {xq[t][2], xq[t][3]}, w0 = {wq[t][0], wq[t][1]}, w1 = {wq[t][2], wq[t][3]};
+            if constexpr (KIND == 1) {
+                acc = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(short4v, x0), __builtin_bit_cast(short4v, w0), acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_4x4x4bf16_1k(__builtin_bit_cast(short4v, x1), __builtin_bit_cast(short4v, w1), acc, 0, 0, 0);
+            } else {
+                acc = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(half4v, x0), __builtin_bit_cast(half4v, w0), acc, 0, 0, 0);
+                acc = __builtin_amdgcn_mfma_f32_4x4x4f16(__builtin_bit_cast(half4v, x1), __builtin_bit_cast(half4v, w1), acc, 0, 0, 0);
+            }
+        }
+        if (it + 1 < iters && grp + 1 < groups) ask(grp + 1); // on its way through the reduction of this group
+        float (*pt)[16] = part[it & 1];
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            float v = acc[i];
+#pragma unroll
+            for (int s = 32; s >= 4; s >>= 1) v += __shfl_xor(v, s);
+            if (lane < 4) pt[wave][i * 4 + j] = v;
+        }
+        __syncthreads(); // (the buffer written two groups ago was read before the barrier of the group in between)
+        if (threadIdx.x < 16) {
+            const uint32_t m = threadIdx.x / 4, col = grp * 4 + threadIdx.x % 4;
+            const float v = (pt[0][threadIdx.x] + pt[1][threadIdx.x]) + (pt[2][threadIdx.x] + pt[3][threadIdx.x]);
+            if (col < a.N && m < a.M) a.C[(uint64_t)m * a.N + col] = asu(v);
+        }
+    }
+}
+
 template <int MM, int KIND>
 __global__ __launch_bounds__(kThreads) void skinny_kt_packed_kernel(const MmArgs a, const void *weights) {
     constexpr int PER = KIND == 3 ? 16 : 8; // weights per lane and trip
@@ -1684,6 +1766,23 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
         int prc = pack_operand(be, y->buf, a.B, a.b_sn, a.b_sk, N, K, kind, true, &pb, &tb, &cb);
         if (prc) return prc;
         const dim3 pgrid((uint32_t)((N + 3) / 4));
+        const int kch = (int)(K / 1024);
+        if (half && M <= 4 && K % 1024 == 0 && (kch == 1 || kch == 2 || kch == 4 || kch == 8) && packed_mfma_ok()) {
+            // all of the activations narrowed into registers, several column groups per workgroup (see the kernel)
+            const uint32_t groups = (uint32_t)((N + 3) / 4), iters = xreg_cols_iters(groups);
+            const dim3 mgrid((groups + iters - 1) / iters);
+#define CG_PACKED_MFMA(KCH)                                                                                              \
+    if (half == 1) hipLaunchKernelGGL((skinny_kt_packed_mfma_kernel<1, KCH>), mgrid, dim3(kThreads), 0, s, a, pb, iters);      \
+    else hipLaunchKernelGGL((skinny_kt_packed_mfma_kernel<2, KCH>), mgrid, dim3(kThreads), 0, s, a, pb, iters);
+            if (kch == 1) { CG_PACKED_MFMA(1) }
+            else if (kch == 2) { CG_PACKED_MFMA(2) }
+            else if (kch == 4) { CG_PACKED_MFMA(4) }
+            else { CG_PACKED_MFMA(8) }
+#undef CG_PACKED_MFMA
+            if (tb) be->pool.free(tb, cb);
+            hipError_t me = hipGetLastError();
+            return me == hipSuccess ? CG_OK : hip_fail(me, "matmul launch");
+        }
 #define CG_PACKED(MM)                                                                                                     \
     if (kind == 1) hipLaunchKernelGGL((skinny_kt_packed_kernel<MM, 1>), pgrid, dim3(kThreads), 0, s, a, pb);                  \
     else if (kind == 2) hipLaunchKernelGGL((skinny_kt_packed_kernel<MM, 2>), pgrid, dim3(kThreads), 0, s, a, pb);             \
