@@ -334,8 +334,10 @@ for _dt in (A.F16, A.BF16):
     @case(f"half_{NAMES[_dt]}_linear_few_rows_narrow_weights", "ulp_" + NAMES[_dt])
     def _(dt=_dt):
         """Decode-time linear layers of a 16-bit dtype (1, 4 and 8 rows; the batch folds into the rows): the weight matrix
-        is narrowed to 2-byte patterns in memory once and read at 2 bytes a weight; the same weight used twice."""
-        shapes = ((1, 512, 300), (4, 2048, 1024), (8, 1024, 640))
+        is narrowed to 2-byte patterns in memory once and read at 2 bytes a weight (up to four rows and K a multiple of 1024:
+        the 4 x 4 x 4 matrix-instruction kernel at its four depths, ragged column counts; else a wave per column); the same
+        weight used twice."""
+        shapes = ((1, 512, 300), (4, 2048, 1024), (8, 1024, 640), (2, 1024, 518), (3, 8192, 262), (4, 4096, 2050))
         data = []
         for i, (B, K, Nn) in enumerate(shapes):
             ux, x = half_inputs(dt, 870 + i, (B, 1, K), 1.0)
