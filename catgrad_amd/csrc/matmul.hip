@@ -43,6 +43,7 @@
 #include "device_utils.hpp"
 
 #include <algorithm>
+#include <type_traits>
 
 namespace cg {
 
@@ -336,9 +337,32 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
                 multiply(kc & 1);
             }
         };
+        // Whole tiles (every tile but a ragged last one) are loaded without a test: a lane's slots sit 32 rows apart at the
+        // same k, so its byte offsets into the operands are fixed (rows beyond the edge are clamped: what they contribute
+        // lands in accumulator rows that are never stored) and a tile is 16 + 16 loads at a base that moves by one tile.
+        uint32_t offa[TileRegs<BM>::slots], offb[TileRegs<BN>::slots];
+#pragma unroll
+        for (int h = 0; h < TileRegs<BM>::slots; h++) {
+            const uint32_t slot = threadIdx.x + h * kThreads, row = min(m0 + slot / (BK / 4), a.M - 1);
+            offa[h] = (uint32_t)(((uint64_t)row * (uint64_t)a.a_sm + (slot % (BK / 4)) * 4) * 4);
+        }
+#pragma unroll
+        for (int h = 0; h < TileRegs<BN>::slots; h++) {
+            const uint32_t slot = threadIdx.x + h * kThreads, row = min(n0 + slot / (BK / 4), a.N - 1);
+            offb[h] = (uint32_t)(((uint64_t)row * (uint64_t)a.b_sn + (slot % (BK / 4)) * 4) * 4);
+        }
+        const bool lean = (uint64_t)a.M * (uint64_t)a.a_sm < (1ull << 30) && (uint64_t)a.N * (uint64_t)a.b_sn < (1ull << 30); // offsets fit 32 bits
         auto ask = [&](TileRegs<BM> &ta, TileRegs<BN> &tb, uint32_t kt) {
-            load_tile<false>(ta, A, a.a_sm, a.a_sk, m0, kt * BK, a.M, a.K, a.a_vec);
-            load_tile<false>(tb, B, a.b_sn, a.b_sk, n0, kt * BK, a.N, a.K, a.b_vec);
+            if (lean && (kt + 1) * BK <= a.K) {
+                const char *pa = reinterpret_cast<const char *>(A + (uint64_t)kt * BK), *pb = reinterpret_cast<const char *>(B + (uint64_t)kt * BK);
+#pragma unroll
+                for (int h = 0; h < TileRegs<BM>::slots; h++) ta.v[h] = *reinterpret_cast<const float4v *>(pa + offa[h]);
+#pragma unroll
+                for (int h = 0; h < TileRegs<BN>::slots; h++) tb.v[h] = *reinterpret_cast<const float4v *>(pb + offb[h]);
+            } else {
+                load_tile<false>(ta, A, a.a_sm, a.a_sk, m0, kt * BK, a.M, a.K, a.a_vec);
+                load_tile<false>(tb, B, a.b_sn, a.b_sk, n0, kt * BK, a.N, a.K, a.b_vec);
+            }
         };
         if (nk > 1) ask(ra, rb, 1); // (tile 0 is in LDS buffer 0 by now)
         for (uint32_t kt = 0; kt < nk; kt++) {
@@ -356,9 +380,47 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
             __syncthreads();
         }
     }
-    for (uint32_t kt = 0; kt < (PACKED ? 0u : nk); kt++) {
+    // Operands whose 16-byte loads are legal everywhere (aligned, unit stride along k or along the rows): a lane's slots keep
+    // their place in every tile, so its byte offsets into the operands are fixed (rows beyond the edge clamped: their values
+    // land in accumulator rows that are never stored) and a whole tile is loaded without a test per slot, at a base that
+    // moves by one tile.  (The generic loader's tests and fallbacks cost the 256 x 256 tile 4 % of its time.)
+    uint32_t offa_kk[TileRegs<BM>::slots], offb_kk[TileRegs<BN>::slots];
+    bool lean_kk = false;
+    // (The 256 x 256 tile with both operands row-contiguous, or with one such operand narrowed to bfloat16, has no registers
+    // left for the offsets.)
+    constexpr bool LEAN = !PACKED && (MT != 4 || (!(A_MFAST && B_NFAST) && !((A_MFAST || B_NFAST) && HALF == 1)));
+    if constexpr (LEAN) {
+        const bool a_ok = A_MFAST ? (a.a_vec && a.a_sm == 1 && a.M % 4 == 0 && a.M >= 4) : (a.a_vec && a.a_sk == 1 && a.a_sm > 0);
+        const bool b_ok = B_NFAST ? (a.b_vec && a.b_sn == 1 && a.N % 4 == 0 && a.N >= 4) : (a.b_vec && a.b_sk == 1 && a.b_sn > 0);
+        const uint64_t a_span = A_MFAST ? (uint64_t)a.K * (uint64_t)a.a_sk : (uint64_t)a.M * (uint64_t)a.a_sm;
+        const uint64_t b_span = B_NFAST ? (uint64_t)a.K * (uint64_t)a.b_sk : (uint64_t)a.N * (uint64_t)a.b_sn;
+        lean_kk = a_ok && b_ok && a.a_sk > 0 && a.b_sk > 0 && a_span < (1ull << 30) && b_span < (1ull << 30); // offsets fit 32 bits
+#pragma unroll
+        for (int h = 0; h < TileRegs<BM>::slots; h++) {
+            const uint32_t slot = threadIdx.x + h * kThreads;
+            if constexpr (A_MFAST) {
+                uint32_t row, k;
+                rows_fast_slot<BM>(slot, row, k);
+                offa_kk[h] = (uint32_t)(((uint64_t)k * (uint64_t)a.a_sk + min(m0 + row, a.M - 4)) * 4);
+            } else {
+                offa_kk[h] = (uint32_t)(((uint64_t)min(m0 + slot / (BK / 4), a.M - 1) * (uint64_t)a.a_sm + (slot % (BK / 4)) * 4) * 4);
+            }
+        }
+#pragma unroll
+        for (int h = 0; h < TileRegs<BN>::slots; h++) {
+            const uint32_t slot = threadIdx.x + h * kThreads;
+            if constexpr (B_NFAST) {
+                uint32_t row, k;
+                rows_fast_slot<BN>(slot, row, k);
+                offb_kk[h] = (uint32_t)(((uint64_t)k * (uint64_t)a.b_sk + min(n0 + row, a.N - 4)) * 4);
+            } else {
+                offb_kk[h] = (uint32_t)(((uint64_t)min(n0 + slot / (BK / 4), a.N - 1) * (uint64_t)a.b_sn + (slot % (BK / 4)) * 4) * 4);
+            }
+        }
+    }
+    auto iterate = [&](const uint32_t kt, auto whole_next) {
         const uint32_t cur = kt & 1;
-        const bool more = kt + 1 < nk;
+        const bool more = decltype(whole_next)::value || kt + 1 < nk;
         const float *la = lds_a(cur), *lb = lds_b(cur);
         // One 8-deep chunk of the tile: lane group g supplies k = 8*kc + 4*g + t to the t-th MFMA,
         // for A and B alike, so one 128-bit LDS read feeds four MFMAs.
@@ -381,7 +443,15 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
         // While a wave is in its burst of matrix instructions it wins issue arbitration against the other
         // wave of its SIMD (which is loading or storing a tile): the two stop advancing in lock-step and
         // their stalls at the barrier no longer coincide.
-        if (more) {
+        if constexpr (decltype(whole_next)::value) {
+            // the next tile is a whole tile of k-contiguous, aligned operands: no test per slot
+            const char *pa = reinterpret_cast<const char *>(A + (uint64_t)(kt + 1) * BK * (A_MFAST ? (uint64_t)a.a_sk : 1ull));
+            const char *pb = reinterpret_cast<const char *>(B + (uint64_t)(kt + 1) * BK * (B_NFAST ? (uint64_t)a.b_sk : 1ull));
+#pragma unroll
+            for (int h = 0; h < TileRegs<BM>::slots; h++) ra.v[h] = *reinterpret_cast<const float4v *>(pa + offa_kk[h]);
+#pragma unroll
+            for (int h = 0; h < TileRegs<BN>::slots; h++) rb.v[h] = *reinterpret_cast<const float4v *>(pb + offb_kk[h]);
+        } else if (more) {
             load_tile<A_MFAST>(ra, A, a.a_sm, a.a_sk, m0, (kt + 1) * BK, a.M, a.K, a.a_vec);
             load_tile<B_NFAST>(rb, B, a.b_sn, a.b_sk, n0, (kt + 1) * BK, a.N, a.K, a.b_vec);
         }
@@ -425,6 +495,14 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
         __builtin_amdgcn_s_setprio(0);
         if (more && (HALF || MT != 4)) stage(ra, rb, cur ^ 1);
         __syncthreads();
+        };
+    {
+        uint32_t kt = 0;
+        if constexpr (LEAN) {
+            if (lean_kk)
+                for (; (kt + 2) * BK <= a.K; kt++) iterate(kt, std::true_type{});
+        }
+        for (; kt < (PACKED ? 0u : nk); kt++) iterate(kt, std::false_type{});
     }
 
     // D layout of v_mfma_f32_32x32x2_f32: lane (li, lg), register v -> row 8*(v/4) + 4*lg + v%4, col li
