@@ -56,9 +56,15 @@ def micro_bench(iters=20):
     out = {}
 
     def run(name, cls, fn, unit, launches_per_call=1, mfma_peak=MFMA_F32_PEAK):
-        for _ in range(3):
-            fn()
-        be.sync()
+        # warm up to steady clocks: the uploads before a line leave the card idle long enough for it to clock down, and
+        # the first few milliseconds of launches after that run up to 15 % slow
+        t_warm = time.perf_counter()
+        while True:
+            for _ in range(3):
+                fn()
+            be.sync()
+            if time.perf_counter() - t_warm >= 0.05:
+                break
         be.profile_enable(cls, 1)
         be.profile_read(cls, reset=True)
         for _ in range(iters):

@@ -103,11 +103,11 @@ template <int TR> struct TileRegs {
 
 __device__ __forceinline__ float ld_guard(const uint32_t *p, bool ok) { return ok ? asf(*p) : 0.0f; }
 
-// Slot -> (first of four rows, k) of a tile whose rows are the unit-stride axis in memory.  The tile is staged K-fastest
-// in LDS, so a lane's four values go to four different LDS rows, one 4-byte store each.  With a whole wave on one k (64
-// row-quads) those stores hit 2 of the 32 banks; with 16 row-quads x 4 consecutive k per wave, and each lane writing its
-// four rows in an order rotated by its row-quad (rows_fast_order), a wave's store covers all 32 banks twice, which is the
-// best 64 lanes can do.  Global loads stay 256 contiguous bytes per k.
+// Slot -> (first of four rows, k) of a tile whose rows are the unit-stride axis in memory: 16 row-quads x 4 consecutive k
+// per wave, global loads of 256 contiguous bytes per k.  An f32 tile keeps that order in LDS (store_tile).  A tile that is
+// narrowed to 16 bits is staged K-fastest (pairs of k share a word), so a lane's four values go to four different LDS
+// rows, one store each; with each lane writing its four rows in an order rotated by its row-quad (rows_fast_order), a
+// wave's store covers all 32 banks twice, which is the best 64 lanes can do (a whole wave on one k would hit 2 banks).
 template <int TR> __device__ __forceinline__ void rows_fast_slot(uint32_t slot, uint32_t &row, uint32_t &k) {
     const uint32_t group = slot / 64, in = slot % 64;
     row = (group % (TR / 64)) * 64 + (in % 16) * 4;
@@ -153,7 +153,8 @@ __device__ __forceinline__ void load_tile(TileRegs<TR> &t, const uint32_t *base,
     }
 }
 
-// Stores the registers K-fastest into an LDS tile [TR][PITCH].
+// Stores the registers into an LDS tile: K-fastest, [TR][PITCH], for k-contiguous operands; rows-fastest, [BK][TR], for
+// row-contiguous ones.
 template <bool ROWS_FAST, int TR> __device__ __forceinline__ void store_tile(const TileRegs<TR> &t, float *lds) {
 #pragma unroll
     for (int h = 0; h < TileRegs<TR>::slots; h++) {
@@ -162,13 +163,11 @@ template <bool ROWS_FAST, int TR> __device__ __forceinline__ void store_tile(con
             uint32_t row = slot / (BK / 4), k = (slot % (BK / 4)) * 4;
             *reinterpret_cast<float4v *>(lds + row * PITCH + k) = t.v[h];
         } else {
+            // rows stay the fastest axis in LDS too, [BK][TR]: one 16-byte store, no transposition (eight lanes cover 32
+            // consecutive words); the fragments are then read a word at a time, 32 consecutive words per half wave
             uint32_t row, k;
             rows_fast_slot<TR>(slot, row, k);
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                const uint32_t j = rows_fast_order(slot, i);
-                lds[(row + j) * PITCH + k] = pick4(t.v[h], j);
-            }
+            *reinterpret_cast<float4v *>(lds + k * TR + row) = t.v[h];
         }
     }
 }
@@ -427,11 +426,23 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
         auto chunk = [&](const int kc) {
             float4v fa[MT], fb[NT];
 #pragma unroll
-            for (int i = 0; i < MT; i++)
-                fa[i] = *reinterpret_cast<const float4v *>(la + (wm + i * 32 + li) * PITCH + kc * 8 + lg * 4);
+            for (int i = 0; i < MT; i++) {
+                if constexpr (A_MFAST) {
 #pragma unroll
-            for (int j = 0; j < NT; j++)
-                fb[j] = *reinterpret_cast<const float4v *>(lb + (wn + j * 32 + li) * PITCH + kc * 8 + lg * 4);
+                    for (int t = 0; t < 4; t++) fa[i][t] = la[(kc * 8 + lg * 4 + t) * BM + wm + i * 32 + li];
+                } else {
+                    fa[i] = *reinterpret_cast<const float4v *>(la + (wm + i * 32 + li) * PITCH + kc * 8 + lg * 4);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < NT; j++) {
+                if constexpr (B_NFAST) {
+#pragma unroll
+                    for (int t = 0; t < 4; t++) fb[j][t] = lb[(kc * 8 + lg * 4 + t) * BN + wn + j * 32 + li];
+                } else {
+                    fb[j] = *reinterpret_cast<const float4v *>(lb + (wn + j * 32 + li) * PITCH + kc * 8 + lg * 4);
+                }
+            }
 #pragma unroll
             for (int t = 0; t < 4; t++)
 #pragma unroll
