@@ -302,40 +302,6 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
         // a 128-bit fragment is the lane's 8 (fp8: 16) consecutive k of its row: lane group g supplies the second half
         // of each 16-deep step (fp8: bytes 0..7 of both groups form one step, bytes 8..15 the next — A and B agree)
         float4v fa[2][MT], fb[2][NT]; // the fragments of the next 16-deep step are read while the current one multiplies
-        auto fragments = [&](const float *la, const float *lb, const int set, const int kc) {
-#pragma unroll
-            for (int i = 0; i < MT; i++)
-                fa[set][i] = *reinterpret_cast<const float4v *>(la + (wm + i * 32 + li) * PITCH + kc * 8 + lg * 4);
-#pragma unroll
-            for (int j = 0; j < NT; j++)
-                fb[set][j] = *reinterpret_cast<const float4v *>(lb + (wn + j * 32 + li) * PITCH + kc * 8 + lg * 4);
-        };
-        auto multiply = [&](const int set) {
-#pragma unroll
-            for (int i = 0; i < MT; i++)
-#pragma unroll
-                for (int j = 0; j < NT; j++) {
-                    if constexpr (HALF == 3) {
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fa[set][i]),
-                                                                            __builtin_bit_cast(bf16x8, fb[set][j]), acc[i][j], 0, 0, 0);
-                    } else if constexpr (HALF == 4) {
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, fa[set][i]),
-                                                                           __builtin_bit_cast(f16x8, fb[set][j]), acc[i][j], 0, 0, 0);
-                    } else {
-                        const long2v pa = __builtin_bit_cast(long2v, fa[set][i]), pb = __builtin_bit_cast(long2v, fb[set][j]);
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(pa[0], pb[0], acc[i][j], 0, 0, 0);
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(pa[1], pb[1], acc[i][j], 0, 0, 0);
-                    }
-                }
-        };
-        // steps [first, last) of the tile; the fragments of step `first` are in set first & 1 already
-        auto steps = [&](const float *la, const float *lb, const int first, const int last) {
-#pragma unroll
-            for (int kc = first; kc < last; kc++) {
-                if (kc + 1 < BK / 8) fragments(la, lb, (kc + 1) & 1, kc + 1);
-                multiply(kc & 1);
-            }
-        };
         // Whole tiles (every tile but a ragged last one) are loaded without a test: a lane's slots sit 32 rows apart at the
         // same k, so its byte offsets into the operands are fixed (rows beyond the edge are clamped: what they contribute
         // lands in accumulator rows that are never stored) and a tile is 16 + 16 loads at a base that moves by one tile.
@@ -363,21 +329,123 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
                 load_tile<false>(tb, B, a.b_sn, a.b_sk, n0, kt * BK, a.N, a.K, a.b_vec);
             }
         };
-        if (nk > 1) ask(ra, rb, 1); // (tile 0 is in LDS buffer 0 by now)
-        for (uint32_t kt = 0; kt < nk; kt++) {
-            // tile kt in buffer kt & 1, tile kt + 1 in ra / rb (asked for in the middle of the previous burst)
-            const uint32_t cur = kt & 1;
-            fragments(lds_a(cur), lds_b(cur), 0, 0);
-            __builtin_amdgcn_s_setprio(1);
-            steps(lds_a(cur), lds_b(cur), 0, BK / 16);
-            if (kt + 1 < nk) {
-                stage(ra, rb, cur ^ 1);
-                if (kt + 2 < nk) ask(ra, rb, kt + 2);
+        // One tile: S steps of 16 (fp8: 32) k.  Set 0 holds the fragments of step 0 when a tile begins; every step reads the
+        // fragments of the next one while it multiplies.  The barrier stands before the LAST step: by then every wave has
+        // read all of this tile's fragments and has staged its share of the next tile into the other buffer, so the first
+        // fragments of the next tile are read behind the barrier, under the last step's matrix instructions, and the matrix
+        // pipe never drains at a tile border.
+        // In the steady state (whole tiles, offsets that fit) the 16 slots of the next tile (one 16-byte LDS store each) and
+        // the 16 loads of the tile after it are dealt out between groups of four matrix instructions of the first S - 1 steps:
+        // a burst of 16 loads (a KB each) blocks the wave's instruction issue for as long as the texture path takes them.
+        constexpr int S = BK / 8;
+        auto frag_a = [&](const float *la, const int set, const int kc, const int i) {
+            fa[set][i] = *reinterpret_cast<const float4v *>(la + (wm + i * 32 + li) * PITCH + kc * 8 + lg * 4);
+        };
+        auto frag_b = [&](const float *lb, const int set, const int kc, const int j) {
+            fb[set][j] = *reinterpret_cast<const float4v *>(lb + (wn + j * 32 + li) * PITCH + kc * 8 + lg * 4);
+        };
+        auto mma_row = [&](const int set, const int i) {
+#pragma unroll
+            for (int j = 0; j < NT; j++) {
+                if constexpr (HALF == 3) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fa[set][i]),
+                                                                        __builtin_bit_cast(bf16x8, fb[set][j]), acc[i][j], 0, 0, 0);
+                } else if constexpr (HALF == 4) {
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, fa[set][i]),
+                                                                       __builtin_bit_cast(f16x8, fb[set][j]), acc[i][j], 0, 0, 0);
+                } else {
+                    const long2v pa = __builtin_bit_cast(long2v, fa[set][i]), pb = __builtin_bit_cast(long2v, fb[set][j]);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(pa[0], pb[0], acc[i][j], 0, 0, 0);
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_fp8_fp8(pa[1], pb[1], acc[i][j], 0, 0, 0);
+                }
             }
-            steps(lds_a(cur), lds_b(cur), BK / 16, BK / 8);
-            __builtin_amdgcn_s_setprio(0);
-            __syncthreads();
+        };
+        static_assert(MT == NT && TileRegs<BM>::slots == 8 && TileRegs<BN>::slots == 8, "the slot schedule below is for the 256 x 256 tile");
+        auto iteration = [&](const uint32_t kt, auto steady) {
+            constexpr bool STEADY = decltype(steady)::value;
+            const uint32_t cur = kt & 1;
+            const bool next = STEADY || kt + 1 < nk;
+            const float *la = lds_a(cur), *lb = lds_b(cur);
+            float *na = lds_a(cur ^ 1), *nb = lds_b(cur ^ 1);
+            const char *pa = reinterpret_cast<const char *>(A + (uint64_t)(kt + 2) * BK), *pb = reinterpret_cast<const char *>(B + (uint64_t)(kt + 2) * BK);
+            auto slot = [&](const int q) { // stage slot q of tile kt + 1, then ask for slot q of tile kt + 2
+                const uint32_t sl = threadIdx.x + (q % 8) * kThreads, row = sl / (BK / 4), k = (sl % (BK / 4)) * 4;
+                if (q < 8) {
+                    *reinterpret_cast<float4v *>(na + row * PITCH + k) = ra.v[q % 8];
+                    ra.v[q % 8] = *reinterpret_cast<const float4v *>(pa + offa[q % 8]);
+                } else {
+                    *reinterpret_cast<float4v *>(nb + row * PITCH + k) = rb.v[q % 8];
+                    rb.v[q % 8] = *reinterpret_cast<const float4v *>(pb + offb[q % 8]);
+                }
+            };
+#pragma unroll
+            for (int kc = 0; kc < S - 1; kc++) {
+#pragma unroll
+                for (int i = 0; i < MT; i++) {
+                    frag_a(la, (kc + 1) & 1, kc + 1, i);
+                    frag_b(lb, (kc + 1) & 1, kc + 1, i);
+                    mma_row(kc & 1, i);
+                    if constexpr (STEADY) {
+                        // 16 slots over 12 groups: every third group takes two
+                        const int g = kc * MT + i, first = g + (g + 2) / 3;
+                        slot(first);
+                        if (g % 3 == 0) slot(first + 1);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+                if constexpr (!STEADY) {
+                    if (kc == S / 2 - 1 && next) {
+                        stage(ra, rb, cur ^ 1);
+                        if (kt + 2 < nk) ask(ra, rb, kt + 2);
+                    }
+                }
+            }
+            asm volatile("" ::: "memory");
+            __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0): this wave's LDS stores have landed (loads in flight stay in flight)
+            __builtin_amdgcn_s_barrier();
+            asm volatile("" ::: "memory");
+#pragma unroll
+            for (int i = 0; i < MT; i++) {
+                if (next) {
+                    frag_a(na, 0, 0, i);
+                    frag_b(nb, 0, 0, i);
+                }
+                mma_row((S - 1) & 1, i);
+                if constexpr (STEADY) __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        static_assert(S % 2 == 0, "the last step multiplies from set 1 while set 0 is refilled");
+        uint32_t kt = 0;
+        if (lean && 3 * BK <= a.K) {
+            // tile 1 is asked for slot by slot in the order the loop consumes the slots: only then does the compiler's count
+            // of loads in flight at the loop's head match the one at its end, and each LDS store waits for its own load
+            // (all but the 15 younger ones) instead of for every load
+            const char *pa = reinterpret_cast<const char *>(A + (uint64_t)BK), *pb = reinterpret_cast<const char *>(B + (uint64_t)BK);
+#pragma unroll
+            for (int h = 0; h < 8; h++) {
+                ra.v[h] = *reinterpret_cast<const float4v *>(pa + offa[h]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int h = 0; h < 8; h++) {
+                rb.v[h] = *reinterpret_cast<const float4v *>(pb + offb[h]);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int i = 0; i < MT; i++) {
+                frag_a(lds_a(0), 0, 0, i);
+                frag_b(lds_b(0), 0, 0, i);
+            }
+            for (; (kt + 3) * BK <= a.K; kt++) iteration(kt, std::true_type{});
+        } else {
+            if (nk > 1) ask(ra, rb, 1); // (tile 0 is in LDS buffer 0 by now)
+#pragma unroll
+            for (int i = 0; i < MT; i++) {
+                frag_a(lds_a(0), 0, 0, i);
+                frag_b(lds_b(0), 0, 0, i);
+            }
         }
+        for (; kt < nk; kt++) iteration(kt, std::false_type{});
     }
     // Operands whose 16-byte loads are legal everywhere (aligned, unit stride along k or along the rows): a lane's slots keep
     // their place in every tile, so its byte offsets into the operands are fixed (rows beyond the edge clamped: their values
