@@ -183,6 +183,8 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef long long2v __attribute__((ext_vector_type(2)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
+typedef int int4v __attribute__((ext_vector_type(4)));
+typedef int int8v __attribute__((ext_vector_type(8)));
 
 // HALF: 1 bfloat16, 2 binary16
 template <int HALF> __device__ __forceinline__ uint32_t pack_halves(float lo, float hi) {
@@ -302,6 +304,7 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
         // a 128-bit fragment is the lane's 8 (fp8: 16) consecutive k of its row: lane group g supplies the second half
         // of each 16-deep step (fp8: bytes 0..7 of both groups form one step, bytes 8..15 the next — A and B agree)
         float4v fa[2][MT], fb[2][NT]; // the fragments of the next 16-deep step are read while the current one multiplies
+        int8v fa8[2], fb8[NT];        // fp8: the 32 bytes a lane feeds to one 64-deep instruction; a ring of two A rows, all of B
         // Whole tiles (every tile but a ragged last one) are loaded without a test: a lane's slots sit 32 rows apart at the
         // same k, so its byte offsets into the operands are fixed (rows beyond the edge are clamped: what they contribute
         // lands in accumulator rows that are never stored) and a tile is 16 + 16 loads at a base that moves by one tile.
@@ -341,6 +344,12 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
         auto frag_a = [&](const float *la, const int set, const int kc, const int i) {
             fa[set][i] = *reinterpret_cast<const float4v *>(la + (wm + i * 32 + li) * PITCH + kc * 8 + lg * 4);
         };
+        auto frag8 = [&](const float *l, const int d, const uint32_t row0) { // the two fragments of double step d of a row
+            const float *p = l + (row0 + li) * PITCH + d * 16 + lg * 4;
+            const int4v lo = __builtin_bit_cast(int4v, *reinterpret_cast<const float4v *>(p));
+            const int4v hi = __builtin_bit_cast(int4v, *reinterpret_cast<const float4v *>(p + 8));
+            return __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7);
+        };
         auto frag_b = [&](const float *lb, const int set, const int kc, const int j) {
             fb[set][j] = *reinterpret_cast<const float4v *>(lb + (wn + j * 32 + li) * PITCH + kc * 8 + lg * 4);
         };
@@ -378,6 +387,64 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
                     rb.v[q % 8] = *reinterpret_cast<const float4v *>(pb + offb[q % 8]);
                 }
             };
+            if constexpr (HALF == 5) {
+                // fp8 runs at twice the 16-bit rate only on the 64-deep instruction (v_mfma_scale_f32_32x32x64_f8f6f4 with
+                // both scales 2^0; the 16-deep fp8 instruction takes the cycles of the 16-bit one): a lane feeds it 32 bytes
+                // of its row, two fragments.  A tile is two such double steps; B's four blocks stay in registers for a double
+                // step and are replaced one by one behind the last row's instructions, A rows go through a ring of two.  The
+                // barrier stands before the last row of the second double step; 16 slots over the 7 rows before it.
+                if constexpr (!STEADY) {
+                    // the first and the last tiles: nothing is carried in registers from one tile to the next (the guarded
+                    // loads need the registers): stage and ask first, then read this tile's fragments as they are needed
+                    if (next) {
+                        stage(ra, rb, cur ^ 1);
+                        if (kt + 2 < nk) ask(ra, rb, kt + 2);
+                    }
+                    fa8[0] = frag8(la, 0, wm);
+#pragma unroll
+                    for (int j = 0; j < NT; j++) fb8[j] = frag8(lb, 0, wn + j * 32);
+                }
+#pragma unroll
+                for (int d = 0; d < 2; d++) {
+#pragma unroll
+                    for (int i = 0; i < MT; i++) {
+                        const bool last = d == 1 && i == MT - 1;
+                        if (last) {
+                            if constexpr (STEADY) {
+                                asm volatile("" ::: "memory");
+                                __builtin_amdgcn_s_waitcnt(0xc07f);
+                                __builtin_amdgcn_s_barrier();
+                                asm volatile("" ::: "memory");
+                                fa8[0] = frag8(na, 0, wm);
+                            }
+                        } else if (i == MT - 1) {
+                            fa8[0] = frag8(la, 1, wm);
+                        } else {
+                            fa8[(i + 1) & 1] = frag8(la, d, wm + (i + 1) * 32);
+                        }
+#pragma unroll
+                        for (int j = 0; j < NT; j++) {
+                            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa8[i & 1], fb8[j], acc[i][j], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+                            if (i == MT - 1) {
+                                if (d == 0) fb8[j] = frag8(lb, 1, wn + j * 32);
+                                else if constexpr (STEADY) fb8[j] = frag8(nb, 0, wn + j * 32);
+                            }
+                        }
+                        if constexpr (STEADY) {
+                            const int g = d * MT + i; // 0..6 before the barrier: 3, 2, 2, 2, 3, 2, 2 slots
+                            if (g < 7) {
+                                const int first = g < 1 ? 0 : g < 5 ? 3 + (g - 1) * 2 : 12 + (g - 5) * 2;
+                                const int count = (g == 0 || g == 4) ? 3 : 2;
+#pragma unroll
+                                for (int c = 0; c < count; c++) slot(first + c);
+                            }
+                            __builtin_amdgcn_sched_barrier(0);
+                        }
+                    }
+                }
+                if constexpr (!STEADY) __syncthreads();
+                return;
+            }
 #pragma unroll
             for (int kc = 0; kc < S - 1; kc++) {
 #pragma unroll
@@ -415,6 +482,19 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
             }
         };
         static_assert(S % 2 == 0, "the last step multiplies from set 1 while set 0 is refilled");
+        auto first_fragments = [&]() {
+            if constexpr (HALF == 5) {
+                fa8[0] = frag8(lds_a(0), 0, wm);
+#pragma unroll
+                for (int j = 0; j < NT; j++) fb8[j] = frag8(lds_b(0), 0, wn + j * 32);
+            } else {
+#pragma unroll
+                for (int i = 0; i < MT; i++) {
+                    frag_a(lds_a(0), 0, 0, i);
+                    frag_b(lds_b(0), 0, 0, i);
+                }
+            }
+        };
         uint32_t kt = 0;
         if (lean && 3 * BK <= a.K) {
             // tile 1 is asked for slot by slot in the order the loop consumes the slots: only then does the compiler's count
@@ -431,19 +511,11 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
                 rb.v[h] = *reinterpret_cast<const float4v *>(pb + offb[h]);
                 __builtin_amdgcn_sched_barrier(0);
             }
-#pragma unroll
-            for (int i = 0; i < MT; i++) {
-                frag_a(lds_a(0), 0, 0, i);
-                frag_b(lds_b(0), 0, 0, i);
-            }
+            first_fragments();
             for (; (kt + 3) * BK <= a.K; kt++) iteration(kt, std::true_type{});
         } else {
             if (nk > 1) ask(ra, rb, 1); // (tile 0 is in LDS buffer 0 by now)
-#pragma unroll
-            for (int i = 0; i < MT; i++) {
-                frag_a(lds_a(0), 0, 0, i);
-                frag_b(lds_b(0), 0, 0, i);
-            }
+            if constexpr (HALF != 5) first_fragments();
         }
         for (; kt < nk; kt++) iteration(kt, std::false_type{});
     }

@@ -285,6 +285,47 @@ def test_format_tensor(hip):
     assert "f32[1,2]" in s and "1.5" in s
 
 
+# ---- the narrow-operand products on the 16-bit and fp8 matrix instructions, many tiles deep -----------------
+@pytest.mark.parametrize("dt", ["bf16", "f16", "fp8"])
+def test_narrow_operand_products_deep_in_k_are_exact_on_integers(hip, dt):
+    """Products that fill the device with 256 x 256 tiles run from operands narrowed in memory, through a loop whose
+    steady state (whole tiles, loads dealt out between the matrix instructions) only starts three tiles deep in k.
+    Small-integer operands make every partial sum an integer that f32 holds exactly, whatever the order of the additions,
+    so the result must equal the rounding of the exact product bit for bit.  K = 1088 is 17 tiles of the 16-bit dtypes and
+    8.5 of fp8 (a ragged last tile); 4000 x 4100 leaves ragged tile edges in both directions.  A second product against a
+    0/1 selection matrix returns columns of the left operand unchanged: every position along k reaches its partner."""
+    import cases_fp8
+    import cases_half
+    rng = np.random.default_rng(77)
+    M, N, K = 4000, 4100, 1088
+    if dt == "fp8":
+        av = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
+        bv = (rng.integers(-1, 2, size=(N, K)) * (rng.random((N, K)) < 0.125)).astype(np.float32)
+        up = lambda v: hip.ndarray_from_vec_fp8(cases_fp8.f8_encode(v), v.shape)
+        rd = lambda t: cases_fp8.read(hip, t)
+        rnd = cases_fp8.f8_round
+    else:
+        code = A.BF16 if dt == "bf16" else A.F16
+        av = rng.integers(-8, 9, size=(M, K)).astype(np.float32)
+        bv = rng.integers(-8, 9, size=(N, K)).astype(np.float32)
+        up = lambda v: cases_half.from_half(hip, code, cases_half.round_to(code, v))
+        rd = lambda t: cases_half.as_f32(code, cases_half.read(hip, t))
+        rnd = lambda x: cases_half.as_f32(code, cases_half.round_to(code, x))
+    a, b = up(av), up(bv)
+    got = rd(hip.matmul(a, hip.transpose(b, 0, 1)))
+    exact = av.astype(np.float64) @ bv.astype(np.float64).T
+    assert np.abs(exact).max() < 2 ** 24
+    exp = rnd(exact.astype(np.float32))
+    bad = np.argwhere(got != exp)
+    assert bad.size == 0, f"{dt}: {len(bad)} mismatches, first {bad[:3].tolist()}"
+    # selection: column n of the result is column sel[n] of the left operand
+    sel = rng.integers(0, K, size=N)
+    pv = np.zeros((N, K), dtype=np.float32)
+    pv[np.arange(N), sel] = 1.0
+    got = rd(hip.matmul(a, hip.transpose(up(pv), 0, 1)))
+    assert np.array_equal(got, av[:, sel])
+
+
 # ---- full-size checks through size-independent properties -----------------------------------
 def test_microbench_shapes_properties(hip):
     """Config-2 shapes: linearity / invariants instead of a CPU recomputation."""
