@@ -190,6 +190,48 @@ def test_random_matmul_shapes_match_oracle(hip, oracle, seed):
     assert float(np.abs(got - ref).max()) <= 1e-3 * scale, f"seed {seed}: M={M} K={K} N={N} batch={batch} xt={xt} yt={yt} pad={pad}"
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_random_wide_tile_products_match_float64(hip, seed):
+    """Products large enough for the 256 x 256 tile (at least 256 tiles), whose loop over k has a lean part (whole tiles of
+    aligned operands at fixed per-lane offsets) and a guarded tail: ragged extents in all three directions, either operand
+    k-contiguous or row-contiguous (a transposed view), slices that break the 16-byte alignment or leave a row pitch that is
+    no multiple of 4, and batches.  Against numpy in float64 (the oracle would take minutes per case); tolerance 1e-3 of
+    sum_k |a| |b| per element, as for every product."""
+    rng = np.random.default_rng(9100 + seed)
+    batch = (2,) if seed % 5 == 4 else ()
+    lo = 2900 if batch else 4097
+    M, N = (int(rng.integers(lo, lo + 600)) for _ in range(2))
+    if seed % 3 == 0:
+        M, N = (M + 3) // 4 * 4, (N + 3) // 4 * 4     # multiples of 4: row-contiguous operands take the lean loads too
+    K = int(rng.choice([33, 64, 96, 100, 128, 200, 257, 512]))
+    xt, yt = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+    pad_x, pad_y = (int(rng.choice([0, 0, 1, 4])) for _ in range(2))
+    x = (rng.standard_normal(batch + ((K, M + pad_x) if xt else (M, K + pad_x)))).astype(np.float32)
+    y = (rng.standard_normal(batch + ((N, K + pad_y) if yt else (K, N + pad_y)))).astype(np.float32)
+    r = len(batch) + 2
+    a, b = hip.from_numpy(x), hip.from_numpy(y)
+    if xt:
+        a = hip.transpose(hip.slice(a, r - 1, pad_x, M) if pad_x else a, r - 2, r - 1)
+        xv = np.swapaxes(x[..., pad_x:], -1, -2)
+    else:
+        a = hip.slice(a, r - 1, pad_x, K) if pad_x else a
+        xv = x[..., pad_x:]
+    if yt:
+        b = hip.transpose(hip.slice(b, r - 1, pad_y, K) if pad_y else b, r - 2, r - 1)
+        yv = np.swapaxes(y[..., pad_y:], -1, -2)
+    else:
+        b = hip.slice(b, r - 1, pad_y, N) if pad_y else b
+        yv = y[..., pad_y:]
+    print(f"seed={seed} batch={batch} M={M} N={N} K={K} xt={xt} yt={yt} pads={pad_x},{pad_y}", flush=True)
+    got = hip.to_numpy(hip.matmul(a, b))
+    x64, y64 = xv.astype(np.float64), yv.astype(np.float64)
+    exact = x64 @ y64
+    scale = np.abs(x64) @ np.abs(y64)
+    assert got.shape == exact.shape == batch + (M, N)
+    err = np.abs(got - exact)
+    assert (err <= 1e-3 * scale).all(), f"seed {seed}: worst {float((err / scale).max()):.3e} at {np.unravel_index(np.argmax(err / scale), err.shape)}"
+
+
 @pytest.mark.parametrize("seed", range(120))
 def test_random_attention_shapes_match_oracle(hip, oracle, seed):
     """The model graphs' attention (repeat_kv, scores, scale, causal mask rows, soft-max, context) at random
