@@ -253,8 +253,10 @@ __global__ __launch_bounds__(kBlock) void decode_attention_kernel(const AttnArgs
 // sum cross the waves through LDS), V is on its way while that happens, and the weighted sum is divided by the
 // row's sum where it is stored.  The workgroups of a batch entry (its query rows read the same K and V) get block
 // indices a multiple of eight apart, which lands them on the same XCD: the second to last read hit in its L2.
-// What bounds a workgroup is its compute unit's path to L2, 64 bytes a clock (K and V of 530 positions take
-// 1.8 us through it), and T x head_dim x 4 multiply-adds on one compute unit: taken up to T = 4096 in one launch and, in
+// What bounds a workgroup is its compute unit's path to L2: measured, a compute unit streams about 60 GB/s (25 bytes a
+// clock) out of L2 however many loads it keeps in flight (a ring of 16 passes per lane instead of two alternating trips
+// of six was no faster), and a workgroup pulls all of K plus its half of V through it (835 KB at T = 2176: 14 us).
+// Taken up to T = 4096 in one launch and, in
 // two segments per row whose results decode_attention_combine_kernel merges, up to 8192; longer caches go to the chunked
 // kernels, which spread a KV head over many workgroups.
 // PASSES x (1024 / LPT) positions per trip to memory.  LOOP: several trips, the next always asked for before the
