@@ -232,6 +232,36 @@ def test_random_wide_tile_products_match_float64(hip, seed):
     assert (err <= 1e-3 * scale).all(), f"seed {seed}: worst {float((err / scale).max()):.3e} at {np.unravel_index(np.argmax(err / scale), err.shape)}"
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_random_wide_tile_products_of_16_bit_dtypes(hip, seed):
+    """The same wide tile with bf16 / f16 tensors that cannot take the narrowed-in-memory path (a batch axis, or k no
+    multiple of 8): f32 words are narrowed on their way into LDS and multiplied on the 16-bit matrix instructions, with
+    either operand k-contiguous or row-contiguous.  Small-integer values: every partial sum is exact in f32, so the result
+    must be the rounding of the exact product, bit for bit."""
+    import cases_half
+    rng = np.random.default_rng(9300 + seed)
+    code = A.BF16 if seed % 2 == 0 else A.F16
+    batch = (2,) if seed % 3 != 2 else ()
+    lo = 2900 if batch else 4097
+    M, N = (int(rng.integers(lo, lo + 300)) for _ in range(2))
+    if seed % 4 == 1:
+        M, N = (M + 3) // 4 * 4, (N + 3) // 4 * 4
+    K = int(rng.choice([96, 130, 200, 264])) if batch else int(rng.choice([100, 130, 203]))
+    xt, yt = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+    xv = rng.integers(-6, 7, size=batch + (M, K)).astype(np.float32)
+    yv = rng.integers(-6, 7, size=batch + (K, N)).astype(np.float32)
+    r = len(batch) + 2
+    up = lambda v: cases_half.from_half(hip, code, cases_half.round_to(code, np.ascontiguousarray(v)))
+    a = hip.transpose(up(np.swapaxes(xv, -1, -2)), r - 2, r - 1) if xt else up(xv)
+    b = hip.transpose(up(np.swapaxes(yv, -1, -2)), r - 2, r - 1) if yt else up(yv)
+    print(f"seed={seed} dtype={'bf16' if code == A.BF16 else 'f16'} batch={batch} M={M} N={N} K={K} xt={xt} yt={yt}", flush=True)
+    got = cases_half.as_f32(code, cases_half.read(hip, hip.matmul(a, b)))
+    exact = (xv.astype(np.float64) @ yv.astype(np.float64)).astype(np.float32)
+    exp = cases_half.as_f32(code, cases_half.round_to(code, exact))
+    bad = np.argwhere(got != exp)
+    assert bad.size == 0, f"seed {seed}: {len(bad)} mismatches, first {bad[:3].tolist()}"
+
+
 @pytest.mark.parametrize("seed", range(120))
 def test_random_attention_shapes_match_oracle(hip, oracle, seed):
     """The model graphs' attention (repeat_kv, scores, scale, causal mask rows, soft-max, context) at random
