@@ -78,7 +78,7 @@ __device__ __forceinline__ void batch_offsets(const MmArgs &a, uint32_t b, int64
 // ------------------------------------------------------------------------------------------
 // MFMA kernel
 // ------------------------------------------------------------------------------------------
-constexpr int BM = 128, BN = 128, BK = 32; // BN = 64 in the narrow variant
+constexpr int BM = 128, BK = 32; // (the kernels shadow BM and define BN from their tile parameters)
 constexpr int PITCH = BK + 4; // words per LDS row: row r starts at bank 4r mod 32
 constexpr size_t gemm_lds_bytes(int bn, int bm = BM, bool half = false) {
     return 2 * (size_t)(bm + bn) * (half ? BK / 2 + 4 : PITCH) * sizeof(float);

@@ -1325,7 +1325,9 @@ for _B, _kvh, _rep, _T, _hd in ((2, 2, 4, 300, 64), (1, 3, 1, 1, 64), (2, 1, 8, 
                                 # batch that does not fill the last eight block indices, caches it takes in two segments and one
                                 # beyond its reach
                                 (4, 8, 4, 2100, 64), (1, 2, 2, 3000, 128), (5, 8, 4, 700, 64), (9, 1, 8, 1100, 128),
-                                (1, 2, 4, 4500, 64), (2, 2, 4, 9000, 64), (1, 1, 2, 5000, 128), (1, 2, 4, 7000, 64)):
+                                (1, 2, 4, 4500, 64), (2, 2, 4, 9000, 64), (1, 1, 2, 5000, 128), (1, 2, 4, 7000, 64),
+                                # few query rows at one sequence (the single-sequence decoder shapes)
+                                (1, 8, 2, 1100, 128), (1, 3, 3, 640, 64), (2, 4, 4, 2049, 64), (1, 2, 4, 513, 64)):
     @case(f"decode_attention_B{_B}_kv{_kvh}_rep{_rep}_T{_T}_hd{_hd}", "ew_abs")
     def _(B=_B, kvh=_kvh, rep=_rep, T=_T, hd=_hd):
         q = f32(400 + T, (B, kvh * rep, 1, hd))
