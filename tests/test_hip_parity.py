@@ -326,6 +326,51 @@ def test_narrow_operand_products_deep_in_k_are_exact_on_integers(hip, dt):
     assert np.array_equal(got, av[:, sel])
 
 
+@pytest.mark.parametrize("dt", ["bf16", "f16", "fp8"])
+def test_narrow_operand_products_carry_special_values(hip, dt):
+    """NaN, infinities (16-bit dtypes) and the largest magnitudes through the narrowed-in-memory products: a NaN operand
+    makes its whole row / column of the result NaN, inf x 0 is NaN, sums beyond the dtype's range come out as infinity
+    (16-bit) or saturate at 448 (fp8), and everything else equals the rounding of the exact product (small integers)."""
+    import cases_fp8
+    import cases_half
+    rng = np.random.default_rng(78)
+    M, N, K = 4096, 4096, 256
+    av = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
+    bv = (rng.integers(-1, 2, size=(N, K)) * (rng.random((N, K)) < 0.125)).astype(np.float32)
+    av[7, 3] = np.nan            # row 7 of the result is NaN
+    bv[11, 200] = np.nan         # column 11 too
+    big = 448.0 if dt == "fp8" else (3.0e38 if dt == "bf16" else 65504.0)
+    av[100] = 0.0                # (nothing else in this row: sums that mix huge and small terms depend on the order of addition)
+    av[100, :4] = big
+    bv[:, :4] = 0.0
+    bv[200, :4] = 1.0            # result[100, 200] = 4 x big exceeds the range
+    bv[201, :4] = [1.0, -1.0, 0.0, 0.0]  # cancels exactly: stays finite
+    if dt != "fp8":
+        av[300, 5] = np.inf
+        bv[400, 5] = 0.0         # inf x 0 = NaN at [300, 400]; elsewhere in row 300: +-inf or NaN by the signs of column 5
+    if dt == "fp8":
+        up = lambda v: hip.ndarray_from_vec_fp8(cases_fp8.f8_encode(v), v.shape)
+        rd = lambda t: cases_fp8.read(hip, t)
+        rnd = cases_fp8.f8_round
+    else:
+        code = A.BF16 if dt == "bf16" else A.F16
+        up = lambda v: cases_half.from_half(hip, code, cases_half.round_to(code, v))
+        rd = lambda t: cases_half.as_f32(code, cases_half.read(hip, t))
+        rnd = lambda x: cases_half.as_f32(code, cases_half.round_to(code, x))
+    got = rd(hip.matmul(up(av), hip.transpose(up(bv), 0, 1)))
+    with np.errstate(invalid="ignore", over="ignore"):
+        a_r, b_r = rnd(av).astype(np.float64), rnd(bv).astype(np.float64)   # (3.0e38 is not a bf16 value: what was uploaded)
+        exact = a_r @ b_r.T
+        exp = rnd(exact.astype(np.float32))
+    same = (got == exp) | (np.isnan(got) & np.isnan(exp))
+    bad = np.argwhere(~same)
+    assert bad.size == 0, f"{dt}: {len(bad)} mismatches, first {bad[:3].tolist()}: got {got[tuple(bad[0])]} expected {exp[tuple(bad[0])]}"
+    assert np.isnan(got[7]).all() and np.isnan(got[:, 11]).all()
+    assert (np.isinf(got[100, 200]) if dt != "fp8" else got[100, 200] == 448.0) and np.isfinite(got[100, 201])
+    if dt != "fp8":
+        assert np.isnan(got[300, 400])
+
+
 # ---- full-size checks through size-independent properties -----------------------------------
 def test_microbench_shapes_properties(hip):
     """Config-2 shapes: linearity / invariants instead of a CPU recomputation."""
