@@ -2102,9 +2102,14 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
         }
 #undef CG_MM_SWITCH
     } else {
-        // the narrow tile when the wide one would leave over a seventh of its columns empty
+        // the narrow tile when the wide one would leave over a seventh of its columns empty, and when the product has at
+        // most one 128 x 128 tile per compute unit: twice the workgroups then fill the chip (4096 x 2048 x 512: 148 -> 83 us)
+        // or at least put two on a unit (8192 x 2048 x 512: 148 -> 145 us); with more tiles than that the wide one wins
+        // (env CG_GEMM_NARROW_BELOW=n moves the limit, for measurements)
         const int64_t cols128 = (N + 127) / 128 * 128, cols64 = (N + 63) / 64 * 64;
-        const bool narrow = cols128 * 7 > cols64 * 8 && !half; // (the 16-bit kernels come in the two square tiles)
+        static const int64_t narrow_below = [] { const char *e = getenv("CG_GEMM_NARROW_BELOW"); return e ? atoll(e) : 256ll; }();
+        const int64_t tiles128 = ((M + BM - 1) / BM) * (cols128 / 128) * (int64_t)batch;
+        const bool narrow = (cols128 * 7 > cols64 * 8 || (tiles128 <= narrow_below && N >= 128)) && !half; // (the 16-bit kernels come in the two square tiles)
         const int bn = narrow ? 64 : 128;
         // the 256 x 256 tile when it covers the chip at least once (env CG_GEMM_BIG=0 switches it off)
         const uint64_t tiles_big = (uint64_t)((M + 255) / 256) * ((N + 255) / 256) * batch;
