@@ -310,7 +310,7 @@ def main():
         "backend_calls": {"prefill": calls[0], "per_decode_step": round(calls[1] / max(T, 1), 1)},
         "backend": sess.backend_name,
         "roofline": {
-            "kernel": "mfma_gemm_kernel (f32 v_mfma_f32_32x32x2; 256x256x32 tiles, 128x128 and 128x64 for small N)",
+            "kernel": "mfma_gemm_kernel (f32 v_mfma_f32_32x32x2; 128x128x32 tiles, two workgroups per compute unit; 128x64 for small products)",
             "bound": "mfma", "achieved": round(mfma_rate / 1e12, 3), "peak": MFMA_F32_PEAK / 1e12, "unit": "TFLOP/s",
             "frac": round(mfma_rate / MFMA_F32_PEAK, 4),
             # from the committed rocprofv3 counter summary of this very workload (null for any other)

@@ -2117,7 +2117,14 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
             const char *e = getenv("CG_GEMM_BIG");
             return !(e && e[0] == '0');
         }();
-        const bool big = big_allowed && !narrow && tiles_big >= 256 && M >= 256 && N >= 256;
+        const bool fits_big = big_allowed && !narrow && tiles_big >= 256 && M >= 256 && N >= 256;
+        // f32 words: since whole tiles are loaded without tests, two workgroups of the 128 x 128 tile per compute unit (two
+        // waves per SIMD covering each other's barriers) are as fast as one of the wide tile or faster — 137-138 against
+        // 134-135 TFLOP/s on the 1B shape's linear layers, and a partial last round costs a quarter as much (8192 x 2048 x
+        // 3072: 755 against 1015 us) — except with a k-contiguous left and a row-contiguous right operand (x.y: 1 % behind).
+        // The 16-bit and fp8 paths keep the wide tile (half the L2 bytes per flop, which is what bounds them).
+        const bool narrow_dtype = half || x->dt == CG_F8;
+        const bool big = fits_big && (narrow_dtype || (!a_mfast && b_nfast));
         uint64_t tiles = big ? tiles_big / batch : (uint64_t)((M + BM - 1) / BM) * ((N + bn - 1) / bn);
         if (tiles > 0x7FFFFFFFull) return fail(CG_ERR_UNSUPPORTED, "matmul: too many tiles");
         dim3 grid((uint32_t)tiles, (uint32_t)batch);
