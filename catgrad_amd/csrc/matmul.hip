@@ -9,16 +9,20 @@
 // axes form one run, the batch is folded into M (one tall GEMM instead of B small ones).
 //
 // Kernels
-//   mfma_gemm_kernel   256 threads = 2x2 waves, one template for three macro tiles: 256x256x32 (each
-//                      wave a 128x128 block as 4x4 v_mfma_f32_32x32x2_f32 accumulators, all 256
-//                      accumulation registers, 144 KiB of LDS) whenever the product has at least
-//                      one such tile per compute unit, 128x128x32 (2x2 accumulators per wave) for
-//                      smaller products, 128x64x32 when N is a small multiple of 64; HALF variants
+//   mfma_gemm_kernel   256 threads = 2x2 waves, one template for three macro tiles: 128x128x32 (2x2
+//                      v_mfma_f32_32x32x2_f32 accumulators per wave, two workgroups per compute unit) for
+//                      f32 products, 128x64x32 when N is a small multiple of 64 or the product has at
+//                      most one 128x128 tile per compute unit, 256x256x32 (each wave a 128x128 block as
+//                      4x4 accumulators, all 256 accumulation registers, 144 KiB of LDS) for the 16-bit
+//                      and fp8 products and for x.y with a row-contiguous right operand when there is at
+//                      least one such tile per compute unit; HALF variants
 //                      narrow the tiles to bf16 / f16 on their way into LDS, or read operands that
 //                      pack_operand_kernel narrowed in memory (bf16 / f16 / fp8), and issue
-//                      v_mfma_f32_32x32x16_{bf16,f16,fp8_fp8}.  A and B tiles are staged K-fastest in LDS
-//                      (pitch 36 words: 128-bit fragment reads and tile stores are both free of
-//                      bank conflicts), two LDS buffers, next tile's global loads in flight during
+//                      v_mfma_f32_32x32x16_{bf16,f16} / v_mfma_scale_f32_32x32x64_f8f6f4.  Tiles of
+//                      k-contiguous operands are staged K-fastest in LDS (pitch 36 words: 128-bit fragment
+//                      reads and tile stores are both free of bank conflicts), those of row-contiguous f32
+//                      operands rows-fastest; whole tiles are loaded at fixed per-lane offsets without
+//                      tests; two LDS buffers, next tile's global loads in flight during
 //                      the MFMAs, XCD-aware tile order.  MFMA-bound: 2*M*N*K flop.
 //   skinny_kt_*        M <= 8 with K-contiguous B rows (decode-time linear layers and q.K^T),
 //                      HBM-bound streams of B (4*K*N bytes):
