@@ -1791,7 +1791,8 @@ static bool packed_mfma_ok() {
 }
 
 // The narrow copy of the [rows, K] view (row stride s_r, k stride s_k, in words) at `ptr` inside `buf`; kept with the buffer
-// when `keep` (the right operand: a weight matrix is narrowed once), else the caller frees *tmp after its launch.
+// when `keep` and the buffer holds none yet (a weight matrix is narrowed once, activations once for the products that
+// share them), else the caller frees *tmp after its launch.
 static int pack_operand(cg_backend *be, Buffer *buf, const uint32_t *ptr, int64_t s_r, int64_t s_k, int64_t rows, int64_t K, int kind,
                         bool keep, const void **packed, void **tmp, size_t *tmp_cls) {
     const int64_t off = ptr - static_cast<const uint32_t *>(buf->ptr);
@@ -2167,7 +2168,8 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
             const void *pa = nullptr, *pb = nullptr;
             void *ta = nullptr, *tb = nullptr;
             size_t ca = 0, cb = 0;
-            int prc = pack_operand(be, x->buf, a.A, a.a_sm, a.a_sk, M, K, kind, false, &pa, &ta, &ca);
+            // (the left operand's narrow copy is kept with its buffer too: q / k / v and gate / up multiply the same activations)
+            int prc = pack_operand(be, x->buf, a.A, a.a_sm, a.a_sk, M, K, kind, true, &pa, &ta, &ca);
             if (!prc) prc = pack_operand(be, y->buf, a.B, a.b_sn, a.b_sk, N, K, kind, true, &pb, &tb, &cb);
             if (!prc) {
                 MmArgs p = a;
