@@ -21,7 +21,7 @@ NEG, SIN, COS, EXP, LOG, FLOOR, ROUND = range(7)
 ADD, SUB, MUL, DIV, POW, LT, GT, GTE, LTE, EQ = range(10)
 
 # enum cg_kernel_class
-K_GEMM_MFMA, K_GEMM_SKINNY, K_GEMM_SIMPLE, K_ELEMENTWISE, K_REDUCE, K_GATHER, K_ATTENTION = range(7)
+K_GEMM_MFMA, K_GEMM_SKINNY, K_GEMM_SIMPLE, K_ELEMENTWISE, K_REDUCE, K_GATHER, K_ATTENTION, K_PACK = range(8)
 
 _P = C.c_void_p
 _PP = C.POINTER(C.c_void_p)
@@ -65,6 +65,7 @@ SIGNATURES = {
     "cg_sum": (_I, [_P, _P, _PP]),
     "cg_max": (_I, [_P, _P, _PP]),
     "cg_argmax": (_I, [_P, _P, _PP]),
+    "cg_noalloc_setup": (_I, [_I]),
     "cg_argmax_rows_noalloc": (_I, [_I, _I, _P, _SZ, _SZ, _P, _P]),
     "cg_topk": (_I, [_P, _P, _SZ, _PP, _PP]),
     "cg_broadcast": (_I, [_P, _P, _SZP, _SZ, _PP]),

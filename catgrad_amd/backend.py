@@ -332,6 +332,10 @@ def load_hip_library():
                 f"{HIP_LIBRARY} is missing: build it with `make -C {os.path.dirname(HIP_LIBRARY)}` "
                 "(or `python -c 'import __graft_entry__ as g; g.build()'`). There is no CPU fallback."
             )
+        try:  # a process that also uses torch must hold ONE HIP runtime, torch's: torch goes first when it is there
+            import torch  # noqa: F401
+        except ImportError:
+            pass
         _hip_lib = A.bind(HIP_LIBRARY)
     return _hip_lib
 

@@ -139,15 +139,22 @@ struct Buffer {
     void *side = nullptr;
     size_t side_cls = 0;
     uint32_t side_blocks = 0;
-    // A narrow copy of one 2-D view of this buffer for the matrix instructions of its dtype (launch_matmul): [rows][k] of
-    // 2-byte (f16 / bf16) or 1-byte (fp8) patterns, k contiguous.  A weight matrix is narrowed once and the copy kept while
-    // the buffer lives; what a view shows never changes (in-place appends write behind it), so the copy stays valid.
-    // Owned (pool memory).
-    void *packed = nullptr;
-    size_t packed_cls = 0;
-    int packed_kind = 0; // 1 bf16, 2 f16, 3 fp8
-    int64_t packed_off = 0, packed_rows = 0, packed_k = 0, packed_sr = 0, packed_sk = 0;
+    // Narrow copies of 2-D views of this buffer for the matrix instructions of its dtype (launch_matmul): [rows][k] of
+    // 2-byte (f16 / bf16) or 1-byte (fp8) patterns, k contiguous, one entry per view (several slices of one weight buffer
+    // each keep theirs; the oldest goes when the list is full).  A weight matrix is narrowed once and the copy kept while
+    // the buffer lives.  Every path that writes into an existing buffer drops the list first (drop_packed), so an entry
+    // always describes what its view shows.  Owned (pool memory).
+    struct Packed {
+        void *ptr = nullptr;
+        size_t cls = 0;
+        int kind = 0; // 1 bf16, 2 f16, 3 fp8
+        int64_t off = 0, rows = 0, k = 0, sr = 0, sk = 0;
+    };
+    std::vector<Packed> packed;
 };
+constexpr size_t kMaxPackedPerBuffer = 4;
+// Frees the narrow copies kept with `b` (to be called before anything is written into a buffer that existed before).
+void drop_packed(Buffer *b);
 
 } // namespace cg
 

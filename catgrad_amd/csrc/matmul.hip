@@ -1790,35 +1790,45 @@ static bool packed_mfma_ok() {
     return ok;
 }
 
-// The narrow copy of the [rows, K] view (row stride s_r, k stride s_k, in words) at `ptr` inside `buf`; kept with the buffer
-// when `keep` and the buffer holds none yet (a weight matrix is narrowed once, activations once for the products that
-// share them), else the caller frees *tmp after its launch.
+// The narrow copy of the [rows, K] view (row stride s_r, k stride s_k, in words) at `ptr` inside `buf`: the copy kept with
+// the buffer for this very view if there is one; else a new one, kept with the buffer when `keep` (a weight matrix is
+// narrowed once, shared activations once for the products that multiply them; the oldest entry makes room when the list is
+// full), else handed to the caller, who frees *tmp after its launch.
 static int pack_operand(cg_backend *be, Buffer *buf, const uint32_t *ptr, int64_t s_r, int64_t s_k, int64_t rows, int64_t K, int kind,
                         bool keep, const void **packed, void **tmp, size_t *tmp_cls) {
     const int64_t off = ptr - static_cast<const uint32_t *>(buf->ptr);
-    if (buf->packed && buf->packed_kind == kind && buf->packed_off == off && buf->packed_rows == rows && buf->packed_k == K &&
-        buf->packed_sr == s_r && buf->packed_sk == s_k) {
-        *packed = buf->packed;
-        return CG_OK;
-    }
+    for (const Buffer::Packed &p : buf->packed)
+        if (p.kind == kind && p.off == off && p.rows == rows && p.k == K && p.sr == s_r && p.sk == s_k) {
+            *packed = p.ptr;
+            return CG_OK;
+        }
     void *dst = nullptr;
     size_t cls = 0;
     int rc = be->pool.alloc((size_t)rows * (size_t)K * (kind == 3 ? 1 : 2), &dst, &cls);
     if (rc) return rc;
     const uint64_t quads = (uint64_t)rows * (uint64_t)(K / 4);
     const dim3 grid((uint32_t)((quads + kThreads - 1) / kThreads));
-    if (kind == 1) hipLaunchKernelGGL(pack_operand_kernel<1>, grid, dim3(kThreads), 0, be->stream, ptr, s_r, s_k, (uint32_t)rows, (uint32_t)K, dst);
-    else if (kind == 2) hipLaunchKernelGGL(pack_operand_kernel<2>, grid, dim3(kThreads), 0, be->stream, ptr, s_r, s_k, (uint32_t)rows, (uint32_t)K, dst);
-    else hipLaunchKernelGGL(pack_operand_kernel<3>, grid, dim3(kThreads), 0, be->stream, ptr, s_r, s_k, (uint32_t)rows, (uint32_t)K, dst);
-    if (keep && !buf->packed) {
-        buf->packed = dst;
-        buf->packed_cls = cls;
-        buf->packed_kind = kind;
-        buf->packed_off = off;
-        buf->packed_rows = rows;
-        buf->packed_k = K;
-        buf->packed_sr = s_r;
-        buf->packed_sk = s_k;
+    {
+        ProfScope prof(be, CG_K_PACK, (double)rows * (double)K * (4.0 + (kind == 3 ? 1.0 : 2.0)));
+        if (kind == 1) hipLaunchKernelGGL(pack_operand_kernel<1>, grid, dim3(kThreads), 0, be->stream, ptr, s_r, s_k, (uint32_t)rows, (uint32_t)K, dst);
+        else if (kind == 2) hipLaunchKernelGGL(pack_operand_kernel<2>, grid, dim3(kThreads), 0, be->stream, ptr, s_r, s_k, (uint32_t)rows, (uint32_t)K, dst);
+        else hipLaunchKernelGGL(pack_operand_kernel<3>, grid, dim3(kThreads), 0, be->stream, ptr, s_r, s_k, (uint32_t)rows, (uint32_t)K, dst);
+    }
+    if (keep) {
+        if (buf->packed.size() >= kMaxPackedPerBuffer) { // stream-ordered free: products already queued on it come first
+            be->pool.free(buf->packed.front().ptr, buf->packed.front().cls);
+            buf->packed.erase(buf->packed.begin());
+        }
+        Buffer::Packed p;
+        p.ptr = dst;
+        p.cls = cls;
+        p.kind = kind;
+        p.off = off;
+        p.rows = rows;
+        p.k = K;
+        p.sr = s_r;
+        p.sk = s_k;
+        buf->packed.push_back(p);
     } else {
         *tmp = dst;
         *tmp_cls = cls;
@@ -2168,8 +2178,10 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
             const void *pa = nullptr, *pb = nullptr;
             void *ta = nullptr, *tb = nullptr;
             size_t ca = 0, cb = 0;
-            // (the left operand's narrow copy is kept with its buffer too: q / k / v and gate / up multiply the same activations)
-            int prc = pack_operand(be, x->buf, a.A, a.a_sm, a.a_sk, M, K, kind, true, &pa, &ta, &ca);
+            // (the left operand's narrow copy is kept with its buffer when somebody else holds the activations too — q / k / v
+            // and gate / up multiply the same ones —; an operand only this product reads is narrowed for it alone)
+            const bool x_shared = x->rc.load() > 1 || x->buf->rc.load() > 1;
+            int prc = pack_operand(be, x->buf, a.A, a.a_sm, a.a_sk, M, K, kind, x_shared, &pa, &ta, &ca);
             if (!prc) prc = pack_operand(be, y->buf, a.B, a.b_sn, a.b_sk, N, K, kind, true, &pb, &tb, &cb);
             if (!prc) {
                 MmArgs p = a;

@@ -472,17 +472,23 @@ static __device__ __align__(256) long long scratch[kNoAllocMaxParts];
 
 constexpr int kNoAllocMaxDevices = 64;
 static std::mutex g_scratch_mu;
-static long long *g_scratch_ptr[kNoAllocMaxDevices] = {};
+static std::atomic<long long *> g_scratch_ptr[kNoAllocMaxDevices] = {};
 
+// Set-up (loads the code object on `device` if need be, so it is not for code under stream capture): leaves the
+// calling thread's current device as it found it.
 int noalloc_setup(int device) {
     if (device < 0 || device >= kNoAllocMaxDevices) return fail(CG_ERR_ARG, "device %d out of range", device);
     std::lock_guard<std::mutex> lk(g_scratch_mu);
-    if (g_scratch_ptr[device]) return CG_OK;
+    if (g_scratch_ptr[device].load(std::memory_order_acquire)) return CG_OK;
+    int prev = -1;
+    CG_HIP(hipGetDevice(&prev));
     CG_HIP(hipSetDevice(device));
     long long *ptr = nullptr;
-    CG_HIP(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
+    const hipError_t e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
+    if (prev != device) (void)hipSetDevice(prev);
+    if (e != hipSuccess) return hip_fail(e, "hipGetSymbolAddress(scratch)");
     if (!ptr) return fail(CG_ERR_DEVICE, "no device address for the scratch array on device %d", device);
-    g_scratch_ptr[device] = ptr;
+    g_scratch_ptr[device].store(ptr, std::memory_order_release);
     return CG_OK;
 }
 
@@ -547,9 +553,12 @@ int launch_any_diff(cg_backend *be, const cg_tensor *x, const cg_tensor *y) { re
 
 } // namespace cg
 
+extern "C" int cg_noalloc_setup(int device) { return cg::noalloc_setup(device); }
+
 // Arg-max over the rows of a dense [rows, n] array of 32-bit words at `x` (device memory) into out[rows] (device
 // memory), queued on `stream`; nothing is allocated and nothing waits.  Same kernels as the segmented arg-max behind
-// cg_argmax, with the per-segment results in the library's fixed scratch array.
+// cg_argmax, with the per-segment results in the library's fixed scratch array, whose address on `device` set-up
+// (cg_noalloc_setup, or cg_backend_create on that device) must have asked for before: the call itself resolves nothing.
 extern "C" int cg_argmax_rows_noalloc(int device, cg_dtype dtype, const void *x, size_t rows, size_t n, uint32_t *out,
                                       void *stream) {
     using namespace cg;
@@ -567,10 +576,15 @@ extern "C" int cg_argmax_rows_noalloc(int device, cg_dtype dtype, const void *x,
                     "argmax without allocation: %zu rows x %u segments exceed the fixed scratch of %u partial results "
                     "(rows x ceil(n / 1024), segments capped at 256)",
                     rows, segs, kNoAllocMaxParts);
-    int rc = noalloc_setup(device); // the first call on a device asks for the array's address there
-    if (rc) return rc;
-    CG_HIP(hipSetDevice(device));
-    long long *part = g_scratch_ptr[device];
+    if (device < 0 || device >= kNoAllocMaxDevices) return fail(CG_ERR_ARG, "device %d out of range", device);
+    long long *part = g_scratch_ptr[device].load(std::memory_order_acquire);
+    if (!part)
+        return fail(CG_ERR_ARG, "argmax without allocation: device %d is not set up (call cg_noalloc_setup or cg_backend_create "
+                                "on it first, outside any stream capture)", device);
+    // the launches go to `device`; the calling thread's current device is put back before the call returns
+    int prev = -1;
+    CG_HIP(hipGetDevice(&prev));
+    if (prev != device) CG_HIP(hipSetDevice(device));
     RowsArgs a;
     memset(&a, 0, sizeof a);
     a.x = static_cast<const char *>(x);
@@ -593,5 +607,6 @@ extern "C" int cg_argmax_rows_noalloc(int device, cg_dtype dtype, const void *x,
         hipLaunchKernelGGL((reduce_segments_final_kernel<kArgmax, true>), dim3(a.rows), dim3(64), 0, s, part, out, segs);
     }
     hipError_t e = hipGetLastError();
+    if (prev != device) (void)hipSetDevice(prev);
     return e == hipSuccess ? CG_OK : hip_fail(e, "argmax without allocation: launch");
 }

@@ -110,11 +110,17 @@ bool is_contiguous(const cg_tensor *t) {
     return true;
 }
 
+void drop_packed(Buffer *b) {
+    if (!b) return;
+    for (Buffer::Packed &p : b->packed) b->be->pool.free(p.ptr, p.cls); // stream-ordered: queued readers come first
+    b->packed.clear();
+}
+
 static void buffer_release(Buffer *b) {
     while (b && b->rc.fetch_sub(1) == 1) {
         if (b->ptr) b->be->pool.free(b->ptr, b->cls);
         if (b->side) b->be->pool.free(b->side, b->side_cls);
-        if (b->packed) b->be->pool.free(b->packed, b->packed_cls);
+        drop_packed(b);
         Buffer *next = b->successor;
         delete b->rs;
         delete b;
@@ -904,6 +910,7 @@ static int try_residual_store(cg_backend *be, const cg_tensor *dst, const Pendin
 }
 
 static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p, bool fresh) {
+    if (!fresh) drop_packed(dst->buf); // a part of a buffer that may have been multiplied before is about to change
     if (be->aot) {
         int grc = try_gated_pair(be, dst, p);
         if (grc == kDeclined) grc = try_residual_store(be, dst, p, fresh);
@@ -1221,6 +1228,7 @@ static int defer_write(cg_backend *be, const cg_tensor *dst, const Pending *prog
         int rc = flush_deferred(be);
         if (rc) return rc;
     }
+    drop_packed(dst->buf);
     DeferredWrite w;
     w.dst = new cg_tensor;
     w.dst->be = be;
@@ -1780,6 +1788,7 @@ static bool try_row_append(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim
         dst.offset = x->offset / (C * R) * (dC * R) + row0 * R;
         const cg_tensor *ins[1] = {src_t};
         int rc;
+        drop_packed(dstbuf);
         if (src_t->pend && may_wait(b, &dst, src_t->pend))
             rc = defer_write(b, &dst, src_t->pend); // the rows are written with the next launch
         else
@@ -1956,6 +1965,7 @@ const char *cg_backend_name(cg_backend *b) { return b ? b->name.c_str() : ""; }
 
 int cg_sync(cg_backend *b) {
     Enter entered(b);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b) return fail(CG_ERR_ARG, "null backend");
     if (int frc = flush_deferred(b)) return frc;
     return wait_and_check(b);
@@ -1963,6 +1973,7 @@ int cg_sync(cg_backend *b) {
 
 int cg_pool_stats(cg_backend *b, size_t *bytes_in_use, size_t *bytes_cached) {
     Enter entered(b);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b) return fail(CG_ERR_ARG, "null backend");
     b->pool.stats(bytes_in_use, bytes_cached);
     // what the backend keeps for itself (iota, results of constant programs) counts as cached
@@ -1974,6 +1985,7 @@ int cg_pool_stats(cg_backend *b, size_t *bytes_in_use, size_t *bytes_cached) {
 
 int cg_pool_trim(cg_backend *b) {
     Enter entered(b);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b) return fail(CG_ERR_ARG, "null backend");
     CG_HIP(hipStreamSynchronize(b->stream));
     const_memo_clear(b);
@@ -1983,6 +1995,7 @@ int cg_pool_trim(cg_backend *b) {
 
 int cg_profile_enable(cg_backend *b, cg_kernel_class cls, unsigned sample_every) {
     Enter entered(b);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b || (int)cls < 0 || (int)cls >= CG_K_CLASSES) return fail(CG_ERR_ARG, "bad profile class");
     b->prof[cls].every = sample_every;
     return CG_OK;
@@ -1990,6 +2003,7 @@ int cg_profile_enable(cg_backend *b, cg_kernel_class cls, unsigned sample_every)
 
 int cg_program_stats(cg_backend *b, uint64_t *compiled, uint64_t *interpreted, int reset) {
     Enter entered(b);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b) return fail(CG_ERR_ARG, "null backend");
     if (compiled) *compiled = b->programs_compiled;
     if (interpreted) *interpreted = b->programs_interpreted;
@@ -1999,6 +2013,7 @@ int cg_program_stats(cg_backend *b, uint64_t *compiled, uint64_t *interpreted, i
 
 int cg_realize(cg_backend *b, cg_tensor *t) {
     Enter entered(b);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b || !t) return fail(CG_ERR_ARG, "null argument");
     return ensure_concrete(t);
 }
@@ -2006,6 +2021,7 @@ int cg_realize(cg_backend *b, cg_tensor *t) {
 int cg_profile_read(cg_backend *b, cg_kernel_class cls, uint64_t *launches, double *milliseconds, double *work,
                     int reset) {
     Enter entered(b);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b || (int)cls < 0 || (int)cls >= CG_K_CLASSES) return fail(CG_ERR_ARG, "bad profile class");
     int rc = wait_and_check(b);
     if (rc) return rc;
@@ -2058,6 +2074,7 @@ static int check_dims(const size_t *dims, size_t rank, int64_t *d64) {
 // ndarray.rs:71-84 — a zero tensor is a uniform constant: no memory, no memset.
 int cg_zeros(cg_backend *b, cg_dtype dtype, const size_t *dims, size_t rank, cg_tensor **out) {
     Enter entered(b);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(dtype)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
     int64_t d[kMaxRank];
@@ -2095,6 +2112,7 @@ static int staged_upload(cg_backend *b, void *dst, const void *src, size_t bytes
 int cg_from_host(cg_backend *b, cg_dtype dtype, const void *data, size_t len, const size_t *dims, size_t rank,
                  cg_tensor **out) {
     Enter entered(b);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(dtype)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
     int64_t d[kMaxRank];
@@ -2151,6 +2169,7 @@ int cg_from_host(cg_backend *b, cg_dtype dtype, const void *data, size_t len, co
 int cg_from_host_bf16_as_f32(cg_backend *b, const uint16_t *bits, size_t len, const size_t *dims, size_t rank,
                              cg_tensor **out) {
     Enter entered(b);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b || !out) return fail(CG_ERR_ARG, "null argument");
     int64_t d[kMaxRank];
     int rc = check_dims(dims, rank, d);
@@ -2190,6 +2209,7 @@ int cg_from_host_bf16_as_f32(cg_backend *b, const uint16_t *bits, size_t len, co
 // rather than reproducing the reference's rounding artefacts.
 int cg_arange(cg_backend *b, size_t end, cg_tensor **out) {
     Enter entered(b);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b || !out) return fail(CG_ERR_ARG, "null argument");
     if (end > (1u << 24)) return fail(CG_ERR_UNSUPPORTED, "arange: end above 2^24 is inexact in the reference");
     int64_t d[1] = {(int64_t)end};
@@ -2272,6 +2292,7 @@ static int copy_out(cg_backend *b, const cg_tensor *t, void *dst, size_t len) {
 // ndarray.rs:50-58.  Non-contiguous views are materialised first (the reference panics).
 int cg_to_host(cg_backend *b, const cg_tensor *t, void *dst, size_t len) {
     Enter entered(b);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b || !t || (!dst && len)) return fail(CG_ERR_ARG, "null argument");
     if ((int64_t)len != numel(t)) return fail(CG_ERR_SHAPE, "to_vec: length mismatch");
     CG_HIP(hipSetDevice(b->device));
@@ -2327,6 +2348,7 @@ static int read_flag(cg_backend *b, int *out) {
 // ndarray.rs:140-149
 int cg_to_bool(cg_backend *b, const cg_tensor *t, int *out) {
     Enter entered(b);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b || !t || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(t->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
     CG_HIP(hipSetDevice(b->device));
@@ -2348,6 +2370,7 @@ int cg_to_bool(cg_backend *b, const cg_tensor *t, int *out) {
 // ndarray.rs:534-541
 int cg_compare(cg_backend *b, const cg_tensor *x, const cg_tensor *y, int *out) {
     Enter entered(b);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b || !x || !y || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt) || !supported(y->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
     if (x->dt != y->dt) return fail(CG_ERR_DTYPE, "compare: dtype mismatch");
@@ -2373,6 +2396,7 @@ int cg_compare(cg_backend *b, const cg_tensor *x, const cg_tensor *y, int *out) 
 // ndarray.rs:60-69 — free-form debug rendering: dtype, shape and the first 16 elements.
 int cg_format_tensor(cg_backend *b, const cg_tensor *t, char *buf, size_t cap) {
     Enter entered(b);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b || !t || !buf || !cap) return fail(CG_ERR_ARG, "null argument");
     CG_HIP(hipSetDevice(b->device));
     size_t n = (size_t)numel(t);
@@ -2450,6 +2474,7 @@ static int retag(cg_backend *b, cg_tensor *x, cg_dtype target, cg_tensor **out) 
 int cg_cast(cg_backend *b, cg_tensor *x, cg_dtype target, cg_tensor **out) {
     Enter entered(b);
     Consume cx(x);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b || !x || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(target) || !supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
     if (target == x->dt) { // identity: hand the same handle back
@@ -2478,6 +2503,7 @@ int cg_cast(cg_backend *b, cg_tensor *x, cg_dtype target, cg_tensor **out) {
 int cg_unary(cg_backend *b, cg_unary_op op, cg_tensor *x, cg_tensor **out) {
     Enter entered(b);
     Consume cx(x);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b || !x || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
     if ((int)op < CG_NEG || (int)op > CG_ROUND) return fail(CG_ERR_ARG, "unknown unary op %d", (int)op);
@@ -2503,6 +2529,7 @@ int cg_unary(cg_backend *b, cg_unary_op op, cg_tensor *x, cg_tensor **out) {
 int cg_binary(cg_backend *b, cg_binary_op op, cg_tensor *x, cg_tensor *y, cg_tensor **out) {
     Enter entered(b);
     Consume cx(x), cy(y);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b || !x || !y || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt) || !supported(y->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
     if ((int)op < CG_ADD || (int)op > CG_EQ) return fail(CG_ERR_ARG, "unknown binary op %d", (int)op);
@@ -2529,6 +2556,7 @@ int cg_binary(cg_backend *b, cg_binary_op op, cg_tensor *x, cg_tensor *y, cg_ten
 int cg_where(cg_backend *b, cg_tensor *mask, cg_tensor *x, cg_tensor *y, cg_tensor **out) {
     Enter entered(b);
     Consume cm(mask), cx(x), cy(y);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b || !mask || !x || !y || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
     if (mask->dt != x->dt || y->dt != x->dt) return fail(CG_ERR_DTYPE, "TypeError: mixed dtypes in where");
@@ -2550,6 +2578,7 @@ int cg_matmul(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **out) {
 }
 static int matmul_entry(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **out) {
     Consume cx(x), cy(y);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b || !x || !y || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt) || !supported(y->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
     if (x->dt != y->dt) return fail(CG_ERR_DTYPE, "TypeError: mixed dtypes in matmul");
@@ -2666,6 +2695,7 @@ static int matmul_entry(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **o
 static int reduce_entry(cg_backend *b, int kind, const char *what, cg_tensor *x, cg_tensor **out) {
     Enter entered(b);
     Consume cx(x);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b || !x || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
     if (x->rank == 0) return fail(CG_ERR_SHAPE, "%s: rank-0 tensor has no last axis", what);
@@ -2724,6 +2754,7 @@ int cg_argmax(cg_backend *b, cg_tensor *x, cg_tensor **out) { return reduce_entr
 int cg_topk(cg_backend *b, cg_tensor *x, size_t k, cg_tensor **values, cg_tensor **indices) {
     Enter entered(b);
     Consume cx(x);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b || !x || !values || !indices) return fail(CG_ERR_ARG, "null argument");
     if (x->dt == CG_U32) return fail(CG_ERR_DTYPE, "Unsupported type for topk");
     if (!is_f(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
@@ -2763,6 +2794,7 @@ int cg_topk(cg_backend *b, cg_tensor *x, size_t k, cg_tensor **values, cg_tensor
 int cg_broadcast(cg_backend *b, cg_tensor *x, const size_t *dims, size_t rank, cg_tensor **out) {
     Enter entered(b);
     Consume cx(x);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b || !x || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
     int64_t d[kMaxRank];
@@ -2821,6 +2853,7 @@ int cg_broadcast(cg_backend *b, cg_tensor *x, const size_t *dims, size_t rank, c
 int cg_reshape(cg_backend *b, cg_tensor *x, const size_t *dims, size_t rank, cg_tensor **out) {
     Enter entered(b);
     Consume cx(x);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b || !x || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
     int64_t d[kMaxRank];
@@ -2903,6 +2936,7 @@ int cg_reshape(cg_backend *b, cg_tensor *x, const size_t *dims, size_t rank, cg_
 int cg_transpose(cg_backend *b, cg_tensor *x, size_t dim0, size_t dim1, cg_tensor **out) {
     Enter entered(b);
     Consume cx(x);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b || !x || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
     if (dim0 >= (size_t)x->rank || dim1 >= (size_t)x->rank) return fail(CG_ERR_RANGE, "transpose: axis out of range");
@@ -2930,6 +2964,7 @@ int cg_transpose(cg_backend *b, cg_tensor *x, size_t dim0, size_t dim1, cg_tenso
 int cg_slice(cg_backend *b, cg_tensor *x, size_t dim, size_t start, size_t len, cg_tensor **out) {
     Enter entered(b);
     Consume cx(x);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b || !x || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
     if (dim >= (size_t)x->rank) return fail(CG_ERR_RANGE, "slice: axis out of range");
@@ -2961,6 +2996,7 @@ int cg_slice(cg_backend *b, cg_tensor *x, size_t dim, size_t start, size_t len, 
 int cg_concat(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor **out) {
     Enter entered(b);
     Consume cx(x), cy(y);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b || !x || !y || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt) || !supported(y->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
     if (x->dt != y->dt) return fail(CG_ERR_DTYPE, "Incompatible types for concatenation");
@@ -3076,6 +3112,7 @@ int cg_concat(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor *
         tail.buf = nullptr;
         if (rc) return rc;
         x->buf->elems = nx + ny;
+        drop_packed(x->buf);
         if (x->buf->side) { // row sums kept for the rows this buffer held so far do not describe the grown tensor
             b->pool.free(x->buf->side, x->buf->side_cls);
             x->buf->side = nullptr;
@@ -3154,6 +3191,7 @@ int cg_concat(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor *
 int cg_index(cg_backend *b, cg_tensor *x, size_t dim, cg_tensor *indices, cg_tensor **out) {
     Enter entered(b);
     Consume cx(x), ci(indices);
+    if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b || !x || !indices || !out) return fail(CG_ERR_ARG, "null argument");
     if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
     if (indices->dt != CG_U32) return fail(CG_ERR_DTYPE, "Invalid input types for indexing");

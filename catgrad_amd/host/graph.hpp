@@ -13,8 +13,10 @@
 // operations layer by layer through the same `tensor_op()` dispatcher.  Differences from the reference, which change
 // the schedule only: shapes, nats and dtypes are computed while recording (the reference evaluates them as
 // operations of the same graph, so an operation that depends on a tensor only through its shape may come later
-// there), and definitions such as nn.sigmoid are inlined (the reference evaluates a definition as one operation of
-// the enclosing term, with its own layers inside).
+// there).
+//
+// A definition (`Module::call`, e.g. nn.sigmoid) is ONE operation of the enclosing term whose body is a term of its
+// own, evaluated with its own layers when the operation's turn comes (interpreter.rs:61-74 `handle_definition`).
 //
 // `If` (core.rs `Operation::If`, interpreter.rs:86-107): the condition tensor is read with `to_bool`, the branch that
 // is taken is a term of its own, evaluated with the remaining operands.
@@ -29,7 +31,7 @@
 namespace cgh {
 
 struct Term : WireTable, OpRecorder {
-    enum Kind { OP, COPY, LOAD, IF };
+    enum Kind { OP, COPY, LOAD, IF, DEFINITION };
     struct Arg { // an operand: a wire, or a value that was known while recording
         int wire = -1;
         Value host;
@@ -37,10 +39,10 @@ struct Term : WireTable, OpRecorder {
     struct Operation {
         Kind kind = OP;
         Op op{TensorOp::Add};
-        std::string path;              // LOAD
-        std::vector<Arg> args;         // OP / IF: in the operation's own operand order; COPY: one wire
+        std::string path;              // LOAD, DEFINITION
+        std::vector<Arg> args;         // OP / IF / DEFINITION: in the operation's own operand order; COPY: one wire
         std::vector<int> targets;
-        std::shared_ptr<Term> then_branch, else_branch; // IF
+        std::shared_ptr<Term> then_branch, else_branch; // IF; DEFINITION: then_branch is the definition's term
     };
     struct Wire {
         Shape shape;
@@ -91,6 +93,8 @@ struct Term : WireTable, OpRecorder {
         auto sh = [&](size_t i) { return a[i].tensor.shape(); };
         auto dt = [&](size_t i) { return a[i].tensor.dtype(); };
         switch (op.op) {
+        case TensorOp::Probe: return {};
+        case TensorOp::Where: return {{sh(1), dt(1)}}; // [mask, x, y]: the type of the values, not of the mask
         case TensorOp::NatToU32: return {{Shape{}, CG_U32}};
         case TensorOp::ScalarF32: return {{Shape{}, CG_F32}};
         case TensorOp::ScalarU32: return {{Shape{}, CG_U32}};
@@ -139,7 +143,7 @@ struct Term : WireTable, OpRecorder {
             s.at(a[1].nat) = a[2].tensor.numel();
             return {{s, dt(0)}};
         }
-        default: return {{sh(0), dt(0)}}; // element-wise: the first operand's type
+        default: return {{sh(0), dt(0)}}; // element-wise maps and comparisons: the operands' common type
         }
     }
 
@@ -188,6 +192,52 @@ struct Term : WireTable, OpRecorder {
             o.args.push_back(std::move(a));
         }
         std::vector<std::pair<Shape, cg_dtype>> result_t;
+        auto branch = [&](auto &&fn) { return record_subterm(i, types, fn, &result_t); };
+        o.then_branch = branch(then_fn);
+        const std::vector<std::pair<Shape, cg_dtype>> then_t = result_t;
+        o.else_branch = branch(else_fn);
+        // both branches have the type of the operation (the reference's type checker rejects anything else)
+        if (then_t != result_t) throw InterpreterError("TypeError: the branches of If disagree in their result types");
+        const int id = (int)ops.size();
+        std::vector<Tensor> out;
+        for (const auto &t : result_t) {
+            const int w = new_wire(t.first, t.second, id);
+            o.targets.push_back(w);
+            out.emplace_back(this, w);
+        }
+        ops.push_back(std::move(o));
+        return out;
+    }
+    // `Module::call` (a Definition operation): `fn` is the definition's body, recorded as a term over sources typed
+    // like `args`.
+    template <class F> std::vector<Tensor> record_definition(Interpreter &i, const std::string &path, std::vector<Tensor> args, F &&fn) {
+        Operation o;
+        o.kind = DEFINITION;
+        o.path = path;
+        std::vector<std::pair<Shape, cg_dtype>> types;
+        for (Tensor &t : args) types.emplace_back(t.shape(), t.dtype());
+        for (Tensor &t : args) {
+            Arg a;
+            a.wire = wire_of(t);
+            o.args.push_back(std::move(a));
+        }
+        std::vector<std::pair<Shape, cg_dtype>> result_t;
+        o.then_branch = record_subterm(i, types, fn, &result_t);
+        const int id = (int)ops.size();
+        std::vector<Tensor> out;
+        for (const auto &t : result_t) {
+            const int w = new_wire(t.first, t.second, id);
+            o.targets.push_back(w);
+            out.emplace_back(this, w);
+        }
+        ops.push_back(std::move(o));
+        return out;
+    }
+    // a term of its own for a branch or a definition: `fn` runs over fresh sources while `i` records into the new term
+    template <class F>
+    static std::shared_ptr<Term> record_subterm(Interpreter &i, const std::vector<std::pair<Shape, cg_dtype>> &types, F &&fn,
+                                                std::vector<std::pair<Shape, cg_dtype>> *result_types_out) {
+        std::vector<std::pair<Shape, cg_dtype>> &result_t = *result_types_out;
         auto branch = [&](auto &&fn) {
             auto term = std::make_shared<Term>();
             std::vector<Tensor> src;
@@ -209,17 +259,7 @@ struct Term : WireTable, OpRecorder {
             }
             return term;
         };
-        o.then_branch = branch(then_fn);
-        o.else_branch = branch(else_fn);
-        const int id = (int)ops.size();
-        std::vector<Tensor> out;
-        for (const auto &t : result_t) {
-            const int w = new_wire(t.first, t.second, id);
-            o.targets.push_back(w);
-            out.emplace_back(this, w);
-        }
-        ops.push_back(std::move(o));
-        return out;
+        return branch(fn);
     }
     std::vector<int> results; // wires handed back by `run` (set by finish / record_if)
     void finish(std::vector<Tensor> outs) {
@@ -281,6 +321,14 @@ struct Term : WireTable, OpRecorder {
                 for (size_t k = 0; k < res.size(); k++) put(o.targets[k], std::move(res[k].tensor));
                 break;
             }
+            case DEFINITION: { // handle_definition: the definition's term, evaluated with the operation's operands
+                std::vector<Tensor> in;
+                for (Arg &a : o.args) in.push_back(take(a.wire));
+                std::vector<Tensor> res = o.then_branch->run(i, std::move(in), in_order);
+                if (res.size() != o.targets.size()) throw InterpreterError("ApplyError: wrong number of results");
+                for (size_t k = 0; k < res.size(); k++) put(o.targets[k], std::move(res[k]));
+                break;
+            }
             case IF: { // handle_if: to_bool of (a clone of) the condition, then the branch's own evaluation
                 Tensor cond = take(o.args[0].wire);
                 std::vector<Tensor> rest;
@@ -310,6 +358,12 @@ template <class F, class G>
 inline std::vector<Tensor> cond(I &i, Tensor c, F &&then_fn, G &&else_fn, std::vector<Tensor> args) {
     if (Term *t = dynamic_cast<Term *>(i.recorder)) return t->record_if(i, std::move(c), std::move(args), then_fn, else_fn);
     return i.backend.to_bool(c) ? then_fn(std::move(args)) : else_fn(std::move(args));
+}
+// `Module::call(builder, args)`: a Definition operation named `path` whose body is `fn`.  Run directly, the body's
+// operations are issued where the call stands, which is the order handle_definition gives them too.
+template <class F> inline std::vector<Tensor> definition(I &i, const std::string &path, F &&fn, std::vector<Tensor> args) {
+    if (Term *t = dynamic_cast<Term *>(i.recorder)) return t->record_definition(i, path, std::move(args), fn);
+    return fn(std::move(args));
 }
 } // namespace ops
 } // namespace cgh

@@ -12,6 +12,8 @@
 #pragma once
 
 #include <cmath>
+#include <cstdio>
+#include <cstdlib>
 #include <map>
 #include <string>
 #include <vector>
@@ -43,16 +45,18 @@ struct InterpreterError : std::runtime_error { // abstract_interpreter/types.rs:
 enum class TensorOp {
     Add, Sub, Mul, Div, Neg, Pow, LT, GT, GTE, LTE, EQ, Cos, Sin, Exp, Log, Floor, Round, Where,
     NatToU32, Cast, MatMul, ScalarF32, ScalarU32, Sum, Max, Argmax, TopK, Broadcast, Reshape, Transpose,
-    Slice, Concat, Arange, Index
+    Slice, Concat, Arange, Index, Probe
 };
 
 struct Op {
     TensorOp op;
     float f32 = 0.0f;   // payload of ScalarF32
     uint32_t u32 = 0;   // payload of ScalarU32
+    std::string label;  // payload of Probe
     Op(TensorOp o) : op(o) {}
     static Op scalar(float v) { Op o(TensorOp::ScalarF32); o.f32 = v; return o; }
     static Op scalar(uint32_t v) { Op o(TensorOp::ScalarU32); o.u32 = v; return o; }
+    static Op probe(std::string l) { Op o(TensorOp::Probe); o.label = std::move(l); return o; }
 };
 
 // Builds an argument / result list by MOVING its items (a braced list would copy,
@@ -177,6 +181,15 @@ inline std::vector<Value> tensor_op(Backend &b, const Op &op, std::vector<Value>
         Tensor x = to_tensor(args[0]), ix = to_tensor(args[2]);
         return vals(Value(b.index(std::move(x), to_nat(args[1]), std::move(ix))));
     }
+    case TensorOp::Probe: { // tensor_op.rs:121-136: a debugging aid with no results; silent unless CATGRAD_PROBE is set
+        if (std::getenv("CATGRAD_PROBE")) {
+            arity(args, 1);
+            Tensor x = to_tensor(args[0]);
+            std::printf("[probe:%s] %s\n", op.label.c_str(), b.format_tensor(x).c_str());
+            std::fflush(stdout);
+        }
+        return {};
+    }
     }
     throw InterpreterError("unknown tensor op");
 }
@@ -227,6 +240,10 @@ inline Tensor mul(I &i, Tensor x, Tensor y) { return i.run1(TensorOp::Mul, vals(
 inline Tensor div(I &i, Tensor x, Tensor y) { return i.run1(TensorOp::Div, vals(std::move(x), std::move(y))); }
 inline Tensor pow(I &i, Tensor x, Tensor y) { return i.run1(TensorOp::Pow, vals(std::move(x), std::move(y))); }
 inline Tensor lt(I &i, Tensor x, Tensor y) { return i.run1(TensorOp::LT, vals(std::move(x), std::move(y))); }
+inline Tensor lte(I &i, Tensor x, Tensor y) { return i.run1(TensorOp::LTE, vals(std::move(x), std::move(y))); }
+inline Tensor gte(I &i, Tensor x, Tensor y) { return i.run1(TensorOp::GTE, vals(std::move(x), std::move(y))); }
+// lang/ops.rs:241-249: the operand is borrowed (`&Var`), so the operation reads a clone; it has no result
+inline void probe(I &i, const std::string &label, const Tensor &x) { i.run(Op::probe(label), vals(Tensor(x))); }
 inline Tensor neg(I &i, Tensor x) { return i.run1(TensorOp::Neg, vals(std::move(x))); }
 inline Tensor exp(I &i, Tensor x) { return i.run1(TensorOp::Exp, vals(std::move(x))); }
 inline Tensor sin(I &i, Tensor x) { return i.run1(TensorOp::Sin, vals(std::move(x))); }

@@ -171,7 +171,7 @@ class LlmModel {
 // hidden.rs:103-132 shaped MLP: Linear(in, hidden) -> nn::Sigmoid -> Linear(hidden, out).
 inline Tensor hidden_mlp(Interpreter &i, size_t in_dim, size_t hidden, size_t out_dim, Tensor x) {
     x = nn::linear(i, in_dim, hidden, "mlp.l1", std::move(x));
-    x = nn::sigmoid(i, std::move(x));
+    x = nn::sigmoid_module(i, std::move(x));
     return nn::linear(i, hidden, out_dim, "mlp.l2", std::move(x));
 }
 

@@ -7,7 +7,7 @@
 #include <cmath>
 #include <limits>
 
-#include "interp.hpp"
+#include "graph.hpp"
 
 namespace cgh {
 namespace nn {
@@ -29,6 +29,22 @@ inline Tensor sigmoid(I &i, Tensor x) {
     Tensor e = exp(i, neg(i, std::move(x)));
     Tensor d = add(i, one, std::move(e)); // one.clone() feeds the division below
     return div(i, std::move(one), std::move(d));
+}
+
+// catgrad/src/stdlib/nn/mod.rs:36-47 with 13-33: `nn::Sigmoid.call(builder, [x])` is a Definition operation at path
+// nn.sigmoid whose body is `sigmoid` (interpreter.rs:61-74 evaluates the body as a term of its own).
+inline Tensor sigmoid_module(I &i, Tensor x) {
+    std::vector<Tensor> args;
+    args.push_back(std::move(x));
+    std::vector<Tensor> r = definition(
+        i, "nn.sigmoid",
+        [&](std::vector<Tensor> a) {
+            std::vector<Tensor> out;
+            out.push_back(sigmoid(i, std::move(a[0])));
+            return out;
+        },
+        std::move(args));
+    return std::move(r[0]);
 }
 
 // catgrad/src/stdlib/nn/mod.rs:143-148
@@ -127,6 +143,33 @@ inline Tensor repeat_interleave(I &i, size_t dim, size_t rep, Tensor x) {
     return reshape(i, sh, std::move(x));
 }
 inline Tensor repeat_kv(I &i, size_t rep, Tensor x) { return repeat_interleave(i, 1, rep, std::move(x)); }
+
+// catgrad-llm-models/src/helpers/tensors.rs:305-334: 1.0 where col <= row + diagonal (lower) / col >= row + diagonal (upper)
+inline Tensor tri_mask(I &i, size_t size, uint32_t diagonal, bool triu) {
+    Shape sh{size, size};
+    Tensor diag = broadcast(i, sh, lit(i, diagonal));
+    Tensor idx = arange(i, size);
+    Tensor row = reshape(i, Shape{size, 1}, idx);
+    Tensor col = reshape(i, Shape{1, size}, std::move(idx));
+    row = broadcast(i, sh, std::move(row));
+    col = broadcast(i, sh, std::move(col));
+    row = add(i, std::move(row), std::move(diag));
+    Tensor mask = triu ? gte(i, std::move(col), std::move(row)) : lte(i, std::move(col), std::move(row));
+    return cast(i, std::move(mask), CG_F32);
+}
+inline Tensor tril_mask(I &i, size_t size, uint32_t diagonal) { return tri_mask(i, size, diagonal, false); }
+
+// catgrad-llm-models/src/helpers/tensors.rs:337-351: cumulative sum along the last axis as a product with the
+// transposed lower-triangular mask
+inline Tensor cumsum(I &i, Tensor x) {
+    Shape sh = shape(x);
+    const size_t ldim = sh.back();
+    sh[sh.size() - 2] = ldim;
+    Tensor lower = tril_mask(i, ldim, 0);
+    lower = transpose(i, 0, 1, std::move(lower));
+    lower = broadcast(i, sh, std::move(lower));
+    return matmul(i, std::move(x), std::move(lower));
+}
 
 // catgrad-llm-models/src/helpers/tensors.rs:207-224
 inline Tensor causal_mask(I &i, size_t seq_len, size_t pos) {

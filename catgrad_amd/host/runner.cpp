@@ -29,6 +29,26 @@ template <class F> static int guarded(F &&f) {
     }
 }
 
+// Runs `body` over `inputs` under the session's schedule: directly (0), or recorded as a term first and evaluated in
+// the reference evaluator's layers (1) or in the order of recording (2).
+template <class F> static std::vector<Tensor> run_scheduled(Interpreter &i, std::vector<Tensor> inputs, F &&body) {
+    if (i.schedule == 0) return body(std::move(inputs));
+    Term term;
+    std::vector<Tensor> src;
+    for (Tensor &t : inputs) src.push_back(term.source(t.shape(), t.dtype()));
+    i.recorder = &term;
+    std::vector<Tensor> r;
+    try {
+        r = body(std::move(src));
+    } catch (...) {
+        i.recorder = nullptr;
+        throw;
+    }
+    i.recorder = nullptr;
+    term.finish(std::move(r));
+    return term.run(i, std::move(inputs), i.schedule == 2);
+}
+
 extern "C" {
 
 const char *cgm_last_error(void) { return g_err.c_str(); }
@@ -103,39 +123,69 @@ int cgm_set_schedule(cgm_session *s, int schedule) {
 int cgm_cond_kat(cgm_session *s, float x, float c, float *out) {
     return guarded([&] {
         Interpreter &i = *s->interp;
-        auto body = [&](Tensor tx, Tensor tc) {
-            Tensor keep = tx; // `x.clone()`: the term also returns x itself in the reference's test
+        std::vector<Tensor> in;
+        in.push_back(i.backend.ndarray_from_vec_f32(&x, 1, Shape{}));
+        in.push_back(i.backend.ndarray_from_vec_f32(&c, 1, Shape{}));
+        std::vector<Tensor> res = run_scheduled(i, std::move(in), [&](std::vector<Tensor> a) {
+            Tensor keep = a[0]; // `x.clone()`: the term also returns x itself in the reference's test
             (void)keep;
             return ops::cond(
-                i, std::move(tc),
-                [&](std::vector<Tensor> a) { return std::vector<Tensor>{ops::add(i, a[0], a[0])}; },
-                [&](std::vector<Tensor> a) { return std::vector<Tensor>{std::move(a[0])}; },
-                std::vector<Tensor>{std::move(tx)});
-        };
-        Tensor tx = i.backend.ndarray_from_vec_f32(&x, 1, Shape{}), tc = i.backend.ndarray_from_vec_f32(&c, 1, Shape{});
-        Tensor res;
-        if (i.schedule == 0) {
-            res = std::move(body(std::move(tx), std::move(tc))[0]);
-        } else {
-            Term term;
-            Tensor sx = term.source(Shape{}, CG_F32), sc = term.source(Shape{}, CG_F32);
-            i.recorder = &term;
-            std::vector<Tensor> r;
-            try {
-                r = body(std::move(sx), std::move(sc));
-            } catch (...) {
-                i.recorder = nullptr;
-                throw;
-            }
-            i.recorder = nullptr;
-            term.finish(std::move(r));
-            std::vector<Tensor> in;
-            in.push_back(std::move(tx));
-            in.push_back(std::move(tc));
-            res = std::move(term.run(i, std::move(in), i.schedule == 2)[0]);
-        }
-        std::vector<uint32_t> v = i.backend.to_vec_bits(std::move(res));
+                i, std::move(a[1]),
+                [&](std::vector<Tensor> b) { return std::vector<Tensor>{ops::add(i, b[0], b[0])}; },
+                [&](std::vector<Tensor> b) { return std::vector<Tensor>{std::move(b[0])}; },
+                std::vector<Tensor>{std::move(a[0])});
+        });
+        std::vector<uint32_t> v = i.backend.to_vec_bits(std::move(res[0]));
         memcpy(out, v.data(), 4);
+    });
+}
+
+int cgm_cond_mismatch(cgm_session *s) {
+    return guarded([&] {
+        Interpreter &i = *s->interp;
+        const float one = 1.0f;
+        std::vector<Tensor> in;
+        in.push_back(i.backend.ndarray_from_vec_f32(&one, 1, Shape{}));
+        in.push_back(i.backend.ndarray_from_vec_f32(&one, 1, Shape{}));
+        run_scheduled(i, std::move(in), [&](std::vector<Tensor> a) {
+            return ops::cond(
+                i, std::move(a[1]),
+                [&](std::vector<Tensor> b) { return std::vector<Tensor>{ops::cast(i, std::move(b[0]), CG_U32)}; },
+                [&](std::vector<Tensor> b) { return std::vector<Tensor>{std::move(b[0])}; },
+                std::vector<Tensor>{std::move(a[0])});
+        });
+    });
+}
+
+int cgm_helper(cgm_session *s, int which, const float *x, const size_t *dims, size_t rank, size_t a0, size_t a1,
+               const char *label, float *out, size_t out_cap, size_t *out_dims, size_t *out_rank) {
+    return guarded([&] {
+        Interpreter &i = *s->interp;
+        Shape shape(dims, dims + rank);
+        size_t n = 1;
+        for (size_t d : shape) n *= d;
+        std::vector<Tensor> in;
+        in.push_back(i.backend.ndarray_from_vec_f32(x, n, shape));
+        std::vector<Tensor> res = run_scheduled(i, std::move(in), [&](std::vector<Tensor> a) {
+            std::vector<Tensor> r;
+            switch (which) {
+            case 0: r.push_back(nn::repeat_kv(i, a0, std::move(a[0]))); break;
+            case 1: r.push_back(nn::repeat_interleave(i, a0, a1, std::move(a[0]))); break;
+            case 2: r.push_back(nn::cumsum(i, std::move(a[0]))); break;
+            case 3:
+                ops::probe(i, label ? label : "", a[0]);
+                r.push_back(std::move(a[0]));
+                break;
+            default: throw InterpreterError("unknown helper");
+            }
+            return r;
+        });
+        Shape rs = res[0].shape();
+        *out_rank = rs.size();
+        for (size_t d = 0; d < rs.size(); d++) out_dims[d] = rs[d];
+        std::vector<uint32_t> v = i.backend.to_vec_bits(std::move(res[0]));
+        if (v.size() > out_cap) throw InterpreterError("helper result larger than the caller's buffer");
+        memcpy(out, v.data(), v.size() * 4);
     });
 }
 
@@ -216,9 +266,14 @@ int cgm_forward_rows(cgm_session *s, const uint32_t *tokens, size_t B, size_t S,
 int cgm_mlp(cgm_session *s, const float *x, size_t rows, size_t in_dim, size_t hidden, size_t out_dim, float *y) {
     return guarded([&] {
         Interpreter &i = *s->interp;
-        Tensor t = i.backend.ndarray_from_vec_f32(x, rows * in_dim, Shape{1, rows, in_dim});
-        Tensor r = hidden_mlp(i, in_dim, hidden, out_dim, std::move(t));
-        std::vector<uint32_t> v = i.backend.to_vec_bits(std::move(r));
+        std::vector<Tensor> in;
+        in.push_back(i.backend.ndarray_from_vec_f32(x, rows * in_dim, Shape{1, rows, in_dim}));
+        std::vector<Tensor> r = run_scheduled(i, std::move(in), [&](std::vector<Tensor> a) {
+            std::vector<Tensor> o;
+            o.push_back(hidden_mlp(i, in_dim, hidden, out_dim, std::move(a[0])));
+            return o;
+        });
+        std::vector<uint32_t> v = i.backend.to_vec_bits(std::move(r[0]));
         memcpy(y, v.data(), v.size() * 4);
     });
 }

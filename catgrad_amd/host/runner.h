@@ -39,6 +39,18 @@ int cgm_set_schedule(cgm_session *s, int schedule);
  * the result's value. */
 int cgm_cond_kat(cgm_session *s, float x, float c, float *out);
 
+/* A term whose If branches disagree in their result types (f32 against u32): under schedules 1 and 2 recording it
+ * fails with a TypeError, as the reference's type checker would; returns nonzero then. */
+int cgm_cond_mismatch(cgm_session *s);
+
+/* One helper composition of catgrad-llm-models/src/helpers/tensors.rs on an f32 tensor x[dims], under the session's
+ * schedule: which 0 = repeat_kv(rep = a0, x); 1 = repeat_interleave(dim = a0, rep = a1, x); 2 = cumsum(x) along the
+ * last axis; 3 = probe(label, x) (catgrad/src/interpreter/tensor_op.rs:121-136: prints "[probe:label] ..." to stdout
+ * when CATGRAD_PROBE is set) and hands x back.  out receives the result (at most out_cap elements), out_dims /
+ * out_rank its shape (out_dims has room for 8 extents). */
+int cgm_helper(cgm_session *s, int which, const float *x, const size_t *dims, size_t rank, size_t a0, size_t a1,
+               const char *label, float *out, size_t out_cap, size_t *out_dims, size_t *out_rank);
+
 /* Prefill + `steps` greedy decode runs.  out_tokens: (steps+1) x B ids.  stats:
  * [prefill_s, decode_s, backend calls in prefill, backend calls in decode]. */
 int cgm_generate(cgm_session *s, const uint32_t *prompt, size_t B, size_t S, size_t steps, size_t max_positions,

@@ -38,6 +38,8 @@ def _host():
             "cgm_set_config": (C.c_int, [P, C.c_int] + [SZ] * 7 + [C.c_float, C.c_float, C.c_int]),
             "cgm_set_schedule": (C.c_int, [P, C.c_int]),
             "cgm_cond_kat": (C.c_int, [P, C.c_float, C.c_float, C.POINTER(C.c_float)]),
+            "cgm_cond_mismatch": (C.c_int, [P]),
+            "cgm_helper": (C.c_int, [P, C.c_int, P, SZP, SZ, SZ, SZ, C.c_char_p, P, SZ, SZP, SZP]),
             "cgm_generate": (C.c_int, [P, P, SZ, SZ, SZ, SZ, P, C.POINTER(C.c_double)]),
             "cgm_generate_with_logits": (C.c_int, [P, P, SZ, SZ, SZ, SZ, P, C.POINTER(C.c_double), P]),
             "cgm_forward": (C.c_int, [P, P, SZ, SZ, SZ, P, P]),
@@ -204,6 +206,26 @@ class Session:
         out = C.c_float()
         self._check(self._lib.cgm_cond_kat(self._s, x, c, C.byref(out)))
         return float(out.value)
+
+    def cond_mismatch(self):
+        """Records a term whose If branches disagree in their result types; raises under schedules 1 and 2."""
+        self._check(self._lib.cgm_cond_mismatch(self._s))
+
+    HELPERS = {"repeat_kv": 0, "repeat_interleave": 1, "cumsum": 2, "probe": 3}
+
+    def helper(self, which: str, x: np.ndarray, a0: int = 0, a1: int = 0, label: str = "", out_cap: int | None = None) -> np.ndarray:
+        """One helper composition of catgrad-llm-models/src/helpers/tensors.rs on an f32 tensor, through the
+        interpreter mirror and the backend, under the session's schedule: repeat_kv(rep=a0), repeat_interleave(dim=a0,
+        rep=a1), cumsum (last axis), probe(label) (prints when CATGRAD_PROBE is set; hands x back)."""
+        x = np.ascontiguousarray(x, dtype=np.float32)
+        dims = (C.c_size_t * max(x.ndim, 1))(*x.shape)
+        cap = out_cap or max(x.size * max(a0, a1, 1), 1)
+        out = np.zeros(cap, dtype=np.float32)
+        od, orank = (C.c_size_t * 8)(), C.c_size_t()
+        self._check(self._lib.cgm_helper(self._s, self.HELPERS[which], x.ctypes.data_as(C.c_void_p), dims, x.ndim, a0, a1,
+                                         label.encode(), out.ctypes.data_as(C.c_void_p), cap, od, C.byref(orank)))
+        shape = tuple(od[i] for i in range(orank.value))
+        return out[: int(np.prod(shape, dtype=np.int64))].reshape(shape)
 
     def generate(self, prompt: np.ndarray, steps: int, max_positions: int | None = None, want_logits: bool = False):
         """Prefill + `steps` greedy decode runs.  Returns (tokens [(steps+1), B], stats dict); with `want_logits`

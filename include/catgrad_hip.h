@@ -139,7 +139,8 @@ typedef enum cg_kernel_class {
     CG_K_REDUCE = 4,      /* work = bytes of the input + output */
     CG_K_GATHER = 5,      /* work = bytes gathered + written */
     CG_K_ATTENTION = 6,   /* one-pass causal attention of a prefill; work = flop of the visible scores and sums */
-    CG_K_CLASSES = 7
+    CG_K_PACK = 7,        /* an operand narrowed to 2- / 1-byte patterns in memory for a product; work = bytes read + written */
+    CG_K_CLASSES = 8
 } cg_kernel_class;
 int cg_profile_enable(cg_backend *b, cg_kernel_class cls, unsigned sample_every);
 /* Element-wise results are computed lazily (fused into their consumer); cg_realize queues
@@ -221,7 +222,11 @@ int cg_argmax(cg_backend *b, cg_tensor *x, cg_tensor **out);
  * (a hipStream_t; null = the default stream) of `device`; the call allocates nothing, frees nothing and does not
  * wait.  Per-segment partial results go to a fixed 128 KiB array that each GPU holds until the process ends:
  * rows * min(256, ceil(n / 1024)) must not exceed 16384 (and rows 65535), else CG_ERR_UNSUPPORTED.  All calls on one
- * GPU share that array: calls that overlap in time on one GPU race; order them on one stream or with events. */
+ * GPU share that array: calls that overlap in time on one GPU race; order them on one stream or with events.
+ * Precondition: cg_noalloc_setup(device) — or cg_backend_create on that device, which includes it — has returned
+ * CG_OK in this process; otherwise CG_ERR_ARG (the call itself never resolves the array's address: that would load
+ * code, which is not allowed under stream capture).  The calling thread's current device is left as it was. */
+int cg_noalloc_setup(int device);
 int cg_argmax_rows_noalloc(int device, cg_dtype dtype, const void *x, size_t rows, size_t n, uint32_t *out,
                            void *stream);
 /* `Backend::topk` (mod.rs:86; ndarray.rs:436-446,696-721). */

@@ -1159,6 +1159,7 @@ int cg_argmax(cg_backend *, cg_tensor *x, cg_tensor **out) {
 
 // The same rule on a dense [rows, n] array in plain memory (the checker's side of the entry point that the GPU
 // library offers to callers that cannot allocate; `device` and `stream` mean nothing here).
+int cg_noalloc_setup(int) { return CG_OK; } // nothing to set up in plain memory
 int cg_argmax_rows_noalloc(int, cg_dtype dtype, const void *x, size_t rows, size_t n, uint32_t *out, void *) {
     if (n == 0) return fail(CG_ERR_SHAPE, "argmax: called `Option::unwrap()` on a `None` value (empty axis)");
     if (rows == 0) return CG_OK;

@@ -2,7 +2,6 @@ import os
 import sys
 
 import pytest
-import torch  # noqa: F401  loaded before any HIP library so that the process holds one HIP runtime (torch's)
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:

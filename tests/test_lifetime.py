@@ -7,7 +7,6 @@ import ctypes as C
 
 import numpy as np
 import pytest
-import torch  # noqa: F401  before the HIP library is loaded (one HIP runtime per process)
 
 from catgrad_amd import _abi as A
 
@@ -58,6 +57,21 @@ def _destroy_then_release(lib):
     lib.cg_backend_destroy(b2)                      # and the ordinary order still does
 
 
+def _calls_after_destroy_fail(lib):
+    """While surviving handles keep a destroyed backend's memory alive, calls on it are refused, not undefined."""
+    b, handles = _survivors(lib)
+    lib.cg_backend_destroy(b)
+    host = np.zeros(4096, np.float32)
+    assert lib.cg_to_host(b, handles[0], host.ctypes.data_as(C.c_void_p), 4096) == A.ERR_ARG
+    assert "cg_backend_destroy" in lib.cg_last_error().decode()
+    out = C.c_void_p()
+    lib.cg_tensor_retain(handles[0])
+    assert lib.cg_unary(b, A.NEG, handles[0], C.byref(out)) == A.ERR_ARG   # (the consumed reference is dropped)
+    assert lib.cg_sync(b) == A.ERR_ARG
+    for h in handles:
+        lib.cg_tensor_release(h)
+
+
 def test_release_after_destroy_oracle():
     from oracle_loader import oracle_library
 
@@ -69,3 +83,10 @@ def test_release_after_destroy_hip():
     from catgrad_amd.backend import load_hip_library
 
     _destroy_then_release(load_hip_library())
+
+
+@pytest.mark.gpu
+def test_calls_on_a_destroyed_backend_fail_hip():
+    from catgrad_amd.backend import load_hip_library
+
+    _calls_after_destroy_fail(load_hip_library())
