@@ -169,6 +169,164 @@ def sample_prompt(cfg, B, S, seed):
     return np.random.default_rng(seed + 1).integers(0, cfg.vocab_size, size=(B, S), dtype=np.uint32)
 
 
+CONFIGS = {
+    5: (4, 2048, 256, "Llama-3.2-1B-shape decoder (hidden 2048, 16 layers, 32/8 heads, MLP 8192, vocab 128256, "
+                      "rope theta 500000, tied lm_head)"),
+    4: (1, 1024, 128, "Qwen3-0.6B-shape decoder (hidden 1024, 28 layers, 16/8 heads of 128, QK-norm, MLP 3072, "
+                      "vocab 151936, tied lm_head)"),
+    3: (1, 512, 16, "SmolLM2-135M-shape decoder (hidden 576, 30 layers, 9/3 heads, MLP 1536, vocab 49152, "
+                    "tied lm_head)"),
+}
+
+
+def measure(config, steps, warmup, batch=None, prefill=None, decode=None, seed=0):
+    """One BASELINE configuration through HipBackend: `warmup` untimed passes, then `steps` timed passes of prefill +
+    greedy decode.  Returns (result dict, the open session, config, params, batch)."""
+    import torch
+
+    from catgrad_amd import _abi as A
+    from catgrad_amd.runner import LLAMA_3_2_1B, QWEN3_0_6B, SMOLLM2_135M, Session, random_params
+
+    cfg = {5: LLAMA_3_2_1B, 4: QWEN3_0_6B, 3: SMOLLM2_135M}[config]
+    dB, dS, dT, cfg_name = CONFIGS[config]
+    B = batch if batch is not None else dB
+    S = prefill if prefill is not None else dS
+    T = decode if decode is not None else dT
+    params = list(random_params(cfg, seed))
+    sess = Session()
+    t_up = time.perf_counter()
+    sess.load_model(cfg, params=params)
+    sess.sync()
+    t_up = time.perf_counter() - t_up
+    weight_bytes = sum(int(w.size) * 4 for _, w in params)
+    prompt = np.random.default_rng(seed).integers(0, cfg.vocab_size, size=(B, S), dtype=np.uint32)
+
+    for _ in range(warmup):
+        sess.generate(prompt, steps=T, max_positions=S + T)
+    sess.profile_enable(A.K_GEMM_MFMA, 1)
+    sess.profile_enable(A.K_GEMM_SKINNY, 8)
+    sess.profile_enable(A.K_ATTENTION, 1)
+    sess.profile_read(A.K_GEMM_MFMA, reset=True)
+    sess.profile_read(A.K_GEMM_SKINNY, reset=True)
+    sess.profile_read(A.K_ATTENTION, reset=True)
+
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    pp_s = tg_s = 0.0
+    calls = (0, 0)
+    tokens = None
+    for _ in range(steps):
+        tokens, st = sess.generate(prompt, steps=T, max_positions=S + T)
+        pp_s += st["prefill_s"]
+        tg_s += st["decode_s"]
+        calls = (st["prefill_calls"], st["decode_calls"])
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+
+    n_m, ms_m, flop_m = sess.profile_read(A.K_GEMM_MFMA)
+    n_s, ms_s, bytes_s = sess.profile_read(A.K_GEMM_SKINNY)
+    n_a, ms_a, flop_a = sess.profile_read(A.K_ATTENTION)
+    sess.profile_enable(A.K_GEMM_MFMA, 0)
+    sess.profile_enable(A.K_GEMM_SKINNY, 0)
+    sess.profile_enable(A.K_ATTENTION, 0)
+    attn_rate = flop_a / (ms_a * 1e-3) if ms_a else 0.0
+    mfma_rate = flop_m / (ms_m * 1e-3) if ms_m else 0.0
+    skinny_rate = bytes_s / (ms_s * 1e-3) if ms_s else 0.0
+
+    K = steps
+    total_tokens = K * B * (S + T)
+    # algorithmic bytes of a decode step: the matmul weights (lm_head included) once, plus K and V
+    # of every layer at the mean cache length of the decode phase
+    hd = cfg.head_dim or cfg.hidden_size // cfg.num_attention_heads
+    weight_elems = cfg.num_hidden_layers * (
+        2 * cfg.hidden_size * cfg.num_attention_heads * hd + 2 * cfg.hidden_size * cfg.num_key_value_heads * hd
+        + 3 * cfg.hidden_size * cfg.intermediate_size) + cfg.vocab_size * cfg.hidden_size
+    kv_elems = 2 * cfg.num_hidden_layers * B * cfg.num_key_value_heads * (S + T / 2.0) * hd
+    step_bytes = int(4 * (weight_elems + kv_elems))
+    step_rate = step_bytes / (tg_s / K / T) if T and tg_s else 0.0
+    # algorithmic flop of the prefill: every linear layer over all positions (lm_head included) + dense attention
+    prefill_flop = 2.0 * B * S * weight_elems + cfg.num_hidden_layers * 4.0 * B * cfg.num_attention_heads * S * S * hd
+    result = {
+        "metric": "tok/s prefill+decode, Llama-3.2-1B-shape f32; % HBM & MFMA roofline",
+        "value": round(total_tokens / (pp_s + tg_s), 2),
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": K,
+        "warmup": warmup,
+        "ms_per_step": round(wall / K * 1e3, 3),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{cfg_name}, random-init f32, batch {B}, prefill {S} random tokens, "
+                        f"{T} greedy decode steps with KV cache",
+            "baseline_config": config,
+            "global_batch": B, "seq_len": S, "decode_steps": T, "parallelism": "single GPU",
+        },
+        "prefill_tok_s": round(K * B * S / pp_s, 2),
+        "decode_tok_s": round(K * B * T / tg_s, 2),
+        "prefill_ms": round(pp_s / K * 1e3, 3),
+        "decode_ms_per_step": round(tg_s / K / T * 1e3, 4),
+        # the whole prefill against the matrix peak: algorithmic flop (all linear layers + dense attention) / prefill time
+        "prefill_flop": prefill_flop,
+        "prefill_mfma_frac": round(prefill_flop / (pp_s / K) / MFMA_F32_PEAK, 4),
+        "backend_calls": {"prefill": calls[0], "per_decode_step": round(calls[1] / max(T, 1), 1)},
+        "backend": sess.backend_name,
+        "roofline": {
+            "kernel": "mfma_gemm_kernel (f32 v_mfma_f32_32x32x2; 128x128x32 tiles, two workgroups per compute unit; 128x64 and "
+                      "split-k variants for products that do not fill the device)",
+            "bound": "mfma", "achieved": round(mfma_rate / 1e12, 3), "peak": MFMA_F32_PEAK / 1e12, "unit": "TFLOP/s",
+            "frac": round(mfma_rate / MFMA_F32_PEAK, 4),
+            # from the committed rocprofv3 counter summary of this very workload (null for any other)
+            "traffic": profiled_traffic() if (config, B, S) == (5, 4, 2048) else None,
+            "traffic_source": "profiles/mfma_gemm_llama1b_prefill_pmc.txt" if (config, B, S) == (5, 4, 2048) else None,
+            "launches_timed": n_m, "avg_launch_ms": round(ms_m / max(n_m, 1), 4),
+            "flop_per_launch_avg": flop_m / max(n_m, 1),
+        },
+        # the one-pass causal attention of the prefill (q.K^T, soft-max, p.V): flop of the visible half only
+        "prefill_attention": {
+            "kernel": "prefill_attention_kernel (f32 v_mfma_f32_32x32x2, 128 query rows x 64 keys per step)",
+            "bound": "mfma", "achieved": round(attn_rate / 1e12, 3), "peak": MFMA_F32_PEAK / 1e12, "unit": "TFLOP/s",
+            "frac": round(attn_rate / MFMA_F32_PEAK, 4), "launches_timed": n_a,
+            "avg_launch_ms": round(ms_a / max(n_a, 1), 4),
+        },
+        "decode_roofline": {
+            "scope": "one decode step, all kernels: every weight matrix and the KV cache are read once",
+            "bound": "hbm", "bytes_per_step": step_bytes, "achieved": round(step_rate / 1e9, 2), "peak": HBM_PEAK / 1e9,
+            "unit": "GB/s", "frac": round(step_rate / HBM_PEAK, 4),
+            "skinny_gemm_kernels": {
+                "kernels": "skinny_kt_wide / skinny_kt_mfma_xreg / skinny_kt_narrow / skinny_nn (M <= 8)",
+                "achieved": round(skinny_rate / 1e9, 2), "unit": "GB/s", "frac": round(skinny_rate / HBM_PEAK, 4),
+                "launches_timed": n_s, "avg_launch_us": round(ms_s / max(n_s, 1) * 1e3, 3),
+            },
+        },
+        # the first decoded tokens of the timed run, for eyeballing across builds; what checks tokens is the CPU sample
+        # below (cpu_baseline.tokens_equal_gpu) and the full-size parity tests (tests/test_hip_config5.py)
+        "first_tokens": tokens[:2].tolist() if tokens is not None else None,
+        # not part of `value`: the one-off upload of the weights from pageable host memory through the
+        # backend's pinned staging buffers (the PCIe-inclusive cost of a cold start)
+        "weights_upload": {"bytes": weight_bytes, "seconds": round(t_up, 3), "GB_per_s": round(weight_bytes / t_up / 1e9, 2)},
+    }
+    return result, sess, cfg, params, B
+
+
+def other_config_line(config, steps=2, warmup=1):
+    """BASELINE configs 3 and 4 beside the headline line: the same measurement in a few seconds, the figures that
+    matter for them (prefill against the matrix peak, decode step against HBM) only."""
+    r, sess, _, _, _ = measure(config, steps, warmup)
+    sess.close()
+    return {
+        "workload": r["config"]["workload"], "steps": steps, "warmup": warmup,
+        "tok_s": r["value"], "prefill_ms": r["prefill_ms"], "prefill_tok_s": r["prefill_tok_s"],
+        "decode_ms_per_step": r["decode_ms_per_step"], "decode_tok_s": r["decode_tok_s"],
+        "prefill_mfma_frac": r["prefill_mfma_frac"], "gemm_kernel_mfma_frac": r["roofline"]["frac"],
+        "prefill_attention_mfma_frac": r["prefill_attention"]["frac"], "decode_hbm_frac": r["decode_roofline"]["frac"],
+        "backend_calls_per_decode_step": r["backend_calls"]["per_decode_step"], "first_tokens": r["first_tokens"],
+    }
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -184,6 +342,8 @@ def main():
     ap.add_argument("--seed", type=int, default=0)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-micro", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true",
+                    help="skip the short runs of BASELINE configs 3 and 4 that the default line carries as `other_configs`")
     ap.add_argument("--cpu-sample", type=int, nargs=3, default=None, metavar=("BATCH", "PREFILL", "DECODE"),
                     help="the CPU baseline's sample (default: the measured batch, prefill 8, 1 decode step)")
     ap.add_argument("--micro-only", action="store_true", help="only the op micro-benchmarks (one JSON line of their own)")
@@ -214,141 +374,19 @@ def main():
 
     import torch  # device-wide synchronisation around the timed region
 
-    from catgrad_amd import _abi as A
-    from catgrad_amd.runner import LLAMA_3_2_1B, QWEN3_0_6B, SMOLLM2_135M, Session, random_params
-
     if not torch.cuda.is_available():
         print("bench.py: no GPU visible; HipBackend has no CPU fallback.", file=sys.stderr)
         sys.exit(1)
 
-    cfg, dB, dS, dT, cfg_name = {
-        5: (LLAMA_3_2_1B, 4, 2048, 256, "Llama-3.2-1B-shape decoder (hidden 2048, 16 layers, 32/8 heads, MLP 8192, vocab 128256, "
-                                        "rope theta 500000, tied lm_head)"),
-        4: (QWEN3_0_6B, 1, 1024, 128, "Qwen3-0.6B-shape decoder (hidden 1024, 28 layers, 16/8 heads of 128, QK-norm, MLP 3072, "
-                                      "vocab 151936, tied lm_head)"),
-        3: (SMOLLM2_135M, 1, 512, 16, "SmolLM2-135M-shape decoder (hidden 576, 30 layers, 9/3 heads, MLP 1536, vocab 49152, "
-                                      "tied lm_head)"),
-    }[args.config]
-    B = args.batch if args.batch is not None else dB
-    S = args.prefill if args.prefill is not None else dS
-    T = args.decode if args.decode is not None else dT
-    params = list(random_params(cfg, args.seed))
-    sess = Session()
-    t_up = time.perf_counter()
-    sess.load_model(cfg, params=params)
-    sess.sync()
-    t_up = time.perf_counter() - t_up
-    weight_bytes = sum(int(w.size) * 4 for _, w in params)
-    prompt = np.random.default_rng(args.seed).integers(0, cfg.vocab_size, size=(B, S), dtype=np.uint32)
-
-    for _ in range(args.warmup):
-        sess.generate(prompt, steps=T, max_positions=S + T)
-    sess.profile_enable(A.K_GEMM_MFMA, 1)
-    sess.profile_enable(A.K_GEMM_SKINNY, 8)
-    sess.profile_enable(A.K_ATTENTION, 1)
-    sess.profile_read(A.K_GEMM_MFMA, reset=True)
-    sess.profile_read(A.K_GEMM_SKINNY, reset=True)
-    sess.profile_read(A.K_ATTENTION, reset=True)
-
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    pp_s = tg_s = 0.0
-    calls = (0, 0)
-    tokens = None
-    for _ in range(args.steps):
-        tokens, st = sess.generate(prompt, steps=T, max_positions=S + T)
-        pp_s += st["prefill_s"]
-        tg_s += st["decode_s"]
-        calls = (st["prefill_calls"], st["decode_calls"])
-    torch.cuda.synchronize()
-    wall = time.perf_counter() - t0
-
-    n_m, ms_m, flop_m = sess.profile_read(A.K_GEMM_MFMA)
-    n_s, ms_s, bytes_s = sess.profile_read(A.K_GEMM_SKINNY)
-    n_a, ms_a, flop_a = sess.profile_read(A.K_ATTENTION)
-    sess.profile_enable(A.K_GEMM_MFMA, 0)
-    sess.profile_enable(A.K_GEMM_SKINNY, 0)
-    sess.profile_enable(A.K_ATTENTION, 0)
-    attn_rate = flop_a / (ms_a * 1e-3) if ms_a else 0.0
-    mfma_rate = flop_m / (ms_m * 1e-3) if ms_m else 0.0
-    skinny_rate = bytes_s / (ms_s * 1e-3) if ms_s else 0.0
-
-    K = args.steps
-    total_tokens = K * B * (S + T)
-    # algorithmic bytes of a decode step: the matmul weights (lm_head included) once, plus K and V
-    # of every layer at the mean cache length of the decode phase
-    hd = cfg.head_dim or cfg.hidden_size // cfg.num_attention_heads
-    weight_elems = cfg.num_hidden_layers * (
-        2 * cfg.hidden_size * cfg.num_attention_heads * hd + 2 * cfg.hidden_size * cfg.num_key_value_heads * hd
-        + 3 * cfg.hidden_size * cfg.intermediate_size) + cfg.vocab_size * cfg.hidden_size
-    kv_elems = 2 * cfg.num_hidden_layers * B * cfg.num_key_value_heads * (S + T / 2.0) * hd
-    step_bytes = int(4 * (weight_elems + kv_elems))
-    step_rate = step_bytes / (tg_s / K / T) if T and tg_s else 0.0
-    result = {
-        "metric": "tok/s prefill+decode, Llama-3.2-1B-shape f32; % HBM & MFMA roofline",
-        "value": round(total_tokens / (pp_s + tg_s), 2),
-        "unit": "tok/s",
-        "n_gpus": 1,
-        "steps": K,
-        "warmup": args.warmup,
-        "ms_per_step": round(wall / K * 1e3, 3),
-        "higher_is_better": True,
-        "scaling": "weak",
-        "vs_baseline": None,
-        "dtype": "f32",
-        "data": "synthetic",
-        "config": {
-            "workload": f"{cfg_name}, random-init f32, batch {B}, prefill {S} random tokens, "
-                        f"{T} greedy decode steps with KV cache",
-            "baseline_config": args.config,
-            "global_batch": B, "seq_len": S, "decode_steps": T, "parallelism": "single GPU",
-        },
-        "prefill_tok_s": round(K * B * S / pp_s, 2),
-        "decode_tok_s": round(K * B * T / tg_s, 2),
-        "prefill_ms": round(pp_s / K * 1e3, 3),
-        "decode_ms_per_step": round(tg_s / K / T * 1e3, 4),
-        "backend_calls": {"prefill": calls[0], "per_decode_step": round(calls[1] / max(T, 1), 1)},
-        "backend": sess.backend_name,
-        "roofline": {
-            "kernel": "mfma_gemm_kernel (f32 v_mfma_f32_32x32x2; 128x128x32 tiles, two workgroups per compute unit; 128x64 for small products)",
-            "bound": "mfma", "achieved": round(mfma_rate / 1e12, 3), "peak": MFMA_F32_PEAK / 1e12, "unit": "TFLOP/s",
-            "frac": round(mfma_rate / MFMA_F32_PEAK, 4),
-            # from the committed rocprofv3 counter summary of this very workload (null for any other)
-            "traffic": profiled_traffic() if (args.config, B, S) == (5, 4, 2048) else None,
-            "traffic_source": "profiles/mfma_gemm_llama1b_prefill_pmc.txt" if (args.config, B, S) == (5, 4, 2048) else None,
-            "launches_timed": n_m, "avg_launch_ms": round(ms_m / max(n_m, 1), 4),
-            "flop_per_launch_avg": flop_m / max(n_m, 1),
-        },
-        # the one-pass causal attention of the prefill (q.K^T, soft-max, p.V): flop of the visible half only
-        "prefill_attention": {
-            "kernel": "prefill_attention_kernel (f32 v_mfma_f32_32x32x2, 128 query rows x 64 keys per step)",
-            "bound": "mfma", "achieved": round(attn_rate / 1e12, 3), "peak": MFMA_F32_PEAK / 1e12, "unit": "TFLOP/s",
-            "frac": round(attn_rate / MFMA_F32_PEAK, 4), "launches_timed": n_a,
-            "avg_launch_ms": round(ms_a / max(n_a, 1), 4),
-        },
-        "decode_roofline": {
-            "scope": "one decode step, all kernels: every weight matrix and the KV cache are read once",
-            "bound": "hbm", "bytes_per_step": step_bytes, "achieved": round(step_rate / 1e9, 2), "peak": HBM_PEAK / 1e9,
-            "unit": "GB/s", "frac": round(step_rate / HBM_PEAK, 4),
-            "skinny_gemm_kernels": {
-                "kernels": "skinny_kt_wide / skinny_kt_mfma_xreg / skinny_kt_narrow / skinny_nn (M <= 8)",
-                "achieved": round(skinny_rate / 1e9, 2), "unit": "GB/s", "frac": round(skinny_rate / HBM_PEAK, 4),
-                "launches_timed": n_s, "avg_launch_us": round(ms_s / max(n_s, 1) * 1e3, 3),
-            },
-        },
-        # the first decoded tokens of the timed run, for eyeballing across builds; what checks tokens is the CPU sample
-        # below (cpu_baseline.tokens_equal_gpu) and the full-size parity tests (tests/test_hip_config5.py)
-        "first_tokens": tokens[:2].tolist() if tokens is not None else None,
-        # not part of `value`: the one-off upload of the weights from pageable host memory through the
-        # backend's pinned staging buffers (the PCIe-inclusive cost of a cold start)
-        "weights_upload": {"bytes": weight_bytes, "seconds": round(t_up, 3), "GB_per_s": round(weight_bytes / t_up / 1e9, 2)},
-    }
+    result, sess, cfg, params, B = measure(args.config, args.steps, args.warmup, args.batch, args.prefill, args.decode, args.seed)
     cpu_sample = args.cpu_sample or [B, 8, 1]
     gpu_sample_tokens = None
     if not args.no_cpu_baseline:   # the CPU sample's prompt through the GPU path too: its tokens are compared below
         gpu_sample_tokens, _ = sess.generate(sample_prompt(cfg, cpu_sample[0], cpu_sample[1], args.seed), steps=cpu_sample[2],
                                              max_positions=cpu_sample[1] + cpu_sample[2])
     sess.close()
+    if args.config == 5 and not args.no_other_configs:
+        result["other_configs"] = {f"config{c}": other_config_line(c) for c in (3, 4)}
     if not args.no_micro:
         result["micro"] = micro_bench()
     if not args.no_cpu_baseline:

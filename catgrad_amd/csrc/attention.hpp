@@ -511,6 +511,270 @@ __global__ __launch_bounds__(kRowBlock) void decode_attention_row_kernel(const A
     }
 }
 
+// The same attention with a workgroup of 1024 threads per (batch entry, KV head) x SEGMENT of the cached positions,
+// all of the group's query rows together: every byte of K and V crosses the path from L2 into a compute unit once
+// (one workgroup per query row pulls K through it once per row and per half of head_dim: six times the traffic, and
+// that path, 25 bytes a clock per unit, is what bounds a launch of this size).  With 256 / (batch entries x KV heads)
+// segments a launch puts one workgroup on every compute unit, each with T / segments positions: 134 KB of K and V at
+// the 1B shape's T = 2100, in flight at once (PASSES x 1024 / LPT positions per trip, K and V of a trip in 2 x PASSES
+// sixteen-byte loads per lane).  A segment leaves its rows' maximum, sum and un-normalised weighted sum of V, as the
+// chunked kernel does; decode_attention_combine_kernel — or the load of the product that reads the result, see
+// AttnPartials — merges the segments.
+// LOOP: several trips, the next always asked for before the current one is used; else one trip covers the segment and
+// the soft-max program's other leaves are asked for before K.  MM: most query rows per KV head (4 or 8).
+constexpr int kSegBlock = 1024;
+constexpr int kSegMaxChunk = 2048; // most positions per workgroup: their scores wait in LDS, MM x 8 KiB
+constexpr size_t seg_lds_bytes(int mm, int hd, uint32_t chunk) {
+    return ((size_t)mm * ((chunk + 63) / 64 * 64) + (size_t)(kSegBlock / 64) * mm * hd) * sizeof(float);
+}
+template <class P, int LPT, int MM, int PASSES, bool LOOP>
+__global__ __launch_bounds__(kSegBlock) void decode_attention_seg_kernel(const AttnArgs g, const FusedArgs a) {
+    constexpr int HD = LPT * 4;
+    constexpr int TPB = kSegBlock / LPT; // positions per pass
+    constexpr int SPAN = TPB * PASSES;    // positions per trip to memory
+    constexpr int WAVES = kSegBlock / 64;
+    constexpr int IPL = LOOP ? 1 : (SPAN + 63) / 64; // positions per lane in the soft-max phase whose leaves wait in registers
+    constexpr int ri0 = reduce_index<P>(0), ri1 = reduce_index<P>(1);
+    constexpr int src0 = P::code[ri0][1], src1 = P::code[ri1][1];
+    static_assert((P::code[ri0][0] & ~kInstrU32) == kRowMax && (P::code[ri1][0] & ~kInstrU32) == kRowSum,
+                  "a soft-max: row maximum, then row sum");
+    extern __shared__ float seg_lds[];
+    const uint32_t cap = (g.chunk + 63) / 64 * 64;
+    float *sc = seg_lds;              // [MM][cap]: scores, then un-normalised weights
+    float *red = seg_lds + MM * cap;  // [WAVES][MM * HD]
+    const uint32_t tid = threadIdx.x, lane = tid % 64, wave = tid / 64;
+    const uint32_t split = blockIdx.x, b = blockIdx.y;
+    const uint32_t t0 = split * g.chunk, n = min(g.T, t0 + g.chunk) - t0; // (the host makes no empty segment)
+    int64_t oq = 0, ok = 0, ov = 0, op = 0;
+    {
+        uint32_t bb = b;
+        // (every axis slot is visited, so that the fields are read from the argument block at once instead of one
+        // dependent scalar load after the other)
+#pragma unroll
+        for (uint32_t d = 0; d < (uint32_t)kMaxBatchAxes; d++) {
+            if (d >= g.nb) break;
+            const uint32_t q = fastdiv(bb, g.bdiv[d]);
+            const int64_t i = (int64_t)(bb - q * g.bd[d]);
+            bb = q;
+            oq += i * g.q_bs[d];
+            ok += i * g.k_bs[d];
+            ov += i * g.v_bs[d];
+            op += i * g.p_bs[d];
+        }
+    }
+    const uint32_t l = tid % LPT, sub = tid / LPT;
+    const uint32_t *kbase = g.Kc + ok + (int64_t)t0 * g.k_st + l * 4;
+    const uint32_t *vbase = g.V + ov + (int64_t)t0 * g.v_st + l * 4;
+    const int64_t k_step = (int64_t)TPB * g.k_st, v_step = (int64_t)TPB * g.v_st;
+    // the trip that starts at `first`: FULL (a tag type) when it lies inside the segment, nothing is checked then
+    auto ask = [&](float4v (&f)[PASSES], const uint32_t *base, int64_t st, int64_t step, uint32_t first, auto full) {
+        const uint32_t *p = base + (int64_t)(first + sub) * st;
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ps++) {
+            if constexpr (decltype(full)::value) {
+                f[ps] = *reinterpret_cast<const float4v *>(p);
+            } else {
+                f[ps] = (float4v){0.f, 0.f, 0.f, 0.f};
+                if (first + sub + ps * TPB < n) f[ps] = *reinterpret_cast<const float4v *>(p);
+            }
+            p += step;
+        }
+    };
+    constexpr std::true_type whole_trip{};
+    constexpr std::false_type ragged{};
+    auto ask_k = [&](float4v (&f)[PASSES], uint32_t first) {
+        if (first + SPAN <= n) ask(f, kbase, g.k_st, k_step, first, whole_trip);
+        else ask(f, kbase, g.k_st, k_step, first, ragged);
+    };
+    auto ask_v = [&](float4v (&f)[PASSES], uint32_t first) {
+        if (first + SPAN <= n) ask(f, vbase, g.v_st, v_step, first, whole_trip);
+        else ask(f, vbase, g.v_st, v_step, first, ragged);
+    };
+    float4v ka[PASSES], kb[LOOP ? PASSES : 1];
+    float4v va[PASSES], vb[LOOP ? PASSES : 1];
+    ask_k(ka, 0);
+    if constexpr (!LOOP) ask_v(va, 0); // the whole segment is in flight from the start: the registers hold both
+    float4v qf[MM];
+#pragma unroll
+    for (int m = 0; m < MM; m++) {
+        qf[m] = (float4v){0.f, 0.f, 0.f, 0.f};
+        if ((uint32_t)m < g.M) qf[m] = *reinterpret_cast<const float4v *>(g.Q + oq + (int64_t)m * g.q_sm + l * 4);
+    }
+    // the soft-max phase gives a wave a query row (waves M.. have none); its lanes take positions lane, lane + 64, ...
+    const uint32_t my_row = wave; // < g.M: this wave runs the program on row my_row
+    int64_t base[P::nleaf + 1];
+    LeafWords<P, 1> w[IPL];
+    if (my_row < g.M) {
+#pragma unroll
+        for (int i = 0; i <= P::nleaf; i++) base[i] = 0;
+        uint32_t rr = (uint32_t)(op / g.T) + my_row; // the row in the program's [rows, T] space
+#pragma unroll
+        for (uint32_t d = 0; d < (uint32_t)kMaxOuter; d++) {
+            if (d >= a.g.nouter) break;
+            const uint32_t q = fastdiv(rr, a.g.odiv[d]);
+            const int64_t i = (int64_t)(rr - q * a.g.od[d]);
+            rr = q;
+#pragma unroll
+            for (int lf = 1; lf < P::nleaf; lf++) base[lf] += i * a.leaf[lf].os[d];
+        }
+        if constexpr (!LOOP) { // nothing waits for them yet
+#pragma unroll
+            for (int c = 0; c < IPL; c++)
+                if (lane + c * 64 < n) aot_fetch_from<P, 1>(a, base, t0 + lane + c * 64, w[c]);
+        }
+    }
+
+    // ---- scores of the segment, all rows of the group
+    auto score = [&](const float4v (&f)[PASSES], uint32_t first, auto full) {
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ps++) {
+            const uint32_t t = first + sub + ps * TPB;
+            if (decltype(full)::value || first + ps * TPB < n) { // the same for the whole workgroup
+#pragma unroll
+                for (int m = 0; m < MM; m++) {
+                    if ((uint32_t)m < g.M) {
+                        float v = fmaf(qf[m][3], f[ps][3], fmaf(qf[m][2], f[ps][2], fmaf(qf[m][1], f[ps][1], qf[m][0] * f[ps][0])));
+                        v = row16_sum(v);
+                        if (LPT == 32) v += __shfl_xor(v, 16);
+                        if (l == 0 && (decltype(full)::value || t < n)) sc[m * cap + t] = v;
+                    }
+                }
+            }
+        }
+    };
+    auto score_at = [&](const float4v (&f)[PASSES], uint32_t first) {
+        if (first + SPAN <= n) score(f, first, whole_trip);
+        else score(f, first, ragged);
+    };
+    if constexpr (LOOP) {
+        for (uint32_t first = 0; first < n; first += 2 * SPAN) {
+            if (first + SPAN < n) ask_k(kb, first + SPAN);
+            score_at(ka, first);
+            if (first + 2 * SPAN < n) ask_k(ka, first + 2 * SPAN);
+            if (first + SPAN < n) score_at(kb, first + SPAN);
+        }
+    } else {
+        score_at(ka, 0);
+    }
+    if constexpr (LOOP) ask_v(va, 0); // on its way through the soft-max
+    __syncthreads();
+
+    // ---- the soft-max program on the segment: local maximum, local sum, un-normalised weights
+    if (my_row < g.M) {
+        const uint32_t m = my_row;
+        uint32_t rs[kMaxRowReduce] = {0, 0, 0};
+        uint32_t acc = row_init(true, true);
+        if constexpr (!LOOP) {
+#pragma unroll
+            for (int c = 0; c < IPL; c++) {
+                const uint32_t i = lane + c * 64;
+                if (i < n) {
+                    w[c].v[0][0] = asu(sc[m * cap + i]); // leaf 0 is the score
+                    const Values<P, 1> s = aot_eval<P, 1, ri0>(w[c], rs, a.fault);
+                    acc = row_merge(true, true, acc, s.v[src0][0]);
+                }
+            }
+        } else {
+            for (uint32_t i = lane; i < n; i += 64) {
+                aot_fetch_from<P, 1>(a, base, t0 + i, w[0]);
+                w[0].v[0][0] = asu(sc[m * cap + i]);
+                const Values<P, 1> s = aot_eval<P, 1, ri0>(w[0], rs, a.fault);
+                acc = row_merge(true, true, acc, s.v[src0][0]);
+            }
+        }
+#pragma unroll
+        for (int sft = 32; sft >= 1; sft >>= 1) acc = row_merge(true, true, acc, (uint32_t)__shfl_xor((int)acc, sft));
+        rs[0] = acc;
+        uint32_t sum = row_init(false, true);
+        if constexpr (!LOOP) {
+#pragma unroll
+            for (int c = 0; c < IPL; c++) {
+                const uint32_t i = lane + c * 64;
+                if (i < n) {
+                    const Values<P, 1> s = aot_eval<P, 1, ri1>(w[c], rs, a.fault);
+                    sum = row_merge(false, true, sum, s.v[src1][0]);
+                    sc[m * cap + i] = asf(s.v[src1][0]); // the un-normalised weight
+                }
+            }
+        } else {
+            for (uint32_t i = lane; i < n; i += 64) {
+                aot_fetch_from<P, 1>(a, base, t0 + i, w[0]);
+                w[0].v[0][0] = asu(sc[m * cap + i]);
+                const Values<P, 1> s = aot_eval<P, 1, ri1>(w[0], rs, a.fault);
+                sum = row_merge(false, true, sum, s.v[src1][0]);
+                sc[m * cap + i] = asf(s.v[src1][0]);
+            }
+        }
+#pragma unroll
+        for (int sft = 32; sft >= 1; sft >>= 1) sum = row_merge(false, true, sum, (uint32_t)__shfl_xor((int)sum, sft));
+        if (lane == 0) {
+            float *ml = g.part_ml + (((uint64_t)b * g.splits + split) * g.M + m) * 2;
+            ml[0] = asf(acc);
+            ml[1] = asf(sum);
+        }
+    }
+    __syncthreads();
+
+    // ---- weights times V: the lane's pieces of V are those of its positions, piece l of head_dim
+    float4v o[MM];
+#pragma unroll
+    for (int m = 0; m < MM; m++) o[m] = (float4v){0.f, 0.f, 0.f, 0.f};
+    auto weigh = [&](const float4v (&f)[PASSES], uint32_t first, auto full) {
+#pragma unroll
+        for (int ps = 0; ps < PASSES; ps++) {
+            const uint32_t t = first + sub + ps * TPB;
+            if (decltype(full)::value || t < n) {
+#pragma unroll
+                for (int m = 0; m < MM; m++) {
+                    if ((uint32_t)m < g.M) {
+                        const float wgt = sc[m * cap + t];
+                        o[m][0] = fmaf(wgt, f[ps][0], o[m][0]);
+                        o[m][1] = fmaf(wgt, f[ps][1], o[m][1]);
+                        o[m][2] = fmaf(wgt, f[ps][2], o[m][2]);
+                        o[m][3] = fmaf(wgt, f[ps][3], o[m][3]);
+                    }
+                }
+            }
+        }
+    };
+    auto weigh_at = [&](const float4v (&f)[PASSES], uint32_t first) {
+        if (first + SPAN <= n) weigh(f, first, whole_trip);
+        else weigh(f, first, ragged);
+    };
+    if constexpr (LOOP) {
+        for (uint32_t first = 0; first < n; first += 2 * SPAN) {
+            if (first + SPAN < n) ask_v(vb, first + SPAN);
+            weigh_at(va, first);
+            if (first + 2 * SPAN < n) ask_v(va, first + 2 * SPAN);
+            if (first + SPAN < n) weigh_at(vb, first + SPAN);
+        }
+    } else {
+        weigh_at(va, 0);
+    }
+    // the wave's position groups (lanes l, l + LPT, ...) first, then the waves through LDS
+#pragma unroll
+    for (int m = 0; m < MM; m++) {
+        if ((uint32_t)m < g.M) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                float v = o[m][j];
+#pragma unroll
+                for (int sft = LPT; sft < 64; sft <<= 1) v += __shfl_xor(v, sft);
+                o[m][j] = v;
+            }
+            if (lane < LPT) *reinterpret_cast<float4v *>(&red[(wave * MM + m) * HD + l * 4]) = o[m];
+        }
+    }
+    __syncthreads();
+    for (uint32_t e = tid; e < g.M * HD; e += kSegBlock) {
+        const uint32_t m = e / HD, d = e % HD;
+        float v = 0.0f;
+#pragma unroll
+        for (int k = 0; k < WAVES; k++) v += red[(k * MM + m) * HD + d];
+        g.part_o[(((uint64_t)b * g.splits + split) * g.M + m) * HD + d] = v;
+    }
+}
+
 // out[b][m][n] = sum_c e^(m_c - g) o_c[n] / sum_c e^(m_c - g) l_c.  A wave per (batch entry, query
 // row): lane c first holds the statistics of chunk c (so each weight e^(m_c - g) is computed once
 // and handed round by lane broadcast), then lane n sums output element n (and n + 64) over the chunks.

@@ -98,6 +98,9 @@ struct cg_backend {
     bool fuse = true; // defer element-wise ops and fuse them (CG_FUSE=0 switches it off)
     bool aot = true;  // use the compiled kernels for listed programs (CG_AOT=0: interpreter only)
     uint64_t programs_compiled = 0, programs_interpreted = 0; // launches of fused programs, by kernel kind
+    // decode-time attention over a cache of at least this many positions runs a workgroup per (KV head, segment of the
+    // cache) (CG_ATTN_SEG_FROM, read when the backend is created; 0: never)
+    int64_t attn_seg_from = 6001;
     bool trace_programs = false; // CG_TRACE_PROGRAMS=1: print each distinct deferred program once, to stderr
     cg::ProfClass prof[CG_K_CLASSES];
     std::vector<cg::ProfPending> prof_pending;

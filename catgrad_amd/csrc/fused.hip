@@ -614,6 +614,23 @@ static int64_t attn_row_halves_below() {
     return n;
 }
 
+// Most segments per KV head (env CG_ATTN_SEG_MAX, for measurements).
+static int64_t attn_seg_max() {
+    static const int64_t n = [] { const char *e = getenv("CG_ATTN_SEG_MAX"); return e ? atoll(e) : 8ll; }();
+    return n;
+}
+
+template <class P, int LPT, int MM, int PASSES, bool LOOP>
+static int launch_seg_kernel(cg_backend *be, const AttnArgs &g, const FusedArgs &a, uint32_t batch) {
+    const size_t lds = seg_lds_bytes(MM, LPT * 4, g.chunk);
+    static const bool lds_ok = hipFuncSetAttribute(reinterpret_cast<const void *>(&decode_attention_seg_kernel<P, LPT, MM, PASSES, LOOP>),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                   (int)seg_lds_bytes(MM, LPT * 4, kSegMaxChunk)) == hipSuccess;
+    if (!lds_ok) return fail(CG_ERR_DEVICE, "decode attention: cannot reserve %zu bytes of LDS", seg_lds_bytes(MM, LPT * 4, kSegMaxChunk));
+    hipLaunchKernelGGL((decode_attention_seg_kernel<P, LPT, MM, PASSES, LOOP>), dim3(g.splits, batch), dim3(kSegBlock), lds, be->stream, g, a);
+    return CG_OK;
+}
+
 int launch_decode_attention(cg_backend *be, const Pending &p, const int64_t *pdims, int prank, const cg_tensor *q,
                             const cg_tensor *kt, const cg_tensor *v, cg_tensor *out) {
     if (int frc = flush_deferred(be)) return frc;
@@ -688,6 +705,59 @@ int launch_decode_attention(cg_backend *be, const Pending &p, const int64_t *pdi
     // T x head_dim x 4 multiply-adds); longer caches in segments of at most kRowMaxT positions per workgroup, merged by the
     // combine kernel.  Everything else goes to the chunked kernel below, which spreads a KV head over many workgroups.
     const int64_t qrows = f1.batch * f1.M;
+    // A workgroup per (batch entry, KV head) and segment of the cache, all of the group's rows together: every byte of K and
+    // V is pulled into a compute unit once.  As many segments as put a workgroup on every compute unit, at most
+    // attn_seg_max() (each segment is one more partial result to merge), each a whole number of passes.  Taken for long
+    // caches, and from 1024 positions when there are more query rows than compute units.  Measured with its combine launch
+    // against the kernels below (batch 4 x 8 KV heads x 4 rows, head_dim 64): 2100 positions 20.4 against 19.7 us (the segment
+    // kernel alone 13.6 against 19.7: what it saves, the combine launch and the hand-over to it cost again), 6000 positions 34.9
+    // against 34.9, 9000 positions 44 against 55, 12000 positions 53 against 64; batch 16 at 2100 positions 42 against 46.
+    if (be->attn_seg_from > 0 && (T >= be->attn_seg_from || (qrows > 256 && T >= 1024))) {
+        const int64_t tpb = hd == 64 ? kSegBlock / 16 : kSegBlock / 32;
+        int64_t want = std::min<int64_t>(attn_seg_max(), std::max<int64_t>(1, 256 / f1.batch));
+        want = std::max<int64_t>(1, std::min<int64_t>(want, T / 64));
+        const int64_t chunk = ((T + want - 1) / want + tpb - 1) / tpb * tpb;
+        if (chunk <= kSegMaxChunk) {
+            g.chunk = (uint32_t)chunk;
+            g.splits = (uint32_t)((T + chunk - 1) / chunk);
+            const size_t o_b = (size_t)f1.batch * g.splits * g.M * hd * 4, ml_b = (size_t)f1.batch * g.splits * g.M * 2 * 4;
+            void *so = nullptr, *sml = nullptr;
+            size_t cso = 0, csml = 0;
+            rc = be->pool.alloc(o_b, &so, &cso);
+            if (rc) return rc;
+            rc = be->pool.alloc(ml_b, &sml, &csml);
+            if (rc) {
+                be->pool.free(so, cso);
+                return rc;
+            }
+            g.part_o = static_cast<float *>(so);
+            g.part_ml = static_cast<float *>(sml);
+            be->programs_compiled++;
+            {
+                ProfScope prof(be, CG_K_GEMM_SKINNY, distinct_bytes(q) + distinct_bytes(kt) + distinct_bytes(v) + distinct_bytes(out));
+                const bool one_trip = chunk <= 5 * tpb;
+                const uint32_t nb = (uint32_t)f1.batch;
+#define CG_SEG_KERNEL(LPT, MMV)                                                                    \
+    rc = one_trip ? launch_seg_kernel<P, LPT, MMV, 5, false>(be, g, a, nb) : launch_seg_kernel<P, LPT, MMV, 4, true>(be, g, a, nb)
+                if (hd == 64 && g.M <= 4) CG_SEG_KERNEL(16, 4);
+                else if (hd == 64) CG_SEG_KERNEL(16, 8);
+                else if (g.M <= 4) CG_SEG_KERNEL(32, 4);
+                else CG_SEG_KERNEL(32, 8);
+#undef CG_SEG_KERNEL
+                if (!rc) {
+                    const uint64_t nrows = (uint64_t)f1.batch * g.M, waves = kBlock / 64;
+                    hipLaunchKernelGGL(decode_attention_combine_kernel, dim3((uint32_t)((nrows + waves - 1) / waves)), dim3(kBlock), 0,
+                                       be->stream, g.part_o, g.part_ml, static_cast<uint32_t *>(out->buf->ptr), g.splits, g.M,
+                                       (uint32_t)hd, nrows);
+                }
+            }
+            be->pool.free(so, cso); // stream-ordered: later users queue behind the combine
+            be->pool.free(sml, csml);
+            if (rc) return rc;
+            hipError_t e = hipGetLastError();
+            return e == hipSuccess ? CG_OK : hip_fail(e, "decode attention launch");
+        }
+    }
     const bool one_launch = T <= std::min<int64_t>(attn_whole_limit(), kRowMaxT) && (T <= 1024 || qrows <= 256);
     const bool segmented = !one_launch && attn_whole_limit() > 0 && T > kRowMaxT && T <= attn_segment_limit() && qrows <= 256;
     if (one_launch || segmented) {

@@ -1906,6 +1906,7 @@ int cg_backend_create(int device, cg_backend **out) {
     b->fuse = !(fuse && fuse[0] == '0');
     const char *aot = getenv("CG_AOT");
     b->aot = !(aot && aot[0] == '0');
+    if (const char *seg = getenv("CG_ATTN_SEG_FROM")) b->attn_seg_from = atoll(seg);
     const char *trace = getenv("CG_TRACE_PROGRAMS");
     b->trace_programs = trace && trace[0] == '1';
     char name[256];

@@ -1327,7 +1327,11 @@ for _B, _kvh, _rep, _T, _hd in ((2, 2, 4, 300, 64), (1, 3, 1, 1, 64), (2, 1, 8, 
                                 (4, 8, 4, 2100, 64), (1, 2, 2, 3000, 128), (5, 8, 4, 700, 64), (9, 1, 8, 1100, 128),
                                 (1, 2, 4, 4500, 64), (2, 2, 4, 9000, 64), (1, 1, 2, 5000, 128), (1, 2, 4, 7000, 64),
                                 # few query rows at one sequence (the single-sequence decoder shapes)
-                                (1, 8, 2, 1100, 128), (1, 3, 3, 640, 64), (2, 4, 4, 2049, 64), (1, 2, 4, 513, 64)):
+                                (1, 8, 2, 1100, 128), (1, 3, 3, 640, 64), (2, 4, 4, 2049, 64), (1, 2, 4, 513, 64),
+                                # a workgroup per KV head and segment of the cache with five to eight query rows per KV head: in one
+                                # trip and in several, both head sizes; a last segment of one position; the longest cache it takes
+                                (3, 2, 8, 700, 64), (1, 1, 8, 3000, 64), (1, 1, 8, 2500, 128), (2, 2, 5, 1281, 64), (1, 1, 2, 16384, 64),
+                                (1, 1, 4, 16500, 64)):
     @case(f"decode_attention_B{_B}_kv{_kvh}_rep{_rep}_T{_T}_hd{_hd}", "ew_abs")
     def _(B=_B, kvh=_kvh, rep=_rep, T=_T, hd=_hd):
         q = f32(400 + T, (B, kvh * rep, 1, hd))

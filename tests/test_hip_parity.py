@@ -37,6 +37,40 @@ def test_hip_matches_closed_form(hip, case):
         assert_close(case.kind, g, e, s, f"{case.name}[{i}]")
 
 
+@pytest.fixture(scope="module")
+def hip_segments():
+    """A backend whose decode-time attention always takes the workgroup-per-(KV head, segment) kernel (by default only
+    long caches do): CG_ATTN_SEG_FROM is read when a backend is created."""
+    import os
+
+    from catgrad_amd import HipBackend
+
+    old = os.environ.get("CG_ATTN_SEG_FROM")
+    os.environ["CG_ATTN_SEG_FROM"] = "1"
+    try:
+        be = HipBackend(0)
+    finally:
+        if old is None:
+            del os.environ["CG_ATTN_SEG_FROM"]
+        else:
+            os.environ["CG_ATTN_SEG_FROM"] = old
+    yield be
+    be.close()
+
+
+@pytest.mark.parametrize("case", [c for c in CASES if c.name.startswith(("decode_attention_", "decode_qkv_rope_append_"))],
+                         ids=lambda c: c.name)
+def test_segment_attention_kernel_matches_closed_form_and_oracle(hip_segments, oracle, case):
+    print(f"case={case.name} (segment kernel)", flush=True)
+    got = case.run(hip_segments)
+    exp = case.expect()
+    ref = case.run(oracle)
+    scales = case.scale() if case.scale else [None] * len(exp)
+    for i, (g, e, r, s) in enumerate(zip(got, exp, ref, scales)):
+        assert_close(case.kind, g, e, s, f"{case.name}[{i}] vs closed form")
+        assert_close(case.kind, g, r, s, f"{case.name}[{i}] vs oracle")
+
+
 @pytest.mark.parametrize("case", KATS["cases"], ids=lambda c: c["name"])
 def test_hip_reference_kat(hip, case):
     check_case(hip, case)
@@ -416,3 +450,33 @@ def test_microbench_shapes_properties(hip):
         ex = a64[bi, r] @ b64[bi]
         sc = np.abs(a64[bi, r]) @ np.abs(b64[bi])
         assert (np.abs(full[bi, r] - ex) <= 1e-3 * sc).all()
+
+
+def test_microbench_dense_reductions(hip):
+    """Config-2 reductions on a DENSE random f32[4096, 8192] (the extent and kernel path the micro-benchmark times):
+    sum within 1e-3 of sum |x| against float64, max exact, argmax bit-exact with the last of equal maxima (planted ties,
+    a row of equal values, a +NaN, -0.0 against +0.0)."""
+    rng = np.random.default_rng(42)
+    x = rng.standard_normal((4096, 8192)).astype(np.float32)
+    x[7, 100] = x[7, 8000] = np.float32(9.5)        # equal maxima: the last one wins
+    x[8, :] = np.float32(-1.25)                      # every element equal: index n - 1
+    x[9, 4321] = np.float32(np.nan)                  # +NaN is greatest in total order for argmax, ignored by max
+    x[10, :] = np.float32(-0.0)
+    x[10, 17] = np.float32(0.0)                      # +0.0 beats -0.0 in total order
+    t = hip.from_numpy(x)
+    s = hip.to_numpy(hip.sum(t.clone()))
+    x64 = x.astype(np.float64)
+    ok = np.ones(4096, bool)
+    ok[9] = False                                    # the NaN row sums to NaN
+    assert s.shape == (4096, 1)
+    assert np.all(np.abs(s[ok, 0] - x64[ok].sum(-1)) <= 1e-3 * np.abs(x64[ok]).sum(-1))
+    assert np.isnan(s[9, 0])
+    m = hip.to_numpy(hip.max(t.clone()))
+    ref_max = np.fmax.reduce(x, axis=-1)             # NaN ignored, as f32::max does (ndarray.rs:656-668)
+    np.testing.assert_array_equal(m[:, 0], ref_max)
+    am = hip.to_numpy(hip.argmax(t))[:, 0]
+    i32 = x.view(np.int32).astype(np.int64)
+    key = np.where(i32 < 0, -(i32 & 0x7FFFFFFF) - 1, i32)   # total_cmp order of the bit patterns (ndarray.rs:670-681)
+    ref_am = (8192 - 1 - np.argmax(key[:, ::-1], axis=-1)).astype(np.uint32)
+    np.testing.assert_array_equal(am, ref_am)
+    assert am[7] == 8000 and am[8] == 8191 and am[9] == 4321 and am[10] == 17
