@@ -855,6 +855,11 @@ struct PrefillArgs {
     uint32_t mask_mul;  // f32 bits of the multiplier of the 0/1 mask
     uint32_t batch;     // folded batch entries (KV heads)
     uint32_t tiles_per_head; // S / 128 when that is whole and heads are whole in M, else 0
+    // Few workgroups (one sequence, a short prompt): the keys of a row tile are cut into `ksplit` parts over grid.y; a part
+    // leaves its rows' running maximum, sum and un-normalised O for prefill_attention_combine_kernel.
+    uint32_t ksplit;    // 1: none
+    float *part_o;      // [ksplit][batch][M][hd]
+    float *part_ml;     // [ksplit][batch][M][2]
 };
 
 constexpr int kPfRows = 128, kPfKeys = 64;
@@ -913,7 +918,10 @@ __global__ __launch_bounds__(kBlock) void prefill_attention_kernel(const AttnArg
         const uint32_t smax = s0 + last < e.S ? s0 + last : e.S - 1;            // the tile may run into the next head
         kmax = min(g.T - 1, e.pos0 + smax);
     }
-    const uint32_t ntiles = kmax / kPfKeys + 1;
+    const uint32_t ntiles_all = kmax / kPfKeys + 1;
+    // this workgroup's share of the key tiles (all of them without a split)
+    const uint32_t per_part = (ntiles_all + e.ksplit - 1) / e.ksplit;
+    const uint32_t it_first = blockIdx.y * per_part, ntiles = min(ntiles_all, it_first + per_part);
 
     // the query rows, as second MFMA operands: chunk c covers d = 8c .. 8c+7, this lane holds 4*lg .. 4*lg+3 of them.
     // The program divides every score by the scale; dividing the query once instead is the same value up to
@@ -958,11 +966,13 @@ __global__ __launch_bounds__(kBlock) void prefill_attention_kernel(const AttnArg
             *reinterpret_cast<float4v *>(&Vs[buf][t][dq * 4]) = vr[h];
         }
     };
-    load_kv(0);
-    store_kv(0);
+    if (it_first < ntiles) { // (a part beyond the last key tile of these rows has nothing to do but to say so)
+        load_kv(it_first * kPfKeys);
+        store_kv(it_first & 1);
+    }
     __syncthreads();
 
-    for (uint32_t it = 0; it < ntiles; it++) {
+    for (uint32_t it = it_first; it < ntiles; it++) {
         const uint32_t cur = it & 1, t0 = it * kPfKeys;
         const bool more = it + 1 < ntiles;
         if (more) load_kv(t0 + kPfKeys);
@@ -1037,6 +1047,26 @@ __global__ __launch_bounds__(kBlock) void prefill_attention_kernel(const AttnArg
         if (more) store_kv(cur ^ 1);
         __syncthreads();
     }
+    if (e.ksplit > 1) { // the part's statistics and un-normalised O; lane group 0 of a wave writes the statistics
+        if (live) {
+            const uint64_t row = ((uint64_t)blockIdx.y * e.batch + b) * g.M + m;
+            float *orow = e.part_o + row * HD;
+#pragma unroll
+            for (int db = 0; db < HD / 32; db++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    float4v o;
+#pragma unroll
+                    for (int r = 0; r < 4; r++) o[r] = acc_o[db][j * 4 + r];
+                    *reinterpret_cast<float4v *>(orow + db * 32 + j * 8 + lg * 4) = o;
+                }
+            if (lg == 0) {
+                e.part_ml[row * 2] = run_max;
+                e.part_ml[row * 2 + 1] = run_sum;
+            }
+        }
+        return;
+    }
     // ---- out[m][d] = O^T[d][m] / l[m]
     if (live) {
         uint32_t *orow = e.out + ((uint64_t)b * g.M + m) * HD;
@@ -1050,4 +1080,34 @@ __global__ __launch_bounds__(kBlock) void prefill_attention_kernel(const AttnArg
                 *reinterpret_cast<float4v *>(orow + db * 32 + j * 8 + lg * 4) = o;
             }
     }
+}
+
+// out[row][d] = sum_p 2^((m_p - g) log2 e) O_p[row][d] / sum_p 2^((m_p - g) log2 e) l_p, g = max_p m_p: the parts of a
+// prefill attention whose keys were cut over several workgroups, merged in the order of the parts.  A thread per four
+// consecutive d of a row.  A part that saw no key of a row has m_p = -inf, l_p = 0 and O_p = 0: weight zero.
+__global__ __launch_bounds__(kBlock) void prefill_attention_combine_kernel(const float *part_o, const float *part_ml, uint32_t *out,
+                                                                           uint32_t parts, uint32_t hd, uint64_t rows) {
+    const uint64_t i = (uint64_t)blockIdx.x * kBlock + threadIdx.x, q = hd / 4;
+    if (i >= rows * q) return;
+    const uint64_t row = i / q;
+    const uint32_t d = (uint32_t)(i % q) * 4;
+    constexpr float kLog2e = 1.4426950408889634f;
+    float g = -INFINITY;
+    for (uint32_t p = 0; p < parts; p++) g = fmaxf(g, part_ml[((uint64_t)p * rows + row) * 2]);
+    float4v num = {0.f, 0.f, 0.f, 0.f};
+    float den = 0.0f;
+    for (uint32_t p = 0; p < parts; p++) {
+        const float *ml = part_ml + ((uint64_t)p * rows + row) * 2;
+        const float w = __builtin_amdgcn_exp2f((ml[0] - g) * kLog2e);
+        const float4v o = *reinterpret_cast<const float4v *>(part_o + ((uint64_t)p * rows + row) * hd + d);
+        den = fmaf(w, ml[1], den);
+        num[0] = fmaf(w, o[0], num[0]);
+        num[1] = fmaf(w, o[1], num[1]);
+        num[2] = fmaf(w, o[2], num[2]);
+        num[3] = fmaf(w, o[3], num[3]);
+    }
+    float4v r;
+#pragma unroll
+    for (int k = 0; k < 4; k++) r[k] = num[k] / den;
+    *reinterpret_cast<float4v *>(out + row * hd + d) = r;
 }

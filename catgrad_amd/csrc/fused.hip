@@ -941,15 +941,51 @@ int launch_prefill_attention(cg_backend *be, const Pending &p, const int64_t *pd
     e.tiles_per_head = S % kPfRows == 0 ? (uint32_t)(S / kPfRows) : 0;
     const uint64_t nblocks = (uint64_t)((f1.M + kPfRows - 1) / kPfRows) * (uint64_t)f1.batch;
     if (nblocks > 0x7FFFFFFFull) return pf_declined(be, 17);
+    // Fewer workgroups than the device takes at once (one sequence; a short prompt): what bounds the launch is the chain of
+    // matrix instructions of the workgroup with the most keys, so the keys of every row tile are cut into parts (at least two
+    // key tiles each, about two workgroups per compute unit in all) and a small second kernel merges the parts.
+    // (env CG_PREFILL_KSPLIT=n forces n parts, 1 = never)
+    static const int forced_split = [] { const char *ev = getenv("CG_PREFILL_KSPLIT"); return ev ? atoi(ev) : 0; }();
+    const int64_t key_tiles = (std::min<int64_t>(T, (int64_t)e.pos0 + S) + kPfKeys - 1) / kPfKeys;
+    int64_t ksplit = forced_split > 0 ? forced_split : std::min<int64_t>((512 + (int64_t)nblocks - 1) / (int64_t)nblocks, 8);
+    ksplit = std::max<int64_t>(1, std::min<int64_t>(ksplit, key_tiles / 2));
+    if (forced_split <= 0 && nblocks >= 256) ksplit = 1;
+    e.ksplit = (uint32_t)ksplit;
+    e.part_o = e.part_ml = nullptr;
+    void *po = nullptr, *pml = nullptr;
+    size_t cpo = 0, cpml = 0;
+    const uint64_t rows = (uint64_t)f1.batch * (uint64_t)f1.M;
+    if (ksplit > 1) {
+        rc = be->pool.alloc((size_t)ksplit * rows * hd * 4, &po, &cpo);
+        if (rc) return rc;
+        rc = be->pool.alloc((size_t)ksplit * rows * 2 * 4, &pml, &cpml);
+        if (rc) {
+            be->pool.free(po, cpo);
+            return rc;
+        }
+        e.part_o = static_cast<float *>(po);
+        e.part_ml = static_cast<float *>(pml);
+    }
     be->programs_compiled++;
-    // flop: the visible half of the [rows, T] rectangle, twice (scores and weighted sum)
-    const double flop = 2.0 * 2.0 * (double)f1.batch * (double)f1.M * (double)hd * ((double)e.pos0 + 0.5 * (double)S);
-    ProfScope prof(be, CG_K_ATTENTION, flop);
-    dim3 grid((uint32_t)nblocks);
-    if (hd == 64)
-        hipLaunchKernelGGL((prefill_attention_kernel<64>), grid, dim3(kBlock), prefill_lds_bytes(64), be->stream, g, e);
-    else
-        hipLaunchKernelGGL((prefill_attention_kernel<128>), grid, dim3(kBlock), prefill_lds_bytes(128), be->stream, g, e);
+    {
+        // flop: the visible half of the [rows, T] rectangle, twice (scores and weighted sum)
+        const double flop = 2.0 * 2.0 * (double)f1.batch * (double)f1.M * (double)hd * ((double)e.pos0 + 0.5 * (double)S);
+        ProfScope prof(be, CG_K_ATTENTION, flop);
+        dim3 grid((uint32_t)nblocks, (uint32_t)ksplit);
+        if (hd == 64)
+            hipLaunchKernelGGL((prefill_attention_kernel<64>), grid, dim3(kBlock), prefill_lds_bytes(64), be->stream, g, e);
+        else
+            hipLaunchKernelGGL((prefill_attention_kernel<128>), grid, dim3(kBlock), prefill_lds_bytes(128), be->stream, g, e);
+        if (ksplit > 1) {
+            const uint64_t items = rows * (uint64_t)(hd / 4);
+            hipLaunchKernelGGL(prefill_attention_combine_kernel, dim3((uint32_t)((items + kBlock - 1) / kBlock)), dim3(kBlock), 0, be->stream,
+                               e.part_o, e.part_ml, e.out, (uint32_t)ksplit, (uint32_t)hd, rows);
+        }
+    }
+    if (ksplit > 1) {
+        be->pool.free(po, cpo); // stream-ordered: later users queue behind the combine
+        be->pool.free(pml, cpml);
+    }
     hipError_t err = hipGetLastError();
     return err == hipSuccess ? CG_OK : hip_fail(err, "prefill attention launch");
 }

@@ -65,6 +65,7 @@ struct MmArgs {
     int64_t a_bs[kMaxBatchAxes], b_bs[kMaxBatchAxes];
     uint32_t batch;
     uint32_t a_vec, b_vec;          // 16-byte loads along the unit-stride axis are legal
+    uint32_t ksplit;                // mfma_gemm_kernel: values of k per workgroup along grid.z (a multiple of 32), 0 = all of K
 };
 
 __device__ __forceinline__ void batch_offsets(const MmArgs &a, uint32_t b, int64_t &oa, int64_t &ob) {
@@ -276,9 +277,14 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
     const uint32_t m0 = tile_m * BM, n0 = tile_n * BN;
     int64_t oa, ob;
     batch_offsets(a, blockIdx.y, oa, ob);
-    const uint32_t *A = a.A + oa;
-    const uint32_t *B = a.B + ob;
-    uint32_t *C = a.C + (uint64_t)blockIdx.y * a.M * a.N;
+    // A product with too few tiles for the device is cut along k over grid.z: this workgroup multiplies k0 .. k0 + Kk and
+    // leaves its tile in slot (batch entry, split) of a.C, which then is scratch memory that splitk_reduce_kernel sums up
+    // in a fixed order.
+    const uint32_t k0 = blockIdx.z * a.ksplit;
+    const uint32_t Kk = a.ksplit ? min(a.K - k0, a.ksplit) : a.K;
+    const uint32_t *A = a.A + oa + (int64_t)k0 * a.a_sk;
+    const uint32_t *B = a.B + ob + (int64_t)k0 * a.b_sk;
+    uint32_t *C = a.C + ((uint64_t)blockIdx.y * gridDim.z + blockIdx.z) * a.M * a.N;
 
     const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x % 64;
     const uint32_t wm = (wave / 2) * (32 * MT), wn = (wave % 2) * (32 * NT); // wave quadrant
@@ -294,9 +300,9 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
 
     TileRegs<BM> ra;
     TileRegs<BN> rb;
-    const uint32_t nk = (a.K + BK - 1) / BK;
-    load_tile<A_MFAST>(ra, A, a.a_sm, a.a_sk, m0, 0, a.M, a.K, a.a_vec);
-    load_tile<B_NFAST>(rb, B, a.b_sn, a.b_sk, n0, 0, a.N, a.K, a.b_vec);
+    const uint32_t nk = (Kk + BK - 1) / BK;
+    load_tile<A_MFAST>(ra, A, a.a_sm, a.a_sk, m0, 0, a.M, Kk, a.a_vec);
+    load_tile<B_NFAST>(rb, B, a.b_sn, a.b_sk, n0, 0, a.N, Kk, a.b_vec);
     stage(ra, rb, 0);
     __syncthreads();
 
@@ -325,15 +331,15 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
         }
         const bool lean = (uint64_t)a.M * (uint64_t)a.a_sm < (1ull << 30) && (uint64_t)a.N * (uint64_t)a.b_sn < (1ull << 30); // offsets fit 32 bits
         auto ask = [&](TileRegs<BM> &ta, TileRegs<BN> &tb, uint32_t kt) {
-            if (lean && (kt + 1) * BK <= a.K) {
+            if (lean && (kt + 1) * BK <= Kk) {
                 const char *pa = reinterpret_cast<const char *>(A + (uint64_t)kt * BK), *pb = reinterpret_cast<const char *>(B + (uint64_t)kt * BK);
 #pragma unroll
                 for (int h = 0; h < TileRegs<BM>::slots; h++) ta.v[h] = *reinterpret_cast<const float4v *>(pa + offa[h]);
 #pragma unroll
                 for (int h = 0; h < TileRegs<BN>::slots; h++) tb.v[h] = *reinterpret_cast<const float4v *>(pb + offb[h]);
             } else {
-                load_tile<false>(ta, A, a.a_sm, a.a_sk, m0, kt * BK, a.M, a.K, a.a_vec);
-                load_tile<false>(tb, B, a.b_sn, a.b_sk, n0, kt * BK, a.N, a.K, a.b_vec);
+                load_tile<false>(ta, A, a.a_sm, a.a_sk, m0, kt * BK, a.M, Kk, a.a_vec);
+                load_tile<false>(tb, B, a.b_sn, a.b_sk, n0, kt * BK, a.N, Kk, a.b_vec);
             }
         };
         // One tile: S steps of 16 (fp8: 32) k.  Set 0 holds the fragments of step 0 when a tile begins; every step reads the
@@ -500,7 +506,7 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
             }
         };
         uint32_t kt = 0;
-        if (lean && 3 * BK <= a.K) {
+        if (lean && 3 * BK <= Kk) {
             // tile 1 is asked for slot by slot in the order the loop consumes the slots: only then does the compiler's count
             // of loads in flight at the loop's head match the one at its end, and each LDS store waits for its own load
             // (all but the 15 younger ones) instead of for every load
@@ -516,7 +522,7 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
                 __builtin_amdgcn_sched_barrier(0);
             }
             first_fragments();
-            for (; (kt + 3) * BK <= a.K; kt++) iteration(kt, std::true_type{});
+            for (; (kt + 3) * BK <= Kk; kt++) iteration(kt, std::true_type{});
         } else {
             if (nk > 1) ask(ra, rb, 1); // (tile 0 is in LDS buffer 0 by now)
             if constexpr (HALF != 5) first_fragments();
@@ -535,8 +541,8 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
     if constexpr (LEAN) {
         const bool a_ok = A_MFAST ? (a.a_vec && a.a_sm == 1 && a.M % 4 == 0 && a.M >= 4) : (a.a_vec && a.a_sk == 1 && a.a_sm > 0);
         const bool b_ok = B_NFAST ? (a.b_vec && a.b_sn == 1 && a.N % 4 == 0 && a.N >= 4) : (a.b_vec && a.b_sk == 1 && a.b_sn > 0);
-        const uint64_t a_span = A_MFAST ? (uint64_t)a.K * (uint64_t)a.a_sk : (uint64_t)a.M * (uint64_t)a.a_sm;
-        const uint64_t b_span = B_NFAST ? (uint64_t)a.K * (uint64_t)a.b_sk : (uint64_t)a.N * (uint64_t)a.b_sn;
+        const uint64_t a_span = A_MFAST ? (uint64_t)Kk * (uint64_t)a.a_sk : (uint64_t)a.M * (uint64_t)a.a_sm;
+        const uint64_t b_span = B_NFAST ? (uint64_t)Kk * (uint64_t)a.b_sk : (uint64_t)a.N * (uint64_t)a.b_sn;
         lean_kk = a_ok && b_ok && a.a_sk > 0 && a.b_sk > 0 && a_span < (1ull << 30) && b_span < (1ull << 30); // offsets fit 32 bits
 #pragma unroll
         for (int h = 0; h < TileRegs<BM>::slots; h++) {
@@ -607,8 +613,8 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
 #pragma unroll
             for (int h = 0; h < TileRegs<BN>::slots; h++) rb.v[h] = *reinterpret_cast<const float4v *>(pb + offb_kk[h]);
         } else if (more) {
-            load_tile<A_MFAST>(ra, A, a.a_sm, a.a_sk, m0, (kt + 1) * BK, a.M, a.K, a.a_vec);
-            load_tile<B_NFAST>(rb, B, a.b_sn, a.b_sk, n0, (kt + 1) * BK, a.N, a.K, a.b_vec);
+            load_tile<A_MFAST>(ra, A, a.a_sm, a.a_sk, m0, (kt + 1) * BK, a.M, Kk, a.a_vec);
+            load_tile<B_NFAST>(rb, B, a.b_sn, a.b_sk, n0, (kt + 1) * BK, a.N, Kk, a.b_vec);
         }
         __builtin_amdgcn_s_setprio(1);
         if constexpr (WIDEN) {
@@ -655,7 +661,7 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
         uint32_t kt = 0;
         if constexpr (LEAN) {
             if (lean_kk)
-                for (; (kt + 2) * BK <= a.K; kt++) iterate(kt, std::true_type{});
+                for (; (kt + 2) * BK <= Kk; kt++) iterate(kt, std::true_type{});
         }
         for (; kt < (PACKED ? 0u : nk); kt++) iterate(kt, std::false_type{});
     }
@@ -1421,6 +1427,22 @@ __global__ __launch_bounds__(kThreads) void skinny_nn_kernel(const MmArgs a, uin
     }
 }
 
+// The same four elements at a time (mn a multiple of 4, both arrays 16-byte aligned): the sums in the same fixed order.
+__global__ __launch_bounds__(kThreads) void splitk_reduce4_kernel(const float4v *part, float4v *C, uint32_t splits, uint32_t mn4, uint64_t total4) {
+    const uint64_t i = (uint64_t)blockIdx.x * kThreads + threadIdx.x;
+    if (i >= total4) return;
+    const uint64_t b = i / mn4, e = i % mn4;
+    float4v v = {0.f, 0.f, 0.f, 0.f};
+    for (uint32_t s = 0; s < splits; s++) {
+        const float4v p = __builtin_nontemporal_load(part + (b * splits + s) * mn4 + e);
+        v[0] += p[0];
+        v[1] += p[1];
+        v[2] += p[2];
+        v[3] += p[3];
+    }
+    C[i] = v;
+}
+
 // C[b][e] = sum over s of part[b][s][e]   (e < M*N)
 __global__ __launch_bounds__(kThreads) void splitk_reduce_kernel(const uint32_t *part, uint32_t *C, uint32_t splits,
                                                                  uint32_t mn, uint64_t total) {
@@ -2142,7 +2164,37 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
         const bool big = fits_big && (narrow_dtype || (!a_mfast && b_nfast));
         uint64_t tiles = big ? tiles_big / batch : (uint64_t)((M + BM - 1) / BM) * ((N + bn - 1) / bn);
         if (tiles > 0x7FFFFFFFull) return fail(CG_ERR_UNSUPPORTED, "matmul: too many tiles");
-        dim3 grid((uint32_t)tiles, (uint32_t)batch);
+        // Too few tiles for the device (the linear layers of a short prefill on a narrow model): cut along k as well, so that
+        // about two workgroups per compute unit run, each with at least 128 values of k; the partial tiles go to scratch memory
+        // and are summed in a fixed order (the same shape always gets the same cut: results are identical from run to run).
+        // (env CG_GEMM_SPLITK=0 switches it off)
+        static const bool splitk_allowed = [] {
+            const char *e = getenv("CG_GEMM_SPLITK");
+            return !(e && e[0] == '0');
+        }();
+        static const int64_t splitk_below = [] { const char *e = getenv("CG_GEMM_SPLITK_BELOW"); return e ? atoll(e) : 256ll; }();
+        static const int64_t splitk_target = [] { const char *e = getenv("CG_GEMM_SPLITK_TARGET"); return e ? atoll(e) : 512ll; }();
+        int64_t splits = 1;
+        uint32_t kchunk = 0;
+        if (splitk_allowed && !narrow_dtype && !big && (int64_t)(tiles * (uint64_t)batch) < splitk_below && K >= 256) {
+            const int64_t wgs = (int64_t)tiles * batch;
+            splits = std::min<int64_t>(std::min<int64_t>((splitk_target + wgs - 1) / wgs, K / 128), 16);
+            kchunk = (uint32_t)(((K + splits - 1) / splits + BK - 1) / BK * BK);
+            splits = (K + kchunk - 1) / kchunk;
+            if (splits < 2) {
+                splits = 1;
+                kchunk = 0;
+            }
+        }
+        void *kscratch = nullptr;
+        size_t kscratch_cls = 0;
+        if (splits > 1) {
+            int src = be->pool.alloc((size_t)batch * splits * M * N * 4, &kscratch, &kscratch_cls);
+            if (src) return src;
+            a.C = static_cast<uint32_t *>(kscratch);
+            a.ksplit = kchunk;
+        }
+        dim3 grid((uint32_t)tiles, (uint32_t)batch, (uint32_t)splits);
         static const bool lds_ok = [] { // the tiles need more than the default 64 KiB of dynamic LDS
             bool ok = true;
 #define CG_LDS(AF, BF)                                                                                                \
@@ -2231,6 +2283,18 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
         }
 #undef CG_GEMM
 #undef CG_GEMM_HALF
+        if (splits > 1) {
+            uint32_t *const dst = static_cast<uint32_t *>(out->buf->ptr);
+            const uint64_t mn = (uint64_t)M * N, total = mn * batch;
+            if (mn % 4 == 0 && reinterpret_cast<uintptr_t>(dst) % 16 == 0)
+                hipLaunchKernelGGL(splitk_reduce4_kernel, dim3((uint32_t)((total / 4 + kThreads - 1) / kThreads)), dim3(kThreads), 0, s,
+                                   static_cast<const float4v *>(kscratch), reinterpret_cast<float4v *>(dst), (uint32_t)splits,
+                                   (uint32_t)(mn / 4), total / 4);
+            else
+                hipLaunchKernelGGL(splitk_reduce_kernel, dim3((uint32_t)((total + kThreads - 1) / kThreads)), dim3(kThreads), 0, s,
+                                   static_cast<const uint32_t *>(kscratch), dst, (uint32_t)splits, (uint32_t)mn, total);
+            be->pool.free(kscratch, kscratch_cls); // stream-ordered: later users queue behind the reduce
+        }
     }
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? CG_OK : hip_fail(e, "matmul launch");

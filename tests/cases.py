@@ -854,6 +854,24 @@ _mm_case("mm_256_tiles_rhs_transposed", (43, 300, 70), (43, 520, 70),
 _mm_case("mm_256_tiles_both_transposed_linear", (300, 16, 68), (5000, 68),
          lambda be, a, b: (be.transpose(a, 0, 1), be.broadcast(be.transpose(b, 0, 1), (16, 68, 5000)), None, None), seed=100)
 
+# products with fewer 128-wide tiles than compute units (the linear layers of a short prefill on a narrow model): cut
+# along k over grid.z, the partial tiles summed in a fixed order.  The linear layers of the Qwen3-0.6B shape at 1024
+# positions and of the SmolLM2-135M shape at 512, a k that is no multiple of the tile depth, a row-contiguous right
+# operand, a transposed left operand, several batch entries.
+def _linear_prep(n_out):
+    return lambda be, a, b: (a, be.broadcast(be.transpose(b, 0, 1), (a.shape[0], b.shape[1], n_out)), None, None)
+
+
+_mm_case("mm_split_k_1024x1024x3072", (1, 1024, 3072), (1024, 3072), _linear_prep(1024), seed=110)
+_mm_case("mm_split_k_1024x2048x1024", (1, 1024, 1024), (2048, 1024), _linear_prep(2048), seed=112)
+_mm_case("mm_split_k_512x576x576", (1, 512, 576), (576, 576), _linear_prep(576), seed=114)
+_mm_case("mm_split_k_512x1536x576", (1, 512, 576), (1536, 576), _linear_prep(1536), seed=116)
+_mm_case("mm_split_k_512x576x1536", (1, 512, 1536), (576, 1536), _linear_prep(576), seed=118)
+_mm_case("mm_split_k_ragged_k", (1, 300, 1000), (200, 1000), _linear_prep(200), seed=120)
+_mm_case("mm_split_k_rhs_rows", (1, 256, 2048), (1, 2048, 384), seed=122)
+_mm_case("mm_split_k_lhs_transposed", (2, 1100, 130), (2, 1100, 260), lambda be, a, b: (be.transpose(a, 1, 2), b, None, None), seed=124)
+_mm_case("mm_split_k_batched", (3, 128, 1024), (3, 1024, 128), seed=126)
+
 
 @case("mm_u32_wrapping")
 def _():
@@ -1435,7 +1453,10 @@ for _B, _K, _kvh, _rep, _T, _hd, _normed in ((4, 2048, 8, 4, 300, 64, True), (1,
 # ---- prefill attention: many query positions per head, causal ---------------------------------------------------------
 for _B, _kvh, _rep, _S, _T, _hd in ((1, 2, 4, 48, 48, 64), (2, 1, 1, 128, 128, 64), (1, 2, 2, 200, 333, 64), (2, 2, 4, 96, 96, 64),
                                      (1, 1, 3, 70, 70, 64), (1, 1, 1, 9, 500, 64), (1, 2, 2, 64, 64, 128), (2, 1, 4, 200, 333, 128),
-                                     (1, 2, 2, 40, 40, 32)):
+                                     (1, 2, 2, 40, 40, 32),
+                                     # few workgroups: the keys of a row tile cut over several of them and merged (parts without a
+                                     # visible key for some rows, a last part of one tile, both head sizes, a prompt behind a cache)
+                                     (1, 2, 2, 1024, 1024, 128), (1, 3, 3, 512, 512, 64), (1, 1, 4, 300, 1500, 64), (2, 1, 2, 130, 777, 128)):
     @case(f"prefill_attention_B{_B}_kv{_kvh}_rep{_rep}_S{_S}_T{_T}_hd{_hd}", "ew_abs")
     def _(B=_B, kvh=_kvh, rep=_rep, S=_S, T=_T, hd=_hd):
         """q [B, H, S, hd] against caches of T >= S positions (the last S of them are the queries' own): row tiles
