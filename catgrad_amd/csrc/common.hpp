@@ -313,24 +313,26 @@ void lazy_mm_release(LazyMm *m);
 // Computes the product if it has not been yet.
 int lazy_mm_force(cg_backend *be, LazyMm *m);
 
+// (No default member initialisers: a Pending holds eight of these and most programs use one or two, so its leaf table
+// starts out uninitialised and only leaf[0 .. nleaf) is ever read.  `LeafView lv{};` gives an empty one: everything zero.)
 struct LeafView {
-    Buffer *buf = nullptr; // retained; null for uniform leaves (and for a lazy product not yet computed)
-    LazyMm *lazy = nullptr; // retained: the leaf is the (row-major) result of this product
-    int64_t strides[kMaxRank] = {0};
-    int64_t offset = 0;
-    bool uniform = false;
-    uint32_t ubits = 0;
+    Buffer *buf; // retained; null for uniform leaves (and for a lazy product not yet computed)
+    LazyMm *lazy; // retained: the leaf is the (row-major) result of this product
+    int64_t strides[kMaxRank];
+    int64_t offset;
+    bool uniform;
+    uint32_t ubits;
     // Piecewise leaf (the deferred form of `concat` along the last axis): positions below
     // `pw_split` of the last axis read the view above, the others read (buf2, strides2,
     // offset2) at position - pw_split; a part may be negated on load (f32 sign flip), which
     // is how rotate_half = concat(-x2, x1) of the rotary embedding stays a leaf.
-    bool pw = false;
-    Buffer *buf2 = nullptr; // retained
-    LazyMm *lazy2 = nullptr; // retained: the second part is a view of this product's result (buf2 null until it is computed)
-    int64_t strides2[kMaxRank] = {0};
-    int64_t offset2 = 0;
-    int64_t pw_split = 0;
-    bool neg1 = false, neg2 = false;
+    bool pw;
+    Buffer *buf2; // retained
+    LazyMm *lazy2; // retained: the second part is a view of this product's result (buf2 null until it is computed)
+    int64_t strides2[kMaxRank];
+    int64_t offset2;
+    int64_t pw_split;
+    bool neg1, neg2;
 };
 
 struct Pending {

@@ -863,8 +863,12 @@ template <int MM> __global__ __launch_bounds__(kThreads) void skinny_kt_wide_res
 // columns per workgroup (one activation load per lane and trip instead of M) when its 2048-wide chunks of k are full.
 // With a single row it is 0.7 us behind the one-column-per-wave kernel at K = 2048 and level with it at K = 8192;
 // it is used all the same, because its residual store and its norm-applying loads save two launches per layer.
-// Chunks of 2048 values of k when K is a multiple of that, of 1024 when of that (hidden sizes like 1024 or 3072).
-static inline int xreg_trips(uint32_t K) { return K % 2048 == 0 ? 8 : K % 1024 == 0 ? 4 : 0; }
+// Chunks of 2048 values of k when K is a multiple of that, of 1024 when of that (hidden sizes like 1024 or 3072); any
+// other K (a multiple of 4 above 256: hidden sizes like 576 or 1536) runs with a ragged last chunk, the waves of a
+// workgroup then interleaved every 64 values of k (xreg_lane_k) so that a short chunk still spreads over all four.
+static inline int xreg_trips(uint32_t K) {
+    return K % 2048 == 0 ? 8 : K % 1024 == 0 ? 4 : (K % 4 == 0 && K > 256) ? (K > 1024 ? 8 : 4) : 0;
+}
 // Column groups per workgroup of the one-chunk gated kernel: as many as leave about two workgroups per compute unit
 // (env CG_XREG_ITERS=n forces n, for measurements).
 static inline uint32_t xreg_cols_iters(uint64_t groups) {
@@ -916,6 +920,15 @@ template <int MM> __global__ __launch_bounds__(kThreads) void skinny_kt_wide_gro
 __device__ __forceinline__ uint32_t norm_divisor(const NormFuse &nf, float sum) {
     const uint32_t mean = apply<kDiv, true>(asu(sum), nf.n_bits, 0, nullptr);
     return apply<kPow, true>(apply<kAdd, true>(mean, nf.eps_bits, 0, nullptr), nf.exp_bits, 0, nullptr);
+}
+// Where a lane's k values lie inside a chunk of TRIPS * 256: trip t covers k0 + kb + ks * t .. + 3.  Whole chunks: a wave
+// takes a quarter of the chunk in a row (2 KiB in a row of each weight row: measured 12 % faster on the gate / up pair than
+// interleaving the waves every 256 bytes).  A ragged last chunk: the waves interleaved every 64 values of k, so that what
+// there is of the chunk is shared by all four.
+template <int TRIPS> __device__ __forceinline__ void xreg_lane_k(uint32_t K, uint32_t wave, uint32_t b, uint32_t &kb, uint32_t &ks) {
+    const bool ragged = K % (TRIPS * 256) != 0;
+    kb = (ragged ? wave * 64 : wave * (TRIPS * 64)) + b * 4;
+    ks = ragged ? 256u : 64u;
 }
 template <int MM, int CG, bool GATED = false, bool RESIDUAL = false, bool NORM = false, int TRIPS = 8>
 __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const uint32_t block_x, const uint32_t block_y,
@@ -970,12 +983,13 @@ __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const 
     }
     // of every chunk of TRIPS * 256 values of k (2048 or 1024) a wave takes a quarter in a row (TRIPS trips of 64)
     static_assert(TRIPS == 8 || TRIPS == 4, "chunks of 2048 or 1024");
-    const uint32_t kb = wave * (TRIPS * 64) + b * 4;
+    uint32_t kb, ks;
+    xreg_lane_k<TRIPS>(a.K, wave, b, kb, ks);
     for (uint32_t k0 = 0; k0 < a.K; k0 += TRIPS * 256) {
         float4v xr[G][TRIPS];
 #pragma unroll
         for (int t = 0; t < TRIPS; t++) {
-            const uint32_t k = k0 + kb + 64 * t;
+            const uint32_t k = k0 + kb + ks * t;
 #pragma unroll
             for (int g = 0; g < G; g++) {
                 xr[g][t] = (float4v){0.f, 0.f, 0.f, 0.f};
@@ -986,7 +1000,7 @@ __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const 
         if constexpr (NORM) {
 #pragma unroll
             for (int t = 0; t < TRIPS; t++) {
-                const uint32_t k = k0 + kb + 64 * t;
+                const uint32_t k = k0 + kb + ks * t;
                 gm[t] = (float4v){0.f, 0.f, 0.f, 0.f};
                 if (k < a.K) gm[t] = *reinterpret_cast<const float4v *>(nf->gamma + k);
             }
@@ -996,7 +1010,7 @@ __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const 
             float4v w[TRIPS];
 #pragma unroll
             for (int t = 0; t < TRIPS; t++) {
-                const uint32_t k = k0 + kb + 64 * t;
+                const uint32_t k = k0 + kb + ks * t;
                 w[t] = (float4v){0.f, 0.f, 0.f, 0.f};
                 if (k < a.K) w[t] = *reinterpret_cast<const float4v *>(wrow[c] + k);
             }
@@ -1154,21 +1168,28 @@ __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_group_rope_kerne
             if (i < nf.blocks * 4) pv[u] = nf.partials[i];
         }
     }
-    const uint32_t kb = wave * (TRIPS * 64) + b * 4;
+    uint32_t kb, ks;
+    xreg_lane_k<TRIPS>(a.K, wave, b, kb, ks);
+    // (a value of k beyond K contributes zeros: only a ragged last chunk has any)
+    auto at = [&](const uint32_t *row, uint32_t k) {
+        float4v v = {0.f, 0.f, 0.f, 0.f};
+        if (k < a.K) v = *reinterpret_cast<const float4v *>(row + k);
+        return v;
+    };
     for (uint32_t k0 = 0; k0 < a.K; k0 += TRIPS * 256) {
         float4v xr[TRIPS];
 #pragma unroll
-        for (int t = 0; t < TRIPS; t++) xr[t] = *reinterpret_cast<const float4v *>(xrow + k0 + kb + 64 * t);
+        for (int t = 0; t < TRIPS; t++) xr[t] = at(xrow, k0 + kb + ks * t);
         float4v gm[NORM ? TRIPS : 1];
         if constexpr (NORM) {
 #pragma unroll
-            for (int t = 0; t < TRIPS; t++) gm[t] = *reinterpret_cast<const float4v *>(nf.gamma + k0 + kb + 64 * t);
+            for (int t = 0; t < TRIPS; t++) gm[t] = at(nf.gamma, k0 + kb + ks * t);
         }
 #pragma unroll
         for (int c = 0; c < 2; c++) {
             float4v w[TRIPS];
 #pragma unroll
-            for (int t = 0; t < TRIPS; t++) w[t] = *reinterpret_cast<const float4v *>(wrow[c] + k0 + kb + 64 * t);
+            for (int t = 0; t < TRIPS; t++) w[t] = at(wrow[c], k0 + kb + ks * t);
             if constexpr (NORM) {
                 if (c == 0) {
 #pragma unroll
@@ -1236,11 +1257,15 @@ __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_cols_gated_kerne
     static_assert(TRIPS == 8 || TRIPS == 4, "chunks of 2048 or 1024");
     const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x % 64;
     const uint32_t j = lane % 4, b = lane / 4;
-    const uint32_t kb = wave * (TRIPS * 64) + b * 4; // this lane's k: kb + 64 t
+    uint32_t kb, ks; // this lane's k: kb + ks t (beyond K, in a chunk that K does not fill: zeros)
+    xreg_lane_k<TRIPS>(a.K, wave, b, kb, ks);
     const uint32_t *xrow = a.A + (int64_t)min(j, a.M - 1) * a.a_sm;
     float4v xr[TRIPS];
 #pragma unroll
-    for (int t = 0; t < TRIPS; t++) xr[t] = *reinterpret_cast<const float4v *>(xrow + kb + 64 * t);
+    for (int t = 0; t < TRIPS; t++) {
+        xr[t] = (float4v){0.f, 0.f, 0.f, 0.f};
+        if (kb + ks * t < a.K) xr[t] = *reinterpret_cast<const float4v *>(xrow + kb + ks * t);
+    }
     float pv[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     float4v gm[NORM ? TRIPS : 1];
     if constexpr (NORM) {
@@ -1250,7 +1275,10 @@ __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_cols_gated_kerne
             if (i < nf.blocks * 4) pv[u] = nf.partials[i];
         }
 #pragma unroll
-        for (int t = 0; t < TRIPS; t++) gm[t] = *reinterpret_cast<const float4v *>(nf.gamma + kb + 64 * t);
+        for (int t = 0; t < TRIPS; t++) {
+            gm[t] = (float4v){0.f, 0.f, 0.f, 0.f};
+            if (kb + ks * t < a.K) gm[t] = *reinterpret_cast<const float4v *>(nf.gamma + kb + ks * t);
+        }
     }
     __shared__ float part[2][4][32];
     __shared__ float nsum[4][4];
@@ -1259,7 +1287,10 @@ __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_cols_gated_kerne
     auto ask = [&](float4v (&w)[TRIPS], const uint32_t *base, uint32_t n0) {
         const uint32_t *row = base + (int64_t)min(n0 + j, a.N - 1) * a.b_sn + kb;
 #pragma unroll
-        for (int t = 0; t < TRIPS; t++) w[t] = __builtin_nontemporal_load(reinterpret_cast<const float4v *>(row + 64 * t));
+        for (int t = 0; t < TRIPS; t++) {
+            w[t] = (float4v){0.f, 0.f, 0.f, 0.f};
+            if (kb + ks * t < a.K) w[t] = __builtin_nontemporal_load(reinterpret_cast<const float4v *>(row + ks * t));
+        }
     };
     auto multiply = [&](float4v &sum, const float4v (&w)[TRIPS]) {
 #pragma unroll
@@ -1688,14 +1719,15 @@ int launch_matmul_gated(cg_backend *be, const cg_tensor *x, const cg_tensor *yg,
     if (!rc) rc = make_mm_args(x, yu, c, &au, &fu);
     if (rc) return rc;
     const bool vec = ag.a_vec && ag.b_vec && au.b_vec && ag.a_sk == 1 && ag.K % 4 == 0;
-    if (fg.batch != 1 || fu.batch != 1 || ag.M > 4 || ag.b_sk != 1 || au.b_sk != 1 || !vec || ag.K <= 256 || ag.N < 2048 ||
+    if (fg.batch != 1 || fu.batch != 1 || ag.M > 4 || ag.b_sk != 1 || au.b_sk != 1 || !vec || ag.K <= 256 || ag.N < 512 ||
         au.N != ag.N || au.K != ag.K || au.M != ag.M || au.b_sn != ag.b_sn)
         return kDeclined;
     if (nf && xreg_trips(ag.K) == 0) return kDeclined;
     const bool short_chunks = xreg_trips(ag.K) == 4; // K a multiple of 1024 but not of 2048
     ProfScope prof(be, CG_K_GEMM_SKINNY, distinct_bytes(x) + distinct_bytes(yg) + distinct_bytes(yu) + distinct_bytes(out));
     const dim3 ggrid((ag.N + 3) / 4);
-    if ((int)ag.K == xreg_trips(ag.K) * 256) { // one chunk of k: see skinny_kt_mfma_xreg_cols_body
+    if (xreg_trips(ag.K) == 0) return kDeclined;
+    if ((int)ag.K <= xreg_trips(ag.K) * 256) { // one chunk of k (full or not): see skinny_kt_mfma_xreg_cols_gated_kernel
         NormFuse none;
         memset(&none, 0, sizeof none);
         const uint32_t groups = (ag.N + 3) / 4, iters = xreg_cols_iters(groups);
@@ -1728,7 +1760,7 @@ int launch_matmul_residual(cg_backend *be, const cg_tensor *x, const cg_tensor *
     int rc = make_mm_args(x, y, static_cast<uint32_t *>(out->buf->ptr) + out->offset, &a, &f);
     if (rc) return rc;
     const bool vec = a.a_vec && a.b_vec && a.a_sk == 1 && a.K % 4 == 0;
-    if (f.batch != 1 || a.M > 8 || a.b_sk != 1 || !vec || a.K <= 256 || a.N < 1024 || a.N >= 8192) return kDeclined;
+    if (f.batch != 1 || a.M > 8 || a.b_sk != 1 || !vec || a.K <= 256 || a.N < 512 || a.N >= 8192) return kDeclined;
     MmResidual r;
     for (int t = 0; t < 4; t++) r.term[t] = t == slot || t >= nterms ? nullptr : terms[t];
     r.slot = (uint32_t)slot;

@@ -151,7 +151,7 @@ Pending::~Pending() {
 
 // Is x (still) the deferred program  h / pow(sum(h * h) / n + eps, e) * gamma  over the rows of a residual stream h
 // [1..4 rows, K] whose kernel left the partial sums of squares (Buffer::side)?  Then a decode-time product can apply
-// the norm while it loads h (K a multiple of 1024) and the norm needs no launch.  Fills nf and the stand-in tensor
+// the norm while it loads h (K a multiple of 4 above 256) and the norm needs no launch.  Fills nf and the stand-in tensor
 // h (a borrowed view of the leaf's buffer: set h->buf to null before it goes out of scope).
 static bool norm_fuse_of(const cg_tensor *x, NormFuse *nf, cg_tensor *h) {
     static const uint8_t code[7][4] = {{kMul, 0, 0, 0},   {kRowSum, 8, 8, 8}, {kDiv, 9, 1, 9},  {kAdd, 10, 2, 10},
@@ -163,7 +163,7 @@ static bool norm_fuse_of(const cg_tensor *x, NormFuse *nf, cg_tensor *h) {
         if (p->ins[i].op != code[i][0] || p->ins[i].a != code[i][1] || p->ins[i].b != code[i][2] || p->ins[i].c != code[i][3]) return false;
     const int r = x->rank;
     const int64_t K = x->dims[r - 1], rows = K > 0 ? numel(x) / K : 0;
-    if (K <= 0 || K % 1024 != 0 || rows < 1 || rows > 4 || p->rowlen != K) return false;
+    if (K <= 256 || K % 4 != 0 || rows < 1 || rows > 4 || p->rowlen != K) return false;
     const LeafView &lh = p->leaf[0], &lg = p->leaf[4];
     if (lh.uniform || lh.pw || lh.lazy || !lh.buf || !lh.buf->side || lh.offset != 0 || (int64_t)lh.buf->side_blocks * 4 != K) return false;
     if (!p->leaf[1].uniform || !p->leaf[2].uniform || !p->leaf[3].uniform) return false;
@@ -208,7 +208,7 @@ static bool residual_sum_open(const cg_tensor *x) {
         if (lv.lazy && !lv.lazy->result) {
             const LazyMm *m = lv.lazy;
             const int64_t N = m->rank > 0 ? m->dims[m->rank - 1] : 0;
-            if (!m->groupable || m->rc.load() != 1 || m->rank != x->rank || N < 1024 || N >= 8192) return false;
+            if (!m->groupable || m->rc.load() != 1 || m->rank != x->rank || N < 512 || N >= 8192) return false;
             open++;
         } else if (!lv.lazy && !lv.buf) {
             return false;
@@ -1254,6 +1254,8 @@ static int ensure_concrete(cg_tensor *t) {
     if (t->split >= 0) { // a split-axis view becomes a plain dense tensor, in place
         std::lock_guard<std::recursive_mutex> lk(g_lazy_mu);
         if (t->split < 0) return CG_OK;
+        const hipError_t she = hipSetDevice(t->be->device);
+        if (she != hipSuccess) return hip_fail(she, "hipSetDevice");
         cg_tensor *m;
         int rc = materialize(t->be, t, &m);
         if (rc) return rc;
@@ -1491,7 +1493,7 @@ static int defer_elementwise(cg_backend *be, int op, cg_dtype in_dt, cg_dtype ou
             if (splice[k]) {
                 reg[k] = splice_program(p, x->pend, sdims, rank, rl > 0 && !x->pend->reduced);
             } else {
-                LeafView lv;
+                LeafView lv{};
                 lv.uniform = x->uniform;
                 lv.ubits = x->ubits;
                 if (!x->uniform) {
@@ -1553,7 +1555,7 @@ static int defer_reduce(cg_backend *be, int kind, cg_tensor *x, const int64_t *o
         src = (uint8_t)(kMaxLeaves + p->ninstr - 1);
     } else {
         p = new Pending;
-        LeafView lv;
+        LeafView lv{};
         lv.uniform = x->uniform;
         lv.ubits = x->ubits;
         if (!x->uniform) {
@@ -2483,7 +2485,7 @@ int cg_cast(cg_backend *b, cg_tensor *x, cg_dtype target, cg_tensor **out) {
         *out = x;
         return CG_OK;
     }
-    CG_HIP(hipSetDevice(b->device));
+    if (!b->fuse) CG_HIP(hipSetDevice(b->device)); // (deferred results: whoever computes them makes the device current)
     if (is_f(x->dt) && is_f(target)) {
         // between floating-point dtypes: the words stay, a narrower target rounds them
         int rc = retag(b, x, target, out);
@@ -2517,7 +2519,7 @@ int cg_unary(cg_backend *b, cg_unary_op op, cg_tensor *x, cg_tensor **out) {
         *out = new_uniform(b, x->dt, x->dims, x->rank, r);
         return CG_OK;
     }
-    CG_HIP(hipSetDevice(b->device));
+    if (!b->fuse) CG_HIP(hipSetDevice(b->device)); // (deferred results: whoever computes them makes the device current)
     const cg_tensor *ins[1] = {x};
     const cg_dtype dt = x->dt;
     int rc = ew_result(b, kNeg + (int)op, dt, dt, x, ins, 1, out);
@@ -2545,7 +2547,7 @@ int cg_binary(cg_backend *b, cg_binary_op op, cg_tensor *x, cg_tensor *y, cg_ten
             return CG_OK;
         }
     }
-    CG_HIP(hipSetDevice(b->device));
+    if (!b->fuse) CG_HIP(hipSetDevice(b->device)); // (deferred results: whoever computes them makes the device current)
     const cg_tensor *ins[2] = {x, y};
     const cg_dtype dt = x->dt;
     int rc = ew_result(b, kAdd + (int)op, dt, dt, x, ins, 2, out);
@@ -2562,7 +2564,7 @@ int cg_where(cg_backend *b, cg_tensor *mask, cg_tensor *x, cg_tensor *y, cg_tens
     if (!supported(x->dt)) return fail(CG_ERR_UNSUPPORTED, "%s", kTodo);
     if (mask->dt != x->dt || y->dt != x->dt) return fail(CG_ERR_DTYPE, "TypeError: mixed dtypes in where");
     if (!same_shape(mask, x) || !same_shape(x, y)) return fail(CG_ERR_SHAPE, "Shape mismatch in operation");
-    CG_HIP(hipSetDevice(b->device));
+    if (!b->fuse) CG_HIP(hipSetDevice(b->device)); // (deferred results: whoever computes them makes the device current)
     const cg_tensor *ins[3] = {mask, x, y};
     return ew_result(b, kWhere, x->dt, x->dt, x, ins, 3, out);
 }
@@ -2595,13 +2597,13 @@ static int matmul_entry(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **o
     for (int i = 0; i < r - 2; i++) od[i] = x->dims[i];
     od[r - 2] = x->dims[r - 2];
     od[r - 1] = y->dims[r - 1];
-    CG_HIP(hipSetDevice(b->device));
     // deferred operands are computed now; a split axis may stay if it is a batch axis (the GEMM walks
     // its two parts as separate batch axes) and the two operands do not disagree about it
     int rc = CG_OK;
     if (b->fuse && x->pend && x->rc.load() == 1 && x->pend->nleaf > 0 && x->pend->leaf[0].lazy &&
         !x->pend->leaf[0].lazy->result && !y->pend && !y->uniform && (y->split < 0 || y->split < r - 2)) {
         // soft-max over a lazy q.K^T, times V: one fused attention pass if the kernel takes the shapes
+        CG_HIP(hipSetDevice(b->device));
         LazyMm *m = x->pend->leaf[0].lazy;
         cg_tensor *o;
         rc = new_dense(b, x->dt, od, r, &o);
@@ -2665,7 +2667,7 @@ static int matmul_entry(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **o
             memcpy(t->dims, od, sizeof t->dims);
             set_row_major(t);
             Pending *p = new Pending;
-            LeafView lv;
+            LeafView lv{};
             lv.lazy = m;
             memcpy(lv.strides, t->strides, sizeof lv.strides);
             add_leaf(p, lv, od, r);
@@ -2679,6 +2681,7 @@ static int matmul_entry(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **o
             return CG_OK;
         }
     }
+    CG_HIP(hipSetDevice(b->device));
     cg_tensor *o;
     rc = new_dense(b, x->dt, od, r, &o);
     if (rc) return rc;
@@ -2705,13 +2708,13 @@ static int reduce_entry(cg_backend *b, int kind, const char *what, cg_tensor *x,
     int64_t od[kMaxRank];
     memcpy(od, x->dims, sizeof od);
     od[x->rank - 1] = 1;
-    CG_HIP(hipSetDevice(b->device));
     cg_tensor *o;
     int rc;
     if (b->fuse && kind != kArgmax && numel(x) > 0) {
         rc = defer_reduce(b, kind, x, od, out);
         if (rc || *out) return rc;
     }
+    CG_HIP(hipSetDevice(b->device));
     rc = new_dense(b, kind == kArgmax ? CG_U32 : x->dt, od, x->rank, &o);
     if (rc) return rc;
     if (numel(o) > 0) {
@@ -3033,7 +3036,7 @@ int cg_concat(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor *
         // Along the last axis the result can stay deferred as one piecewise leaf when each
         // operand is a plain view, or the negation of one (rotate_half of the rotary embedding,
         // helpers/rope.rs:423-427): its consumer then reads both halves in place.
-        LeafView lv;
+        LeafView lv{};
         // a part may also be a view of a decode-time product that has not been computed yet: it stays open, so that a
         // rotary embedding over it can still run in the product's own store (see try_rope_stores)
         auto part = [&](cg_tensor *t, Buffer **buf, LazyMm **lazy, int64_t *strides, int64_t *offset, bool *neg) {

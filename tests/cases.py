@@ -1182,7 +1182,7 @@ for _B, _K, _N in ((4, 512, 4096), (1, 2048, 8192), (3, 388, 4100), (8, 512, 409
 
 
 # ---- residual adds around a decode-time linear layer (the o / down projection of a decoder layer) -------------------
-for _B, _K, _N in ((4, 512, 2048), (8, 260, 2052), (1, 1024, 4096), (4, 512, 512), (4, 2048, 2048), (3, 4096, 2052), (2, 2048, 4100), (1, 3072, 2048), (4, 1024, 2052)):
+for _B, _K, _N in ((4, 512, 2048), (8, 260, 2052), (1, 1024, 4096), (4, 512, 512), (4, 512, 256), (4, 2048, 2048), (3, 4096, 2052), (2, 2048, 4100), (1, 3072, 2048), (4, 1024, 2052)):
     @case(f"linear_residual_B{_B}_K{_K}_N{_N}", "red")
     def _(B=_B, K=_K, Nn=_N):
         """Sums of three dense terms and a lazy product in the two association orders and every operand
@@ -1369,7 +1369,10 @@ def _np_rope(x, cos, sin):
 
 
 for _B, _K, _kvh, _rep, _T, _hd, _normed in ((4, 2048, 8, 4, 300, 64, True), (1, 1024, 2, 2, 256, 128, False), (2, 2048, 4, 1, 131, 64, True),
-                                              (3, 512, 4, 2, 200, 64, False), (4, 2048, 2, 4, 512, 32, False)):
+                                              (3, 512, 4, 2, 200, 64, False), (3, 256, 4, 2, 200, 64, False), (4, 2048, 2, 4, 512, 32, False),
+                                              # hidden sizes that are no multiple of 1024: a ragged chunk of k in the fused store
+                                              (1, 576, 3, 3, 200, 64, True), (4, 576, 3, 3, 300, 64, False), (2, 1536, 4, 2, 131, 64, True),
+                                              (3, 2560, 2, 4, 260, 128, True)):
     @case(f"decode_qkv_rope_append_B{_B}_K{_K}_kv{_kvh}_rep{_rep}_T{_T}_hd{_hd}{'_normed' if _normed else ''}", "red",
           (lambda n=2 * 3: [np.float64(4.0)] * n))   # projections of order one, rows of the caches likewise: 1e-3 of 4
     def _(B=_B, K=_K, kvh=_kvh, rep=_rep, T=_T, hd=_hd, normed=_normed):
@@ -1541,8 +1544,10 @@ def _rmsnorm_ops(be, h, gamma, n, shp):
     return be.mul(be.div(h, be.broadcast(rms.move(), shp).move()).move(), be.broadcast(gamma.move(), shp).move())
 
 
-for _B, _H, _F, _read_norms in ((4, 2048, 4096, False), (2, 2048, 4096, True), (3, 4096, 8192, False), (4, 512, 4096, False), (1, 2048, 4096, False),
-                                 (1, 1024, 3072, False), (4, 3072, 4096, False)):
+for _B, _H, _F, _read_norms in ((4, 2048, 4096, False), (2, 2048, 4096, True), (3, 4096, 8192, False), (4, 512, 4096, False), (4, 256, 4096, False), (1, 2048, 4096, False),
+                                 (1, 1024, 3072, False), (4, 3072, 4096, False),
+                                 # hidden and MLP sizes that are no multiples of 1024 (ragged chunks of k, few columns)
+                                 (1, 576, 1536, False), (4, 576, 1536, True), (2, 1536, 2560, False), (3, 2560, 6912, False)):
     @case(f"decoder_block_B{_B}_H{_H}_F{_F}{'_norms_read' if _read_norms else ''}", "red",
           (lambda n=5 + 2 * _read_norms: [np.float64(4.0)] * n))   # every output is of order one: 1e-3 of 4
     def _(B=_B, H=_H, F=_F, read_norms=_read_norms):

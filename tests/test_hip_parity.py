@@ -187,13 +187,15 @@ def test_decode_attention_runs_as_one_fused_pass(hip):
 def test_norms_run_in_the_products_behind_them(hip):
     """The dense part of a decoder layer at decode time (hidden 2048, 4 rows): four skinny-product launches — o
     projection + residual add, gate / up / SiLU with the first norm in its loads, down projection + residual add,
-    q / k / v with the second norm in their loads — and no launch for the norms or the adds.  With hidden 512
-    the products' kernels do not take the norms, which then run on their own: same values either way."""
+    q / k / v with the second norm in their loads — and no launch for the norms or the adds (hidden 512
+    and up, any multiple of 4).  With hidden 256 the products' kernels do not take the norms, which then run on their own:
+    same values either way."""
     from catgrad_amd import _abi as A
     from cases import by_name
 
     classes = (A.K_GEMM_SKINNY, A.K_ELEMENTWISE, A.K_REDUCE)
-    for name, fused in (("decoder_block_B4_H2048_F4096", True), ("decoder_block_B1_H1024_F3072", True), ("decoder_block_B4_H512_F4096", False)):
+    for name, fused in (("decoder_block_B4_H2048_F4096", True), ("decoder_block_B1_H1024_F3072", True), ("decoder_block_B4_H512_F4096", True),
+                        ("decoder_block_B1_H576_F1536", True), ("decoder_block_B4_H256_F4096", False)):
         c = by_name(name)
         hip.sync()
         for cls in classes:
@@ -206,7 +208,7 @@ def test_norms_run_in_the_products_behind_them(hip):
         if fused:
             assert counts == (4, 0, 0), (name, counts)
         else:
-            assert counts[0] == 4 and counts[1] + counts[2] >= 2, (name, counts)
+            assert counts[0] >= 4 and counts[1] + counts[2] >= 2, (name, counts)
         for g, e in zip(got, c.expect()):
             np.testing.assert_allclose(g, e, rtol=1e-3, atol=4e-3)
 
@@ -215,12 +217,13 @@ def test_programs_absorbed_by_decode_time_products(hip):
     """gate and up projection of a decode step plus the SiLU program between them and the next product:
     one skinny-product launch and no element-wise launch; a pair the kernel does not take (8 rows) runs as
     a grouped product plus the compiled program and gives the same kind of result.  Likewise the residual
-    adds around a product (eight sums per case): absorbed at 2048 columns, separate launches at 512."""
+    adds around a product (eight sums per case): absorbed from 512 columns on, separate launches at 256."""
     from catgrad_amd import _abi as A
     from cases import by_name
 
     for name, launches in (("linear_gated_B4_K512_N4096", (1, 0)), ("linear_gated_B8_K512_N4096", (1, 1)),
-                           ("linear_residual_B4_K512_N2048", (8, 0)), ("linear_residual_B4_K512_N512", (8, 8))):
+                           ("linear_residual_B4_K512_N2048", (8, 0)), ("linear_residual_B4_K512_N512", (8, 0)),
+                           ("linear_residual_B4_K512_N256", (8, 8))):
         c = by_name(name)
         hip.sync()
         for cls in (A.K_GEMM_SKINNY, A.K_ELEMENTWISE):
@@ -239,13 +242,15 @@ def test_rotary_embedding_and_cache_append_run_in_the_products_store(hip):
     """Two decode steps of an attention block (hidden 2048, 4 rows; hidden 1024, 1 row): the element-wise launches
     that remain are the two moves of the caches into buffers with room (first append) and the four read-backs of
     cache rows the case asks for; the rotary embedding of q and k and the writes of the new k / v rows cost none.
-    With hidden 512 the products' kernel does not take the store and they run as a launch of their own per step."""
+    With hidden 256 the products' kernel does not take the store and they run as a launch of their own per step."""
     from catgrad_amd import _abi as A
     from cases import by_name
 
     for name, ew in (("decode_qkv_rope_append_B4_K2048_kv8_rep4_T300_hd64_normed", 6),
                      ("decode_qkv_rope_append_B1_K1024_kv2_rep2_T256_hd128", 6),
-                     ("decode_qkv_rope_append_B3_K512_kv4_rep2_T200_hd64", None)):
+                     ("decode_qkv_rope_append_B3_K512_kv4_rep2_T200_hd64", 6),
+                     ("decode_qkv_rope_append_B1_K576_kv3_rep3_T200_hd64_normed", 6),
+                     ("decode_qkv_rope_append_B3_K256_kv4_rep2_T200_hd64", None)):
         c = by_name(name)
         hip.sync()
         hip.profile_enable(A.K_ELEMENTWISE, 1)
