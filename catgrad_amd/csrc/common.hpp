@@ -101,6 +101,9 @@ struct cg_backend {
     // decode-time attention over a cache of at least this many positions runs a workgroup per (KV head, segment of the
     // cache) (CG_ATTN_SEG_FROM, read when the backend is created; 0: never)
     int64_t attn_seg_from = 6001;
+    bool narrow_storage = true;  // tensors of the narrow float dtypes keep 2- / 1-byte elements in memory (CG_NARROW_STORAGE=0: 32-bit words)
+    int64_t narrow_from = 65536; // ... from this many elements on (CG_NARROW_FROM); smaller tensors stay 32-bit words: the kernels of a
+                                 // decode step, which address words, never meet a narrow operand that way
     bool trace_programs = false; // CG_TRACE_PROGRAMS=1: print each distinct deferred program once, to stderr
     cg::ProfClass prof[CG_K_CLASSES];
     std::vector<cg::ProfPending> prof_pending;
@@ -121,6 +124,16 @@ struct RowStore {
     std::vector<int64_t> fill;
 };
 
+// How the elements of a buffer lie in memory.  32-bit words (f32 and u32 values; also values of the narrow float dtypes,
+// each held exactly in an f32 word), or the narrow dtypes' own patterns: 2 bytes per element for bfloat16 / binary16, 1 for
+// fp8 (E4M3).  A format is a property of the BUFFER, not of the dtype tag of a tensor that views it: what a narrow buffer
+// holds are exactly representable values, so a tensor of any floating-point dtype may view it.  Kernels either take the
+// format from their operand descriptors (element-wise kernels, fused programs, copies, gathers, the narrow-operand matrix
+// products) or ask for words (device_ptr), which a narrow buffer answers with a widened copy that it makes once and keeps.
+enum : int { kFmtWords = 0, kFmtBF16 = 1, kFmtF16 = 2, kFmtF8 = 3 };
+inline int fmt_of(cg_dtype d) { return d == CG_BF16 ? kFmtBF16 : d == CG_F16 ? kFmtF16 : d == CG_F8 ? kFmtF8 : kFmtWords; }
+inline size_t fmt_bytes(int fmt) { return fmt == kFmtWords ? 4 : fmt == kFmtF8 ? 1 : 2; }
+
 inline uint64_t next_buffer_id() {
     static std::atomic<uint64_t> n{1};
     return n.fetch_add(1);
@@ -132,6 +145,9 @@ struct Buffer {
     void *ptr = nullptr;
     size_t cls = 0;
     int64_t elems = 0;           // elements in use from the start of the buffer (grows with in-place appends); <= cls / 4
+    int fmt = kFmtWords;         // element format (see above); a narrow buffer is never appended to or written in place
+    Buffer *wide = nullptr;      // retained: this narrow buffer's elements as 32-bit words, made when a kernel that only
+                                 // reads words first needed them (device_ptr)
     cg_backend *be = nullptr;
     RowStore *rs = nullptr;      // owned
     bool constant = false;       // the contents depend on constants only (iota, programs over such buffers)
@@ -212,14 +228,23 @@ void release(cg_tensor *t);
 inline void retain(cg_tensor *t) { t->rc.fetch_add(1, std::memory_order_relaxed); }
 // Fresh row-major tensor with pool memory (none when numel == 0).
 // `reserve_elems` asks for a buffer with room for at least that many elements.
-int new_dense(cg_backend *be, cg_dtype dt, const int64_t *dims, int rank, cg_tensor **out, int64_t reserve_elems = 0);
+// `fmt`: the element format of the new buffer (a narrow one only for results whose producer stores that format).
+int new_dense(cg_backend *be, cg_dtype dt, const int64_t *dims, int rank, cg_tensor **out, int64_t reserve_elems = 0,
+              int fmt = kFmtWords);
+// The narrowest format that results of dtype dt with n elements are stored in (small results stay words: the kernels of a
+// decode step address words).
+int result_fmt(const cg_backend *be, cg_dtype dt, int64_t n);
 // Fresh uniform tensor (no memory).
 cg_tensor *new_uniform(cg_backend *be, cg_dtype dt, const int64_t *dims, int rank, uint32_t bits);
 // New handle sharing t's buffer and metadata.
 cg_tensor *new_view(const cg_tensor *t);
-// Device address of element 0 of the view; allocates the 4-byte backing word of a
-// uniform tensor on first use.
+// Device address of element 0 of the view, for kernels that READ 32-bit words; allocates the 4-byte backing word of a
+// uniform tensor on first use.  A view of a narrow buffer is answered from the buffer's widened copy (made on first
+// use, kept with the buffer).  Never for a destination: a kernel that writes takes device_ptr_fmt.
 int device_ptr(const cg_tensor *t, const void **ptr);
+// The same in the buffer's own format: *fmt says how the elements behind *ptr lie in memory.
+int device_ptr_fmt(const cg_tensor *t, const void **ptr, int *fmt);
+inline bool is_narrow_buf(const Buffer *b) { return b && b->fmt != kFmtWords; }
 
 // ---- magic-number division for 32-bit indices (Granlund-Montgomery round-up) ----
 struct FastDiv {
@@ -236,6 +261,7 @@ struct Operand {
     int64_t is;                // element stride of the inner axis
     uint32_t uniform;          // 1: take `ubits`, never dereference ptr
     uint32_t ubits;
+    uint32_t fmt;              // element format of the memory behind ptr (kFmtWords, ...): loads widen, stores narrow
 };
 
 struct EwGeom {
@@ -356,6 +382,7 @@ struct ViewDesc {
     uint32_t ubits;
     const char *ptr; // device address of the view's first element (unused when uniform)
     int64_t vec_period = 0; // > 0: 16-byte vectors are only allowed if this divides by 4 (a piecewise leaf's split)
+    int fmt = kFmtWords;    // element format of the memory behind ptr
 };
 // Collapses the iteration space shared by `n` views of shape `dims` (v[0] is the output)
 // and fills geometry + operands.  keep_last_axis: never merge the last axis into the one
@@ -420,6 +447,8 @@ int launch_fill_word(cg_backend *be, void *ptr, uint32_t bits);
 int launch_bf16_widen(cg_backend *be, const void *src, void *dst, uint64_t n);
 // binary16 bit patterns widened to f32
 int launch_f16_widen(cg_backend *be, const void *src, void *dst, uint64_t n);
+// n elements of format `fmt` widened to 32-bit words
+int launch_widen(cg_backend *be, int fmt, const void *src, void *dst, uint64_t n);
 // f32 words holding bfloat16 / binary16 values -> their 16-bit patterns (exact)
 int launch_narrow16(cg_backend *be, cg_dtype dt, const void *src, void *dst, uint64_t n);
 // fp8 (E4M3) bytes <-> 32-bit words holding the same values

@@ -13,11 +13,91 @@ __device__ __forceinline__ uint32_t fastdiv(uint32_t n, const FastDiv &f) {
 __device__ __forceinline__ float asf(uint32_t b) { return __uint_as_float(b); }
 __device__ __forceinline__ uint32_t asu(float f) { return __float_as_uint(f); }
 
+// The f32 word of one element of a narrow format, and back (exact: a word that is stored narrow holds a value of the format).
+__device__ __forceinline__ uint32_t f8_word_of_dev(uint8_t b);
+__device__ __forceinline__ uint8_t f8_byte_of_dev(uint32_t u);
+
+// VEC consecutive elements (element stride o.is) of a NARROW operand, widened to f32 words.
+template <int VEC>
+__device__ __forceinline__ void load_narrow(const Operand &o, int64_t off, uint32_t (&r)[VEC]) {
+    if (o.fmt == kFmtF8) {
+        const uint8_t *p = reinterpret_cast<const uint8_t *>(o.ptr) + off;
+        if (VEC == 4 && o.is == 1) {
+            const uint32_t t = *reinterpret_cast<const uint32_t *>(p);
+#pragma unroll
+            for (int j = 0; j < VEC; j++) r[j] = f8_word_of_dev((uint8_t)(t >> (8 * j)));
+        } else if (o.is == 0) {
+            const uint32_t t = f8_word_of_dev(*p);
+#pragma unroll
+            for (int j = 0; j < VEC; j++) r[j] = t;
+        } else {
+#pragma unroll
+            for (int j = 0; j < VEC; j++) r[j] = f8_word_of_dev(p[(int64_t)j * o.is]);
+        }
+        return;
+    }
+    const uint16_t *p = reinterpret_cast<const uint16_t *>(o.ptr) + off;
+    uint16_t h[VEC];
+    if (VEC == 4 && o.is == 1) {
+        const uint2 t = *reinterpret_cast<const uint2 *>(p);
+        h[0] = (uint16_t)t.x;
+        h[1 % VEC] = (uint16_t)(t.x >> 16);
+        h[2 % VEC] = (uint16_t)t.y;
+        h[3 % VEC] = (uint16_t)(t.y >> 16);
+    } else if (o.is == 0) {
+        const uint16_t t = *p;
+#pragma unroll
+        for (int j = 0; j < VEC; j++) h[j] = t;
+    } else {
+#pragma unroll
+        for (int j = 0; j < VEC; j++) h[j] = p[(int64_t)j * o.is];
+    }
+#pragma unroll
+    for (int j = 0; j < VEC; j++)
+        r[j] = o.fmt == kFmtBF16 ? (uint32_t)h[j] << 16 : __float_as_uint(__half2float(__ushort_as_half(h[j])));
+}
+
+// f32 words that hold values of a narrow format, stored as that format's patterns.
+template <int VEC>
+__device__ __forceinline__ void store_narrow(const Operand &o, int64_t off, const uint32_t (&r)[VEC]) {
+    if (o.fmt == kFmtF8) {
+        uint8_t *p = reinterpret_cast<uint8_t *>(const_cast<char *>(o.ptr)) + off;
+        if (VEC == 4 && o.is == 1) {
+            uint32_t t = 0;
+#pragma unroll
+            for (int j = 0; j < VEC; j++) t |= (uint32_t)f8_byte_of_dev(r[j]) << (8 * j);
+            *reinterpret_cast<uint32_t *>(p) = t;
+        } else {
+#pragma unroll
+            for (int j = 0; j < VEC; j++) p[(int64_t)j * o.is] = f8_byte_of_dev(r[j]);
+        }
+        return;
+    }
+    uint16_t h[VEC];
+#pragma unroll
+    for (int j = 0; j < VEC; j++)
+        h[j] = o.fmt == kFmtBF16 ? (uint16_t)(r[j] >> 16) : __half_as_ushort(__float2half_rn(__uint_as_float(r[j])));
+    uint16_t *p = reinterpret_cast<uint16_t *>(const_cast<char *>(o.ptr)) + off;
+    if (VEC == 4 && o.is == 1) {
+        uint2 t;
+        t.x = (uint32_t)h[0] | ((uint32_t)h[1 % VEC] << 16);
+        t.y = (uint32_t)h[2 % VEC] | ((uint32_t)h[3 % VEC] << 16);
+        *reinterpret_cast<uint2 *>(p) = t;
+    } else {
+#pragma unroll
+        for (int j = 0; j < VEC; j++) p[(int64_t)j * o.is] = h[j];
+    }
+}
+
 template <int VEC, bool STREAM = false>
 __device__ __forceinline__ void load_words(const Operand &o, int64_t off, uint32_t (&r)[VEC]) {
     if (o.uniform) {
 #pragma unroll
         for (int j = 0; j < VEC; j++) r[j] = o.ubits;
+        return;
+    }
+    if (o.fmt != kFmtWords) { // (the same for every lane: the format is a launch parameter)
+        load_narrow<VEC>(o, off, r);
         return;
     }
     const uint32_t *p = reinterpret_cast<const uint32_t *>(o.ptr) + off;
@@ -42,6 +122,10 @@ __device__ __forceinline__ void load_words(const Operand &o, int64_t off, uint32
 // evicting the operands that are still being read.
 template <int VEC, bool STREAM = false>
 __device__ __forceinline__ void store_words(const Operand &o, int64_t off, const uint32_t (&r)[VEC]) {
+    if (o.fmt != kFmtWords) {
+        store_narrow<VEC>(o, off, r);
+        return;
+    }
     uint32_t *p = reinterpret_cast<uint32_t *>(const_cast<char *>(o.ptr)) + off;
     if (VEC == 4 && o.is == 1) {
         if (STREAM) {
@@ -109,6 +193,9 @@ __host__ __device__ __forceinline__ uint32_t f8_word_of(uint8_t b) {
     if (e != 0) return sign | ((e + 120u) << 23) | (m << 20);
     return sign | __builtin_bit_cast(uint32_t, (float)m * (1.0f / 512.0f));
 }
+
+__device__ __forceinline__ uint32_t f8_word_of_dev(uint8_t b) { return f8_word_of(b); }
+__device__ __forceinline__ uint8_t f8_byte_of_dev(uint32_t u) { return f8_byte_of(u); }
 
 // One scalar application of OP on raw 32-bit words.  F = operands are f32.
 template <int OP, bool F>

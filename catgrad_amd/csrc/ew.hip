@@ -249,6 +249,7 @@ __global__ __launch_bounds__(kBlock) void transpose_copy_kernel(const TransposeA
 static int try_transpose_copy(cg_backend *be, const EwArgs &a) {
     const EwGeom &g = a.g;
     if (a.in[0].uniform || a.out.is != 1 || a.in[0].is == 1 || a.in[0].is == 0 || g.nouter < 1) return kDeclined;
+    if (a.in[0].fmt != kFmtWords || a.out.fmt != kFmtWords) return kDeclined; // (the tiles are 32-bit words)
     int td = -1; // the outer axis along which the source is unit-stride
     for (uint32_t d = 0; d < g.nouter; d++)
         if (a.in[0].os[d] == 1 && g.od[d] >= 16) td = (int)d;
@@ -403,6 +404,10 @@ int launch_narrow8(cg_backend *be, const void *src, void *dst, uint64_t n) {
     return e == hipSuccess ? CG_OK : hip_fail(e, "fp8 narrowing launch");
 }
 
+int launch_widen(cg_backend *be, int fmt, const void *src, void *dst, uint64_t n) {
+    return fmt == kFmtBF16 ? launch_bf16_widen(be, src, dst, n) : fmt == kFmtF16 ? launch_f16_widen(be, src, dst, n) : launch_f8_widen(be, src, dst, n);
+}
+
 int launch_fill_word(cg_backend *be, void *ptr, uint32_t bits) {
     hipLaunchKernelGGL(fill_word_kernel, dim3(1), dim3(1), 0, be->stream, static_cast<uint32_t *>(ptr), bits);
     hipError_t e = hipGetLastError();
@@ -418,13 +423,35 @@ int launch_gather(cg_backend *be, const cg_tensor *x, int dim, const cg_tensor *
     if (D > 0xFFFFFFFFll || inner > 0xFFFFFFFFll || outer * J > 0xFFFFFFFFll)
         return fail(CG_ERR_UNSUPPORTED, "index: extents above 2^32-1");
     const void *xp, *ip;
-    int rc = device_ptr(x, &xp);
+    int rc = device_ptr(idx, &ip);
     if (rc) return rc;
-    rc = device_ptr(idx, &ip);
-    if (rc) return rc;
-    int64_t istride = idx->uniform ? 0 : (idx->rank == 1 ? idx->strides[0] : 1);
+    // Rows of a narrow source that are whole 32-bit words long and start on one are gathered as those words (2 or 1 bytes
+    // per element moved); the result keeps the format, or, a small one, is widened afterwards.  Other narrow sources are
+    // read through their widened copy.
+    const int xf = x->buf ? x->buf->fmt : kFmtWords, of = out->buf->fmt;
+    const int64_t eb = (int64_t)fmt_bytes(xf);
+    const bool as_bytes = xf != kFmtWords && inner * eb % 4 == 0 && x->offset * eb % 4 == 0;
+    if (of != kFmtWords && !(as_bytes && of == xf)) return fail(CG_ERR_ARG, "internal error: gather into a narrow buffer of another layout");
+    void *tmp = nullptr;
+    size_t tmp_cls = 0;
     uint32_t *op = static_cast<uint32_t *>(out->buf->ptr);
-    bool vec4 = inner % 4 == 0 && reinterpret_cast<uintptr_t>(xp) % 16 == 0;
+    const int64_t out_elems = outer * J * inner;
+    if (as_bytes) {
+        int f;
+        rc = device_ptr_fmt(x, &xp, &f);
+        if (rc) return rc;
+        inner = inner * eb / 4;
+        if (of == kFmtWords) {
+            rc = be->pool.alloc((size_t)(out_elems * eb), &tmp, &tmp_cls);
+            if (rc) return rc;
+            op = static_cast<uint32_t *>(tmp);
+        }
+    } else {
+        rc = device_ptr(x, &xp);
+        if (rc) return rc;
+    }
+    int64_t istride = idx->uniform ? 0 : (idx->rank == 1 ? idx->strides[0] : 1);
+    bool vec4 = inner % 4 == 0 && reinterpret_cast<uintptr_t>(xp) % 16 == 0 && reinterpret_cast<uintptr_t>(op) % 16 == 0;
     uint32_t vec = vec4 ? 4 : 1;
     uint32_t ipr = (uint32_t)(inner / vec);
     uint64_t total = (uint64_t)outer * J * ipr;
@@ -440,6 +467,11 @@ int launch_gather(cg_backend *be, const cg_tensor *x, int dim, const cg_tensor *
                            static_cast<const uint32_t *>(ip), istride, op, (uint32_t)D, (uint32_t)inner,
                            make_fastdiv(ipr), ipr, make_fastdiv((uint32_t)J), (uint32_t)J, total, be->fault_dev);
     hipError_t e = hipGetLastError();
+    if (tmp) { // stream-ordered free: the widening kernel queued here reads it first
+        if (e == hipSuccess) rc = launch_widen(be, xf, tmp, out->buf->ptr, (uint64_t)out_elems);
+        be->pool.free(tmp, tmp_cls);
+        if (e == hipSuccess) return rc;
+    }
     return e == hipSuccess ? CG_OK : hip_fail(e, "gather launch");
 }
 

@@ -459,7 +459,7 @@ int fill_args(cg_backend *be, const Pending &p, const int64_t *dims, int rank, c
     int64_t out_strides[kMaxRank];
     if (out) {
         const void *op;
-        int rc = device_ptr(out, &op);
+        int rc = device_ptr_fmt(out, &op, &v[0].fmt); // (a destination: the buffer itself, in its own format)
         if (rc) return rc;
         v[0].strides = out->strides;
         v[0].uniform = false;
@@ -489,7 +489,8 @@ int fill_args(cg_backend *be, const Pending &p, const int64_t *dims, int rank, c
             if (lrc) return lrc;
             src = lv.lazy->result;
         }
-        v[l + 1].ptr = lv.uniform || !src ? nullptr : static_cast<const char *>(src->ptr) + lv.offset * 4;
+        v[l + 1].fmt = lv.uniform || !src ? kFmtWords : src->fmt;
+        v[l + 1].ptr = lv.uniform || !src ? nullptr : static_cast<const char *>(src->ptr) + lv.offset * (int64_t)fmt_bytes(v[l + 1].fmt);
         v[l + 1].vec_period = 0;
         if (lv.pw) { // its second part is planned as one more view, and the row axis stays on its own
             pw_leaf = l;
@@ -504,14 +505,15 @@ int fill_args(cg_backend *be, const Pending &p, const int64_t *dims, int rank, c
                 if (lrc) return lrc;
                 src2 = lv.lazy2->result;
             }
-            w.ptr = static_cast<const char *>(src2->ptr) + lv.offset2 * 4;
+            w.fmt = src2->fmt;
+            w.ptr = static_cast<const char *>(src2->ptr) + lv.offset2 * (int64_t)fmt_bytes(w.fmt);
             w.vec_period = lv.pw_split;
         }
         if (!lv.uniform) {
             double n = 1.0;
             for (int i = 0; i < rank; i++)
                 if (lv.strides[i] != 0 || dims[i] <= 1) n *= (double)dims[i];
-            if (!(lv.lazy && skip_lazy)) bytes += 4.0 * n;
+            if (!(lv.lazy && skip_lazy)) bytes += (double)fmt_bytes(v[l + 1].fmt) * n;
         }
     }
     Operand ops[kMaxViews + 1];

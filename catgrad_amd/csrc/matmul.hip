@@ -1571,19 +1571,13 @@ int fold_matmul(const cg_tensor *x, const cg_tensor *y, MmFold *f) {
 }
 
 // Kernel arguments of x . y -> c (row-major); the folded extents come back in *f.
-static int make_mm_args(const cg_tensor *x, const cg_tensor *y, void *c, MmArgs *ap, MmFold *fp) {
+// The geometry of x . y (everything of MmArgs but the operands' addresses and what depends on them).
+static int mm_geometry(const cg_tensor *x, const cg_tensor *y, void *c, MmArgs *ap, MmFold *fp) {
     MmArgs &a = *ap;
     memset(&a, 0, sizeof a);
-    const void *pa, *pb;
-    int rc = device_ptr(x, &pa);
-    if (rc) return rc;
-    rc = device_ptr(y, &pb);
-    if (rc) return rc;
-    a.A = static_cast<const uint32_t *>(pa);
-    a.B = static_cast<const uint32_t *>(pb);
     a.C = static_cast<uint32_t *>(c);
     MmFold &f = *fp;
-    rc = fold_matmul(x, y, &f);
+    int rc = fold_matmul(x, y, &f);
     if (rc) return rc;
     const int64_t M = f.M, N = f.N, K = f.K, batch = f.batch;
     const int w = f.nb;
@@ -1598,21 +1592,62 @@ static int make_mm_args(const cg_tensor *x, const cg_tensor *y, void *c, MmArgs 
     a.K = (uint32_t)K;
     a.nb = (uint32_t)w;
     a.batch = (uint32_t)batch;
-    bool a_al = reinterpret_cast<uintptr_t>(pa) % 16 == 0, b_al = reinterpret_cast<uintptr_t>(pb) % 16 == 0;
     for (int d = 0; d < w; d++) {
         a.bd[d] = (uint32_t)f.bd[d];
         a.bdiv[d] = make_fastdiv(a.bd[d]);
         a.a_bs[d] = f.a_bs[d];
         a.b_bs[d] = f.b_bs[d];
-        if (a.a_bs[d] % 4) a_al = false;
-        if (a.b_bs[d] % 4) b_al = false;
     }
-    // 16-byte loads run along the unit-stride axis; the other axis' stride must keep alignment
-    const bool a_kfast = a.a_sk == 1 || K == 1, a_mfast = !a_kfast && a.a_sm == 1;
-    const bool b_kfast = a.b_sk == 1 || K == 1, b_nfast = !b_kfast && a.b_sn == 1;
-    a.a_vec = a_al && ((a.a_sk == 1 && a.a_sm % 4 == 0) || (a_mfast && a.a_sk % 4 == 0));
-    a.b_vec = b_al && ((a.b_sk == 1 && a.b_sn % 4 == 0) || (b_nfast && a.b_sk % 4 == 0));
     return CG_OK;
+}
+
+// The 32-bit words of one operand (`left`: x, else y) and whether 16-byte loads may run along its unit-stride axis.  An
+// operand that lies in memory in a narrow format is read through its widened copy, unless the caller takes it as it
+// lies (`native`: then the address stays null and the operand counts as unaligned).
+static int mm_operand(const cg_tensor *t, bool left, bool native, MmArgs *ap) {
+    MmArgs &a = *ap;
+    const void *p = nullptr;
+    if (!native) {
+        int rc = device_ptr(t, &p);
+        if (rc) return rc;
+    }
+    bool al = !native && reinterpret_cast<uintptr_t>(p) % 16 == 0;
+    for (uint32_t d = 0; d < a.nb; d++)
+        if ((left ? a.a_bs[d] : a.b_bs[d]) % 4) al = false;
+    // 16-byte loads run along the unit-stride axis; the other axis' stride must keep alignment
+    if (left) {
+        a.A = static_cast<const uint32_t *>(p);
+        const bool kfast = a.a_sk == 1 || a.K == 1, mfast = !kfast && a.a_sm == 1;
+        a.a_vec = al && ((a.a_sk == 1 && a.a_sm % 4 == 0) || (mfast && a.a_sk % 4 == 0));
+    } else {
+        a.B = static_cast<const uint32_t *>(p);
+        const bool kfast = a.b_sk == 1 || a.K == 1, nfast = !kfast && a.b_sn == 1;
+        a.b_vec = al && ((a.b_sk == 1 && a.b_sn % 4 == 0) || (nfast && a.b_sk % 4 == 0));
+    }
+    return CG_OK;
+}
+
+static int make_mm_args(const cg_tensor *x, const cg_tensor *y, void *c, MmArgs *ap, MmFold *fp) {
+    int rc = mm_geometry(x, y, c, ap, fp);
+    if (!rc) rc = mm_operand(x, true, false, ap);
+    if (!rc) rc = mm_operand(y, false, false, ap);
+    return rc;
+}
+
+// The buffer that device_ptr's address of t lies in: the widened copy for a view of a narrow buffer.
+static Buffer *words_buffer(const cg_tensor *t) { return is_narrow_buf(t->buf) ? t->buf->wide : t->buf; }
+
+// May the [rows, K] view of t (row stride s_r, k stride s_k, in elements) be multiplied as it lies in memory, by the
+// kernels of narrow kind `kind` (1 bf16, 2 f16, 3 fp8)?  Its buffer holds that very format, k is contiguous and every row
+// starts on a 16-byte boundary.  dense: the rows must also follow each other without gaps.
+static bool native_rows(const cg_tensor *t, int kind, int64_t s_r, int64_t s_k, int64_t K, bool dense) {
+    if (!t->buf || t->uniform || t->buf->fmt != kind) return false;
+    const int64_t eb = (int64_t)fmt_bytes(kind);
+    if (s_k != 1 || s_r * eb % 16 != 0 || t->offset * eb % 16 != 0) return false;
+    return !dense || s_r == K;
+}
+static const void *native_ptr(const cg_tensor *t) {
+    return static_cast<const char *>(t->buf->ptr) + t->offset * (int64_t)fmt_bytes(t->buf->fmt);
 }
 
 int launch_matmul_group(cg_backend *be, const cg_tensor *x, const cg_tensor *const *ys, cg_tensor *const *outs, int n,
@@ -2031,7 +2066,7 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
     if (int frc = flush_deferred(be)) return frc;
     MmArgs a;
     MmFold f;
-    int rc = make_mm_args(x, y, out->buf->ptr, &a, &f);
+    int rc = mm_geometry(x, y, out->buf->ptr, &a, &f);
     if (rc) return rc;
     const int64_t M = f.M, N = f.N, K = f.K, batch = f.batch;
     const bool a_mfast = !(a.a_sk == 1 || K == 1) && a.a_sm == 1;
@@ -2040,7 +2075,48 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
     if (batch > 65535) return fail(CG_ERR_UNSUPPORTED, "matmul: more than 65535 batch entries after folding");
     const bool f32 = is_f(x->dt);
     const int half = x->dt == CG_BF16 ? 1 : x->dt == CG_F16 ? 2 : 0; // operands of the 16-bit matrix instructions
+    const int kind = half ? half : x->dt == CG_F8 ? 3 : 0;           // the narrow kernels' operand format (0: none)
     hipStream_t s = be->stream;
+
+    // ---- the tiled kernels' plan (used by the last branch below; here because it decides how operands are addressed) ----
+    // the narrow tile when the wide one would leave over a seventh of its columns empty, and when the product has at
+    // most one 128 x 128 tile per compute unit: twice the workgroups then fill the chip (4096 x 2048 x 512: 148 -> 83 us)
+    // or at least put two on a unit (8192 x 2048 x 512: 148 -> 145 us); with more tiles than that the wide one wins
+    // (env CG_GEMM_NARROW_BELOW=n moves the limit, for measurements)
+    const int64_t cols128 = (N + 127) / 128 * 128, cols64 = (N + 63) / 64 * 64;
+    static const int64_t narrow_below = [] { const char *e = getenv("CG_GEMM_NARROW_BELOW"); return e ? atoll(e) : 256ll; }();
+    const int64_t tiles128 = ((M + BM - 1) / BM) * (cols128 / 128) * (int64_t)batch;
+    const bool narrow = (cols128 * 7 > cols64 * 8 || (tiles128 <= narrow_below && N >= 128)) && !half; // (the 16-bit kernels come in the two square tiles)
+    const int bn = narrow ? 64 : 128;
+    // the 256 x 256 tile when it covers the chip at least once (env CG_GEMM_BIG=0 switches it off)
+    const uint64_t tiles_big = (uint64_t)((M + 255) / 256) * ((N + 255) / 256) * batch;
+    static const bool big_allowed = [] {
+        const char *e = getenv("CG_GEMM_BIG");
+        return !(e && e[0] == '0');
+    }();
+    const bool fits_big = big_allowed && !narrow && tiles_big >= 256 && M >= 256 && N >= 256;
+    // f32 words: since whole tiles are loaded without tests, two workgroups of the 128 x 128 tile per compute unit (two
+    // waves per SIMD covering each other's barriers) are as fast as one of the wide tile or faster — 137-138 against
+    // 134-135 TFLOP/s on the 1B shape's linear layers, and a partial last round costs a quarter as much (8192 x 2048 x
+    // 3072: 755 against 1015 us) — except with a k-contiguous left and a row-contiguous right operand (x.y: 1 % behind).
+    // The 16-bit and fp8 paths keep the wide tile (half the L2 bytes per flop, which is what bounds them).
+    const bool narrow_dtype = kind != 0;
+    const bool big = fits_big && (narrow_dtype || (!a_mfast && b_nfast));
+    // Operands of a narrow dtype in a product big enough for the 256 x 256 tile are multiplied from 2-byte / 1-byte
+    // patterns: as they lie in memory when their buffer holds that format, else narrowed in memory first (the right
+    // operand once per buffer) (env CG_GEMM_PACKED=0 switches it off).
+    const bool big_packed = f32 && K != 0 && M > 8 && kind && packed_narrow_ok() && big && batch == 1 && K % (kind == 3 ? 16 : 8) == 0 && x->buf && y->buf;
+
+    // ---- the operands' addresses -------------------------------------------------------------------------------------
+    const bool x_native = big_packed && native_rows(x, kind, a.a_sm, a.a_sk, K, false);
+    rc = mm_operand(x, true, x_native, &a);
+    if (rc) return rc;
+    // a decode-time linear layer of a narrow dtype reads its weight matrix at 2 or 1 bytes a weight (see below)
+    const bool skinny_packed = f32 && K != 0 && M <= (half ? 8 : 2) && packed_narrow_ok() && kind && batch == 1 && a.a_sk == 1 && a.a_vec &&
+                               a.a_sm % 4 == 0 && K % 16 == 0 && K >= 256 && N >= 64 && y->buf;
+    const bool y_native = (skinny_packed && native_rows(y, kind, a.b_sn, a.b_sk, K, true)) || (big_packed && native_rows(y, kind, a.b_sn, a.b_sk, K, false));
+    rc = mm_operand(y, false, y_native, &a);
+    if (rc) return rc;
     const double flop = 2.0 * (double)M * (double)N * (double)K * (double)batch;
     const double bytes = distinct_bytes(x) + distinct_bytes(y) + distinct_bytes(out);
     const bool simple = K == 0 || !f32, skinny = !simple && M <= 8 && (a.b_sk == 1 || a.b_sn == 1);
@@ -2052,16 +2128,15 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
             hipLaunchKernelGGL((simple_gemm_kernel<true>), grid, dim3(kThreads), 0, s, a);
         else
             hipLaunchKernelGGL((simple_gemm_kernel<false>), grid, dim3(kThreads), 0, s, a);
-    } else if (M <= (half ? 8 : 2) && packed_narrow_ok() && (half || x->dt == CG_F8) && batch == 1 && a.a_sk == 1 && a.a_vec && a.a_sm % 4 == 0 &&
-               K % 16 == 0 && K >= 256 && N >= 64 && y->buf) {
-        // a decode-time linear layer of a narrow dtype: the weight matrix narrowed in memory once, read at 2 or 1 bytes a weight
+    } else if (skinny_packed) {
+        // a decode-time linear layer of a narrow dtype: the weight matrix in memory as its dtype's patterns (as uploaded, or
+        // narrowed once), read at 2 or 1 bytes a weight
         // (measured on 2048 x 8192: one row 10.7 instead of 15.6 us for the 16-bit dtypes, 13.2 instead of 15.4 for fp8; with
         // four rows the loads of the activations bound both kernels alike, and widening fp8 costs more than it saves)
-        const int kind = half ? half : 3;
-        const void *pb = nullptr;
+        const void *pb = y_native ? native_ptr(y) : nullptr;
         void *tb = nullptr;
         size_t cb = 0;
-        int prc = pack_operand(be, y->buf, a.B, a.b_sn, a.b_sk, N, K, kind, true, &pb, &tb, &cb);
+        int prc = y_native ? CG_OK : pack_operand(be, words_buffer(y), a.B, a.b_sn, a.b_sk, N, K, kind, true, &pb, &tb, &cb);
         if (prc) return prc;
         const dim3 pgrid((uint32_t)((N + 3) / 4));
         const int kch = (int)(K / 1024);
@@ -2171,29 +2246,6 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
         }
 #undef CG_MM_SWITCH
     } else {
-        // the narrow tile when the wide one would leave over a seventh of its columns empty, and when the product has at
-        // most one 128 x 128 tile per compute unit: twice the workgroups then fill the chip (4096 x 2048 x 512: 148 -> 83 us)
-        // or at least put two on a unit (8192 x 2048 x 512: 148 -> 145 us); with more tiles than that the wide one wins
-        // (env CG_GEMM_NARROW_BELOW=n moves the limit, for measurements)
-        const int64_t cols128 = (N + 127) / 128 * 128, cols64 = (N + 63) / 64 * 64;
-        static const int64_t narrow_below = [] { const char *e = getenv("CG_GEMM_NARROW_BELOW"); return e ? atoll(e) : 256ll; }();
-        const int64_t tiles128 = ((M + BM - 1) / BM) * (cols128 / 128) * (int64_t)batch;
-        const bool narrow = (cols128 * 7 > cols64 * 8 || (tiles128 <= narrow_below && N >= 128)) && !half; // (the 16-bit kernels come in the two square tiles)
-        const int bn = narrow ? 64 : 128;
-        // the 256 x 256 tile when it covers the chip at least once (env CG_GEMM_BIG=0 switches it off)
-        const uint64_t tiles_big = (uint64_t)((M + 255) / 256) * ((N + 255) / 256) * batch;
-        static const bool big_allowed = [] {
-            const char *e = getenv("CG_GEMM_BIG");
-            return !(e && e[0] == '0');
-        }();
-        const bool fits_big = big_allowed && !narrow && tiles_big >= 256 && M >= 256 && N >= 256;
-        // f32 words: since whole tiles are loaded without tests, two workgroups of the 128 x 128 tile per compute unit (two
-        // waves per SIMD covering each other's barriers) are as fast as one of the wide tile or faster — 137-138 against
-        // 134-135 TFLOP/s on the 1B shape's linear layers, and a partial last round costs a quarter as much (8192 x 2048 x
-        // 3072: 755 against 1015 us) — except with a k-contiguous left and a row-contiguous right operand (x.y: 1 % behind).
-        // The 16-bit and fp8 paths keep the wide tile (half the L2 bytes per flop, which is what bounds them).
-        const bool narrow_dtype = half || x->dt == CG_F8;
-        const bool big = fits_big && (narrow_dtype || (!a_mfast && b_nfast));
         uint64_t tiles = big ? tiles_big / batch : (uint64_t)((M + BM - 1) / BM) * ((N + bn - 1) / bn);
         if (tiles > 0x7FFFFFFFull) return fail(CG_ERR_UNSUPPORTED, "matmul: too many tiles");
         // Too few tiles for the device (the linear layers of a short prefill on a narrow model): cut along k as well, so that
@@ -2251,29 +2303,24 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
             return ok;
         }();
         if (!lds_ok) return fail(CG_ERR_DEVICE, "matmul: cannot reserve %zu bytes of LDS", gemm_lds_bytes(128));
-        // Operands of a narrow dtype in a product big enough for the 256 x 256 tile: narrowed in memory first (the right
-        // operand once per buffer), then multiplied from 2-byte / 1-byte patterns (env CG_GEMM_PACKED=0 switches it off).
-        static const bool packed_allowed = [] {
-            const char *e = getenv("CG_GEMM_PACKED");
-            return !(e && e[0] == '0');
-        }();
-        const int kind = half ? half : x->dt == CG_F8 ? 3 : 0;
-        if (kind && packed_allowed && big && batch == 1 && K % (kind == 3 ? 16 : 8) == 0 && x->buf && y->buf) {
-            const void *pa = nullptr, *pb = nullptr;
+        if (big_packed) {
+            const void *pa = x_native ? native_ptr(x) : nullptr, *pb = y_native ? native_ptr(y) : nullptr;
             void *ta = nullptr, *tb = nullptr;
             size_t ca = 0, cb = 0;
             // (the left operand's narrow copy is kept with its buffer when somebody else holds the activations too — q / k / v
             // and gate / up multiply the same ones —; an operand only this product reads is narrowed for it alone)
             const bool x_shared = x->rc.load() > 1 || x->buf->rc.load() > 1;
-            int prc = pack_operand(be, x->buf, a.A, a.a_sm, a.a_sk, M, K, kind, x_shared, &pa, &ta, &ca);
-            if (!prc) prc = pack_operand(be, y->buf, a.B, a.b_sn, a.b_sk, N, K, kind, true, &pb, &tb, &cb);
+            int prc = x_native ? CG_OK : pack_operand(be, words_buffer(x), a.A, a.a_sm, a.a_sk, M, K, kind, x_shared, &pa, &ta, &ca);
+            if (!prc && !y_native) prc = pack_operand(be, words_buffer(y), a.B, a.b_sn, a.b_sk, N, K, kind, true, &pb, &tb, &cb);
             if (!prc) {
                 MmArgs p = a;
-                const int64_t kw = K / (kind == 3 ? 4 : 2); // words per row
+                const int64_t per = kind == 3 ? 4 : 2;      // elements per 32-bit word
+                const int64_t kw = K / per;                 // words per row
                 p.A = static_cast<const uint32_t *>(pa);
                 p.B = static_cast<const uint32_t *>(pb);
                 p.K = (uint32_t)kw;
-                p.a_sm = p.b_sn = kw;
+                p.a_sm = x_native ? a.a_sm / per : kw; // (a view taken as it lies keeps its own row pitch)
+                p.b_sn = y_native ? a.b_sn / per : kw;
                 p.a_sk = p.b_sk = 1;
                 p.a_vec = p.b_vec = 1;
                 if (kind == 1) hipLaunchKernelGGL((mfma_gemm_kernel<false, false, 4, 4, 3>), grid, dim3(kThreads), gemm_lds_bytes(256, 256), s, p);

@@ -121,6 +121,7 @@ static void buffer_release(Buffer *b) {
         if (b->ptr) b->be->pool.free(b->ptr, b->cls);
         if (b->side) b->be->pool.free(b->side, b->side_cls);
         drop_packed(b);
+        buffer_release(b->wide); // (a widened copy has none of its own: one level deep)
         Buffer *next = b->successor;
         delete b->rs;
         delete b;
@@ -166,6 +167,7 @@ static bool norm_fuse_of(const cg_tensor *x, NormFuse *nf, cg_tensor *h) {
     if (K <= 256 || K % 4 != 0 || rows < 1 || rows > 4 || p->rowlen != K) return false;
     const LeafView &lh = p->leaf[0], &lg = p->leaf[4];
     if (lh.uniform || lh.pw || lh.lazy || !lh.buf || !lh.buf->side || lh.offset != 0 || (int64_t)lh.buf->side_blocks * 4 != K) return false;
+    if (is_narrow_buf(lh.buf) || is_narrow_buf(lg.buf)) return false; // (the kernels read 32-bit words)
     if (!p->leaf[1].uniform || !p->leaf[2].uniform || !p->leaf[3].uniform) return false;
     if (lg.uniform || lg.pw || lg.lazy || !lg.buf || lg.offset % 4 != 0) return false;
     int64_t st = 1;
@@ -321,7 +323,7 @@ static void set_row_major(cg_tensor *t) {
     }
 }
 
-int new_dense(cg_backend *be, cg_dtype dt, const int64_t *dims, int rank, cg_tensor **out, int64_t reserve_elems) {
+int new_dense(cg_backend *be, cg_dtype dt, const int64_t *dims, int rank, cg_tensor **out, int64_t reserve_elems, int fmt) {
     cg_tensor *t = alloc_tensor(be);
     t->be = be;
     t->dt = dt;
@@ -332,7 +334,7 @@ int new_dense(cg_backend *be, cg_dtype dt, const int64_t *dims, int rank, cg_ten
     if (n > 0) {
         Buffer *b = new Buffer;
         b->be = be;
-        int rc = be->pool.alloc((size_t)(n > reserve_elems ? n : reserve_elems) * 4, &b->ptr, &b->cls);
+        int rc = be->pool.alloc((size_t)(n > reserve_elems ? n : reserve_elems) * fmt_bytes(fmt), &b->ptr, &b->cls);
         if (rc) {
             delete b;
             delete t;
@@ -340,6 +342,7 @@ int new_dense(cg_backend *be, cg_dtype dt, const int64_t *dims, int rank, cg_ten
             return rc;
         }
         b->elems = n;
+        b->fmt = fmt;
         t->buf = b;
     }
     *out = t;
@@ -378,8 +381,68 @@ cg_tensor *new_view(const cg_tensor *t) {
     return v;
 }
 
+int result_fmt(const cg_backend *be, cg_dtype dt, int64_t n) {
+    return be->narrow_storage && is_narrow(dt) && n >= be->narrow_from ? fmt_of(dt) : kFmtWords;
+}
+
+// The words of a narrow buffer: its widened copy, made now if nobody needed it before.
+static int wide_of(Buffer *b, Buffer **out) {
+    std::lock_guard<std::recursive_mutex> lk(g_lazy_mu);
+    if (!b->wide) {
+        Buffer *w = new Buffer;
+        w->be = b->be;
+        int rc = b->be->pool.alloc((size_t)b->elems * 4, &w->ptr, &w->cls);
+        if (!rc) rc = launch_widen(b->be, b->fmt, b->ptr, w->ptr, (uint64_t)b->elems);
+        if (rc) {
+            buffer_release(w);
+            return rc;
+        }
+        w->elems = b->elems;
+        w->constant = b->constant;
+        b->wide = w;
+    }
+    *out = b->wide;
+    return CG_OK;
+}
+
+// The handle's view moves from a narrow buffer to that buffer's widened copy (the values stay; every holder of the handle
+// sees it).  For the paths that go on writing into the buffer behind a tensor.
+static int make_words(cg_tensor *t) {
+    if (t->pend || !is_narrow_buf(t->buf)) return CG_OK;
+    std::lock_guard<std::recursive_mutex> lk(g_lazy_mu);
+    Buffer *w;
+    int rc = wide_of(t->buf, &w);
+    if (rc) return rc;
+    w->rc.fetch_add(1);
+    Buffer *old = t->buf;
+    t->buf = w;
+    if (old->rc.load() == 1) { // nobody else sees the narrow buffer: the copy is the handle's alone from here on
+        old->wide = nullptr;
+        w->rc.fetch_sub(1);
+    }
+    buffer_release(old);
+    return CG_OK;
+}
+
+int device_ptr_fmt(const cg_tensor *t, const void **ptr, int *fmt) {
+    if (t->buf && !t->pend && t->buf->fmt != kFmtWords) {
+        *fmt = t->buf->fmt;
+        *ptr = static_cast<const char *>(t->buf->ptr) + t->offset * (int64_t)fmt_bytes(t->buf->fmt);
+        return CG_OK;
+    }
+    *fmt = kFmtWords;
+    return device_ptr(t, ptr);
+}
+
 int device_ptr(const cg_tensor *t, const void **ptr) {
     if (t->pend) return fail(CG_ERR_ARG, "internal error: address of a deferred tensor requested");
+    if (t->buf && t->buf->fmt != kFmtWords) {
+        Buffer *w;
+        int rc = wide_of(t->buf, &w);
+        if (rc) return rc;
+        *ptr = static_cast<const char *>(w->ptr) + t->offset * 4;
+        return CG_OK;
+    }
     if (!t->buf) {
         if (!t->uniform || numel(t) == 0) {
             *ptr = nullptr;
@@ -466,10 +529,11 @@ int plan_views(const int64_t *vdims, int vrank, const ViewDesc *v, int n, bool k
         o.ubits = v[k].ubits;
         o.ptr = v[k].uniform ? nullptr : v[k].ptr;
         o.is = st[k][r - 1];
+        o.fmt = v[k].uniform ? (uint32_t)kFmtWords : (uint32_t)v[k].fmt;
         for (int d = 0; d < r - 1; d++) o.os[d] = st[k][r - 2 - d];
         if (v[k].vec_period > 0 && v[k].vec_period % 4) vec4 = false;
         if (!o.uniform && o.is == 1) {
-            if (reinterpret_cast<uintptr_t>(o.ptr) % 16) vec4 = false;
+            if (reinterpret_cast<uintptr_t>(o.ptr) % (4 * fmt_bytes((int)o.fmt))) vec4 = false; // four elements per access
             for (int d = 0; d < r - 1; d++)
                 if (o.os[d] % 4) vec4 = false;
         }
@@ -497,9 +561,10 @@ int plan_elementwise(const cg_tensor *const *views, int n, EwGeom *g, Operand *o
         v[k].uniform = views[k]->uniform;
         v[k].ubits = views[k]->ubits;
         v[k].ptr = nullptr;
+        v[k].fmt = kFmtWords;
         if (!views[k]->uniform) {
             const void *p;
-            int rc = device_ptr(views[k], &p);
+            int rc = device_ptr_fmt(views[k], &p, &v[k].fmt);
             if (rc) return rc;
             v[k].ptr = static_cast<const char *>(p);
         }
@@ -560,7 +625,7 @@ double distinct_bytes(const cg_tensor *t) {
     double n = 1.0;
     for (int i = 0; i < t->rank; i++)
         if (t->strides[i] != 0 || t->dims[i] <= 1) n *= (double)t->dims[i];
-    return 4.0 * n;
+    return (double)fmt_bytes(t->buf && !t->pend ? t->buf->fmt : kFmtWords) * n;
 }
 
 // ---- helpers for the entry points -------------------------------------------------------
@@ -669,7 +734,13 @@ static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p, b
 // Row-major copy of a view (the materialising half of reshape / to_vec).
 static int materialize(cg_backend *be, const cg_tensor *x, cg_tensor **out) {
     cg_tensor *o;
-    int rc = new_dense(be, x->dt, x->dims, x->rank, &o);
+    // a copy of a view of a narrow buffer keeps the buffer's format (whatever dtype tags the view); a program without row
+    // reductions stores the format of its dtype
+    int fmt = kFmtWords;
+    if (x->pend) fmt = x->pend->nred == 0 ? result_fmt(be, x->dt, numel(x)) : kFmtWords;
+    else if (is_narrow_buf(x->buf) && be->narrow_storage && numel(x) >= be->narrow_from) fmt = x->buf->fmt;
+    else if (x->buf) fmt = result_fmt(be, x->dt, numel(x));
+    int rc = new_dense(be, x->dt, x->dims, x->rank, &o, 0, fmt);
     if (rc) return rc;
     if (numel(x) > 0 && x->split >= 0) {
         // copy through the physical (rank + 1) shape: the split axis becomes two axes on both sides
@@ -891,7 +962,7 @@ static int try_residual_store(cg_backend *be, const cg_tensor *dst, const Pendin
             slot = l;
         } else {
             const Buffer *b = lv.lazy ? lv.lazy->result : lv.buf;
-            if (!b) return kDeclined;
+            if (!b || is_narrow_buf(b)) return kDeclined;
             terms[l] = static_cast<const uint32_t *>(b->ptr) + lv.offset;
         }
     }
@@ -911,7 +982,9 @@ static int try_residual_store(cg_backend *be, const cg_tensor *dst, const Pendin
 
 static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p, bool fresh) {
     if (!fresh) drop_packed(dst->buf); // a part of a buffer that may have been multiplied before is about to change
-    if (be->aot) {
+    const bool narrow_dst = is_narrow_buf(dst->buf);
+    if (narrow_dst && p.nred > 0) return fail(CG_ERR_ARG, "internal error: a narrow buffer written by a kernel that stores words");
+    if (be->aot && !narrow_dst) {
         int grc = try_gated_pair(be, dst, p);
         if (grc == kDeclined) grc = try_residual_store(be, dst, p, fresh);
         if (grc != kDeclined) return grc;
@@ -932,7 +1005,7 @@ static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p, b
             const int kind = (last.op & ~kInstrU32) == kRowMax ? kMax : kSum;
             const bool f32 = !(last.op & kInstrU32);
             cg_tensor *out = const_cast<cg_tensor *>(dst);
-            if (p.ninstr == 1 && !p.leaf[last.a].uniform) {
+            if (p.ninstr == 1 && !p.leaf[last.a].uniform && !is_narrow_buf(p.leaf[last.a].buf)) { // (those kernels read words)
                 cg_tensor leaf;
                 leaf_as_tensor(p, last.a, &space, f32 ? CG_F32 : CG_U32, &leaf);
                 leaf.be = be;
@@ -1116,7 +1189,8 @@ static int try_rope_stores(cg_backend *be, std::vector<DeferredWrite> &w, const 
     for (int i = 0; i < n; i++) {
         const Pending &p = *w[i].prog;
         const cg_tensor *dst = w[i].dst;
-        if (p.reduced || p.nred || p.overflow || dst->dt != CG_F32 || dst->rank != 4 || dst->dims[2] != 1 || dst->split >= 0) return kDeclined;
+        if (p.reduced || p.nred || p.overflow || dst->dt != CG_F32 || dst->rank != 4 || dst->dims[2] != 1 || dst->split >= 0 || is_narrow_buf(dst->buf))
+            return kDeclined;
         const int64_t B = dst->dims[0], H = dst->dims[1], hd = dst->dims[3];
         if (hd < 8 || hd % 8 || dst->strides[3] != 1) return kDeclined;
         const LeafView *lx = nullptr, *lc = nullptr, *ls = nullptr, *lr = nullptr;
@@ -1143,7 +1217,7 @@ static int try_rope_stores(cg_backend *be, std::vector<DeferredWrite> &w, const 
             return (B == 1 || s[0] == N) && (H == 1 || s[1] == hd) && s[3] == 1 && off == want_off;
         };
         auto row_table = [&](const LeafView *l) { // one row of hd factors, the same for every batch entry and head
-            return l->buf && !l->uniform && !l->pw && !l->lazy && (B == 1 || l->strides[0] == 0) && (H == 1 || l->strides[1] == 0) &&
+            return l->buf && !is_narrow_buf(l->buf) && !l->uniform && !l->pw && !l->lazy && (B == 1 || l->strides[0] == 0) && (H == 1 || l->strides[1] == 0) &&
                    l->strides[3] == 1;
         };
         if (!whole(lx->strides, lx->offset, 0)) return kDeclined;
@@ -1307,7 +1381,12 @@ static int ensure_concrete(cg_tensor *t) {
     }
     Buffer *b = new Buffer;
     b->be = be;
-    int rc = be->pool.alloc((size_t)numel(t) * 4, &b->ptr, &b->cls);
+    // a big result of a narrow dtype is stored as that dtype's patterns by the program kernels (not by the row-reduce and
+    // product-store paths, which write words)
+    bool plain = t->pend->nred == 0 && !t->pend->reduced;
+    for (int l = 0; l < t->pend->nleaf; l++) plain = plain && !t->pend->leaf[l].lazy && !t->pend->leaf[l].lazy2;
+    b->fmt = plain ? result_fmt(be, t->dt, numel(t)) : kFmtWords;
+    int rc = be->pool.alloc((size_t)numel(t) * fmt_bytes(b->fmt), &b->ptr, &b->cls);
     if (rc) {
         delete b;
         return rc;
@@ -1739,6 +1818,11 @@ static bool try_row_append(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim
     }
     if (outer <= 1 || outer > 65536 || min_os % R) return false;
     if (numel(x) * 4 < 65536) return false; // not worth the bookkeeping
+    if (is_narrow_buf(x->buf)) { // rows are appended to 32-bit words
+        hipError_t she = hipSetDevice(b->device);
+        *status = she == hipSuccess ? make_words(x) : hip_fail(she, "hipSetDevice");
+        if (*status) return true;
+    }
     Buffer *src = x->buf;
     RowStore *rs = src->rs;
     const int64_t C = rs ? rs->C : min_os / R;
@@ -1909,6 +1993,8 @@ int cg_backend_create(int device, cg_backend **out) {
     const char *aot = getenv("CG_AOT");
     b->aot = !(aot && aot[0] == '0');
     if (const char *seg = getenv("CG_ATTN_SEG_FROM")) b->attn_seg_from = atoll(seg);
+    if (const char *ns = getenv("CG_NARROW_STORAGE")) b->narrow_storage = ns[0] != '0';
+    if (const char *nf = getenv("CG_NARROW_FROM")) b->narrow_from = std::max<int64_t>(atoll(nf), 2);
     const char *trace = getenv("CG_TRACE_PROGRAMS");
     b->trace_programs = trace && trace[0] == '1';
     char name[256];
@@ -2140,11 +2226,14 @@ int cg_from_host(cg_backend *b, cg_dtype dtype, const void *data, size_t len, co
         return CG_OK;
     }
     cg_tensor *t;
-    rc = new_dense(b, dtype, d, (int)rank, &t);
+    const int fmt = result_fmt(b, dtype, (int64_t)n);
+    rc = new_dense(b, dtype, d, (int)rank, &t, 0, fmt);
     if (rc) return rc;
     if (n) {
         CG_HIP(hipSetDevice(b->device));
-        if (is_narrow(dtype)) { // 2- or 1-byte elements: uploaded as they are, widened to 32-bit words on the device
+        if (fmt != kFmtWords) { // kept as they come: 2 or 1 bytes per element
+            rc = staged_upload(b, t->buf->ptr, data, n * host_bytes(dtype));
+        } else if (is_narrow(dtype)) { // a small tensor: uploaded as it is, widened to 32-bit words on the device
             void *tmp = nullptr;
             size_t cls = 0;
             const size_t eb = host_bytes(dtype);
@@ -2324,6 +2413,17 @@ int cg_to_host(cg_backend *b, const cg_tensor *t, void *dst, size_t len) {
         const void *p;
         void *half = nullptr;
         size_t cls = 0;
+        if (src->buf && src->buf->fmt == fmt_of(t->dt)) { // the patterns are in memory as they are wanted
+            int sf;
+            rc = flush_deferred(b);
+            if (!rc) rc = device_ptr_fmt(src, &p, &sf);
+            if (!rc) {
+                hipError_t e = hipMemcpyAsync(dst, p, len * eb, hipMemcpyDeviceToHost, b->stream);
+                rc = e == hipSuccess ? wait_and_check(b) : hip_fail(e, "device to host copy");
+            }
+            release(tmp);
+            return rc;
+        }
         rc = device_ptr(src, &p);
         if (!rc) rc = b->pool.alloc(len * eb, &half, &cls);
         if (!rc) {
@@ -3096,7 +3196,7 @@ int cg_concat(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor *
     // has room behind it, y is appended in place and x's handle is returned with the larger
     // extent — one copy of y instead of a copy of everything accumulated so far.
     if (outermost && nx > 0 && ny > 0 && !x->uniform && x->rc.load() == 1 && x->buf && x->buf->rc.load() == 1 &&
-        x->offset == 0 && is_contiguous(x) && (size_t)(nx + ny) * 4 <= x->buf->cls) {
+        x->offset == 0 && is_contiguous(x) && !is_narrow_buf(x->buf) && (size_t)(nx + ny) * 4 <= x->buf->cls) {
         cg_tensor tail;
         tail.be = b;
         tail.buf = x->buf;
@@ -3158,7 +3258,11 @@ int cg_concat(cg_backend *b, cg_tensor *x, cg_tensor *y, size_t dim, cg_tensor *
         }
     }
     // a stack that starts growing gets room for as much again, so later appends stay in place
-    int rc = new_dense(b, x->dt, od, x->rank, &o, outermost && !constant ? 2 * (nx + ny) : 0);
+    // (a stack that may grow in place holds words; other big results of a narrow dtype are stored narrow, written by the
+    // copy / program kernels of the two halves)
+    const bool growing = outermost && !constant;
+    const bool by_rows = (x->pend && (x->pend->nred > 0 || x->pend->reduced)) || (y->pend && (y->pend->nred > 0 || y->pend->reduced));
+    int rc = new_dense(b, x->dt, od, x->rank, &o, growing ? 2 * (nx + ny) : 0, growing || by_rows ? kFmtWords : result_fmt(b, x->dt, nx + ny));
     if (rc) return rc;
     if (constant) const_memo_insert(b, ckey, o->buf);
     const cg_tensor *parts[2] = {x, y};
@@ -3205,14 +3309,12 @@ int cg_index(cg_backend *b, cg_tensor *x, size_t dim, cg_tensor *indices, cg_ten
     int64_t od[kMaxRank];
     memcpy(od, x->dims, sizeof od);
     od[dim] = J;
-    cg_tensor *o;
-    int rc = new_dense(b, x->dt, od, x->rank, &o);
-    if (rc) return rc;
-    if (numel(o) > 0) {
-        if (x->dims[dim] == 0) {
-            release(o);
-            return fail(CG_ERR_RANGE, "index: index out of bounds for an axis of length 0");
-        }
+    cg_tensor *o = nullptr;
+    int64_t on = 1;
+    for (int i = 0; i < x->rank; i++) on *= od[i];
+    int rc = CG_OK;
+    if (on > 0) {
+        if (x->dims[dim] == 0) return fail(CG_ERR_RANGE, "index: index out of bounds for an axis of length 0");
         // the gather kernel wants a row-major source and a 1-D index vector
         cg_tensor *xs = nullptr, *is = nullptr;
         const cg_tensor *src = x, *idx = indices;
@@ -3226,6 +3328,17 @@ int cg_index(cg_backend *b, cg_tensor *x, size_t dim, cg_tensor *indices, cg_ten
             rc = materialize(b, indices, &is);
             idx = is;
         }
+        // rows of a narrow source are gathered as they lie in memory; a big result keeps the source's format
+        if (!rc) {
+            int ofmt = kFmtWords;
+            if (is_narrow_buf(src->buf) && b->narrow_storage && on >= b->narrow_from) {
+                int64_t inner = 1;
+                for (int i = (int)dim + 1; i < x->rank; i++) inner *= x->dims[i];
+                const int64_t eb = (int64_t)fmt_bytes(src->buf->fmt);
+                if (inner * eb % 4 == 0 && src->offset * eb % 4 == 0) ofmt = src->buf->fmt; // (whole 32-bit words per row: see launch_gather)
+            }
+            rc = new_dense(b, x->dt, od, x->rank, &o, 0, ofmt);
+        }
         if (!rc) rc = launch_gather(b, src, (int)dim, idx, o);
         release(xs);
         release(is);
@@ -3233,6 +3346,9 @@ int cg_index(cg_backend *b, cg_tensor *x, size_t dim, cg_tensor *indices, cg_ten
             release(o);
             return rc;
         }
+    } else {
+        rc = new_dense(b, x->dt, od, x->rank, &o);
+        if (rc) return rc;
     }
     *out = o;
     return CG_OK;

@@ -71,6 +71,101 @@ def test_segment_attention_kernel_matches_closed_form_and_oracle(hip_segments, o
         assert_close(case.kind, g, r, s, f"{case.name}[{i}] vs oracle")
 
 
+@pytest.fixture(scope="module")
+def hip_narrow_everywhere():
+    """A backend that keeps EVERY tensor of a narrow float dtype as 2- / 1-byte patterns (by default only tensors of 65536
+    elements and more): the small tensors of the 16-bit and fp8 cases then take the narrow-format loads and stores of every
+    kernel, the widened copies of the kernels that address words, and the declines of the decode-time fusions."""
+    from backends import backend_with_env
+
+    be = backend_with_env(CG_NARROW_FROM="2")
+    yield be
+    be.close()
+
+
+@pytest.fixture(scope="module")
+def hip_words_only():
+    """A backend that keeps tensors of the narrow float dtypes as 32-bit words (CG_NARROW_STORAGE=0)."""
+    from backends import backend_with_env
+
+    be = backend_with_env(CG_NARROW_STORAGE="0")
+    yield be
+    be.close()
+
+
+@pytest.mark.parametrize("case", [c for c in CASES if c.name.startswith(("half_", "fp8_"))], ids=lambda c: c.name)
+def test_narrow_storage_of_small_tensors_matches_oracle(hip_narrow_everywhere, hip_words_only, oracle, case):
+    print(f"case={case.name} (narrow storage from 2 elements)", flush=True)
+    got = case.run(hip_narrow_everywhere)
+    wide = case.run(hip_words_only)
+    ref = case.run(oracle)
+    scales = case.scale() if case.scale else [None] * len(ref)
+    assert len(got) == len(ref) == len(wide)
+    for i, (g, w, e, s) in enumerate(zip(got, wide, ref, scales)):
+        assert g.dtype == e.dtype
+        assert_close(case.kind, g, e, s, f"{case.name}[{i}]")
+        assert_close(case.kind, w, e, s, f"{case.name}[{i}] (32-bit words)")
+    if case.expect is not None:
+        for i, (g, e, s) in enumerate(zip(got, case.expect(), scales)):
+            assert_close(case.kind, g, e, s, f"{case.name}[{i}] vs closed form")
+
+
+def test_narrow_tensors_occupy_their_own_width(hip, oracle):
+    """A bf16 tensor of 8192 x 8192 and an fp8 tensor of the same shape take 128 and 64 MiB of device memory; the sum
+    and the product of two such tensors, a strided view, a concat, a gather and a row sum of them are stored / computed
+    as the oracle does, and nothing but the pool's rounding is held afterwards."""
+    import cases_fp8
+    import cases_half
+
+    hip.sync()
+    hip.pool_trim()
+    base = hip.pool_stats()[0]
+    n = 8192
+    ua, a = cases_half.bf16_values(9101, (n, n), 1.0)
+    ub, b = cases_half.bf16_values(9102, (n, n), 1.0)
+    ta, tb = cases_half.from_half(hip, A.BF16, ua), cases_half.from_half(hip, A.BF16, ub)
+    held = hip.pool_stats()[0] - base
+    assert 2 * n * n * 2 <= held <= 2 * n * n * 2 + (64 << 20), held          # 2 bytes per element (+ size classes)
+    tsum = hip.add(ta, tb)
+    got = cases_half.as_f32(A.BF16, cases_half.read(hip, tsum))
+    exp = cases_half.as_f32(A.BF16, cases_half.round_to(A.BF16, a + b))
+    assert np.array_equal(got, exp)
+    held = hip.pool_stats()[0] - base
+    assert held <= 3 * n * n * 2 + (96 << 20), held                           # the sum is stored narrow as well
+    # a strided view (every other row, transposed) materialised by reshape; a row sum; a gather of rows
+    view = hip.reshape(hip.transpose(hip.slice(tsum, 0, 1, n - 1), 0, 1), (n * (n - 1),))
+    got = cases_half.as_f32(A.BF16, cases_half.read(hip, view))
+    assert np.array_equal(got, exp[1:].T.reshape(-1))
+    del view
+    rows = cases_half.as_f32(A.BF16, cases_half.read(hip, hip.sum(tsum)))
+    ref = exp.astype(np.float64).sum(-1, keepdims=True)
+    assert np.all(np.abs(rows - ref) <= 2.0 ** -7 * np.abs(ref) + 1e-3 * np.abs(exp).sum(-1, keepdims=True))
+    idx = np.array([5, 8191, 0, 5, 4096], np.uint32)
+    few = cases_half.as_f32(A.BF16, cases_half.read(hip, hip.index(tsum, 0, hip.from_numpy(idx))))
+    assert np.array_equal(few, exp[idx])
+    many = np.arange(0, n, 3, dtype=np.uint32)[::-1].copy()
+    big = cases_half.as_f32(A.BF16, cases_half.read(hip, hip.index(tsum, 0, hip.from_numpy(many))))
+    assert np.array_equal(big, exp[many])
+    cols = cases_half.as_f32(A.BF16, cases_half.read(hip, hip.index(tsum, 1, hip.from_numpy(idx))))
+    assert np.array_equal(cols, exp[:, idx])
+    cat = cases_half.as_f32(A.BF16, cases_half.read(hip, hip.concat(hip.slice(tsum, 1, 0, 100), hip.slice(ta, 1, 7, 33), 1)))
+    assert np.array_equal(cat, np.concatenate([exp[:, :100], a[:, 7:40]], 1))
+    del tsum, ta, tb
+    # fp8: 1 byte per element
+    rng = np.random.default_rng(9103)
+    codes = rng.integers(0, 256, (n, n), dtype=np.uint8)
+    codes[(codes & 0x7F) == 0x7F] = 0x38                                        # no NaNs: 1.0 instead
+    t8 = hip.ndarray_from_vec_fp8(codes, codes.shape)
+    held = hip.pool_stats()[0] - base
+    assert n * n <= held <= n * n + (32 << 20), held
+    back = hip.to_numpy(hip.reshape(hip.transpose(t8, 0, 1), (n * n,)))
+    assert back.dtype == np.uint8 and np.array_equal(back.reshape(n, n), codes.T)
+    del t8
+    hip.sync()
+    hip.pool_trim()
+    assert hip.pool_stats()[0] - base <= (1 << 20)
+
+
 @pytest.mark.parametrize("case", KATS["cases"], ids=lambda c: c["name"])
 def test_hip_reference_kat(hip, case):
     check_case(hip, case)
