@@ -109,6 +109,15 @@ def micro_bench(iters=20):
         run(f"linear_{tag}_8192x2048x8192", A.K_GEMM_MFMA, lambda: be.matmul(be.cast(x32, dt), wv), "TFLOP/s", mfma_peak=peak)
         del wn, wv
     del x32, w32
+    # the same kernels on tensors that lie in memory as 2-byte patterns (bf16): 2 bytes per element read and written
+    ab = be.cast(be.from_numpy(rng.standard_normal((n, n), dtype=np.float32)), A.BF16)
+    bb = be.cast(be.from_numpy(rng.standard_normal((n, n), dtype=np.float32)), A.BF16)
+    be.realize(ab), be.realize(bb)
+    run("add_bf16_8192x8192", A.K_ELEMENTWISE, lambda: be.realize(be.add(ab, bb)), "GB/s")
+    run("sum_last_bf16_8192x8192", A.K_REDUCE, lambda: be.realize(be.sum(ab)), "GB/s")
+    run("transpose_bf16_8192x8192_materialised", A.K_ELEMENTWISE,
+        lambda: be.realize(be.reshape(be.transpose(ab, 0, 1), (n * n,))), "GB/s")
+    del ab, bb
     # the strided / indexing kernels of the path: a materialised transpose, concat along the outermost and the innermost
     # axis, the embedding gather of the 1B-shape prefill and a sum over a non-last axis (8 bytes per element moved,
     # 4 per element reduced)

@@ -387,13 +387,15 @@ struct ViewDesc {
 // Collapses the iteration space shared by `n` views of shape `dims` (v[0] is the output)
 // and fills geometry + operands.  keep_last_axis: never merge the last axis into the one
 // before it (reductions need it on its own).
+// allow_vec8: work items of 8 elements when some operand lies in memory in a narrow format (its 16-byte access) and the
+// extents and every operand's alignment allow it (the caller's kernel must have that instantiation).
 int plan_views(const int64_t *dims, int rank, const ViewDesc *v, int n, bool keep_last_axis, EwGeom *g, Operand *ops,
-               bool allow_vec4 = true);
+               bool allow_vec4 = true, bool allow_vec8 = false);
 
 // Collapses the iteration space shared by `n` views of identical shape (views[0] is
 // the output) and fills geometry + operands.  Returns CG_ERR_UNSUPPORTED when the
 // space exceeds 2^32-1 work items.
-int plan_elementwise(const cg_tensor *const *views, int n, EwGeom *g, Operand *ops);
+int plan_elementwise(const cg_tensor *const *views, int n, EwGeom *g, Operand *ops, bool allow_vec8 = false);
 
 // Times one launch with a pair of events on the backend's stream when the kernel class
 // is being sampled; the pair is resolved by the next call that waits for the device.
@@ -429,7 +431,8 @@ enum EwOp : int {
 constexpr bool is_row_reduce(int op) { return (op & ~0x80) == kRowSum || (op & ~0x80) == kRowMax; }
 
 // out = op(ins...) element-wise; all views have out's shape.  `out` may be a strided view.
-int launch_elementwise(cg_backend *be, int op, cg_dtype dt, const cg_tensor *out, const cg_tensor *const *ins, int nin);
+// round_op: kRoundBF16 / kRoundF16 / kRoundF8 applied to the (f32) result before it is stored, 0: none.
+int launch_elementwise(cg_backend *be, int op, cg_dtype dt, const cg_tensor *out, const cg_tensor *const *ins, int nin, int round_op = 0);
 // True when the program of `p` can be register-allocated for the interpreter kernels.
 bool fused_program_fits(const Pending &p);
 // Evaluates `p` for every element of shape `dims` into `out` (a dense or strided view of that shape).

@@ -17,15 +17,23 @@ __device__ __forceinline__ uint32_t asu(float f) { return __float_as_uint(f); }
 __device__ __forceinline__ uint32_t f8_word_of_dev(uint8_t b);
 __device__ __forceinline__ uint8_t f8_byte_of_dev(uint32_t u);
 
-// VEC consecutive elements (element stride o.is) of a NARROW operand, widened to f32 words.
+// VEC consecutive elements (element stride o.is) of a NARROW operand, widened to f32 words.  VEC 4 or 8 with unit stride:
+// one load of 8 or 16 bytes (16-bit formats), of 4 or 8 bytes (fp8); the planner has checked the alignment.
 template <int VEC>
 __device__ __forceinline__ void load_narrow(const Operand &o, int64_t off, uint32_t (&r)[VEC]) {
     if (o.fmt == kFmtF8) {
         const uint8_t *p = reinterpret_cast<const uint8_t *>(o.ptr) + off;
-        if (VEC == 4 && o.is == 1) {
-            const uint32_t t = *reinterpret_cast<const uint32_t *>(p);
+        if (VEC >= 4 && o.is == 1) {
+            uint32_t t[VEC >= 8 ? 2 : 1];
+            if (VEC >= 8) {
+                const uint2 q = *reinterpret_cast<const uint2 *>(p);
+                t[0] = q.x;
+                t[VEC >= 8 ? 1 : 0] = q.y;
+            } else {
+                t[0] = *reinterpret_cast<const uint32_t *>(p);
+            }
 #pragma unroll
-            for (int j = 0; j < VEC; j++) r[j] = f8_word_of_dev((uint8_t)(t >> (8 * j)));
+            for (int j = 0; j < VEC; j++) r[j] = f8_word_of_dev((uint8_t)(t[j / 4] >> (8 * (j % 4))));
         } else if (o.is == 0) {
             const uint32_t t = f8_word_of_dev(*p);
 #pragma unroll
@@ -38,12 +46,21 @@ __device__ __forceinline__ void load_narrow(const Operand &o, int64_t off, uint3
     }
     const uint16_t *p = reinterpret_cast<const uint16_t *>(o.ptr) + off;
     uint16_t h[VEC];
-    if (VEC == 4 && o.is == 1) {
-        const uint2 t = *reinterpret_cast<const uint2 *>(p);
-        h[0] = (uint16_t)t.x;
-        h[1 % VEC] = (uint16_t)(t.x >> 16);
-        h[2 % VEC] = (uint16_t)t.y;
-        h[3 % VEC] = (uint16_t)(t.y >> 16);
+    if (VEC >= 4 && o.is == 1) {
+        uint32_t t[VEC / 2 > 0 ? VEC / 2 : 1];
+        if (VEC >= 8) {
+            const uint4 q = *reinterpret_cast<const uint4 *>(p);
+            t[0] = q.x;
+            t[1 % (VEC / 2 > 0 ? VEC / 2 : 1)] = q.y;
+            t[2 % (VEC / 2 > 0 ? VEC / 2 : 1)] = q.z;
+            t[3 % (VEC / 2 > 0 ? VEC / 2 : 1)] = q.w;
+        } else {
+            const uint2 q = *reinterpret_cast<const uint2 *>(p);
+            t[0] = q.x;
+            t[1 % (VEC / 2 > 0 ? VEC / 2 : 1)] = q.y;
+        }
+#pragma unroll
+        for (int j = 0; j < VEC; j++) h[j] = (uint16_t)(t[j / 2] >> (16 * (j % 2)));
     } else if (o.is == 0) {
         const uint16_t t = *p;
 #pragma unroll
@@ -58,15 +75,23 @@ __device__ __forceinline__ void load_narrow(const Operand &o, int64_t off, uint3
 }
 
 // f32 words that hold values of a narrow format, stored as that format's patterns.
-template <int VEC>
+template <int VEC, bool STREAM = false>
 __device__ __forceinline__ void store_narrow(const Operand &o, int64_t off, const uint32_t (&r)[VEC]) {
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    typedef uint32_t u2 __attribute__((ext_vector_type(2)));
     if (o.fmt == kFmtF8) {
         uint8_t *p = reinterpret_cast<uint8_t *>(const_cast<char *>(o.ptr)) + off;
-        if (VEC == 4 && o.is == 1) {
-            uint32_t t = 0;
+        if (VEC >= 4 && o.is == 1) {
+            uint32_t t[VEC >= 8 ? 2 : 1] = {};
 #pragma unroll
-            for (int j = 0; j < VEC; j++) t |= (uint32_t)f8_byte_of_dev(r[j]) << (8 * j);
-            *reinterpret_cast<uint32_t *>(p) = t;
+            for (int j = 0; j < VEC; j++) t[j / 4] |= (uint32_t)f8_byte_of_dev(r[j]) << (8 * (j % 4));
+            if (VEC >= 8) {
+                const u2 v = {t[0], t[VEC >= 8 ? 1 : 0]};
+                if (STREAM) __builtin_nontemporal_store(v, reinterpret_cast<u2 *>(p));
+                else *reinterpret_cast<u2 *>(p) = v;
+            } else {
+                *reinterpret_cast<uint32_t *>(p) = t[0];
+            }
         } else {
 #pragma unroll
             for (int j = 0; j < VEC; j++) p[(int64_t)j * o.is] = f8_byte_of_dev(r[j]);
@@ -78,11 +103,20 @@ __device__ __forceinline__ void store_narrow(const Operand &o, int64_t off, cons
     for (int j = 0; j < VEC; j++)
         h[j] = o.fmt == kFmtBF16 ? (uint16_t)(r[j] >> 16) : __half_as_ushort(__float2half_rn(__uint_as_float(r[j])));
     uint16_t *p = reinterpret_cast<uint16_t *>(const_cast<char *>(o.ptr)) + off;
-    if (VEC == 4 && o.is == 1) {
-        uint2 t;
-        t.x = (uint32_t)h[0] | ((uint32_t)h[1 % VEC] << 16);
-        t.y = (uint32_t)h[2 % VEC] | ((uint32_t)h[3 % VEC] << 16);
-        *reinterpret_cast<uint2 *>(p) = t;
+    if (VEC >= 4 && o.is == 1) {
+        constexpr int W = VEC / 2 > 0 ? VEC / 2 : 1;
+        uint32_t t[W];
+#pragma unroll
+        for (int j = 0; j < W; j++) t[j] = (uint32_t)h[(2 * j) % VEC] | ((uint32_t)h[(2 * j + 1) % VEC] << 16);
+        if (VEC >= 8) {
+            const u4 v = {t[0], t[1 % W], t[2 % W], t[3 % W]};
+            if (STREAM) __builtin_nontemporal_store(v, reinterpret_cast<u4 *>(p));
+            else *reinterpret_cast<u4 *>(p) = v;
+        } else {
+            const u2 v = {t[0], t[1 % W]};
+            if (STREAM) __builtin_nontemporal_store(v, reinterpret_cast<u2 *>(p));
+            else *reinterpret_cast<u2 *>(p) = v;
+        }
     } else {
 #pragma unroll
         for (int j = 0; j < VEC; j++) p[(int64_t)j * o.is] = h[j];
@@ -101,13 +135,16 @@ __device__ __forceinline__ void load_words(const Operand &o, int64_t off, uint32
         return;
     }
     const uint32_t *p = reinterpret_cast<const uint32_t *>(o.ptr) + off;
-    if (VEC == 4 && o.is == 1) {
+    if (VEC >= 4 && o.is == 1) {
         typedef uint32_t u4 __attribute__((ext_vector_type(4)));
-        u4 t = STREAM ? __builtin_nontemporal_load(reinterpret_cast<const u4 *>(p)) : *reinterpret_cast<const u4 *>(p);
-        r[0] = t[0];
-        r[1 % VEC] = t[1];
-        r[2 % VEC] = t[2];
-        r[3 % VEC] = t[3];
+#pragma unroll
+        for (int q = 0; q < VEC / 4; q++) {
+            const u4 t = STREAM ? __builtin_nontemporal_load(reinterpret_cast<const u4 *>(p) + q) : reinterpret_cast<const u4 *>(p)[q];
+            r[(4 * q) % VEC] = t[0];
+            r[(4 * q + 1) % VEC] = t[1];
+            r[(4 * q + 2) % VEC] = t[2];
+            r[(4 * q + 3) % VEC] = t[3];
+        }
     } else if (o.is == 0) {
         uint32_t t = *p;
 #pragma unroll
@@ -123,17 +160,17 @@ __device__ __forceinline__ void load_words(const Operand &o, int64_t off, uint32
 template <int VEC, bool STREAM = false>
 __device__ __forceinline__ void store_words(const Operand &o, int64_t off, const uint32_t (&r)[VEC]) {
     if (o.fmt != kFmtWords) {
-        store_narrow<VEC>(o, off, r);
+        store_narrow<VEC, STREAM>(o, off, r);
         return;
     }
     uint32_t *p = reinterpret_cast<uint32_t *>(const_cast<char *>(o.ptr)) + off;
-    if (VEC == 4 && o.is == 1) {
-        if (STREAM) {
-            typedef uint32_t u4 __attribute__((ext_vector_type(4)));
-            u4 v = {r[0], r[1 % VEC], r[2 % VEC], r[3 % VEC]};
-            __builtin_nontemporal_store(v, reinterpret_cast<u4 *>(p));
-        } else {
-            *reinterpret_cast<uint4 *>(p) = make_uint4(r[0], r[1 % VEC], r[2 % VEC], r[3 % VEC]);
+    if (VEC >= 4 && o.is == 1) {
+        typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+        for (int q = 0; q < VEC / 4; q++) {
+            const u4 v = {r[(4 * q) % VEC], r[(4 * q + 1) % VEC], r[(4 * q + 2) % VEC], r[(4 * q + 3) % VEC]};
+            if (STREAM) __builtin_nontemporal_store(v, reinterpret_cast<u4 *>(p) + q);
+            else reinterpret_cast<u4 *>(p)[q] = v;
         }
     } else {
 #pragma unroll

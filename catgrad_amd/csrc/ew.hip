@@ -16,6 +16,7 @@
 #include "device_utils.hpp"
 
 #include <algorithm>
+#include <type_traits>
 
 namespace cg {
 
@@ -30,6 +31,7 @@ struct EwArgs {
     Operand out;
     Operand in[3];
     uint32_t *fault;
+    uint32_t round; // kRoundBF16 / kRoundF16 / kRoundF8: the result is rounded to that format before it is stored; 0: not
 };
 
 // FLAT: the iteration space collapsed to a single axis (no index arithmetic at all).
@@ -87,6 +89,13 @@ __global__ __launch_bounds__(kBlock) void ew_kernel(const EwArgs a) {
 #pragma unroll
             for (int j = 0; j < VEC; j++)
                 r[j] = apply<OP, F>(x[u][0][j], NIN > 1 ? x[u][1 % NIN][j] : 0u, NIN > 2 ? x[u][2 % NIN][j] : 0u, a.fault);
+            if (F && a.round) { // (the same for every lane: a launch parameter)
+#pragma unroll
+                for (int j = 0; j < VEC; j++)
+                    r[j] = a.round == kRoundBF16 ? apply<kRoundBF16, true>(r[j], 0u, 0u, a.fault)
+                           : a.round == kRoundF16 ? apply<kRoundF16, true>(r[j], 0u, 0u, a.fault)
+                                                  : apply<kRoundF8, true>(r[j], 0u, 0u, a.fault);
+            }
             if (a.g.total >= kStreamItems) store_words<VEC, true>(a.out, off[u][0], r);
             else store_words<VEC>(a.out, off[u][0], r);
         }
@@ -98,7 +107,12 @@ template <int OP, bool F, int NIN> int launch_variants(cg_backend *be, const EwA
     if (blocks == 0) return CG_OK;
     dim3 grid((uint32_t)blocks), block(kBlock);
     bool flat = a.g.nouter == 0;
-    if (a.g.vec == 4) {
+    if (a.g.vec == 8) {
+        if (flat)
+            hipLaunchKernelGGL((ew_kernel<OP, F, NIN, 8, true>), grid, block, 0, be->stream, a);
+        else
+            hipLaunchKernelGGL((ew_kernel<OP, F, NIN, 8, false>), grid, block, 0, be->stream, a);
+    } else if (a.g.vec == 4) {
         if (flat)
             hipLaunchKernelGGL((ew_kernel<OP, F, NIN, 4, true>), grid, block, 0, be->stream, a);
         else
@@ -180,10 +194,10 @@ __global__ __launch_bounds__(kBlock) void gather_kernel(const uint32_t *__restri
 // line with one of the two.  Here a workgroup moves a 64 x 64 tile through LDS: 16-byte loads along the source's
 // unit-stride axis, 16-byte stores along the destination's.  HBM-bound: 8 bytes per element.
 struct TransposeArgs {
-    const uint32_t *src;
-    uint32_t *dst;
+    const char *src;
+    char *dst;
     uint32_t I, T;            // extents of the destination's fast axis (i) and of the source's fast axis (t)
-    int64_t src_is, dst_ts;   // source stride along i, destination stride along t (the other two are 1)
+    int64_t src_is, dst_ts;   // source stride along i, destination stride along t (the other two are 1), in elements
     uint32_t tiles_i, tiles_t;
     uint32_t nrest;           // further axes, innermost first
     uint32_t rd[kMaxOuter];
@@ -192,8 +206,12 @@ struct TransposeArgs {
     uint32_t vec;             // 1: every 16-byte access of a whole tile is aligned
 };
 
-__global__ __launch_bounds__(kBlock) void transpose_copy_kernel(const TransposeArgs a) {
+// EB: bytes per element (4: 32-bit words; 2 / 1: the narrow formats, moved as they lie).  A 16-byte piece holds 16 / EB
+// elements; in LDS every element has a 32-bit word of its own, so the exchange is the same for every width.
+template <int EB> __global__ __launch_bounds__(kBlock) void transpose_copy_kernel(const TransposeArgs a) {
     constexpr int TS = 64, PITCH = TS + 1;
+    constexpr int PER = 16 / EB, PIECES = TS / PER, RPP = kBlock / PIECES, PASSES = TS / RPP;
+    typedef typename std::conditional<EB == 4, uint32_t, typename std::conditional<EB == 2, uint16_t, uint8_t>::type>::type E;
     __shared__ uint32_t tile[TS][PITCH]; // [i][t]
     // tiles are walked along diagonals: neighbouring workgroups then differ in BOTH their source rows and their
     // destination rows, which spreads the strided side of the copy over the memory channels
@@ -210,54 +228,63 @@ __global__ __launch_bounds__(kBlock) void transpose_copy_kernel(const TransposeA
         so += i * a.src_rs[d];
         dofs += i * a.dst_rs[d];
     }
+    const E *const src = reinterpret_cast<const E *>(a.src);
+    E *const dst = reinterpret_cast<E *>(a.dst);
     const uint32_t i0 = ti * TS, t0 = tt * TS;
     const bool whole = a.vec && i0 + TS <= a.I && t0 + TS <= a.T;
-    const uint32_t q = threadIdx.x % 16, r = threadIdx.x / 16; // a quarter-row of 16-byte pieces, 16 rows per pass
+    const uint32_t q = threadIdx.x % PIECES, r = threadIdx.x / PIECES; // a row of 16-byte pieces, RPP rows per pass
     typedef uint32_t u4 __attribute__((ext_vector_type(4)));
     if (whole) {
-        u4 v[4];
+        u4 v[PASSES];
 #pragma unroll
-        for (int k = 0; k < 4; k++) // row i0 + r + 16k of the source, pieces t0 + 4q .. + 3
-            v[k] = __builtin_nontemporal_load(reinterpret_cast<const u4 *>(a.src + so + (int64_t)(i0 + r + 16 * k) * a.src_is + t0 + 4 * q));
+        for (int k = 0; k < PASSES; k++) // row i0 + r + RPP k of the source, elements t0 + PER q .. + PER - 1
+            v[k] = __builtin_nontemporal_load(reinterpret_cast<const u4 *>(src + so + (int64_t)(i0 + r + RPP * k) * a.src_is + t0 + PER * q));
 #pragma unroll
-        for (int k = 0; k < 4; k++) {
-            uint32_t *row = tile[r + 16 * k];
-            row[4 * q] = v[k][0];
-            row[4 * q + 1] = v[k][1];
-            row[4 * q + 2] = v[k][2];
-            row[4 * q + 3] = v[k][3];
+        for (int k = 0; k < PASSES; k++) {
+            uint32_t *row = tile[r + RPP * k];
+#pragma unroll
+            for (int j = 0; j < PER; j++) {
+                const uint32_t word = v[k][j * EB / 4];
+                row[PER * q + j] = EB == 4 ? word : EB == 2 ? (word >> (16 * (j % 2))) & 0xFFFFu : (word >> (8 * (j % 4))) & 0xFFu;
+            }
         }
         __syncthreads();
 #pragma unroll
-        for (int k = 0; k < 4; k++) { // row t0 + r + 16k of the destination, pieces i0 + 4q .. + 3
-            const uint32_t t = r + 16 * k;
-            const u4 o = {tile[4 * q][t], tile[4 * q + 1][t], tile[4 * q + 2][t], tile[4 * q + 3][t]};
-            __builtin_nontemporal_store(o, reinterpret_cast<u4 *>(a.dst + dofs + (int64_t)(t0 + t) * a.dst_ts + i0 + 4 * q));
+        for (int k = 0; k < PASSES; k++) { // row t0 + r + RPP k of the destination, elements i0 + PER q .. + PER - 1
+            const uint32_t t = r + RPP * k;
+            u4 o = {0u, 0u, 0u, 0u};
+#pragma unroll
+            for (int j = 0; j < PER; j++) {
+                const uint32_t e = tile[PER * q + j][t];
+                o[j * EB / 4] |= EB == 4 ? e : EB == 2 ? e << (16 * (j % 2)) : e << (8 * (j % 4));
+            }
+            __builtin_nontemporal_store(o, reinterpret_cast<u4 *>(dst + dofs + (int64_t)(t0 + t) * a.dst_ts + i0 + PER * q));
         }
         return;
     }
     // ragged or unaligned tile: element by element, still along the fast axis of each side
     const uint32_t c = threadIdx.x % 64, w = threadIdx.x / 64;
     for (uint32_t k = w; k < TS; k += 4)
-        if (i0 + k < a.I && t0 + c < a.T) tile[k][c] = a.src[so + (int64_t)(i0 + k) * a.src_is + t0 + c];
+        if (i0 + k < a.I && t0 + c < a.T) tile[k][c] = src[so + (int64_t)(i0 + k) * a.src_is + t0 + c];
     __syncthreads();
     for (uint32_t k = w; k < TS; k += 4)
-        if (t0 + k < a.T && i0 + c < a.I) a.dst[dofs + (int64_t)(t0 + k) * a.dst_ts + i0 + c] = tile[c][k];
+        if (t0 + k < a.T && i0 + c < a.I) dst[dofs + (int64_t)(t0 + k) * a.dst_ts + i0 + c] = (E)tile[c][k];
 }
 
 // Takes a planned copy (a.out, a.in[0]) when it is a transposition worth tiling; kDeclined otherwise.
 static int try_transpose_copy(cg_backend *be, const EwArgs &a) {
     const EwGeom &g = a.g;
     if (a.in[0].uniform || a.out.is != 1 || a.in[0].is == 1 || a.in[0].is == 0 || g.nouter < 1) return kDeclined;
-    if (a.in[0].fmt != kFmtWords || a.out.fmt != kFmtWords) return kDeclined; // (the tiles are 32-bit words)
+    if (a.in[0].fmt != a.out.fmt || a.round) return kDeclined; // (elements are moved as they lie)
+    const int64_t eb = (int64_t)fmt_bytes((int)a.out.fmt), per = 16 / eb; // bytes per element, elements per 16-byte access
     int td = -1; // the outer axis along which the source is unit-stride
     for (uint32_t d = 0; d < g.nouter; d++)
         if (a.in[0].os[d] == 1 && g.od[d] >= 16) td = (int)d;
     if (td < 0 || g.inner < 16) return kDeclined;
     TransposeArgs t;
     memset(&t, 0, sizeof t);
-    t.src = reinterpret_cast<const uint32_t *>(a.in[0].ptr);
-    t.dst = reinterpret_cast<uint32_t *>(const_cast<char *>(a.out.ptr));
+    t.src = a.in[0].ptr;
+    t.dst = const_cast<char *>(a.out.ptr);
     t.I = g.inner;
     t.T = g.od[td];
     t.src_is = a.in[0].is;
@@ -266,37 +293,40 @@ static int try_transpose_copy(cg_backend *be, const EwArgs &a) {
     t.tiles_i = (t.I + 63) / 64;
     t.tiles_t = (t.T + 63) / 64;
     uint64_t blocks = (uint64_t)t.tiles_i * t.tiles_t;
-    bool vec = reinterpret_cast<uintptr_t>(t.src) % 16 == 0 && reinterpret_cast<uintptr_t>(t.dst) % 16 == 0 && t.src_is % 4 == 0 &&
-               t.dst_ts % 4 == 0;
+    bool vec = reinterpret_cast<uintptr_t>(t.src) % 16 == 0 && reinterpret_cast<uintptr_t>(t.dst) % 16 == 0 && t.src_is % per == 0 &&
+               t.dst_ts % per == 0;
     for (uint32_t d = 0; d < g.nouter; d++) {
         if ((int)d == td) continue;
         t.rd[t.nrest] = g.od[d];
         t.rdiv[t.nrest] = make_fastdiv(g.od[d]);
         t.src_rs[t.nrest] = a.in[0].os[d];
         t.dst_rs[t.nrest] = a.out.os[d];
-        if (a.in[0].os[d] % 4 || a.out.os[d] % 4) vec = false;
+        if (a.in[0].os[d] % per || a.out.os[d] % per) vec = false;
         blocks *= g.od[d];
         t.nrest++;
     }
     if (blocks == 0 || blocks > 0x7FFFFFFFull) return kDeclined;
     t.vec = vec ? 1u : 0u;
-    hipLaunchKernelGGL(transpose_copy_kernel, dim3((uint32_t)blocks), dim3(kBlock), 0, be->stream, t);
+    if (eb == 4) hipLaunchKernelGGL(transpose_copy_kernel<4>, dim3((uint32_t)blocks), dim3(kBlock), 0, be->stream, t);
+    else if (eb == 2) hipLaunchKernelGGL(transpose_copy_kernel<2>, dim3((uint32_t)blocks), dim3(kBlock), 0, be->stream, t);
+    else hipLaunchKernelGGL(transpose_copy_kernel<1>, dim3((uint32_t)blocks), dim3(kBlock), 0, be->stream, t);
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? CG_OK : hip_fail(e, "transposing copy launch");
 }
 
-int launch_elementwise(cg_backend *be, int op, cg_dtype dt, const cg_tensor *out, const cg_tensor *const *ins, int nin) {
+int launch_elementwise(cg_backend *be, int op, cg_dtype dt, const cg_tensor *out, const cg_tensor *const *ins, int nin, int round_op) {
     if (int frc = flush_deferred(be)) return frc;
     const cg_tensor *views[4] = {out, nullptr, nullptr, nullptr};
     for (int k = 0; k < nin; k++) views[k + 1] = ins[k];
     EwArgs a;
     memset(&a, 0, sizeof a);
     Operand ops[4];
-    int rc = plan_elementwise(views, nin + 1, &a.g, ops);
+    int rc = plan_elementwise(views, nin + 1, &a.g, ops, true);
     if (rc) return rc;
     a.out = ops[0];
     for (int k = 0; k < nin; k++) a.in[k] = ops[k + 1];
     a.fault = be->fault_dev;
+    a.round = (uint32_t)round_op;
     double work = distinct_bytes(out);
     for (int k = 0; k < nin; k++) work += distinct_bytes(ins[k]);
     ProfScope prof(be, CG_K_ELEMENTWISE, work);

@@ -36,7 +36,9 @@ struct RowsArgs {
     uint32_t od[kMaxOuter];
     FastDiv odiv[kMaxOuter];
     int64_t os[kMaxOuter];
-    uint32_t vec;         // 4: rows are unit-stride and 16-byte aligned
+    uint32_t vec;         // 4: rows are unit-stride and 16-byte aligned; 8: the same for rows of a narrow format (one access of
+                          // 16 bytes, fp8 8 bytes, holds 8 elements)
+    uint32_t fmt;         // how the elements lie in memory (kFmtWords, ...); narrow formats: reduce_rows_kernel only
 };
 
 __device__ __forceinline__ int32_t total_key(uint32_t bits) { // Rust f32::total_cmp
@@ -111,7 +113,39 @@ template <int K, bool F, int TPR> __global__ __launch_bounds__(kBlock) void redu
     const uint32_t row = blockIdx.x * RPB + threadIdx.x / TPR;
     const bool live = row < a.rows;
     Acc<K, F> acc;
-    if (live) {
+    if (live && a.fmt != kFmtWords) { // (the same for every lane: a launch parameter)
+        Operand o;
+        o.ptr = a.x;
+        o.is = a.sn;
+        o.uniform = 0;
+        o.fmt = a.fmt;
+        const int64_t base = row_offset(row, a.nouter, a.od, a.odiv, a.os);
+        if (a.vec == 8) {
+            const uint32_t nv = a.n / 8;
+            uint32_t i = lane;
+            for (; i + TPR < nv; i += 2 * TPR) { // two independent loads in flight per lane per trip
+                uint32_t t0[8], t1[8];
+                load_narrow<8>(o, base + 8 * (int64_t)i, t0);
+                load_narrow<8>(o, base + 8 * (int64_t)(i + TPR), t1);
+#pragma unroll
+                for (int j = 0; j < 8; j++) acc.take(t0[j], 8 * i + j);
+#pragma unroll
+                for (int j = 0; j < 8; j++) acc.take(t1[j], 8 * (i + TPR) + j);
+            }
+            if (i < nv) {
+                uint32_t t0[8];
+                load_narrow<8>(o, base + 8 * (int64_t)i, t0);
+#pragma unroll
+                for (int j = 0; j < 8; j++) acc.take(t0[j], 8 * i + j);
+            }
+        } else {
+            for (uint32_t i = lane; i < a.n; i += TPR) {
+                uint32_t t[1];
+                load_narrow<1>(o, base + (int64_t)i * a.sn, t);
+                acc.take(t[0], i);
+            }
+        }
+    } else if (live) {
         const uint32_t *p = reinterpret_cast<const uint32_t *>(a.x) + row_offset(row, a.nouter, a.od, a.odiv, a.os);
         if (a.vec == 4) {
             const uint32_t nv = a.n / 4;
@@ -228,11 +262,14 @@ template <int MODE, bool F, int VEC> __global__ __launch_bounds__(kBlock) void a
     if (hit) *a.flag = 1u;
 }
 
-int fill_rows_args(const cg_tensor *x, RowsArgs *a) {
+// native: a view of a narrow buffer is described as it lies in memory (for reduce_rows_kernel); else as 32-bit words
+int fill_rows_args(const cg_tensor *x, RowsArgs *a, bool native = false) {
     memset(a, 0, sizeof *a);
     const void *p;
-    int rc = device_ptr(x, &p);
+    int fmt = kFmtWords;
+    int rc = native ? device_ptr_fmt(x, &p, &fmt) : device_ptr(x, &p);
     if (rc) return rc;
+    a->fmt = (uint32_t)fmt;
     a->x = static_cast<const char *>(p);
     int r = x->rank;
     int64_t n = x->dims[r - 1];
@@ -258,14 +295,15 @@ int fill_rows_args(const cg_tensor *x, RowsArgs *a) {
     a->rows = (uint32_t)rows;
     a->n = (uint32_t)n;
     a->nouter = (uint32_t)w;
-    bool vec = !x->uniform && a->sn == 1 && n % 4 == 0 && reinterpret_cast<uintptr_t>(p) % 16 == 0;
+    const int64_t per = fmt == kFmtWords ? 4 : 8; // elements per vector access
+    bool vec = !x->uniform && a->sn == 1 && n % per == 0 && reinterpret_cast<uintptr_t>(p) % (fmt == kFmtF8 ? 8 : 16) == 0;
     for (int d = 0; d < w; d++) {
         a->od[d] = (uint32_t)dims[w - 1 - d];
         a->odiv[d] = make_fastdiv(a->od[d]);
         a->os[d] = st[w - 1 - d];
-        if (a->os[d] % 4) vec = false;
+        if (a->os[d] % per) vec = false;
     }
-    a->vec = vec ? 4 : 1;
+    a->vec = vec ? (uint32_t)per : 1;
     return CG_OK;
 }
 
@@ -427,9 +465,16 @@ template <int K, bool F> int launch_cols(cg_backend *be, const RowsArgs &a) {
     return e == hipSuccess ? CG_OK : hip_fail(e, "column reduction launch");
 }
 
+// Which kernels launch_rows picks: 1 the column kernels, 2 the segmented ones, 0 a row per 4 .. 256 lanes.
+static int rows_route(const RowsArgs &a) {
+    if (a.sn != 1 && a.nouter >= 1 && a.os[0] == 1 && a.od[0] >= 16 && a.n >= 8) return 1;
+    return a.rows <= 64 && a.n >= 32768 ? 2 : 0;
+}
+
 template <int K, bool F> int launch_rows(cg_backend *be, const RowsArgs &a) {
-    if (a.sn != 1 && a.nouter >= 1 && a.os[0] == 1 && a.od[0] >= 16 && a.n >= 8) return launch_cols<K, F>(be, a);
-    if (a.rows <= 64 && a.n >= 32768) {
+    if (rows_route(a) != 0 && a.fmt != kFmtWords) return fail(CG_ERR_ARG, "internal error: a narrow operand in a reduction kernel that reads words");
+    if (rows_route(a) == 1) return launch_cols<K, F>(be, a);
+    if (rows_route(a) == 2) {
         uint32_t segs = std::min<uint32_t>(256, (a.n + 1023) / 1024);
         const uint32_t seglen = ((a.n + segs - 1) / segs + 3) / 4 * 4;
         segs = (a.n + seglen - 1) / seglen;
@@ -495,7 +540,8 @@ int noalloc_setup(int device) {
 int launch_reduce(cg_backend *be, int kind, const cg_tensor *x, cg_tensor *out) {
     if (int frc = flush_deferred(be)) return frc;
     RowsArgs a;
-    int rc = fill_rows_args(x, &a);
+    int rc = fill_rows_args(x, &a, true);
+    if (!rc && a.fmt != kFmtWords && rows_route(a) != 0) rc = fill_rows_args(x, &a); // those kernels read words
     if (rc) return rc;
     a.out = static_cast<uint32_t *>(out->buf->ptr);
     bool f = is_f(x->dt);

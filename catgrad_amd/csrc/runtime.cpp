@@ -481,7 +481,7 @@ FastDiv make_fastdiv(uint32_t d) {
 }
 
 int plan_views(const int64_t *vdims, int vrank, const ViewDesc *v, int n, bool keep_last_axis, EwGeom *g,
-               Operand *ops, bool allow_vec4) {
+               Operand *ops, bool allow_vec4, bool allow_vec8) {
     int r = 0;
     int64_t dims[kMaxRank];
     int64_t st[kMaxViews + 1][kMaxRank];
@@ -522,6 +522,7 @@ int plan_views(const int64_t *vdims, int vrank, const ViewDesc *v, int n, bool k
         if (dims[i] > 0xFFFFFFFFll) return fail(CG_ERR_UNSUPPORTED, "axis extent above 2^32-1 elements");
     int64_t inner = dims[r - 1];
     bool vec4 = allow_vec4 && inner % 4 == 0;
+    bool vec8 = allow_vec4 && allow_vec8 && inner % 8 == 0, any_narrow = false;
     for (int k = 0; k < n; k++) {
         Operand &o = ops[k];
         memset(&o, 0, sizeof o);
@@ -532,15 +533,23 @@ int plan_views(const int64_t *vdims, int vrank, const ViewDesc *v, int n, bool k
         o.fmt = v[k].uniform ? (uint32_t)kFmtWords : (uint32_t)v[k].fmt;
         for (int d = 0; d < r - 1; d++) o.os[d] = st[k][r - 2 - d];
         if (v[k].vec_period > 0 && v[k].vec_period % 4) vec4 = false;
+        if (v[k].vec_period > 0 && v[k].vec_period % 8) vec8 = false;
         if (!o.uniform && o.is == 1) {
-            if (reinterpret_cast<uintptr_t>(o.ptr) % (4 * fmt_bytes((int)o.fmt))) vec4 = false; // four elements per access
-            for (int d = 0; d < r - 1; d++)
+            const size_t eb = fmt_bytes((int)o.fmt);
+            any_narrow = any_narrow || o.fmt != kFmtWords;
+            if (reinterpret_cast<uintptr_t>(o.ptr) % (4 * eb)) vec4 = false; // four elements per access
+            // eight: one access of 16 (16-bit formats) or 8 bytes (fp8), two of 16 bytes for words
+            if (reinterpret_cast<uintptr_t>(o.ptr) % (eb == 4 ? 16 : 8 * eb)) vec8 = false;
+            for (int d = 0; d < r - 1; d++) {
                 if (o.os[d] % 4) vec4 = false;
+                if (o.os[d] % (eb == 4 ? 4 : 8)) vec8 = false;
+            }
         }
     }
+    vec8 = vec8 && vec4 && any_narrow;
     g->nouter = (uint32_t)(r - 1);
     g->inner = (uint32_t)inner;
-    g->vec = vec4 ? 4 : 1;
+    g->vec = vec8 ? 8 : vec4 ? 4 : 1;
     g->ipr = (uint32_t)(inner / g->vec);
     g->ipr_div = make_fastdiv(g->ipr ? g->ipr : 1);
     uint64_t total = g->ipr;
@@ -554,7 +563,7 @@ int plan_views(const int64_t *vdims, int vrank, const ViewDesc *v, int n, bool k
     return CG_OK;
 }
 
-int plan_elementwise(const cg_tensor *const *views, int n, EwGeom *g, Operand *ops) {
+int plan_elementwise(const cg_tensor *const *views, int n, EwGeom *g, Operand *ops, bool allow_vec8) {
     ViewDesc v[kMaxViews];
     for (int k = 0; k < n; k++) {
         v[k].strides = views[k]->strides;
@@ -569,7 +578,7 @@ int plan_elementwise(const cg_tensor *const *views, int n, EwGeom *g, Operand *o
             v[k].ptr = static_cast<const char *>(p);
         }
     }
-    return plan_views(views[0]->dims, views[0]->rank, v, n, false, g, ops);
+    return plan_views(views[0]->dims, views[0]->rank, v, n, false, g, ops, true, allow_vec8);
 }
 
 // ---- launch timing ---------------------------------------------------------------------
@@ -1005,7 +1014,7 @@ static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p, b
             const int kind = (last.op & ~kInstrU32) == kRowMax ? kMax : kSum;
             const bool f32 = !(last.op & kInstrU32);
             cg_tensor *out = const_cast<cg_tensor *>(dst);
-            if (p.ninstr == 1 && !p.leaf[last.a].uniform && !is_narrow_buf(p.leaf[last.a].buf)) { // (those kernels read words)
+            if (p.ninstr == 1 && !p.leaf[last.a].uniform) {
                 cg_tensor leaf;
                 leaf_as_tensor(p, last.a, &space, f32 ? CG_F32 : CG_U32, &leaf);
                 leaf.be = be;
@@ -1015,6 +1024,22 @@ static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p, b
             }
             if (p.ninstr > 1 && last.a == kMaxLeaves + p.ninstr - 2)
                 return launch_fused_reduce(be, kind, f32, p, p.ninstr - 1, space.dims, space.rank, out);
+        }
+        // the same of a narrow dtype, whose result is rounded to the dtype: the reduction kernels, then the rounding of
+        // the few results where they stand
+        const Instr first = p.ins[0];
+        if (p.reduced && p.nred == 1 && p.ninstr == 2 && is_row_reduce(first.op) && !(first.op & kInstrU32) && first.a < kMaxLeaves &&
+            !p.leaf[first.a].uniform && last.a == kMaxLeaves && (last.op == kRoundBF16 || last.op == kRoundF16 || last.op == kRoundF8) &&
+            is_contiguous(dst)) {
+            cg_tensor *out = const_cast<cg_tensor *>(dst);
+            cg_tensor leaf;
+            leaf_as_tensor(p, first.a, &space, CG_F32, &leaf);
+            leaf.be = be;
+            int rc = launch_reduce(be, first.op == kRowMax ? kMax : kSum, &leaf, out);
+            leaf.buf = nullptr;
+            const cg_tensor *ins[1] = {out};
+            if (!rc) rc = launch_elementwise(be, last.op, CG_F32, out, ins, 1);
+            return rc;
         }
         return launch_fused_rows(be, dst, p, space.dims, space.rank);
     }
@@ -1047,7 +1072,11 @@ static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p, b
         }
         return rc;
     }
-    if (p.ninstr == 1 && !piecewise) {
+    // one operation, or one operation of a narrow dtype with the rounding of its result behind it: the single-op kernel
+    const bool op_and_round = p.ninstr == 2 && !(p.ins[0].op & kInstrU32) && p.ins[1].a == kMaxLeaves &&
+                              (p.ins[1].op == kRoundBF16 || p.ins[1].op == kRoundF16 || p.ins[1].op == kRoundF8) &&
+                              p.ins[0].a < kMaxLeaves && p.ins[0].b < kMaxLeaves && p.ins[0].c < kMaxLeaves;
+    if ((p.ninstr == 1 || op_and_round) && !piecewise) {
         const Instr in = p.ins[0];
         const int op = in.op & ~kInstrU32;
         const cg_dtype dt = (in.op & kInstrU32) ? CG_U32 : CG_F32;
@@ -1059,7 +1088,7 @@ static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p, b
             leaf_as_tensor(p, regs[k], dst, dt, &tmp[k]);
             ins[k] = &tmp[k];
         }
-        int rc = launch_elementwise(be, op, dt, dst, ins, nin);
+        int rc = launch_elementwise(be, op, dt, dst, ins, nin, op_and_round ? p.ins[1].op : 0);
         for (int k = 0; k < nin; k++) tmp[k].buf = nullptr;
         return rc;
     }

@@ -63,12 +63,16 @@ typedef struct cg_tensor cg_tensor;   /* `HipBackend::BackendTensor` */
 typedef enum cg_dtype {
     CG_F32 = 0,
     CG_F16 = 1,  /* IEEE binary16; NdArrayBackend has todo!() here (ndarray.rs:7-9), CandleBackend implements it */
-    CG_BF16 = 2, /* bfloat16; idem.  Both: 2-byte elements at the boundary (cg_from_host / cg_to_host), held as
-                    32-bit words inside; every op computes in f32 on exactly held values and rounds its result
-                    to the dtype (nearest, ties to even); sums and products accumulate in f32 and round once */
+    CG_BF16 = 2, /* bfloat16; idem.  Both: 2-byte elements at the boundary (cg_from_host / cg_to_host) and in device memory
+                    (tensors of 65536 elements and more: uploads, element-wise results, copies, gathers, concats; smaller
+                    tensors and the results of products and row reductions are held as 32-bit words, each holding its value
+                    exactly); every op computes in f32 on exactly held values and rounds its result to the dtype (nearest,
+                    ties to even); sums and products accumulate in f32 and round once */
     CG_F8 = 3,   /* float8::F8E4M3 (candle.rs:9,382): 4 exponent bits (bias 7), 3 mantissa bits, no infinities, largest
-                    finite value 448; same model: 1-byte elements at the boundary, 32-bit words inside, every result
-                    rounded to nearest even and saturated to +-448.  NdArrayBackend has todo!() here too */
+                    finite value 448; same model: 1-byte elements at the boundary and in device memory (same rule), every
+                    result rounded to nearest even and saturated to +-448.  NdArrayBackend has todo!() here too.
+                    (CG_NARROW_STORAGE=0 in the environment when a backend is created keeps every tensor as 32-bit words;
+                    CG_NARROW_FROM=n moves the limit of 65536 elements.) */
     CG_U32 = 4
 } cg_dtype;
 
