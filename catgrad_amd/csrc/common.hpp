@@ -334,6 +334,17 @@ struct LazyMm {
     // are computed by one grouped launch.  `be` is set while the product is listed as open.
     bool groupable = false;
     cg_backend *be = nullptr;
+    // A product whose value is x . y with an RMS norm over every run of hn_hd columns applied to it (see RopeStore::hgamma):
+    // what became of `rmsnorm(reshape(x . y, [rows * heads, hd]))` when the product was still open.  Computed either by the
+    // kernel that also embeds and stores the heads (try_rope_stores), or, when something else needs it first, as the
+    // product followed by the kept program hn_prog (whose leaf 0 then reads the plain product).
+    bool head_norm = false;
+    Buffer *hn_gamma = nullptr; // retained
+    int64_t hn_gamma_off = 0;
+    uint32_t hn_hd = 0, hn_n_bits = 0, hn_eps_bits = 0, hn_exp_bits = 0;
+    Pending *hn_prog = nullptr; // owned
+    int64_t hn_dims[kMaxRank] = {0};
+    int hn_rank = 0;
 };
 void lazy_mm_release(LazyMm *m);
 // Computes the product if it has not been yet.
@@ -506,11 +517,15 @@ int launch_matmul_group(cg_backend *be, const cg_tensor *x, const cg_tensor *con
 // Where the columns of a decode-time product go when the rotary embedding and the write into a KV cache (or into q's own
 // buffer) run in the product's store: column n = head * hd + d of row b goes to dst[b * sb + head * sh + d], after
 // out[d] = cos[d] * x[d] + sin[d] * rot[d], rot = concat(-x[hd/2..], x[..hd/2]) when `rope` (cos, sin: hd words each).
+// hgamma: when set, every head of a row (hd columns) first goes through an RMS norm of its own, x / pow(sum(x * x) / n +
+// eps, e) * hgamma[d] (the q / k norm of Qwen3, qwen3.rs:249-279): a workgroup then owns a whole head.
 struct RopeStore {
     uint32_t *dst;
     int64_t sb, sh;
     const uint32_t *cos, *sin;
     uint32_t hd, rope;
+    const uint32_t *hgamma;
+    uint32_t hn_n_bits, hn_eps_bits, hn_exp_bits;
 };
 // The products x . ys[i] (one row per batch entry, the same x) with such a store each; kDeclined when the shapes are not
 // the grouped kernel's.  nf as in launch_matmul_group.

@@ -616,9 +616,10 @@ static int64_t attn_row_halves_below() {
     return n;
 }
 
-// Most segments per KV head (env CG_ATTN_SEG_MAX, for measurements).
+// Most segments per KV head (env CG_ATTN_SEG_MAX, for measurements).  With few (batch entry, KV head) groups many segments
+// pay: one group of 8 KV heads with head_dim 128 at 4500 positions 18.7 us with up to 32 segments, 24.0 with up to 16.
 static int64_t attn_seg_max() {
-    static const int64_t n = [] { const char *e = getenv("CG_ATTN_SEG_MAX"); return e ? atoll(e) : 8ll; }();
+    static const int64_t n = [] { const char *e = getenv("CG_ATTN_SEG_MAX"); return e ? atoll(e) : 32ll; }();
     return n;
 }
 
@@ -714,7 +715,13 @@ int launch_decode_attention(cg_backend *be, const Pending &p, const int64_t *pdi
     // against the kernels below (batch 4 x 8 KV heads x 4 rows, head_dim 64): 2100 positions 20.4 against 19.7 us (the segment
     // kernel alone 13.6 against 19.7: what it saves, the combine launch and the hand-over to it cost again), 6000 positions 34.9
     // against 34.9, 9000 positions 44 against 55, 12000 positions 53 against 64; batch 16 at 2100 positions 42 against 46.
-    if (be->attn_seg_from > 0 && (T >= be->attn_seg_from || (qrows > 256 && T >= 1024))) {
+    // With at most 8 groups (a single sequence) the kernels below leave most of the device idle and the segments win from 2560
+    // positions on: 8 KV heads, head_dim 128: 3000 positions 17.2 against 28.3 us, 12000 positions 31.7 against 59.0; 3 KV
+    // heads, head_dim 64: 4500 positions 16.7 against 20.0, 12000 positions 22.1 against 40.5 (2100 positions: 15.8 against 15.8).
+    // (Merging the segments inside the kernel — the workgroup that counts itself last at a device-scope counter reads the
+    // others' results — was measured and costs what the combine launch costs: the stores must reach memory, the count must come
+    // back and the loads go out again, 6 to 7 us in all; with a release / acquire fence per workgroup 24.0 against 19.3 us.)
+    if (be->attn_seg_from > 0 && (T >= be->attn_seg_from || (qrows > 256 && T >= 1024) || (f1.batch <= 8 && T >= 2560))) {
         const int64_t tpb = hd == 64 ? kSegBlock / 16 : kSegBlock / 32;
         int64_t want = std::min<int64_t>(attn_seg_max(), std::max<int64_t>(1, 256 / f1.batch));
         want = std::max<int64_t>(1, std::min<int64_t>(want, T / 64));

@@ -21,6 +21,7 @@ namespace cg {
 static thread_local std::string g_err;
 static std::recursive_mutex g_lazy_mu; // guards lazy backing of uniform tensors and of deferred ones (computing one may compute another)
 static int ensure_concrete(cg_tensor *t);
+static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p, bool fresh);
 
 int fail(int code, const char *fmt, ...) {
     char buf[512];
@@ -210,7 +211,7 @@ static bool residual_sum_open(const cg_tensor *x) {
         if (lv.lazy && !lv.lazy->result) {
             const LazyMm *m = lv.lazy;
             const int64_t N = m->rank > 0 ? m->dims[m->rank - 1] : 0;
-            if (!m->groupable || m->rc.load() != 1 || m->rank != x->rank || N < 512 || N >= 8192) return false;
+            if (!m->groupable || m->head_norm || m->rc.load() != 1 || m->rank != x->rank || N < 512 || N >= 8192) return false;
             open++;
         } else if (!lv.lazy && !lv.buf) {
             return false;
@@ -238,18 +239,46 @@ void lazy_mm_release(LazyMm *m) {
         release(m->x);
         release(m->y);
         buffer_release(m->result);
+        buffer_release(m->hn_gamma);
+        delete m->hn_prog;
         delete m;
     }
 }
 
 int lazy_mm_force(cg_backend *be, LazyMm *m) {
     if (m->result) return CG_OK;
+    if (m->head_norm) {
+        // nobody took it with the norm in the store: the plain product, then the kept norm program over it
+        lazy_mm_close(m);
+        if (m->x->pend) {
+            int xrc = ensure_concrete(m->x);
+            if (xrc) return xrc;
+        }
+        cg_tensor *raw = nullptr, *o = nullptr;
+        int rc = new_dense(be, CG_F32, m->dims, m->rank, &raw);
+        if (!rc) rc = launch_matmul(be, m->x, m->y, raw);
+        if (!rc) rc = new_dense(be, CG_F32, m->hn_dims, m->hn_rank, &o);
+        if (!rc) {
+            LeafView &l0 = m->hn_prog->leaf[0];
+            buffer_release(l0.buf);
+            l0.buf = raw->buf;
+            l0.buf->rc.fetch_add(1);
+            rc = run_pending(be, o, *m->hn_prog, true);
+        }
+        if (!rc) {
+            m->result = o->buf;
+            o->buf = nullptr;
+        }
+        release(o);
+        release(raw);
+        return rc;
+    }
     if (m->groupable && m->be) {
         // the other open products with the same left operand go along in the same launch
         LazyMm *grp[4] = {m};
         int n = 1;
         for (LazyMm *o : be->lazy_open)
-            if (o != m && !o->result && o->x == m->x && n < 4) grp[n++] = o;
+            if (o != m && !o->result && !o->head_norm && o->x == m->x && n < 4) grp[n++] = o;
         NormFuse nf;
         cg_tensor h;
         const bool normed = m->x->pend && norm_fuse_of(m->x, &nf, &h);
@@ -738,7 +767,8 @@ static int wait_and_check(cg_backend *be) {
 }
 
 // fresh: dst is the whole of a buffer allocated for this very result (nothing else lives in it).
-static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p, bool fresh = false);
+static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p, bool fresh);
+static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p) { return run_pending(be, dst, p, false); }
 
 // Row-major copy of a view (the materialising half of reshape / to_vec).
 static int materialize(cg_backend *be, const cg_tensor *x, cg_tensor **out) {
@@ -896,7 +926,7 @@ static int try_gated_pair(cg_backend *be, const cg_tensor *dst, const Pending &p
     const LeafView &lg = p.leaf[0], &lc = p.leaf[1], &lu = p.leaf[2];
     if (!lc.uniform || lg.uniform || lu.uniform || lg.pw || lu.pw || !lg.lazy || !lu.lazy || lg.lazy == lu.lazy) return kDeclined;
     LazyMm *mg = lg.lazy, *mu = lu.lazy;
-    if (mg->result || mu->result || !mg->groupable || !mu->groupable || mg->x != mu->x || mg->rc.load() != 1 ||
+    if (mg->result || mu->result || mg->head_norm || mu->head_norm || !mg->groupable || !mu->groupable || mg->x != mu->x || mg->rc.load() != 1 ||
         mu->rc.load() != 1 || mg->rank != dst->rank || mu->rank != dst->rank)
         return kDeclined;
     // both leaves are the whole products, read in place
@@ -963,7 +993,7 @@ static int try_residual_store(cg_backend *be, const cg_tensor *dst, const Pendin
         }
         if (lv.lazy && !lv.lazy->result) {
             LazyMm *m = lv.lazy;
-            if (slot >= 0 || !m->groupable || m->rc.load() != 1 || lv.offset != 0 || m->rank != dst->rank) return kDeclined;
+            if (slot >= 0 || !m->groupable || m->head_norm || m->rc.load() != 1 || lv.offset != 0 || m->rank != dst->rank) return kDeclined;
             for (int d = 0; d < dst->rank; d++)
                 if (m->dims[d] != dst->dims[d]) return kDeclined;
             for (LazyMm *o : be->lazy_open)
@@ -1241,7 +1271,7 @@ static int try_rope_stores(cg_backend *be, std::vector<DeferredWrite> &w, const 
         const int64_t N = m->dims[m->rank - 1];
         int64_t rows = 1;
         for (int d = 0; d + 1 < m->rank; d++) rows *= m->dims[d];
-        if (H * hd != N || rows != B || B > 4) return kDeclined;
+        if (H * hd != N || rows != B || B > 4 || (m->head_norm && m->hn_hd != (uint32_t)hd)) return kDeclined;
         auto whole = [&](const int64_t *s, int64_t off, int64_t want_off) { // the view [B, H, 1, hd] of the product's rows, from `want_off`
             return (B == 1 || s[0] == N) && (H == 1 || s[1] == hd) && s[3] == 1 && off == want_off;
         };
@@ -1258,6 +1288,12 @@ static int try_rope_stores(cg_backend *be, std::vector<DeferredWrite> &w, const 
             st[i].cos = static_cast<const uint32_t *>(lc->buf->ptr) + lc->offset;
             st[i].sin = static_cast<const uint32_t *>(ls->buf->ptr) + ls->offset;
             st[i].rope = 1;
+        }
+        if (m->head_norm) { // the heads' own RMS norm ahead of the embedding
+            st[i].hgamma = static_cast<const uint32_t *>(m->hn_gamma->ptr) + m->hn_gamma_off;
+            st[i].hn_n_bits = m->hn_n_bits;
+            st[i].hn_eps_bits = m->hn_eps_bits;
+            st[i].hn_exp_bits = m->hn_exp_bits;
         }
         st[i].dst = static_cast<uint32_t *>(dst->buf->ptr) + dst->offset;
         st[i].sb = B > 1 ? dst->strides[0] : 0;
@@ -1694,6 +1730,73 @@ static int defer_reduce(cg_backend *be, int kind, cg_tensor *x, const int64_t *o
     return CG_OK;
 }
 
+// x: the deferred RMS norm  v / pow(sum(v * v) / n + eps, e) * gamma  over the rows of [R, hd], v the whole of a decode-time
+// product [rows <= 4, N = heads * hd] that nobody has needed yet (the q / k norm of Qwen3, qwen3.rs:249-279).  Then x
+// becomes a plain view of a NEW open product that carries the norm (LazyMm::head_norm): the views, the rotary embedding and
+// the cache write that follow treat it like any open product, and the kernel that stores the embedded heads norms them on
+// the way (try_rope_stores).  False: not that shape; x is untouched.
+static bool head_norm_lazy(cg_tensor *x) {
+    static const uint8_t code[7][4] = {{kMul, 0, 0, 0},   {kRowSum, 8, 8, 8}, {kDiv, 9, 1, 9},  {kAdd, 10, 2, 10},
+                                       {kPow, 11, 3, 11}, {kDiv, 0, 12, 0},   {kMul, 13, 4, 13}};
+    const Pending *p = x->pend;
+    cg_backend *be = x->be;
+    if (!p || !be->aot || !be->fuse || x->dt != CG_F32 || x->rank != 2 || x->split >= 0) return false;
+    if (p->nleaf != 5 || p->ninstr != 7 || p->nred != 1 || p->reduced || p->overflow) return false;
+    for (int i = 0; i < 7; i++)
+        if (p->ins[i].op != code[i][0] || p->ins[i].a != code[i][1] || p->ins[i].b != code[i][2] || p->ins[i].c != code[i][3]) return false;
+    const int64_t R = x->dims[0], hd = x->dims[1];
+    if (hd < 16 || hd > 128 || hd % 16 || p->rowlen != hd || R < 1) return false;
+    const LeafView &lx = p->leaf[0], &lg = p->leaf[4];
+    if (lx.uniform || lx.pw || !lx.lazy || lx.lazy->result || lx.offset != 0 || lx.strides[1] != 1 || (R > 1 && lx.strides[0] != hd)) return false;
+    LazyMm *m = lx.lazy;
+    if (!m->groupable || !m->be || m->head_norm || m->rc.load() != 1 || m->rank < 1) return false;
+    int64_t n = 1;
+    for (int d = 0; d < m->rank; d++) n *= m->dims[d];
+    const int64_t N = m->dims[m->rank - 1], K = m->x->rank > 0 ? m->x->dims[m->x->rank - 1] : 0;
+    if (n != R * hd || N % hd || n / N > 4 || K <= 256 || K > 1024 || K % 4) return false; // (what the head-per-workgroup kernel takes)
+    if (!p->leaf[1].uniform || !p->leaf[2].uniform || !p->leaf[3].uniform) return false;
+    if (lg.uniform || lg.pw || lg.lazy || !lg.buf || is_narrow_buf(lg.buf) || lg.strides[1] != 1 || (R > 1 && lg.strides[0] != 0)) return false;
+    LazyMm *m2 = new LazyMm;
+    m2->x = m->x;
+    retain(m2->x);
+    m2->y = m->y;
+    retain(m2->y);
+    memcpy(m2->dims, m->dims, sizeof m2->dims);
+    m2->rank = m->rank;
+    m2->groupable = true;
+    m2->be = be;
+    be->lazy_open.push_back(m2);
+    m2->head_norm = true;
+    m2->hn_gamma = lg.buf;
+    m2->hn_gamma->rc.fetch_add(1);
+    m2->hn_gamma_off = lg.offset;
+    m2->hn_hd = (uint32_t)hd;
+    m2->hn_n_bits = p->leaf[1].ubits;
+    m2->hn_eps_bits = p->leaf[2].ubits;
+    m2->hn_exp_bits = p->leaf[3].ubits;
+    m2->hn_prog = new Pending(*p); // for whoever needs the value without the fused store: leaf 0 will read the plain product
+    lazy_mm_release(m2->hn_prog->leaf[0].lazy);
+    m2->hn_prog->leaf[0].lazy = nullptr;
+    m2->hn_prog->leaf[0].buf = nullptr;
+    memcpy(m2->hn_dims, x->dims, sizeof m2->hn_dims);
+    m2->hn_rank = x->rank;
+    Pending *np = new Pending;
+    LeafView lv{};
+    lv.lazy = m2;
+    lv.strides[0] = hd;
+    lv.strides[1] = 1;
+    add_leaf(np, lv, x->dims, x->rank);
+    lazy_mm_release(m2); // the leaf holds it now
+    Instr in;
+    in.op = (uint8_t)kCopy;
+    in.a = in.b = in.c = 0;
+    emit_instr(np, in);
+    Pending *old = x->pend;
+    x->pend = np;
+    delete old; // the plain product goes with it, never computed
+    return true;
+}
+
 // A view of a deferred tensor is the same program over re-strided leaves.  `fn` rewrites
 // one leaf (strides/offset) for the new shape; returns false when that leaf cannot be
 // viewed that way (then the tensor is made concrete and the caller takes the normal path).
@@ -1701,7 +1804,7 @@ template <class F>
 static int pending_view(cg_tensor *x, const int64_t *dims, int rank, F &&fn, cg_tensor **out, bool *handled) {
     *handled = false;
     if (!x->pend) return CG_OK;
-    if (x->pend->nred > 0) return ensure_concrete(x); // rows do not survive re-striding
+    if (x->pend->nred > 0 && !head_norm_lazy(x)) return ensure_concrete(x); // rows do not survive re-striding
     for (int l = 0; l < x->pend->nleaf; l++)
         if (x->pend->leaf[l].pw) return ensure_concrete(x); // nor does a split of the last axis
     int64_t n = 1;

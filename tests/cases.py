@@ -1372,8 +1372,12 @@ for _B, _K, _kvh, _rep, _T, _hd, _normed in ((4, 2048, 8, 4, 300, 64, True), (1,
                                               (3, 512, 4, 2, 200, 64, False), (3, 256, 4, 2, 200, 64, False), (4, 2048, 2, 4, 512, 32, False),
                                               # hidden sizes that are no multiple of 1024: a ragged chunk of k in the fused store
                                               (1, 576, 3, 3, 200, 64, True), (4, 576, 3, 3, 300, 64, False), (2, 1536, 4, 2, 131, 64, True),
-                                              (3, 2560, 2, 4, 260, 128, True)):
-    @case(f"decode_qkv_rope_append_B{_B}_K{_K}_kv{_kvh}_rep{_rep}_T{_T}_hd{_hd}{'_normed' if _normed else ''}", "red",
+                                              (3, 2560, 2, 4, 260, 128, True),
+                                              # q and k with an RMS norm per head ahead of the embedding (the Qwen3 attention block):
+                                              # the shapes whose store takes the norm (hidden up to 1024), and ones that do not
+                                              (1, 1024, 8, 2, 300, 128, "qk_normed"), (4, 1024, 2, 2, 200, 64, "qk"), (2, 576, 3, 3, 131, 64, "qk_normed"),
+                                              (3, 512, 2, 1, 257, 32, "qk"), (1, 2048, 2, 2, 100, 128, "qk_normed"), (2, 256, 2, 2, 90, 64, "qk")):
+    @case(f"decode_qkv_rope_append_B{_B}_K{_K}_kv{_kvh}_rep{_rep}_T{_T}_hd{_hd}{('_' + _normed) if isinstance(_normed, str) else '_normed' if _normed else ''}", "red",
           (lambda n=2 * 3: [np.float64(4.0)] * n))   # projections of order one, rows of the caches likewise: 1e-3 of 4
     def _(B=_B, K=_K, kvh=_kvh, rep=_rep, T=_T, hd=_hd, normed=_normed):
         """Two decode steps of an attention block (llama.rs:285-345): the q / k / v projections of one activation row
@@ -1383,6 +1387,8 @@ for _B, _K, _kvh, _rep, _T, _hd, _normed in ((4, 2048, 8, 4, 300, 64, True), (1,
         behind it), attention over the grown caches.  Where the extents allow it the embedding and the append run in
         the stores of the three products."""
         H = kvh * rep
+        qk = isinstance(normed, str)            # an RMS norm over head_dim on q and k (qwen3.rs:249-279)
+        normed = normed in (True, "qk_normed")
         r_ = np.random.default_rng(4400 + K + T)
         sc = np.float32(1.0 / np.sqrt(K))
         xs = [r_.standard_normal((B, 1, K)).astype(np.float32) for _ in range(2)]
@@ -1396,6 +1402,8 @@ for _B, _K, _kvh, _rep, _T, _hd, _normed in ((4, 2048, 8, 4, 300, 64, True), (1,
         cv = r_.standard_normal((B, kvh, T, hd)).astype(np.float32)
         ang = r_.uniform(0, 6.28, (T + 2, hd)).astype(np.float32)
         cos_t, sin_t = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+        gq = (1.0 + 0.1 * r_.standard_normal(hd)).astype(np.float32)
+        gk = (1.0 + 0.1 * r_.standard_normal(hd)).astype(np.float32)
 
         def run(be):
             k_cache, v_cache = be.from_numpy(ck), be.from_numpy(cv)
@@ -1424,6 +1432,14 @@ for _B, _K, _kvh, _rep, _T, _hd, _normed in ((4, 2048, 8, 4, 300, 64, True), (1,
                     return be.add(be.mul(c.move(), t.move()).move(), be.mul(s_.move(), rot.move()).move())
 
                 q, k, v = heads(q, H), heads(k, kvh), heads(v, kvh)
+                if qk:
+                    def head_norm(t, n, g):
+                        flat = be.reshape(t.move(), (B * n, hd))
+                        normed_t = _rmsnorm_ops(be, flat, be.from_numpy(g), hd, (B * n, hd))
+                        del flat   # (the graph interpreter gives every handle away at its last use)
+                        return be.reshape(normed_t.move(), (B, n, 1, hd))
+
+                    q, k = head_norm(q, H, gq), head_norm(k, kvh, gk)
                 q, k = rope(q, H), rope(k, kvh)
                 k_cache = be.concat(k_cache.move(), k.move(), 2)
                 v_cache = be.concat(v_cache.move(), v.move(), 2)
@@ -1444,6 +1460,9 @@ for _B, _K, _kvh, _rep, _T, _hd, _normed in ((4, 2048, 8, 4, 300, 64, True), (1,
                 q = (x @ wq.astype(f8).T).reshape(B, 1, H, hd).transpose(0, 2, 1, 3)
                 k = (x @ wk.astype(f8).T).reshape(B, 1, kvh, hd).transpose(0, 2, 1, 3)
                 v = (x @ wv.astype(f8).T).reshape(B, 1, kvh, hd).transpose(0, 2, 1, 3)
+                if qk:
+                    q = q / np.sqrt((q * q).mean(-1, keepdims=True) + 1e-5) * gq.astype(f8)
+                    k = k / np.sqrt((k * k).mean(-1, keepdims=True) + 1e-5) * gk.astype(f8)
                 c, s_ = cos_t[pos].astype(f8), sin_t[pos].astype(f8)
                 q, k = _np_rope(q, c, s_), _np_rope(k, c, s_)
                 K_, V_ = np.concatenate([K_, k], 2), np.concatenate([V_, v], 2)
