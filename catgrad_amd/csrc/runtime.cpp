@@ -1044,7 +1044,7 @@ static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p, b
             const int kind = (last.op & ~kInstrU32) == kRowMax ? kMax : kSum;
             const bool f32 = !(last.op & kInstrU32);
             cg_tensor *out = const_cast<cg_tensor *>(dst);
-            if (p.ninstr == 1 && !p.leaf[last.a].uniform) {
+            if (p.ninstr == 1 && !p.leaf[last.a].uniform && !p.leaf[last.a].pw) { // (a plain view: a two-part leaf is not one tensor)
                 cg_tensor leaf;
                 leaf_as_tensor(p, last.a, &space, f32 ? CG_F32 : CG_U32, &leaf);
                 leaf.be = be;
@@ -1059,7 +1059,8 @@ static int run_pending(cg_backend *be, const cg_tensor *dst, const Pending &p, b
         // the few results where they stand
         const Instr first = p.ins[0];
         if (p.reduced && p.nred == 1 && p.ninstr == 2 && is_row_reduce(first.op) && !(first.op & kInstrU32) && first.a < kMaxLeaves &&
-            !p.leaf[first.a].uniform && last.a == kMaxLeaves && (last.op == kRoundBF16 || last.op == kRoundF16 || last.op == kRoundF8) &&
+            !p.leaf[first.a].uniform && !p.leaf[first.a].pw && last.a == kMaxLeaves &&
+            (last.op == kRoundBF16 || last.op == kRoundF16 || last.op == kRoundF8) &&
             is_contiguous(dst)) {
             cg_tensor *out = const_cast<cg_tensor *>(dst);
             cg_tensor leaf;

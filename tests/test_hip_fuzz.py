@@ -150,6 +150,79 @@ def test_random_graph_matches_oracle(hip, oracle, seed):
         np.testing.assert_allclose(g, e, rtol=1e-4, atol=1e-5 * max(1.0, n.hi), err_msg=f"seed {seed} output {i}")
 
 
+class AsNarrow:
+    """A backend seen through a narrow float dtype: f32 arrays go up as their roundings to the dtype, results come back
+    widened, and a cast to F32 is a cast to the dtype — so the graphs above run as graphs of that dtype, every op rounding
+    its result to it."""
+
+    def __init__(self, be, dt):
+        self._be, self._dt = be, dt
+
+    def __getattr__(self, name):
+        return getattr(self._be, name)
+
+    def from_numpy(self, arr):
+        import cases_fp8
+        import cases_half
+
+        arr = np.asarray(arr)
+        if arr.dtype != np.float32:
+            return self._be.from_numpy(arr)
+        if self._dt == A.BF16:
+            return self._be.ndarray_from_vec_bf16(cases_half.bf16_round_bits(arr), arr.shape)
+        if self._dt == A.F16:
+            return self._be.ndarray_from_vec_f16(arr.astype(np.float16), arr.shape)
+        return self._be.ndarray_from_vec_fp8(cases_fp8.f8_encode(cases_fp8.f8_round(arr)), arr.shape)
+
+    def to_numpy(self, t):
+        import cases_fp8
+        import cases_half
+
+        a = self._be.to_numpy(t)
+        if a.dtype == np.uint16:
+            return cases_half.bf16_widen(a)
+        if a.dtype == np.float16:
+            return a.astype(np.float32)
+        return cases_fp8.f8_decode(a) if a.dtype == np.uint8 else a
+
+    def cast(self, t, dt):
+        return self._be.cast(t, self._dt if dt == A.F32 else dt)
+
+
+@pytest.fixture(scope="module")
+def hip_all_narrow():
+    """A backend that stores every tensor of a narrow dtype as 2- / 1-byte patterns, however small."""
+    from backends import backend_with_env
+
+    be = backend_with_env(CG_NARROW_FROM="2")
+    yield be
+    be.close()
+
+
+@pytest.mark.parametrize("seed", range(120))
+@pytest.mark.parametrize("dt", ["bf16", "f16", "fp8"])
+def test_random_graph_in_narrow_dtypes_matches_oracle(hip, hip_all_narrow, oracle, dt, seed):
+    """The same random graphs on bf16 / f16 / fp8 tensors, on the default backend (tensors of these sizes are 32-bit
+    words) and on one that keeps every tensor as 2- / 1-byte patterns: strided, broadcast, sliced and piecewise views of
+    narrow buffers, gathers, row programs and casts over them.  Every op rounds to the dtype on both sides, so exact
+    ancestry stays bit-exact; ops whose f32 result may differ in the last place (exp, sin, cos, sums) may differ by one
+    unit in the last place of the dtype."""
+    code, ulp = {"bf16": (A.BF16, 2.0 ** -8), "f16": (A.F16, 2.0 ** -11), "fp8": (A.F8, 2.0 ** -4)}[dt]
+    rng = np.random.default_rng(1000 + seed)
+    inputs, nodes, outs = random_graph(rng)
+    ref = evaluate(AsNarrow(oracle, code), inputs, nodes, outs)
+    for be in (hip, hip_all_narrow):
+        got = evaluate(AsNarrow(be, code), inputs, nodes, outs)
+        for i, (n, g, e) in enumerate(zip(outs, got, ref)):
+            assert g.shape == e.shape == n.shape and g.dtype == e.dtype
+            same = (g == e) | (np.isnan(g) & np.isnan(e))
+            if n.exact:
+                assert same.all(), f"seed {seed} output {i} (exact ancestry)"
+            else:
+                ok = same | (np.abs(g - e) <= 2 * ulp * np.maximum(np.abs(e), 2.0 ** -6 * max(1.0, n.hi)))
+                assert ok.all(), f"seed {seed} output {i}: worst {float(np.nanmax(np.abs(g - e)))}"
+
+
 @pytest.mark.parametrize("seed", range(200))
 def test_random_matmul_shapes_match_oracle(hip, oracle, seed):
     """[.., M, K] x [.., K, N] at random extents, either operand possibly a transposed or sliced view, the
