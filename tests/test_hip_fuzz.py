@@ -360,7 +360,7 @@ def test_random_attention_shapes_match_oracle(hip, oracle, seed):
     np.testing.assert_allclose(got, ref, rtol=1e-4, atol=2e-5, err_msg=f"seed {seed}: B={B} kvh={kvh} rep={rep} hd={hd} S={S} T={T}")
 
 
-@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("seed", range(28))
 def test_random_decoder_blocks_match_oracle(hip, oracle, seed):
     """The dense part of a decoder layer at decode time (residual add in the store of the o / down product, RMS norm in
     the loads of the products behind it, gated pair) with random row counts and widths, and with the results — norms and
@@ -370,9 +370,14 @@ def test_random_decoder_blocks_match_oracle(hip, oracle, seed):
 
     rng = np.random.default_rng(7000 + seed)
     B = int(rng.integers(1, 6))
-    H = int(rng.choice([2048, 2048, 4096, 1024, 3072, 512]))
-    F = int(rng.choice([4096, 6144, 8192]))
-    kv = int(rng.choice([256, 512, 2048]))
+    if seed < 12:
+        H = int(rng.choice([2048, 2048, 4096, 1024, 3072, 512]))
+        F = int(rng.choice([4096, 6144, 8192]))
+        kv = int(rng.choice([256, 512, 2048]))
+    else:   # widths that are no multiples of 1024 (ragged chunks of k, few columns)
+        H = int(rng.choice([576, 640, 960, 1536, 2560, 260, 1028]))
+        F = int(rng.choice([1536, 2560, 6912, 1540, 512]))
+        kv = int(rng.choice([192, 320, 576, 128]))
     sc = np.float32(1.0 / np.sqrt(H))
     r = lambda *s: rng.standard_normal(s).astype(np.float32)  # noqa: E731
     x0, a0 = r(B, 1, H), r(B, 1, H)
@@ -413,25 +418,29 @@ def test_random_decoder_blocks_match_oracle(hip, oracle, seed):
         np.testing.assert_allclose(gx, rx, rtol=1e-4, atol=1e-4)
 
 
-@pytest.mark.parametrize("seed", range(24))
+@pytest.mark.parametrize("seed", range(48))
 def test_random_attention_block_steps_match_oracle(hip, oracle, seed):
     """Decode steps of a whole attention block (q / k / v projections, heads split off, rotary embedding, cache append,
     attention) at random row counts, widths, head counts and sizes and cache lengths, with or without an RMS norm of a
     residual stream in front, and with random extra holders of the intermediate handles (a clone of a projection or of
     a roped tensor that is read later, the roped q read back before the attention): who else holds a product decides
-    whether the embedding and the append may run in the products' store.  1e-3 of the values' scale (order one)."""
+    whether the embedding and the append may run in the products' store.  From seed 24 on: hidden sizes that are no
+    multiples of 1024, and (half of them) an RMS norm per head on q and k between the projection and the embedding, as in
+    the Qwen3 block, with random holders of the normed tensors too.  1e-3 of the values' scale (order one)."""
     import cases
 
     rng = np.random.default_rng(11000 + seed)
     B = int(rng.integers(1, 6))
-    K = int(rng.choice([1024, 2048, 2048, 3072, 512]))
+    K = int(rng.choice([1024, 2048, 2048, 3072, 512])) if seed < 24 else int(rng.choice([576, 1024, 1024, 960, 1536, 640, 2048]))
     hd = int(rng.choice([64, 64, 128, 32]))
+    qk = seed >= 24 and bool(rng.random() < 0.6)
     kvh, rep = int(rng.integers(1, 5)), int(rng.choice([1, 2, 4]))
     H = kvh * rep
     T = int(rng.choice([int(rng.integers(1, 40)), int(rng.integers(200, 700)), int(rng.integers(1000, 2300))]))
     steps = int(rng.integers(1, 4))
     normed = bool(rng.random() < 0.5)
     keep = {n: bool(rng.random() < 0.2) for n in ("q_raw", "k_raw", "v_raw", "q_rope", "k_rope")}
+    keep.update({n: qk and bool(rng.random() < 0.15) for n in ("q_norm", "k_norm")})
     read_q_first = bool(rng.random() < 0.25)
     sc = np.float32(1.0 / np.sqrt(K))
     r = lambda *s: rng.standard_normal(s).astype(np.float32)  # noqa: E731
@@ -441,6 +450,7 @@ def test_random_attention_block_steps_match_oracle(hip, oracle, seed):
     ck, cv = r(B, kvh, T, hd), r(B, kvh, T, hd)
     ang = rng.uniform(0, 6.28, (T + steps, hd)).astype(np.float32)
     cos_t, sin_t = np.cos(ang).astype(np.float32), np.sin(ang).astype(np.float32)
+    gq, gk = (1 + 0.1 * r(hd)).astype(np.float32), (1 + 0.1 * r(hd)).astype(np.float32)
 
     def run(be):
         k_cache, v_cache = be.from_numpy(ck), be.from_numpy(cv)
@@ -473,6 +483,18 @@ def test_random_attention_block_steps_match_oracle(hip, oracle, seed):
                 return be.add(be.mul(c.move(), t.move()).move(), be.mul(s_.move(), rot.move()).move())
 
             q, k, v = heads(q, H), heads(k, kvh), heads(v, kvh)
+            if qk:
+                def head_norm(t, n, g):
+                    flat = be.reshape(t.move(), (B * n, hd))
+                    nt = cases._rmsnorm_ops(be, flat, be.from_numpy(g), hd, (B * n, hd))
+                    del flat
+                    return be.reshape(nt.move(), (B, n, 1, hd))
+
+                q, k = head_norm(q, H, gq), head_norm(k, kvh, gk)
+                if keep["q_norm"]:
+                    held["q_norm"] = q.clone()
+                if keep["k_norm"]:
+                    held["k_norm"] = k.clone()
             q, k = rope(q, H), rope(k, kvh)
             if keep["q_rope"]:
                 held["q_rope"] = q.clone()
@@ -490,7 +512,7 @@ def test_random_attention_block_steps_match_oracle(hip, oracle, seed):
 
     got, ref = run(hip), run(oracle)
     assert len(got) == len(ref)
-    what = f"seed {seed}: B={B} K={K} hd={hd} kvh={kvh} rep={rep} T={T} steps={steps} normed={normed} keep={keep} read_q_first={read_q_first}"
+    what = f"seed {seed}: B={B} K={K} hd={hd} kvh={kvh} rep={rep} T={T} steps={steps} normed={normed} qk={qk} keep={keep} read_q_first={read_q_first}"
     for i, (g, e) in enumerate(zip(got, ref)):
         assert g.shape == e.shape, what
         err = float(np.abs(g.astype(np.float64) - e).max())
