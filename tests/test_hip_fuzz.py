@@ -335,6 +335,61 @@ def test_random_wide_tile_products_of_16_bit_dtypes(hip, seed):
     assert bad.size == 0, f"seed {seed}: {len(bad)} mismatches, first {bad[:3].tolist()}"
 
 
+@pytest.mark.parametrize("seed", range(18))
+def test_random_products_of_operands_that_lie_narrow(hip, seed):
+    """Products of bf16 / f16 / fp8 tensors that lie in memory as 2- / 1-byte patterns (uploads of 65536 elements and
+    more): big ones (the 256 x 256 tile of narrow operands) and few-row ones (a decode-time linear layer), with the
+    operands whole — multiplied as they lie —, or cut by slices that move the first element off a 16-byte boundary, leave
+    a row pitch that is no multiple of 16 bytes or take a window of the rows (then narrowed or widened first), or
+    transposed so that k is not contiguous.  Small-integer values: every partial sum is exact in f32, so the result must
+    be the rounding of the exact product, bit for bit."""
+    import cases_fp8
+    import cases_half
+
+    rng = np.random.default_rng(9300 + seed)
+    dt = ("bf16", "f16", "fp8")[seed % 3]
+    few = seed % 2 == 1
+    M = int(rng.integers(1, 9)) if few else int(rng.integers(4097, 4400))
+    N = int(rng.integers(300, 2000)) if few else int(rng.integers(4097, 4400))
+    K = int(rng.choice([256, 512, 1024, 2048])) if few else int(rng.choice([64, 128, 192, 256]))
+    row_pad = int(rng.choice([0, 0, 8, 16, 3]))         # extra columns in the weight's rows (a slice takes K of them)
+    col_off = int(rng.choice([0, 0, 8, 16, 1])) if row_pad else 0
+    col_off = min(col_off, row_pad)
+    row_off = int(rng.choice([0, 0, 5, 64]))             # rows skipped at the top of the weight
+    yt = bool(rng.random() < 0.2)                         # the weight as [K, N] (k not contiguous)
+    lim = 3 if dt == "fp8" else 6
+    xv = rng.integers(-lim, lim + 1, size=(M, K)).astype(np.float32)
+    wv = rng.integers(-lim, lim + 1, size=(N + row_off, K + row_pad)).astype(np.float32)
+
+    def up(v):
+        v = np.ascontiguousarray(v)
+        if dt == "fp8":
+            return hip.ndarray_from_vec_fp8(cases_fp8.f8_encode(v), v.shape)
+        code = A.BF16 if dt == "bf16" else A.F16
+        return cases_half.from_half(hip, code, cases_half.round_to(code, v))
+
+    a = up(xv)
+    if yt:
+        b = up(np.ascontiguousarray(wv[row_off:, col_off:col_off + K].T))
+    else:
+        w = up(wv)
+        if row_off:
+            w = hip.slice(w, 0, row_off, N)
+        if row_pad:
+            w = hip.slice(w, 1, col_off, K)
+        b = hip.transpose(w, 0, 1)
+    print(f"seed={seed} dtype={dt} M={M} N={N} K={K} row_pad={row_pad} col_off={col_off} row_off={row_off} yt={yt}", flush=True)
+    got = hip.to_numpy(hip.matmul(a, b))
+    exact = (xv.astype(np.float64) @ wv[row_off:, col_off:col_off + K].astype(np.float64).T).astype(np.float32)
+    if dt == "fp8":
+        got, exp = cases_fp8.f8_decode(got), cases_fp8.f8_round(exact)
+    else:
+        code = A.BF16 if dt == "bf16" else A.F16
+        got, exp = cases_half.as_f32(code, got), cases_half.as_f32(code, cases_half.round_to(code, exact))
+    bad = np.argwhere(got != exp)
+    assert bad.size == 0, f"seed {seed}: {len(bad)} mismatches, first {bad[:3].tolist()}"
+
+
 @pytest.mark.parametrize("seed", range(120))
 def test_random_attention_shapes_match_oracle(hip, oracle, seed):
     """The model graphs' attention (repeat_kv, scores, scale, causal mask rows, soft-max, context) at random
