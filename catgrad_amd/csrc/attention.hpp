@@ -1,4 +1,4 @@
-// Decode-time attention in one pass (included by fused.hip after aot_programs.hpp).
+// Decode-time attention in one pass (included by attention.hip after interp.hpp).
 //
 // A decode step issues, per layer, q.K^T (at most 8 query rows per KV head after the GQA
 // group is folded into rows), the soft-max program over the scores, and p.V.  Each of the

@@ -12,8 +12,7 @@
 // Arithmetic follows NdArrayBackend (catgrad/src/interpreter/backend/ndarray.rs):
 // IEEE f32 with one rounding per operation (the file is compiled with
 // -ffp-contract=off), accurate libm-grade sin/cos/exp/log/pow, wrapping u32.
-#include "common.hpp"
-#include "device_utils.hpp"
+#include "ew_kernel.hpp"
 
 #include <algorithm>
 #include <type_traits>
@@ -21,115 +20,6 @@
 namespace cg {
 
 namespace {
-
-constexpr int kBlock = 256;
-constexpr int kUnroll = 4;
-constexpr uint64_t kStreamItems = 4u << 20; // work items (64 MiB of 16-byte vectors) from which outputs stream past the caches
-
-struct EwArgs {
-    EwGeom g;
-    Operand out;
-    Operand in[3];
-    uint32_t *fault;
-    uint32_t round; // kRoundBF16 / kRoundF16 / kRoundF8: the result is rounded to that format before it is stored; 0: not
-};
-
-// FLAT: the iteration space collapsed to a single axis (no index arithmetic at all).
-template <int OP, bool F, int NIN, int VEC, bool FLAT>
-__global__ __launch_bounds__(kBlock) void ew_kernel(const EwArgs a) {
-    const uint64_t base = (uint64_t)blockIdx.x * (kBlock * kUnroll) + threadIdx.x;
-    int64_t off[kUnroll][4];
-    bool live[kUnroll];
-#pragma unroll
-    for (int u = 0; u < kUnroll; u++) {
-        uint64_t v64 = base + (uint64_t)u * kBlock;
-        live[u] = v64 < a.g.total;
-        uint32_t v = (uint32_t)v64;
-        if (FLAT) {
-            int64_t e = (int64_t)v * VEC;
-            off[u][0] = e * a.out.is;
-#pragma unroll
-            for (int k = 0; k < NIN; k++) off[u][k + 1] = e * a.in[k].is;
-        } else {
-            uint32_t row = fastdiv(v, a.g.ipr_div);
-            int64_t e = (int64_t)(v - row * a.g.ipr) * VEC;
-            int64_t oo = e * a.out.is;
-            int64_t oi[3];
-#pragma unroll
-            for (int k = 0; k < NIN; k++) oi[k] = e * a.in[k].is;
-            for (uint32_t d = 0; d < a.g.nouter; d++) {
-                uint32_t q = fastdiv(row, a.g.odiv[d]);
-                int64_t i = (int64_t)(row - q * a.g.od[d]);
-                row = q;
-                oo += i * a.out.os[d];
-#pragma unroll
-                for (int k = 0; k < NIN; k++) oi[k] += i * a.in[k].os[d];
-            }
-            off[u][0] = oo;
-#pragma unroll
-            for (int k = 0; k < NIN; k++) off[u][k + 1] = oi[k];
-        }
-    }
-    uint32_t x[kUnroll][3][VEC];
-#pragma unroll
-    for (int u = 0; u < kUnroll; u++)
-        if (live[u]) {
-#pragma unroll
-            for (int k = 0; k < NIN; k++) {
-                // fully collapsed space: a unit-stride operand is read exactly once, so it need not
-                // displace anything from the caches either
-                if (FLAT && a.g.total >= kStreamItems) load_words<VEC, true>(a.in[k], off[u][k + 1], x[u][k]);
-                else load_words<VEC>(a.in[k], off[u][k + 1], x[u][k]);
-            }
-        }
-#pragma unroll
-    for (int u = 0; u < kUnroll; u++)
-        if (live[u]) {
-            uint32_t r[VEC];
-#pragma unroll
-            for (int j = 0; j < VEC; j++)
-                r[j] = apply<OP, F>(x[u][0][j], NIN > 1 ? x[u][1 % NIN][j] : 0u, NIN > 2 ? x[u][2 % NIN][j] : 0u, a.fault);
-            if (F && a.round) { // (the same for every lane: a launch parameter)
-#pragma unroll
-                for (int j = 0; j < VEC; j++)
-                    r[j] = a.round == kRoundBF16 ? apply<kRoundBF16, true>(r[j], 0u, 0u, a.fault)
-                           : a.round == kRoundF16 ? apply<kRoundF16, true>(r[j], 0u, 0u, a.fault)
-                                                  : apply<kRoundF8, true>(r[j], 0u, 0u, a.fault);
-            }
-            if (a.g.total >= kStreamItems) store_words<VEC, true>(a.out, off[u][0], r);
-            else store_words<VEC>(a.out, off[u][0], r);
-        }
-}
-
-template <int OP, bool F, int NIN> int launch_variants(cg_backend *be, const EwArgs &a) {
-    uint64_t per_block = (uint64_t)kBlock * kUnroll;
-    uint64_t blocks = (a.g.total + per_block - 1) / per_block;
-    if (blocks == 0) return CG_OK;
-    dim3 grid((uint32_t)blocks), block(kBlock);
-    bool flat = a.g.nouter == 0;
-    if (a.g.vec == 8) {
-        if (flat)
-            hipLaunchKernelGGL((ew_kernel<OP, F, NIN, 8, true>), grid, block, 0, be->stream, a);
-        else
-            hipLaunchKernelGGL((ew_kernel<OP, F, NIN, 8, false>), grid, block, 0, be->stream, a);
-    } else if (a.g.vec == 4) {
-        if (flat)
-            hipLaunchKernelGGL((ew_kernel<OP, F, NIN, 4, true>), grid, block, 0, be->stream, a);
-        else
-            hipLaunchKernelGGL((ew_kernel<OP, F, NIN, 4, false>), grid, block, 0, be->stream, a);
-    } else {
-        if (flat)
-            hipLaunchKernelGGL((ew_kernel<OP, F, NIN, 1, true>), grid, block, 0, be->stream, a);
-        else
-            hipLaunchKernelGGL((ew_kernel<OP, F, NIN, 1, false>), grid, block, 0, be->stream, a);
-    }
-    hipError_t e = hipGetLastError();
-    return e == hipSuccess ? CG_OK : hip_fail(e, "element-wise kernel launch");
-}
-
-template <int OP, int NIN> int launch_by_dtype(cg_backend *be, cg_dtype dt, const EwArgs &a) {
-    return is_f(dt) ? launch_variants<OP, true, NIN>(be, a) : launch_variants<OP, false, NIN>(be, a);
-}
 
 __global__ void arange_kernel(uint32_t *out, uint32_t n) {
     uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -334,29 +224,9 @@ int launch_elementwise(cg_backend *be, int op, cg_dtype dt, const cg_tensor *out
         const int trc = try_transpose_copy(be, a);
         if (trc != kDeclined) return trc;
     }
-    switch (op) {
-#define CG_EW1(OP) case OP: return launch_by_dtype<OP, 1>(be, dt, a);
-#define CG_EW2(OP) case OP: return launch_by_dtype<OP, 2>(be, dt, a);
-    CG_EW1(kNeg)
-    case kSin: return launch_variants<kSin, true, 1>(be, a);
-    case kCos: return launch_variants<kCos, true, 1>(be, a);
-    case kExp: return launch_variants<kExp, true, 1>(be, a);
-    case kLog: return launch_variants<kLog, true, 1>(be, a);
-    case kFloor: return launch_variants<kFloor, true, 1>(be, a);
-    case kRound: return launch_variants<kRound, true, 1>(be, a);
-    case kRoundBF16: return launch_variants<kRoundBF16, true, 1>(be, a);
-    case kRoundF16: return launch_variants<kRoundF16, true, 1>(be, a);
-    case kRoundF8: return launch_variants<kRoundF8, true, 1>(be, a);
-    CG_EW2(kAdd) CG_EW2(kSub) CG_EW2(kMul) CG_EW2(kDiv) CG_EW2(kPow)
-    CG_EW2(kLt) CG_EW2(kGt) CG_EW2(kGte) CG_EW2(kLte) CG_EW2(kEq)
-    case kWhere: return launch_by_dtype<kWhere, 3>(be, dt, a);
-    case kCastF2U: return launch_variants<kCastF2U, true, 1>(be, a);
-    case kCastU2F: return launch_variants<kCastU2F, false, 1>(be, a);
-    case kCopy: return launch_variants<kCopy, false, 1>(be, a);
-#undef CG_EW1
-#undef CG_EW2
-    default: return fail(CG_ERR_ARG, "unknown element-wise op %d", op);
-    }
+    return a.g.vec == 8   ? launch_ew_vec<8>(be, op, dt, a)
+           : a.g.vec == 4 ? launch_ew_vec<4>(be, op, dt, a)
+                          : launch_ew_vec<1>(be, op, dt, a);
 }
 
 int launch_arange(cg_backend *be, cg_tensor *out) {
