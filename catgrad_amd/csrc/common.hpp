@@ -104,6 +104,7 @@ struct cg_backend {
     bool narrow_storage = true;  // tensors of the narrow float dtypes keep 2- / 1-byte elements in memory (CG_NARROW_STORAGE=0: 32-bit words)
     int64_t narrow_from = 65536; // ... from this many elements on (CG_NARROW_FROM); smaller tensors stay 32-bit words: the kernels of a
                                  // decode step, which address words, never meet a narrow operand that way
+    int compute_units = 256;     // of the device (a persistent kernel launches one workgroup for each)
     bool trace_programs = false; // CG_TRACE_PROGRAMS=1: print each distinct deferred program once, to stderr
     cg::ProfClass prof[CG_K_CLASSES];
     std::vector<cg::ProfPending> prof_pending;
@@ -480,6 +481,8 @@ int launch_topk(cg_backend *be, const cg_tensor *x, int64_t k, cg_tensor *vals, 
 int launch_any_positive(cg_backend *be, const cg_tensor *x);
 int launch_any_diff(cg_backend *be, const cg_tensor *x, const cg_tensor *y);
 
+// out == nullptr: nothing is launched; CG_OK if this product would run on the kernel that can round a narrow dtype's
+// result in its store (then `out` may hold that dtype's format), kDeclined if not.
 int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_tensor *out);
 
 // The batch structure of x . y after collapsing: batch axes that both operands walk as one run

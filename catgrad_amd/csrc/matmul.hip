@@ -66,6 +66,7 @@ struct MmArgs {
     uint32_t batch;
     uint32_t a_vec, b_vec;          // 16-byte loads along the unit-stride axis are legal
     uint32_t ksplit;                // mfma_gemm_kernel: values of k per workgroup along grid.z (a multiple of 32), 0 = all of K
+    uint32_t c_fmt;                 // mfma_gemm_dlds_kernel: kFmtWords, or the operands' narrow format: C holds its patterns, rounded in the store
 };
 
 __device__ __forceinline__ void batch_offsets(const MmArgs &a, uint32_t b, int64_t &oa, int64_t &ob) {
@@ -187,6 +188,9 @@ constexpr int PITCH_H = BK / 2 + 4;
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
 typedef long long2v __attribute__((ext_vector_type(2)));
+typedef float float2v __attribute__((ext_vector_type(2)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t uint4v __attribute__((ext_vector_type(4)));
 typedef int int4v __attribute__((ext_vector_type(4)));
 typedef int int8v __attribute__((ext_vector_type(8)));
@@ -680,6 +684,360 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
                 }
             }
         }
+}
+
+// ------------------------------------------------------------------------------------------
+// The 256 x 256 tile of operands that lie narrow in memory, fed by loads that go from memory straight into LDS
+// (global_load_lds_dwordx4): no tile registers, no LDS stores, so what a workgroup has in flight is bounded by LDS
+// instead of by registers.  The register-staged kernel above keeps one tile step (64 KB) in flight per compute unit
+// and a step lasts as long as a trip to memory (about 2 us under load, 31 GB/s per unit, whatever the matrix pipes
+// could take); here a step is 64 bytes of k per row (32 values of 16 bits, 64 of fp8), a stage is 32 KB and LDS holds a
+// ring of kDldsStages of them: one being multiplied, the others in flight.
+// A row's 64 bytes are four 16-byte columns; column c of row r sits at column c ^ ((r >> 1) & 3) of the row's place, so
+// that the eight lanes of a 128-bit fragment read (eight consecutive rows, one logical column) cover all 32 banks.  A
+// load instruction of a wave fills 1 KB = 16 consecutive rows in lane order: lane l fetches row l / 4, logical column
+// (l % 4) ^ ((row >> 1) & 3).
+// HALF: 3 bfloat16, 4 binary16 (two 16-deep steps per stage), 5 fp8 (one 64-deep step per stage).  a.K counts 32-bit
+// words and is a multiple of 64 (whole turns of the ring); rows beyond the edge are clamped as above.
+// ------------------------------------------------------------------------------------------
+constexpr int kDldsStages = 4;
+constexpr uint32_t kDldsOperandBytes = 256 * 64, kDldsStageBytes = 2 * kDldsOperandBytes;
+constexpr size_t kDldsLdsBytes = (size_t)kDldsStages * kDldsStageBytes;
+
+template <int HALF, bool NARROW_OUT> __global__ __launch_bounds__(kThreads) void mfma_gemm_dlds_kernel(const MmArgs a) {
+    constexpr int NS = kDldsStages;
+    static_assert(NS == 4, "the last stages of a tile below are written out for a ring of four");
+    extern __shared__ float lds_dyn[];
+    typedef __attribute__((address_space(3))) char lds_char;
+    lds_char *const lds = (lds_char *)lds_dyn;
+
+    // Tile order as in mfma_gemm_kernel: a run of tiles per XCD, down a column of kGroupM row tiles first.  The grid is one
+    // workgroup per compute unit (or per tile if there are fewer); workgroup b takes tiles b, b + grid, b + 2 grid, ...
+    const uint32_t tiles_n = (a.N + 255) / 256, tiles_m = (a.M + 255) / 256;
+    const uint32_t ntiles = tiles_m * tiles_n;
+    auto tile_origin = [&](const uint32_t vb, uint32_t &m0, uint32_t &n0) {
+        const uint32_t xcd = vb % kXcds, slot = vb / kXcds;
+        const uint32_t q = ntiles / kXcds, r = ntiles % kXcds;
+        const uint32_t lin = xcd * q + (xcd < r ? xcd : r) + slot;
+        const uint32_t per_group = kGroupM * tiles_n;
+        const uint32_t group = lin / per_group, in_group = lin % per_group;
+        const uint32_t first_m = group * kGroupM;
+        const uint32_t gsize = (tiles_m - first_m) < kGroupM ? (tiles_m - first_m) : kGroupM;
+        m0 = (first_m + in_group % gsize) * 256;
+        n0 = (in_group / gsize) * 256;
+    };
+
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x / 64), lane = threadIdx.x % 64;
+    const uint32_t wm = (wave / 2) * 128, wn = (wave % 2) * 128;
+    const uint32_t li = lane % 32, lg = lane / 32;
+
+    // this lane's share of a stage: instruction q of wave w fills rows 64 w + 16 q .. + 15 of an operand's place
+    uint32_t offa[4], offb[4];
+    auto set_offa = [&](const uint32_t m0) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const uint32_t row = wave * 64 + q * 16 + lane / 4, col = (lane % 4) ^ ((row >> 1) & 3);
+            offa[q] = (uint32_t)((uint64_t)min(m0 + row, a.M - 1) * (uint64_t)a.a_sm * 4 + col * 16);
+        }
+    };
+    auto set_offb = [&](const uint32_t n0) {
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const uint32_t row = wave * 64 + q * 16 + lane / 4, col = (lane % 4) ^ ((row >> 1) & 3);
+            offb[q] = (uint32_t)((uint64_t)min(n0 + row, a.N - 1) * (uint64_t)a.b_sn * 4 + col * 16);
+        }
+    };
+    const char *const ga = reinterpret_cast<const char *>(a.A), *const gb = reinterpret_cast<const char *>(a.B);
+    // load q of stage kt (of the tile whose offsets are set): 0..3 the four of A, 4..7 the four of B
+    auto issue = [&](const uint32_t kt, const int q) {
+        const char *const p = (q < 4 ? ga : gb) + (uint64_t)kt * 64 + (q < 4 ? offa[q & 3] : offb[q & 3]);
+        lds_char *const l = lds + (kt % NS) * kDldsStageBytes + (q < 4 ? 0u : kDldsOperandBytes) + wave * 4096 + (q & 3) * 1024;
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)p, (__attribute__((address_space(3))) void *)l, 16, 0, 0);
+    };
+    // fragment addresses: row li of a 32-row block, logical column c -> byte li * 64 + ((c ^ sw) * 16)
+    const uint32_t sw = (li >> 1) & 3;
+    auto frag = [&](const uint32_t stage_base, const uint32_t row0, const uint32_t c) {
+        return *reinterpret_cast<const __attribute__((address_space(3))) float4v *>(lds + stage_base + (row0 + li) * 64 + ((c ^ sw) * 16));
+    };
+
+    float16v acc[4][4];
+    auto clear = [&]() {
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+#pragma unroll
+                for (int v = 0; v < 16; v++) acc[i][j][v] = 0.0f;
+    };
+    // D layout of the 32 x 32 instructions: lane (li, lg), register v -> row 8 (v / 4) + 4 lg + v % 4, column li.  A whole
+    // tile is stored at a per-lane 32-bit offset from addresses that are the same for every lane (M N < 2^30).
+    // With NARROW_OUT the result is rounded to the operands' format here (what the separate rounding pass over the f32 result
+    // would give, bit for bit) and stored as its patterns, a quarter or an eighth of the bytes of that f32 result and pass:
+    // lanes exchange values so that each stores 32 bits — two columns of one row (16-bit: lanes pair up, the even lane takes
+    // the first of two rows, the odd lane the second) or four (fp8: a quad transposes its 4 x 4 values).
+    auto pattern = [&](const float x) -> uint32_t {
+        if constexpr (HALF == 3) return round_bf16_bits(asu(x)) >> 16;
+        else if constexpr (HALF == 4) return (uint32_t)__half_as_ushort(__float2half_rn(x));
+        else return (uint32_t)f8_byte_of(round_f8_bits(asu(x)));
+    };
+    const uint32_t lane_off = ((wm + 4 * lg) * a.N + wn + li) * 4;
+    const uint32_t sub = HALF == 5 ? (li & 3) : (li & 1); // this lane's row among the 4 (2) that its group exchanges
+    const uint32_t lane_off_narrow = ((wm + 4 * lg + sub) * a.N + wn + li - sub) * (HALF == 5 ? 1 : 2);
+    // v_perm_b32 selectors of the quad's transposition (byte values 0..3: the second source's bytes, 4..7: the first's, 12: zero)
+    const uint32_t quad_sel_a = (0x0C0C0C0Cu & ~(0xFFu << (8 * sub)) & ~(0xFFu << (8 * ((sub + 1) & 3)))) | (sub << (8 * sub)) | ((4 + sub) << (8 * ((sub + 1) & 3)));
+    const uint32_t quad_sel_b = (0x0C0C0C0Cu & ~(0xFFu << (8 * ((sub + 2) & 3))) & ~(0xFFu << (8 * ((sub + 3) & 3)))) | (sub << (8 * ((sub + 2) & 3))) |
+                                ((4 + sub) << (8 * ((sub + 3) & 3)));
+    auto store = [&](const uint32_t m0, const uint32_t n0) {
+        const bool whole = m0 + 256 <= a.M && n0 + 256 <= a.N;
+        if (whole && !NARROW_OUT) {
+            char *const base = reinterpret_cast<char *>(a.C) + ((uint64_t)m0 * a.N + n0) * 4;
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+#pragma unroll
+                    for (int v = 0; v < 16; v++) {
+                        const uint32_t r = i * 32 + 8 * (v / 4) + (v % 4);
+                        // (written out: the compiler would keep a 64-bit address per row in vector registers)
+                        asm volatile("global_store_dword %0, %1, %2" ::"v"(lane_off), "v"(acc[i][j][v]), "s"(base + ((uint64_t)r * a.N + j * 32) * 4) : "memory");
+                    }
+                    __builtin_amdgcn_sched_barrier(0); // (a block at a time: its 16 values pass through 16 registers)
+                }
+            return;
+        }
+        if (whole) {
+            constexpr uint32_t EB = HALF == 5 ? 1 : 2;
+            char *const base = reinterpret_cast<char *>(a.C) + ((uint64_t)m0 * a.N + n0) * EB;
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    if constexpr (HALF != 5) {
+#pragma unroll
+                        for (int v = 0; v < 16; v += 2) {
+                            // v_cvt_pk_{bf16,f16}_f32 round two values as the rounding pass does (all 2^32 patterns compared)
+                            const float2v pair = {acc[i][j][v], acc[i][j][v + 1]};
+                            uint32_t mine;
+                            if constexpr (HALF == 3) mine = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, bf16x2));
+                            else mine = __builtin_bit_cast(uint32_t, __builtin_convertvector(pair, f16x2));
+                            const uint32_t theirs = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mine, 0xB1, 0xF, 0xF, true); // the pair's other lane
+                            // even lane: its and the other's first row; odd lane: the other's and its second row
+                            const uint32_t two = __builtin_amdgcn_perm(theirs, mine, sub ? 0x03020706u : 0x05040100u);
+                            const uint32_t r = i * 32 + 8 * (v / 4) + (v % 4);
+                            asm volatile("global_store_dword %0, %1, %2" ::"v"(lane_off_narrow), "v"(two), "s"(base + ((uint64_t)r * a.N + j * 32) * 2) : "memory");
+                        }
+                    } else {
+#pragma unroll
+                        for (int v = 0; v < 16; v += 4) {
+                            // v_cvt_pk_fp8_f32 rounds as the rounding pass does once the magnitude is clamped to 448 (it holds no
+                            // infinities) and NaNs are set apart: they become the clamped pattern 0x7e, which the 0x7f below completes
+                            // (all 2^32 patterns compared)
+                            float xs[4];
+                            uint32_t nans = 0;
+#pragma unroll
+                            for (int k = 0; k < 4; k++) {
+                                const uint32_t u = asu(acc[i][j][v + k]), mag = u & 0x7FFFFFFFu;
+                                xs[k] = asf(min(mag, 0x43E00000u) | (u & 0x80000000u));
+                                nans |= mag > 0x7F800000u ? 0x7Fu << (8 * k) : 0u;
+                            }
+                            int packed = __builtin_amdgcn_cvt_pk_fp8_f32(xs[0], xs[1], 0, false);
+                            packed = __builtin_amdgcn_cvt_pk_fp8_f32(xs[2], xs[3], packed, true);
+                            const uint32_t mine = (uint32_t)packed | nans; // byte k: row k of this lane's column
+                            // lane q of the quad keeps row q: byte q of every lane's word, at the place of that lane's column
+                            const uint32_t r1 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mine, 0x39, 0xF, 0xF, true); // of lane q + 1
+                            const uint32_t r2 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mine, 0x4E, 0xF, 0xF, true); // of lane q + 2
+                            const uint32_t r3 = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)mine, 0x93, 0xF, 0xF, true); // of lane q + 3
+                            const uint32_t four = __builtin_amdgcn_perm(r1, mine, quad_sel_a) | __builtin_amdgcn_perm(r3, r2, quad_sel_b);
+                            const uint32_t r = i * 32 + 8 * (v / 4);
+                            asm volatile("global_store_dword %0, %1, %2" ::"v"(lane_off_narrow), "v"(four), "s"(base + ((uint64_t)r * a.N + j * 32)) : "memory");
+                        }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            return;
+        }
+#pragma unroll
+        for (int i = 0; i < 4; i++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const uint32_t col = n0 + wn + j * 32 + li;
+                if (col < a.N) {
+#pragma unroll
+                    for (int v = 0; v < 16; v++) {
+                        const uint32_t row = m0 + wm + i * 32 + 8 * (v / 4) + 4 * lg + (v % 4);
+                        if (row < a.M) {
+                            const uint64_t at = (uint64_t)row * a.N + col;
+                            if constexpr (!NARROW_OUT) a.C[at] = asu(acc[i][j][v]);
+                            else if constexpr (HALF == 5) reinterpret_cast<uint8_t *>(a.C)[at] = (uint8_t)pattern(acc[i][j][v]);
+                            else reinterpret_cast<uint16_t *>(a.C)[at] = (uint16_t)pattern(acc[i][j][v]);
+                        }
+                    }
+                }
+                __builtin_amdgcn_sched_barrier(0);
+            }
+    };
+
+    const uint32_t nk = a.K / 16; // a multiple of NS: stage kt of every tile sits in place kt % NS of the ring
+    uint32_t vb = blockIdx.x, m0, n0;
+    tile_origin(vb, m0, n0);
+    set_offa(m0);
+    set_offb(n0);
+    // A wave's loads wait for each other in the texture path (a KB each), and while one waits the wave issues nothing:
+    // they are dealt out one behind every group of matrix instructions.  The first half of stage kt asks for the second
+    // half of the loads (B) of the stage 3 ahead, its second half (behind the barrier, when the place of stage kt is free) for
+    // the first half (A) of the stage 4 ahead.  The stages of a workgroup's tiles form one stream: the last four stages of a
+    // tile ask for the first stages of the next, and the matrix pipes pause at a tile's end only for the stores of the result.
+#pragma unroll
+    for (int s = 0; s < NS - 1; s++)
+#pragma unroll
+        for (int q = 0; q < 8; q++) issue(s, q);
+#pragma unroll
+    for (int q = 0; q < 4; q++) issue(NS - 1, q);
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0x0f70 | (20 & 15) | ((20 >> 4) << 14)); // vmcnt(20): stage 0 is in LDS
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+
+    // wait until at most `stages` younger stages are in flight and every fragment read has returned, then meet the others:
+    // the next stage is in LDS for everybody, and nobody reads the current stage's place any more.  (Loads finish in the
+    // order asked for; the stores of a finished tile share the counter and only make the wait longer than needed.)
+    auto meet = [&](auto stages) {
+        constexpr uint32_t n = decltype(stages)::value * 8;
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(0x0070 | (n & 15) | ((n >> 4) << 14)); // vmcnt(n) lgkmcnt(0)
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+    };
+    typedef std::integral_constant<int, 2> Y2;
+    typedef std::true_type Ask;
+
+    if constexpr (HALF != 5) {
+        float4v fa[2][4], fb[2][4];
+        auto mma_row = [&](const int set, const int i) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                if constexpr (HALF == 3)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, fa[set][i]),
+                                                                        __builtin_bit_cast(bf16x8, fb[set][j]), acc[i][j], 0, 0, 0);
+                else
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, fa[set][i]),
+                                                                       __builtin_bit_cast(f16x8, fb[set][j]), acc[i][j], 0, 0, 0);
+            }
+        };
+        // step c of a stage: lane group g supplies the 8 values of k at 16 c + 8 g: logical column 2 c + g
+        auto read = [&](const uint32_t kt, const int set, const int c, const int i) {
+            const uint32_t base = (kt % NS) * kDldsStageBytes;
+            fa[set][i] = frag(base, wm + i * 32, c * 2 + lg);
+            fb[set][i] = frag(base + kDldsOperandBytes, wn + i * 32, c * 2 + lg);
+        };
+#pragma unroll
+        for (int i = 0; i < 4; i++) read(0, 0, 0, i);
+        // YOUNGER: stages younger than the next one that may still be in flight when this stage meets the others (-1: the
+        // last stage of the last tile); FIRST / SECOND: the loads dealt out in the two halves are those of stages fkt / skt
+        auto stage = [&](const uint32_t kt, auto younger, auto first, auto second, const uint32_t fkt, const uint32_t skt) {
+            constexpr int YOUNGER = decltype(younger)::value;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                read(kt, 1, 1, i);
+                mma_row(0, i);
+                if constexpr (decltype(first)::value) issue(fkt, 4 + i);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+            if constexpr (YOUNGER >= 0) meet(std::integral_constant<uint32_t, (uint32_t)(YOUNGER < 0 ? 0 : YOUNGER)>{});
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                if constexpr (YOUNGER >= 0) read(kt + 1, 0, 0, i);
+                mma_row(1, i);
+                if constexpr (decltype(second)::value) issue(skt, i);
+                __builtin_amdgcn_sched_barrier(0);
+            }
+        };
+        for (;;) {
+            // (a workgroup's last tile asks for its own first stages again: one way through the loop, and loads nobody reads)
+            const uint32_t nvb = vb + gridDim.x;
+            const bool more = nvb < ntiles;
+            uint32_t nm0, nn0;
+            tile_origin(more ? nvb : vb, nm0, nn0);
+            clear();
+            uint32_t kt = 0;
+            for (; kt + NS < nk; kt++) stage(kt, Y2{}, Ask{}, Ask{}, kt + NS - 1, kt + NS);
+            set_offa(nm0);
+            stage(kt, Y2{}, Ask{}, Ask{}, kt + NS - 1, 0);
+            set_offb(nn0);
+            stage(kt + 1, Y2{}, Ask{}, Ask{}, 0, 1);
+            stage(kt + 2, Y2{}, Ask{}, Ask{}, 1, 2);
+            stage(kt + 3, Y2{}, Ask{}, Ask{}, 2, 3);
+            store(m0, n0);
+            if (!more) break;
+            vb = nvb, m0 = nm0, n0 = nn0;
+        }
+    } else {
+        // fp8: a lane feeds the 64-deep instruction 32 bytes of its row — logical columns g and 2 + g (A and B agree on
+        // which bytes of the 64 they are).  The fragments of a stage sit in one of two register sets, the stage's parity;
+        // the next stage's are read behind the barrier, under the second half of this stage's instructions.
+        int8v fa8[2][4], fb8[2][4];
+        auto read8 = [&](const uint32_t kt, const int set, const int i) {
+            const uint32_t base = (kt % NS) * kDldsStageBytes;
+            const int4v alo = __builtin_bit_cast(int4v, frag(base, wm + i * 32, lg)), ahi = __builtin_bit_cast(int4v, frag(base, wm + i * 32, 2 + lg));
+            fa8[set][i] = __builtin_shufflevector(alo, ahi, 0, 1, 2, 3, 4, 5, 6, 7);
+            const int4v blo = __builtin_bit_cast(int4v, frag(base + kDldsOperandBytes, wn + i * 32, lg)),
+                        bhi = __builtin_bit_cast(int4v, frag(base + kDldsOperandBytes, wn + i * 32, 2 + lg));
+            fb8[set][i] = __builtin_shufflevector(blo, bhi, 0, 1, 2, 3, 4, 5, 6, 7);
+        };
+        auto mma8 = [&](const int set, const int i, const int j) {
+            acc[i][j] = __builtin_amdgcn_mfma_scale_f32_32x32x64_f8f6f4(fa8[set][i], fb8[set][j], acc[i][j], 0, 0, 0, 0x7f7f7f7f, 0, 0x7f7f7f7f);
+        };
+#pragma unroll
+        for (int i = 0; i < 4; i++) read8(0, 0, i);
+        // (a load behind every second matrix instruction, which is twice as long as a 16-bit one)
+        auto stage8 = [&](const uint32_t kt, const int set, auto younger, auto first, auto second, const uint32_t fkt, const uint32_t skt) {
+            constexpr int YOUNGER = decltype(younger)::value;
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    mma8(set, i, 2 * h);
+                    mma8(set, i, 2 * h + 1);
+                    if constexpr (decltype(first)::value) issue(fkt, 4 + 2 * i + h);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            if constexpr (YOUNGER >= 0) meet(std::integral_constant<uint32_t, (uint32_t)(YOUNGER < 0 ? 0 : YOUNGER)>{});
+#pragma unroll
+            for (int i = 2; i < 4; i++)
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    if constexpr (YOUNGER >= 0) read8(kt + 1, set ^ 1, 2 * (i - 2) + h);
+                    mma8(set, i, 2 * h);
+                    mma8(set, i, 2 * h + 1);
+                    if constexpr (decltype(second)::value) issue(skt, 2 * (i - 2) + h);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+        };
+        for (;;) {
+            const uint32_t nvb = vb + gridDim.x;
+            const bool more = nvb < ntiles;
+            uint32_t nm0, nn0;
+            tile_origin(more ? nvb : vb, nm0, nn0);
+            clear();
+            uint32_t kt = 0;
+            for (; kt + NS < nk; kt += 2) {
+                stage8(kt, 0, Y2{}, Ask{}, Ask{}, kt + NS - 1, kt + NS);
+                stage8(kt + 1, 1, Y2{}, Ask{}, Ask{}, kt + NS, kt + NS + 1);
+            }
+            set_offa(nm0);
+            stage8(kt, 0, Y2{}, Ask{}, Ask{}, kt + NS - 1, 0);
+            set_offb(nn0);
+            stage8(kt + 1, 1, Y2{}, Ask{}, Ask{}, 0, 1);
+            stage8(kt + 2, 0, Y2{}, Ask{}, Ask{}, 1, 2);
+            stage8(kt + 3, 1, Y2{}, Ask{}, Ask{}, 2, 3);
+            store(m0, n0);
+            if (!more) break;
+            vb = nvb, m0 = nm0, n0 = nn0;
+        }
+    }
+    // (loads into LDS must not outlive the workgroup: its LDS passes to the next one)
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_waitcnt(0x0070); // vmcnt(0) lgkmcnt(0)
 }
 
 // ------------------------------------------------------------------------------------------
@@ -2208,7 +2566,7 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
     if (int frc = flush_deferred(be)) return frc;
     MmArgs a;
     MmFold f;
-    int rc = mm_geometry(x, y, out->buf->ptr, &a, &f);
+    int rc = mm_geometry(x, y, out ? out->buf->ptr : nullptr, &a, &f);
     if (rc) return rc;
     const int64_t M = f.M, N = f.N, K = f.K, batch = f.batch;
     const bool a_mfast = !(a.a_sk == 1 || K == 1) && a.a_sm == 1;
@@ -2259,6 +2617,24 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
     const bool y_native = (skinny_packed && native_rows(y, kind, a.b_sn, a.b_sk, K, true)) || (big_packed && native_rows(y, kind, a.b_sn, a.b_sk, K, false));
     rc = mm_operand(y, false, y_native, &a);
     if (rc) return rc;
+    // Whole stages of 64 bytes of k in whole turns of the ring, 16-byte rows, byte offsets that fit 32 bits: the wide tile
+    // fed by loads straight into LDS (env CG_GEMM_DLDS=0: the register-staged one).  Only that kernel can round the result
+    // to the operands' format in its store; without `out` the call just says whether this product would run on it.
+    static const bool dlds_allowed = [] {
+        const char *e = getenv("CG_GEMM_DLDS");
+        return !(e && e[0] == '0');
+    }();
+    const int64_t per = kind == 3 ? 4 : 2;           // elements per 32-bit word
+    const int64_t kw = kind ? K / per : 0;           // words per row
+    const int64_t a_pitch = x_native ? a.a_sm / per : kw, b_pitch = y_native ? a.b_sn / per : kw; // (a view taken as it lies keeps its own row pitch)
+    const bool dlds = big_packed && dlds_allowed && kw % (16 * kDldsStages) == 0 && a_pitch % 4 == 0 && b_pitch % 4 == 0 &&
+                      (!x_native || reinterpret_cast<uintptr_t>(native_ptr(x)) % 16 == 0) && (!y_native || reinterpret_cast<uintptr_t>(native_ptr(y)) % 16 == 0) &&
+                      (uint64_t)M * (uint64_t)a_pitch * 4 < (1ull << 32) && (uint64_t)N * (uint64_t)b_pitch * 4 < (1ull << 32) &&
+                      (uint64_t)M * (uint64_t)N < (1ull << 30);
+    const bool can_round = dlds && N % 4 == 0 && kind != 3; // (fp8 results take the separate rounding pass)
+    if (!out) return can_round ? CG_OK : kDeclined;
+    const int c_fmt = out->buf->fmt;
+    if (c_fmt != kFmtWords && !can_round) return fail(CG_ERR_ARG, "matmul: a narrow result needs the kernel that rounds in its store");
     const double flop = 2.0 * (double)M * (double)N * (double)K * (double)batch;
     const double bytes = distinct_bytes(x) + distinct_bytes(y) + distinct_bytes(out);
     const bool simple = K == 0 || !f32, skinny = !simple && M <= 8 && (a.b_sk == 1 || a.b_sn == 1);
@@ -2456,16 +2832,33 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
             if (!prc && !y_native) prc = pack_operand(be, words_buffer(y), a.B, a.b_sn, a.b_sk, N, K, kind, true, &pb, &tb, &cb);
             if (!prc) {
                 MmArgs p = a;
-                const int64_t per = kind == 3 ? 4 : 2;      // elements per 32-bit word
-                const int64_t kw = K / per;                 // words per row
                 p.A = static_cast<const uint32_t *>(pa);
                 p.B = static_cast<const uint32_t *>(pb);
                 p.K = (uint32_t)kw;
-                p.a_sm = x_native ? a.a_sm / per : kw; // (a view taken as it lies keeps its own row pitch)
-                p.b_sn = y_native ? a.b_sn / per : kw;
+                p.a_sm = a_pitch;
+                p.b_sn = b_pitch;
                 p.a_sk = p.b_sk = 1;
                 p.a_vec = p.b_vec = 1;
-                if (kind == 1) hipLaunchKernelGGL((mfma_gemm_kernel<false, false, 4, 4, 3>), grid, dim3(kThreads), gemm_lds_bytes(256, 256), s, p);
+                p.c_fmt = (uint32_t)c_fmt;
+                static const bool dlds_ok = [] {
+                    bool ok = true;
+#define CG_DLDS_LDS(H, NARROW)                                                                                                 \
+    ok &= hipFuncSetAttribute(reinterpret_cast<const void *>(&mfma_gemm_dlds_kernel<H, NARROW>), hipFuncAttributeMaxDynamicSharedMemorySize, \
+                              (int)kDldsLdsBytes) == hipSuccess;
+                    CG_DLDS_LDS(3, false) CG_DLDS_LDS(3, true) CG_DLDS_LDS(4, false) CG_DLDS_LDS(4, true) CG_DLDS_LDS(5, false)
+#undef CG_DLDS_LDS
+                    return ok;
+                }();
+                if (dlds && !dlds_ok) prc = fail(CG_ERR_DEVICE, "matmul: cannot reserve %zu bytes of LDS", kDldsLdsBytes);
+                else if (dlds) {
+                    const dim3 pgrid((uint32_t)std::min<uint64_t>(tiles, (uint64_t)be->compute_units)); // its workgroups walk the tiles
+                    const bool narrow_out = c_fmt != kFmtWords;
+                    if (kind == 1 && narrow_out) hipLaunchKernelGGL((mfma_gemm_dlds_kernel<3, true>), pgrid, dim3(kThreads), kDldsLdsBytes, s, p);
+                    else if (kind == 1) hipLaunchKernelGGL((mfma_gemm_dlds_kernel<3, false>), pgrid, dim3(kThreads), kDldsLdsBytes, s, p);
+                    else if (kind == 2 && narrow_out) hipLaunchKernelGGL((mfma_gemm_dlds_kernel<4, true>), pgrid, dim3(kThreads), kDldsLdsBytes, s, p);
+                    else if (kind == 2) hipLaunchKernelGGL((mfma_gemm_dlds_kernel<4, false>), pgrid, dim3(kThreads), kDldsLdsBytes, s, p);
+                    else hipLaunchKernelGGL((mfma_gemm_dlds_kernel<5, false>), pgrid, dim3(kThreads), kDldsLdsBytes, s, p);
+                } else if (kind == 1) hipLaunchKernelGGL((mfma_gemm_kernel<false, false, 4, 4, 3>), grid, dim3(kThreads), gemm_lds_bytes(256, 256), s, p);
                 else if (kind == 2) hipLaunchKernelGGL((mfma_gemm_kernel<false, false, 4, 4, 4>), grid, dim3(kThreads), gemm_lds_bytes(256, 256), s, p);
                 else hipLaunchKernelGGL((mfma_gemm_kernel<false, false, 4, 4, 5>), grid, dim3(kThreads), gemm_lds_bytes(256, 256), s, p);
             }

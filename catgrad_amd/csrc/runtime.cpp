@@ -2130,6 +2130,7 @@ int cg_backend_create(int device, cg_backend **out) {
     if (const char *nf = getenv("CG_NARROW_FROM")) b->narrow_from = std::max<int64_t>(atoll(nf), 2);
     const char *trace = getenv("CG_TRACE_PROGRAMS");
     b->trace_programs = trace && trace[0] == '1';
+    b->compute_units = std::max(prop.multiProcessorCount, 1);
     char name[256];
     snprintf(name, sizeof name, "hip:%s (%s, %d CUs)%s", prop.gcnArchName, prop.name, prop.multiProcessorCount,
              b->fuse ? "" : " [unfused]");
@@ -2804,15 +2805,16 @@ int cg_where(cg_backend *b, cg_tensor *mask, cg_tensor *x, cg_tensor *y, cg_tens
 
 // ---- contraction / reductions ---------------------------------------------------------------------
 // ndarray.rs:176-183, 750-816
-static int matmul_entry(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **out);
+static int matmul_entry(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **out, bool *rounded);
 // The 16-bit float dtypes: products of exactly held values, summed in f32, rounded once.
 int cg_matmul(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **out) {
     Enter entered(b);
     const cg_dtype dt = x ? x->dt : CG_F32;
-    int rc = matmul_entry(b, x, y, out);
-    return rc ? rc : round_result(b, dt, out);
+    bool rounded = false; // (by the product's own store)
+    int rc = matmul_entry(b, x, y, out, &rounded);
+    return rc || rounded ? rc : round_result(b, dt, out);
 }
-static int matmul_entry(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **out) {
+static int matmul_entry(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **out, bool *rounded) {
     Consume cx(x), cy(y);
     if (b && b->owner_gone) return fail(CG_ERR_ARG, "backend used after cg_backend_destroy");
     if (!b || !x || !y || !out) return fail(CG_ERR_ARG, "null argument");
@@ -2915,8 +2917,18 @@ static int matmul_entry(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **o
         }
     }
     CG_HIP(hipSetDevice(b->device));
+    // A big product of a narrow dtype whose result is stored narrow rounds in its own store when the kernel it runs on can
+    // (asked first: launch_matmul without a result), and leaves the patterns; otherwise f32 words, rounded by the caller.
+    int64_t n_res = 1;
+    for (int i = 0; i < r; i++) n_res *= od[i];
+    int fmt = is_narrow(x->dt) && n_res > 0 ? result_fmt(b, x->dt, n_res) : kFmtWords;
+    if (fmt != kFmtWords) {
+        rc = launch_matmul(b, x, y, nullptr);
+        if (rc == kDeclined) fmt = kFmtWords;
+        else if (rc) return rc;
+    }
     cg_tensor *o;
-    rc = new_dense(b, x->dt, od, r, &o);
+    rc = new_dense(b, x->dt, od, r, &o, 0, fmt);
     if (rc) return rc;
     if (numel(o) > 0) {
         rc = launch_matmul(b, x, y, o);
@@ -2925,6 +2937,7 @@ static int matmul_entry(cg_backend *b, cg_tensor *x, cg_tensor *y, cg_tensor **o
             return rc;
         }
     }
+    *rounded = fmt != kFmtWords;
     *out = o;
     return CG_OK;
 }

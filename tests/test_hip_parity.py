@@ -510,6 +510,62 @@ def test_narrow_operand_products_carry_special_values(hip, dt):
         assert np.isnan(got[300, 400])
 
 
+def _narrow_codec(hip, dt):
+    import cases_fp8
+    import cases_half
+    if dt == "fp8":
+        up = lambda v: hip.ndarray_from_vec_fp8(cases_fp8.f8_encode(v), v.shape)
+        rd = lambda t: cases_fp8.read(hip, t)
+        rnd = cases_fp8.f8_round
+    else:
+        code = A.BF16 if dt == "bf16" else A.F16
+        up = lambda v: cases_half.from_half(hip, code, cases_half.round_to(code, v))
+        rd = lambda t: cases_half.as_f32(code, cases_half.read(hip, t))
+        rnd = lambda x: cases_half.as_f32(code, cases_half.round_to(code, x))
+    return up, rd, rnd
+
+
+def _small_integers(rng, dt, M, N, K):
+    if dt == "fp8":
+        av = rng.integers(-2, 3, size=(M, K)).astype(np.float32)
+        bv = (rng.integers(-1, 2, size=(N, K)) * (rng.random((N, K)) < 0.125)).astype(np.float32)
+    else:
+        av = rng.integers(-8, 9, size=(M, K)).astype(np.float32)
+        bv = rng.integers(-8, 9, size=(N, K)).astype(np.float32)
+    return av, bv
+
+
+@pytest.mark.parametrize("dt", ["bf16", "f16", "fp8"])
+@pytest.mark.parametrize("shape", ["ragged_edges", "partial_last_round"])
+def test_narrow_operand_products_through_the_lds_ring_are_exact_on_integers(hip, hip_words_only, dt, shape):
+    """Rows of k that are whole turns of the four-stage ring (multiples of 128 values of the 16-bit dtypes, of 256 of fp8)
+    take the kernel whose loads go straight into LDS and whose workgroups walk the tiles: one per compute unit, so 17 x 16
+    tiles end with a round in which few workgroups have a tile left, and 32 x 33 tiles take four full rounds and a partial
+    one.  The 16-bit dtypes round the result in that kernel's store (two columns per lane, exchanged between neighbours);
+    with 32-bit storage (the second backend) the same kernel stores f32 words and the rounding pass follows.  Small
+    integers make the exact product the only right answer (see the test above); 4000 x 4100 leaves ragged tiles at both
+    edges, which take the guarded store; a sliced left operand has a row pitch of twice its width."""
+    rng = np.random.default_rng(79)
+    M, N, K = (4000, 4100, 1280) if shape == "ragged_edges" else (8192, 8448, 256)
+    av, bv = _small_integers(rng, dt, M, N, K)
+    exp32 = av @ bv.T                                   # (sgemm on small integers: every partial sum is exact)
+    assert np.abs(exp32).max() < 2 ** 24
+    for be in (hip, hip_words_only):
+        print(f"dt={dt} shape={shape} storage={'words' if be is hip_words_only else 'narrow'}", flush=True)
+        up, rd, rnd = _narrow_codec(be, dt)
+        exp = rnd(exp32)
+        a, b = up(av), up(bv)
+        got = rd(be.matmul(a, be.transpose(b, 0, 1)))
+        bad = np.argwhere(got != exp)
+        assert bad.size == 0, f"{dt}: {len(bad)} mismatches, first {bad[:3].tolist()}"
+        if shape == "ragged_edges":
+            # the left operand as the right half of a tensor twice as wide
+            wide = up(np.concatenate([np.zeros_like(av), av], axis=1))
+            got = rd(be.matmul(be.slice(wide, 1, K, K), be.transpose(b, 0, 1)))
+            assert np.array_equal(got, exp)
+        del a, b, got
+
+
 # ---- full-size checks through size-independent properties -----------------------------------
 def test_microbench_shapes_properties(hip):
     """Config-2 shapes: linearity / invariants instead of a CPU recomputation."""
