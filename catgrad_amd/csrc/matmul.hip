@@ -693,10 +693,11 @@ __global__ __launch_bounds__(kThreads) void mfma_gemm_kernel(const MmArgs a) {
 // and a step lasts as long as a trip to memory (about 2 us under load, 31 GB/s per unit, whatever the matrix pipes
 // could take); here a step is 64 bytes of k per row (32 values of 16 bits, 64 of fp8), a stage is 32 KB and LDS holds a
 // ring of kDldsStages of them: one being multiplied, the others in flight.
-// A row's 64 bytes are four 16-byte columns; column c of row r sits at column c ^ ((r >> 1) & 3) of the row's place, so
-// that the eight lanes of a 128-bit fragment read (eight consecutive rows, one logical column) cover all 32 banks.  A
-// load instruction of a wave fills 1 KB = 16 consecutive rows in lane order: lane l fetches row l / 4, logical column
-// (l % 4) ^ ((row >> 1) & 3).
+// A row's 64 bytes are four 16-byte columns; column c of row r sits at column c ^ ((r >> 2) & 3) of the row's place, so
+// that the sixteen lanes that a 128-bit fragment read serves at a time (sixteen consecutive rows, one logical column)
+// cover all 64 banks (counted: no bank conflicts; with (r >> 1) & 3, which spreads eight rows over 32 banks, every read
+// took two turns).  A load instruction of a wave fills 1 KB = 16 consecutive rows in lane order: lane l fetches row
+// l / 4, logical column (l % 4) ^ ((row >> 2) & 3).
 // HALF: 3 bfloat16, 4 binary16 (two 16-deep steps per stage), 5 fp8 (one 64-deep step per stage).  a.K counts 32-bit
 // words and is a multiple of 64 (whole turns of the ring); rows beyond the edge are clamped as above.
 // ------------------------------------------------------------------------------------------
@@ -736,14 +737,14 @@ template <int HALF, bool NARROW_OUT> __global__ __launch_bounds__(kThreads) void
     auto set_offa = [&](const uint32_t m0) {
 #pragma unroll
         for (int q = 0; q < 4; q++) {
-            const uint32_t row = wave * 64 + q * 16 + lane / 4, col = (lane % 4) ^ ((row >> 1) & 3);
+            const uint32_t row = wave * 64 + q * 16 + lane / 4, col = (lane % 4) ^ ((row >> 2) & 3);
             offa[q] = (uint32_t)((uint64_t)min(m0 + row, a.M - 1) * (uint64_t)a.a_sm * 4 + col * 16);
         }
     };
     auto set_offb = [&](const uint32_t n0) {
 #pragma unroll
         for (int q = 0; q < 4; q++) {
-            const uint32_t row = wave * 64 + q * 16 + lane / 4, col = (lane % 4) ^ ((row >> 1) & 3);
+            const uint32_t row = wave * 64 + q * 16 + lane / 4, col = (lane % 4) ^ ((row >> 2) & 3);
             offb[q] = (uint32_t)((uint64_t)min(n0 + row, a.N - 1) * (uint64_t)a.b_sn * 4 + col * 16);
         }
     };
@@ -755,7 +756,7 @@ template <int HALF, bool NARROW_OUT> __global__ __launch_bounds__(kThreads) void
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)p, (__attribute__((address_space(3))) void *)l, 16, 0, 0);
     };
     // fragment addresses: row li of a 32-row block, logical column c -> byte li * 64 + ((c ^ sw) * 16)
-    const uint32_t sw = (li >> 1) & 3;
+    const uint32_t sw = (li >> 2) & 3;
     auto frag = [&](const uint32_t stage_base, const uint32_t row0, const uint32_t c) {
         return *reinterpret_cast<const __attribute__((address_space(3))) float4v *>(lds + stage_base + (row0 + li) * 64 + ((c ^ sw) * 16));
     };
@@ -850,6 +851,7 @@ template <int HALF, bool NARROW_OUT> __global__ __launch_bounds__(kThreads) void
                             const uint32_t four = __builtin_amdgcn_perm(r1, mine, quad_sel_a) | __builtin_amdgcn_perm(r3, r2, quad_sel_b);
                             const uint32_t r = i * 32 + 8 * (v / 4);
                             asm volatile("global_store_dword %0, %1, %2" ::"v"(lane_off_narrow), "v"(four), "s"(base + ((uint64_t)r * a.N + j * 32)) : "memory");
+                            __builtin_amdgcn_sched_barrier(0);
                         }
                     }
                     __builtin_amdgcn_sched_barrier(0);
@@ -2631,7 +2633,7 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
                       (!x_native || reinterpret_cast<uintptr_t>(native_ptr(x)) % 16 == 0) && (!y_native || reinterpret_cast<uintptr_t>(native_ptr(y)) % 16 == 0) &&
                       (uint64_t)M * (uint64_t)a_pitch * 4 < (1ull << 32) && (uint64_t)N * (uint64_t)b_pitch * 4 < (1ull << 32) &&
                       (uint64_t)M * (uint64_t)N < (1ull << 30);
-    const bool can_round = dlds && N % 4 == 0 && kind != 3; // (fp8 results take the separate rounding pass)
+    const bool can_round = dlds && N % 4 == 0;
     if (!out) return can_round ? CG_OK : kDeclined;
     const int c_fmt = out->buf->fmt;
     if (c_fmt != kFmtWords && !can_round) return fail(CG_ERR_ARG, "matmul: a narrow result needs the kernel that rounds in its store");
@@ -2845,7 +2847,7 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
 #define CG_DLDS_LDS(H, NARROW)                                                                                                 \
     ok &= hipFuncSetAttribute(reinterpret_cast<const void *>(&mfma_gemm_dlds_kernel<H, NARROW>), hipFuncAttributeMaxDynamicSharedMemorySize, \
                               (int)kDldsLdsBytes) == hipSuccess;
-                    CG_DLDS_LDS(3, false) CG_DLDS_LDS(3, true) CG_DLDS_LDS(4, false) CG_DLDS_LDS(4, true) CG_DLDS_LDS(5, false)
+                    CG_DLDS_LDS(3, false) CG_DLDS_LDS(3, true) CG_DLDS_LDS(4, false) CG_DLDS_LDS(4, true) CG_DLDS_LDS(5, false) CG_DLDS_LDS(5, true)
 #undef CG_DLDS_LDS
                     return ok;
                 }();
@@ -2857,6 +2859,7 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
                     else if (kind == 1) hipLaunchKernelGGL((mfma_gemm_dlds_kernel<3, false>), pgrid, dim3(kThreads), kDldsLdsBytes, s, p);
                     else if (kind == 2 && narrow_out) hipLaunchKernelGGL((mfma_gemm_dlds_kernel<4, true>), pgrid, dim3(kThreads), kDldsLdsBytes, s, p);
                     else if (kind == 2) hipLaunchKernelGGL((mfma_gemm_dlds_kernel<4, false>), pgrid, dim3(kThreads), kDldsLdsBytes, s, p);
+                    else if (narrow_out) hipLaunchKernelGGL((mfma_gemm_dlds_kernel<5, true>), pgrid, dim3(kThreads), kDldsLdsBytes, s, p);
                     else hipLaunchKernelGGL((mfma_gemm_dlds_kernel<5, false>), pgrid, dim3(kThreads), kDldsLdsBytes, s, p);
                 } else if (kind == 1) hipLaunchKernelGGL((mfma_gemm_kernel<false, false, 4, 4, 3>), grid, dim3(kThreads), gemm_lds_bytes(256, 256), s, p);
                 else if (kind == 2) hipLaunchKernelGGL((mfma_gemm_kernel<false, false, 4, 4, 4>), grid, dim3(kThreads), gemm_lds_bytes(256, 256), s, p);
