@@ -96,16 +96,16 @@ def micro_bench(iters=20):
     y = be.from_numpy(rng.standard_normal((16, 1024, 1024), dtype=np.float32))
     run("bmm_f32_16x1024x1024x1024", A.K_GEMM_MFMA, lambda: be.matmul(x, y), "TFLOP/s")
     del x, y
-    # a linear layer of the 1B-shape prefill on the narrow dtypes (the reduced-precision row of the path): operands narrowed
-    # to 2-byte / 1-byte patterns in memory (the weight once, the activations — new ones every launch — inside the timed launch), then the 16-bit /
-    # fp8 matrix instructions; against their dense peaks
+    # a linear layer of the 1B-shape prefill on the narrow dtypes (the reduced-precision row of the path): both operands lie
+    # in memory as 2-byte / 1-byte patterns (the weight cast once, the activations by a cast per launch, which is an
+    # element-wise launch of its own) and are multiplied as they lie on the 16-bit / fp8 matrix instructions, the result
+    # rounded to the dtype in the product's store; against the dense peaks of those instructions
     x32 = be.from_numpy(rng.standard_normal((1, 8192, 2048), dtype=np.float32) * np.float32(0.25))
     w32 = be.from_numpy(rng.standard_normal((8192, 2048), dtype=np.float32) * np.float32(0.25))
     for dt, tag, peak in ((A.BF16, "bf16", 2.5e15), (A.F8, "fp8", 5.0e15)):
         wn = be.cast(w32, dt)
         be.realize(wn)
         wv = be.broadcast(be.transpose(wn, 0, 1), (1, 2048, 8192))
-        # fresh activations per launch (the library keeps a buffer's narrowed copy, as it does the weight's)
         run(f"linear_{tag}_8192x2048x8192", A.K_GEMM_MFMA, lambda: be.matmul(be.cast(x32, dt), wv), "TFLOP/s", mfma_peak=peak)
         del wn, wv
     del x32, w32
