@@ -390,6 +390,57 @@ def test_random_products_of_operands_that_lie_narrow(hip, seed):
     assert bad.size == 0, f"seed {seed}: {len(bad)} mismatches, first {bad[:3].tolist()}"
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_random_products_through_the_lds_ring(hip, seed):
+    """Big products of narrow operands whose rows of k are whole turns of the four-stage LDS ring (random multiples of 128
+    values of the 16-bit dtypes, of 256 of fp8): the kernel whose workgroups walk the tiles, at random extents (ragged
+    tiles, more or fewer tiles than four rounds), with a result width that is a multiple of 4 (rounded in the product's
+    store) or not (f32 result and the rounding pass), the weight whole or as a window of wider rows.  Small integers: the
+    rounding of the exact product, bit for bit."""
+    import cases_fp8
+    import cases_half
+
+    rng = np.random.default_rng(9400 + seed)
+    dt = ("bf16", "f16", "fp8")[seed % 3]
+    M = int(rng.integers(3600, 5200))
+    N = int(rng.integers(3600, 5200))
+    if seed % 2 == 0:
+        N -= N % 4
+    if M * N < 256 * 65536 + 300000:       # (at least 256 tiles of 256 x 256)
+        M = 4200
+    K = (256 * int(rng.integers(1, 5))) if dt == "fp8" else (128 * int(rng.integers(1, 11)))
+    row_pad = int(rng.choice([0, 0, 16, 32]))
+    col_off = int(rng.choice([0, 16])) if row_pad else 0
+    col_off = min(col_off, row_pad)
+    lim = 3 if dt == "fp8" else 6
+    xv = rng.integers(-lim, lim + 1, size=(M, K)).astype(np.float32)
+    wv = rng.integers(-lim, lim + 1, size=(N, K + row_pad)).astype(np.float32)
+    if dt == "fp8":
+        wv *= (rng.random(wv.shape) < 0.25)        # (sums stay small enough for fp8's few exact integers to matter)
+
+    def up(v):
+        v = np.ascontiguousarray(v)
+        if dt == "fp8":
+            return hip.ndarray_from_vec_fp8(cases_fp8.f8_encode(v), v.shape)
+        code = A.BF16 if dt == "bf16" else A.F16
+        return cases_half.from_half(hip, code, cases_half.round_to(code, v))
+
+    w = up(wv)
+    if row_pad:
+        w = hip.slice(w, 1, col_off, K)
+    print(f"seed={seed} dtype={dt} M={M} N={N} K={K} row_pad={row_pad} col_off={col_off}", flush=True)
+    got = hip.to_numpy(hip.matmul(up(xv), hip.transpose(w, 0, 1)))
+    exact = xv @ wv[:, col_off:col_off + K].T          # (sgemm on small integers: exact)
+    assert np.abs(exact).max() < 2 ** 24
+    if dt == "fp8":
+        got, exp = cases_fp8.f8_decode(got), cases_fp8.f8_round(exact)
+    else:
+        code = A.BF16 if dt == "bf16" else A.F16
+        got, exp = cases_half.as_f32(code, got), cases_half.as_f32(code, cases_half.round_to(code, exact))
+    bad = np.argwhere(got != exp)
+    assert bad.size == 0, f"seed {seed}: {len(bad)} mismatches, first {bad[:3].tolist()}"
+
+
 @pytest.mark.parametrize("seed", range(120))
 def test_random_attention_shapes_match_oracle(hip, oracle, seed):
     """The model graphs' attention (repeat_kv, scores, scale, causal mask rows, soft-max, context) at random
