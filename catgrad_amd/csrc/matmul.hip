@@ -1285,15 +1285,15 @@ __device__ __forceinline__ uint32_t norm_divisor(const NormFuse &nf, float sum) 
 // takes a quarter of the chunk in a row (2 KiB in a row of each weight row: measured 12 % faster on the gate / up pair than
 // interleaving the waves every 256 bytes).  A ragged last chunk: the waves interleaved every 64 values of k, so that what
 // there is of the chunk is shared by all four.
-template <int TRIPS> __device__ __forceinline__ void xreg_lane_k(uint32_t K, uint32_t wave, uint32_t b, uint32_t &kb, uint32_t &ks) {
-    const bool ragged = K % (TRIPS * 256) != 0;
+// WHOLE: K is known to be whole chunks (the kernels branch once, at their top: loads without a test per trip).
+template <int TRIPS, bool WHOLE = false> __device__ __forceinline__ void xreg_lane_k(uint32_t K, uint32_t wave, uint32_t b, uint32_t &kb, uint32_t &ks) {
+    const bool ragged = !WHOLE && K % (TRIPS * 256) != 0;
     kb = (ragged ? wave * 64 : wave * (TRIPS * 64)) + b * 4;
     ks = ragged ? 256u : 64u;
 }
-template <int MM, int CG, bool GATED = false, bool RESIDUAL = false, bool NORM = false, int TRIPS = 8>
-__device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const uint32_t block_x, const uint32_t block_y,
-                                                         const uint32_t *second = nullptr, const uint32_t one = 0,
-                                                         const MmResidual *res = nullptr, const NormFuse *nf = nullptr) {
+template <bool WHOLE, int MM, int CG, bool GATED, bool RESIDUAL, bool NORM, int TRIPS>
+__device__ __forceinline__ void skinny_kt_mfma_xreg_body_impl(const MmArgs &a, const uint32_t block_x, const uint32_t block_y, const uint32_t *second,
+                                                              const uint32_t one, const MmResidual *res, const NormFuse *nf) {
     static_assert(!NORM || MM == 4, "the norm's row sums are kept for four rows");
     static_assert(!GATED || CG == 2, "a gated pair is two column groups");
     static_assert(!(GATED && RESIDUAL), "one epilogue at a time");
@@ -1344,7 +1344,7 @@ __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const 
     // of every chunk of TRIPS * 256 values of k (2048 or 1024) a wave takes a quarter in a row (TRIPS trips of 64)
     static_assert(TRIPS == 8 || TRIPS == 4, "chunks of 2048 or 1024");
     uint32_t kb, ks;
-    xreg_lane_k<TRIPS>(a.K, wave, b, kb, ks);
+    xreg_lane_k<TRIPS, WHOLE>(a.K, wave, b, kb, ks);
     for (uint32_t k0 = 0; k0 < a.K; k0 += TRIPS * 256) {
         float4v xr[G][TRIPS];
 #pragma unroll
@@ -1353,7 +1353,7 @@ __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const 
 #pragma unroll
             for (int g = 0; g < G; g++) {
                 xr[g][t] = (float4v){0.f, 0.f, 0.f, 0.f};
-                if (k < a.K) xr[g][t] = *reinterpret_cast<const float4v *>(xrow[g] + k);
+                if (WHOLE || k < a.K) xr[g][t] = *reinterpret_cast<const float4v *>(xrow[g] + k);
             }
         }
         float4v gm[NORM ? TRIPS : 1]; // asked for with the activations, multiplied in once the first weights are on their way
@@ -1362,7 +1362,7 @@ __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const 
             for (int t = 0; t < TRIPS; t++) {
                 const uint32_t k = k0 + kb + ks * t;
                 gm[t] = (float4v){0.f, 0.f, 0.f, 0.f};
-                if (k < a.K) gm[t] = *reinterpret_cast<const float4v *>(nf->gamma + k);
+                if (WHOLE || k < a.K) gm[t] = *reinterpret_cast<const float4v *>(nf->gamma + k);
             }
         }
 #pragma unroll
@@ -1372,7 +1372,7 @@ __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const 
             for (int t = 0; t < TRIPS; t++) {
                 const uint32_t k = k0 + kb + ks * t;
                 w[t] = (float4v){0.f, 0.f, 0.f, 0.f};
-                if (k < a.K) w[t] = *reinterpret_cast<const float4v *>(wrow[c] + k);
+                if (WHOLE || k < a.K) w[t] = *reinterpret_cast<const float4v *>(wrow[c] + k);
             }
             if constexpr (NORM) {
                 if (c == 0) {
@@ -1457,6 +1457,13 @@ __device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const 
         }
     }
 }
+template <int MM, int CG, bool GATED = false, bool RESIDUAL = false, bool NORM = false, int TRIPS = 8>
+__device__ __forceinline__ void skinny_kt_mfma_xreg_body(const MmArgs &a, const uint32_t block_x, const uint32_t block_y,
+                                                         const uint32_t *second = nullptr, const uint32_t one = 0,
+                                                         const MmResidual *res = nullptr, const NormFuse *nf = nullptr) {
+    if (a.K % (TRIPS * 256) == 0) skinny_kt_mfma_xreg_body_impl<true, MM, CG, GATED, RESIDUAL, NORM, TRIPS>(a, block_x, block_y, second, one, res, nf);
+    else skinny_kt_mfma_xreg_body_impl<false, MM, CG, GATED, RESIDUAL, NORM, TRIPS>(a, block_x, block_y, second, one, res, nf);
+}
 
 template <int MM, int CG, int TRIPS = 8> __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_kernel(const MmArgs a) {
     skinny_kt_mfma_xreg_body<MM, CG, false, false, false, TRIPS>(a, blockIdx.x, blockIdx.y);
@@ -1496,8 +1503,8 @@ __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_group_norm_kerne
 struct RopeGroup {
     RopeStore s[kMaxGroup];
 };
-template <bool NORM, int TRIPS>
-__global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_group_rope_kernel(const MmGroup g, const RopeGroup rg, const NormFuse nf) {
+template <bool WHOLE, bool NORM, int TRIPS>
+__device__ __forceinline__ void skinny_kt_mfma_xreg_group_rope_impl(const MmGroup &g, const RopeGroup &rg, const NormFuse &nf) {
     static_assert(TRIPS == 8 || TRIPS == 4, "chunks of 2048 or 1024");
     uint32_t bx;
     const uint32_t p = group_problem(g, bx);
@@ -1529,11 +1536,11 @@ __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_group_rope_kerne
         }
     }
     uint32_t kb, ks;
-    xreg_lane_k<TRIPS>(a.K, wave, b, kb, ks);
+    xreg_lane_k<TRIPS, WHOLE>(a.K, wave, b, kb, ks);
     // (a value of k beyond K contributes zeros: only a ragged last chunk has any)
     auto at = [&](const uint32_t *row, uint32_t k) {
         float4v v = {0.f, 0.f, 0.f, 0.f};
-        if (k < a.K) v = *reinterpret_cast<const float4v *>(row + k);
+        if (WHOLE || k < a.K) v = *reinterpret_cast<const float4v *>(row + k);
         return v;
     };
     for (uint32_t k0 = 0; k0 < a.K; k0 += TRIPS * 256) {
@@ -1601,6 +1608,11 @@ __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_group_rope_kerne
         if (threadIdx.x < 32 && col < a.N && m < a.M) rs.dst[(int64_t)m * rs.sb + (int64_t)(col / rs.hd) * rs.sh + col % rs.hd] = v;
     }
 }
+template <bool NORM, int TRIPS>
+__global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_group_rope_kernel(const MmGroup g, const RopeGroup rg, const NormFuse nf) {
+    if (g.p[0].K % (TRIPS * 256) == 0) skinny_kt_mfma_xreg_group_rope_impl<true, NORM, TRIPS>(g, rg, nf); // (the problems of a group share k)
+    else skinny_kt_mfma_xreg_group_rope_impl<false, NORM, TRIPS>(g, rg, nf);
+}
 
 // The same store for products whose heads go through an RMS norm of their own first (RopeStore::hgamma): the norm needs
 // the sum of squares over all hd columns of a head, and workgroups cannot exchange values inside a launch for less than a
@@ -1616,8 +1628,8 @@ __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_group_rope_kerne
 // that each multiply the whole head (its weights reach three of them out of L2) and store a quarter of it were measured
 // too: 29 to 35 us, every compute unit still has to pull a whole head.
 constexpr int kHeadThreads = 1024;
-template <bool NORM>
-__global__ __launch_bounds__(kHeadThreads) void skinny_kt_head_rope_kernel(const MmGroup g, const RopeGroup rg, const NormFuse nf) {
+template <bool WHOLE, bool NORM>
+__device__ __forceinline__ void skinny_kt_head_rope_impl(const MmGroup &g, const RopeGroup &rg, const NormFuse &nf) {
     constexpr int TRIPS = 4;
     uint32_t head;
     const uint32_t p = group_problem(g, head);
@@ -1626,10 +1638,10 @@ __global__ __launch_bounds__(kHeadThreads) void skinny_kt_head_rope_kernel(const
     const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x % 64, team = wave / 4, tw = wave % 4;
     const uint32_t j = lane % 4, b = lane / 4;
     uint32_t kb, ks;
-    xreg_lane_k<TRIPS>(a.K, tw, b, kb, ks);
+    xreg_lane_k<TRIPS, WHOLE>(a.K, tw, b, kb, ks);
     auto at = [&](const uint32_t *row, uint32_t k) { // (a value of k beyond K contributes zeros)
         float4v v = {0.f, 0.f, 0.f, 0.f};
-        if (k < a.K) v = *reinterpret_cast<const float4v *>(row + k);
+        if (WHOLE || k < a.K) v = *reinterpret_cast<const float4v *>(row + k);
         return v;
     };
     const uint32_t groups = rs.hd / 4, col0 = head * rs.hd; // (groups is a multiple of 4: every team makes every trip)
@@ -1639,7 +1651,7 @@ __global__ __launch_bounds__(kHeadThreads) void skinny_kt_head_rope_kernel(const
 #pragma unroll
         for (int t = 0; t < TRIPS; t++) {
             ww[t] = (float4v){0.f, 0.f, 0.f, 0.f};
-            if (kb + ks * t < a.K) ww[t] = __builtin_nontemporal_load(reinterpret_cast<const float4v *>(row + kb + ks * t));
+            if (WHOLE || kb + ks * t < a.K) ww[t] = __builtin_nontemporal_load(reinterpret_cast<const float4v *>(row + kb + ks * t));
         }
     };
     ask(w, team);
@@ -1734,6 +1746,11 @@ __global__ __launch_bounds__(kHeadThreads) void skinny_kt_head_rope_kernel(const
     }
     if (mine) rs.dst[(int64_t)m * rs.sb + (int64_t)head * rs.sh + d] = v;
 }
+template <bool NORM>
+__global__ __launch_bounds__(kHeadThreads) void skinny_kt_head_rope_kernel(const MmGroup g, const RopeGroup rg, const NormFuse nf) {
+    if (g.p[0].K % 1024 == 0) skinny_kt_head_rope_impl<true, NORM>(g, rg, nf); // (one chunk of 4 trips x 256)
+    else skinny_kt_head_rope_impl<false, NORM>(g, rg, nf);
+}
 
 // The gated pair when K is exactly one chunk (TRIPS * 256: the hidden size of the model): the workgroup asks for its
 // share of the activations (and of gamma, and of the row sums of an RMS norm) ONCE and walks `iters` consecutive
@@ -1744,20 +1761,19 @@ __global__ __launch_bounds__(kHeadThreads) void skinny_kt_head_rope_kernel(const
 // the 128 MiB of gate + up, more leave too few workgroups in flight.  For q / k / v and o (a quarter of the columns)
 // one group per workgroup stays the fastest.  Weights are read with the non-temporal hint.
 // M <= 4, batch folded away (one batch entry).  Epilogues as in skinny_kt_mfma_xreg_body.
-template <bool NORM, int TRIPS>
-__global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_cols_gated_kernel(const MmArgs a, const uint32_t *second, uint32_t one,
-                                                                                  uint32_t iters, const NormFuse nf) {
+template <bool WHOLE, bool NORM, int TRIPS>
+__device__ __forceinline__ void skinny_kt_mfma_xreg_cols_gated_impl(const MmArgs &a, const uint32_t *second, uint32_t one, uint32_t iters, const NormFuse &nf) {
     static_assert(TRIPS == 8 || TRIPS == 4, "chunks of 2048 or 1024");
     const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x % 64;
     const uint32_t j = lane % 4, b = lane / 4;
     uint32_t kb, ks; // this lane's k: kb + ks t (beyond K, in a chunk that K does not fill: zeros)
-    xreg_lane_k<TRIPS>(a.K, wave, b, kb, ks);
+    xreg_lane_k<TRIPS, WHOLE>(a.K, wave, b, kb, ks);
     const uint32_t *xrow = a.A + (int64_t)min(j, a.M - 1) * a.a_sm;
     float4v xr[TRIPS];
 #pragma unroll
     for (int t = 0; t < TRIPS; t++) {
         xr[t] = (float4v){0.f, 0.f, 0.f, 0.f};
-        if (kb + ks * t < a.K) xr[t] = *reinterpret_cast<const float4v *>(xrow + kb + ks * t);
+        if (WHOLE || kb + ks * t < a.K) xr[t] = *reinterpret_cast<const float4v *>(xrow + kb + ks * t);
     }
     float pv[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     float4v gm[NORM ? TRIPS : 1];
@@ -1770,7 +1786,7 @@ __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_cols_gated_kerne
 #pragma unroll
         for (int t = 0; t < TRIPS; t++) {
             gm[t] = (float4v){0.f, 0.f, 0.f, 0.f};
-            if (kb + ks * t < a.K) gm[t] = *reinterpret_cast<const float4v *>(nf.gamma + kb + ks * t);
+            if (WHOLE || kb + ks * t < a.K) gm[t] = *reinterpret_cast<const float4v *>(nf.gamma + kb + ks * t);
         }
     }
     __shared__ float part[2][4][32];
@@ -1782,7 +1798,7 @@ __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_cols_gated_kerne
 #pragma unroll
         for (int t = 0; t < TRIPS; t++) {
             w[t] = (float4v){0.f, 0.f, 0.f, 0.f};
-            if (kb + ks * t < a.K) w[t] = __builtin_nontemporal_load(reinterpret_cast<const float4v *>(row + ks * t));
+            if (WHOLE || kb + ks * t < a.K) w[t] = __builtin_nontemporal_load(reinterpret_cast<const float4v *>(row + ks * t));
         }
     };
     auto multiply = [&](float4v &sum, const float4v (&w)[TRIPS]) {
@@ -1853,6 +1869,12 @@ __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_cols_gated_kerne
             if (col < a.N && m < a.M) a.C[(uint64_t)m * a.N + col] = r;
         }
     }
+}
+template <bool NORM, int TRIPS>
+__global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_cols_gated_kernel(const MmArgs a, const uint32_t *second, uint32_t one,
+                                                                                  uint32_t iters, const NormFuse nf) {
+    if (a.K % (TRIPS * 256) == 0) skinny_kt_mfma_xreg_cols_gated_impl<true, NORM, TRIPS>(a, second, one, iters, nf);
+    else skinny_kt_mfma_xreg_cols_gated_impl<false, NORM, TRIPS>(a, second, one, iters, nf);
 }
 
 // Vectorised skinny kernel for short K (K <= 4*LPC, e.g. q.K^T of a decode step with
