@@ -56,6 +56,14 @@ CG_PROGRAM(RowsRmsNormAdd2b, 7, 0x38, -1, {16, 0, 1, 0}, {16, 8, 2, 8}, {18, 9, 
 CG_PROGRAM(RowsSoftmaxCausal, 5, 0x12, -1, {19, 0, 1, 0}, {149, 2, 3, 2}, {169, 9, 9, 9}, {18, 10, 4, 10}, {16, 8, 11, 8},
            {49, 12, 12, 12}, {17, 12, 13, 12}, {3, 14, 14, 14}, {48, 15, 15, 15}, {19, 15, 16, 15})
 
+// The same program for launches whose leaves and result all lie in 32-bit words (every tensor of an f32 model): the kernels
+// compiled for WordsOnly<P> carry no code for the narrow formats.
+template <class P> struct WordsOnly : P {
+    static constexpr bool words_only = true;
+};
+template <class P, class = void> struct words_only_of : std::false_type {};
+template <class P> struct words_only_of<P, std::void_t<decltype(P::words_only)>> : std::true_type {};
+
 template <class... P> struct ProgramList {};
 using MapPrograms = ProgramList<MapRope, MapSiluMul, MapResidual3a, MapResidual3b>;
 using RowsPrograms = ProgramList<RowsRmsNorm, RowsRmsNormAdd, RowsRmsNormAdd2a, RowsRmsNormAdd2b, RowsSoftmaxCausal>;
@@ -121,14 +129,14 @@ __device__ __forceinline__ void aot_load_leaf(const FusedArgs &a, const int64_t 
         for (int j = 0; j < VEC; j++) t[j] = a.leaf[L].ubits;
     } else if constexpr (L == P::pw) {
         const bool second = e >= a.pw_split;
-        if (second) load_words<VEC>(a.leaf2, off[P::nleaf], t);
-        else load_words<VEC>(a.leaf[L], off[L], t);
+        if (second) load_words<VEC, false, words_only_of<P>::value>(a.leaf2, off[P::nleaf], t);
+        else load_words<VEC, false, words_only_of<P>::value>(a.leaf[L], off[L], t);
         if ((a.pw_neg >> (second ? 1 : 0)) & 1u) {
 #pragma unroll
             for (int j = 0; j < VEC; j++) t[j] ^= 0x80000000u;
         }
     } else {
-        load_words<VEC>(a.leaf[L], off[L], t);
+        load_words<VEC, false, words_only_of<P>::value>(a.leaf[L], off[L], t);
     }
 }
 
@@ -170,7 +178,7 @@ template <class P, int VEC> __device__ __forceinline__ void aot_map_body(const F
     }
     const uint32_t rs[kMaxRowReduce] = {0, 0, 0};
     aot_run<P, VEC>(s, rs, a.fault, std::make_integer_sequence<int, P::ninstr>{});
-    store_words<VEC>(a.out, oo, s.v[kMaxLeaves + P::ninstr - 1]);
+    store_words<VEC, false, words_only_of<P>::value>(a.out, oo, s.v[kMaxLeaves + P::ninstr - 1]);
 }
 template <class P, int VEC> __global__ __launch_bounds__(kBlock) void aot_map_kernel(const FusedArgs a) {
     aot_map_body<P, VEC>(a, blockIdx.x);
@@ -333,7 +341,7 @@ __global__ __launch_bounds__(kBlock) void aot_rows_kernel(const FusedArgs a, uin
             const uint32_t it = lane + c * TPR;
             if (it < items) {
                 const Values<P, VEC> s = aot_eval<P, VEC, P::ninstr>(cache[c], rs, a.fault);
-                store_words<VEC>(a.out, obase + (int64_t)it * VEC * a.out.is, s.v[kMaxLeaves + P::ninstr - 1]);
+                store_words<VEC, false, words_only_of<P>::value>(a.out, obase + (int64_t)it * VEC * a.out.is, s.v[kMaxLeaves + P::ninstr - 1]);
             }
         }
     } else {
@@ -341,15 +349,25 @@ __global__ __launch_bounds__(kBlock) void aot_rows_kernel(const FusedArgs a, uin
             LeafWords<P, VEC> w;
             aot_fetch<P, VEC>(a, base, it, w);
             const Values<P, VEC> s = aot_eval<P, VEC, P::ninstr>(w, rs, a.fault);
-            store_words<VEC>(a.out, obase + (int64_t)it * VEC * a.out.is, s.v[kMaxLeaves + P::ninstr - 1]);
+            store_words<VEC, false, words_only_of<P>::value>(a.out, obase + (int64_t)it * VEC * a.out.is, s.v[kMaxLeaves + P::ninstr - 1]);
         }
     }
 }
 
 // ---- dispatch ---------------------------------------------------------------------------------------
+inline bool all_words(const FusedArgs &a) {
+    bool words = a.out.fmt == kFmtWords && a.leaf2.fmt == kFmtWords;
+    for (uint32_t l = 0; l < a.nleaf; l++) words &= a.leaf[l].fmt == kFmtWords;
+    return words;
+}
 template <class P> void aot_map_launch(const FusedArgs &a, dim3 grid, hipStream_t s) {
-    if (a.g.vec == 4)
+    const bool words = all_words(a);
+    if (a.g.vec == 4 && words)
+        hipLaunchKernelGGL((aot_map_kernel<WordsOnly<P>, 4>), grid, dim3(kBlock), 0, s, a);
+    else if (a.g.vec == 4)
         hipLaunchKernelGGL((aot_map_kernel<P, 4>), grid, dim3(kBlock), 0, s, a);
+    else if (words)
+        hipLaunchKernelGGL((aot_map_kernel<WordsOnly<P>, 1>), grid, dim3(kBlock), 0, s, a);
     else
         hipLaunchKernelGGL((aot_map_kernel<P, 1>), grid, dim3(kBlock), 0, s, a);
 }
@@ -388,8 +406,13 @@ template <class P, class... Rest>
 bool aot_rows_dispatch(const Pending &p, const FusedArgs &a, uint32_t *rowout, int tpr, dim3 grid, hipStream_t s,
                        ProgramList<P, Rest...>) {
     if (program_matches<P>(p)) {
-        if (a.g.vec == 4)
+        const bool words = all_words(a);
+        if (a.g.vec == 4 && words)
+            aot_rows_launch<WordsOnly<P>, 4>(a, rowout, tpr, grid, s);
+        else if (a.g.vec == 4)
             aot_rows_launch<P, 4>(a, rowout, tpr, grid, s);
+        else if (words)
+            aot_rows_launch<WordsOnly<P>, 1>(a, rowout, tpr, grid, s);
         else
             aot_rows_launch<P, 1>(a, rowout, tpr, grid, s);
         return true;

@@ -123,14 +123,16 @@ __device__ __forceinline__ void store_narrow(const Operand &o, int64_t off, cons
     }
 }
 
-template <int VEC, bool STREAM = false>
+// WORDS: the caller knows that the operand lies in 32-bit words (kernels compiled for launches whose operands all do:
+// without the narrow formats' code between its loads a program keeps them all in flight).
+template <int VEC, bool STREAM = false, bool WORDS = false>
 __device__ __forceinline__ void load_words(const Operand &o, int64_t off, uint32_t (&r)[VEC]) {
     if (o.uniform) {
 #pragma unroll
         for (int j = 0; j < VEC; j++) r[j] = o.ubits;
         return;
     }
-    if (o.fmt != kFmtWords) { // (the same for every lane: the format is a launch parameter)
+    if (!WORDS && o.fmt != kFmtWords) { // (the same for every lane: the format is a launch parameter)
         load_narrow<VEC>(o, off, r);
         return;
     }
@@ -157,9 +159,9 @@ __device__ __forceinline__ void load_words(const Operand &o, int64_t off, uint32
 
 // STREAM: the output is far larger than the caches; non-temporal stores keep it from
 // evicting the operands that are still being read.
-template <int VEC, bool STREAM = false>
+template <int VEC, bool STREAM = false, bool WORDS = false>
 __device__ __forceinline__ void store_words(const Operand &o, int64_t off, const uint32_t (&r)[VEC]) {
-    if (o.fmt != kFmtWords) {
+    if (!WORDS && o.fmt != kFmtWords) {
         store_narrow<VEC, STREAM>(o, off, r);
         return;
     }
