@@ -57,7 +57,7 @@ static int launch_seg_kernel(cg_backend *be, const AttnArgs &g, const FusedArgs 
 int launch_decode_attention(cg_backend *be, const Pending &p, const int64_t *pdims, int prank, const cg_tensor *q,
                             const cg_tensor *kt, const cg_tensor *v, cg_tensor *out) {
     if (int frc = flush_deferred(be)) return frc;
-    using P = RowsSoftmaxCausal;
+    using P = WordsOnly<RowsSoftmaxCausal>; // (the scores of an open product are f32, and so is all that meets them)
     if (!be->aot || !program_matches<P>(p) || !p.leaf[0].lazy || p.leaf[0].lazy->result || p.reduced) return kDeclined;
     cg_tensor pd; // the soft-max result as a dense descriptor: the left operand of p.V
     pd.rank = prank;
@@ -92,6 +92,7 @@ int launch_decode_attention(cg_backend *be, const Pending &p, const int64_t *pdi
     bool full;
     rc = fill_args(be, p, pdims, prank, nullptr, true, &a, &leaf_bytes, &full, -1, true);
     if (rc) return rc;
+    if (!all_words(a)) return kDeclined;
     uint64_t rows = 1;
     for (uint32_t d = 0; d < a.g.nouter; d++) rows *= a.g.od[d];
     if (a.g.inner != (uint32_t)T || rows != (uint64_t)f1.batch * (uint64_t)f1.M) return kDeclined;

@@ -79,6 +79,11 @@ struct cg_backend {
     uint32_t *fault_dev = nullptr;
     uint32_t *flag_dev = nullptr;   // 4-byte scratch for to_bool / compare
     uint32_t *flag_host = nullptr;  // pinned landing zone for it
+    // small read-backs (the tokens of a decode step): a kernel copies the words into pinned, device-visible memory and
+    // writes a sequence number behind them; the host polls it instead of waiting for the stream (CG_FAST_READBACK=0: never)
+    uint32_t *rb_host = nullptr, *rb_dev = nullptr;
+    uint32_t rb_seq = 0;
+    bool fast_readback = true;
     // host-to-device staging: two pinned buffers used in turn, each guarded by an event
     void *stage[2] = {nullptr, nullptr};
     hipEvent_t stage_ev[2] = {nullptr, nullptr};
@@ -457,6 +462,12 @@ int launch_fused_reduce(cg_backend *be, int kind, bool f32, const Pending &p, in
 // reduced: `out` is dense with one element per row; else `out` is a (strided) view of shape `dims`.
 int launch_fused_rows(cg_backend *be, const cg_tensor *out, const Pending &p, const int64_t *dims, int rank);
 int launch_arange(cg_backend *be, cg_tensor *out);
+// Copies n <= kReadbackWords words to be->rb_dev and then stores `seq` at word kReadbackWords of it, visible to the host.
+constexpr uint32_t kReadbackWords = 1024;
+int launch_small_readback(cg_backend *be, const uint32_t *src, uint32_t n, uint32_t seq);
+// A few words from the host travel with the launch, as kernel arguments: n <= kUploadWords words to dst.
+constexpr uint32_t kUploadWords = 64;
+int launch_small_upload(cg_backend *be, uint32_t *dst, const uint32_t *host_words, uint32_t n);
 int launch_fill_word(cg_backend *be, void *ptr, uint32_t bits);
 // dst[i] = (uint32_t)src[i] << 16 : bfloat16 bit patterns widened to f32
 int launch_bf16_widen(cg_backend *be, const void *src, void *dst, uint64_t n);

@@ -229,6 +229,35 @@ int launch_elementwise(cg_backend *be, int op, cg_dtype dt, const cg_tensor *out
                           : launch_ew_vec<1>(be, op, dt, a);
 }
 
+__global__ void small_readback_kernel(const uint32_t *src, uint32_t n, uint32_t *dst, uint32_t seq) {
+    for (uint32_t i = threadIdx.x; i < n; i += blockDim.x) dst[i] = src[i];
+    __threadfence_system();
+    __syncthreads();
+    if (threadIdx.x == 0) __hip_atomic_store(dst + kReadbackWords, seq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
+struct UploadWords {
+    uint32_t w[kUploadWords];
+};
+__global__ void small_upload_kernel(uint32_t *dst, const UploadWords v, uint32_t n) {
+    if (threadIdx.x < n) dst[threadIdx.x] = v.w[threadIdx.x];
+}
+
+int launch_small_upload(cg_backend *be, uint32_t *dst, const uint32_t *host_words, uint32_t n) {
+    UploadWords v;
+    memset(&v, 0, sizeof v);
+    memcpy(v.w, host_words, (size_t)n * 4);
+    hipLaunchKernelGGL(small_upload_kernel, dim3(1), dim3(kUploadWords), 0, be->stream, dst, v, n);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CG_OK : hip_fail(e, "upload launch");
+}
+
+int launch_small_readback(cg_backend *be, const uint32_t *src, uint32_t n, uint32_t seq) {
+    hipLaunchKernelGGL(small_readback_kernel, dim3(1), dim3(256), 0, be->stream, src, n, be->rb_dev, seq);
+    hipError_t e = hipGetLastError();
+    return e == hipSuccess ? CG_OK : hip_fail(e, "read-back launch");
+}
+
 int launch_arange(cg_backend *be, cg_tensor *out) {
     uint32_t n = (uint32_t)out->dims[0];
     hipLaunchKernelGGL(arange_kernel, dim3((n + 255) / 256), dim3(256), 0, be->stream,

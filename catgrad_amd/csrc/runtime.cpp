@@ -10,6 +10,7 @@
 #include "common.hpp"
 
 #include <algorithm>
+#include <chrono>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -757,6 +758,27 @@ static bool same_shape(const cg_tensor *a, const cg_tensor *b) {
 static int wait_and_check(cg_backend *be) {
     CG_HIP(hipStreamSynchronize(be->stream));
     if (!be->prof_pending.empty()) prof_drain(be);
+    uint32_t f = *reinterpret_cast<volatile uint32_t *>(be->fault_host);
+    if (f) {
+        *reinterpret_cast<volatile uint32_t *>(be->fault_host) = 0;
+        if (f & kFaultIndexRange) return fail(CG_ERR_RANGE, "index: index out of bounds (detected on device)");
+        if (f & kFaultDivZero) return fail(CG_ERR_RANGE, "attempt to divide by zero (detected on device)");
+    }
+    return CG_OK;
+}
+
+// The read-back kernel with sequence number `seq` has run (and with it everything before it on the stream): polls the word
+// it writes last.  Launch timings that wait to be read need the stream itself; so does a device that does not answer
+// within a tenth of a second (a fault: the stream's own wait reports it).
+static int wait_for_readback(cg_backend *be, uint32_t seq) {
+    if (be->prof_pending.size() > 2048) return wait_and_check(be);
+    volatile uint32_t *word = be->rb_host + kReadbackWords;
+    const auto t0 = std::chrono::steady_clock::now();
+    for (uint32_t spins = 0; *word != seq; spins++) {
+        if ((spins & 1023) == 1023 && std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(100)) return wait_and_check(be);
+        __builtin_ia32_pause();
+    }
+    std::atomic_thread_fence(std::memory_order_acquire);
     uint32_t f = *reinterpret_cast<volatile uint32_t *>(be->fault_host);
     if (f) {
         *reinterpret_cast<volatile uint32_t *>(be->fault_host) = 0;
@@ -2119,6 +2141,10 @@ int cg_backend_create(int device, cg_backend **out) {
     CG_HIP(hipHostMalloc((void **)&b->fault_host, 64, hipHostMallocMapped));
     memset(b->fault_host, 0, 64);
     CG_HIP(hipHostGetDevicePointer((void **)&b->fault_dev, b->fault_host, 0));
+    CG_HIP(hipHostMalloc((void **)&b->rb_host, (kReadbackWords + 16) * 4, hipHostMallocMapped));
+    memset(b->rb_host, 0, (kReadbackWords + 16) * 4);
+    CG_HIP(hipHostGetDevicePointer((void **)&b->rb_dev, b->rb_host, 0));
+    if (const char *fr = getenv("CG_FAST_READBACK")) b->fast_readback = fr[0] != '0';
     CG_HIP(hipHostMalloc((void **)&b->flag_host, 64, hipHostMallocDefault));
     CG_HIP(hipMalloc((void **)&b->flag_dev, 64));
     const char *fuse = getenv("CG_FUSE"); // CG_FUSE=0: run every element-wise op as its own kernel
@@ -2151,6 +2177,7 @@ static void backend_teardown(cg_backend *b) {
     }
     (void)hipHostFree(b->flag_host);
     (void)hipHostFree(b->fault_host);
+    (void)hipHostFree(b->rb_host);
     (void)hipStreamDestroy(b->stream);
     delete b;
 }
@@ -2313,6 +2340,9 @@ int cg_zeros(cg_backend *b, cg_dtype dtype, const size_t *dims, size_t rank, cg_
 // copy into one buffer overlaps the DMA out of the other, nothing waits for the device unless
 // a buffer is still in flight, and `src` may be freed on return.
 static int staged_upload(cg_backend *b, void *dst, const void *src, size_t bytes) {
+    // (a few words — the tokens of a decode step — go as the arguments of a small kernel: no staging buffer, no event)
+    if (b->fast_readback && bytes % 4 == 0 && bytes <= kUploadWords * 4 && reinterpret_cast<uintptr_t>(dst) % 4 == 0)
+        return launch_small_upload(b, static_cast<uint32_t *>(dst), static_cast<const uint32_t *>(src), (uint32_t)(bytes / 4));
     const char *s = static_cast<const char *>(src);
     char *d = static_cast<char *>(dst);
     for (size_t off = 0; off < bytes; off += kStageBytes) {
@@ -2507,7 +2537,14 @@ static int copy_out(cg_backend *b, const cg_tensor *t, void *dst, size_t len) {
     }
     const void *p;
     int rc = device_ptr(src, &p);
-    if (!rc) {
+    if (!rc && b->fast_readback && len <= kReadbackWords) {
+        // a few words (the tokens of a decode step): copied by a kernel into pinned memory that the host polls — neither
+        // the runtime's staged copy nor its wake-up stands between the last kernel of a step and the first of the next
+        const uint32_t seq = ++b->rb_seq;
+        rc = launch_small_readback(b, static_cast<const uint32_t *>(p), (uint32_t)len, seq);
+        if (!rc) rc = wait_for_readback(b, seq);
+        if (!rc) memcpy(dst, b->rb_host, len * 4);
+    } else if (!rc) {
         hipError_t e = hipMemcpyAsync(dst, p, len * 4, hipMemcpyDeviceToHost, b->stream);
         rc = e == hipSuccess ? wait_and_check(b) : hip_fail(e, "device to host copy");
     }
