@@ -63,6 +63,50 @@ struct ProfPending {
 } // namespace cg
 
 namespace cg {
+// Objects that every backend call makes and drops (tensor handles, deferred programs, lazy products, buffer records) come
+// from free lists of their own instead of the C library's heap, whose arena lock the runtime's own threads contend for: a
+// sampling profile of a launch-bound decode step had a fifth of the host's time in malloc / free and their lock.
+template <class T> struct Pooled {
+    // one list per type for the whole process, behind a flag that is almost never contended (a backend's calls are
+    // serialised by its own lock); it is never destroyed, so handles dropped while the process exits still find it
+    struct List {
+        std::atomic_flag busy = ATOMIC_FLAG_INIT;
+        std::vector<void *> free;
+    };
+    static List &list() {
+        static List *l = new List;
+        return *l;
+    }
+    static void *operator new(size_t n) {
+        if (n == sizeof(T)) {
+            List &l = list();
+            while (l.busy.test_and_set(std::memory_order_acquire)) {
+            }
+            void *p = nullptr;
+            if (!l.free.empty()) {
+                p = l.free.back();
+                l.free.pop_back();
+            }
+            l.busy.clear(std::memory_order_release);
+            if (p) return p;
+        }
+        return ::operator new(n);
+    }
+    static void operator delete(void *p, size_t n) {
+        if (!p) return;
+        if (n == sizeof(T)) {
+            List &l = list();
+            while (l.busy.test_and_set(std::memory_order_acquire)) {
+            }
+            const bool keep = l.free.size() < 1024;
+            if (keep) l.free.push_back(p);
+            l.busy.clear(std::memory_order_release);
+            if (keep) return;
+        }
+        ::operator delete(p);
+    }
+};
+
 struct LazyMm;
 struct DeferredWrite;
 struct Buffer;
@@ -145,7 +189,7 @@ inline uint64_t next_buffer_id() {
     return n.fetch_add(1);
 }
 
-struct Buffer {
+struct Buffer : Pooled<Buffer> {
     std::atomic<long> rc{1};
     const uint64_t id = next_buffer_id(); // never reused, unlike the address: what keys of kept results name
     void *ptr = nullptr;
@@ -191,7 +235,7 @@ struct Pending;
 // 0 is a broadcast axis.  `uniform` marks a tensor all of whose elements equal `ubits`
 // (rank-0 constants, zeros, and every view of them): such tensors own no memory until a
 // kernel needs to address them, and kernels take their value as an immediate.
-struct cg_tensor {
+struct cg_tensor : cg::Pooled<cg_tensor> {
     std::atomic<long> rc{1};
     cg_backend *be = nullptr;
     cg::Buffer *buf = nullptr;
@@ -327,7 +371,7 @@ struct NormFuse {
     uint32_t n_bits, eps_bits, exp_bits;
 };
 
-struct LazyMm {
+struct LazyMm : Pooled<LazyMm> {
     std::atomic<long> rc{1};
     // retained operands; y is concrete, x is concrete or (groupable products only) still the deferred RMS norm
     // of a residual stream with partial sums, see norm_fuse_of
@@ -378,7 +422,7 @@ struct LeafView {
     bool neg1, neg2;
 };
 
-struct Pending {
+struct Pending : Pooled<Pending> {
     int nleaf = 0, ninstr = 0;
     bool expensive = false; // holds pow / exp / log / sin / cos
     int nred = 0;           // row-reduce instructions in the program
