@@ -566,6 +566,34 @@ def test_narrow_operand_products_through_the_lds_ring_are_exact_on_integers(hip,
         del a, b, got
 
 
+@pytest.mark.parametrize("n", [2, 63, 64, 65, 1023, 1024, 1025, 5000])
+def test_small_uploads_and_read_backs_on_both_paths(hip, n):
+    """Up to 64 words go up as the arguments of a small kernel and up to 1024 come back through pinned memory that the host
+    polls; beyond that, and with CG_FAST_READBACK=0, the runtime's staged copies and the stream's own wait do it.  Both
+    paths, at the limits, f32 and u32, a view that has to be gathered first, and a read-back right behind a long launch."""
+    from backends import backend_with_env
+
+    rng = np.random.default_rng(n)
+    xv = rng.standard_normal(n).astype(np.float32)
+    iv = rng.integers(0, 2 ** 32, size=n, dtype=np.uint32)
+    big = rng.standard_normal((2048, 2048)).astype(np.float32)
+    slow = backend_with_env(CG_FAST_READBACK="0")
+    try:
+        for be in (hip, slow):
+            assert np.array_equal(be.to_numpy(be.from_numpy(xv)), xv)
+            assert np.array_equal(be.to_numpy(be.from_numpy(iv)), iv)
+            x2 = be.from_numpy(np.stack([xv, -xv]))
+            assert np.array_equal(be.to_numpy(be.slice(be.transpose(x2, 0, 1), 1, 1, 1)), -xv.reshape(n, 1))
+            # behind a launch of a few hundred microseconds: the words must be those of the finished product
+            b = be.from_numpy(big)
+            p = be.matmul(b, b)
+            got = be.to_numpy(be.slice(be.reshape(p, (2048 * 2048,)), 0, 7, min(n, 1024)))
+            ref = (big.astype(np.float64) @ big.astype(np.float64)).reshape(-1)[7:7 + min(n, 1024)]
+            np.testing.assert_allclose(got, ref, rtol=1e-3, atol=1e-2)
+    finally:
+        slow.close()
+
+
 # ---- full-size checks through size-independent properties -----------------------------------
 def test_microbench_shapes_properties(hip):
     """Config-2 shapes: linearity / invariants instead of a CPU recomputation."""
