@@ -139,10 +139,13 @@ int launch_decode_attention(cg_backend *be, const Pending &p, const int64_t *pdi
     // With at most 8 groups (a single sequence) the kernels below leave most of the device idle and the segments win from 2560
     // positions on: 8 KV heads, head_dim 128: 3000 positions 17.2 against 28.3 us, 12000 positions 31.7 against 59.0; 3 KV
     // heads, head_dim 64: 4500 positions 16.7 against 20.0, 12000 positions 22.1 against 40.5 (2100 positions: 15.8 against 15.8).
+    // So a single sequence takes the segments from 128 Ki cached values per KV head on (1024 positions of head_dim 128, 2048
+    // of 64): the Qwen3-0.6B shape's decode step (8 KV heads, head_dim 128, 16 query rows, 1024 to 1152 positions) takes 1.45
+    // to 1.53 ms with them against 1.64 to 1.66 ms with its 32 workgroups of the kernel below.
     // (Merging the segments inside the kernel — the workgroup that counts itself last at a device-scope counter reads the
     // others' results — was measured and costs what the combine launch costs: the stores must reach memory, the count must come
     // back and the loads go out again, 6 to 7 us in all; with a release / acquire fence per workgroup 24.0 against 19.3 us.)
-    if (be->attn_seg_from > 0 && (T >= be->attn_seg_from || (qrows > 256 && T >= 1024) || (f1.batch <= 8 && T >= 2560))) {
+    if (be->attn_seg_from > 0 && (T >= be->attn_seg_from || (qrows > 256 && T >= 1024) || (f1.batch <= 8 && T * hd >= 131072))) {
         const int64_t tpb = hd == 64 ? kSegBlock / 16 : kSegBlock / 32;
         int64_t want = std::min<int64_t>(attn_seg_max(), std::max<int64_t>(1, 256 / f1.batch));
         want = std::max<int64_t>(1, std::min<int64_t>(want, T / 64));

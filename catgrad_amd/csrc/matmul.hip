@@ -1614,117 +1614,41 @@ __global__ __launch_bounds__(kThreads) void skinny_kt_mfma_xreg_group_rope_kerne
     else skinny_kt_mfma_xreg_group_rope_impl<false, NORM, TRIPS>(g, rg, nf);
 }
 
-// The same store for products whose heads go through an RMS norm of their own first (RopeStore::hgamma): the norm needs
-// the sum of squares over all hd columns of a head, and workgroups cannot exchange values inside a launch for less than a
-// launch costs, so a workgroup of 1024 threads owns one head of one product.  Its sixteen waves are four teams of four; a
-// team multiplies one group of four columns at a time (the four waves share K as in the kernels above), the teams take the
-// head's column groups in turn, the next group's weights on their way.  K is at most one chunk of 1024 (the activations of
-// a row stay in registers).
-// A compute unit streams about 25 GB/s on its own, however deep its loads are queued (a ring of four register sets per
-// team, straight-line code, unconditional loads: no faster), so with one workgroup per head the launch is as slow as its
-// heads are few: 23 us for the 32 heads of 128 x 1024 of the Qwen3-0.6B shape against 8.9 us for the
-// eight-columns-per-workgroup kernel.  It still pays: the two norm launches and the embedding launch behind the product
-// (5 + 5 + 4.6 us and three hand-overs) go away, 2.46 -> 2.11 ms per decode step of that shape.  Four workgroups per head
-// that each multiply the whole head (its weights reach three of them out of L2) and store a quarter of it were measured
-// too: 29 to 35 us, every compute unit still has to pull a whole head.
-constexpr int kHeadThreads = 1024;
-template <bool WHOLE, bool NORM>
-__device__ __forceinline__ void skinny_kt_head_rope_impl(const MmGroup &g, const RopeGroup &rg, const NormFuse &nf) {
-    constexpr int TRIPS = 4;
-    uint32_t head;
-    const uint32_t p = group_problem(g, head);
-    const MmArgs &a = g.p[p];
-    const RopeStore &rs = rg.s[p];
-    const uint32_t wave = threadIdx.x / 64, lane = threadIdx.x % 64, team = wave / 4, tw = wave % 4;
-    const uint32_t j = lane % 4, b = lane / 4;
-    uint32_t kb, ks;
-    xreg_lane_k<TRIPS, WHOLE>(a.K, tw, b, kb, ks);
-    auto at = [&](const uint32_t *row, uint32_t k) { // (a value of k beyond K contributes zeros)
-        float4v v = {0.f, 0.f, 0.f, 0.f};
-        if (WHOLE || k < a.K) v = *reinterpret_cast<const float4v *>(row + k);
-        return v;
-    };
-    const uint32_t groups = rs.hd / 4, col0 = head * rs.hd; // (groups is a multiple of 4: every team makes every trip)
-    float4v w[TRIPS], wn[TRIPS];
-    auto ask = [&](float4v (&ww)[TRIPS], uint32_t grp) {
-        const uint32_t *row = a.B + (int64_t)min(col0 + grp * 4 + j, a.N - 1) * a.b_sn;
-#pragma unroll
-        for (int t = 0; t < TRIPS; t++) {
-            ww[t] = (float4v){0.f, 0.f, 0.f, 0.f};
-            if (WHOLE || kb + ks * t < a.K) ww[t] = __builtin_nontemporal_load(reinterpret_cast<const float4v *>(row + kb + ks * t));
-        }
-    };
-    ask(w, team);
-    const uint32_t *xrow = a.A + (int64_t)min(j, a.M - 1) * a.a_sm;
-    float4v xr[TRIPS];
-#pragma unroll
-    for (int t = 0; t < TRIPS; t++) xr[t] = at(xrow, kb + ks * t);
-    // the thread's (row, column) of the head in the last phase, and that column's factors: asked for before the walk along K
+// The store above for products whose heads go through an RMS norm of their own first (RopeStore::hgamma, the q / k norm of
+// Qwen3): the norm needs the sum of squares over all hd columns of a head, which lie with hd / 8 workgroups of the
+// eight-columns-per-workgroup kernel, and workgroups cannot exchange values inside a launch for less than a launch costs.
+// So that kernel leaves those products plain (rows already divided by the input norm) in scratch memory, N columns a row,
+// and this small launch finishes them: a workgroup per head of a product, a thread per (row, column) of the head; the
+// head's norm, the embedding and the store, op for op as the stand-alone programs.  Measured against one launch with a
+// workgroup of 1024 threads per head (a compute unit streams about 25 GB/s on its own however deep its loads are queued,
+// so that launch is as slow as its heads are few: 23 to 29 us for the 32 heads of 128 x 1024 of the Qwen3-0.6B shape):
+// 9 + 3 us and a hand-over, 1.94 -> 1.66 ms per decode step of that shape.
+struct HeadFinish {
+    RopeStore s[kMaxGroup];
+    const uint32_t *src[kMaxGroup];
+    uint32_t N[kMaxGroup];
+    uint32_t first[kMaxGroup + 1]; // prefix sums of the products' head counts
+    uint32_t n, M;
+};
+constexpr int kFinishThreads = 512;
+__global__ __launch_bounds__(kFinishThreads) void head_norm_rope_finish_kernel(const HeadFinish f) {
+    uint32_t p = 0;
+    while (p + 1 < f.n && blockIdx.x >= f.first[p + 1]) p++;
+    const uint32_t head = blockIdx.x - f.first[p];
+    const RopeStore &rs = f.s[p];
     const uint32_t e = threadIdx.x, m = e / rs.hd, d = e % rs.hd;
-    const bool mine = e < a.M * rs.hd; // (M <= 4, hd <= 128: at most 512 threads)
-    uint32_t hg = 0, cs = 0, sn = 0;
+    const bool mine = e < f.M * rs.hd; // (M <= 4, hd <= 128: at most 512 threads)
+    uint32_t hg = 0, cs = 0, sn = 0, v = 0;
+    if (mine) v = f.src[p][(int64_t)m * f.N[p] + head * rs.hd + d];
     if (mine && rs.hgamma) hg = rs.hgamma[d];
     if (mine && rs.rope) {
         cs = rs.cos[d];
         sn = rs.sin[d];
     }
-    __shared__ float nsum[4][4];
-    if constexpr (NORM) {
-        // (x / d * gamma) . w = ((x * gamma) . w) / d, d from the partial sums of squares that came with x
-#pragma unroll
-        for (int t = 0; t < TRIPS; t++) {
-            const float4v gm = at(nf.gamma, kb + ks * t);
-#pragma unroll
-            for (int q = 0; q < 4; q++) xr[t][q] = asf(apply<kMul, true>(asu(xr[t][q]), asu(gm[q]), 0, nullptr));
-        }
-        if (threadIdx.x < kThreads) { // the first four waves put the row sums together, always in the same order
-            float s = 0.0f;
-            for (uint32_t i = threadIdx.x; i < nf.blocks * 4; i += kThreads) s += nf.partials[i];
-#pragma unroll
-            for (int sh = 32; sh >= 4; sh >>= 1) s += __shfl_xor(s, sh);
-            if (lane < 4) nsum[wave][lane] = s;
-        }
-    }
-    __shared__ float part[2][kHeadThreads / 64][16];
-    __shared__ float hv[4][128], hy[4][128]; // the head's columns of every row: products, then normed values
-    for (uint32_t it = 0, grp = team; grp < groups; it++, grp += 4) {
-        if (grp + 4 < groups) ask(wn, grp + 4);
-        float4v acc = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int t = 0; t < TRIPS; t++) {
-            acc = __builtin_amdgcn_mfma_f32_4x4x1f32(xr[t][0], w[t][0], acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_4x4x1f32(xr[t][1], w[t][1], acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_4x4x1f32(xr[t][2], w[t][2], acc, 0, 0, 0);
-            acc = __builtin_amdgcn_mfma_f32_4x4x1f32(xr[t][3], w[t][3], acc, 0, 0, 0);
-        }
-#pragma unroll
-        for (int i = 0; i < 4; i++) {
-            float v = acc[i];
-#pragma unroll
-            for (int s = 32; s >= 4; s >>= 1) v += __shfl_xor(v, s);
-            if (lane < 4) part[it & 1][wave][i * 4 + j] = v;
-        }
-        __syncthreads(); // (the buffer written two trips ago was read before the barrier of the trip in between)
-        if (threadIdx.x < 64) { // (team, row, column) of this trip's four groups
-            const uint32_t tm = threadIdx.x / 16, t = threadIdx.x % 16, row = t / 4, c = t % 4;
-            const float (*pt)[16] = part[it & 1];
-            hv[row][(it * 4 + tm) * 4 + c] = (pt[tm * 4][t] + pt[tm * 4 + 1][t]) + (pt[tm * 4 + 2][t] + pt[tm * 4 + 3][t]);
-        }
-#pragma unroll
-        for (int t = 0; t < TRIPS; t++) w[t] = wn[t];
-    }
-    __syncthreads();
-    // ---- the head's values, one thread per (row, column): norm of the input rows, norm of the head, embedding, store
-    uint32_t v = 0;
-    if (mine) {
-        v = asu(hv[m][d]);
-        if constexpr (NORM) v = apply<kDiv, true>(v, norm_divisor(nf, (nsum[0][m] + nsum[1][m]) + (nsum[2][m] + nsum[3][m])), 0, nullptr);
-    }
+    __shared__ float hv[4][128], hy[4][128];
     if (rs.hgamma) { // (the same for the whole workgroup)
-        if constexpr (NORM) {
-            if (mine) hv[m][d] = asf(v);
-            __syncthreads();
-        }
+        if (mine) hv[m][d] = asf(v);
+        __syncthreads();
         if (mine) {
             float ss = 0.0f; // the row's sum of squares, its columns in order
             for (uint32_t c = 0; c < rs.hd; c++) ss += hv[m][c] * hv[m][c];
@@ -1745,11 +1669,6 @@ __device__ __forceinline__ void skinny_kt_head_rope_impl(const MmGroup &g, const
         }
     }
     if (mine) rs.dst[(int64_t)m * rs.sb + (int64_t)head * rs.sh + d] = v;
-}
-template <bool NORM>
-__global__ __launch_bounds__(kHeadThreads) void skinny_kt_head_rope_kernel(const MmGroup g, const RopeGroup rg, const NormFuse nf) {
-    if (g.p[0].K % 1024 == 0) skinny_kt_head_rope_impl<true, NORM>(g, rg, nf); // (one chunk of 4 trips x 256)
-    else skinny_kt_head_rope_impl<false, NORM>(g, rg, nf);
 }
 
 // The gated pair when K is exactly one chunk (TRIPS * 256: the hidden size of the model): the workgroup asks for its
@@ -2226,7 +2145,7 @@ int launch_matmul_group_rope(cg_backend *be, const cg_tensor *x, const cg_tensor
     memset(&rg, 0, sizeof rg);
     double bytes = distinct_bytes(x);
     uint32_t blocks = 0;
-    bool by_head = false; // some product's heads are normed: a workgroup per head (see skinny_kt_head_rope_kernel)
+    bool by_head = false; // some product's heads are normed: two launches (see head_norm_rope_finish_kernel)
     for (int i = 0; i < n; i++) by_head = by_head || stores[i].hgamma != nullptr;
     for (int i = 0; i < n; i++) {
         MmFold f;
@@ -2238,10 +2157,10 @@ int launch_matmul_group_rope(cg_backend *be, const cg_tensor *x, const cg_tensor
         if (f.batch != 1 || !xreg_narrow(a.M, a.K) || a.b_sk != 1 || !vec || a.N >= 8192) return kDeclined;
         if (i > 0 && (a.M != g.p[0].M || a.K != g.p[0].K || a.a_sm != g.p[0].a_sm)) return kDeclined;
         if (st.hd < 8 || st.hd % 8 || a.N % st.hd || !st.dst || (st.rope && (!st.cos || !st.sin))) return kDeclined;
-        if (by_head && (a.K > 1024 || st.hd % 16 || st.hd > 128)) return kDeclined;
+        if (by_head && (st.hd % 16 || st.hd > 128)) return kDeclined;
         rg.s[i] = st;
         g.first[i] = blocks;
-        blocks += by_head ? a.N / st.hd : a.N / 8;
+        blocks += a.N / 8;
         bytes += distinct_bytes(ys[i]) + 4.0 * (double)a.M * a.N;
     }
     g.first[n] = blocks;
@@ -2250,16 +2169,47 @@ int launch_matmul_group_rope(cg_backend *be, const cg_tensor *x, const cg_tensor
     memset(&none, 0, sizeof none);
     const bool wide = xreg_trips(g.p[0].K) == 8;
     ProfScope prof(be, CG_K_GEMM_SKINNY, bytes);
-    if (by_head) {
-        if (nf) hipLaunchKernelGGL(skinny_kt_head_rope_kernel<true>, dim3(blocks), dim3(kHeadThreads), 0, be->stream, g, rg, *nf);
-        else hipLaunchKernelGGL(skinny_kt_head_rope_kernel<false>, dim3(blocks), dim3(kHeadThreads), 0, be->stream, g, rg, none);
-        hipError_t he = hipGetLastError();
-        return he == hipSuccess ? CG_OK : hip_fail(he, "grouped matmul launch (a head per workgroup)");
+    HeadFinish hf;
+    void *tmp = nullptr;
+    size_t tmp_cls = 0;
+    uint32_t finish_heads = 0;
+    if (by_head) { // the normed products go to scratch memory as they are (see head_norm_rope_finish_kernel)
+        memset(&hf, 0, sizeof hf);
+        hf.M = g.p[0].M;
+        uint64_t words = 0;
+        for (int i = 0; i < n; i++)
+            if (stores[i].hgamma) words += (uint64_t)g.p[i].M * g.p[i].N;
+        if (int arc = be->pool.alloc(words * 4, &tmp, &tmp_cls)) return arc;
+        uint32_t *at = static_cast<uint32_t *>(tmp);
+        uint32_t heads = 0;
+        for (int i = 0; i < n; i++) {
+            if (!stores[i].hgamma) continue;
+            const uint32_t k = hf.n++;
+            hf.s[k] = stores[i];
+            hf.src[k] = at;
+            hf.N[k] = g.p[i].N;
+            hf.first[k] = heads;
+            heads += g.p[i].N / stores[i].hd;
+            RopeStore &plain = rg.s[i]; // column n of row m to at[m * N + n]
+            plain.dst = at;
+            plain.sb = g.p[i].N;
+            plain.sh = stores[i].hd;
+            plain.rope = 0;
+            plain.hgamma = nullptr;
+            at += (uint64_t)g.p[i].M * g.p[i].N;
+        }
+        hf.first[hf.n] = heads;
+        finish_heads = heads;
     }
     if (nf && wide) hipLaunchKernelGGL((skinny_kt_mfma_xreg_group_rope_kernel<true, 8>), dim3(blocks), dim3(kThreads), 0, be->stream, g, rg, *nf);
     else if (nf) hipLaunchKernelGGL((skinny_kt_mfma_xreg_group_rope_kernel<true, 4>), dim3(blocks), dim3(kThreads), 0, be->stream, g, rg, *nf);
     else if (wide) hipLaunchKernelGGL((skinny_kt_mfma_xreg_group_rope_kernel<false, 8>), dim3(blocks), dim3(kThreads), 0, be->stream, g, rg, none);
     else hipLaunchKernelGGL((skinny_kt_mfma_xreg_group_rope_kernel<false, 4>), dim3(blocks), dim3(kThreads), 0, be->stream, g, rg, none);
+    if (by_head) {
+        const uint32_t threads = (hf.M * 128 + 63) / 64 * 64;
+        hipLaunchKernelGGL(head_norm_rope_finish_kernel, dim3(finish_heads), dim3(threads), 0, be->stream, hf);
+        be->pool.free(tmp, tmp_cls); // stream-ordered: later users queue behind the finishing launch
+    }
     hipError_t e = hipGetLastError();
     return e == hipSuccess ? CG_OK : hip_fail(e, "grouped matmul with rotary store launch");
 }

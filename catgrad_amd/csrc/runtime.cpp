@@ -1776,7 +1776,7 @@ static bool head_norm_lazy(cg_tensor *x) {
     int64_t n = 1;
     for (int d = 0; d < m->rank; d++) n *= m->dims[d];
     const int64_t N = m->dims[m->rank - 1], K = m->x->rank > 0 ? m->x->dims[m->x->rank - 1] : 0;
-    if (n != R * hd || N % hd || n / N > 4 || K <= 256 || K > 1024 || K % 4) return false; // (what the head-per-workgroup kernel takes)
+    if (n != R * hd || N % hd || n / N > 4 || K <= 256 || K % 4) return false; // (what the kernels of launch_matmul_group_rope take)
     if (!p->leaf[1].uniform || !p->leaf[2].uniform || !p->leaf[3].uniform) return false;
     if (lg.uniform || lg.pw || lg.lazy || !lg.buf || is_narrow_buf(lg.buf) || lg.strides[1] != 1 || (R > 1 && lg.strides[0] != 0)) return false;
     LazyMm *m2 = new LazyMm;

@@ -537,7 +537,7 @@ def test_random_attention_block_steps_match_oracle(hip, oracle, seed):
 
     rng = np.random.default_rng(11000 + seed)
     B = int(rng.integers(1, 6))
-    K = int(rng.choice([1024, 2048, 2048, 3072, 512])) if seed < 24 else int(rng.choice([576, 1024, 1024, 960, 1536, 640, 2048]))
+    K = int(rng.choice([1024, 2048, 2048, 3072, 512])) if seed < 24 else int(rng.choice([576, 1024, 1024, 960, 1536, 640, 2048, 2560, 4096]))
     hd = int(rng.choice([64, 64, 128, 32]))
     qk = seed >= 24 and bool(rng.random() < 0.6)
     kvh, rep = int(rng.integers(1, 5)), int(rng.choice([1, 2, 4]))
