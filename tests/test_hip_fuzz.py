@@ -7,12 +7,17 @@ piecewise leaves, views of deferred results) in combinations the hand-written ca
 node carries a bound on its magnitude, graphs stay below 1e6, and the comparison is the element-wise tolerance of
 the contract (rtol 1e-4) plus an absolute term of 1e-5 of the node's bound, which covers differences that a
 subtraction of nearly equal values amplifies."""
+import os
+
 import numpy as np
 import pytest
 
 from catgrad_amd import _abi as A
 
 pytestmark = pytest.mark.gpu
+
+# CG_FUZZ_SEED_OFFSET=n runs every seeded test below on seeds n, n + 1, ... instead of 0, 1, ... (more of the same fuzz)
+SEED0 = int(os.environ.get("CG_FUZZ_SEED_OFFSET", "0"))
 
 LIMIT = 1e6
 
@@ -138,7 +143,7 @@ def evaluate(be, inputs, nodes, outs):
     return [got[id(n)] for n in outs]
 
 
-@pytest.mark.parametrize("seed", range(400))
+@pytest.mark.parametrize("seed", range(SEED0, SEED0 + 400))
 def test_random_graph_matches_oracle(hip, oracle, seed):
     rng = np.random.default_rng(1000 + seed)
     inputs, nodes, outs = random_graph(rng)
@@ -199,7 +204,7 @@ def hip_all_narrow():
     be.close()
 
 
-@pytest.mark.parametrize("seed", range(120))
+@pytest.mark.parametrize("seed", range(SEED0, SEED0 + 120))
 @pytest.mark.parametrize("dt", ["bf16", "f16", "fp8"])
 def test_random_graph_in_narrow_dtypes_matches_oracle(hip, hip_all_narrow, oracle, dt, seed):
     """The same random graphs on bf16 / f16 / fp8 tensors, on the default backend (tensors of these sizes are 32-bit
@@ -223,7 +228,7 @@ def test_random_graph_in_narrow_dtypes_matches_oracle(hip, hip_all_narrow, oracl
                 assert ok.all(), f"seed {seed} output {i}: worst {float(np.nanmax(np.abs(g - e)))}"
 
 
-@pytest.mark.parametrize("seed", range(200))
+@pytest.mark.parametrize("seed", range(SEED0, SEED0 + 200))
 def test_random_matmul_shapes_match_oracle(hip, oracle, seed):
     """[.., M, K] x [.., K, N] at random extents, either operand possibly a transposed or sliced view, the
     result possibly consumed by an element-wise op first.  Tolerance: 1e-3 of the result's largest magnitude."""
@@ -263,7 +268,7 @@ def test_random_matmul_shapes_match_oracle(hip, oracle, seed):
     assert float(np.abs(got - ref).max()) <= 1e-3 * scale, f"seed {seed}: M={M} K={K} N={N} batch={batch} xt={xt} yt={yt} pad={pad}"
 
 
-@pytest.mark.parametrize("seed", range(16))
+@pytest.mark.parametrize("seed", range(SEED0, SEED0 + 16))
 def test_random_wide_tile_products_match_float64(hip, seed):
     """Products large enough for the 256 x 256 tile (at least 256 tiles), whose loop over k has a lean part (whole tiles of
     aligned operands at fixed per-lane offsets) and a guarded tail: ragged extents in all three directions, either operand
@@ -305,7 +310,7 @@ def test_random_wide_tile_products_match_float64(hip, seed):
     assert (err <= 1e-3 * scale).all(), f"seed {seed}: worst {float((err / scale).max()):.3e} at {np.unravel_index(np.argmax(err / scale), err.shape)}"
 
 
-@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("seed", range(SEED0, SEED0 + 12))
 def test_random_wide_tile_products_of_16_bit_dtypes(hip, seed):
     """The same wide tile with bf16 / f16 tensors that cannot take the narrowed-in-memory path (a batch axis, or k no
     multiple of 8): f32 words are narrowed on their way into LDS and multiplied on the 16-bit matrix instructions, with
@@ -335,7 +340,7 @@ def test_random_wide_tile_products_of_16_bit_dtypes(hip, seed):
     assert bad.size == 0, f"seed {seed}: {len(bad)} mismatches, first {bad[:3].tolist()}"
 
 
-@pytest.mark.parametrize("seed", range(18))
+@pytest.mark.parametrize("seed", range(SEED0, SEED0 + 18))
 def test_random_products_of_operands_that_lie_narrow(hip, seed):
     """Products of bf16 / f16 / fp8 tensors that lie in memory as 2- / 1-byte patterns (uploads of 65536 elements and
     more): big ones (the 256 x 256 tile of narrow operands) and few-row ones (a decode-time linear layer), with the
@@ -390,7 +395,7 @@ def test_random_products_of_operands_that_lie_narrow(hip, seed):
     assert bad.size == 0, f"seed {seed}: {len(bad)} mismatches, first {bad[:3].tolist()}"
 
 
-@pytest.mark.parametrize("seed", range(12))
+@pytest.mark.parametrize("seed", range(SEED0, SEED0 + 12))
 def test_random_products_through_the_lds_ring(hip, seed):
     """Big products of narrow operands whose rows of k are whole turns of the four-stage LDS ring (random multiples of 128
     values of the 16-bit dtypes, of 256 of fp8): the kernel whose workgroups walk the tiles, at random extents (ragged
@@ -441,7 +446,7 @@ def test_random_products_through_the_lds_ring(hip, seed):
     assert bad.size == 0, f"seed {seed}: {len(bad)} mismatches, first {bad[:3].tolist()}"
 
 
-@pytest.mark.parametrize("seed", range(120))
+@pytest.mark.parametrize("seed", range(SEED0, SEED0 + 120))
 def test_random_attention_shapes_match_oracle(hip, oracle, seed):
     """The model graphs' attention (repeat_kv, scores, scale, causal mask rows, soft-max, context) at random
     batch / head / query / cache extents: decode steps (one query), speculative-width chunks and prefill chunks
@@ -466,7 +471,7 @@ def test_random_attention_shapes_match_oracle(hip, oracle, seed):
     np.testing.assert_allclose(got, ref, rtol=1e-4, atol=2e-5, err_msg=f"seed {seed}: B={B} kvh={kvh} rep={rep} hd={hd} S={S} T={T}")
 
 
-@pytest.mark.parametrize("seed", range(28))
+@pytest.mark.parametrize("seed", range(SEED0, SEED0 + 28))
 def test_random_decoder_blocks_match_oracle(hip, oracle, seed):
     """The dense part of a decoder layer at decode time (residual add in the store of the o / down product, RMS norm in
     the loads of the products behind it, gated pair) with random row counts and widths, and with the results — norms and
@@ -524,7 +529,7 @@ def test_random_decoder_blocks_match_oracle(hip, oracle, seed):
         np.testing.assert_allclose(gx, rx, rtol=1e-4, atol=1e-4)
 
 
-@pytest.mark.parametrize("seed", range(48))
+@pytest.mark.parametrize("seed", range(SEED0, SEED0 + 48))
 def test_random_attention_block_steps_match_oracle(hip, oracle, seed):
     """Decode steps of a whole attention block (q / k / v projections, heads split off, rotary embedding, cache append,
     attention) at random row counts, widths, head counts and sizes and cache lengths, with or without an RMS norm of a
