@@ -1374,9 +1374,11 @@ for _B, _K, _kvh, _rep, _T, _hd, _normed in ((4, 2048, 8, 4, 300, 64, True), (1,
                                               (1, 576, 3, 3, 200, 64, True), (4, 576, 3, 3, 300, 64, False), (2, 1536, 4, 2, 131, 64, True),
                                               (3, 2560, 2, 4, 260, 128, True),
                                               # q and k with an RMS norm per head ahead of the embedding (the Qwen3 attention block):
-                                              # the shapes whose store takes the norm (hidden up to 1024), and ones that do not
+                                              # shapes whose products leave the norm to the launch behind their store (any hidden
+                                              # size above 256; head sizes that are no powers of two), and one that does not
                                               (1, 1024, 8, 2, 300, 128, "qk_normed"), (4, 1024, 2, 2, 200, 64, "qk"), (2, 576, 3, 3, 131, 64, "qk_normed"),
-                                              (3, 512, 2, 1, 257, 32, "qk"), (1, 2048, 2, 2, 100, 128, "qk_normed"), (2, 256, 2, 2, 90, 64, "qk")):
+                                              (3, 512, 2, 1, 257, 32, "qk"), (1, 2048, 2, 2, 100, 128, "qk_normed"), (2, 256, 2, 2, 90, 64, "qk"),
+                                              (4, 2560, 4, 2, 77, 96, "qk_normed"), (2, 1280, 2, 3, 63, 80, "qk"), (3, 4096, 1, 4, 40, 48, "qk_normed")):
     @case(f"decode_qkv_rope_append_B{_B}_K{_K}_kv{_kvh}_rep{_rep}_T{_T}_hd{_hd}{('_' + _normed) if isinstance(_normed, str) else '_normed' if _normed else ''}", "red",
           (lambda n=2 * 3: [np.float64(4.0)] * n))   # projections of order one, rows of the caches likewise: 1e-3 of 4
     def _(B=_B, K=_K, kvh=_kvh, rep=_rep, T=_T, hd=_hd, normed=_normed):

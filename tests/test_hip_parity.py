@@ -351,6 +351,11 @@ def test_rotary_embedding_and_cache_append_run_in_the_products_store(hip):
                      ("decode_qkv_rope_append_B4_K1024_kv2_rep2_T200_hd64_qk", 6),
                      ("decode_qkv_rope_append_B2_K576_kv3_rep3_T131_hd64_qk_normed", 6),
                      ("decode_qkv_rope_append_B1_K2048_kv2_rep2_T100_hd128_qk_normed", 6),
+                     # (head sizes other than 64 and 128: the attention's soft-max is a launch of its own per step)
+                     ("decode_qkv_rope_append_B4_K2560_kv4_rep2_T77_hd96_qk_normed", 8),
+                     ("decode_qkv_rope_append_B2_K1280_kv2_rep3_T63_hd80_qk", 8),
+                     # (k and v of 48 columns are below what the products' kernels take)
+                     ("decode_qkv_rope_append_B3_K4096_kv1_rep4_T40_hd48_qk_normed", None),
                      ("decode_qkv_rope_append_B3_K256_kv4_rep2_T200_hd64", None)):
         c = by_name(name)
         hip.sync()
