@@ -414,6 +414,53 @@ __global__ __launch_bounds__(kBlock) void reduce_cols_kernel(const RowsArgs a, u
     }
 }
 
+// The same in ONE launch when there are outputs enough for every compute unit: a workgroup owns 32 neighbouring outputs (a
+// 128-byte line per step of the reduced axis), eight lanes of 16 bytes side by side and 32 groups of lanes that take the
+// steps in turn, eight loads in flight per lane; the groups meet in LDS and are merged in a fixed order.  No segments, no
+// partial results in memory, no second launch.
+template <int K, bool F>
+__global__ __launch_bounds__(kBlock) void reduce_cols_narrow_kernel(const RowsArgs a, uint32_t tiles0) {
+    constexpr uint32_t CH = 32, G = kBlock / 8; // outputs per workgroup, groups of lanes
+    typedef uint32_t u4 __attribute__((ext_vector_type(4)));
+    const uint32_t lx = threadIdx.x % 8, ly = threadIdx.x / 8;
+    const uint32_t tile = blockIdx.x % tiles0;
+    uint32_t rest = blockIdx.x / tiles0;
+    const uint32_t rest_index = rest;
+    int64_t base = 0;
+    for (uint32_t d = 1; d < a.nouter; d++) {
+        const uint32_t q = fastdiv(rest, a.odiv[d]);
+        base += (int64_t)(rest - q * a.od[d]) * a.os[d];
+        rest = q;
+    }
+    const uint32_t r0 = tile * CH + lx * 4; // (od[0] is a multiple of 32)
+    const uint32_t *p = reinterpret_cast<const uint32_t *>(a.x) + base + r0;
+    Acc<K, F> acc[4];
+    uint32_t i = ly;
+    for (; i + 7 * G < a.n; i += 8 * G) {
+        u4 t[8];
+#pragma unroll
+        for (int u = 0; u < 8; u++) t[u] = __builtin_nontemporal_load(reinterpret_cast<const u4 *>(p + (int64_t)(i + u * G) * a.sn));
+#pragma unroll
+        for (int u = 0; u < 8; u++)
+#pragma unroll
+            for (int v = 0; v < 4; v++) acc[v].take(t[u][v], i + u * G);
+    }
+    for (; i < a.n; i += G) {
+        const u4 t = __builtin_nontemporal_load(reinterpret_cast<const u4 *>(p + (int64_t)i * a.sn));
+#pragma unroll
+        for (int v = 0; v < 4; v++) acc[v].take(t[v], i);
+    }
+    __shared__ long long meet[G][CH];
+#pragma unroll
+    for (int v = 0; v < 4; v++) meet[ly][lx * 4 + v] = acc[v].pack();
+    __syncthreads();
+    if (threadIdx.x < CH) {
+        Acc<K, F> r = Acc<K, F>::unpack(meet[0][threadIdx.x]);
+        for (uint32_t g = 1; g < G; g++) r.merge(Acc<K, F>::unpack(meet[g][threadIdx.x]));
+        a.out[(uint64_t)rest_index * a.od[0] + tile * CH + threadIdx.x] = r.result();
+    }
+}
+
 template <int K, bool F>
 __global__ __launch_bounds__(kBlock) void reduce_cols_final_kernel(const long long *part, uint32_t *out, uint32_t segs, uint32_t rows) {
     // 64 neighbouring outputs per workgroup; the four waves split the segments (independent loads) and meet in LDS
@@ -438,6 +485,16 @@ template <int K, bool F> int launch_cols(cg_backend *be, const RowsArgs &a) {
     const uint32_t ch = vec ? 256 : 64, tiles0 = (R0 + ch - 1) / ch;
     const uint64_t blocks = (uint64_t)tiles0 * (a.rows / R0);
     if (blocks > 0x7FFFFFFFull) return fail(CG_ERR_UNSUPPORTED, "reduction extents above 2^31-1 workgroups");
+    // outputs enough for a workgroup of 32 on every compute unit and a long axis: one launch (env CG_COLS_NARROW=0: never)
+    static const bool narrow_allowed = [] { const char *e = getenv("CG_COLS_NARROW"); return !(e && e[0] == '0'); }();
+    if (narrow_allowed && vec && R0 % 32 == 0 && (uint64_t)(R0 / 32) * (a.rows / R0) >= 256 && a.n >= 1024) {
+        const uint64_t nblocks = (uint64_t)(R0 / 32) * (a.rows / R0);
+        if (nblocks <= 0x7FFFFFFFull) {
+            hipLaunchKernelGGL((reduce_cols_narrow_kernel<K, F>), dim3((uint32_t)nblocks), dim3(kBlock), 0, be->stream, a, R0 / 32);
+            hipError_t ne = hipGetLastError();
+            return ne == hipSuccess ? CG_OK : hip_fail(ne, "column reduction launch");
+        }
+    }
     // segments along the reduced axis until about 1024 workgroups are in flight (measured best on 8192 x 8192: 54.5 us against
     // 60 at 512 and 56.5 at 2048 and 4096; env CG_COLS_BLOCKS for measurements), at least 64 steps each
     static const uint64_t want = [] { const char *e = getenv("CG_COLS_BLOCKS"); return e ? (uint64_t)atoll(e) : 1024ull; }();

@@ -647,6 +647,35 @@ def test_microbench_shapes_properties(hip):
         assert (np.abs(full[bi, r] - ex) <= 1e-3 * sc).all()
 
 
+@pytest.mark.parametrize("shape", [(1500, 8192), (2, 1100, 4096), (8192, 8192)])
+def test_reductions_over_a_strided_axis_with_many_outputs(hip, shape):
+    """`sum` / `max` / `argmax` over the last axis of a transposed view with 8192 outputs and a long reduced axis (the
+    extents of the micro-benchmark's sum over axis 0, a ragged length, a batched one): the shapes that take the one-launch
+    column kernel.  sum within 1e-3 of sum |x| against float64, max exact, argmax bit-exact (planted ties: the last wins)."""
+    rng = np.random.default_rng(77 + len(shape))
+    x = rng.standard_normal(shape).astype(np.float32)
+    n = shape[-2]
+    x[..., 5, 64] = x[..., n - 3, 64] = np.float32(9.5)      # equal maxima down a column: the last one wins
+    x[..., :, 65] = np.float32(-1.25)                         # a column of equal values: index n - 1
+    x[..., 700, 66] = np.float32(np.nan)                      # +NaN: greatest for argmax, ignored by max, NaN sum
+    t = hip.transpose(hip.from_numpy(x), len(shape) - 2, len(shape) - 1)
+    xt = np.swapaxes(x, -1, -2)
+    x64 = xt.astype(np.float64)
+    s = hip.to_numpy(hip.sum(t.clone()))[..., 0]
+    ok = ~np.isnan(x64.sum(-1))
+    assert s.shape == xt.shape[:-1]
+    assert np.all(np.abs(s[ok] - x64.sum(-1)[ok]) <= 1e-3 * np.abs(x64).sum(-1)[ok])
+    assert np.isnan(s[~ok]).all() and (~ok).sum() == int(np.prod(shape[:-2]))
+    m = hip.to_numpy(hip.max(t.clone()))[..., 0]
+    np.testing.assert_array_equal(m, np.fmax.reduce(xt, axis=-1))
+    am = hip.to_numpy(hip.argmax(t))[..., 0]
+    i32 = np.ascontiguousarray(xt).view(np.int32).astype(np.int64)
+    key = np.where(i32 < 0, -(i32 & 0x7FFFFFFF) - 1, i32)    # total_cmp order of the bit patterns (ndarray.rs:670-681)
+    ref_am = (n - 1 - np.argmax(key[..., ::-1], axis=-1)).astype(np.uint32)
+    np.testing.assert_array_equal(am, ref_am)
+    assert (am[..., 64] == n - 3).all() and (am[..., 65] == n - 1).all() and (am[..., 66] == 700).all()
+
+
 def test_microbench_dense_reductions(hip):
     """Config-2 reductions on a DENSE random f32[4096, 8192] (the extent and kernel path the micro-benchmark times):
     sum within 1e-3 of sum |x| against float64, max exact, argmax bit-exact with the last of equal maxima (planted ties,
