@@ -2562,6 +2562,13 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
     const int64_t tiles128 = ((M + BM - 1) / BM) * (cols128 / 128) * (int64_t)batch;
     const bool narrow = (cols128 * 7 > cols64 * 8 || (tiles128 <= narrow_below && N >= 128)) && !half; // (the 16-bit kernels come in the two square tiles)
     const int bn = narrow ? 64 : 128;
+    // the 64 x 64 tile when even the narrow tile leaves most compute units without one (the linear layers of a short prompt on
+    // a narrow model: 512 x 576 is 36 tiles of 128 x 64): twice the workgroups, each cut along k half as often
+    // below 128 tiles of 128 x 64 — the SmolLM2-135M shape's prefill of 512 tokens 7.34 -> 6.84 ms, the Qwen3-0.6B shape's of
+    // 1024 unchanged (env CG_GEMM_TINY_BELOW=n moves the limit, for measurements; 0: never)
+    static const int64_t tiny_below = [] { const char *e = getenv("CG_GEMM_TINY_BELOW"); return e ? atoll(e) : 128ll; }();
+    const bool tiny = narrow && !kind && ((M + BM - 1) / BM) * (cols64 / 64) * (int64_t)batch < tiny_below && M > 64;
+    const int bm = tiny ? 64 : BM;
     // the 256 x 256 tile when it covers the chip at least once (env CG_GEMM_BIG=0 switches it off)
     const uint64_t tiles_big = (uint64_t)((M + 255) / 256) * ((N + 255) / 256) * batch;
     static const bool big_allowed = [] {
@@ -2738,7 +2745,7 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
         }
 #undef CG_MM_SWITCH
     } else {
-        uint64_t tiles = big ? tiles_big / batch : (uint64_t)((M + BM - 1) / BM) * ((N + bn - 1) / bn);
+        uint64_t tiles = big ? tiles_big / batch : (uint64_t)((M + bm - 1) / bm) * ((N + bn - 1) / bn);
         if (tiles > 0x7FFFFFFFull) return fail(CG_ERR_UNSUPPORTED, "matmul: too many tiles");
         // Too few tiles for the device (the linear layers of a short prefill on a narrow model): cut along k as well, so that
         // about two workgroups per compute unit run, each with at least 128 values of k; the partial tiles go to scratch memory
@@ -2858,6 +2865,8 @@ int launch_matmul(cg_backend *be, const cg_tensor *x, const cg_tensor *y, cg_ten
             CG_GEMM_HALF(AF, BF, 2);                                                                               \
         } else if (big)                                                                                            \
             hipLaunchKernelGGL((mfma_gemm_kernel<AF, BF, 4, 4>), grid, dim3(kThreads), gemm_lds_bytes(256, 256), s, a); \
+        else if (tiny)                                                                                             \
+            hipLaunchKernelGGL((mfma_gemm_kernel<AF, BF, 1, 1>), grid, dim3(kThreads), gemm_lds_bytes(64, 64), s, a); \
         else if (narrow)                                                                                           \
             hipLaunchKernelGGL((mfma_gemm_kernel<AF, BF, 1>), grid, dim3(kThreads), gemm_lds_bytes(64), s, a);     \
         else                                                                                                       \
